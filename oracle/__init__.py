@@ -1,0 +1,258 @@
+"""CPU checker for the HIP backend — TEST INFRASTRUCTURE ONLY.
+
+``oracle.lib``   ctypes view of ``libvv_oracle.so`` (our restatement of the
+                 reference's ``src/cpu`` layer kernels, ``vv_oracle.c``).
+``oracle.ref``   ctypes view of ``_ref/libvv_ref_cpu.so`` — the reference's own
+                 ``src/cpu/cpu_kernels.c`` compiled by ``oracle/Makefile`` — or
+                 ``None`` when that file was not built.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` import this package. The shipped library never does.
+
+All array arguments are C-contiguous numpy arrays; FP16 tensors travel as
+``uint16`` bit patterns so that nothing is converted behind the caller's back.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libvv_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libvv_ref_cpu.so")
+
+_u16p = C.POINTER(C.c_uint16)
+_f32p = C.POINTER(C.c_float)
+_i32p = C.POINTER(C.c_int32)
+
+
+def build(force: bool = False) -> None:
+    """Compile the checker (and ``_ref`` when the reference tree is present)."""
+    if force or not os.path.exists(_LIB_PATH) or \
+            os.path.getmtime(_LIB_PATH) < os.path.getmtime(os.path.join(_HERE, "vv_oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libvv_oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    if force or not os.path.exists(_REF_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "ref"], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    lib.vvo_half_to_float.restype = C.c_float
+    lib.vvo_half_to_float.argtypes = [C.c_uint16]
+    lib.vvo_float_to_half_rne.restype = C.c_uint16
+    lib.vvo_float_to_half_rne.argtypes = [C.c_float]
+    lib.vvo_widen_f16.argtypes = [_u16p, _f32p, C.c_size_t]
+    lib.vvo_narrow_f32_rne.argtypes = [_f32p, _u16p, C.c_size_t]
+    lib.vvo_rmsnorm_f32.argtypes = [_f32p, _u16p, _f32p, C.c_int, C.c_int, C.c_float]
+    lib.vvo_rope_f32.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]
+    lib.vvo_swiglu_f32.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    lib.vvo_residual_add_f32.argtypes = [_f32p, _f32p, C.c_int]
+    lib.vvo_embedding_f32.argtypes = [_u16p, _i32p, _f32p, C.c_int, C.c_int]
+    lib.vvo_rmsnorm_f16.argtypes = [_u16p, _u16p, _f32p, _u16p, C.c_int, C.c_int, C.c_float]
+    lib.vvo_residual_add_f16.argtypes = [_u16p, _u16p, C.c_size_t]
+    lib.vvo_add_rmsnorm_f16.argtypes = [_u16p, _u16p, _u16p, _f32p, _u16p,
+                                        C.c_int, C.c_int, C.c_float]
+    lib.vvo_rope_f16.argtypes = [_u16p, _f32p, _u16p, C.c_int, C.c_int, C.c_int,
+                                 C.c_int, C.c_float]
+    lib.vvo_swiglu_f16.argtypes = [_u16p, _u16p, _f32p, _u16p, C.c_size_t]
+    lib.vvo_swiglu_fused_f16.argtypes = [_u16p, _f32p, _u16p, C.c_int, C.c_int]
+    lib.vvo_embedding_f16.argtypes = [_u16p, _i32p, _u16p, C.c_int, C.c_int]
+    lib.vvo_bias_add_f16.argtypes = [_u16p, _u16p, C.c_int, C.c_int]
+    lib.vvo_fill_normal_f16.argtypes = [_u16p, C.c_size_t, C.c_uint64, C.c_double, C.c_double]
+    lib.vvo_fill_normal_f32.argtypes = [_f32p, C.c_size_t, C.c_uint64, C.c_double, C.c_double]
+    lib.vvo_fill_ids.argtypes = [_i32p, C.c_size_t, C.c_uint64, C.c_int32]
+    lib.vvo_threads.restype = C.c_int
+    lib.vvo_set_threads.argtypes = [C.c_int]
+    for name in ("vvo_rmsnorm_f32", "vvo_rope_f32", "vvo_swiglu_f32", "vvo_residual_add_f32",
+                 "vvo_embedding_f32", "vvo_rmsnorm_f16", "vvo_residual_add_f16",
+                 "vvo_add_rmsnorm_f16", "vvo_rope_f16", "vvo_swiglu_f16",
+                 "vvo_swiglu_fused_f16", "vvo_embedding_f16", "vvo_bias_add_f16"):
+        getattr(lib, name).restype = C.c_int
+    return lib
+
+
+def _load_ref():
+    """The reference's compiled CPU kernels (include/vibevoice/cpu_kernels.h names)."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    ref = C.CDLL(_REF_PATH)
+    vp = C.c_void_p
+    ref.vv_rmsnorm_cpu.argtypes = [_f32p, vp, _f32p, C.c_int, C.c_int, C.c_float]
+    ref.vv_rope_cpu.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]
+    ref.vv_swiglu_cpu.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    ref.vv_residual_add_cpu.argtypes = [_f32p, _f32p, C.c_int]
+    ref.vv_embedding_cpu.argtypes = [vp, _i32p, _f32p, C.c_int, C.c_int]
+    for name in ("vv_rmsnorm_cpu", "vv_rope_cpu", "vv_swiglu_cpu", "vv_residual_add_cpu",
+                 "vv_embedding_cpu", "vv_cpu_threads", "vv_cpu_physical_cores"):
+        getattr(ref, name).restype = C.c_int
+    ref.vv_cpu_simd_name.restype = C.c_char_p
+    return ref
+
+
+lib = _load()
+ref = _load_ref()
+
+
+# ── small numpy conveniences ────────────────────────────────────────────────
+
+def _p(a: np.ndarray, ty):
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
+    return a.ctypes.data_as(ty)
+
+
+def _check(st: int, what: str) -> None:
+    if st != 0:
+        raise RuntimeError(f"oracle {what} returned status {st}")
+
+
+def widen(h: np.ndarray) -> np.ndarray:
+    """uint16 FP16 bits -> float32, exactly."""
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, dtype=np.float32)
+    lib.vvo_widen_f16(_p(h, _u16p), _p(out, _f32p), h.size)
+    return out
+
+
+def narrow(f: np.ndarray) -> np.ndarray:
+    """float32 -> uint16 FP16 bits, round-to-nearest-even."""
+    f = np.ascontiguousarray(f, dtype=np.float32)
+    out = np.empty(f.shape, dtype=np.uint16)
+    lib.vvo_narrow_f32_rne(_p(f, _f32p), _p(out, _u16p), f.size)
+    return out
+
+
+def normal_f16(shape, seed: int, mean: float = 0.0, std: float = 1.0) -> np.ndarray:
+    out = np.empty(shape, dtype=np.uint16)
+    lib.vvo_fill_normal_f16(_p(out, _u16p), out.size, seed, mean, std)
+    return out
+
+
+def normal_f32(shape, seed: int, mean: float = 0.0, std: float = 1.0) -> np.ndarray:
+    out = np.empty(shape, dtype=np.float32)
+    lib.vvo_fill_normal_f32(_p(out, _f32p), out.size, seed, mean, std)
+    return out
+
+
+def ids(n: int, seed: int, bound: int) -> np.ndarray:
+    out = np.empty(n, dtype=np.int32)
+    lib.vvo_fill_ids(_p(out, _i32p), n, seed, bound)
+    return out
+
+
+def rmsnorm_f32(x: np.ndarray, w16: np.ndarray, eps: float) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    _check(lib.vvo_rmsnorm_f32(_p(x, _f32p), _p(w16, _u16p), _p(out, _f32p), rows, n, eps),
+           "rmsnorm_f32")
+    return out
+
+
+def rope_f32(x: np.ndarray, position_offset: int, theta: float) -> np.ndarray:
+    """x: [rows, n_heads, head_dim] float32; returns the rotated copy."""
+    v = np.array(x, dtype=np.float32, order="C", copy=True)
+    rows, n_heads, head_dim = v.shape
+    _check(lib.vvo_rope_f32(_p(v, _f32p), rows, n_heads, head_dim, position_offset, theta),
+           "rope_f32")
+    return v
+
+
+def swiglu_f32(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    gate = np.ascontiguousarray(gate, dtype=np.float32)
+    up = np.ascontiguousarray(up, dtype=np.float32)
+    out = np.empty_like(gate)
+    _check(lib.vvo_swiglu_f32(_p(gate, _f32p), _p(up, _f32p), _p(out, _f32p), gate.size),
+           "swiglu_f32")
+    return out
+
+
+def residual_add_f32(x: np.ndarray, y: np.ndarray) -> np.ndarray:
+    v = np.array(x, dtype=np.float32, order="C", copy=True)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    _check(lib.vvo_residual_add_f32(_p(v, _f32p), _p(y, _f32p), v.size), "residual_add_f32")
+    return v
+
+
+def embedding_f32(table16: np.ndarray, tok: np.ndarray) -> np.ndarray:
+    hidden = table16.shape[1]
+    tok = np.ascontiguousarray(tok, dtype=np.int32)
+    out = np.empty((tok.size, hidden), dtype=np.float32)
+    _check(lib.vvo_embedding_f32(_p(table16, _u16p), _p(tok, _i32p), _p(out, _f32p),
+                                 tok.size, hidden), "embedding_f32")
+    return out
+
+
+def rmsnorm_f16(x16: np.ndarray, w16: np.ndarray, eps: float):
+    """-> (ref float32, rne uint16) for the vv_rmsnorm_dev contract."""
+    rows, n = x16.shape
+    ref_ = np.empty((rows, n), dtype=np.float32)
+    rne = np.empty((rows, n), dtype=np.uint16)
+    _check(lib.vvo_rmsnorm_f16(_p(x16, _u16p), _p(w16, _u16p), _p(ref_, _f32p), _p(rne, _u16p),
+                               rows, n, eps), "rmsnorm_f16")
+    return ref_, rne
+
+
+def residual_add_f16(x16: np.ndarray, y16: np.ndarray) -> np.ndarray:
+    v = np.array(x16, dtype=np.uint16, order="C", copy=True)
+    _check(lib.vvo_residual_add_f16(_p(v, _u16p), _p(y16, _u16p), v.size), "residual_add_f16")
+    return v
+
+
+def add_rmsnorm_f16(res16: np.ndarray, x16: np.ndarray, w16: np.ndarray, eps: float):
+    """-> (updated residual uint16, normed ref float32, normed rne uint16)."""
+    rows, n = res16.shape
+    r = np.array(res16, dtype=np.uint16, order="C", copy=True)
+    ref_ = np.empty((rows, n), dtype=np.float32)
+    rne = np.empty((rows, n), dtype=np.uint16)
+    _check(lib.vvo_add_rmsnorm_f16(_p(r, _u16p), _p(x16, _u16p), _p(w16, _u16p), _p(ref_, _f32p),
+                                   _p(rne, _u16p), rows, n, eps), "add_rmsnorm_f16")
+    return r, ref_, rne
+
+
+def rope_f16(x16: np.ndarray, position_offset: int, theta: float):
+    rows, n_heads, head_dim = x16.shape
+    ref_ = np.empty(x16.shape, dtype=np.float32)
+    rne = np.empty(x16.shape, dtype=np.uint16)
+    _check(lib.vvo_rope_f16(_p(x16, _u16p), _p(ref_, _f32p), _p(rne, _u16p), rows, n_heads,
+                            head_dim, position_offset, theta), "rope_f16")
+    return ref_, rne
+
+
+def swiglu_f16(g16: np.ndarray, u16: np.ndarray):
+    ref_ = np.empty(g16.shape, dtype=np.float32)
+    rne = np.empty(g16.shape, dtype=np.uint16)
+    _check(lib.vvo_swiglu_f16(_p(g16, _u16p), _p(u16, _u16p), _p(ref_, _f32p), _p(rne, _u16p),
+                              g16.size), "swiglu_f16")
+    return ref_, rne
+
+
+def swiglu_fused_f16(gu16: np.ndarray):
+    rows, two_inter = gu16.shape
+    inter = two_inter // 2
+    ref_ = np.empty((rows, inter), dtype=np.float32)
+    rne = np.empty((rows, inter), dtype=np.uint16)
+    _check(lib.vvo_swiglu_fused_f16(_p(gu16, _u16p), _p(ref_, _f32p), _p(rne, _u16p),
+                                    rows, inter), "swiglu_fused_f16")
+    return ref_, rne
+
+
+def embedding_f16(table16: np.ndarray, tok: np.ndarray) -> np.ndarray:
+    hidden = table16.shape[1]
+    tok = np.ascontiguousarray(tok, dtype=np.int32)
+    out = np.empty((tok.size, hidden), dtype=np.uint16)
+    _check(lib.vvo_embedding_f16(_p(table16, _u16p), _p(tok, _i32p), _p(out, _u16p),
+                                 tok.size, hidden), "embedding_f16")
+    return out
+
+
+def bias_add_f16(out16: np.ndarray, bias16: np.ndarray) -> np.ndarray:
+    v = np.array(out16, dtype=np.uint16, order="C", copy=True)
+    M, N = v.shape
+    _check(lib.vvo_bias_add_f16(_p(v, _u16p), _p(bias16, _u16p), M, N), "bias_add_f16")
+    return v

@@ -1,0 +1,343 @@
+/*
+ * vv_oracle.c — CPU restatement of vibevoice.c's src/cpu layer kernels.
+ *
+ * TEST INFRASTRUCTURE ONLY (see vv_oracle.h). Build with
+ *   gcc -O2 -fopenmp -ffp-contract=off -fPIC -shared vv_oracle.c -lm
+ * No -ffast-math, no -march: the reference builds src/cpu/cpu_kernels.c with
+ * plain -O3 (CMakeLists.txt:111-128), so products and sums are unfused and in
+ * source order, and libm's powf/cosf/sinf/expf/sqrtf are the scalar glibc
+ * ones. Keeping that here is what makes the low bits reproducible.
+ */
+#include "vv_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+enum { VVO_OK = 0, VVO_ERR_NULL_PTR = -2 };   /* types.h:19,23 */
+
+/* ── FP16 conversions ─────────────────────────────────────────────────── */
+
+float vvo_half_to_float(uint16_t h) {
+    /* types.h:107-129: exact widening. Written here as three value classes:
+     * inf/NaN keep the payload, subnormals are an integer times 2^-24, and
+     * normals shift the exponent bias from 15 to 127. */
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t mag = h & 0x7FFFu;
+    union { uint32_t u; float f; } v;
+    if (mag >= 0x7C00u) {
+        v.u = sign | 0x7F800000u | ((mag & 0x3FFu) << 13);
+    } else if (mag < 0x0400u) {
+        v.f = (float)mag * 0x1p-24f;          /* exact: mag < 2^10 */
+        v.u |= sign;
+    } else {
+        v.u = sign | ((mag << 13) + (112u << 23));
+    }
+    return v.f;
+}
+
+uint16_t vvo_float_to_half_rne(float f) {
+    /* types.h:171-196: round-to-nearest-even. The subnormal range is rounded
+     * by the FPU itself (adding 0.5f leaves round(|f| * 2^24) in the low
+     * mantissa bits under the default rounding mode); normals add the
+     * classic 0xFFF + lsb bias before dropping 13 bits. */
+    union { float f; uint32_t u; } v;
+    v.f = f;
+    const uint16_t sign = (uint16_t)((v.u >> 16) & 0x8000u);
+    uint32_t a = v.u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);       /* NaN */
+    if (a >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);      /* -> inf */
+    if (a < 0x38800000u) {                                        /* < 2^-14 */
+        union { float f; uint32_t u; } t;
+        v.u = a;
+        t.f = v.f + 0.5f;
+        return (uint16_t)(sign | (t.u - 0x3F000000u));
+    }
+    a += 0xC8000000u + 0xFFFu + ((a >> 13) & 1u);   /* rebias 127 -> 15 */
+    return (uint16_t)(sign | (a >> 13));
+}
+
+void vvo_widen_f16(const uint16_t* in, float* out, size_t n) {
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++) out[i] = vvo_half_to_float(in[i]);
+}
+
+void vvo_narrow_f32_rne(const float* in, uint16_t* out, size_t n) {
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++) out[i] = vvo_float_to_half_rne(in[i]);
+}
+
+/* ── the five reference kernels, FP32 activations ─────────────────────── */
+
+int vvo_rmsnorm_f32(const float* input, const uint16_t* weight_f16,
+                    float* output, int rows, int n, float eps) {
+    /* cpu_kernels.c:1432-1451. Per row: double sum of squares in index
+     * order, one float reciprocal square root, then (x * inv) * w. */
+    if (!input || !weight_f16 || !output) return VVO_ERR_NULL_PTR;
+    int r;
+#pragma omp parallel for schedule(static)
+    for (r = 0; r < rows; r++) {
+        const float* x = input + (size_t)r * n;
+        float* y = output + (size_t)r * n;
+        double sumsq = 0.0;
+        for (int i = 0; i < n; i++) {
+            const double xi = (double)x[i];
+            sumsq += xi * xi;
+        }
+        const float mean = (float)(sumsq / n);
+        const float inv = 1.0f / sqrtf(mean + eps);
+        for (int i = 0; i < n; i++) {
+            const float scaled = x[i] * inv;
+            y[i] = scaled * vvo_half_to_float(weight_f16[i]);
+        }
+    }
+    return VVO_OK;
+}
+
+int vvo_rope_f32(float* x, int rows, int n_heads, int head_dim,
+                 int position_offset, float theta) {
+    /* cpu_kernels.c:1453-1478. Rotate-half pairing (i, i + head_dim/2); the
+     * frequency, angle, cosine and sine are all float, recomputed per head
+     * exactly as the reference does (same libm calls, same arguments). */
+    if (!x) return VVO_ERR_NULL_PTR;
+    const int half = head_dim / 2;
+    int r;
+#pragma omp parallel for schedule(static)
+    for (r = 0; r < rows; r++) {
+        const int pos = position_offset + r;
+        for (int h = 0; h < n_heads; h++) {
+            float* v = x + ((size_t)r * n_heads + h) * head_dim;
+            for (int i = 0; i < half; i++) {
+                const float expo = -2.0f * (float)i / (float)head_dim;
+                const float freq = powf(theta, expo);
+                const float ang = (float)pos * freq;
+                const float c = cosf(ang);
+                const float s = sinf(ang);
+                const float a = v[i];
+                const float b = v[i + half];
+                const float ac = a * c, bs = b * s;
+                const float as = a * s, bc = b * c;
+                v[i] = ac - bs;
+                v[i + half] = as + bc;
+            }
+        }
+    }
+    return VVO_OK;
+}
+
+int vvo_swiglu_f32(const float* gate, const float* up, float* output, int n) {
+    /* cpu_kernels.c:1536-1548: (g / (1 + expf(-g))) * u. Safe for
+     * output == gate: element i is read before it is written. */
+    if (!gate || !up || !output) return VVO_ERR_NULL_PTR;
+    int i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < n; i++) {
+        const float g = gate[i];
+        const float denom = 1.0f + expf(-g);
+        const float silu = g / denom;
+        output[i] = silu * up[i];
+    }
+    return VVO_OK;
+}
+
+int vvo_residual_add_f32(float* x, const float* y, int n) {
+    /* cpu_kernels.c:1550-1558 */
+    if (!x || !y) return VVO_ERR_NULL_PTR;
+    int i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < n; i++) x[i] = x[i] + y[i];
+    return VVO_OK;
+}
+
+int vvo_embedding_f32(const uint16_t* table_f16, const int32_t* ids,
+                      float* output, int rows, int hidden) {
+    /* cpu_kernels.c:1560-1568: single-threaded row copy, widened to FP32
+     * (f16_row, :587-596). Row offsets are size_t; ids are not checked. */
+    if (!table_f16 || !ids || !output) return VVO_ERR_NULL_PTR;
+    for (int r = 0; r < rows; r++) {
+        const uint16_t* src = table_f16 + (size_t)ids[r] * (size_t)hidden;
+        float* dst = output + (size_t)r * (size_t)hidden;
+        for (int i = 0; i < hidden; i++) dst[i] = vvo_half_to_float(src[i]);
+    }
+    return VVO_OK;
+}
+
+/* ── device-contract forms ─────────────────────────────────────────────── */
+
+static void emit(const float* src, float* out_ref, uint16_t* out_rne, size_t n) {
+    if (out_ref && out_ref != src) memcpy(out_ref, src, n * sizeof(float));
+    if (out_rne) vvo_narrow_f32_rne(src, out_rne, n);
+}
+
+int vvo_rmsnorm_f16(const uint16_t* x, const uint16_t* w, float* out_ref,
+                    uint16_t* out_rne, int rows, int n, float eps) {
+    if (!x || !w) return VVO_ERR_NULL_PTR;
+    const size_t total = (size_t)rows * (size_t)n;
+    float* xin = (float*)malloc((total ? total : 1) * sizeof(float));
+    float* y = (float*)malloc((total ? total : 1) * sizeof(float));
+    if (!xin || !y) { free(xin); free(y); return -3; }
+    vvo_widen_f16(x, xin, total);
+    const int st = vvo_rmsnorm_f32(xin, w, y, rows, n, eps);
+    if (st == VVO_OK) emit(y, out_ref, out_rne, total);
+    free(xin); free(y);
+    return st;
+}
+
+int vvo_residual_add_f16(uint16_t* x, const uint16_t* y, size_t n) {
+    if (!x || !y) return VVO_ERR_NULL_PTR;
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++) {
+        float a = vvo_half_to_float(x[i]);
+        const float b = vvo_half_to_float(y[i]);
+        /* the same FP32 add vvo_residual_add_f32 does, then one RNE round */
+        a = a + b;
+        x[i] = vvo_float_to_half_rne(a);
+    }
+    return VVO_OK;
+}
+
+int vvo_add_rmsnorm_f16(uint16_t* residual, const uint16_t* x,
+                        const uint16_t* w, float* normed_ref,
+                        uint16_t* normed_rne, int rows, int n, float eps) {
+    if (!residual || !x || !w) return VVO_ERR_NULL_PTR;
+    const int st = vvo_residual_add_f16(residual, x, (size_t)rows * (size_t)n);
+    if (st != VVO_OK) return st;
+    return vvo_rmsnorm_f16(residual, w, normed_ref, normed_rne, rows, n, eps);
+}
+
+int vvo_rope_f16(const uint16_t* x, float* out_ref, uint16_t* out_rne,
+                 int rows, int n_heads, int head_dim, int position_offset,
+                 float theta) {
+    if (!x) return VVO_ERR_NULL_PTR;
+    const size_t total = (size_t)rows * (size_t)n_heads * (size_t)head_dim;
+    float* v = (float*)malloc((total ? total : 1) * sizeof(float));
+    if (!v) return -3;
+    vvo_widen_f16(x, v, total);
+    const int st = vvo_rope_f32(v, rows, n_heads, head_dim, position_offset, theta);
+    if (st == VVO_OK) emit(v, out_ref, out_rne, total);
+    free(v);
+    return st;
+}
+
+int vvo_swiglu_f16(const uint16_t* gate, const uint16_t* up, float* out_ref,
+                   uint16_t* out_rne, size_t n) {
+    if (!gate || !up) return VVO_ERR_NULL_PTR;
+    /* chunked so that n beyond INT_MAX never reaches the int-sized kernel */
+    const size_t chunk = (size_t)1 << 22;
+    float* g = (float*)malloc(chunk * sizeof(float));
+    float* u = (float*)malloc(chunk * sizeof(float));
+    if (!g || !u) { free(g); free(u); return -3; }
+    for (size_t off = 0; off < n; off += chunk) {
+        const size_t m = n - off < chunk ? n - off : chunk;
+        vvo_widen_f16(gate + off, g, m);
+        vvo_widen_f16(up + off, u, m);
+        vvo_swiglu_f32(g, u, g, (int)m);        /* in place, as decoder.c:1473 */
+        emit(g, out_ref ? out_ref + off : NULL, out_rne ? out_rne + off : NULL, m);
+    }
+    free(g); free(u);
+    return VVO_OK;
+}
+
+int vvo_swiglu_fused_f16(const uint16_t* gate_up, float* out_ref,
+                         uint16_t* out_rne, int rows, int inter) {
+    if (!gate_up) return VVO_ERR_NULL_PTR;
+    for (int r = 0; r < rows; r++) {
+        const uint16_t* g = gate_up + (size_t)r * 2u * (size_t)inter;
+        const size_t o = (size_t)r * (size_t)inter;
+        const int st = vvo_swiglu_f16(g, g + inter, out_ref ? out_ref + o : NULL,
+                                      out_rne ? out_rne + o : NULL, (size_t)inter);
+        if (st != VVO_OK) return st;
+    }
+    return VVO_OK;
+}
+
+int vvo_embedding_f16(const uint16_t* table, const int32_t* ids,
+                      uint16_t* out, int rows, int hidden) {
+    if (!table || !ids || !out) return VVO_ERR_NULL_PTR;
+    for (int r = 0; r < rows; r++)
+        memcpy(out + (size_t)r * (size_t)hidden,
+               table + (size_t)ids[r] * (size_t)hidden,
+               (size_t)hidden * sizeof(uint16_t));
+    return VVO_OK;
+}
+
+int vvo_bias_add_f16(uint16_t* out, const uint16_t* bias, int M, int N) {
+    if (!out || !bias) return VVO_ERR_NULL_PTR;
+    int m;
+#pragma omp parallel for schedule(static)
+    for (m = 0; m < M; m++) {
+        uint16_t* row = out + (size_t)m * (size_t)N;
+        for (int j = 0; j < N; j++) {
+            const float v = vvo_half_to_float(row[j]) + vvo_half_to_float(bias[j]);
+            row[j] = vvo_float_to_half_rne(v);
+        }
+    }
+    return VVO_OK;
+}
+
+/* ── seeded inputs ─────────────────────────────────────────────────────── */
+
+static inline uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+/* One standard normal per (seed, i): Box-Muller on two counter-based draws. */
+static inline double normal_at(uint64_t seed, uint64_t i) {
+    const uint64_t base = seed * 0xD1342543DE82EF95ull + 2u * i;
+    const uint64_t a = splitmix64(base), b = splitmix64(base + 1u);
+    const double u1 = ((double)(a >> 11) + 1.0) * 0x1p-53;   /* (0, 1] */
+    const double u2 = (double)(b >> 11) * 0x1p-53;           /* [0, 1) */
+    return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
+}
+
+void vvo_fill_normal_f32(float* out, size_t n, uint64_t seed,
+                         double mean, double std) {
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++)
+        out[i] = (float)(mean + std * normal_at(seed, (uint64_t)i));
+}
+
+void vvo_fill_normal_f16(uint16_t* out, size_t n, uint64_t seed,
+                         double mean, double std) {
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++)
+        out[i] = vvo_float_to_half_rne(
+            (float)(mean + std * normal_at(seed, (uint64_t)i)));
+}
+
+void vvo_fill_ids(int32_t* out, size_t n, uint64_t seed, int32_t bound) {
+    long i;
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < (long)n; i++) {
+        const uint64_t r = splitmix64(seed * 0xA0761D6478BD642Full + (uint64_t)i);
+        /* multiply-shift maps 64 random bits onto [0, bound) */
+        out[i] = (int32_t)(((unsigned __int128)r * (uint64_t)bound) >> 64);
+    }
+}
+
+int vvo_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+void vvo_set_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}

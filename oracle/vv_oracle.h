@@ -1,0 +1,113 @@
+/*
+ * vv_oracle.h — CPU restatement of vibevoice.c's src/cpu layer kernels.
+ *
+ * TEST INFRASTRUCTURE ONLY. This library is the checker for the HIP backend:
+ * tests, the smoke check and the benchmark's cpu_baseline leg link it; the
+ * shipped library (libvibevoice_hip.so) never does and has no CPU fallback.
+ *
+ * Two families of functions:
+ *   vvo_*_f32   the reference's CPU kernels, restated operation by operation
+ *               (FP32 activations, FP16 weights/table), one function per
+ *               reference function, each citing the lines it follows;
+ *   vvo_*_f16   the same arithmetic applied to the device contract of
+ *               include/vibevoice/device.h (FP16 tensors in and out): inputs
+ *               are widened exactly, the f32 kernel runs, and the result is
+ *               returned both as FP32 ("ref", what the tolerance is measured
+ *               against) and rounded to FP16 with round-to-nearest-even
+ *               ("rne", what a device kernel that made no other error stores).
+ *
+ * Parity status (what pins each function is listed in tests/test_oracle_*.py):
+ *   every function below is pinned by the compiled reference (oracle/_ref,
+ *   bit-for-bit) where that builds, by committed golden vectors made from it,
+ *   and by closed forms / invariants that do not retype its formula.
+ */
+#ifndef VV_ORACLE_H
+#define VV_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* FP16 <-> FP32. Follows include/vibevoice/types.h:107-129 (half -> float,
+ * exact, subnormals/inf/NaN included) and types.h:171-196 (float -> half,
+ * round-to-nearest-even; NaN -> quiet NaN with the sign kept). */
+float    vvo_half_to_float(uint16_t h);
+uint16_t vvo_float_to_half_rne(float f);
+void     vvo_widen_f16(const uint16_t* in, float* out, size_t n);
+void     vvo_narrow_f32_rne(const float* in, uint16_t* out, size_t n);
+
+/* src/cpu/cpu_kernels.c:1432-1451 */
+int vvo_rmsnorm_f32(const float* input, const uint16_t* weight_f16,
+                    float* output, int rows, int n, float eps);
+/* src/cpu/cpu_kernels.c:1453-1478 */
+int vvo_rope_f32(float* x, int rows, int n_heads, int head_dim,
+                 int position_offset, float theta);
+/* src/cpu/cpu_kernels.c:1536-1548 */
+int vvo_swiglu_f32(const float* gate, const float* up, float* output, int n);
+/* src/cpu/cpu_kernels.c:1550-1558 */
+int vvo_residual_add_f32(float* x, const float* y, int n);
+/* src/cpu/cpu_kernels.c:1560-1568 with f16_row :587-596 */
+int vvo_embedding_f32(const uint16_t* table_f16, const int32_t* ids,
+                      float* output, int rows, int hidden);
+
+/* ── device-contract forms (FP16 in, FP32 ref + FP16 rne out) ──────────── */
+
+/* vv_rmsnorm_dev contract (device.h:490-492). out_ref/out_rne may be NULL. */
+int vvo_rmsnorm_f16(const uint16_t* x, const uint16_t* w, float* out_ref,
+                    uint16_t* out_rne, int rows, int n, float eps);
+
+/* vv_residual_add_dev contract (device.h:512): x = half_rn(float(x)+float(y)),
+ * the rounding src/cuda/conv_vae.cu:29-31 applies. Bit-exact target. */
+int vvo_residual_add_f16(uint16_t* x, const uint16_t* y, size_t n);
+
+/* Fused residual-add + RMSNorm = vv_residual_add_dev followed by
+ * vv_rmsnorm_dev on the rounded sum (decoder.c:950-960). residual is updated
+ * in place (bit-exact target); normed as for vvo_rmsnorm_f16. */
+int vvo_add_rmsnorm_f16(uint16_t* residual, const uint16_t* x,
+                        const uint16_t* w, float* normed_ref,
+                        uint16_t* normed_rne, int rows, int n, float eps);
+
+/* vv_rope_dev contract (device.h:500-502); x is not modified. */
+int vvo_rope_f16(const uint16_t* x, float* out_ref, uint16_t* out_rne,
+                 int rows, int n_heads, int head_dim, int position_offset,
+                 float theta);
+
+/* vv_swiglu_dev contract (device.h:504-506). */
+int vvo_swiglu_f16(const uint16_t* gate, const uint16_t* up, float* out_ref,
+                   uint16_t* out_rne, size_t n);
+
+/* vv_swiglu_fused_dev contract (device.h:508-510): gate_up is [rows, 2*inter],
+ * gate in columns [0,inter), up in [inter, 2*inter). */
+int vvo_swiglu_fused_f16(const uint16_t* gate_up, float* out_ref,
+                         uint16_t* out_rne, int rows, int inter);
+
+/* vv_embedding_dev contract (device.h:486-488): FP16 bits copied. */
+int vvo_embedding_f16(const uint16_t* table, const int32_t* ids,
+                      uint16_t* out, int rows, int hidden);
+
+/* vv_bias_add_dev contract (device.h:513-514; src/cuda/conv_vae.cu:54-67):
+ * out[m,n] = half_rn(float(out[m,n]) + float(bias[n])). Bit-exact target. */
+int vvo_bias_add_f16(uint16_t* out, const uint16_t* bias, int M, int N);
+
+/* ── seeded inputs (the same bytes go to the oracle and to the GPU) ────── */
+
+/* N(mean, std) rounded to FP16 (RNE). Counter-based: element i depends only
+ * on (seed, i), so any slice can be regenerated. */
+void vvo_fill_normal_f16(uint16_t* out, size_t n, uint64_t seed,
+                         double mean, double std);
+void vvo_fill_normal_f32(float* out, size_t n, uint64_t seed,
+                         double mean, double std);
+/* uniform int32 on [0, bound) */
+void vvo_fill_ids(int32_t* out, size_t n, uint64_t seed, int32_t bound);
+
+/* OpenMP threads the *_f32 kernels will use (1 if built without OpenMP). */
+int vvo_threads(void);
+void vvo_set_threads(int n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VV_ORACLE_H */
