@@ -1,0 +1,306 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused layer kernels at the Qwen2-7B prefill shape.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only NAME]
+
+One "step" is one pass of the hot path over a T = 14449 token prompt:
+  gather+norm   vv_embedding_rmsnorm_dev   table [152064,3584] -> hidden, normed
+  add+norm      vv_add_rmsnorm_dev         residual, x [T,3584] -> residual, normed
+  rope          vv_rope_qk_dev             Q [T,28,128], K [T,4,128] in place
+  swiglu        vv_swiglu_dev              gate, up [T,18944] -> out
+All inputs are resident in HBM before the timed region. Buffers rotate over
+several distinct sets so that no launch finds its data in the last-level cache
+left by the previous one. Reported:
+  value      algorithmic bytes of one step / wall time of one step (GB/s), K steps
+             timed between device synchronisations;
+  kernels    per kernel: HIP-event time of back-to-back launches, GB/s on the
+             algorithmic byte count, rows/s, fraction of the 8 TB/s HBM peak;
+  roofline   the dominant kernel (SwiGLU: 63 % of the step's bytes);
+  cpu_baseline  the reference's CPU kernels (or our restatement of them) on the
+             host's cores, on the same T = 14449 step (about 10 s including input generation).
+Prints one JSON line on stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+T_FULL, H, I_FF, V, NQ, NK, HD = 14449, 3584, 18944, 152064, 28, 4, 128
+EPS, THETA = 1e-6, 1e6
+HBM_PEAK_GBPS = 8000.0           # MI355X HBM3E, published peak
+CPU_SAMPLE_ROWS = T_FULL         # the whole step: ~0.3 s per pass on 8-16 host cores
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(T: int) -> dict:
+    """FP16 I/O bytes each kernel must move, per launch."""
+    return {
+        "gather+norm": 6 * T * H + 4 * T + 2 * H,      # read row + id, write hidden + normed
+        "add+norm": 8 * T * H + 2 * H,                 # read x, residual; write residual, normed
+        "rope": 4 * T * (NQ + NK) * HD,                # read + write Q and K
+        "swiglu": 6 * T * I_FF,                        # read gate, up; write out
+    }
+
+
+class Workload:
+    """Device buffers for `nsets` rotating copies of the step's tensors."""
+
+    def __init__(self, torch, dev, T: int, nsets: int):
+        self.torch, self.dev, self.T, self.nsets = torch, dev, T, nsets
+        gen = torch.Generator(device="cuda").manual_seed(0)
+
+        def randn(*shape, std=1.0, mean=0.0):
+            return (torch.randn(*shape, generator=gen, device="cuda") * std + mean).half()
+
+        self.table = randn(V, H, std=0.02)
+        self.weight = randn(H, std=0.1, mean=1.0)
+        self.sets = []
+        for s in range(nsets):
+            d = {
+                "ids": torch.randint(0, V, (T,), generator=gen, device="cuda", dtype=torch.int32),
+                "hidden": torch.empty(T, H, dtype=torch.float16, device="cuda"),
+                "normed": torch.empty(T, H, dtype=torch.float16, device="cuda"),
+                "residual": randn(T, H),
+                "x": randn(T, H),
+                "q": randn(T, NQ, HD),
+                "k": randn(T, NK, HD),
+                "gate": randn(T, I_FF, std=2.0),
+                "up": randn(T, I_FF, std=2.0),
+                "out": torch.empty(T, I_FF, dtype=torch.float16, device="cuda"),
+            }
+            self.sets.append(d)
+        torch.cuda.synchronize()
+
+    def launch(self, name: str, i: int, st: int) -> None:
+        d, dev, T = self.sets[i % self.nsets], self.dev, self.T
+        if name == "gather+norm":
+            rc = dev.vv_embedding_rmsnorm_dev(self.table.data_ptr(), d["ids"].data_ptr(),
+                                              self.weight.data_ptr(), d["hidden"].data_ptr(),
+                                              d["normed"].data_ptr(), T, H, EPS, st)
+        elif name == "add+norm":
+            rc = dev.vv_add_rmsnorm_dev(d["residual"].data_ptr(), d["x"].data_ptr(),
+                                        self.weight.data_ptr(), d["normed"].data_ptr(),
+                                        T, H, EPS, st)
+        elif name == "rope":
+            rc = dev.vv_rope_qk_dev(d["q"].data_ptr(), d["k"].data_ptr(), T, NQ, NK, HD, 0, None,
+                                    THETA, st)
+        elif name == "swiglu":
+            rc = dev.vv_swiglu_dev(d["gate"].data_ptr(), d["up"].data_ptr(), d["out"].data_ptr(),
+                                   T * I_FF, st)
+        else:
+            raise KeyError(name)
+        if rc != 0:
+            raise RuntimeError(f"{name} returned status {rc}")
+
+
+KERNELS = ["gather+norm", "add+norm", "rope", "swiglu"]
+
+
+def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: int):
+    """HIP events on the launch stream around `launches` back-to-back launches;
+    returns (best, median) seconds per launch over `reps` repetitions."""
+    per = []
+    for _ in range(reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(launches):
+            wl.launch(name, i, st)
+        e1.record()
+        e1.synchronize()
+        per.append(e0.elapsed_time(e1) * 1e-3 / launches)
+    per.sort()
+    return per[0], per[len(per) // 2]
+
+
+def cpu_baseline(rows: int) -> dict:
+    """The CPU path of the same step on `rows` rows: warm-up, then best of five
+    (bench/benchmark.c:197-211). FP32 activations, so its byte count is its own."""
+    import ctypes as C
+
+    import numpy as np
+
+    import oracle
+
+    f32p, i32p = C.POINTER(C.c_float), C.POINTER(C.c_int32)
+    use_ref = oracle.ref is not None
+    if use_ref:
+        threads = oracle.ref.vv_cpu_threads()     # one per physical core, pinned; OMP_NUM_THREADS wins
+        simd = oracle.ref.vv_cpu_simd_name().decode()
+    else:
+        threads, simd = oracle.lib.vvo_threads(), "scalar"
+    vocab = 8192                                   # a table slice: the gather cost is per row
+    table = oracle.normal_f16((vocab, H), 1, std=0.02)
+    ids = oracle.ids(rows, 2, vocab)
+    w = oracle.normal_f16((H,), 3, mean=1.0, std=0.1)
+    hidden = np.empty((rows, H), np.float32)
+    normed = np.empty((rows, H), np.float32)
+    resid = oracle.normal_f32((rows, H), 4)
+    x = oracle.normal_f32((rows, H), 5)
+    q = oracle.normal_f32((rows, NQ, HD), 6)
+    k = oracle.normal_f32((rows, NK, HD), 7)
+    gate = oracle.normal_f32((rows, I_FF), 8, std=2.0)
+    up = oracle.normal_f32((rows, I_FF), 9, std=2.0)
+    out = np.empty((rows, I_FF), np.float32)
+
+    def p(a, ty=f32p):
+        return a.ctypes.data_as(ty)
+
+    if use_ref:
+        r = oracle.ref
+        steps = {
+            "gather+norm": lambda: (r.vv_embedding_cpu(table.ctypes.data, p(ids, i32p), p(hidden), rows, H),
+                                    r.vv_rmsnorm_cpu(p(hidden), w.ctypes.data, p(normed), rows, H, C.c_float(EPS))),
+            "add+norm": lambda: (r.vv_residual_add_cpu(p(resid), p(x), rows * H),
+                                 r.vv_rmsnorm_cpu(p(resid), w.ctypes.data, p(normed), rows, H, C.c_float(EPS))),
+            "rope": lambda: (r.vv_rope_cpu(p(q), rows, NQ, HD, 0, C.c_float(THETA)),
+                             r.vv_rope_cpu(p(k), rows, NK, HD, 0, C.c_float(THETA))),
+            "swiglu": lambda: (r.vv_swiglu_cpu(p(gate), p(up), p(out), rows * I_FF),),
+        }
+    else:
+        u16p = C.POINTER(C.c_uint16)
+        o = oracle.lib
+        steps = {
+            "gather+norm": lambda: (o.vvo_embedding_f32(p(table, u16p), p(ids, i32p), p(hidden), rows, H),
+                                    o.vvo_rmsnorm_f32(p(hidden), p(w, u16p), p(normed), rows, H, EPS)),
+            "add+norm": lambda: (o.vvo_residual_add_f32(p(resid), p(x), rows * H),
+                                 o.vvo_rmsnorm_f32(p(resid), p(w, u16p), p(normed), rows, H, EPS)),
+            "rope": lambda: (o.vvo_rope_f32(p(q), rows, NQ, HD, 0, THETA),
+                             o.vvo_rope_f32(p(k), rows, NK, HD, 0, THETA)),
+            "swiglu": lambda: (o.vvo_swiglu_f32(p(gate), p(up), p(out), rows * I_FF),),
+        }
+    # the CPU path's own traffic: FP32 activations, FP16 weights/table
+    cpu_bytes = {
+        "gather+norm": rows * (4 + 2 * H) + 4 * rows * H + 8 * rows * H + 2 * H,
+        "add+norm": 12 * rows * H + 8 * rows * H + 2 * H,
+        "rope": 8 * rows * (NQ + NK) * HD,
+        "swiglu": 12 * rows * I_FF,
+    }
+    per, total = {}, 0.0
+    for name in KERNELS:
+        fn = steps[name]
+        assert all(rc == 0 for rc in fn())                  # warm-up
+        best = float("inf")
+        for _ in range(5):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        per[name] = {"ms": best * 1e3, "rows_per_s": rows / best,
+                     "GBps_own_bytes": cpu_bytes[name] / best / 1e9}
+        total += best
+        log(f"  cpu {name:12s} {best * 1e3:9.2f} ms  {rows / best:12.0f} rows/s")
+    return {
+        "value": sum(cpu_bytes.values()) / total / 1e9,
+        "unit": "GB/s (on the CPU path's own FP32 byte count)",
+        "cores": threads,
+        "kind": "reference" if use_ref else "port",
+        "simd": simd,
+        "sample": f"the same step on {rows} of {T_FULL} rows (embedding table cut to {vocab} "
+                  "rows), best of 5 after a warm-up call",
+        "rows_per_s": rows / total,
+        "ms_per_step_sample": total * 1e3,
+        "kernels": per,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--rows", type=int, default=T_FULL, help="prompt length T")
+    ap.add_argument("--sets", type=int, default=3, help="rotating buffer sets")
+    ap.add_argument("--launches", type=int, default=20, help="back-to-back launches per event pair")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--only", default=None, help="time only this kernel (profiling aid)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every op is row-independent and this build uses no "
+              "second device; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from __graft_entry__ import load_device
+
+    dev = load_device()                              # raises if the HIP library is not built
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU: there is no CPU fallback for the HIP backend")
+    torch.cuda.set_device(0)
+    T = args.rows
+    name_buf = torch.cuda.get_device_name(0)
+    log(f"device: {name_buf}; T={T}, sets={args.sets}")
+    wl = Workload(torch, dev, T, args.sets)
+    st = torch.cuda.current_stream().cuda_stream
+    bytes_per = algorithmic_bytes(T)
+    kernels = [args.only] if args.only else KERNELS
+
+    # ── whole step: W warm-up steps, then exactly K timed steps ──
+    for i in range(args.warmup):
+        for name in kernels:
+            wl.launch(name, i, st)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        for name in kernels:
+            wl.launch(name, i, st)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    step_bytes = sum(bytes_per[n] for n in kernels)
+    value = step_bytes / (wall / args.steps) / 1e9
+    log(f"step: {ms_per_step:.4f} ms, {value:.1f} GB/s over {step_bytes / 1e6:.1f} MB")
+
+    # ── per kernel, HIP events on the launch stream ──
+    per = {}
+    for name in kernels:
+        best, med = time_kernel(torch, wl, name, args.launches, 5, st)
+        per[name] = {
+            "bytes": bytes_per[name],
+            "us_median": med * 1e6, "us_best": best * 1e6,
+            "GBps": bytes_per[name] / med / 1e9,
+            "frac_of_peak": bytes_per[name] / med / 1e9 / HBM_PEAK_GBPS,
+            "rows_per_s": T / med,
+        }
+        log(f"  {name:12s} {med * 1e6:9.2f} us  {per[name]['GBps']:8.1f} GB/s  "
+            f"{100 * per[name]['frac_of_peak']:5.1f} % of peak  {T / med:12.0f} rows/s")
+
+    dominant = max(kernels, key=lambda n: bytes_per[n])
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(dominant, {}).get("hbm_bytes_per_launch")
+    result = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) for RMSNorm/RoPE/SwiGLU at T=14449",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "storage_dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"Qwen2-7B fused layer kernels, one prefill pass at T={T}: "
+                               "embedding gather+RMSNorm, residual-add+RMSNorm, RoPE(Q,K), SwiGLU",
+                   "hidden": H, "intermediate": I_FF, "vocab": V, "q_heads": NQ, "kv_heads": NK,
+                   "head_dim": HD, "rows": T, "buffer_sets": args.sets},
+        "pct_of_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "rows_per_s": T / (wall / args.steps),
+        "kernels": per,
+        "roofline": {"kernel": dominant, "bound": "hbm", "achieved": per[dominant]["GBps"],
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": per[dominant]["frac_of_peak"], "traffic": traffic},
+    }
+    if not args.no_cpu:
+        log(f"cpu baseline on {CPU_SAMPLE_ROWS} rows ...")
+        result["cpu_baseline"] = cpu_baseline(CPU_SAMPLE_ROWS)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,205 @@
+/*
+ * vibevoice_hip.h — C ABI of libvibevoice_hip.so, the MI355X (gfx950) backend
+ * for vibevoice.c's accelerator seam.
+ *
+ * Every symbol below that carries a "replaces" citation has the name,
+ * argument list and status-code behaviour of the declaration of the same name
+ * in the reference's include/vibevoice/device.h, so the C engine above that
+ * header links against this library unchanged. Symbols marked "addition" do
+ * not exist in the reference: they are the fused forms of adjacent reference
+ * calls and follow the same conventions.
+ *
+ * Conventions (device.h:16-20):
+ *   - `void* stream` is a hipStream_t; NULL is the legacy default stream;
+ *   - tensors are FP16, row-major, contiguous; pointers are device pointers;
+ *   - every op enqueues on `stream` and returns at once with VV_OK or a
+ *     negative vv_status_t; no op allocates, synchronises, throws or aborts,
+ *     and none keeps state between calls, so concurrent calls on different
+ *     streams from different host threads are safe and every op is
+ *     graph-capturable;
+ *   - a size of zero rows/elements is VV_OK with nothing launched.
+ */
+#ifndef VIBEVOICE_HIP_H
+#define VIBEVOICE_HIP_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes: the values of include/vibevoice/types.h:18-58 that this
+ * backend returns. When the reference's types.h is already included its enum
+ * is used instead. */
+#ifndef VV_TYPES_H
+typedef enum vv_status {
+    VV_OK               = 0,
+    VV_ERR_INVALID_ARG  = -1,
+    VV_ERR_NULL_PTR     = -2,
+    VV_ERR_UNSUPPORTED  = -7,
+    VV_ERR_CUDA         = -100,   /* a runtime (HIP) call failed            */
+    VV_ERR_CUDA_OOM     = -101,   /* device allocation: out of memory       */
+    VV_ERR_CUDA_LAUNCH  = -102    /* a kernel launch was rejected           */
+} vv_status_t;
+#endif
+
+/* ── Transformer layer ops: the hot path ───────────────────────────────── */
+
+/* output[r,:] = table[ids[r],:], FP16 bits copied. ids are not range-checked
+ * (as in the reference); row offsets are 64-bit.
+ * replaces device.h:486-488 (src/cuda/embedding.cu:59-74). */
+vv_status_t vv_embedding_dev(const void* table, const int32_t* ids, void* output,
+                             int seq_len, int hidden_size, void* stream);
+
+/* output = x * (1/sqrt(mean(x^2)+eps)) * weight per row, FP32 arithmetic,
+ * one FP16 rounding. input != output.
+ * replaces device.h:490-492 (src/cuda/rmsnorm.cu:82-100). */
+vv_status_t vv_rmsnorm_dev(const void* input, const void* weight, void* output,
+                           int seq_len, int hidden_size, float eps, void* stream);
+
+/* Rotate-half RoPE in place over [seq_len, n_heads, head_dim]; the first row
+ * is at position `*d_position` when d_position is non-NULL (read on the
+ * device, so a captured launch can be replayed), else at position_offset.
+ * head_dim must be even and at most 256, else VV_ERR_UNSUPPORTED.
+ * replaces device.h:500-502 (src/cuda/rope.cu:89-103). */
+vv_status_t vv_rope_dev(void* x, int seq_len, int n_heads, int head_dim,
+                        int position_offset, const int* d_position, float theta,
+                        void* stream);
+
+/* output = silu(gate) * up elementwise; output may alias gate (or up).
+ * replaces device.h:504-506 (src/cuda/swiglu.cu:79-103). */
+vv_status_t vv_swiglu_dev(const void* gate, const void* up, void* output,
+                          int n_elements, void* stream);
+
+/* The same with gate and up as the two halves of one [rows, 2*inter] buffer.
+ * replaces device.h:508-510 (declared there; no CUDA definition exists, Metal:
+ * src/metal/mtl_transformer.c:88-97). */
+vv_status_t vv_swiglu_fused_dev(const void* gate_up, void* output, int rows,
+                                int inter, void* stream);
+
+/* x = half_rn(float(x) + float(y)), in place.
+ * replaces device.h:512 (src/cuda/conv_vae.cu:37-47). */
+vv_status_t vv_residual_add_dev(void* x, const void* y, int total, void* stream);
+
+/* output[m,n] = half_rn(float(output[m,n]) + float(bias[n])), in place.
+ * replaces device.h:513-514 (src/cuda/conv_vae.cu:72-84). */
+vv_status_t vv_bias_add_dev(void* output, const void* bias, int M, int N,
+                            void* stream);
+
+/* replaces device.h:717-720 (src/cuda/conv_vae.cu:100-116). */
+vv_status_t vv_fp32_to_fp16_dev(const void* in_fp32, void* out_fp16, int n,
+                                void* stream);
+vv_status_t vv_fp16_to_fp32_dev(const void* in_fp16, void* out_fp32, int n,
+                                void* stream);
+
+/* ── Fused forms (additions) ───────────────────────────────────────────── */
+
+/* addition: vv_residual_add_dev(residual, x) followed by
+ * vv_rmsnorm_dev(residual, weight, normed) in one pass over the rows — the
+ * adjacent calls at src/inference/decoder.c:950-960 and :988 -> :810. The
+ * updated residual (bit-identical to the two-call sequence) is written back in
+ * place and the norm reads that rounded FP16 value, as the two calls would.
+ * 8*T*H bytes of traffic instead of 10*T*H. */
+vv_status_t vv_add_rmsnorm_dev(void* residual, const void* x, const void* weight,
+                               void* normed, int seq_len, int hidden_size,
+                               float eps, void* stream);
+
+/* addition: vv_rope_dev on Q [seq_len, n_q_heads, head_dim] and on
+ * K [seq_len, n_kv_heads, head_dim] in one launch (decoder.c:850-855), the
+ * cosine/sine of a position computed once and shared by all heads of both.
+ * Either of q, k may be NULL (its head count is then ignored). */
+vv_status_t vv_rope_qk_dev(void* q, void* k, int seq_len, int n_q_heads,
+                           int n_kv_heads, int head_dim, int position_offset,
+                           const int* d_position, float theta, void* stream);
+
+/* addition: vv_bias_add_dev on Q and K followed by vv_rope_qk_dev — the
+ * projection epilogue of decoder.c:825-855 (bias, then rotation) in one pass.
+ * The biased value is rounded to FP16 before it is rotated, as the two calls
+ * would. q_bias [n_q_heads*head_dim], k_bias [n_kv_heads*head_dim]; either
+ * may be NULL (no bias for that tensor). */
+vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias,
+                                const void* k_bias, int seq_len, int n_q_heads,
+                                int n_kv_heads, int head_dim, int position_offset,
+                                const int* d_position, float theta, void* stream);
+
+/* addition: vv_embedding_dev(table, ids, hidden) followed by
+ * vv_rmsnorm_dev(hidden, weight, normed): the first-layer chain
+ * src/inference/pipeline.c:2309 -> decoder.c:810. hidden is bit-exact. */
+vv_status_t vv_embedding_rmsnorm_dev(const void* table, const int32_t* ids,
+                                     const void* weight, void* hidden, void* normed,
+                                     int seq_len, int hidden_size, float eps,
+                                     void* stream);
+
+/* ── Device, memory, streams, events, graphs: the runtime half ─────────── */
+
+/* replaces device.h:39-45 (src/cuda/cuda_utils.cu:20-99). Copies with a NULL
+ * stream are synchronous; with a stream they are ordered on it. */
+vv_status_t vv_dev_alloc(void** ptr, size_t size);
+vv_status_t vv_dev_alloc_pinned(void** ptr, size_t size);
+vv_status_t vv_dev_free(void* ptr);
+vv_status_t vv_dev_free_pinned(void* ptr);
+vv_status_t vv_dev_memcpy_h2d(void* dst, const void* src, size_t size, void* stream);
+vv_status_t vv_dev_memcpy_d2h(void* dst, const void* src, size_t size, void* stream);
+vv_status_t vv_dev_memcpy_d2d(void* dst, const void* src, size_t size, void* stream);
+
+/* Copy `size` bytes to dst_base + (*d_index) * size, the index read on the
+ * device. replaces device.h:54-55 (cuda_utils.cu:131-154). */
+vv_status_t vv_dev_memcpy_d2d_at(void* dst_base, const void* src, size_t size,
+                                 const int* d_index, void* stream);
+
+/* replaces device.h:56 and :65-66 (cuda_utils.cu:418-422, :213-218). The
+ * stream-ordered form is a fill kernel, so it may be captured into a graph. */
+vv_status_t vv_dev_memset(void* ptr, int value, size_t size);
+vv_status_t vv_dev_memset_async(void* ptr, int value, size_t size, void* stream);
+
+/* replaces device.h:67-75 (cuda_utils.cu:229-271). Both kinds of stream are
+ * created at the default priority on this backend. */
+vv_status_t vv_dev_stream_create(void** stream);
+vv_status_t vv_dev_stream_create_background(void** stream);
+vv_status_t vv_dev_stream_destroy(void* stream);
+vv_status_t vv_dev_stream_sync(void* stream);
+
+/* replaces device.h:76-101 (cuda_utils.cu:276-292, :327-349, :409-412).
+ * sm_count reports compute units. */
+vv_status_t vv_dev_set_device(int device_id);
+vv_status_t vv_dev_get_device_info(int device_id, size_t* total_mem,
+                                   size_t* free_mem, int* sm_count);
+int         vv_dev_device_count(void);
+vv_status_t vv_dev_get_device_name(int device_id, char* buf, size_t buf_size);
+bool        vv_dev_host_shares_memory(int device_id);
+
+/* replaces device.h:111-121 (cuda_utils.cu:301-325). */
+vv_status_t vv_dev_memcpy_peer(void* dst, int dst_device, const void* src,
+                               int src_device, size_t size, void* stream);
+vv_status_t vv_dev_enable_peer(int device, int peer);
+
+/* replaces device.h:125-130, :872 (cuda_utils.cu:362-424). Registering
+ * existing host memory is declined with VV_ERR_UNSUPPORTED (the caller at
+ * decoder.c:289 then keeps its pageable copy path); unregister is VV_OK. */
+vv_status_t vv_dev_event_create(void** ev);
+vv_status_t vv_dev_event_destroy(void* ev);
+vv_status_t vv_dev_event_record(void* ev, void* stream);
+vv_status_t vv_dev_event_sync(void* ev);
+vv_status_t vv_dev_stream_wait_event(void* stream, void* ev);
+vv_status_t vv_dev_host_register(void* p, size_t n);
+vv_status_t vv_dev_host_unregister(void* p);
+
+/* replaces device.h:133. Returns "HIP". */
+const char* vv_dev_backend_name(void);
+
+/* replaces device.h:152-160 (cuda_utils.cu:158-204). */
+vv_status_t vv_dev_graph_begin(void* stream);
+vv_status_t vv_dev_graph_end(void* stream, void** graph_exec);
+vv_status_t vv_dev_graph_launch(void* graph_exec, void* stream);
+void        vv_dev_graph_destroy(void* graph_exec);
+
+/* *dst = *src + delta on the stream. replaces device.h:163
+ * (cuda_utils.cu:126-130). */
+vv_status_t vv_pos_add_dev(int* dst, const int* src, int delta, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VIBEVOICE_HIP_H */

@@ -1,0 +1,108 @@
+"""CPU checks of the drop-in boundary: the library loads, exports exactly the
+symbols include/vibevoice_hip.h declares, and the argument checks that need no
+GPU behave as the reference's do (NULL -> VV_ERR_NULL_PTR, empty -> VV_OK)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from __graft_entry__ import ROOT, load_device
+
+dev = load_device()
+HEADER = os.path.join(ROOT, "include", "vibevoice_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_python_and_library_agree():
+    declared = declared_symbols()
+    assert len(declared) >= 47
+    assert sorted(dev.SIGNATURES) == declared
+    out = subprocess.check_output(["nm", "-D", "--defined-only", dev.LIB_PATH], text=True)
+    exported = sorted(l.split()[-1] for l in out.splitlines() if " T " in l and " vv_" in l)
+    assert exported == declared
+
+
+def test_library_is_gfx950_only_and_does_not_link_the_oracle():
+    out = subprocess.check_output(["ldd", dev.LIB_PATH], text=True)
+    assert "libamdhip64" in out
+    assert "oracle" not in out and "vv_ref" not in out and "gomp" not in out
+    blob = open(dev.LIB_PATH, "rb").read()
+    assert b"gfx950" in blob
+    for other in (b"gfx942", b"gfx90a", b"sm_80"):
+        assert other not in blob
+
+
+def test_backend_name():
+    assert dev.vv_dev_backend_name() == b"HIP"
+    assert dev.vv_dev_host_shares_memory(0) is False
+
+
+P = 0x1000   # a non-null, 16-byte aligned stand-in; never dereferenced by these calls
+
+
+@pytest.mark.parametrize("call", [
+    lambda: dev.vv_embedding_dev(None, P, P, 4, 3584, None),
+    lambda: dev.vv_embedding_dev(P, None, P, 4, 3584, None),
+    lambda: dev.vv_embedding_dev(P, P, None, 4, 3584, None),
+    lambda: dev.vv_rmsnorm_dev(None, P, P, 4, 3584, 1e-6, None),
+    lambda: dev.vv_rmsnorm_dev(P, None, P, 4, 3584, 1e-6, None),
+    lambda: dev.vv_rmsnorm_dev(P, P, None, 4, 3584, 1e-6, None),
+    lambda: dev.vv_rope_dev(None, 4, 28, 128, 0, None, 1e6, None),
+    lambda: dev.vv_rope_qk_dev(None, None, 4, 28, 4, 128, 0, None, 1e6, None),
+    lambda: dev.vv_swiglu_dev(None, P, P, 64, None),
+    lambda: dev.vv_swiglu_dev(P, None, P, 64, None),
+    lambda: dev.vv_swiglu_dev(P, P, None, 64, None),
+    lambda: dev.vv_swiglu_fused_dev(None, P, 2, 64, None),
+    lambda: dev.vv_residual_add_dev(None, P, 64, None),
+    lambda: dev.vv_residual_add_dev(P, None, 64, None),
+    lambda: dev.vv_bias_add_dev(None, P, 2, 64, None),
+    lambda: dev.vv_add_rmsnorm_dev(None, P, P, P, 4, 3584, 1e-6, None),
+    lambda: dev.vv_add_rmsnorm_dev(P, P, P, None, 4, 3584, 1e-6, None),
+    lambda: dev.vv_embedding_rmsnorm_dev(P, None, P, P, P, 4, 3584, 1e-6, None),
+    lambda: dev.vv_pos_add_dev(None, P, 1, None),
+    lambda: dev.vv_dev_memcpy_d2d_at(P, P, 16, None, None),
+    lambda: dev.vv_dev_alloc(None, 16),
+    lambda: dev.vv_dev_memset_async(None, 0, 16, None),
+    lambda: dev.vv_dev_event_record(None, None),
+    lambda: dev.vv_dev_graph_launch(None, None),
+])
+def test_null_pointer_is_an_error_not_a_crash(call):
+    assert call() == dev.VV_ERR_NULL_PTR
+
+
+@pytest.mark.parametrize("call", [
+    lambda: dev.vv_embedding_dev(P, P, P, 0, 3584, None),
+    lambda: dev.vv_rmsnorm_dev(P, P, P, 0, 3584, 1e-6, None),
+    lambda: dev.vv_rmsnorm_dev(P, P, P, -3, 3584, 1e-6, None),
+    lambda: dev.vv_rope_dev(P, 0, 28, 128, 0, None, 1e6, None),
+    lambda: dev.vv_rope_dev(P, 4, 0, 128, 0, None, 1e6, None),
+    lambda: dev.vv_swiglu_dev(P, P, P, 0, None),
+    lambda: dev.vv_swiglu_fused_dev(P, P, 0, 64, None),
+    lambda: dev.vv_residual_add_dev(P, P, 0, None),
+    lambda: dev.vv_bias_add_dev(P, P, 0, 64, None),
+    lambda: dev.vv_add_rmsnorm_dev(P, P, P, P, 0, 3584, 1e-6, None),
+    lambda: dev.vv_embedding_rmsnorm_dev(P, P, P, P, P, 0, 3584, 1e-6, None),
+    lambda: dev.vv_dev_memcpy_d2d_at(P, P, 0, P, None),
+    lambda: dev.vv_dev_free(None),
+    lambda: dev.vv_dev_free_pinned(None),
+    lambda: dev.vv_dev_stream_destroy(None),
+    lambda: dev.vv_dev_event_destroy(None),
+    lambda: dev.vv_dev_host_unregister(None),
+])
+def test_empty_work_is_ok_and_launches_nothing(call):
+    assert call() == dev.VV_OK
+
+
+def test_declined_arguments():
+    assert dev.vv_rope_dev(P, 4, 2, 127, 0, None, 1e4, None) == dev.VV_ERR_UNSUPPORTED
+    assert dev.vv_rope_dev(P, 4, 2, 1024, 0, None, 1e4, None) == dev.VV_ERR_UNSUPPORTED
+    assert dev.vv_dev_graph_begin(None) == dev.VV_ERR_INVALID_ARG
+    assert dev.vv_dev_host_register(P, 4096) == dev.VV_ERR_UNSUPPORTED
+    assert dev.vv_dev_host_register(None, 4096) == dev.VV_ERR_NULL_PTR
+    dev.vv_dev_graph_destroy(None)      # no-op, must not crash

@@ -1,0 +1,248 @@
+// Rotary position embedding (rotate-half pairing) on Q and K, in place.
+//
+// What is shared and what is streamed:
+//   - cos/sin depend only on (position, pair index), not on the head. A
+//     workgroup owns kPosPerBlock consecutive positions; its 256 threads first
+//     compute those positions' head_dim/2 cosines and sines once into LDS
+//     (LDS is justified here: every head of Q and K at that position reuses
+//     the same 2 x 64 values), then stream the heads through.
+//   - head_dim = 128 is 16 chunks; the pair (d, d+64) is chunk c with chunk
+//     c+8, so a lane that loads chunks c and c+8 of one head rotates 8 pairs
+//     without talking to any other lane. 28 Q heads + 4 K heads = 256 such
+//     lane tasks per position: one per thread of the workgroup.
+//   - frequencies: inv_freq[i] = powf(theta, -2i/head_dim) is computed on the
+//     HOST with the C library's powf and passed by value in the kernel
+//     arguments. The angle (float)pos * inv_freq reaches ~1e4 rad at long
+//     prompts, where one FP32 ulp of the angle is ~1e-3 rad, so a frequency
+//     that differs by one ulp from the CPU path's would be visible; the host
+//     value is bit-identical to what the CPU kernels compute. The device then
+//     forms the angle with one FP32 multiply and calls the full-range sincosf
+//     (never the fast intrinsics, whose error grows with |angle|).
+#include <math.h>
+
+#include "vv_common.hpp"
+
+namespace vv {
+namespace {
+
+constexpr int kMaxPairs = 128;      // head_dim <= 256
+constexpr int kPosPerBlock = 4;     // positions per workgroup in the head_dim-128 kernel
+
+struct FreqTable {
+    float f[kMaxPairs];
+};
+
+struct RopeArgs {
+    h16* q;                 // [rows, nq, head_dim] or nullptr
+    h16* k;                 // [rows, nk, head_dim] or nullptr
+    const h16* q_bias;      // [nq * head_dim] or nullptr
+    const h16* k_bias;      // [nk * head_dim] or nullptr
+    const int* d_position;  // device int with the first row's position, or nullptr
+    int rows, nq, nk, head_dim, position_offset;
+};
+
+__device__ __forceinline__ Chunk add_bias(const Chunk& v, const Chunk& b) {
+    const f32x8 x = unpack(v), y = unpack(b);
+    f32x8 r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = x[i] + y[i];
+    return pack(r);      // rounded to FP16 before the rotation, as bias_add then rope would
+}
+
+// The rotation itself, in the CPU path's arithmetic: four products, one
+// subtraction, one addition, none of them fused, so that the only difference
+// from the CPU result is the last bits of sin/cos.
+struct Pair {
+    float lo, hi;
+};
+__device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
+#pragma clang fp contract(off)
+    const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+    Pair r;
+    r.lo = ac - bs;
+    r.hi = as + bc;
+    return r;
+}
+
+// head_dim == 128, 16-byte aligned tensors.
+template <bool kBias>
+__global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
+    __shared__ __attribute__((aligned(16))) float cs_cos[kPosPerBlock][64];
+    __shared__ __attribute__((aligned(16))) float cs_sin[kPosPerBlock][64];
+
+    const int first = a.d_position ? *a.d_position : a.position_offset;
+    const int row0 = (int)blockIdx.x * kPosPerBlock;
+
+    {   // phase 1: thread t -> (position t / 64, pair t % 64)
+        const int p = (int)threadIdx.x >> 6, i = (int)threadIdx.x & 63;
+        const int pos = first + row0 + p;
+        const float ang = (float)pos * freqs.f[i];
+        float s, c;
+        sincosf(ang, &s, &c);
+        cs_cos[p][i] = c;
+        cs_sin[p][i] = s;
+    }
+    __syncthreads();
+
+    const int heads = a.nq + a.nk;
+    const int tasks = heads * 8;                 // (head, chunk-pair) per position
+    const int rows_here = min(kPosPerBlock, a.rows - row0);
+
+    for (int p = 0; p < rows_here; ++p) {
+        const size_t row = (size_t)(row0 + p);
+        for (int t = (int)threadIdx.x; t < tasks; t += kBlock) {
+            const int head = t >> 3, c = t & 7;
+            h16* base;
+            const h16* bias = nullptr;
+            if (head < a.nq) {
+                base = a.q + (row * (size_t)a.nq + (size_t)head) * 128u;
+                if (kBias && a.q_bias) bias = a.q_bias + (size_t)head * 128u;
+            } else {
+                base = a.k + (row * (size_t)a.nk + (size_t)(head - a.nq)) * 128u;
+                if (kBias && a.k_bias) bias = a.k_bias + (size_t)(head - a.nq) * 128u;
+            }
+            Chunk* lo_p = reinterpret_cast<Chunk*>(base) + c;
+            Chunk* hi_p = lo_p + 8;
+            Chunk lo = load_chunk(lo_p), hi = load_chunk(hi_p);
+            if (kBias && bias) {
+                const Chunk* bp = reinterpret_cast<const Chunk*>(bias) + c;
+                lo = add_bias(lo, load_chunk(bp));
+                hi = add_bias(hi, load_chunk(bp + 8));
+            }
+            const f32x8 x0 = unpack(lo), x1 = unpack(hi);
+            const f32x8 cv = *reinterpret_cast<const f32x8*>(&cs_cos[p][c * 8]);
+            const f32x8 sv = *reinterpret_cast<const f32x8*>(&cs_sin[p][c * 8]);
+            f32x8 y0, y1;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const Pair r = rotate(x0[i], x1[i], cv[i], sv[i]);
+                y0[i] = r.lo;
+                y1[i] = r.hi;
+            }
+            store_chunk(lo_p, pack(y0));
+            store_chunk(hi_p, pack(y1));
+        }
+    }
+}
+
+// Any even head_dim <= 256, any alignment: one workgroup per position,
+// 2-byte accesses.
+__global__ __launch_bounds__(kBlock) void rope_generic(RopeArgs a, FreqTable freqs) {
+    __shared__ float cs_cos[kMaxPairs];
+    __shared__ float cs_sin[kMaxPairs];
+    const int half = a.head_dim / 2;
+    const int first = a.d_position ? *a.d_position : a.position_offset;
+    const size_t row = blockIdx.x;
+    const int pos = first + (int)row;
+    for (int i = (int)threadIdx.x; i < half; i += kBlock) {
+        const float ang = (float)pos * freqs.f[i];
+        float s, c;
+        sincosf(ang, &s, &c);
+        cs_cos[i] = c;
+        cs_sin[i] = s;
+    }
+    __syncthreads();
+    const int heads = a.nq + a.nk;
+    const int tasks = heads * half;
+    for (int t = (int)threadIdx.x; t < tasks; t += kBlock) {
+        const int head = t / half, i = t - head * half;
+        h16* v;
+        const h16* bias = nullptr;
+        if (head < a.nq) {
+            v = a.q + (row * (size_t)a.nq + (size_t)head) * (size_t)a.head_dim;
+            if (a.q_bias) bias = a.q_bias + (size_t)head * (size_t)a.head_dim;
+        } else {
+            v = a.k + (row * (size_t)a.nk + (size_t)(head - a.nq)) * (size_t)a.head_dim;
+            if (a.k_bias) bias = a.k_bias + (size_t)(head - a.nq) * (size_t)a.head_dim;
+        }
+        h16 h0 = v[i], h1 = v[i + half];
+        if (bias) {
+            h0 = (h16)((float)h0 + (float)bias[i]);
+            h1 = (h16)((float)h1 + (float)bias[i + half]);
+        }
+        const float x0 = (float)h0, x1 = (float)h1;
+        const float c = cs_cos[i], s = cs_sin[i];
+        const Pair r = rotate(x0, x1, c, s);
+        v[i] = (h16)r.lo;
+        v[i + half] = (h16)r.hi;
+    }
+}
+
+// The table depends only on (theta, head_dim); each host thread remembers the
+// last one it built (thread-local, so concurrent callers never share state).
+const FreqTable& host_freqs(float theta, int head_dim) {
+    thread_local FreqTable table;
+    thread_local float cached_theta = 0.0f;
+    thread_local int cached_dim = 0;
+    if (cached_dim != head_dim || cached_theta != theta) {
+        const int half = head_dim / 2;
+        for (int i = 0; i < kMaxPairs; ++i)
+            table.f[i] = i < half ? powf(theta, -2.0f * (float)i / (float)head_dim) : 0.0f;
+        cached_theta = theta;
+        cached_dim = head_dim;
+    }
+    return table;
+}
+
+vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias, int rows,
+                        int nq, int nk, int head_dim, int position_offset,
+                        const int* d_position, float theta, hipStream_t st) {
+    if (!q) nq = 0;
+    if (!k) nk = 0;
+    if (nq < 0 || nk < 0) return VV_ERR_INVALID_ARG;
+    if (rows <= 0 || nq + nk == 0 || head_dim <= 0) return VV_OK;
+    if ((head_dim & 1) || head_dim > 2 * kMaxPairs) return VV_ERR_UNSUPPORTED;
+
+    RopeArgs a;
+    a.q = nq ? static_cast<h16*>(q) : nullptr;
+    a.k = nk ? static_cast<h16*>(k) : nullptr;
+    a.q_bias = nq ? static_cast<const h16*>(q_bias) : nullptr;
+    a.k_bias = nk ? static_cast<const h16*>(k_bias) : nullptr;
+    a.d_position = d_position;
+    a.rows = rows; a.nq = nq; a.nk = nk; a.head_dim = head_dim;
+    a.position_offset = position_offset;
+    const FreqTable& freqs = host_freqs(theta, head_dim);
+    const bool has_bias = a.q_bias || a.k_bias;
+
+    const bool fast = head_dim == 128 && (!a.q || aligned16(a.q)) && (!a.k || aligned16(a.k)) &&
+                      (!a.q_bias || aligned16(a.q_bias)) && (!a.k_bias || aligned16(a.k_bias));
+    if (fast) {
+        const dim3 grid((unsigned)((rows + kPosPerBlock - 1) / kPosPerBlock));
+        if (has_bias) rope128<true><<<grid, kBlock, 0, st>>>(a, freqs);
+        else          rope128<false><<<grid, kBlock, 0, st>>>(a, freqs);
+    } else {
+        rope_generic<<<dim3((unsigned)rows), kBlock, 0, st>>>(a, freqs);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_rope_dev(void* x, int seq_len, int n_heads, int head_dim, int position_offset,
+                        const int* d_position, float theta, void* stream) {
+    if (!x) return VV_ERR_NULL_PTR;
+    return vv::launch_rope(x, nullptr, nullptr, nullptr, seq_len, n_heads, 0, head_dim,
+                           position_offset, d_position, theta, vv::as_stream(stream));
+}
+
+vv_status_t vv_rope_qk_dev(void* q, void* k, int seq_len, int n_q_heads, int n_kv_heads,
+                           int head_dim, int position_offset, const int* d_position, float theta,
+                           void* stream) {
+    if (!q && !k) return VV_ERR_NULL_PTR;
+    return vv::launch_rope(q, k, nullptr, nullptr, seq_len, n_q_heads, n_kv_heads, head_dim,
+                           position_offset, d_position, theta, vv::as_stream(stream));
+}
+
+vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias, const void* k_bias,
+                                int seq_len, int n_q_heads, int n_kv_heads, int head_dim,
+                                int position_offset, const int* d_position, float theta,
+                                void* stream) {
+    if (!q && !k) return VV_ERR_NULL_PTR;
+    return vv::launch_rope(q, k, q_bias, k_bias, seq_len, n_q_heads, n_kv_heads, head_dim,
+                           position_offset, d_position, theta, vv::as_stream(stream));
+}
+
+}  // extern "C"

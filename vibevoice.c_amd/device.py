@@ -1,0 +1,98 @@
+"""ctypes view of libvibevoice_hip.so, one Python callable per C symbol.
+
+Names, argument order and status codes are those of the C ABI
+(include/vibevoice_hip.h, which mirrors the reference's
+include/vibevoice/device.h): every function takes raw device addresses
+(Python ints, e.g. ``tensor.data_ptr()``), a ``stream`` handle (0 = default
+stream) and returns the ``vv_status_t`` integer. Nothing is converted, copied
+or computed on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+VV_OK = 0
+VV_ERR_INVALID_ARG = -1
+VV_ERR_NULL_PTR = -2
+VV_ERR_UNSUPPORTED = -7
+VV_ERR_CUDA = -100
+VV_ERR_CUDA_OOM = -101
+VV_ERR_CUDA_LAUNCH = -102
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
+                        "libvibevoice_hip.so")
+
+_vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+
+# symbol -> (restype, argtypes); the complete export list of include/vibevoice_hip.h
+SIGNATURES = {
+    "vv_embedding_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "vv_rmsnorm_dev": (_i, [_vp, _vp, _vp, _i, _i, _f, _vp]),
+    "vv_rope_dev": (_i, [_vp, _i, _i, _i, _i, _vp, _f, _vp]),
+    "vv_swiglu_dev": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "vv_swiglu_fused_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vv_residual_add_dev": (_i, [_vp, _vp, _i, _vp]),
+    "vv_bias_add_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vv_fp32_to_fp16_dev": (_i, [_vp, _vp, _i, _vp]),
+    "vv_fp16_to_fp32_dev": (_i, [_vp, _vp, _i, _vp]),
+    "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
+    "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
+    "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
+    "vv_embedding_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
+    "vv_dev_alloc": (_i, [C.POINTER(_vp), _sz]),
+    "vv_dev_alloc_pinned": (_i, [C.POINTER(_vp), _sz]),
+    "vv_dev_free": (_i, [_vp]),
+    "vv_dev_free_pinned": (_i, [_vp]),
+    "vv_dev_memcpy_h2d": (_i, [_vp, _vp, _sz, _vp]),
+    "vv_dev_memcpy_d2h": (_i, [_vp, _vp, _sz, _vp]),
+    "vv_dev_memcpy_d2d": (_i, [_vp, _vp, _sz, _vp]),
+    "vv_dev_memcpy_d2d_at": (_i, [_vp, _vp, _sz, _vp, _vp]),
+    "vv_dev_memset": (_i, [_vp, _i, _sz]),
+    "vv_dev_memset_async": (_i, [_vp, _i, _sz, _vp]),
+    "vv_dev_stream_create": (_i, [C.POINTER(_vp)]),
+    "vv_dev_stream_create_background": (_i, [C.POINTER(_vp)]),
+    "vv_dev_stream_destroy": (_i, [_vp]),
+    "vv_dev_stream_sync": (_i, [_vp]),
+    "vv_dev_set_device": (_i, [_i]),
+    "vv_dev_get_device_info": (_i, [_i, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_i)]),
+    "vv_dev_device_count": (_i, []),
+    "vv_dev_get_device_name": (_i, [_i, C.c_char_p, _sz]),
+    "vv_dev_host_shares_memory": (C.c_bool, [_i]),
+    "vv_dev_memcpy_peer": (_i, [_vp, _i, _vp, _i, _sz, _vp]),
+    "vv_dev_enable_peer": (_i, [_i, _i]),
+    "vv_dev_event_create": (_i, [C.POINTER(_vp)]),
+    "vv_dev_event_destroy": (_i, [_vp]),
+    "vv_dev_event_record": (_i, [_vp, _vp]),
+    "vv_dev_event_sync": (_i, [_vp]),
+    "vv_dev_stream_wait_event": (_i, [_vp, _vp]),
+    "vv_dev_host_register": (_i, [_vp, _sz]),
+    "vv_dev_host_unregister": (_i, [_vp]),
+    "vv_dev_backend_name": (C.c_char_p, []),
+    "vv_dev_graph_begin": (_i, [_vp]),
+    "vv_dev_graph_end": (_i, [_vp, C.POINTER(_vp)]),
+    "vv_dev_graph_launch": (_i, [_vp, _vp]),
+    "vv_dev_graph_destroy": (None, [_vp]),
+    "vv_pos_add_dev": (_i, [_vp, _vp, _i, _vp]),
+}
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python vibevoice.c_amd/build.py` "
+            "(there is no CPU fallback for the HIP backend)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the ABI lost a symbol
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+# module-level callables with the C names
+for _name in SIGNATURES:
+    globals()[_name] = getattr(lib, _name)
+del _name
