@@ -39,11 +39,11 @@ __device__ __forceinline__ Chunk apply2(const Chunk& a, const Chunk& b) {
 
 template <int kOp>
 __device__ __forceinline__ h16 apply2(h16 a, h16 b) {
-    return (kOp == kSwiglu) ? (h16)swiglu1((float)a, (float)b) : (h16)((float)a + (float)b);
+    return to_half((kOp == kSwiglu) ? swiglu1((float)a, (float)b) : ((float)a + (float)b));
 }
 
 // out[i] = op(a[i], b[i]) over nchunks chunks, then the (< 8) trailing halves.
-template <int kOp>
+template <int kOp, bool kStream>
 __global__ __launch_bounds__(kBlock) void binary_chunks(const Chunk* a, const Chunk* b,
                                                         Chunk* out, size_t nchunks,
                                                         int tail_halves) {
@@ -52,12 +52,12 @@ __global__ __launch_bounds__(kBlock) void binary_chunks(const Chunk* a, const Ch
     if (base + (size_t)(kUnroll - 1) * kBlock < nchunks) {
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            va[j] = load_chunk(a + base + (size_t)j * kBlock);
-            vb[j] = load_chunk(b + base + (size_t)j * kBlock);
+            va[j] = load_chunk_as<kStream>(a + base + (size_t)j * kBlock);
+            vb[j] = load_chunk_as<kStream>(b + base + (size_t)j * kBlock);
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j)
-            store_chunk(out + base + (size_t)j * kBlock, apply2<kOp>(va[j], vb[j]));
+            store_chunk_as<kStream>(out + base + (size_t)j * kBlock, apply2<kOp>(va[j], vb[j]));
     } else {
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
@@ -92,9 +92,14 @@ vv_status_t launch_binary(const void* a, const void* b, void* out, size_t n, hip
         const size_t nchunks = n / 8;
         const int tail = (int)(n % 8);
         const size_t blocks = nchunks ? (nchunks + kChunksPerBlock - 1) / kChunksPerBlock : 1;
-        binary_chunks<kOp><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
-            static_cast<const Chunk*>(a), static_cast<const Chunk*>(b), static_cast<Chunk*>(out),
-            nchunks, tail);
+        if (use_streaming(3u * n * 2u))
+            binary_chunks<kOp, true><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
+                static_cast<const Chunk*>(a), static_cast<const Chunk*>(b),
+                static_cast<Chunk*>(out), nchunks, tail);
+        else
+            binary_chunks<kOp, false><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
+                static_cast<const Chunk*>(a), static_cast<const Chunk*>(b),
+                static_cast<Chunk*>(out), nchunks, tail);
     } else {
         const size_t blocks = (n + kBlock - 1) / kBlock;
         binary_halves<kOp><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
@@ -158,13 +163,13 @@ __global__ __launch_bounds__(kBlock) void bias_add_chunks(Chunk* out, const Chun
 __global__ __launch_bounds__(kBlock) void bias_add_halves(h16* out, const h16* __restrict__ bias,
                                                           size_t total, int n) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < total) out[i] = (h16)((float)out[i] + (float)bias[i % (size_t)n]);
+    if (i < total) out[i] = to_half((float)out[i] + (float)bias[i % (size_t)n]);
 }
 
 __global__ __launch_bounds__(kBlock) void f32_to_f16(const float* __restrict__ in,
                                                      h16* __restrict__ out, size_t n) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) out[i] = (h16)in[i];
+    if (i < n) out[i] = to_half(in[i]);
 }
 
 __global__ __launch_bounds__(kBlock) void f16_to_f32(const h16* __restrict__ in,

@@ -28,7 +28,7 @@ __device__ __forceinline__ float inv_rms(float sumsq, int n, float eps) {
 // ── one wave per row, row held in registers ──────────────────────────────
 // kCpl = chunks per lane (row width <= 512 * kCpl halves); kFull = the row is
 // exactly 64 * kCpl chunks, so no lane is ever idle and loads are unpredicated.
-template <int kCpl, int kMode, bool kFull>
+template <int kCpl, int kMode, bool kFull, bool kStream>
 __global__ __launch_bounds__(kBlock) void norm_rows_wave(
     const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
     const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float eps) {
@@ -50,8 +50,8 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
         if (kFull || c < nchunks) {
-            a[j] = load_chunk(s + c);
-            if (kMode == kAdd) b[j] = load_chunk(state + out_base + c);
+            a[j] = load_chunk_as<kStream>(s + c);
+            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
         }
     }
 
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
 #pragma unroll
         for (int j = 0; j < kCpl; ++j) {
             const int c = j * kWave + lane;
-            if (kFull || c < nchunks) store_chunk(state + out_base + c, a[j]);
+            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
         }
         return;
     }
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
 #pragma unroll
         for (int j = 0; j < kCpl; ++j) {
             const int c = j * kWave + lane;
-            if (kFull || c < nchunks) store_chunk(state + out_base + c, a[j]);
+            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
         }
     }
 
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
             const f32x8 g = unpack(w[j]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
-            store_chunk(normed + out_base + c, pack(x));
+            store_chunk_as<kStream>(normed + out_base + c, pack(x));
         }
     }
 }
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_block(
             for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
         } else {
             h16 v = s[c];
-            if (kMode == kAdd) v = (h16)((float)st[c] + (float)v);
+            if (kMode == kAdd) v = to_half((float)st[c] + (float)v);
             if (kMode != kPlain) st[c] = v;
             acc = fmaf((float)v, (float)v, acc);
         }
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_block(
             for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
             store_chunk(out + c, pack(x));
         } else {
-            out[c] = (h16)(((float)again[c] * inv) * (float)weight[c]);
+            out[c] = to_half(((float)again[c] * inv) * (float)weight[c]);
         }
     }
 }
@@ -188,20 +188,24 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         const dim3 grid((unsigned)((rows + kWavesPerBlock - 1) / kWavesPerBlock));
         const int cpl = (nchunks + kWave - 1) / kWave;
         const bool full = nchunks == cpl * kWave;
-#define VV_ROWS_CASE(N)                                                                      \
-    case N:                                                                                  \
-        if (full)                                                                            \
-            norm_rows_wave<N, kMode, true><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, \
-                                                                     nchunks, eps);          \
-        else                                                                                 \
-            norm_rows_wave<N, kMode, false><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows,\
-                                                                      nchunks, eps);         \
+        // bytes this launch streams: 2 tensors (plain, gather-only), 3 (gather+norm), 4 (add+norm)
+        const size_t tensors = kMode == kAdd ? 4 : (kMode == kGather ? 3 : 2);
+        const bool stream = use_streaming(tensors * (size_t)rows * (size_t)hidden * 2u);
+#define VV_ROWS_LAUNCH(N, F, S) \
+    norm_rows_wave<N, kMode, F, S><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, nchunks, eps)
+#define VV_ROWS_CASE(N)                                       \
+    case N:                                                   \
+        if (full && stream)       VV_ROWS_LAUNCH(N, true, true);   \
+        else if (full)            VV_ROWS_LAUNCH(N, true, false);  \
+        else if (stream)          VV_ROWS_LAUNCH(N, false, true);  \
+        else                      VV_ROWS_LAUNCH(N, false, false); \
         break;
         switch (cpl) {
             VV_ROWS_CASE(1) VV_ROWS_CASE(2) VV_ROWS_CASE(3) VV_ROWS_CASE(4)
             VV_ROWS_CASE(5) VV_ROWS_CASE(6) VV_ROWS_CASE(7) VV_ROWS_CASE(8)
         }
 #undef VV_ROWS_CASE
+#undef VV_ROWS_LAUNCH
         return launch_status();
     }
     if (vec) {

@@ -65,7 +65,7 @@ __device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
 }
 
 // head_dim == 128, 16-byte aligned tensors.
-template <bool kBias>
+template <bool kBias, bool kStream>
 __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
     __shared__ __attribute__((aligned(16))) float cs_cos[kPosPerBlock][64];
     __shared__ __attribute__((aligned(16))) float cs_sin[kPosPerBlock][64];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
             }
             Chunk* lo_p = reinterpret_cast<Chunk*>(base) + c;
             Chunk* hi_p = lo_p + 8;
-            Chunk lo = load_chunk(lo_p), hi = load_chunk(hi_p);
+            Chunk lo = load_chunk_as<kStream>(lo_p), hi = load_chunk_as<kStream>(hi_p);
             if (kBias && bias) {
                 const Chunk* bp = reinterpret_cast<const Chunk*>(bias) + c;
                 lo = add_bias(lo, load_chunk(bp));
@@ -119,8 +119,8 @@ __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
                 y0[i] = r.lo;
                 y1[i] = r.hi;
             }
-            store_chunk(lo_p, pack(y0));
-            store_chunk(hi_p, pack(y1));
+            store_chunk_as<kStream>(lo_p, pack(y0));
+            store_chunk_as<kStream>(hi_p, pack(y1));
         }
     }
 }
@@ -157,14 +157,14 @@ __global__ __launch_bounds__(kBlock) void rope_generic(RopeArgs a, FreqTable fre
         }
         h16 h0 = v[i], h1 = v[i + half];
         if (bias) {
-            h0 = (h16)((float)h0 + (float)bias[i]);
-            h1 = (h16)((float)h1 + (float)bias[i + half]);
+            h0 = to_half((float)h0 + (float)bias[i]);
+            h1 = to_half((float)h1 + (float)bias[i + half]);
         }
         const float x0 = (float)h0, x1 = (float)h1;
         const float c = cs_cos[i], s = cs_sin[i];
         const Pair r = rotate(x0, x1, c, s);
-        v[i] = (h16)r.lo;
-        v[i + half] = (h16)r.hi;
+        v[i] = to_half(r.lo);
+        v[i + half] = to_half(r.hi);
     }
 }
 
@@ -208,8 +208,11 @@ vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias
                       (!a.q_bias || aligned16(a.q_bias)) && (!a.k_bias || aligned16(a.k_bias));
     if (fast) {
         const dim3 grid((unsigned)((rows + kPosPerBlock - 1) / kPosPerBlock));
-        if (has_bias) rope128<true><<<grid, kBlock, 0, st>>>(a, freqs);
-        else          rope128<false><<<grid, kBlock, 0, st>>>(a, freqs);
+        const bool stream = use_streaming(2u * (size_t)rows * (size_t)(nq + nk) * 128u * 2u);
+        if (has_bias && stream)  rope128<true, true><<<grid, kBlock, 0, st>>>(a, freqs);
+        else if (has_bias)       rope128<true, false><<<grid, kBlock, 0, st>>>(a, freqs);
+        else if (stream)         rope128<false, true><<<grid, kBlock, 0, st>>>(a, freqs);
+        else                     rope128<false, false><<<grid, kBlock, 0, st>>>(a, freqs);
     } else {
         rope_generic<<<dim3((unsigned)rows), kBlock, 0, st>>>(a, freqs);
     }

@@ -10,6 +10,9 @@
 //     a captured graph and replay correctly.
 #include <stdio.h>
 
+#include <algorithm>
+#include <vector>
+
 #include "vv_common.hpp"
 
 namespace vv {
@@ -46,6 +49,40 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(unsigned char* ptr, unsign
     for (size_t i = gid; i < chunks; i += stride) mid[i] = c;
 }
 
+// ── captures in flight on this host thread ───────────────────────────────
+// An uncapturable call (a synchronisation, an allocation, a synchronous copy)
+// made while this thread is capturing must fail the capture rather than run.
+// The HIP runtime does mark such a capture invalid, but it then leaves the
+// stream in that state for good: hipStreamEndCapture reports the error without
+// ending the capture, and every later launch on the stream fails. The caller
+// of a broken capture reissues its work on the same stream, so this backend
+// ends the capture itself, cleanly, BEFORE the offending runtime call would
+// wedge it: the recorded graph is discarded, the stream is remembered as
+// "broken", and vv_dev_graph_end on it reports the failure. Capture is
+// thread-local (hipStreamCaptureModeThreadLocal), so thread-local lists suffice
+// and other threads' streams are never touched.
+thread_local std::vector<hipStream_t> tl_capturing;
+thread_local std::vector<hipStream_t> tl_broken;
+
+bool break_captures_of_this_thread() {
+    if (tl_capturing.empty()) return false;
+    for (hipStream_t s : tl_capturing) {
+        hipGraph_t g = nullptr;
+        if (hipStreamEndCapture(s, &g) == hipSuccess && g) (void)hipGraphDestroy(g);
+        tl_broken.push_back(s);
+    }
+    tl_capturing.clear();
+    (void)hipGetLastError();
+    return true;
+}
+
+bool forget(std::vector<hipStream_t>& v, hipStream_t s) {
+    auto it = std::find(v.begin(), v.end(), s);
+    if (it == v.end()) return false;
+    v.erase(it);
+    return true;
+}
+
 vv_status_t rt(hipError_t e) {
     if (e == hipSuccess) return VV_OK;
     (void)hipGetLastError();          // do not let the failure leak into the next call
@@ -56,6 +93,7 @@ vv_status_t copy(void* dst, const void* src, size_t size, hipMemcpyKind kind, vo
     if (size == 0) return VV_OK;
     if (!dst || !src) return VV_ERR_NULL_PTR;
     if (stream) return rt(hipMemcpyAsync(dst, src, size, kind, as_stream(stream)));
+    if (break_captures_of_this_thread()) return VV_ERR_CUDA;   // synchronous copy
     return rt(hipMemcpy(dst, src, size, kind));
 }
 
@@ -66,6 +104,7 @@ extern "C" {
 
 vv_status_t vv_dev_alloc(void** ptr, size_t size) {
     if (!ptr) return VV_ERR_NULL_PTR;
+    if (vv::break_captures_of_this_thread()) { *ptr = nullptr; return VV_ERR_CUDA; }
     const hipError_t e = hipMalloc(ptr, size);
     if (e == hipErrorOutOfMemory) { (void)hipGetLastError(); *ptr = nullptr; return VV_ERR_CUDA_OOM; }
     if (e != hipSuccess) { *ptr = nullptr; return vv::rt(e); }
@@ -74,6 +113,7 @@ vv_status_t vv_dev_alloc(void** ptr, size_t size) {
 
 vv_status_t vv_dev_alloc_pinned(void** ptr, size_t size) {
     if (!ptr) return VV_ERR_NULL_PTR;
+    if (vv::break_captures_of_this_thread()) { *ptr = nullptr; return VV_ERR_CUDA; }
     const hipError_t e = hipHostMalloc(ptr, size, hipHostMallocDefault);
     if (e != hipSuccess) { *ptr = nullptr; return vv::rt(e); }
     return VV_OK;
@@ -81,11 +121,13 @@ vv_status_t vv_dev_alloc_pinned(void** ptr, size_t size) {
 
 vv_status_t vv_dev_free(void* ptr) {
     if (!ptr) return VV_OK;
+    vv::break_captures_of_this_thread();      // hipFree synchronises the device
     return vv::rt(hipFree(ptr));
 }
 
 vv_status_t vv_dev_free_pinned(void* ptr) {
     if (!ptr) return VV_OK;
+    vv::break_captures_of_this_thread();
     return vv::rt(hipHostFree(ptr));
 }
 
@@ -145,6 +187,7 @@ vv_status_t vv_dev_memset_async(void* ptr, int value, size_t size, void* stream)
 
 vv_status_t vv_dev_memset(void* ptr, int value, size_t size) {
     if (!ptr) return VV_ERR_NULL_PTR;
+    if (vv::break_captures_of_this_thread()) return VV_ERR_CUDA;
     return vv::rt(hipMemset(ptr, value, size));
 }
 
@@ -163,11 +206,27 @@ vv_status_t vv_dev_stream_create_background(void** stream) {
 
 vv_status_t vv_dev_stream_destroy(void* stream) {
     if (!stream) return VV_OK;
+    if (vv::forget(vv::tl_capturing, vv::as_stream(stream))) {
+        hipGraph_t g = nullptr;
+        if (hipStreamEndCapture(vv::as_stream(stream), &g) == hipSuccess && g)
+            (void)hipGraphDestroy(g);
+        (void)hipGetLastError();
+    }
+    vv::forget(vv::tl_broken, vv::as_stream(stream));
     return vv::rt(hipStreamDestroy(vv::as_stream(stream)));
 }
 
 vv_status_t vv_dev_stream_sync(void* stream) {
-    if (stream) return vv::rt(hipStreamSynchronize(vv::as_stream(stream)));
+    if (stream) {
+        hipStream_t s = vv::as_stream(stream);
+        if (std::find(vv::tl_capturing.begin(), vv::tl_capturing.end(), s) !=
+            vv::tl_capturing.end()) {
+            vv::break_captures_of_this_thread();
+            return VV_ERR_CUDA;               // a capturing stream cannot be waited on
+        }
+        return vv::rt(hipStreamSynchronize(s));
+    }
+    if (vv::break_captures_of_this_thread()) return VV_ERR_CUDA;
     return vv::rt(hipDeviceSynchronize());
 }
 
@@ -281,12 +340,19 @@ const char* vv_dev_backend_name(void) { return "HIP"; }
 
 vv_status_t vv_dev_graph_begin(void* stream) {
     if (!stream) return VV_ERR_INVALID_ARG;      // the default stream cannot be captured
-    return vv::rt(hipStreamBeginCapture(vv::as_stream(stream), hipStreamCaptureModeThreadLocal));
+    hipStream_t s = vv::as_stream(stream);
+    vv::forget(vv::tl_broken, s);
+    const vv_status_t st = vv::rt(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    if (st == VV_OK) vv::tl_capturing.push_back(s);
+    return st;
 }
 
 vv_status_t vv_dev_graph_end(void* stream, void** graph_exec) {
     if (!stream || !graph_exec) return VV_ERR_NULL_PTR;
     *graph_exec = nullptr;
+    // Ended early by an uncapturable call: nothing was kept, the stream is usable.
+    if (vv::forget(vv::tl_broken, vv::as_stream(stream))) return VV_ERR_CUDA;
+    vv::forget(vv::tl_capturing, vv::as_stream(stream));
     hipGraph_t graph = nullptr;
     const hipError_t e = hipStreamEndCapture(vv::as_stream(stream), &graph);
     if (e != hipSuccess || !graph) {

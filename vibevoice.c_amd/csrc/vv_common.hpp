@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/vibevoice_hip.h"
 
@@ -29,8 +30,15 @@ static_assert(sizeof(Chunk) == 16, "Chunk must be 16 bytes");
 __device__ __forceinline__ Chunk load_chunk(const Chunk* p) { return *p; }
 __device__ __forceinline__ void store_chunk(Chunk* p, const Chunk& c) { *p = c; }
 
-// Streaming forms: the data is touched once, so it should not displace lines
-// that other kernels will reuse (the "nt" bit on global_load/global_store).
+// Streaming forms (the "nt" bit on global_load/global_store): the line is
+// touched once and should be the first to leave the caches. On MI355X a plain
+// copy moves 5.7 TB/s with ordinary accesses and 6.3 TB/s with these; the
+// hosts pick them when a launch's footprint exceeds what the last-level cache
+// could keep for the next kernel anyway (kStreamBytes), and ordinary accesses
+// below that, so a decode step or a prefill chunk leaves its output cached for
+// the GEMM that consumes it.
+constexpr size_t kStreamBytes = (size_t)96 << 20;
+
 __device__ __forceinline__ Chunk load_chunk_stream(const Chunk* p) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
@@ -44,6 +52,17 @@ __device__ __forceinline__ void store_chunk_stream(Chunk* p, const Chunk& c) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+template <bool kStream>
+__device__ __forceinline__ Chunk load_chunk_as(const Chunk* p) {
+    if constexpr (kStream) return load_chunk_stream(p);
+    else return load_chunk(p);
+}
+template <bool kStream>
+__device__ __forceinline__ void store_chunk_as(Chunk* p, const Chunk& c) {
+    if constexpr (kStream) store_chunk_stream(p, c);
+    else store_chunk(p, c);
+}
+
 __device__ __forceinline__ f32x8 unpack(const Chunk& c) {
     const h16x8 h = __builtin_bit_cast(h16x8, c);
     f32x8 f;
@@ -53,11 +72,20 @@ __device__ __forceinline__ f32x8 unpack(const Chunk& c) {
 }
 
 // FP32 -> FP16 with round-to-nearest-even (v_cvt_f16_f32 under the default
-// rounding mode), packed back into one chunk.
+// rounding mode). The empty asm makes the FP32 value opaque at this point:
+// without it the compiler may fold a preceding multiply by a widened FP16
+// operand into v_fma_mixlo_f16 with a +0 addend, which turns a product of -0
+// into +0 (observed in the 2-byte SwiGLU path).
+__device__ __forceinline__ h16 to_half(float v) {
+    asm("" : "+v"(v));
+    return (h16)v;
+}
+
+// Eight of them, packed back into one chunk.
 __device__ __forceinline__ Chunk pack(const f32x8& f) {
     h16x8 h;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = (h16)f[i];
+    for (int i = 0; i < 8; ++i) h[i] = to_half(f[i]);
     return __builtin_bit_cast(Chunk, h);
 }
 
@@ -95,6 +123,16 @@ __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63); }
 
 // ── host helpers ─────────────────────────────────────────────────────────
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Streaming accesses for launches of at least kStreamBytes; the environment
+// variable VV_HIP_STREAM=0 / 1 forces them off / on (for A/B measurements).
+inline bool use_streaming(size_t launch_bytes) {
+    static const int forced = [] {
+        const char* e = getenv("VV_HIP_STREAM");
+        return (e && (e[0] == '0' || e[0] == '1')) ? e[0] - '0' : -1;
+    }();
+    return forced >= 0 ? forced == 1 : launch_bytes >= kStreamBytes;
+}
 
 inline vv_status_t launch_status() {
     return hipGetLastError() == hipSuccess ? VV_OK : VV_ERR_CUDA_LAUNCH;

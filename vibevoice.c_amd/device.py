@@ -78,6 +78,16 @@ SIGNATURES = {
 
 
 def _load() -> C.CDLL:
+    # A process must hold ONE HIP runtime. PyTorch wheels bundle their own
+    # libamdhip64.so.7; if this library were loaded first it would pull in the
+    # system copy and a later `import torch` would bring a second one (observed:
+    # a segmentation fault at torch's first device call). Importing torch first
+    # makes the loader reuse torch's copy for this library (same SONAME). In a
+    # process without torch the system runtime is used.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python vibevoice.c_amd/build.py` "
