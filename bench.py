@@ -222,6 +222,10 @@ def main() -> int:
     ap.add_argument("--launches", type=int, default=20, help="back-to-back launches per event pair")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default=None, help="time only this kernel (profiling aid)")
+    ap.add_argument("--reps", type=int, default=5, help="event-timed repetitions per kernel")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
+                         "five times: the known-size reference for rocprofv3 byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every op is row-independent and this build uses no "
@@ -240,6 +244,16 @@ def main() -> int:
     log(f"device: {name_buf}; T={T}, sets={args.sets}")
     wl = Workload(torch, dev, T, args.sets)
     st = torch.cuda.current_stream().cuda_stream
+    if args.calibrate:
+        n = 256 << 20
+        src = torch.ones(n, dtype=torch.uint8, device="cuda")
+        dst = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+        for _ in range(5):
+            assert dev.vv_dev_memcpy_d2d_at(dst.data_ptr(), src.data_ptr(), n, idx.data_ptr(), st) == 0
+        torch.cuda.synchronize()
+        assert bool((dst == 1).all())
+        del src, dst
     bytes_per = algorithmic_bytes(T)
     kernels = [args.only] if args.only else KERNELS
 
@@ -262,7 +276,7 @@ def main() -> int:
     # ── per kernel, HIP events on the launch stream ──
     per = {}
     for name in kernels:
-        best, med = time_kernel(torch, wl, name, args.launches, 5, st)
+        best, med = time_kernel(torch, wl, name, args.launches, args.reps, st)
         per[name] = {
             "bytes": bytes_per[name],
             "us_median": med * 1e6, "us_best": best * 1e6,

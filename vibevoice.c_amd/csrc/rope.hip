@@ -64,19 +64,74 @@ __device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
     return r;
 }
 
-// head_dim == 128, 16-byte aligned tensors.
-template <bool kBias, bool kStream>
-__global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
+// head_dim == 128, 16-byte aligned tensors, at most kMaxFastHeads heads in all.
+//
+// A workgroup owns `posb` consecutive positions (4 when Q+K is 32 heads). Work
+// item = (position, head, chunk pair); thread t takes items t, t+256, ... — at
+// most kItems of them. Order inside the kernel: issue every global load of the
+// thread's items first, THEN compute the cos/sin table (one (position, pair)
+// per thread, full-range sincosf) and cross the barrier, so the memory latency
+// runs under the transcendental work; then rotate and store.
+constexpr int kItems = 4;
+constexpr int kMaxFastHeads = kItems * kBlock / 8;   // 128: one position per workgroup
+
+template <bool kBias, bool kStream, bool kExact>   // kExact: 32 heads, 256 items per position
+__global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs, int posb) {
     __shared__ __attribute__((aligned(16))) float cs_cos[kPosPerBlock][64];
     __shared__ __attribute__((aligned(16))) float cs_sin[kPosPerBlock][64];
 
     const int first = a.d_position ? *a.d_position : a.position_offset;
-    const int row0 = (int)blockIdx.x * kPosPerBlock;
+    const int row0 = (int)blockIdx.x * posb;
+    const int tasks = (a.nq + a.nk) * 8;            // (head, chunk pair) per position
+    const int items = min(posb, a.rows - row0) * tasks;
+    // Fetched before the tensor loads are issued: memory returns in issue order,
+    // so waiting for this value later does not wait for the tensor data.
+    float my_freq = freqs.f[threadIdx.x & 63];
 
-    {   // phase 1: thread t -> (position t / 64, pair t % 64)
+    // Loads are unconditional (an item past the end re-reads the last valid
+    // one and is simply not stored): straight-line code lets the compiler count
+    // outstanding loads exactly instead of draining them all at the first use.
+    Chunk* lo_p[kItems];
+    Chunk lo[kItems], hi[kItems];
+    int p_of[kItems], c_of[kItems];
+    bool live[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int want = (int)threadIdx.x + k * kBlock;
+        live[k] = want < items;
+        const int item = live[k] ? want : items - 1;
+        const int p = kExact ? item >> 8 : item / tasks;
+        const int t = kExact ? item & 255 : item - p * tasks;
+        const int head = t >> 3, c = t & 7;
+        const size_t row = (size_t)(row0 + p);
+        h16* base = head < a.nq
+            ? a.q + (row * (size_t)a.nq + (size_t)head) * 128u
+            : a.k + (row * (size_t)a.nk + (size_t)(head - a.nq)) * 128u;
+        lo_p[k] = reinterpret_cast<Chunk*>(base) + c;
+        lo[k] = load_chunk_as<kStream>(lo_p[k]);
+        hi[k] = load_chunk_as<kStream>(lo_p[k] + 8);
+        p_of[k] = p;
+        c_of[k] = c;
+        if (kBias) {
+            const h16* bias = head < a.nq
+                ? (a.q_bias ? a.q_bias + (size_t)head * 128u : nullptr)
+                : (a.k_bias ? a.k_bias + (size_t)(head - a.nq) * 128u : nullptr);
+            if (bias) {
+                const Chunk* bp = reinterpret_cast<const Chunk*>(bias) + c;
+                lo[k] = add_bias(lo[k], load_chunk(bp));
+                hi[k] = add_bias(hi[k], load_chunk(bp + 8));
+            }
+        }
+    }
+
+    // Use point of my_freq, outside any branch, so its load stays where it was
+    // written (ahead of the tensor loads) and only it is waited for here.
+    asm volatile("" : "+v"(my_freq));
+
+    if ((int)threadIdx.x < posb * 64) {      // thread t -> (position t / 64, pair t % 64)
         const int p = (int)threadIdx.x >> 6, i = (int)threadIdx.x & 63;
         const int pos = first + row0 + p;
-        const float ang = (float)pos * freqs.f[i];
+        const float ang = (float)pos * my_freq;
         float s, c;
         sincosf(ang, &s, &c);
         cs_cos[p][i] = c;
@@ -84,34 +139,12 @@ __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
     }
     __syncthreads();
 
-    const int heads = a.nq + a.nk;
-    const int tasks = heads * 8;                 // (head, chunk-pair) per position
-    const int rows_here = min(kPosPerBlock, a.rows - row0);
-
-    for (int p = 0; p < rows_here; ++p) {
-        const size_t row = (size_t)(row0 + p);
-        for (int t = (int)threadIdx.x; t < tasks; t += kBlock) {
-            const int head = t >> 3, c = t & 7;
-            h16* base;
-            const h16* bias = nullptr;
-            if (head < a.nq) {
-                base = a.q + (row * (size_t)a.nq + (size_t)head) * 128u;
-                if (kBias && a.q_bias) bias = a.q_bias + (size_t)head * 128u;
-            } else {
-                base = a.k + (row * (size_t)a.nk + (size_t)(head - a.nq)) * 128u;
-                if (kBias && a.k_bias) bias = a.k_bias + (size_t)(head - a.nq) * 128u;
-            }
-            Chunk* lo_p = reinterpret_cast<Chunk*>(base) + c;
-            Chunk* hi_p = lo_p + 8;
-            Chunk lo = load_chunk_as<kStream>(lo_p), hi = load_chunk_as<kStream>(hi_p);
-            if (kBias && bias) {
-                const Chunk* bp = reinterpret_cast<const Chunk*>(bias) + c;
-                lo = add_bias(lo, load_chunk(bp));
-                hi = add_bias(hi, load_chunk(bp + 8));
-            }
-            const f32x8 x0 = unpack(lo), x1 = unpack(hi);
-            const f32x8 cv = *reinterpret_cast<const f32x8*>(&cs_cos[p][c * 8]);
-            const f32x8 sv = *reinterpret_cast<const f32x8*>(&cs_sin[p][c * 8]);
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (live[k]) {
+            const f32x8 x0 = unpack(lo[k]), x1 = unpack(hi[k]);
+            const f32x8 cv = *reinterpret_cast<const f32x8*>(&cs_cos[p_of[k]][c_of[k] * 8]);
+            const f32x8 sv = *reinterpret_cast<const f32x8*>(&cs_sin[p_of[k]][c_of[k] * 8]);
             f32x8 y0, y1;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -119,8 +152,8 @@ __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs) {
                 y0[i] = r.lo;
                 y1[i] = r.hi;
             }
-            store_chunk_as<kStream>(lo_p, pack(y0));
-            store_chunk_as<kStream>(hi_p, pack(y1));
+            store_chunk_as<kStream>(lo_p[k], pack(y0));
+            store_chunk_as<kStream>(lo_p[k] + 8, pack(y1));
         }
     }
 }
@@ -204,15 +237,24 @@ vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias
     const FreqTable& freqs = host_freqs(theta, head_dim);
     const bool has_bias = a.q_bias || a.k_bias;
 
-    const bool fast = head_dim == 128 && (!a.q || aligned16(a.q)) && (!a.k || aligned16(a.k)) &&
+    const bool fast = head_dim == 128 && nq + nk <= kMaxFastHeads &&
+                      (!a.q || aligned16(a.q)) && (!a.k || aligned16(a.k)) &&
                       (!a.q_bias || aligned16(a.q_bias)) && (!a.k_bias || aligned16(a.k_bias));
     if (fast) {
-        const dim3 grid((unsigned)((rows + kPosPerBlock - 1) / kPosPerBlock));
+        // as many positions per workgroup as kItems items per thread allow, at most 4
+        int posb = kItems * kBlock / ((nq + nk) * 8);
+        if (posb > kPosPerBlock) posb = kPosPerBlock;
+        const dim3 grid((unsigned)((rows + posb - 1) / posb));
         const bool stream = use_streaming(2u * (size_t)rows * (size_t)(nq + nk) * 128u * 2u);
-        if (has_bias && stream)  rope128<true, true><<<grid, kBlock, 0, st>>>(a, freqs);
-        else if (has_bias)       rope128<true, false><<<grid, kBlock, 0, st>>>(a, freqs);
-        else if (stream)         rope128<false, true><<<grid, kBlock, 0, st>>>(a, freqs);
-        else                     rope128<false, false><<<grid, kBlock, 0, st>>>(a, freqs);
+        const bool exact = (nq + nk) * 8 == kBlock;
+#define VV_ROPE_LAUNCH(B, S, E) rope128<B, S, E><<<grid, kBlock, 0, st>>>(a, freqs, posb)
+#define VV_ROPE_PICK(B, S) (exact ? VV_ROPE_LAUNCH(B, S, true) : VV_ROPE_LAUNCH(B, S, false))
+        if (has_bias && stream)  VV_ROPE_PICK(true, true);
+        else if (has_bias)       VV_ROPE_PICK(true, false);
+        else if (stream)         VV_ROPE_PICK(false, true);
+        else                     VV_ROPE_PICK(false, false);
+#undef VV_ROPE_PICK
+#undef VV_ROPE_LAUNCH
     } else {
         rope_generic<<<dim3((unsigned)rows), kBlock, 0, st>>>(a, freqs);
     }
