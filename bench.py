@@ -48,6 +48,12 @@ def algorithmic_bytes(T: int) -> dict:
         "add+norm": 8 * T * H + 2 * H,                 # read x, residual; write residual, normed
         "rope": 4 * T * (NQ + NK) * HD,                # read + write Q and K
         "swiglu": 6 * T * I_FF,                        # read gate, up; write out
+        # unfused reference-API forms, timed only with --unfused (not part of the step)
+        "embedding": T * (4 + 4 * H),
+        "rmsnorm": 4 * T * H + 2 * H,
+        "residual_add": 6 * T * H,
+        "rope_q": 4 * T * NQ * HD,
+        "rope_k": 4 * T * NK * HD,
     }
 
 
@@ -96,6 +102,18 @@ class Workload:
         elif name == "swiglu":
             rc = dev.vv_swiglu_dev(d["gate"].data_ptr(), d["up"].data_ptr(), d["out"].data_ptr(),
                                    T * I_FF, st)
+        elif name == "embedding":
+            rc = dev.vv_embedding_dev(self.table.data_ptr(), d["ids"].data_ptr(),
+                                      d["hidden"].data_ptr(), T, H, st)
+        elif name == "rmsnorm":
+            rc = dev.vv_rmsnorm_dev(d["x"].data_ptr(), self.weight.data_ptr(),
+                                    d["normed"].data_ptr(), T, H, EPS, st)
+        elif name == "residual_add":
+            rc = dev.vv_residual_add_dev(d["residual"].data_ptr(), d["x"].data_ptr(), T * H, st)
+        elif name == "rope_q":
+            rc = dev.vv_rope_dev(d["q"].data_ptr(), T, NQ, HD, 0, None, THETA, st)
+        elif name == "rope_k":
+            rc = dev.vv_rope_dev(d["k"].data_ptr(), T, NK, HD, 0, None, THETA, st)
         else:
             raise KeyError(name)
         if rc != 0:
@@ -103,6 +121,7 @@ class Workload:
 
 
 KERNELS = ["gather+norm", "add+norm", "rope", "swiglu"]
+UNFUSED = ["embedding", "rmsnorm", "residual_add", "rope_q", "rope_k"]
 
 
 def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: int):
@@ -223,6 +242,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only", default=None, help="time only this kernel (profiling aid)")
     ap.add_argument("--reps", type=int, default=5, help="event-timed repetitions per kernel")
+    ap.add_argument("--unfused", action="store_true",
+                    help="also time the unfused reference-API calls (reported under 'unfused')")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
                          "five times: the known-size reference for rocprofv3 byte counters")
@@ -287,6 +308,16 @@ def main() -> int:
         log(f"  {name:12s} {med * 1e6:9.2f} us  {per[name]['GBps']:8.1f} GB/s  "
             f"{100 * per[name]['frac_of_peak']:5.1f} % of peak  {T / med:12.0f} rows/s")
 
+    unfused = {}
+    if args.unfused:
+        for name in UNFUSED:
+            best, med = time_kernel(torch, wl, name, args.launches, args.reps, st)
+            unfused[name] = {"bytes": bytes_per[name], "us_median": med * 1e6,
+                             "GBps": bytes_per[name] / med / 1e9,
+                             "frac_of_peak": bytes_per[name] / med / 1e9 / HBM_PEAK_GBPS}
+            log(f"  {name:12s} {med * 1e6:9.2f} us  {unfused[name]['GBps']:8.1f} GB/s  "
+                f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (unfused form)")
+
     dominant = max(kernels, key=lambda n: bytes_per[n])
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
@@ -309,6 +340,8 @@ def main() -> int:
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": per[dominant]["frac_of_peak"], "traffic": traffic},
     }
+    if unfused:
+        result["unfused"] = unfused
     if not args.no_cpu:
         log(f"cpu baseline on {CPU_SAMPLE_ROWS} rows ...")
         result["cpu_baseline"] = cpu_baseline(CPU_SAMPLE_ROWS)

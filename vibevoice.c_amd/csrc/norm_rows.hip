@@ -20,9 +20,13 @@ enum RowMode : int {
     kGatherOnly = 3  // state = src[ids[row]]
 };
 
-__device__ __forceinline__ float inv_rms(float sumsq, int n, float eps) {
-    const float mean = sumsq / (float)n;
-    return 1.0f / sqrtf(mean + eps);
+// 1 / sqrt(mean(x^2) + eps) with the hardware reciprocal square root (1 ulp of
+// FP32, i.e. ~1e-7 relative against an FP16 result whose own rounding is 5e-4).
+// Every lane of every wave of a row evaluates this, so it has to be a handful
+// of instructions: the correctly rounded divide + sqrt + divide sequence is
+// ~60 and was a measurable share of the VALU time with one chunk per thread.
+__device__ __forceinline__ float inv_rms(float sumsq, float inv_n, float eps) {
+    return __builtin_amdgcn_rsqf(sumsq * inv_n + eps);
 }
 
 // ── one wave per row, row held in registers ──────────────────────────────
@@ -31,7 +35,8 @@ __device__ __forceinline__ float inv_rms(float sumsq, int n, float eps) {
 template <int kCpl, int kMode, bool kFull, bool kStream>
 __global__ __launch_bounds__(kBlock) void norm_rows_wave(
     const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
-    const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float eps) {
+    const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float inv_n,
+    float eps) {
     const int row = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
     if (row >= rows) return;
     const int lane = lane_id();
@@ -43,14 +48,18 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
     const size_t out_base = (size_t)row * (size_t)nchunks;
 
     // Issue every load of the row before the first use: kCpl (or 2*kCpl)
-    // independent 16-byte loads in flight per lane.
+    // independent 16-byte loads in flight per lane. Gathered table rows are
+    // read with ordinary loads even in streaming launches: measured on MI355X,
+    // a row gather with streaming loads runs 10 % slower (5.3 vs 5.9 TB/s for
+    // gather + two outputs), and a table row may well be needed again.
+    constexpr bool kStreamSrc = kStream && !(kMode == kGather || kMode == kGatherOnly);
     Chunk a[kCpl];
     Chunk b[kCpl];
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
         if (kFull || c < nchunks) {
-            a[j] = load_chunk_as<kStream>(s + c);
+            a[j] = load_chunk_as<kStreamSrc>(s + c);
             if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
         }
     }
@@ -98,11 +107,97 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
         }
     }
 
-    const float inv = inv_rms(wave_sum(acc), nchunks * 8, eps);
+    const float inv = inv_rms(wave_sum(acc), inv_n, eps);
 
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
+        if (kFull || c < nchunks) {
+            f32x8 x = unpack(a[j]);
+            const f32x8 g = unpack(w[j]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
+            store_chunk_as<kStream>(normed + out_base + c, pack(x));
+        }
+    }
+}
+
+// ── one workgroup per row, one chunk per thread ──────────────────────────
+// blockDim = the row's chunk count rounded up to whole waves (448 threads = 7
+// waves for hidden 3584), kCpt chunks per thread for rows wider than 1024
+// chunks. Every wave is light (one or two 16-byte loads per lane), which is the
+// shape the memory system rewards: a pure copy with this structure moves
+// 6.4 TB/s for the add+norm traffic pattern against 5.8 TB/s with one wave per
+// row. Sum of squares: DPP reduction inside each wave, then one float per wave
+// through LDS and a single barrier.
+constexpr int kMaxWgThreads = 1024;
+
+template <int kCpt, int kMode, bool kStream, bool kFull>   // kFull: nchunks == kCpt * blockDim.x
+__global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
+    const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
+    const Chunk* __restrict__ weight, Chunk* normed, int nchunks, float inv_n, float eps) {
+    __shared__ float partial[kMaxWgThreads / kWave];
+    const size_t row = blockIdx.x;
+    const int t = (int)threadIdx.x;
+    const int nthreads = (int)blockDim.x;
+
+    size_t src_row = row;
+    if (kMode == kGather || kMode == kGatherOnly) src_row = (size_t)ids[row];
+    const Chunk* s = src + src_row * (size_t)nchunks;
+    const size_t out_base = row * (size_t)nchunks;
+    constexpr bool kStreamSrc = kStream && !(kMode == kGather || kMode == kGatherOnly);
+
+    Chunk a[kCpt], b[kCpt], w[kCpt];
+#pragma unroll
+    for (int j = 0; j < kCpt; ++j) {
+        const int c = j * nthreads + t;
+        if (kFull || c < nchunks) {
+            a[j] = load_chunk_as<kStreamSrc>(s + c);
+            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
+            if (kMode != kGatherOnly) w[j] = load_chunk(weight + c);
+        }
+    }
+    if (kMode == kGatherOnly) {
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
+        }
+        return;
+    }
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kCpt; ++j) {
+        const int c = j * nthreads + t;
+        if (kFull || c < nchunks) {
+            f32x8 x = unpack(a[j]);
+            if (kMode == kAdd) {
+                const f32x8 r = unpack(b[j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = r[i] + x[i];
+                // stored residual = FP16 rounding of the sum; the norm reads that value
+                a[j] = pack(x);
+                x = unpack(a[j]);
+            }
+            if (kMode == kAdd || kMode == kGather)
+                store_chunk_as<kStream>(state + out_base + c, a[j]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
+        }
+    }
+
+    acc = wave_sum(acc);
+    if (lane_id() == 0) partial[t >> 6] = acc;
+    __syncthreads();
+    float total = 0.0f;
+    const int nwaves = nthreads >> 6;
+    for (int i = 0; i < nwaves; ++i) total += partial[i];
+    const float inv = inv_rms(total, inv_n, eps);
+
+#pragma unroll
+    for (int j = 0; j < kCpt; ++j) {
+        const int c = j * nthreads + t;
         if (kFull || c < nchunks) {
             f32x8 x = unpack(a[j]);
             const f32x8 g = unpack(w[j]);
@@ -120,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
 template <int kMode, typename T>   // T = Chunk (8 halves at a time) or h16
 __global__ __launch_bounds__(kBlock) void norm_rows_block(
     const T* src, T* state, const int32_t* __restrict__ ids, const T* __restrict__ weight,
-    T* normed, int units, int hidden, float eps) {
+    T* normed, int units, float inv_n, float eps) {
     __shared__ float partial[kWavesPerBlock];
     const int row = (int)blockIdx.x;
     size_t src_row = (size_t)row;
@@ -157,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_block(
     if (lane_id() == 0) partial[threadIdx.x >> 6] = acc;
     __syncthreads();
     const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
-    const float inv = inv_rms(total, hidden, eps);
+    const float inv = inv_rms(total, inv_n, eps);
 
     const T* again = (kMode == kPlain) ? s : st;
     for (int c = (int)threadIdx.x; c < units; c += kBlock) {
@@ -180,6 +275,36 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
     const bool vec = (hidden % 8 == 0) && aligned16(src) && aligned16(state) &&
                      aligned16(weight) && aligned16(normed);
     const int nchunks = hidden / 8;
+    const float inv_n = 1.0f / (float)hidden;
+    static const bool use_wave = [] {
+        const char* e = getenv("VV_HIP_ROWS");
+        return e && e[0] == 'w' && e[1] == 'a';       // VV_HIP_ROWS=wave: A/B aid
+    }();
+    if (vec && !use_wave && nchunks <= 3 * kMaxWgThreads) {
+        const int cpt = (nchunks + kMaxWgThreads - 1) / kMaxWgThreads;
+        int threads = ((nchunks + cpt - 1) / cpt + kWave - 1) / kWave * kWave;
+        const size_t tensors = kMode == kAdd ? 4 : (kMode == kGather ? 3 : 2);
+        const bool stream = use_streaming(tensors * (size_t)rows * (size_t)hidden * 2u);
+        const Chunk* s = static_cast<const Chunk*>(src);
+        Chunk* stt = static_cast<Chunk*>(state);
+        const Chunk* w = static_cast<const Chunk*>(weight);
+        Chunk* o = static_cast<Chunk*>(normed);
+        const dim3 grid((unsigned)rows);
+        const bool full = nchunks == cpt * threads;
+#define VV_WG_LAUNCH(C, S, F) \
+    norm_rows_wg<C, kMode, S, F><<<grid, threads, 0, st>>>(s, stt, ids, w, o, nchunks, inv_n, eps)
+#define VV_WG_CASE(C)                                        \
+    case C:                                                  \
+        if (stream && full)  VV_WG_LAUNCH(C, true, true);    \
+        else if (stream)     VV_WG_LAUNCH(C, true, false);   \
+        else if (full)       VV_WG_LAUNCH(C, false, true);   \
+        else                 VV_WG_LAUNCH(C, false, false);  \
+        break;
+        switch (cpt) { VV_WG_CASE(1) VV_WG_CASE(2) VV_WG_CASE(3) }
+#undef VV_WG_CASE
+#undef VV_WG_LAUNCH
+        return launch_status();
+    }
     if (vec && nchunks <= 8 * kWave) {
         const Chunk* s = static_cast<const Chunk*>(src);
         Chunk* stt = static_cast<Chunk*>(state);
@@ -192,7 +317,7 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         const size_t tensors = kMode == kAdd ? 4 : (kMode == kGather ? 3 : 2);
         const bool stream = use_streaming(tensors * (size_t)rows * (size_t)hidden * 2u);
 #define VV_ROWS_LAUNCH(N, F, S) \
-    norm_rows_wave<N, kMode, F, S><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, nchunks, eps)
+    norm_rows_wave<N, kMode, F, S><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, nchunks, inv_n, eps)
 #define VV_ROWS_CASE(N)                                       \
     case N:                                                   \
         if (full && stream)       VV_ROWS_LAUNCH(N, true, true);   \
@@ -211,11 +336,11 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
     if (vec) {
         norm_rows_block<kMode, Chunk><<<dim3((unsigned)rows), kBlock, 0, st>>>(
             static_cast<const Chunk*>(src), static_cast<Chunk*>(state), ids,
-            static_cast<const Chunk*>(weight), static_cast<Chunk*>(normed), nchunks, hidden, eps);
+            static_cast<const Chunk*>(weight), static_cast<Chunk*>(normed), nchunks, inv_n, eps);
     } else {
         norm_rows_block<kMode, h16><<<dim3((unsigned)rows), kBlock, 0, st>>>(
             static_cast<const h16*>(src), static_cast<h16*>(state), ids,
-            static_cast<const h16*>(weight), static_cast<h16*>(normed), hidden, hidden, eps);
+            static_cast<const h16*>(weight), static_cast<h16*>(normed), hidden, inv_n, eps);
     }
     return launch_status();
 }
