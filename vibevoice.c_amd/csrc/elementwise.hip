@@ -1,19 +1,21 @@
 // Flat elementwise kernels: SwiGLU, residual add, bias add, FP32 <-> FP16.
 //
 // Each is a single pass over contiguous FP16 data, bound by HBM bandwidth. A
-// thread moves kUnroll 16-byte chunks per input, all of its loads issued before
-// the first use, the chunks of one instruction contiguous across the wave
-// (64 lanes x 16 B = 1 KiB per load instruction). Every thread reads all of its
-// chunks before it writes any of them and no other thread touches those
-// chunks, so an output that aliases an input exactly (out == gate, the way the
-// decoder calls SwiGLU) is safe. Unaligned pointers take a 2-byte kernel.
+// thread moves ONE 16-byte chunk per input and a workgroup is ONE wave: the
+// chunks of a load instruction are contiguous across the wave (64 lanes x 16 B
+// = 1 KiB), and the grid is as many light, short-lived waves as there are KiB.
+// Measured for SwiGLU at T = 14449 (1.64 GB per launch): 1 chunk/thread in
+// 64-thread workgroups 84.3 % of the HBM peak, in 256-thread workgroups 82.7 %,
+// 4 chunks/thread in 256-thread workgroups 75.9-79.6 %. Every thread reads its
+// chunk before it writes it and no other thread touches that chunk, so an
+// output that aliases an input exactly (out == gate, the way the decoder calls
+// SwiGLU) is safe. Unaligned pointers take a 2-byte kernel.
 #include "vv_common.hpp"
 
 namespace vv {
 namespace {
 
-constexpr int kUnroll = 4;                       // chunks per thread per input
-constexpr int kChunksPerBlock = kBlock * kUnroll;
+constexpr int kEwBlock = kWave;                  // one wave per workgroup
 
 // silu(g) * u in the oracle's association, (g / (1 + e^-g)) * u, with the
 // hardware exponential and reciprocal: exp2(-g * log2 e) and rcp are each
@@ -44,31 +46,14 @@ __device__ __forceinline__ h16 apply2(h16 a, h16 b) {
 
 // out[i] = op(a[i], b[i]) over nchunks chunks, then the (< 8) trailing halves.
 template <int kOp, bool kStream>
-__global__ __launch_bounds__(kBlock) void binary_chunks(const Chunk* a, const Chunk* b,
-                                                        Chunk* out, size_t nchunks,
-                                                        int tail_halves) {
-    const size_t base = (size_t)blockIdx.x * kChunksPerBlock + threadIdx.x;
-    Chunk va[kUnroll], vb[kUnroll];
-    if (base + (size_t)(kUnroll - 1) * kBlock < nchunks) {
-#pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            va[j] = load_chunk_as<kStream>(a + base + (size_t)j * kBlock);
-            vb[j] = load_chunk_as<kStream>(b + base + (size_t)j * kBlock);
-        }
-#pragma unroll
-        for (int j = 0; j < kUnroll; ++j)
-            store_chunk_as<kStream>(out + base + (size_t)j * kBlock, apply2<kOp>(va[j], vb[j]));
-    } else {
-#pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            const size_t c = base + (size_t)j * kBlock;
-            if (c < nchunks) { va[j] = load_chunk(a + c); vb[j] = load_chunk(b + c); }
-        }
-#pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            const size_t c = base + (size_t)j * kBlock;
-            if (c < nchunks) store_chunk(out + c, apply2<kOp>(va[j], vb[j]));
-        }
+__global__ __launch_bounds__(kEwBlock) void binary_chunks(const Chunk* a, const Chunk* b,
+                                                          Chunk* out, size_t nchunks,
+                                                          int tail_halves) {
+    const size_t c = (size_t)blockIdx.x * kEwBlock + threadIdx.x;
+    if (c < nchunks) {
+        const Chunk va = load_chunk_as<kStream>(a + c);
+        const Chunk vb = load_chunk_as<kStream>(b + c);
+        store_chunk_as<kStream>(out + c, apply2<kOp>(va, vb));
     }
     if (tail_halves > 0 && blockIdx.x == 0 && (int)threadIdx.x < tail_halves) {
         const h16* ta = reinterpret_cast<const h16*>(a + nchunks);
@@ -91,13 +76,13 @@ vv_status_t launch_binary(const void* a, const void* b, void* out, size_t n, hip
     if (aligned16(a) && aligned16(b) && aligned16(out)) {
         const size_t nchunks = n / 8;
         const int tail = (int)(n % 8);
-        const size_t blocks = nchunks ? (nchunks + kChunksPerBlock - 1) / kChunksPerBlock : 1;
+        const size_t blocks = nchunks ? (nchunks + kEwBlock - 1) / kEwBlock : 1;
         if (use_streaming(3u * n * 2u))
-            binary_chunks<kOp, true><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
+            binary_chunks<kOp, true><<<dim3((unsigned)blocks), kEwBlock, 0, st>>>(
                 static_cast<const Chunk*>(a), static_cast<const Chunk*>(b),
                 static_cast<Chunk*>(out), nchunks, tail);
         else
-            binary_chunks<kOp, false><<<dim3((unsigned)blocks), kBlock, 0, st>>>(
+            binary_chunks<kOp, false><<<dim3((unsigned)blocks), kEwBlock, 0, st>>>(
                 static_cast<const Chunk*>(a), static_cast<const Chunk*>(b),
                 static_cast<Chunk*>(out), nchunks, tail);
     } else {
@@ -108,55 +93,37 @@ vv_status_t launch_binary(const void* a, const void* b, void* out, size_t n, hip
     return launch_status();
 }
 
-// gate and up are the two halves of each [2*inter] row. One workgroup column
-// per row (blockIdx.y), chunks of the row spread over blockIdx.x.
-__global__ __launch_bounds__(kBlock) void swiglu_fused_chunks(const Chunk* gate_up, Chunk* out,
-                                                              int inter_chunks) {
-    const size_t row = blockIdx.y;
-    const Chunk* g = gate_up + row * 2u * (size_t)inter_chunks;
-    const Chunk* u = g + inter_chunks;
-    Chunk* o = out + row * (size_t)inter_chunks;
-    const int base = (int)blockIdx.x * kChunksPerBlock + (int)threadIdx.x;
-    Chunk vg[kUnroll], vu[kUnroll];
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-        const int c = base + j * kBlock;
-        if (c < inter_chunks) { vg[j] = load_chunk(g + c); vu[j] = load_chunk(u + c); }
-    }
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-        const int c = base + j * kBlock;
-        if (c < inter_chunks) store_chunk(o + c, apply2<kSwiglu>(vg[j], vu[j]));
+// gate and up are the two halves of each [2*inter] row; flat over the output.
+__global__ __launch_bounds__(kEwBlock) void swiglu_fused_chunks(const Chunk* gate_up, Chunk* out,
+                                                                size_t total_chunks,
+                                                                int inter_chunks) {
+    const size_t c = (size_t)blockIdx.x * kEwBlock + threadIdx.x;
+    if (c < total_chunks) {
+        const size_t row = c / (size_t)inter_chunks, col = c - row * (size_t)inter_chunks;
+        const Chunk* g = gate_up + row * 2u * (size_t)inter_chunks + col;
+        store_chunk(out + c, apply2<kSwiglu>(load_chunk(g), load_chunk(g + inter_chunks)));
     }
 }
 
 __global__ __launch_bounds__(kBlock) void swiglu_fused_halves(const h16* gate_up, h16* out,
-                                                              int inter) {
-    const size_t row = blockIdx.y;
-    const int c = (int)blockIdx.x * kBlock + (int)threadIdx.x;
-    if (c >= inter) return;
-    const h16* g = gate_up + row * 2u * (size_t)inter;
-    out[row * (size_t)inter + c] = apply2<kSwiglu>(g[c], g[inter + c]);
+                                                              size_t total, int inter) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < total) {
+        const size_t row = i / (size_t)inter, col = i - row * (size_t)inter;
+        const h16* g = gate_up + row * 2u * (size_t)inter + col;
+        out[i] = apply2<kSwiglu>(g[0], g[inter]);
+    }
 }
 
 // out[m, :] += bias[:]. Chunked form: a row is n_chunks chunks, the bias chunk
 // index is the chunk's column, found with one 64-bit modulo per chunk.
-__global__ __launch_bounds__(kBlock) void bias_add_chunks(Chunk* out, const Chunk* __restrict__ bias,
-                                                          size_t total_chunks, int row_chunks) {
-    const size_t base = (size_t)blockIdx.x * kChunksPerBlock + threadIdx.x;
-    Chunk v[kUnroll];
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-        const size_t c = base + (size_t)j * kBlock;
-        if (c < total_chunks) v[j] = load_chunk(out + c);
-    }
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-        const size_t c = base + (size_t)j * kBlock;
-        if (c < total_chunks) {
-            const Chunk bv = load_chunk(bias + (c % (size_t)row_chunks));
-            store_chunk(out + c, apply2<kResidual>(v[j], bv));
-        }
+__global__ __launch_bounds__(kEwBlock) void bias_add_chunks(Chunk* out, const Chunk* __restrict__ bias,
+                                                            size_t total_chunks, int row_chunks) {
+    const size_t c = (size_t)blockIdx.x * kEwBlock + threadIdx.x;
+    if (c < total_chunks) {
+        const Chunk v = load_chunk(out + c);
+        const Chunk bv = load_chunk(bias + (c % (size_t)row_chunks));
+        store_chunk(out + c, apply2<kResidual>(v, bv));
     }
 }
 
@@ -202,16 +169,17 @@ vv_status_t vv_swiglu_fused_dev(const void* gate_up, void* output, int rows, int
     if (!gate_up || !output) return VV_ERR_NULL_PTR;
     if (rows <= 0 || inter <= 0) return VV_OK;
     hipStream_t st = vv::as_stream(stream);
+    const size_t total = (size_t)rows * (size_t)inter;
     if (inter % 8 == 0 && vv::aligned16(gate_up) && vv::aligned16(output)) {
-        const int ic = inter / 8;
-        const dim3 grid((unsigned)((ic + vv::kChunksPerBlock - 1) / vv::kChunksPerBlock),
-                        (unsigned)rows);
-        vv::swiglu_fused_chunks<<<grid, vv::kBlock, 0, st>>>(
-            static_cast<const vv::Chunk*>(gate_up), static_cast<vv::Chunk*>(output), ic);
+        const size_t chunks = total / 8;
+        vv::swiglu_fused_chunks<<<dim3((unsigned)((chunks + vv::kEwBlock - 1) / vv::kEwBlock)),
+                                  vv::kEwBlock, 0, st>>>(
+            static_cast<const vv::Chunk*>(gate_up), static_cast<vv::Chunk*>(output), chunks,
+            inter / 8);
     } else {
-        const dim3 grid((unsigned)((inter + vv::kBlock - 1) / vv::kBlock), (unsigned)rows);
-        vv::swiglu_fused_halves<<<grid, vv::kBlock, 0, st>>>(
-            static_cast<const vv::h16*>(gate_up), static_cast<vv::h16*>(output), inter);
+        vv::swiglu_fused_halves<<<dim3((unsigned)((total + vv::kBlock - 1) / vv::kBlock)),
+                                  vv::kBlock, 0, st>>>(
+            static_cast<const vv::h16*>(gate_up), static_cast<vv::h16*>(output), total, inter);
     }
     return vv::launch_status();
 }
@@ -223,8 +191,8 @@ vv_status_t vv_bias_add_dev(void* output, const void* bias, int M, int N, void* 
     const size_t total = (size_t)M * (size_t)N;
     if (N % 8 == 0 && vv::aligned16(output) && vv::aligned16(bias)) {
         const size_t chunks = total / 8;
-        const size_t blocks = (chunks + vv::kChunksPerBlock - 1) / vv::kChunksPerBlock;
-        vv::bias_add_chunks<<<dim3((unsigned)blocks), vv::kBlock, 0, st>>>(
+        const size_t blocks = (chunks + vv::kEwBlock - 1) / vv::kEwBlock;
+        vv::bias_add_chunks<<<dim3((unsigned)blocks), vv::kEwBlock, 0, st>>>(
             static_cast<vv::Chunk*>(output), static_cast<const vv::Chunk*>(bias), chunks, N / 8);
     } else {
         const size_t blocks = (total + vv::kBlock - 1) / vv::kBlock;

@@ -1,13 +1,19 @@
 // Row kernels: RMSNorm, residual-add + RMSNorm, embedding gather (+ RMSNorm).
 //
 // All of them stream [rows, hidden] FP16 once and are bound by HBM bandwidth.
-// Layout of the fast path: ONE WAVE OWNS ONE ROW and keeps it in registers
-// (hidden = 3584 is 448 16-byte chunks = 7 per lane), so the row is read from
-// memory exactly once, the sum of squares is reduced across the 64 lanes with
-// DPP permutes, and no LDS and no barrier are involved. A 256-thread workgroup
-// is four independent rows. Rows that do not fit that shape (hidden not a
-// multiple of 8, wider than 4096, or unaligned pointers) take a
-// workgroup-per-row kernel with a two-pass loop.
+// Layout of the fast path: ONE WORKGROUP OWNS ONE ROW (or two), ONE 16-BYTE
+// CHUNK PER THREAD, the chunk kept in registers between the sum-of-squares pass
+// and the scaling pass, so a row is read from memory exactly once. hidden =
+// 3584 is 448 chunks = a 448-thread workgroup of 7 waves. The sum of squares
+// is reduced inside each wave with DPP permutes, across the waves through 7
+// floats of LDS and one barrier. Rows wider than 1024 chunks use 2 or 3 chunks
+// per thread; widths that are not a multiple of 8, rows wider than 3072
+// chunks, or unaligned pointers take a two-pass workgroup-per-row kernel.
+//
+// Why light threads: on MI355X a copy with this structure moves 6.4 TB/s for
+// the add+norm traffic pattern, one with a whole row per wave (7 chunks per
+// lane, 14 loads in flight per lane, no LDS) 5.8 TB/s; the measured kernels
+// follow (add+norm 66.6 vs 71.0 us at 14449 rows).
 #include "vv_common.hpp"
 
 namespace vv {
@@ -29,99 +35,6 @@ __device__ __forceinline__ float inv_rms(float sumsq, float inv_n, float eps) {
     return __builtin_amdgcn_rsqf(sumsq * inv_n + eps);
 }
 
-// ── one wave per row, row held in registers ──────────────────────────────
-// kCpl = chunks per lane (row width <= 512 * kCpl halves); kFull = the row is
-// exactly 64 * kCpl chunks, so no lane is ever idle and loads are unpredicated.
-template <int kCpl, int kMode, bool kFull, bool kStream>
-__global__ __launch_bounds__(kBlock) void norm_rows_wave(
-    const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
-    const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float inv_n,
-    float eps) {
-    const int row = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
-    if (row >= rows) return;
-    const int lane = lane_id();
-
-    size_t src_row = (size_t)row;
-    if (kMode == kGather || kMode == kGatherOnly)
-        src_row = (size_t)__builtin_amdgcn_readfirstlane(ids[row]);
-    const Chunk* s = src + src_row * (size_t)nchunks;
-    const size_t out_base = (size_t)row * (size_t)nchunks;
-
-    // Issue every load of the row before the first use: kCpl (or 2*kCpl)
-    // independent 16-byte loads in flight per lane. Gathered table rows are
-    // read with ordinary loads even in streaming launches: measured on MI355X,
-    // a row gather with streaming loads runs 10 % slower (5.3 vs 5.9 TB/s for
-    // gather + two outputs), and a table row may well be needed again.
-    constexpr bool kStreamSrc = kStream && !(kMode == kGather || kMode == kGatherOnly);
-    Chunk a[kCpl];
-    Chunk b[kCpl];
-#pragma unroll
-    for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (kFull || c < nchunks) {
-            a[j] = load_chunk_as<kStreamSrc>(s + c);
-            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
-        }
-    }
-
-    if (kMode == kGatherOnly) {
-#pragma unroll
-        for (int j = 0; j < kCpl; ++j) {
-            const int c = j * kWave + lane;
-            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
-        }
-        return;
-    }
-
-    Chunk w[kCpl];
-#pragma unroll
-    for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (kFull || c < nchunks) w[j] = load_chunk(weight + c);
-    }
-
-    float acc = 0.0f;
-#pragma unroll
-    for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (kFull || c < nchunks) {
-            f32x8 x = unpack(a[j]);
-            if (kMode == kAdd) {
-                const f32x8 r = unpack(b[j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) x[i] = r[i] + x[i];
-                // The stored residual is the FP16 rounding of the sum, and the
-                // norm reads that rounded value (what add-then-norm would see).
-                a[j] = pack(x);
-                x = unpack(a[j]);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
-        }
-    }
-    if (kMode == kAdd || kMode == kGather) {
-#pragma unroll
-        for (int j = 0; j < kCpl; ++j) {
-            const int c = j * kWave + lane;
-            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
-        }
-    }
-
-    const float inv = inv_rms(wave_sum(acc), inv_n, eps);
-
-#pragma unroll
-    for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (kFull || c < nchunks) {
-            f32x8 x = unpack(a[j]);
-            const f32x8 g = unpack(w[j]);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
-            store_chunk_as<kStream>(normed + out_base + c, pack(x));
-        }
-    }
-}
-
 // ── one workgroup per row, one chunk per thread ──────────────────────────
 // blockDim = the row's chunk count rounded up to whole waves (448 threads = 7
 // waves for hidden 3584), kCpt chunks per thread for rows wider than 1024
@@ -132,78 +45,100 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
 // through LDS and a single barrier.
 constexpr int kMaxWgThreads = 1024;
 
-template <int kCpt, int kMode, bool kStream, bool kFull>   // kFull: nchunks == kCpt * blockDim.x
+template <int kCpt, int kRows, int kMode, bool kStream, bool kFull>   // kFull: nchunks == kCpt * blockDim.x
 __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
     const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
-    const Chunk* __restrict__ weight, Chunk* normed, int nchunks, float inv_n, float eps) {
-    __shared__ float partial[kMaxWgThreads / kWave];
-    const size_t row = blockIdx.x;
+    const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float inv_n,
+    float eps) {
+    __shared__ float partial[kRows][kMaxWgThreads / kWave];
     const int t = (int)threadIdx.x;
     const int nthreads = (int)blockDim.x;
+    const int row0 = (int)blockIdx.x * kRows;
+    constexpr bool kGathers = kMode == kGather || kMode == kGatherOnly;
+    constexpr bool kStreamSrc = kStream && !kGathers;
 
-    size_t src_row = row;
-    if (kMode == kGather || kMode == kGatherOnly) src_row = (size_t)ids[row];
-    const Chunk* s = src + src_row * (size_t)nchunks;
-    const size_t out_base = row * (size_t)nchunks;
-    constexpr bool kStreamSrc = kStream && !(kMode == kGather || kMode == kGatherOnly);
-
-    Chunk a[kCpt], b[kCpt], w[kCpt];
+    // kRows consecutive rows share the workgroup: one weight load serves them
+    // all, and their loads are all in flight before the first use. A row past
+    // the end (odd row count) re-reads the last row and is not stored.
+    Chunk a[kRows][kCpt], b[kRows][kCpt], w[kCpt];
+    bool live[kRows];
+    size_t out_base[kRows];
 #pragma unroll
-    for (int j = 0; j < kCpt; ++j) {
-        const int c = j * nthreads + t;
-        if (kFull || c < nchunks) {
-            a[j] = load_chunk_as<kStreamSrc>(s + c);
-            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
-            if (kMode != kGatherOnly) w[j] = load_chunk(weight + c);
+    for (int r = 0; r < kRows; ++r) {
+        live[r] = kRows == 1 || row0 + r < rows;
+        const int row = live[r] ? row0 + r : rows - 1;
+        const size_t src_row = kGathers ? (size_t)ids[row] : (size_t)row;
+        const Chunk* s = src + src_row * (size_t)nchunks;
+        out_base[r] = (size_t)row * (size_t)nchunks;
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            if (kFull || c < nchunks) {
+                a[r][j] = load_chunk_as<kStreamSrc>(s + c);
+                if (kMode == kAdd) b[r][j] = load_chunk_as<kStream>(state + out_base[r] + c);
+            }
         }
     }
     if (kMode == kGatherOnly) {
 #pragma unroll
-        for (int j = 0; j < kCpt; ++j) {
-            const int c = j * nthreads + t;
-            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
-        }
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int j = 0; j < kCpt; ++j) {
+                const int c = j * nthreads + t;
+                if ((kFull || c < nchunks) && live[r])
+                    store_chunk_as<kStream>(state + out_base[r] + c, a[r][j]);
+            }
         return;
     }
-
-    float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < kCpt; ++j) {
         const int c = j * nthreads + t;
-        if (kFull || c < nchunks) {
-            f32x8 x = unpack(a[j]);
-            if (kMode == kAdd) {
-                const f32x8 r = unpack(b[j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) x[i] = r[i] + x[i];
-                // stored residual = FP16 rounding of the sum; the norm reads that value
-                a[j] = pack(x);
-                x = unpack(a[j]);
-            }
-            if (kMode == kAdd || kMode == kGather)
-                store_chunk_as<kStream>(state + out_base + c, a[j]);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
-        }
+        if (kFull || c < nchunks) w[j] = load_chunk(weight + c);
     }
 
-    acc = wave_sum(acc);
-    if (lane_id() == 0) partial[t >> 6] = acc;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            if (kFull || c < nchunks) {
+                f32x8 x = unpack(a[r][j]);
+                if (kMode == kAdd) {
+                    const f32x8 res = unpack(b[r][j]);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) x[i] = res[i] + x[i];
+                    // stored residual = FP16 rounding of the sum; the norm reads that value
+                    a[r][j] = pack(x);
+                    x = unpack(a[r][j]);
+                }
+                if ((kMode == kAdd || kMode == kGather) && live[r])
+                    store_chunk_as<kStream>(state + out_base[r] + c, a[r][j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
+            }
+        }
+        acc = wave_sum(acc);
+        if (lane_id() == 0) partial[r][t >> 6] = acc;
+    }
     __syncthreads();
-    float total = 0.0f;
     const int nwaves = nthreads >> 6;
-    for (int i = 0; i < nwaves; ++i) total += partial[i];
-    const float inv = inv_rms(total, inv_n, eps);
 
 #pragma unroll
-    for (int j = 0; j < kCpt; ++j) {
-        const int c = j * nthreads + t;
-        if (kFull || c < nchunks) {
-            f32x8 x = unpack(a[j]);
-            const f32x8 g = unpack(w[j]);
+    for (int r = 0; r < kRows; ++r) {
+        float total = 0.0f;
+        for (int i = 0; i < nwaves; ++i) total += partial[r][i];
+        const float inv = inv_rms(total, inv_n, eps);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
-            store_chunk_as<kStream>(normed + out_base + c, pack(x));
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            if ((kFull || c < nchunks) && live[r]) {
+                f32x8 x = unpack(a[r][j]);
+                const f32x8 g = unpack(w[j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
+                store_chunk_as<kStream>(normed + out_base[r] + c, pack(x));
+            }
         }
     }
 }
@@ -276,11 +211,7 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
                      aligned16(weight) && aligned16(normed);
     const int nchunks = hidden / 8;
     const float inv_n = 1.0f / (float)hidden;
-    static const bool use_wave = [] {
-        const char* e = getenv("VV_HIP_ROWS");
-        return e && e[0] == 'w' && e[1] == 'a';       // VV_HIP_ROWS=wave: A/B aid
-    }();
-    if (vec && !use_wave && nchunks <= 3 * kMaxWgThreads) {
+    if (vec && nchunks <= 3 * kMaxWgThreads) {
         const int cpt = (nchunks + kMaxWgThreads - 1) / kMaxWgThreads;
         int threads = ((nchunks + cpt - 1) / cpt + kWave - 1) / kWave * kWave;
         const size_t tensors = kMode == kAdd ? 4 : (kMode == kGather ? 3 : 2);
@@ -289,48 +220,35 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         Chunk* stt = static_cast<Chunk*>(state);
         const Chunk* w = static_cast<const Chunk*>(weight);
         Chunk* o = static_cast<Chunk*>(normed);
-        const dim3 grid((unsigned)rows);
         const bool full = nchunks == cpt * threads;
-#define VV_WG_LAUNCH(C, S, F) \
-    norm_rows_wg<C, kMode, S, F><<<grid, threads, 0, st>>>(s, stt, ids, w, o, nchunks, inv_n, eps)
-#define VV_WG_CASE(C)                                        \
-    case C:                                                  \
-        if (stream && full)  VV_WG_LAUNCH(C, true, true);    \
-        else if (stream)     VV_WG_LAUNCH(C, true, false);   \
-        else if (full)       VV_WG_LAUNCH(C, false, true);   \
-        else                 VV_WG_LAUNCH(C, false, false);  \
-        break;
-        switch (cpt) { VV_WG_CASE(1) VV_WG_CASE(2) VV_WG_CASE(3) }
-#undef VV_WG_CASE
+        // Two rows per workgroup for the narrow (one chunk per thread) case once there
+        // are enough rows to fill the chip several times over; VV_HIP_ROWS_PER_WG=1|2 forces.
+        static const int forced_rows = [] {
+            const char* e = getenv("VV_HIP_ROWS_PER_WG");
+            return (e && (e[0] == '1' || e[0] == '2')) ? e[0] - '0' : 0;
+        }();
+        // Measured at T = 14449, hidden 3584: two rows per workgroup is faster for the
+        // one-input modes (norm 37.3 -> 34.6 us, gather+norm 58.8 -> 55.2 us) and
+        // slightly slower for add+norm (66.6 -> 67.5 us), which already has two loads
+        // per thread in flight.
+        const int rpw = forced_rows ? forced_rows
+                                    : ((cpt == 1 && rows >= 4096 && kMode != kAdd) ? 2 : 1);
+        const bool two = rpw == 2 && cpt == 1;
+        const dim3 grid((unsigned)(two ? (rows + 1) / 2 : rows));
+#define VV_WG_LAUNCH(C, R, S, F)                                                          \
+    norm_rows_wg<C, R, kMode, S, F><<<grid, threads, 0, st>>>(s, stt, ids, w, o, rows, nchunks, \
+                                                              inv_n, eps)
+#define VV_WG_PICK(C, R)                                     \
+        if (stream && full)  VV_WG_LAUNCH(C, R, true, true);    \
+        else if (stream)     VV_WG_LAUNCH(C, R, true, false);   \
+        else if (full)       VV_WG_LAUNCH(C, R, false, true);   \
+        else                 VV_WG_LAUNCH(C, R, false, false);
+        if (two) { VV_WG_PICK(1, 2) }
+        else if (cpt == 1) { VV_WG_PICK(1, 1) }
+        else if (cpt == 2) { VV_WG_PICK(2, 1) }
+        else { VV_WG_PICK(3, 1) }
+#undef VV_WG_PICK
 #undef VV_WG_LAUNCH
-        return launch_status();
-    }
-    if (vec && nchunks <= 8 * kWave) {
-        const Chunk* s = static_cast<const Chunk*>(src);
-        Chunk* stt = static_cast<Chunk*>(state);
-        const Chunk* w = static_cast<const Chunk*>(weight);
-        Chunk* o = static_cast<Chunk*>(normed);
-        const dim3 grid((unsigned)((rows + kWavesPerBlock - 1) / kWavesPerBlock));
-        const int cpl = (nchunks + kWave - 1) / kWave;
-        const bool full = nchunks == cpl * kWave;
-        // bytes this launch streams: 2 tensors (plain, gather-only), 3 (gather+norm), 4 (add+norm)
-        const size_t tensors = kMode == kAdd ? 4 : (kMode == kGather ? 3 : 2);
-        const bool stream = use_streaming(tensors * (size_t)rows * (size_t)hidden * 2u);
-#define VV_ROWS_LAUNCH(N, F, S) \
-    norm_rows_wave<N, kMode, F, S><<<grid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, nchunks, inv_n, eps)
-#define VV_ROWS_CASE(N)                                       \
-    case N:                                                   \
-        if (full && stream)       VV_ROWS_LAUNCH(N, true, true);   \
-        else if (full)            VV_ROWS_LAUNCH(N, true, false);  \
-        else if (stream)          VV_ROWS_LAUNCH(N, false, true);  \
-        else                      VV_ROWS_LAUNCH(N, false, false); \
-        break;
-        switch (cpl) {
-            VV_ROWS_CASE(1) VV_ROWS_CASE(2) VV_ROWS_CASE(3) VV_ROWS_CASE(4)
-            VV_ROWS_CASE(5) VV_ROWS_CASE(6) VV_ROWS_CASE(7) VV_ROWS_CASE(8)
-        }
-#undef VV_ROWS_CASE
-#undef VV_ROWS_LAUNCH
         return launch_status();
     }
     if (vec) {

@@ -66,16 +66,19 @@ __device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
 
 // head_dim == 128, 16-byte aligned tensors, at most kMaxFastHeads heads in all.
 //
-// A workgroup owns `posb` consecutive positions (4 when Q+K is 32 heads). Work
-// item = (position, head, chunk pair); thread t takes items t, t+256, ... — at
-// most kItems of them. Order inside the kernel: issue every global load of the
+// A workgroup owns `posb` consecutive positions. Work item = (position, head,
+// chunk pair); thread t takes items t, t+256, ... — kItems of them. For the
+// 32 heads of Qwen2-7B's Q+K that is one position per workgroup and ONE item
+// per thread: measured at T = 14449, 1 / 2 / 4 items per thread give 38.3 /
+// 39.4 / 40.9 us — the memory system rewards many light workgroups — so more
+// items per thread are used only when a position has more than 256 of them. Order inside the kernel: issue every global load of the
 // thread's items first, THEN compute the cos/sin table (one (position, pair)
 // per thread, full-range sincosf) and cross the barrier, so the memory latency
 // runs under the transcendental work; then rotate and store.
-constexpr int kItems = 4;
-constexpr int kMaxFastHeads = kItems * kBlock / 8;   // 128: one position per workgroup
+constexpr int kMaxItems = 4;
+constexpr int kMaxFastHeads = kMaxItems * kBlock / 8;   // 128: one position per workgroup
 
-template <bool kBias, bool kStream, bool kExact>   // kExact: 32 heads, 256 items per position
+template <bool kBias, bool kStream, bool kExact, int kItems>   // kExact: 32 heads, 256 items per position
 __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs, int posb) {
     __shared__ __attribute__((aligned(16))) float cs_cos[kPosPerBlock][64];
     __shared__ __attribute__((aligned(16))) float cs_sin[kPosPerBlock][64];
@@ -241,19 +244,34 @@ vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias
                       (!a.q || aligned16(a.q)) && (!a.k || aligned16(a.k)) &&
                       (!a.q_bias || aligned16(a.q_bias)) && (!a.k_bias || aligned16(a.k_bias));
     if (fast) {
-        // as many positions per workgroup as kItems items per thread allow, at most 4
-        int posb = kItems * kBlock / ((nq + nk) * 8);
+        // items per thread: enough for one position, then as many positions per
+        // workgroup as fit (at most kPosPerBlock); VV_ROPE_ITEMS=1|2|4 forces (A/B aid)
+        static const int forced_items = getenv("VV_ROPE_ITEMS") ? atoi(getenv("VV_ROPE_ITEMS")) : 0;
+        const int tasks = (nq + nk) * 8;
+        int items = forced_items ? forced_items : 1;
+        while (items * kBlock < tasks) items *= 2;          // <= kMaxItems by the head limit
+        if (items == 3) items = 4;
+        int posb = items * kBlock / tasks;
         if (posb > kPosPerBlock) posb = kPosPerBlock;
+        if (posb < 1) posb = 1;
         const dim3 grid((unsigned)((rows + posb - 1) / posb));
         const bool stream = use_streaming(2u * (size_t)rows * (size_t)(nq + nk) * 128u * 2u);
         const bool exact = (nq + nk) * 8 == kBlock;
-#define VV_ROPE_LAUNCH(B, S, E) rope128<B, S, E><<<grid, kBlock, 0, st>>>(a, freqs, posb)
-#define VV_ROPE_PICK(B, S) (exact ? VV_ROPE_LAUNCH(B, S, true) : VV_ROPE_LAUNCH(B, S, false))
+#define VV_ROPE_LAUNCH(B, S, E, I) rope128<B, S, E, I><<<grid, kBlock, 0, st>>>(a, freqs, posb)
+#define VV_ROPE_ITEMS(B, S, E)                          \
+    do {                                                \
+        if (items == 1)      VV_ROPE_LAUNCH(B, S, E, 1); \
+        else if (items == 2) VV_ROPE_LAUNCH(B, S, E, 2); \
+        else                 VV_ROPE_LAUNCH(B, S, E, 4); \
+    } while (0)
+#define VV_ROPE_PICK(B, S) \
+    do { if (exact) VV_ROPE_ITEMS(B, S, true); else VV_ROPE_ITEMS(B, S, false); } while (0)
         if (has_bias && stream)  VV_ROPE_PICK(true, true);
         else if (has_bias)       VV_ROPE_PICK(true, false);
         else if (stream)         VV_ROPE_PICK(false, true);
         else                     VV_ROPE_PICK(false, false);
 #undef VV_ROPE_PICK
+#undef VV_ROPE_ITEMS
 #undef VV_ROPE_LAUNCH
     } else {
         rope_generic<<<dim3((unsigned)rows), kBlock, 0, st>>>(a, freqs);
