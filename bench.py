@@ -60,15 +60,15 @@ def algorithmic_bytes(T: int) -> dict:
 class Workload:
     """Device buffers for `nsets` rotating copies of the step's tensors."""
 
-    def __init__(self, torch, dev, T: int, nsets: int):
+    def __init__(self, torch, dev, T: int, nsets: int, table=None, weight=None):
         self.torch, self.dev, self.T, self.nsets = torch, dev, T, nsets
         gen = torch.Generator(device="cuda").manual_seed(0)
 
         def randn(*shape, std=1.0, mean=0.0):
             return (torch.randn(*shape, generator=gen, device="cuda") * std + mean).half()
 
-        self.table = randn(V, H, std=0.02)
-        self.weight = randn(H, std=0.1, mean=1.0)
+        self.table = table if table is not None else randn(V, H, std=0.02)
+        self.weight = weight if weight is not None else randn(H, std=0.1, mean=1.0)
         self.sets = []
         for s in range(nsets):
             d = {
@@ -318,6 +318,16 @@ def main() -> int:
             log(f"  {name:12s} {med * 1e6:9.2f} us  {unfused[name]['GBps']:8.1f} GB/s  "
                 f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (unfused form)")
 
+    # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
+    decode = {}
+    if not args.only:
+        wl1 = Workload(torch, dev, 1, 1, table=wl.table, weight=wl.weight)
+        for name in KERNELS:
+            best, med = time_kernel(torch, wl1, name, 200, 3, st)
+            decode[name] = {"us_median": med * 1e6, "bytes": algorithmic_bytes(1)[name]}
+        log("  decode (T=1) us per launch: " +
+            ", ".join(f"{n} {d['us_median']:.2f}" for n, d in decode.items()))
+
     dominant = max(kernels, key=lambda n: bytes_per[n])
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
@@ -342,6 +352,8 @@ def main() -> int:
     }
     if unfused:
         result["unfused"] = unfused
+    if decode:
+        result["decode_T1_us"] = decode
     if not args.no_cpu:
         log(f"cpu baseline on {CPU_SAMPLE_ROWS} rows ...")
         result["cpu_baseline"] = cpu_baseline(CPU_SAMPLE_ROWS)
