@@ -106,3 +106,48 @@ def test_declined_arguments():
     assert dev.vv_dev_host_register(P, 4096) == dev.VV_ERR_UNSUPPORTED
     assert dev.vv_dev_host_register(None, 4096) == dev.VV_ERR_NULL_PTR
     dev.vv_dev_graph_destroy(None)      # no-op, must not crash
+
+
+# ── the declined remainder of the seam ──────────────────────────────────────
+
+STUB_PATH = os.path.join(os.path.dirname(dev.LIB_PATH), "libvibevoice_hip_unsupported.so")
+
+
+def test_unsupported_library_declines_everything_and_overlaps_nothing():
+    import ctypes as C
+    out = subprocess.check_output(["nm", "-D", "--defined-only", STUB_PATH], text=True)
+    stubs = sorted(l.split()[-1] for l in out.splitlines() if " T vv_" in l)
+    assert len(stubs) == 59
+    assert not set(stubs) & set(dev.SIGNATURES)          # no symbol defined twice
+    lib = C.CDLL(STUB_PATH)
+    zero = {"vv_attn_resolve", "vv_attn_decode_shape", "vv_gqa_decode_shape", "vv_attn_scratch_bytes",
+            "vv_gqa_decode_scratch_bytes", "vv_i8_head_argmax_scratch_bytes"}
+    for name in stubs:
+        fn = getattr(lib, name)
+        if name == "vv_gemm_cleanup":
+            fn.restype = None
+            fn()
+        elif name in zero:
+            fn.restype = C.c_size_t
+            assert fn(1, 2, 3) == 0
+        else:
+            fn.restype = C.c_int
+            assert fn(None, None, None, 4, 5, None) == dev.VV_ERR_UNSUPPORTED, name
+
+
+REF_HEADER = "/root/reference/include/vibevoice/device.h"
+
+
+@pytest.mark.skipif(not os.path.exists(REF_HEADER), reason="reference tree not present")
+def test_the_two_libraries_define_every_symbol_of_the_reference_seam():
+    text = re.sub(r"/\*.*?\*/", "", open(REF_HEADER).read(), flags=re.S)
+    wanted = set(re.findall(r"^\s*(?:vv_status_t|int|size_t|void|bool|const char\*)\s+(vv_[a-z0-9_]+)\s*\(",
+                            text, flags=re.M))
+    have = set()
+    for path in (dev.LIB_PATH, STUB_PATH):
+        out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
+        have |= {l.split()[-1] for l in out.splitlines() if " T vv_" in l}
+    assert len(wanted) >= 100 and not (wanted - have), sorted(wanted - have)
+    # what we add beyond the reference's seam: the fused entry points only
+    assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
+                             "vv_embedding_rmsnorm_dev"}

@@ -22,3 +22,19 @@ def test_c_program_links_and_passes():
 def test_c_program_is_built_against_the_public_header():
     src = open(os.path.join(HERE, "c", "abi_layer_ops.c")).read()
     assert '#include "vibevoice_hip.h"' in src and "hip_runtime" not in src
+
+
+REF_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_device_memory_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(REF_EXE),
+                    reason="oracle/_ref/test_device_memory_hip not built (needs the reference tree)")
+def test_reference_own_device_memory_test_passes_on_this_backend():
+    """The reference's tests/test_device_memory.c, compiled unmodified by
+    oracle/Makefile and linked against libvibevoice_hip.so: copies, fills,
+    device-side index, events, pinned memory, graph capture/replay/break."""
+    res = subprocess.run([REF_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-1000:])
+    assert res.returncode == 0, res.stdout[-2000:]
+    assert "all device memory checks passed" in res.stdout and "FAIL" not in res.stdout

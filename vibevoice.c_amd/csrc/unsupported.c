@@ -1,0 +1,71 @@
+/*
+ * unsupported.c — the rest of the accelerator seam, declined.
+ *
+ * vibevoice.c's device.h declares ~100 symbols and a binary links exactly one
+ * backend, so a backend that accelerates only part of the op set still has to
+ * DEFINE every symbol. The contract for an op a backend does not implement is
+ * "return VV_ERR_UNSUPPORTED having launched nothing", which the callers that
+ * have a fallback take (include/vibevoice/device.h:468-470; precedent:
+ * src/metal/metal_stubs.c:1-30, src/device/device_none.c:129-483).
+ *
+ * This file is that remainder for libvibevoice_hip: every device.h symbol the
+ * HIP library does not define (dense/quantised GEMM and GEMV, attention, KV
+ * cache, LM head, VAE, BitNet, int8 activation quantisers). It builds into its
+ * own small library, libvibevoice_hip_unsupported.so, which a full engine link
+ * adds next to libvibevoice_hip.so; the layer-op library's own export list
+ * stays exactly what include/vibevoice_hip.h declares.
+ *
+ * The definitions take no named parameters on purpose: none of them reads an
+ * argument, and under the x86-64 System V calling convention the caller owns
+ * argument setup and cleanup, so one unprototyped definition serves whatever
+ * argument list device.h gives the symbol. Size queries return 0 and shape /
+ * backend queries return 0, as device_none.c does (its vv_attn_resolve answer,
+ * VV_ATTN_FA1, is the enum's zero).
+ */
+#include <stddef.h>
+
+#define VV_ERR_UNSUPPORTED (-7) /* include/vibevoice/types.h:27 */
+
+#define VV_DECLINE(name) int name() { return VV_ERR_UNSUPPORTED; }
+#define VV_ZERO_INT(name) int name() { return 0; }
+#define VV_ZERO_SIZE(name) size_t name() { return 0; }
+
+/* quantised linear layers (device.h:168-294) */
+VV_DECLINE(vv_nf4_gemv_dev)      VV_DECLINE(vv_nf4_gemm_dev)      VV_DECLINE(vv_dequant_nf4_dev)
+VV_DECLINE(vv_awq_gemv_dev)      VV_DECLINE(vv_awq_gemm_dev)      VV_DECLINE(vv_dequant_awq_dev)
+VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_dequant_int8_dev)
+VV_DECLINE(vv_w4a16_gemv_dev)    VV_DECLINE(vv_w4a16_gemv_multi_dev)
+VV_DECLINE(vv_w4a16_gather_dev)  VV_DECLINE(vv_w4a16_gemm_dev)    VV_DECLINE(vv_w4a16_dequant_dev)
+
+/* int8 activations and W8A8 / W4A8 linears (device.h:320-410) */
+VV_DECLINE(vv_act_quant_dev)     VV_DECLINE(vv_rmsnorm_q8_dev)    VV_DECLINE(vv_swiglu_q8_dev)
+VV_DECLINE(vv_col_absmax_dev)    VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)
+VV_DECLINE(vv_i8_linear_multi_dev)
+
+/* dense FP16 GEMM (device.h:423-482) */
+VV_DECLINE(vv_gemm_fp16_dev)     VV_DECLINE(vv_gemm_fp16_tile_dev) VV_DECLINE(vv_skinny_linear_dev)
+VV_DECLINE(vv_gemm_fp16_nn_dev)
+void vv_gemm_cleanup() {}
+
+/* attention and KV cache (device.h:545-700) */
+VV_ZERO_INT(vv_attn_resolve)     VV_ZERO_SIZE(vv_attn_scratch_bytes) VV_ZERO_INT(vv_attn_decode_shape)
+VV_DECLINE(vv_attn_prefill)      VV_DECLINE(vv_attn_decode)
+VV_DECLINE(vv_kv_store_dev)      VV_DECLINE(vv_kv_page_map_dev)
+VV_ZERO_SIZE(vv_gqa_decode_scratch_bytes) VV_ZERO_INT(vv_gqa_decode_shape)
+VV_DECLINE(vv_gqa_attention_decode_dev)   VV_DECLINE(vv_gqa_attention_prefill_cached_dev)
+VV_DECLINE(vv_gqa_attention_prefill_dev)  VV_DECLINE(vv_gqa_attention_decode_q_dev)
+VV_DECLINE(vv_gqa_attention_prefill_q_dev)
+VV_DECLINE(vv_kv_quant_store_dev) VV_DECLINE(vv_kv_dequant_dev)
+
+/* LM head (device.h:707-715) */
+VV_DECLINE(vv_lm_head_gemv_dev)  VV_DECLINE(vv_argmax_dev)
+
+/* Conv-VAE speech encoder (device.h:762-870) */
+VV_DECLINE(vv_vae_conv_dev)      VV_DECLINE(vv_vae_tail_dev)      VV_DECLINE(vv_vae_rms_dev)
+VV_DECLINE(vv_vae_mixer_dev)     VV_DECLINE(vv_vae_im2col_dev)    VV_DECLINE(vv_vae_conv_gemm_dev)
+VV_DECLINE(vv_vae_gemm_nn_dev)   VV_DECLINE(vv_vae_gemm_tn_dev)   VV_DECLINE(vv_vae_f32_to_f16_dev)
+
+/* BitNet (device.h:888-942) */
+VV_DECLINE(vv_act_quant_i8_dev)  VV_DECLINE(vv_ternary_gemm_dev)  VV_DECLINE(vv_i8_gemm_dev)
+VV_DECLINE(vv_i8s_requant_dev)
+VV_ZERO_SIZE(vv_i8_head_argmax_scratch_bytes) VV_DECLINE(vv_i8_head_argmax_dev)
