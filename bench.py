@@ -54,6 +54,9 @@ def algorithmic_bytes(T: int) -> dict:
         "residual_add": 6 * T * H,
         "rope_q": 4 * T * NQ * HD,
         "rope_k": 4 * T * NK * HD,
+        # int8-activation fused forms: FP16 in, int8 + scale + per-32 sums out
+        "rmsnorm_q8": 2 * T * H + 2 * H + T * H + 4 * T + T * H // 8,
+        "swiglu_q8": 4 * T * I_FF + T * I_FF + 4 * T + T * I_FF // 8,
     }
 
 
@@ -86,6 +89,14 @@ class Workload:
             self.sets.append(d)
         torch.cuda.synchronize()
 
+    def q8_buffers(self):
+        if not hasattr(self, "_q8"):
+            t = self.torch
+            self._q8 = (t.empty(self.T * I_FF, dtype=t.int8, device="cuda"),
+                        t.empty(self.T, dtype=t.float32, device="cuda"),
+                        t.empty(self.T * I_FF // 32, dtype=t.int32, device="cuda"))
+        return self._q8
+
     def launch(self, name: str, i: int, st: int) -> None:
         d, dev, T = self.sets[i % self.nsets], self.dev, self.T
         if name == "gather+norm":
@@ -110,6 +121,14 @@ class Workload:
                                     d["normed"].data_ptr(), T, H, EPS, st)
         elif name == "residual_add":
             rc = dev.vv_residual_add_dev(d["residual"].data_ptr(), d["x"].data_ptr(), T * H, st)
+        elif name == "rmsnorm_q8":
+            q = self.q8_buffers()
+            rc = dev.vv_rmsnorm_q8_dev(d["x"].data_ptr(), self.weight.data_ptr(), T, H, EPS, 0,
+                                       q[0].data_ptr(), q[1].data_ptr(), q[2].data_ptr(), st)
+        elif name == "swiglu_q8":
+            q = self.q8_buffers()
+            rc = dev.vv_swiglu_q8_dev(d["gate"].data_ptr(), d["up"].data_ptr(), T, I_FF, 0,
+                                      q[0].data_ptr(), q[1].data_ptr(), q[2].data_ptr(), st)
         elif name == "rope_q":
             rc = dev.vv_rope_dev(d["q"].data_ptr(), T, NQ, HD, 0, None, THETA, st)
         elif name == "rope_k":
@@ -121,7 +140,7 @@ class Workload:
 
 
 KERNELS = ["gather+norm", "add+norm", "rope", "swiglu"]
-UNFUSED = ["embedding", "rmsnorm", "residual_add", "rope_q", "rope_k"]
+UNFUSED = ["embedding", "rmsnorm", "residual_add", "rope_q", "rope_k", "rmsnorm_q8", "swiglu_q8"]
 
 
 def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: int):
@@ -243,7 +262,8 @@ def main() -> int:
     ap.add_argument("--only", default=None, help="time only this kernel (profiling aid)")
     ap.add_argument("--reps", type=int, default=5, help="event-timed repetitions per kernel")
     ap.add_argument("--unfused", action="store_true",
-                    help="also time the unfused reference-API calls (reported under 'unfused')")
+                    help="also time the unfused reference-API calls and the int8-activation fused "
+                         "forms (reported under 'unfused'; not part of the step)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
                          "five times: the known-size reference for rocprofv3 byte counters")
@@ -316,7 +336,7 @@ def main() -> int:
                              "GBps": bytes_per[name] / med / 1e9,
                              "frac_of_peak": bytes_per[name] / med / 1e9 / HBM_PEAK_GBPS}
             log(f"  {name:12s} {med * 1e6:9.2f} us  {unfused[name]['GBps']:8.1f} GB/s  "
-                f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (unfused form)")
+                f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (not part of the step)")
 
     # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
     decode = {}

@@ -94,6 +94,33 @@ vv_status_t vv_fp32_to_fp16_dev(const void* in_fp32, void* out_fp16, int n,
 vv_status_t vv_fp16_to_fp32_dev(const void* in_fp16, void* out_fp32, int n,
                                 void* stream);
 
+/* ── Per-token int8 activations (the W8A8 / W4A8 front end) ─────────────── */
+
+/* Per row: sx[m] = max|v| / 127, xq = clamp(round-half-even(v * 127 / max|v|),
+ * +-127), where v is the FP16 value the unfused op would have written, so a
+ * fused row is bit-identical to "op, then vv_act_quant_dev" and to the CPU
+ * quantiser on those values. `layout` is the order of the int8 values inside
+ * each run of 32 columns (0 natural, 1 nibble, 2 W4-GEMV, 3 W4-MMA: the
+ * reference's include/vibevoice/q8.h); `xsum` (may be NULL) receives the sum of
+ * xq over each run, [M][K/32]. K % 32 != 0, K > 22528 or pointers that are not
+ * 16-byte (inputs) / 8-byte (xq) aligned: VV_ERR_UNSUPPORTED, nothing launched;
+ * M <= 0, K <= 0 or a bad layout: VV_ERR_INVALID_ARG.
+ * replace device.h:320-334 (src/cuda/act_quant.cu:226-275). */
+vv_status_t vv_act_quant_dev(const void* x, int M, int K, int layout, int8_t* xq,
+                             float* sx, int32_t* xsum, void* stream);
+/* RMSNorm fused with the quantiser; K < 256: VV_ERR_UNSUPPORTED. */
+vv_status_t vv_rmsnorm_q8_dev(const void* x, const void* weight, int M, int K,
+                              float eps, int layout, int8_t* xq, float* sx,
+                              int32_t* xsum, void* stream);
+/* SwiGLU fused with the quantiser. */
+vv_status_t vv_swiglu_q8_dev(const void* gate, const void* up, int M, int K,
+                             int layout, int8_t* xq, float* sx, int32_t* xsum,
+                             void* stream);
+/* acc[k] = max(acc[k], max_m |x[m,k]|), x FP16 [M,K], acc FP32 [K] updated in
+ * place (SmoothQuant calibration). replaces device.h:343-344
+ * (src/cuda/act_quant.cu:277-313). */
+vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* stream);
+
 /* ── Fused forms (additions) ───────────────────────────────────────────── */
 
 /* addition: vv_residual_add_dev(residual, x) followed by

@@ -67,6 +67,10 @@ def _load():
     lib.vvo_fill_normal_f16.argtypes = [_u16p, C.c_size_t, C.c_uint64, C.c_double, C.c_double]
     lib.vvo_fill_normal_f32.argtypes = [_f32p, C.c_size_t, C.c_uint64, C.c_double, C.c_double]
     lib.vvo_fill_ids.argtypes = [_i32p, C.c_size_t, C.c_uint64, C.c_int32]
+    lib.vvo_q8_pos.restype = C.c_int
+    lib.vvo_q8_pos.argtypes = [C.c_int, C.c_int]
+    lib.vvo_quant_act_q8.restype = C.c_int
+    lib.vvo_quant_act_q8.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8), _f32p, _i32p]
     lib.vvo_threads.restype = C.c_int
     lib.vvo_set_threads.argtypes = [C.c_int]
     for name in ("vvo_rmsnorm_f32", "vvo_rope_f32", "vvo_swiglu_f32", "vvo_residual_add_f32",
@@ -92,6 +96,10 @@ def _load_ref():
                  "vv_embedding_cpu", "vv_cpu_threads", "vv_cpu_physical_cores"):
         getattr(ref, name).restype = C.c_int
     ref.vv_cpu_simd_name.restype = C.c_char_p
+    if hasattr(ref, "vv_quant_act_q8_cpu"):
+        ref.vv_quant_act_q8_cpu.restype = C.c_int
+        ref.vv_quant_act_q8_cpu.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8),
+                                            _f32p, _i32p]
     return ref
 
 
@@ -256,3 +264,16 @@ def bias_add_f16(out16: np.ndarray, bias16: np.ndarray) -> np.ndarray:
     M, N = v.shape
     _check(lib.vvo_bias_add_f16(_p(v, _u16p), _p(bias16, _u16p), M, N), "bias_add_f16")
     return v
+
+
+def quant_act_q8(x: np.ndarray, layout: int, want_xsum: bool = True):
+    """float32 [M,K] -> (int8 [M,K] in `layout`, float32 scale [M], int32 xsum [M,K/32] or None)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    xq = np.empty((M, K), dtype=np.int8)
+    sx = np.empty(M, dtype=np.float32)
+    xs = np.empty((M, K // 32), dtype=np.int32) if want_xsum else None
+    _check(lib.vvo_quant_act_q8(_p(x, _f32p), M, K, layout, xq.ctypes.data_as(C.POINTER(C.c_int8)),
+                                _p(sx, _f32p), _p(xs, _i32p) if want_xsum else None),
+           "quant_act_q8")
+    return xq, sx, xs

@@ -281,6 +281,57 @@ int vvo_bias_add_f16(uint16_t* out, const uint16_t* bias, int M, int N) {
     return VVO_OK;
 }
 
+/* ── per-token int8 activation quantiser ──────────────────────────────── */
+
+int vvo_q8_pos(int layout, int j) {
+    /* q8.h:56-66. The W4 layouts mirror a 16-byte chunk of packed 4-bit
+     * weights: column j lives in 32-bit word (j/2)%4 at nibble slot
+     * j/8 + 4*(j%2). */
+    const int odd = j & 1, word = (j >> 1) & 3, slot = (j >> 3) + 4 * odd;
+    if (layout == 1) return odd ? 16 + (j >> 1) : (j >> 1);
+    if (layout == 2) return 8 * word + 4 * (slot & 1) + (slot >> 1);
+    if (layout == 3) return 16 * odd + 4 * word + (slot & 3);
+    return j;
+}
+
+int vvo_quant_act_q8(const float* x, int M, int K, int layout, int8_t* xq,
+                     float* sx, int32_t* xsum) {
+    /* cpu_int8.c:158-196. All FP32: one division for the scale, one for its
+     * reciprocal, one multiply and one round-half-even per element. */
+    if (!x || !xq || !sx) return VVO_ERR_NULL_PTR;
+    if (M <= 0 || K <= 0 || (K % 32) != 0) return -1;
+    if (layout < 0 || layout > 3) return -1;
+    int where[32];
+    for (int j = 0; j < 32; j++) where[j] = vvo_q8_pos(layout, j);
+    int m;
+#pragma omp parallel for schedule(static) if (M > 4)
+    for (m = 0; m < M; m++) {
+        const float* row = x + (size_t)m * K;
+        int8_t* out = xq + (size_t)m * K;
+        float amax = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const float a = fabsf(row[k]);
+            if (a > amax) amax = a;
+        }
+        const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+        sx[m] = amax / 127.0f;
+        for (int run = 0; run < K / 32; run++) {
+            int total = 0;
+            for (int j = 0; j < 32; j++) {
+                const float scaled = row[run * 32 + j] * inv;
+                float r = rintf(scaled);
+                if (r > 127.0f) r = 127.0f;
+                if (r < -127.0f) r = -127.0f;
+                const int q = (int)r;
+                total += q;
+                out[run * 32 + where[j]] = (int8_t)q;
+            }
+            if (xsum) xsum[(size_t)m * (K / 32) + run] = total;
+        }
+    }
+    return VVO_OK;
+}
+
 /* ── seeded inputs ─────────────────────────────────────────────────────── */
 
 static inline uint64_t splitmix64(uint64_t z) {

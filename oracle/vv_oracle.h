@@ -92,6 +92,20 @@ int vvo_embedding_f16(const uint16_t* table, const int32_t* ids,
  * out[m,n] = half_rn(float(out[m,n]) + float(bias[n])). Bit-exact target. */
 int vvo_bias_add_f16(uint16_t* out, const uint16_t* bias, int M, int N);
 
+/* ── per-token int8 activation quantiser (the W8A8 / W4A8 path's front end) ─ */
+
+/* Where column j (0..31) of a 32-column run is stored, per layout
+ * (include/vibevoice/q8.h:19-66): 0 natural, 1 nibble (16 even columns, then
+ * 16 odd), 2 W4 GEMV, 3 W4 MMA. */
+int vvo_q8_pos(int layout, int j);
+
+/* src/cpu/cpu_int8.c:158-196 (vv_quant_act_q8_cpu): per row, amax = max|x|,
+ * sx = amax/127, xq = clamp(rint(x * (127/amax)), +-127) stored at the
+ * layout's position inside each run of 32; xsum (optional) = the sum of xq over
+ * each run. K must be a multiple of 32. Bit-exact target for the device. */
+int vvo_quant_act_q8(const float* x, int M, int K, int layout, int8_t* xq,
+                     float* sx, int32_t* xsum);
+
 /* ── seeded inputs (the same bytes go to the oracle and to the GPU) ────── */
 
 /* N(mean, std) rounded to FP16 (RNE). Counter-based: element i depends only

@@ -7,7 +7,8 @@ oracle/Makefile compiles from the reference's src/cpu/cpu_kernels.c):
 
 The fixture holds inputs and the reference's outputs for its five layer
 kernels (vv_rmsnorm_cpu, vv_rope_cpu, vv_swiglu_cpu, vv_residual_add_cpu,
-vv_embedding_cpu) at small shapes. It is data only: no reference source text.
+vv_embedding_cpu) at small shapes. It also holds the int8 activation quantiser's outputs (vv_quant_act_q8_cpu)
+in all four layouts. It is data only: no reference source text.
 Inputs come from a local numpy generator and are stored in the file, so the
 fixture does not depend on any generator staying stable.
 """
@@ -85,6 +86,21 @@ def main() -> None:
     assert ref.vv_embedding_cpu(table.ctypes.data, p(ids, i32p), p(e, f32p), ids.size, 72) == 0
     out["emb_table"], out["emb_ids"] = table, ids
     out["emb_y_bits"] = e.view(np.uint32)     # bits: NaN payloads survive the file
+
+    # Int8 activation quantiser (src/cpu/cpu_int8.c), all four layouts.
+    i8p = C.POINTER(C.c_int8)
+    xq_in = (3.0 * rng.standard_normal((4, 256))).astype(np.float16).astype(np.float32)
+    xq_in[1] = 0.0
+    xq_in[2, :6] = [127.0, 0.5, 1.5, 2.5, -0.5, -126.5]
+    xq_in[2, 6:] *= 0.01
+    out["q8_x"] = xq_in
+    for layout in range(4):
+        q = np.empty((4, 256), np.int8)
+        sx = np.empty(4, np.float32)
+        xs = np.empty((4, 8), np.int32)
+        assert ref.vv_quant_act_q8_cpu(p(xq_in, f32p), 4, 256, layout, q.ctypes.data_as(i8p),
+                                       p(sx, f32p), p(xs, i32p)) == 0
+        out[f"q8_q{layout}"], out[f"q8_sx{layout}"], out[f"q8_xs{layout}"] = q, sx, xs
 
     path = os.path.join(HERE, "cpu_kernels_golden.npz")
     np.savez_compressed(path, **out)

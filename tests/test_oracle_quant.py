@@ -1,0 +1,107 @@
+"""Pins the oracle's int8 activation quantiser (oracle/vv_oracle.c:
+vvo_quant_act_q8, vvo_q8_pos) — the checker for vv_act_quant_dev and the fused
+*_q8 kernels: against the compiled reference (src/cpu/cpu_int8.c), against a
+numpy restatement written from the documented definition, and against the
+layouts' descriptions in the reference's q8.h."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+
+needs_ref = pytest.mark.skipif(oracle.ref is None or not hasattr(oracle.ref, "vv_quant_act_q8_cpu"),
+                               reason="oracle/_ref not built here")
+
+
+def layout_table(layout):
+    return [oracle.lib.vvo_q8_pos(layout, j) for j in range(32)]
+
+
+def test_layouts_match_their_descriptions():
+    """q8.h:19-47 describes each layout in words; build each table from the words."""
+    assert layout_table(0) == list(range(32))
+    # nibble: the 16 even columns, then the 16 odd ones
+    want = [0] * 32
+    for n, j in enumerate(list(range(0, 32, 2)) + list(range(1, 32, 2))):
+        want[j] = n
+    assert layout_table(1) == want
+    # W4A16 GPU layout: column j sits in word t = (j/2)%4 at nibble slot s = j/8 + 4*(j%2)
+    gemv, mma = [0] * 32, [0] * 32
+    for j in range(32):
+        t, s = (j // 2) % 4, j // 8 + 4 * (j % 2)
+        # GEMV: positions 8t..8t+3 are the even slots (0,2,4,6), 8t+4..8t+7 the odd ones
+        gemv[j] = 8 * t + (4 if s % 2 else 0) + s // 2
+        # MMA: slots 0..3 of word t at 4t..4t+3, slots 4..7 at 16+4t..16+4t+3
+        mma[j] = (16 if s >= 4 else 0) + 4 * t + s % 4
+    assert layout_table(2) == gemv and layout_table(3) == mma
+    for lay in range(4):
+        assert sorted(layout_table(lay)) == list(range(32))       # a permutation
+
+
+def numpy_quant(x, layout):
+    x = x.astype(np.float32)
+    amax = np.abs(x).max(axis=1)
+    with np.errstate(divide="ignore"):
+        inv = np.where(amax > 0, np.float32(127.0) / amax, np.float32(0)).astype(np.float32)
+    sx = (amax / np.float32(127.0)).astype(np.float32)
+    q = np.clip(np.rint((x * inv[:, None]).astype(np.float32)), -127, 127).astype(np.int32)
+    M, K = x.shape
+    runs = q.reshape(M, K // 32, 32)
+    out = np.empty_like(runs)
+    out[:, :, layout_table(layout)] = runs
+    return out.reshape(M, K).astype(np.int8), sx, runs.sum(axis=2).astype(np.int32)
+
+
+@pytest.mark.parametrize("layout", [0, 1, 2, 3])
+def test_quantiser_against_numpy_restatement(layout):
+    x = oracle.widen(oracle.normal_f16((9, 3584), 11 + layout, std=3.0))
+    x[2] = 0.0                                        # zero row: scale 0, all zeros
+    x[3, 5] = 1000.0                                  # one outlier sets the scale
+    x[4] = np.float32(0.5)                            # ties: 0.5*inv lands on .5 values
+    q, sx, xs = oracle.quant_act_q8(x, layout)
+    wq, wsx, wxs = numpy_quant(x, layout)
+    assert np.array_equal(q, wq) and np.array_equal(sx, wsx) and np.array_equal(xs, wxs)
+    assert not q[2].any() and sx[2] == 0.0
+    assert np.abs(q.astype(np.int32)).max() == 127 and q.min() >= -127
+    # round-half-even, not half-away: 2.5 -> 2, 3.5 -> 4 (amax 127 makes inv exactly 1)
+    t = np.zeros((1, 32), np.float32)
+    t[0, :5] = [127.0, 2.5, 3.5, -2.5, -0.5]
+    tq, _, _ = oracle.quant_act_q8(t, 0)
+    assert tq[0, :5].tolist() == [127, 2, 4, -2, 0]
+
+
+@needs_ref
+@pytest.mark.parametrize("M,K", [(1, 32), (7, 1536), (5, 3584), (3, 18944), (2, 22528)])
+def test_quantiser_equals_compiled_reference(M, K):
+    x = oracle.widen(oracle.normal_f16((M, K), M + K, std=4.0))
+    i8p, f32p, i32p = C.POINTER(C.c_int8), C.POINTER(C.c_float), C.POINTER(C.c_int32)
+    for layout in range(4):
+        q, sx, xs = oracle.quant_act_q8(x, layout)
+        rq, rsx, rxs = np.empty_like(q), np.empty_like(sx), np.empty_like(xs)
+        assert oracle.ref.vv_quant_act_q8_cpu(x.ctypes.data_as(f32p), M, K, layout, rq.ctypes.data_as(i8p),
+                                              rsx.ctypes.data_as(f32p), rxs.ctypes.data_as(i32p)) == 0
+        assert np.array_equal(q, rq) and np.array_equal(sx.view(np.uint32), rsx.view(np.uint32))
+        assert np.array_equal(xs, rxs)
+
+
+def test_quantiser_against_golden_vectors():
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "cpu_kernels_golden.npz"))
+    for layout in range(4):
+        q, sx, xs = oracle.quant_act_q8(gold["q8_x"], layout)
+        assert np.array_equal(q, gold[f"q8_q{layout}"]), layout
+        assert np.array_equal(sx.view(np.uint32), gold[f"q8_sx{layout}"].view(np.uint32))
+        assert np.array_equal(xs, gold[f"q8_xs{layout}"])
+
+
+def test_quantiser_argument_checks():
+    x = np.zeros((2, 64), np.float32)
+    q = np.zeros((2, 64), np.int8)
+    sx = np.zeros(2, np.float32)
+    i8p, f32p = C.POINTER(C.c_int8), C.POINTER(C.c_float)
+    call = oracle.lib.vvo_quant_act_q8
+    assert call(x.ctypes.data_as(f32p), 2, 64, 0, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == 0
+    assert call(x.ctypes.data_as(f32p), 2, 48, 0, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -1
+    assert call(x.ctypes.data_as(f32p), 2, 64, 4, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -1
+    assert call(None, 2, 64, 0, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -2

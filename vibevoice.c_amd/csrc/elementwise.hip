@@ -10,23 +10,12 @@
 // chunk before it writes it and no other thread touches that chunk, so an
 // output that aliases an input exactly (out == gate, the way the decoder calls
 // SwiGLU) is safe. Unaligned pointers take a 2-byte kernel.
-#include "vv_common.hpp"
+#include "row_math.hpp"
 
 namespace vv {
 namespace {
 
 constexpr int kEwBlock = kWave;                  // one wave per workgroup
-
-// silu(g) * u in the oracle's association, (g / (1 + e^-g)) * u, with the
-// hardware exponential and reciprocal: exp2(-g * log2 e) and rcp are each
-// accurate to about 1 ulp of FP32, three orders below the FP16 rounding of the
-// result. Large |g| needs no special case: e^-g -> inf gives rcp -> 0 and
-// g * 0 = -0 (the oracle's -65504 / inf), e^-g -> 0 gives g itself.
-__device__ __forceinline__ float swiglu1(float g, float u) {
-    const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
-    const float silu = g * __builtin_amdgcn_rcpf(1.0f + e);
-    return silu * u;
-}
 
 enum EwOp : int { kSwiglu = 0, kResidual = 1 };
 

@@ -14,7 +14,7 @@
 // the add+norm traffic pattern, one with a whole row per wave (7 chunks per
 // lane, 14 loads in flight per lane, no LDS) 5.8 TB/s; the measured kernels
 // follow (add+norm 66.6 vs 71.0 us at 14449 rows).
-#include "vv_common.hpp"
+#include "row_math.hpp"
 
 namespace vv {
 namespace {
@@ -26,15 +26,6 @@ enum RowMode : int {
     kGatherOnly = 3  // state = src[ids[row]]
 };
 
-// 1 / sqrt(mean(x^2) + eps) with the hardware reciprocal square root (1 ulp of
-// FP32, i.e. ~1e-7 relative against an FP16 result whose own rounding is 5e-4).
-// Every lane of every wave of a row evaluates this, so it has to be a handful
-// of instructions: the correctly rounded divide + sqrt + divide sequence is
-// ~60 and was a measurable share of the VALU time with one chunk per thread.
-__device__ __forceinline__ float inv_rms(float sumsq, float inv_n, float eps) {
-    return __builtin_amdgcn_rsqf(sumsq * inv_n + eps);
-}
-
 // ── one workgroup per row, one chunk per thread ──────────────────────────
 // blockDim = the row's chunk count rounded up to whole waves (448 threads = 7
 // waves for hidden 3584), kCpt chunks per thread for rows wider than 1024
@@ -43,8 +34,6 @@ __device__ __forceinline__ float inv_rms(float sumsq, float inv_n, float eps) {
 // 6.4 TB/s for the add+norm traffic pattern against 5.8 TB/s with one wave per
 // row. Sum of squares: DPP reduction inside each wave, then one float per wave
 // through LDS and a single barrier.
-constexpr int kMaxWgThreads = 1024;
-
 template <int kCpt, int kRows, int kMode, bool kStream, bool kFull>   // kFull: nchunks == kCpt * blockDim.x
 __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
     const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
@@ -114,8 +103,7 @@ __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
                 }
                 if ((kMode == kAdd || kMode == kGather) && live[r])
                     store_chunk_as<kStream>(state + out_base[r] + c, a[r][j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc = fmaf(x[i], x[i], acc);
+                acc = chunk_sumsq(x, acc);
             }
         }
         acc = wave_sum(acc);
@@ -132,13 +120,8 @@ __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
 #pragma unroll
         for (int j = 0; j < kCpt; ++j) {
             const int c = j * nthreads + t;
-            if ((kFull || c < nchunks) && live[r]) {
-                f32x8 x = unpack(a[r][j]);
-                const f32x8 g = unpack(w[j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) x[i] = (x[i] * inv) * g[i];
-                store_chunk_as<kStream>(normed + out_base[r] + c, pack(x));
-            }
+            if ((kFull || c < nchunks) && live[r])
+                store_chunk_as<kStream>(normed + out_base[r] + c, scale_chunk(a[r][j], inv, w[j]));
         }
     }
 }

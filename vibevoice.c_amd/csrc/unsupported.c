@@ -10,7 +10,7 @@
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
  * HIP library does not define (dense/quantised GEMM and GEMV, attention, KV
- * cache, LM head, VAE, BitNet, int8 activation quantisers). It builds into its
+ * cache, LM head, VAE, BitNet). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
  * stays exactly what include/vibevoice_hip.h declares.
@@ -37,10 +37,8 @@ VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_
 VV_DECLINE(vv_w4a16_gemv_dev)    VV_DECLINE(vv_w4a16_gemv_multi_dev)
 VV_DECLINE(vv_w4a16_gather_dev)  VV_DECLINE(vv_w4a16_gemm_dev)    VV_DECLINE(vv_w4a16_dequant_dev)
 
-/* int8 activations and W8A8 / W4A8 linears (device.h:320-410) */
-VV_DECLINE(vv_act_quant_dev)     VV_DECLINE(vv_rmsnorm_q8_dev)    VV_DECLINE(vv_swiglu_q8_dev)
-VV_DECLINE(vv_col_absmax_dev)    VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)
-VV_DECLINE(vv_i8_linear_multi_dev)
+/* W8A8 / W4A8 linears (device.h:362-410); the activation quantisers are implemented */
+VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)   VV_DECLINE(vv_i8_linear_multi_dev)
 
 /* dense FP16 GEMM (device.h:423-482) */
 VV_DECLINE(vv_gemm_fp16_dev)     VV_DECLINE(vv_gemm_fp16_tile_dev) VV_DECLINE(vv_skinny_linear_dev)

@@ -116,6 +116,23 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
+// The same butterfly with max instead of +, for row-wise absmax.
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
+                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
+// Integer sum over each quad of lanes (lanes 4q..4q+3), left in all four.
+__device__ __forceinline__ int quad_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
+    return v;
+}
+
 __device__ __forceinline__ int wave_in_block() {
     return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }

@@ -36,6 +36,10 @@ SIGNATURES = {
     "vv_bias_add_dev": (_i, [_vp, _vp, _i, _i, _vp]),
     "vv_fp32_to_fp16_dev": (_i, [_vp, _vp, _i, _vp]),
     "vv_fp16_to_fp32_dev": (_i, [_vp, _vp, _i, _vp]),
+    "vv_act_quant_dev": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "vv_rmsnorm_q8_dev": (_i, [_vp, _vp, _i, _i, _f, _i, _vp, _vp, _vp, _vp]),
+    "vv_swiglu_q8_dev": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "vv_col_absmax_dev": (_i, [_vp, _i, _i, _vp, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
