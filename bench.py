@@ -160,6 +160,64 @@ def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: in
     return per[0], per[len(per) // 2]
 
 
+def decode_graph_leg(torch, dev, wl1) -> dict:
+    """One token's worth of this library's launches (per layer: norm -> RoPE(Q,K) with the
+    position read from device memory -> add+norm -> SwiGLU -> add+norm), issued directly and
+    as a captured graph replayed; the position advances inside the graph (vv_pos_add_dev)."""
+    import ctypes as C
+    d = wl1.sets[0]
+    w = wl1.weight.data_ptr()
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    s = C.c_void_p()
+    assert dev.vv_dev_stream_create(C.byref(s)) == 0
+    st = s.value
+    layers = 28
+
+    def issue():
+        n = 0
+        for _ in range(layers):
+            assert dev.vv_rmsnorm_dev(d["hidden"].data_ptr(), w, d["normed"].data_ptr(), 1, H, EPS, st) == 0
+            assert dev.vv_rope_qk_dev(d["q"].data_ptr(), d["k"].data_ptr(), 1, NQ, NK, HD, 0,
+                                      pos.data_ptr(), THETA, st) == 0
+            assert dev.vv_add_rmsnorm_dev(d["residual"].data_ptr(), d["x"].data_ptr(), w,
+                                          d["normed"].data_ptr(), 1, H, EPS, st) == 0
+            assert dev.vv_swiglu_dev(d["gate"].data_ptr(), d["up"].data_ptr(), d["gate"].data_ptr(),
+                                     I_FF, st) == 0
+            assert dev.vv_add_rmsnorm_dev(d["residual"].data_ptr(), d["x"].data_ptr(), w,
+                                          d["normed"].data_ptr(), 1, H, EPS, st) == 0
+            n += 5
+        assert dev.vv_pos_add_dev(pos.data_ptr(), pos.data_ptr(), 1, st) == 0
+        return n + 1
+
+    torch.cuda.synchronize()
+    launches = issue()
+    assert dev.vv_dev_stream_sync(st) == 0
+    reps = 20
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        issue()
+    assert dev.vv_dev_stream_sync(st) == 0
+    eager = (time.perf_counter() - t0) / reps
+    assert dev.vv_dev_graph_begin(st) == 0
+    issue()
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(st, C.byref(g)) == 0 and g.value
+    for _ in range(3):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    before = int(pos.item())
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    replay = (time.perf_counter() - t0) / reps
+    assert int(pos.item()) == before + reps          # every replay advanced the device-side position
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(st)
+    return {"launches": launches, "eager_us": eager * 1e6, "replay_us": replay * 1e6,
+            "replay_us_per_launch": replay * 1e6 / launches}
+
+
 def cpu_baseline(rows: int) -> dict:
     """The CPU path of the same step on `rows` rows: warm-up, then best of five
     (bench/benchmark.c:197-211). FP32 activations, so its byte count is its own."""
@@ -348,6 +406,13 @@ def main() -> int:
         log("  decode (T=1) us per launch: " +
             ", ".join(f"{n} {d['us_median']:.2f}" for n, d in decode.items()))
 
+    # ── the decode step's layer ops as one captured graph (28 layers x 5 launches) ──
+    graph = {}
+    if not args.only:
+        graph = decode_graph_leg(torch, dev, wl1)
+        log(f"  decode graph: {graph['launches']} launches, eager {graph['eager_us']:.1f} us, "
+            f"graph replay {graph['replay_us']:.1f} us ({graph['replay_us_per_launch']:.2f} us/launch)")
+
     dominant = max(kernels, key=lambda n: bytes_per[n])
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
@@ -374,6 +439,8 @@ def main() -> int:
         result["unfused"] = unfused
     if decode:
         result["decode_T1_us"] = decode
+    if graph:
+        result["decode_graph"] = graph
     if not args.no_cpu:
         log(f"cpu baseline on {CPU_SAMPLE_ROWS} rows ...")
         result["cpu_baseline"] = cpu_baseline(CPU_SAMPLE_ROWS)
