@@ -55,6 +55,7 @@ def algorithmic_bytes(T: int) -> dict:
         "rope_q": 4 * T * NQ * HD,
         "rope_k": 4 * T * NK * HD,
         # int8-activation fused forms: FP16 in, int8 + scale + per-32 sums out
+        "act_quant": 2 * T * H + T * H + 4 * T + T * H // 8,
         "rmsnorm_q8": 2 * T * H + 2 * H + T * H + 4 * T + T * H // 8,
         "swiglu_q8": 4 * T * I_FF + T * I_FF + 4 * T + T * I_FF // 8,
     }
@@ -121,6 +122,10 @@ class Workload:
                                     d["normed"].data_ptr(), T, H, EPS, st)
         elif name == "residual_add":
             rc = dev.vv_residual_add_dev(d["residual"].data_ptr(), d["x"].data_ptr(), T * H, st)
+        elif name == "act_quant":
+            q = self.q8_buffers()
+            rc = dev.vv_act_quant_dev(d["x"].data_ptr(), T, H, 0, q[0].data_ptr(), q[1].data_ptr(),
+                                      q[2].data_ptr(), st)
         elif name == "rmsnorm_q8":
             q = self.q8_buffers()
             rc = dev.vv_rmsnorm_q8_dev(d["x"].data_ptr(), self.weight.data_ptr(), T, H, EPS, 0,
@@ -140,7 +145,8 @@ class Workload:
 
 
 KERNELS = ["gather+norm", "add+norm", "rope", "swiglu"]
-UNFUSED = ["embedding", "rmsnorm", "residual_add", "rope_q", "rope_k", "rmsnorm_q8", "swiglu_q8"]
+UNFUSED = ["embedding", "rmsnorm", "residual_add", "rope_q", "rope_k", "act_quant", "rmsnorm_q8",
+           "swiglu_q8"]
 
 
 def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: int):

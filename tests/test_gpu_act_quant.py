@@ -73,7 +73,7 @@ def test_quantisers_reference_shapes(M, K):
     assert np.array_equal(bits_of(d_x), x) and np.array_equal(bits_of(d_x2), x2)   # inputs untouched
 
 
-@pytest.mark.parametrize("K", [32, 256, 2048, 8192, 8224, 16384, 22528])
+@pytest.mark.parametrize("K", [32, 256, 288, 1024, 2048, 4096, 4128, 8192, 8224, 16384, 22528])
 def test_quantiser_widths_and_rounding(K):
     """Widths at the edges of the 1/2/3-chunks-per-thread ranges, and ties."""
     M = 5
@@ -88,6 +88,16 @@ def test_quantiser_widths_and_rounding(K):
         assert np.array_equal(q, rq) and np.array_equal(sx, rsx) and np.array_equal(xs, rxs), (K, layout)
     q, _, _ = run_quant("act_quant", d_x, None, None, M, K, 0)
     assert q[0, 0] == 127 and not q[0, 1:].any()
+    # the fused norm at the same widths (one wave per row up to 4096, workgroup per row beyond)
+    if K >= 256:
+        x2 = oracle.normal_f16((M, K), K + 1, std=1.5)
+        w = oracle.normal_f16((K,), 9, mean=1.0, std=0.2)
+        d_x2, d_w = to_dev(x2), to_dev(w)
+        hy = oracle.widen(unfused_fp16("rmsnorm_q8", d_x2, None, d_w, M, K))
+        for layout in range(4):
+            q, sx, xs = run_quant("rmsnorm_q8", d_x2, None, d_w, M, K, layout)
+            rq, rsx, rxs = oracle.quant_act_q8(hy, layout)
+            assert np.array_equal(q, rq) and np.array_equal(sx, rsx) and np.array_equal(xs, rxs), (K, layout)
 
 
 def test_quantiser_status_codes():

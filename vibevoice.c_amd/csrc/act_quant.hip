@@ -38,16 +38,6 @@ __device__ __forceinline__ int q8_pos(int layout, int j) {
     }
 }
 
-__device__ __forceinline__ float block_max(float v, float* partial) {
-    v = wave_max(v);
-    if (lane_id() == 0) partial[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float m = 0.0f;
-    const int nwaves = (int)blockDim.x >> 6;
-    for (int i = 0; i < nwaves; ++i) m = fmaxf(m, partial[i]);
-    return m;
-}
-
 // max |v| over the 8 halves of a chunk, in packed FP16 (exact: max and abs do
 // not round): 4 masks + 3 v_pk_max_f16 instead of 8 conversions and 8 maxima.
 __device__ __forceinline__ float chunk_absmax(const Chunk& c) {
@@ -90,79 +80,192 @@ __device__ __forceinline__ void quantise_chunk(const Chunk& h, float to_q, uint3
     hi = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
 }
 
-template <int kCpt, int kSrc, bool kStream>
+// One workgroup per row (kRows = 1 in every launch; several rows per workgroup
+// were measured and bought nothing: these kernels are bound by instruction
+// issue, not by loads in flight), kCpt chunks per thread.
+template <int kCpt, int kRows, int kSrc, bool kStream>
 __global__ __launch_bounds__(kMaxWgThreads) void quant_rows_wg(
-    const Chunk* a_in, const Chunk* __restrict__ b_in, int nchunks, float inv_n, float eps,
-    int layout, int8_t* __restrict__ xq, float* __restrict__ sx, int32_t* __restrict__ xsum) {
-    __shared__ float partial_sum[kMaxWgWaves];
-    __shared__ float partial_max[kMaxWgWaves];
+    const Chunk* a_in, const Chunk* __restrict__ b_in, int rows, int nchunks, float inv_n,
+    float eps, int layout, int8_t* __restrict__ xq, float* __restrict__ sx,
+    int32_t* __restrict__ xsum) {
+    __shared__ float partial_sum[kRows][kMaxWgWaves];
+    __shared__ float partial_max[kRows][kMaxWgWaves];
     __shared__ __attribute__((aligned(8))) unsigned char stage[kMaxWgThreads * 8];
 
-    const size_t row = blockIdx.x;
     const int t = (int)threadIdx.x;
     const int nthreads = (int)blockDim.x;
-    const size_t in_base = row * (size_t)nchunks;
+    const int row0 = (int)blockIdx.x * kRows;
 
-    // ── the op: FP16 values h[] exactly as the unfused kernel would store them ──
-    Chunk h[kCpt], b[kCpt];
+    // ── the op: FP16 values h[][] exactly as the unfused kernel would store them ──
+    Chunk h[kRows][kCpt], b[kRows][kCpt];
+    bool live_row[kRows];
+    size_t row_of[kRows];
 #pragma unroll
-    for (int j = 0; j < kCpt; ++j) {
-        const int c = j * nthreads + t;
-        if (c < nchunks) {
-            h[j] = load_chunk_as<kStream>(a_in + in_base + c);
-            if (kSrc == kQNorm) b[j] = load_chunk(b_in + c);                        // weight
-            if (kSrc == kQSwiglu) b[j] = load_chunk_as<kStream>(b_in + in_base + c);  // up
+    for (int r = 0; r < kRows; ++r) {
+        live_row[r] = kRows == 1 || row0 + r < rows;
+        row_of[r] = (size_t)(live_row[r] ? row0 + r : rows - 1);   // a dead row re-reads the last one
+        const size_t in_base = row_of[r] * (size_t)nchunks;
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            if (c < nchunks) {
+                h[r][j] = load_chunk_as<kStream>(a_in + in_base + c);
+                if (kSrc == kQNorm) b[r][j] = load_chunk(b_in + c);                        // weight
+                if (kSrc == kQSwiglu) b[r][j] = load_chunk_as<kStream>(b_in + in_base + c);  // up
+            }
         }
     }
     if (kSrc == kQNorm) {
-        float acc = 0.0f;
+        float acc[kRows];
 #pragma unroll
-        for (int j = 0; j < kCpt; ++j)
-            if (j * nthreads + t < nchunks) acc = chunk_sumsq(unpack(h[j]), acc);
-        const float inv = inv_rms(block_sum(acc, partial_sum), inv_n, eps);
+        for (int r = 0; r < kRows; ++r) {
+            acc[r] = 0.0f;
 #pragma unroll
-        for (int j = 0; j < kCpt; ++j)
-            if (j * nthreads + t < nchunks) h[j] = scale_chunk(h[j], inv, b[j]);
+            for (int j = 0; j < kCpt; ++j)
+                if (j * nthreads + t < nchunks) acc[r] = chunk_sumsq(unpack(h[r][j]), acc[r]);
+        }
+        block_sum_n<kRows>(acc, partial_sum);
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+            const float inv = inv_rms(acc[r], inv_n, eps);
+#pragma unroll
+            for (int j = 0; j < kCpt; ++j)
+                if (j * nthreads + t < nchunks) h[r][j] = scale_chunk(h[r][j], inv, b[r][j]);
+        }
     } else if (kSrc == kQSwiglu) {
 #pragma unroll
-        for (int j = 0; j < kCpt; ++j)
-            if (j * nthreads + t < nchunks) h[j] = swiglu_chunk(h[j], b[j]);
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int j = 0; j < kCpt; ++j)
+                if (j * nthreads + t < nchunks) h[r][j] = swiglu_chunk(h[r][j], b[r][j]);
     }
 
-    // ── the scale: absmax over the row ──
-    float amax = 0.0f;
+    // ── the scale: absmax over each row ──
+    float amax[kRows];
 #pragma unroll
-    for (int j = 0; j < kCpt; ++j) {
-        if (j * nthreads + t < nchunks) amax = fmaxf(amax, chunk_absmax(h[j]));
+    for (int r = 0; r < kRows; ++r) {
+        amax[r] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j)
+            if (j * nthreads + t < nchunks) amax[r] = fmaxf(amax[r], chunk_absmax(h[r][j]));
     }
-    amax = block_max(amax, partial_max);
-    const float to_q = amax > 0.0f ? 127.0f / amax : 0.0f;   // correctly rounded divisions,
-    if (t == 0) sx[row] = amax / 127.0f;                     // as on the CPU
+    block_max_n<kRows>(amax, partial_max);
 
     // ── quantise, sum per run of 32, place, store ──
-    int8_t* out_row = xq + row * (size_t)nchunks * 8u;
 #pragma unroll
-    for (int j = 0; j < kCpt; ++j) {
-        const int c = j * nthreads + t;
-        const bool live = c < nchunks;       // a quad is live or dead as a whole (K % 32 == 0)
+    for (int r = 0; r < kRows; ++r) {
+        const float to_q = amax[r] > 0.0f ? 127.0f / amax[r] : 0.0f;   // correctly rounded
+        if (t == 0 && live_row[r]) sx[row_of[r]] = amax[r] / 127.0f;    // divisions, as on the CPU
+        int8_t* out_row = xq + row_of[r] * (size_t)nchunks * 8u;
+#pragma unroll
+        for (int j = 0; j < kCpt; ++j) {
+            const int c = j * nthreads + t;
+            const bool live = c < nchunks && live_row[r];   // a quad is live or dead as a whole
+            uint32_t lo = 0, hi = 0;
+            float run_part = 0.0f;
+            if (c < nchunks) quantise_chunk(h[r][j], to_q, lo, hi, run_part);
+            const int total = quad_sum((int)run_part);
+            if (live && xsum && (t & 3) == 0)
+                xsum[row_of[r] * (size_t)(nchunks >> 2) + (size_t)(c >> 2)] = total;
+            if (layout != 0) {
+                // Exchange inside the quad through LDS: byte i of this chunk is column
+                // 8*(t&3)+i of its run and belongs at q8_pos of that; then each thread
+                // takes back the 8 consecutive bytes it will store. Same wave, in-order
+                // LDS queue: no barrier.
+                unsigned char* run = stage + (t >> 2) * 32;
+                const int j0 = (t & 3) * 8;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t word = i < 4 ? lo : hi;
+                    run[q8_pos(layout, j0 + i)] = (unsigned char)(word >> (8 * (i & 3)));
+                }
+                const uint2 placed = *reinterpret_cast<const uint2*>(stage + t * 8);
+                lo = placed.x;
+                hi = placed.y;
+            }
+            if (live) {
+                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                const u32x2 v = {lo, hi};
+                u32x2* dst = reinterpret_cast<u32x2*>(out_row + (size_t)c * 8u);
+                if (kStream) __builtin_nontemporal_store(v, dst);
+                else *dst = v;
+            }
+        }
+    }
+}
+
+// ── RMSNorm + quantise for rows of at most 512 chunks: one wave per row ───
+// The quantiser's arithmetic is fixed cost per THREAD (two reductions, two
+// divisions, addressing) plus ~10 VALU operations per element, against only
+// 3 bytes of traffic per element: with one chunk per thread the kernel is
+// bound by instruction issue, not by HBM (46.8 us at 14449 x 3584, the plain
+// quantiser 35.5 us against 27.9 us with four chunks per thread). Here a lane
+// holds kCpl chunks — chunk j*64 + lane, exactly the chunk that lane `lane` of
+// wave j holds in vv_rmsnorm_dev's workgroup — so the sum of squares can be
+// formed in vv_rmsnorm_dev's order (per chunk, then the same DPP tree per group
+// of 64 chunks, then the groups in order) without LDS or barriers, and the FP16
+// values stay bit-identical to the unfused op's.
+template <int kCpl, bool kStream>
+__global__ __launch_bounds__(kBlock) void quant_norm_wave(
+    const Chunk* __restrict__ x, const Chunk* __restrict__ weight, int rows, int nchunks,
+    float inv_n, float eps, int layout, int8_t* __restrict__ xq, float* __restrict__ sx,
+    int32_t* __restrict__ xsum) {
+    __shared__ __attribute__((aligned(8))) unsigned char stage[kWavesPerBlock][kWave * 8];
+    const int wave = wave_in_block();
+    const int row = (int)blockIdx.x * kWavesPerBlock + wave;
+    if (row >= rows) return;
+    const int lane = lane_id();
+    const size_t in_base = (size_t)row * (size_t)nchunks;
+
+    Chunk h[kCpl], w[kCpl];
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        if (c < nchunks) {
+            h[j] = load_chunk_as<kStream>(x + in_base + c);
+            w[j] = load_chunk(weight + c);
+        }
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        const float acc = c < nchunks ? chunk_sumsq(unpack(h[j]), 0.0f) : 0.0f;
+        total += wave_sum(acc);          // group j = wave j of the unfused kernel, added in order
+    }
+    const float inv = inv_rms(total, inv_n, eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        if (j * kWave + lane < nchunks) {
+            h[j] = scale_chunk(h[j], inv, w[j]);
+            amax = fmaxf(amax, chunk_absmax(h[j]));
+        }
+    }
+    amax = wave_max(amax);
+    const float to_q = amax > 0.0f ? 127.0f / amax : 0.0f;
+    if (lane == 0) sx[row] = amax / 127.0f;
+
+    int8_t* out_row = xq + (size_t)row * (size_t)nchunks * 8u;
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        const bool live = c < nchunks;
         uint32_t lo = 0, hi = 0;
         float run_part = 0.0f;
         if (live) quantise_chunk(h[j], to_q, lo, hi, run_part);
-        const int total = quad_sum((int)run_part);
-        if (live && xsum && (t & 3) == 0) xsum[row * (size_t)(nchunks >> 2) + (size_t)(c >> 2)] = total;
-        if (layout != 0) {
-            // Exchange inside the quad through LDS: byte i of this chunk is column
-            // 8*(t&3)+i of its run and belongs at q8_pos of that; then each thread
-            // takes back the 8 consecutive bytes it will store. Same wave, in-order
-            // LDS queue: no barrier.
-            unsigned char* run = stage + (t >> 2) * 32;
-            const int j0 = (t & 3) * 8;
+        const int total_q = quad_sum((int)run_part);
+        if (live && xsum && (lane & 3) == 0)
+            xsum[(size_t)row * (size_t)(nchunks >> 2) + (size_t)(c >> 2)] = total_q;
+        if (layout != 0) {               // place the bytes inside the quad through LDS (see above)
+            unsigned char* run = stage[wave] + (lane >> 2) * 32;
+            const int j0 = (lane & 3) * 8;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint32_t word = i < 4 ? lo : hi;
                 run[q8_pos(layout, j0 + i)] = (unsigned char)(word >> (8 * (i & 3)));
             }
-            const uint2 placed = *reinterpret_cast<const uint2*>(stage + t * 8);
+            const uint2 placed = *reinterpret_cast<const uint2*>(stage[wave] + lane * 8);
             lo = placed.x;
             hi = placed.y;
         }
@@ -192,7 +295,35 @@ template <int kSrc>
 vv_status_t launch_quant(const void* a, const void* b, int M, int K, float eps, int layout,
                          int8_t* xq, float* sx, int32_t* xsum, hipStream_t st) {
     const int nchunks = K / 8;
-    const int cpt = (nchunks + kMaxWgThreads - 1) / kMaxWgThreads;            // 1..3
+    if (kSrc == kQNorm && nchunks <= 8 * kWave && !getenv("VV_Q8_LIGHT_NORM")) {
+        const float inv_k = 1.0f / (float)K;
+        const bool nt = use_streaming((size_t)M * (size_t)K * 3u);
+        const dim3 g((unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock));
+        const Chunk* px = static_cast<const Chunk*>(a);
+        const Chunk* pw = static_cast<const Chunk*>(b);
+#define VV_QN(C)                                                                                  \
+    case C:                                                                                       \
+        if (nt) quant_norm_wave<C, true><<<g, kBlock, 0, st>>>(px, pw, M, nchunks, inv_k, eps, layout, \
+                                                               xq, sx, xsum);                     \
+        else quant_norm_wave<C, false><<<g, kBlock, 0, st>>>(px, pw, M, nchunks, inv_k, eps, layout,   \
+                                                             xq, sx, xsum);                       \
+        break;
+        switch ((nchunks + kWave - 1) / kWave) {
+            VV_QN(1) VV_QN(2) VV_QN(3) VV_QN(4) VV_QN(5) VV_QN(6) VV_QN(7) VV_QN(8)
+        }
+#undef VV_QN
+        return launch_status();
+    }
+    // chunks per thread: VV_Q8_CPT forces (A/B aid), else the smallest that fits 1024 threads
+    static const int forced_cpt = getenv("VV_Q8_CPT") ? atoi(getenv("VV_Q8_CPT")) : 0;
+    int cpt = (nchunks + kMaxWgThreads - 1) / kMaxWgThreads;            // 1..3
+    // Without a reduction inside the op the mapping is free: four chunks per thread
+    // amortise the per-thread cost (plain quantiser 35.5 -> 27.9 us at 14449 x 3584).
+    // The fused norm must keep vv_rmsnorm_dev's mapping (same summation order).
+    if (kSrc == kQPlain && cpt < 4 && nchunks >= 4 * kWave) cpt = 4;
+    if (forced_cpt > cpt && kSrc != kQNorm) cpt = forced_cpt;
+    if (cpt == 5 || cpt == 6) cpt = 7;
+    if (cpt > 8) cpt = 8;
     const int threads = ((nchunks + cpt - 1) / cpt + kWave - 1) / kWave * kWave;
     const float inv_n = 1.0f / (float)K;
     const size_t in_tensors = kSrc == kQSwiglu ? 2 : 1;
@@ -200,12 +331,19 @@ vv_status_t launch_quant(const void* a, const void* b, int M, int K, float eps, 
     const Chunk* pa = static_cast<const Chunk*>(a);
     const Chunk* pb = static_cast<const Chunk*>(b);
     const dim3 grid((unsigned)M);
-#define VV_Q_LAUNCH(C, S) \
-    quant_rows_wg<C, kSrc, S><<<grid, threads, 0, st>>>(pa, pb, nchunks, inv_n, eps, layout, xq, sx, xsum)
-#define VV_Q_CASE(C) \
-    case C: if (stream) VV_Q_LAUNCH(C, true); else VV_Q_LAUNCH(C, false); break;
-    switch (cpt) { VV_Q_CASE(1) VV_Q_CASE(2) VV_Q_CASE(3) }
-#undef VV_Q_CASE
+#define VV_Q_LAUNCH(C, R, S)                                                                   \
+    quant_rows_wg<C, R, kSrc, S><<<grid, threads, 0, st>>>(pa, pb, M, nchunks, inv_n, eps, layout, \
+                                                          xq, sx, xsum)
+#define VV_Q_PICK(C, R) do { if (stream) VV_Q_LAUNCH(C, R, true); else VV_Q_LAUNCH(C, R, false); } while (0)
+    switch (cpt) {
+        case 1: VV_Q_PICK(1, 1); break;
+        case 2: VV_Q_PICK(2, 1); break;
+        case 3: VV_Q_PICK(3, 1); break;
+        case 4: VV_Q_PICK(4, 1); break;
+        case 7: VV_Q_PICK(7, 1); break;
+        default: VV_Q_PICK(8, 1); break;
+    }
+#undef VV_Q_PICK
 #undef VV_Q_LAUNCH
     return launch_status();
 }

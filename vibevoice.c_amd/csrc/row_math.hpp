@@ -44,6 +44,42 @@ __device__ __forceinline__ float block_sum(float acc, float* partial) {
     return total;
 }
 
+// The same for kN independent values at once (kN rows sharing a workgroup): one
+// barrier for all of them. `partial` is kN x kMaxWgWaves floats of LDS.
+template <int kN>
+__device__ __forceinline__ void block_sum_n(float (&acc)[kN], float (*partial)[kMaxWgWaves]) {
+#pragma unroll
+    for (int r = 0; r < kN; ++r) {
+        const float w = wave_sum(acc[r]);
+        if (lane_id() == 0) partial[r][threadIdx.x >> 6] = w;
+    }
+    __syncthreads();
+    const int nwaves = (int)blockDim.x >> 6;
+#pragma unroll
+    for (int r = 0; r < kN; ++r) {
+        float total = 0.0f;
+        for (int i = 0; i < nwaves; ++i) total += partial[r][i];
+        acc[r] = total;
+    }
+}
+
+template <int kN>
+__device__ __forceinline__ void block_max_n(float (&v)[kN], float (*partial)[kMaxWgWaves]) {
+#pragma unroll
+    for (int r = 0; r < kN; ++r) {
+        const float w = wave_max(v[r]);
+        if (lane_id() == 0) partial[r][threadIdx.x >> 6] = w;
+    }
+    __syncthreads();
+    const int nwaves = (int)blockDim.x >> 6;
+#pragma unroll
+    for (int r = 0; r < kN; ++r) {
+        float m = 0.0f;
+        for (int i = 0; i < nwaves; ++i) m = fmaxf(m, partial[r][i]);
+        v[r] = m;
+    }
+}
+
 // (x * inv) * w per element, two roundings, then one FP16 rounding.
 __device__ __forceinline__ Chunk scale_chunk(const Chunk& x16, float inv, const Chunk& w16) {
     f32x8 x = unpack(x16);
