@@ -71,6 +71,10 @@ def _load():
     lib.vvo_q8_pos.argtypes = [C.c_int, C.c_int]
     lib.vvo_quant_act_q8.restype = C.c_int
     lib.vvo_quant_act_q8.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8), _f32p, _i32p]
+    lib.vvo_gemm_f16w.restype = C.c_int
+    lib.vvo_gemm_f16w.argtypes = [_f32p, _u16p, _u16p, _f32p, C.c_int, C.c_int, C.c_int]
+    lib.vvo_attention_prefill_f32.restype = C.c_int
+    lib.vvo_attention_prefill_f32.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 7
     lib.vvo_threads.restype = C.c_int
     lib.vvo_set_threads.argtypes = [C.c_int]
     for name in ("vvo_rmsnorm_f32", "vvo_rope_f32", "vvo_swiglu_f32", "vvo_residual_add_f32",
@@ -96,6 +100,10 @@ def _load_ref():
                  "vv_embedding_cpu", "vv_cpu_threads", "vv_cpu_physical_cores"):
         getattr(ref, name).restype = C.c_int
     ref.vv_cpu_simd_name.restype = C.c_char_p
+    ref.vv_gemm_f16w_cpu.restype = C.c_int
+    ref.vv_gemm_f16w_cpu.argtypes = [_f32p, vp, vp, _f32p, C.c_int, C.c_int, C.c_int]
+    ref.vv_attention_prefill_cpu.restype = C.c_int
+    ref.vv_attention_prefill_cpu.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 6 + [C.c_bool]
     if hasattr(ref, "vv_quant_act_q8_cpu"):
         ref.vv_quant_act_q8_cpu.restype = C.c_int
         ref.vv_quant_act_q8_cpu.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8),
@@ -277,3 +285,28 @@ def quant_act_q8(x: np.ndarray, layout: int, want_xsum: bool = True):
                                 _p(sx, _f32p), _p(xs, _i32p) if want_xsum else None),
            "quant_act_q8")
     return xq, sx, xs
+
+
+def gemm_f16w(x: np.ndarray, w16: np.ndarray, bias16=None) -> np.ndarray:
+    """float32 x [M,K] times FP16 weight bits [N,K] (transposed) + FP16 bias bits [N]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    N = w16.shape[0]
+    out = np.empty((M, N), dtype=np.float32)
+    _check(lib.vvo_gemm_f16w(_p(x, _f32p), _p(w16, _u16p),
+                             _p(bias16, _u16p) if bias16 is not None else None,
+                             _p(out, _f32p), M, N, K), "gemm_f16w")
+    return out
+
+
+def attention_prefill_f32(q, k, v, q_offset: int, kv_len: int, causal: bool = True) -> np.ndarray:
+    """q [rows, n_q, hd], k/v [kv_len, n_kv, hd] float32 -> out like q."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    rows, n_q, hd = q.shape
+    out = np.empty_like(q)
+    _check(lib.vvo_attention_prefill_f32(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), _p(out, _f32p),
+                                         n_q, k.shape[1], hd, rows, q_offset, kv_len, int(causal)),
+           "attention_prefill_f32")
+    return out

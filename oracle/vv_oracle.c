@@ -332,6 +332,69 @@ int vvo_quant_act_q8(const float* x, int M, int K, int layout, int8_t* xq,
     return VVO_OK;
 }
 
+/* ── the layer's two contractions ─────────────────────────────────────── */
+
+int vvo_gemm_f16w(const float* x, const uint16_t* w, const uint16_t* bias,
+                  float* out, int M, int N, int K) {
+    if (!x || !w || !out) return VVO_ERR_NULL_PTR;
+    int n;
+#pragma omp parallel for schedule(static)
+    for (n = 0; n < N; n++) {
+        const uint16_t* wr = w + (size_t)n * K;
+        const float b = bias ? vvo_half_to_float(bias[n]) : 0.0f;
+        for (int m = 0; m < M; m++) {
+            const float* xr = x + (size_t)m * K;
+            double acc = 0.0;
+            for (int k = 0; k < K; k++) acc += (double)xr[k] * (double)vvo_half_to_float(wr[k]);
+            out[(size_t)m * N + n] = (float)acc + b;
+        }
+    }
+    return VVO_OK;
+}
+
+int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
+                              float* out, int n_q_heads, int n_kv_heads,
+                              int head_dim, int rows, int q_offset, int kv_len,
+                              int causal) {
+    /* cpu_kernels.c:1480-1525. Per (row, head): running maximum m, running
+     * denominator l, output rescaled by expf(m_old - m_new) at every key. */
+    if (!q || !k || !v || !out) return VVO_ERR_NULL_PTR;
+    const int group = n_q_heads / n_kv_heads;
+    const size_t q_stride = (size_t)n_q_heads * head_dim;
+    const size_t kv_stride = (size_t)n_kv_heads * head_dim;
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    int r;
+#pragma omp parallel for schedule(static)
+    for (r = 0; r < rows; r++) {
+        for (int h = 0; h < n_q_heads; h++) {
+            const int kvh = h / group;
+            const int q_abs = q_offset + r;
+            int limit = kv_len;
+            if (causal && q_abs + 1 < kv_len) limit = q_abs + 1;
+            const float* qv = q + (size_t)r * q_stride + (size_t)h * head_dim;
+            float* ov = out + (size_t)r * q_stride + (size_t)h * head_dim;
+            float m_run = -INFINITY, l_run = 0.0f;
+            for (int d = 0; d < head_dim; d++) ov[d] = 0.0f;
+            for (int t = 0; t < limit; t++) {
+                const float* kt = k + (size_t)t * kv_stride + (size_t)kvh * head_dim;
+                const float* vt = v + (size_t)t * kv_stride + (size_t)kvh * head_dim;
+                float dot = 0.0f;
+                for (int d = 0; d < head_dim; d++) dot += qv[d] * kt[d];
+                const float sc = dot * scale;
+                const float m_new = sc > m_run ? sc : m_run;
+                const float a = (m_run == -INFINITY) ? 0.0f : expf(m_run - m_new);
+                const float p = expf(sc - m_new);
+                for (int d = 0; d < head_dim; d++) ov[d] = ov[d] * a + p * vt[d];
+                l_run = l_run * a + p;
+                m_run = m_new;
+            }
+            const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+            for (int d = 0; d < head_dim; d++) ov[d] *= inv;
+        }
+    }
+    return VVO_OK;
+}
+
 /* ── seeded inputs ─────────────────────────────────────────────────────── */
 
 static inline uint64_t splitmix64(uint64_t z) {

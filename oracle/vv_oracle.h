@@ -106,6 +106,24 @@ int vvo_q8_pos(int layout, int j);
 int vvo_quant_act_q8(const float* x, int M, int K, int layout, int8_t* xq,
                      float* sx, int32_t* xsum);
 
+/* ── the layer's two contractions (checkers for the layer runner) ─────── */
+
+/* out[m,n] = sum_k x[m,k] * w[n,k] + bias[n]; x FP32 [M,K], w FP16 [N,K],
+ * bias FP16 [N] or NULL. The reference's CPU kernel (src/cpu/cpu_kernels.c:
+ * 1325-1360) sums in a SIMD-dependent order; this is the double-accumulated
+ * form its own test holds it to at 1e-5 (tests/test_cpu_kernels.c:128-147). */
+int vvo_gemm_f16w(const float* x, const uint16_t* w, const uint16_t* bias,
+                  float* out, int M, int N, int K);
+
+/* src/cpu/cpu_kernels.c:1480-1525: causal GQA attention, one pass with an
+ * online softmax. q, out [rows, n_q_heads, head_dim]; k, v [kv_len,
+ * n_kv_heads, head_dim]; query r sits at absolute position q_offset + r and
+ * sees keys 0 .. min(q_offset + r + 1, kv_len) - 1 when causal. */
+int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
+                              float* out, int n_q_heads, int n_kv_heads,
+                              int head_dim, int rows, int q_offset, int kv_len,
+                              int causal);
+
 /* ── seeded inputs (the same bytes go to the oracle and to the GPU) ────── */
 
 /* N(mean, std) rounded to FP16 (RNE). Counter-based: element i depends only
