@@ -121,6 +121,22 @@ vv_status_t vv_swiglu_q8_dev(const void* gate, const void* up, int M, int K,
  * (src/cuda/act_quant.cu:277-313). */
 vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* stream);
 
+/* ── Dense linear layers ───────────────────────────────────────────────── */
+
+/* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32
+ * accumulation on the matrix cores. beta == 0 never reads C. M <= 8 streams
+ * the weight rows once (one wave per output column); larger M runs 32x64,
+ * 64x64 or 128x128 workgroup tiles, all of which add K in the same order and
+ * so give the same bits for an element. K % 8 != 0 or A/B off 16 bytes take a
+ * scalar kernel. M <= 0 or N <= 0: VV_OK, nothing launched.
+ * replaces device.h:423-425 (src/cuda/gemm.cu). */
+vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N,
+                             int K, float alpha, float beta, void* stream);
+/* The 128x128 tile alone, whatever M. replaces device.h:432-434. */
+vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
+                                  int N, int K, float alpha, float beta,
+                                  void* stream);
+
 /* ── Fused forms (additions) ───────────────────────────────────────────── */
 
 /* addition: vv_residual_add_dev(residual, x) followed by

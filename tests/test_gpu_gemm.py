@@ -1,0 +1,107 @@
+"""GPU parity tests of the dense FP16 GEMM (C = alpha * A * B^T + beta * C)
+through the C ABI, against the oracle's double-accumulated product.
+
+Bars: the stated one for FP16 outputs (scaled error <= 2e-3) and an
+elementwise one of our own: half an FP16 ulp of the exact value plus 1e-5 of
+sum_k |a||b| (FP32 accumulation over K <= 18944 stays well inside that).
+Bit-exact: every tile shape against the 128x128 tile (same K order), beta = 0
+never reading C, M <= 0 / N <= 0 launching nothing.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import FP16_TOL, bits_of, dev, ok, stream, to_dev
+from conftest import scaled_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def exact(a_bits, b_bits, c_bits, alpha, beta):
+    a = oracle.widen(a_bits)
+    ref = alpha * oracle.gemm_f16w(a, b_bits).astype(np.float64)
+    if beta != 0.0:
+        ref = ref + beta * oracle.widen(c_bits).astype(np.float64)
+    mag = abs(alpha) * (np.abs(a).astype(np.float64) @ np.abs(oracle.widen(b_bits)).astype(np.float64).T)
+    return ref, mag
+
+
+def check(got_bits, ref, mag, what):
+    got = oracle.widen(got_bits).astype(np.float64)
+    err = scaled_rel_err(got, ref)
+    assert err <= FP16_TOL, f"{what}: scaled error {err:.3e}"
+    with np.errstate(over="ignore"):
+        ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64)
+    bound = 0.5 * ulp + 1e-5 * mag + 2.0 ** -25
+    worst = float(np.max(np.abs(got - ref) / bound))
+    assert worst <= 1.0, f"{what}: {worst:.3f}x the elementwise bound"
+
+
+def run(fn, d_a, d_b, d_c, M, N, K, alpha=1.0, beta=0.0):
+    ok(fn(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr(), M, N, K, alpha, beta, stream()))
+    return bits_of(d_c)
+
+
+SHAPES = [(1, 64, 64), (1, 3584, 3584), (3, 512, 3584), (8, 1000, 1536), (9, 64, 64),
+          (29, 3584, 3584), (29, 512, 3584), (33, 4608, 1536), (64, 256, 512), (100, 128, 72),
+          (285, 3584, 3584), (130, 101, 200), (257, 37, 8), (48, 512, 256), (70, 3584, 18944)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm_against_oracle_and_tile(M, N, K):
+    a = oracle.normal_f16((M, K), 100 + M)
+    b = oracle.normal_f16((N, K), 200 + N, std=K ** -0.5)
+    d_a, d_b = to_dev(a), to_dev(b)
+    d_c = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    got = run(dev.vv_gemm_fp16_dev, d_a, d_b, d_c, M, N, K)     # beta = 0 over NaNs
+    ref, mag = exact(a, b, None, 1.0, 0.0)
+    check(got, ref, mag, f"gemm {M}x{N}x{K}")
+    d_t = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    tile = run(dev.vv_gemm_fp16_tile_dev, d_a, d_b, d_t, M, N, K)
+    check(tile, ref, mag, f"tile {M}x{N}x{K}")
+    if M > 8:
+        assert np.array_equal(got, tile), "tile shapes must agree bit for bit"
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (5, 100, 64), (29, 256, 512), (200, 264, 136)])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 1.0), (0.5, -2.0), (-1.25, 0.0)])
+def test_gemm_alpha_beta(M, N, K, alpha, beta):
+    a = oracle.normal_f16((M, K), 1)
+    b = oracle.normal_f16((N, K), 2, std=K ** -0.5)
+    c = oracle.normal_f16((M, N), 3)
+    ref, mag = exact(a, b, c, alpha, beta)
+    mag = mag + abs(beta) * np.abs(oracle.widen(c))
+    for fn in (dev.vv_gemm_fp16_dev, dev.vv_gemm_fp16_tile_dev):
+        got = run(fn, to_dev(a), to_dev(b), to_dev(c), M, N, K, alpha, beta)
+        check(got, ref, mag, f"alpha {alpha} beta {beta}")
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 40, 131), (20, 33, 7), (70, 130, 100)])
+def test_gemm_scalar_path(M, N, K):
+    """K % 8 != 0, and operands that start 2 bytes off a 16-byte boundary."""
+    a = oracle.normal_f16((M, K), 4)
+    b = oracle.normal_f16((N, K), 5, std=K ** -0.5)
+    ref, mag = exact(a, b, None, 1.0, 0.0)
+    d_c = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    check(run(dev.vv_gemm_fp16_dev, to_dev(a), to_dev(b), d_c, M, N, K), ref, mag, "odd K")
+    pad = torch.zeros(M * K + 1, dtype=torch.float16, device="cuda")
+    pad[1:] = to_dev(a).reshape(-1)
+    d_c.zero_()
+    ok(dev.vv_gemm_fp16_dev(pad.data_ptr() + 2, to_dev(b).data_ptr(), d_c.data_ptr(), M, N, K,
+                            1.0, 0.0, stream()))
+    check(bits_of(d_c), ref, mag, "misaligned A")
+
+
+def test_gemm_edges():
+    d = torch.ones(64, dtype=torch.float16, device="cuda")
+    p = d.data_ptr()
+    assert dev.vv_gemm_fp16_dev(None, p, p, 1, 1, 8, 1.0, 0.0, stream()) == dev.VV_ERR_NULL_PTR
+    assert dev.vv_gemm_fp16_dev(p, p, p, 0, 8, 8, 1.0, 0.0, stream()) == dev.VV_OK
+    assert dev.vv_gemm_fp16_tile_dev(p, p, p, 4, 0, 8, 1.0, 0.0, stream()) == dev.VV_OK
+    assert bits_of(d).tolist() == [0x3C00] * 64
+    # K == 0: C = beta * C
+    c = to_dev(oracle.normal_f16((2, 8), 9))
+    want = (2.0 * oracle.widen(bits_of(c))).astype(np.float16).view(np.uint16)
+    ok(dev.vv_gemm_fp16_dev(p, p, c.data_ptr(), 2, 8, 0, 1.0, 2.0, stream()))
+    assert np.array_equal(bits_of(c), want)

@@ -1,0 +1,307 @@
+// Dense linear layers: C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C, all FP16
+// row-major, FP32 accumulation.
+//
+// Both operands are contiguous along K, which is what the CDNA4 matrix core
+// wants: v_mfma_f32_32x32x16_f16 takes, per lane, eight consecutive K values
+// of one row of each operand. Three kernels:
+//
+//   gemm_tile<BM,BN,WM,WN>  workgroup tile BM x BN over WM x WN waves, K in
+//                           slabs of 64 staged through LDS (double-buffered,
+//                           16-byte slots XOR-swizzled so that the 32 rows a
+//                           ds_read_b128 touches fall in distinct banks). The
+//                           weight rows are the MFMA's A operand and the
+//                           activation rows its B operand, so a lane ends up
+//                           with four CONSECUTIVE output columns of one output
+//                           row: 8-byte stores. Every tile shape adds the K
+//                           slabs in the same order, so all of them produce
+//                           the same bits for the same element.
+//   gemv_rows<MR>           M <= 8 (a decode step): one wave per output
+//                           column streams that weight row once with
+//                           non-temporal 16-byte loads and keeps MR dot
+//                           products; bound by the weight bytes.
+//   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
+#include "vv_common.hpp"
+
+namespace vv {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kSlab = 64;                 // K values per LDS slab
+constexpr int kSlabChunks = kSlab / 8;    // 16-byte slots per slab row
+
+// Slot swizzle: rows are 128 B = 32 banks apart, so two rows share a 64-bank
+// line; XOR-ing the slot with (row / 2) % 8 spreads any 16 consecutive rows
+// reading the same logical slot over all 64 banks.
+__device__ __forceinline__ int swz(int row, int slot) { return slot ^ ((row >> 1) & 7); }
+
+__device__ __forceinline__ float finish(float acc, float alpha, float beta, h16 old) {
+    return alpha * acc + beta * (float)old;
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
+    const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
+    int K, float alpha, float beta, int vec_store) {
+    constexpr int NT = WM * WN * kWave;
+    constexpr int TM = BM / WM / 32;          // 32x32 MFMA tiles per wave along M
+    constexpr int TN = BN / WN / 32;          // and along N
+    constexpr int LA = BM * kSlabChunks / NT; // 16-byte loads per thread per slab, A
+    constexpr int LB = BN * kSlabChunks / NT;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiles are 32x32 multiples");
+    static_assert(LA >= 1 && LB >= 1 && (BM * kSlabChunks) % NT == 0 && (BN * kSlabChunks) % NT == 0,
+                  "slab loads must divide evenly over the threads");
+
+    __shared__ Chunk sA[2][BM * kSlabChunks];
+    __shared__ Chunk sB[2][BN * kSlabChunks];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int m_blk = (int)blockIdx.y * BM;
+    const int n_blk = (int)blockIdx.x * BN;
+    const int kchunks = K / 8;
+    const int nslabs = (K + kSlab - 1) / kSlab;
+
+    Chunk ra[LA], rb[LB];
+    const Chunk zero = {{0u, 0u, 0u, 0u}};
+
+    auto fetch = [&](int slab) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
+            const int gm = min(m_blk + row, M - 1);
+            const int kc = slab * kSlabChunks + slot;
+            ra[i] = kc < kchunks
+                        ? load_chunk(reinterpret_cast<const Chunk*>(A + (size_t)gm * K) + kc)
+                        : zero;
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
+            const int gn = min(n_blk + row, N - 1);
+            const int kc = slab * kSlabChunks + slot;
+            rb[i] = kc < kchunks
+                        ? load_chunk(reinterpret_cast<const Chunk*>(B + (size_t)gn * K) + kc)
+                        : zero;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
+            sA[buf][row * kSlabChunks + swz(row, slot)] = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
+            sB[buf][row * kSlabChunks + swz(row, slot)] = rb[i];
+        }
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+
+    const int frow = lane & 31;       // operand row inside a 32x32 tile
+    const int fhalf = lane >> 5;      // which 8 of the step's 16 K values
+
+    for (int slab = 0; slab < nslabs; ++slab) {
+        const int buf = slab & 1;
+        if (slab + 1 < nslabs) fetch(slab + 1);
+#pragma unroll
+        for (int step = 0; step < kSlab / 16; ++step) {
+            const int slot = step * 2 + fhalf;
+            h16x8 fw[TN], fx[TM];
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                const int row = (wn * TN + a) * 32 + frow;
+                fw[a] = __builtin_bit_cast(h16x8, sB[buf][row * kSlabChunks + swz(row, slot)]);
+            }
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int row = (wm * TM + b) * 32 + frow;
+                fx[b] = __builtin_bit_cast(h16x8, sA[buf][row * kSlabChunks + swz(row, slot)]);
+            }
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[a], fx[b], acc[a][b],
+                                                                       0, 0, 0);
+        }
+        if (slab + 1 < nslabs) stage(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Result register 4g + r of lane l holds column n0 + 8g + 4(l / 32) + r of
+    // row m0 + l % 32.
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const int m = m_blk + (wm * TM + b) * 32 + frow;
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n_blk + (wn * TN + a) * 32 + 8 * g + 4 * fhalf;
+                if (n >= N) continue;
+                if (vec_store && n + 3 < N) {
+                    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+                    h16x4 old = {0, 0, 0, 0};
+                    if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+                    h16x4 o;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        o[r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old[r]));
+                    *reinterpret_cast<h16x4*>(crow + n) = o;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < N) {
+                            const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                            crow[n + r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old));
+                        }
+                }
+            }
+        }
+    }
+}
+
+// One wave per output column n; MR rows of A share each weight chunk.
+template <int MR>
+__global__ __launch_bounds__(kBlock) void gemv_rows(const h16* __restrict__ A,
+                                                    const h16* __restrict__ B,
+                                                    h16* __restrict__ C, int M, int N, int K,
+                                                    float alpha, float beta) {
+    const int n = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
+    if (n >= N) return;
+    const int lane = lane_id();
+    const int kchunks = K / 8;
+    const Chunk* w = reinterpret_cast<const Chunk*>(B + (size_t)n * K);
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+#pragma unroll 4
+    for (int c = lane; c < kchunks; c += kWave) {
+        const f32x8 wf = unpack(load_chunk_stream(w + c));
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            if (m < M) {
+                const f32x8 xf =
+                    unpack(load_chunk(reinterpret_cast<const Chunk*>(A + (size_t)m * K) + c));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[m] = fmaf(xf[i], wf[i], acc[m]);
+            }
+        }
+    }
+    float mine = 0.0f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float s = wave_sum(acc[m]);
+        if (lane == m) mine = s;
+    }
+    if (lane < M && lane < MR) {
+        h16* c = C + (size_t)lane * N + n;
+        const h16 old = beta != 0.0f ? *c : (h16)0.0f;
+        *c = to_half(finish(mine, alpha, beta, old));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gemm_naive(const h16* A, const h16* B, h16* C, int M,
+                                                     int N, int K, float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= (size_t)M * N) return;
+    const int m = (int)(i / N), n = (int)(i % N);
+    const h16* a = A + (size_t)m * K;
+    const h16* b = B + (size_t)n * K;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) acc = fmaf((float)a[k], (float)b[k], acc);
+    const h16 old = beta != 0.0f ? C[i] : (h16)0.0f;
+    C[i] = to_half(finish(acc, alpha, beta, old));
+}
+
+template <int BM, int BN, int WM, int WN>
+void launch_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                 float beta, hipStream_t st) {
+    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    gemm_tile<BM, BN, WM, WN><<<grid, WM * WN * kWave, 0, st>>>(
+        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K,
+        alpha, beta, vec);
+}
+
+enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3 };
+
+vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
+                 float beta, void* stream, int choice, bool allow_gemv) {
+    if (!A || !B || !C) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0) return VV_OK;
+    if (K < 0) return VV_ERR_INVALID_ARG;
+    hipStream_t st = as_stream(stream);
+    const h16* a = static_cast<const h16*>(A);
+    const h16* b = static_cast<const h16*>(B);
+    h16* c = static_cast<h16*>(C);
+
+    if (K % 8 != 0 || !aligned16(A) || !aligned16(B)) {
+        const size_t blocks = ((size_t)M * N + kBlock - 1) / kBlock;
+        gemm_naive<<<dim3((unsigned)blocks), kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        return launch_status();
+    }
+    if (allow_gemv && M <= 8) {
+        const dim3 grid((unsigned)((N + kWavesPerBlock - 1) / kWavesPerBlock));
+        if (M == 1) gemv_rows<1><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        else if (M <= 4) gemv_rows<4><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        else gemv_rows<8><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        return launch_status();
+    }
+    if (choice == kAuto) {
+        // The largest tile that still gives every compute unit a workgroup.
+        const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+        const long wg64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+        choice = (M > 64 && wg128 >= 256) ? k128 : (M > 32 && wg64 >= 128) ? k64
+                 : (M > 32) ? k64 : k32;
+    }
+    switch (choice) {
+        case k128: launch_tile<128, 128, 2, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k64:  launch_tile<64, 64, 2, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        default:   launch_tile<32, 64, 1, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+    }
+    return launch_status();
+}
+
+int forced_tile() {
+    static const int v = [] {
+        const char* e = getenv("VV_GEMM_TILE");
+        return e ? atoi(e) : 0;
+    }();
+    return (v >= 0 && v <= 3) ? v : 0;
+}
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N, int K,
+                             float alpha, float beta, void* stream) {
+    return vv::gemm(A, B, C, M, N, K, alpha, beta, stream, vv::forced_tile(), true);
+}
+
+vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M, int N, int K,
+                                  float alpha, float beta, void* stream) {
+    return vv::gemm(A, B, C, M, N, K, alpha, beta, stream, vv::k128, false);
+}
+
+}  // extern "C"

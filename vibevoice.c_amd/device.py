@@ -40,6 +40,8 @@ SIGNATURES = {
     "vv_rmsnorm_q8_dev": (_i, [_vp, _vp, _i, _i, _f, _i, _vp, _vp, _vp, _vp]),
     "vv_swiglu_q8_dev": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vv_col_absmax_dev": (_i, [_vp, _i, _i, _vp, _vp]),
+    "vv_gemm_fp16_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _f, _vp]),
+    "vv_gemm_fp16_tile_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _f, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
