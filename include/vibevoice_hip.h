@@ -137,6 +137,66 @@ vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
                                   int N, int K, float alpha, float beta,
                                   void* stream);
 
+/* ── Attention over an FP16 KV cache ───────────────────────────────────── */
+
+/* One layer of a KV cache as the attention kernels see it: k, v are
+ * [row][n_kv_heads][head_dim] FP16, row = position, or with a (device)
+ * page_table position t lives at row page_table[t / 64] * 64 + t % 64.
+ * Same layout as device.h:527-536. */
+typedef struct vv_kv_view {
+    const void* k;
+    const void* v;
+    const void* k_meta;       /* quantised formats only: unused here */
+    const void* v_meta;
+    const int*  page_table;   /* device memory, or NULL */
+    int         format;       /* vv_kv_format_t; only VV_KV_FP16 (0) is served */
+    int         n_kv_heads;
+    int         head_dim;
+} vv_kv_view_t;
+
+/* The backend a context should name (never VV_ATTN_AUTO = 0). All backend
+ * names run the same kernels here; a format other than FP16 answers
+ * VV_ATTN_FA1 (1) and the attention calls then decline.
+ * replaces device.h:545-546 (src/cuda/attention_fi.cu:554-583). */
+int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
+                    int n_kv_heads, int head_dim);
+/* n_q_heads * 64 * (head_dim + 2) floats: the decode slices' partial states.
+ * replaces device.h:554 (attention_fi.cu:585-589). */
+size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim);
+/* The number of slices the decode splits `cache_len` positions into: 1, 2,
+ * 4 ... 64, doubling as the length passes 256, 512, ... A captured decode
+ * step is valid while this stays equal. replaces device.h:562-563. */
+int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len);
+/* q_len query rows at absolute positions q_offset.. against the first kv_len
+ * positions of the cache; Q, O [q_len][n_q_heads][head_dim] FP16; causal:
+ * query p sees positions <= p. head_dim 128 with 16-byte aligned pointers
+ * runs on the matrix cores, any other head_dim <= 256 a wave per row.
+ * A format other than FP16, head_dim > 256 or n_q_heads % n_kv_heads != 0:
+ * VV_ERR_UNSUPPORTED. replaces device.h:575-578 (attention_fi.cu:600-632). */
+vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv,
+                            void* out, int n_q_heads, int q_len, int q_offset,
+                            int kv_len, bool causal, void* scratch, void* stream);
+/* One query row per head against the whole cache. cache_len sizes the launch;
+ * d_cache_len (device int, or NULL) holds the exact length and need only be in
+ * the same vv_attn_decode_shape() bucket. scratch: vv_attn_scratch_bytes()
+ * of device memory owned by the caller (may be NULL while the shape is 1).
+ * replaces device.h:586-589 (attention_fi.cu:634-660). */
+vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv,
+                           void* out, int n_q_heads, int cache_len,
+                           const int* d_cache_len, void* scratch, void* stream);
+/* Copy K/V rows [n_positions][n_kv_heads][head_dim] into an FP16 cache layer
+ * at positions pos.. (or *d_pos..), through page_table when it is set.
+ * Other formats: VV_ERR_UNSUPPORTED. replaces device.h:597-602. */
+vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_store,
+                            void* v_store, void* k_meta, void* v_meta, void* k_ref,
+                            bool build_ref, int n_kv_heads, int head_dim, int pos,
+                            const int* d_pos, int n_positions, int kv_format,
+                            const int* page_table, void* stream);
+/* page_table[first + i] = pages[i], i < n, ordered on the stream; `pages` is
+ * host memory, consumed before the call returns. replaces device.h:610-611. */
+vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages,
+                               void* stream);
+
 /* ── Fused forms (additions) ───────────────────────────────────────────── */
 
 /* addition: vv_residual_add_dev(residual, x) followed by

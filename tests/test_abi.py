@@ -108,6 +108,22 @@ def test_declined_arguments():
     dev.vv_dev_graph_destroy(None)      # no-op, must not crash
 
 
+def test_attention_host_queries():
+    """The three attention queries run on the host and launch nothing."""
+    AUTO, FA1, FA2, FI = 0, 1, 2, 3
+    for requested in (AUTO, FA1, FA2, FI):
+        for paged in (False, True):
+            got = dev.vv_attn_resolve(requested, 0, paged, 28, 4, 128)
+            assert got in (FA1, FA2, FI) and (requested in (AUTO, got) or paged)
+            assert dev.vv_attn_resolve(requested, 3, paged, 28, 4, 128) == FA1     # not an FP16 cache
+    assert dev.vv_attn_resolve(FA1, 0, True, 28, 4, 128) != FA1                    # fa1 never pages
+    assert dev.vv_attn_scratch_bytes(28, 4, 128) == 28 * 64 * 130 * 4
+    shapes = [dev.vv_attn_decode_shape(FA2, 28, 4, n) for n in range(1, 20000, 37)]
+    assert shapes == sorted(shapes) and shapes[0] == 1 and shapes[-1] == 64
+    assert set(shapes) <= {1, 2, 4, 8, 16, 32, 64}
+    assert dev.vv_attn_decode_shape(FA2, 28, 4, 256) == 1 and dev.vv_attn_decode_shape(FA2, 28, 4, 257) == 2
+
+
 # ── the declined remainder of the seam ──────────────────────────────────────
 
 STUB_PATH = os.path.join(os.path.dirname(dev.LIB_PATH), "libvibevoice_hip_unsupported.so")
@@ -117,10 +133,10 @@ def test_unsupported_library_declines_everything_and_overlaps_nothing():
     import ctypes as C
     out = subprocess.check_output(["nm", "-D", "--defined-only", STUB_PATH], text=True)
     stubs = sorted(l.split()[-1] for l in out.splitlines() if " T vv_" in l)
-    assert len(stubs) == 55
+    assert len(stubs) == 48
     assert not set(stubs) & set(dev.SIGNATURES)          # no symbol defined twice
     lib = C.CDLL(STUB_PATH)
-    zero = {"vv_attn_resolve", "vv_attn_decode_shape", "vv_gqa_decode_shape", "vv_attn_scratch_bytes",
+    zero = {"vv_gqa_decode_shape",
             "vv_gqa_decode_scratch_bytes", "vv_i8_head_argmax_scratch_bytes"}
     for name in stubs:
         fn = getattr(lib, name)
@@ -148,6 +164,7 @@ def test_the_two_libraries_define_every_symbol_of_the_reference_seam():
         out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
         have |= {l.split()[-1] for l in out.splitlines() if " T vv_" in l}
     assert len(wanted) >= 100 and not (wanted - have), sorted(wanted - have)
-    # what we add beyond the reference's seam: the fused entry points only
+    # beyond device.h: the fused entry points, and the two kv_quant.h symbols
+    # (kv_quant.h:96-101) the decoder links against, declined
     assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
-                             "vv_embedding_rmsnorm_dev"}
+                             "vv_embedding_rmsnorm_dev", "vv_kv_rotate_dev", "vv_kv_unrotate_dev"}

@@ -1,0 +1,551 @@
+// Causal grouped-query attention over an FP16 KV cache: the prefill form
+// (q_len rows against the first kv_len positions) and the decode form (one
+// row per head against the whole cache), plus the FP16 cache store.
+//
+// Q, O are [rows][n_q_heads][head_dim]; the cache is [row][n_kv_heads]
+// [head_dim], row = position, or, with a page table, page_table[t / 64] * 64
+// + t % 64. Every kernel keeps the softmax online (running maximum and
+// denominator in FP32, in the base-2 domain: v_exp_f32 is 2^x).
+//
+//   prefill128   head_dim 128 on the matrix cores. A workgroup owns 128
+//                query rows of one head, a wave 32 of them; keys come in
+//                tiles of 64 through LDS. The products are computed
+//                TRANSPOSED: S^T = K Q^T puts one query row in each lane
+//                (lane % 32) with 32 of the tile's keys in its registers, so
+//                the row maximum and sum are register reductions plus one
+//                exchange with lane ^ 32, the rescale of O is one factor per
+//                lane, and the probabilities, rounded to FP16, are already
+//                laid out as the B operand of O^T = V^T P^T. V is transposed
+//                on its way into LDS (four keys of one channel per 8-byte
+//                slot) so the A operand of that product is two 8-byte reads.
+//   decode_part  one query row: bound by the cache bytes. A workgroup takes
+//                one KV head and one slice of the positions; 16 lanes share a
+//                key row (16 bytes each), all query heads of the group reuse
+//                it from registers. Slices leave (max, sum, unnormalised O)
+//                in the caller's scratch and decode_merge folds them.
+//   rows_generic any head_dim <= 256, any alignment: one wave per (row, head).
+#include "vv_common.hpp"
+
+namespace vv {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kPage = 64;            // positions per page (include/vibevoice/kv_quant.h:52)
+constexpr int kFormatFp16 = 0;       // VV_KV_FP16
+constexpr int kMaxParts = 64;        // decode slices per KV head
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float other_half(float v) { return __shfl_xor(v, 32); }
+
+__device__ __forceinline__ int cache_row(const int* page_table, int t) {
+    return page_table ? page_table[t / kPage] * kPage + t % kPage : t;
+}
+
+// ── prefill, head_dim 128 ────────────────────────────────────────────────
+constexpr int kD = 128;
+constexpr int kQTile = 128;          // query rows per workgroup (32 per wave)
+constexpr int kKeyTile = 64;         // keys per LDS tile
+constexpr int kVtStride = kKeyTile + 4;   // halves per transposed-V row: 136 B
+
+__global__ __launch_bounds__(kBlock) void prefill128(
+    const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
+    const int* __restrict__ page_table, h16* __restrict__ O, int n_q_heads, int n_kv_heads,
+    int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
+    __shared__ Chunk sK[kKeyTile * (kD / 8)];          // [key][16 slots], slot ^ (key & 15)
+    __shared__ __align__(16) h16 sVt[kD * kVtStride];  // [channel][key]
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int col = lane & 31;        // this lane's query row inside the wave's 32
+    const int half = lane >> 5;
+    const int head = (int)blockIdx.y;
+    const int kvh = head / (n_q_heads / n_kv_heads);
+    const int q0 = (int)blockIdx.x * kQTile;
+    const int qw0 = q0 + wave * 32;
+    const int qrow = qw0 + col;
+    const int q_abs = q_offset + qrow;
+    const size_t kv_stride = (size_t)n_kv_heads * kD;
+
+    // Keys any row of the workgroup / of this wave may see.
+    int wg_limit = kv_len, wave_limit = qw0 < q_len ? kv_len : 0;
+    if (causal) {
+        wg_limit = min(kv_len, q_offset + min(q0 + kQTile, q_len));
+        wave_limit = qw0 < q_len ? min(kv_len, q_offset + min(qw0 + 32, q_len)) : 0;
+    }
+
+    h16x8 qf[kD / 16];
+    {
+        const h16* qp = Q + ((size_t)min(qrow, q_len - 1) * n_q_heads + head) * kD;
+#pragma unroll
+        for (int s = 0; s < kD / 16; ++s)
+            qf[s] = __builtin_bit_cast(h16x8,
+                                       load_chunk(reinterpret_cast<const Chunk*>(qp) + 2 * s + half));
+    }
+
+    f32x16 oacc[kD / 32];
+#pragma unroll
+    for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    for (int t0 = 0; t0 < wg_limit; t0 += kKeyTile) {
+        __syncthreads();
+        // K tile: four 16-byte slots per thread.
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q = tid + i * kBlock, r = q >> 4, slot = q & 15;
+            const int row = cache_row(page_table, min(t0 + r, kv_len - 1));
+            sK[r * 16 + (slot ^ (r & 15))] =
+                load_chunk(reinterpret_cast<const Chunk*>(Kc + (size_t)row * kv_stride + kvh * kD) + slot);
+        }
+        // V tile, transposed: a thread takes four consecutive keys of one
+        // 8-channel chunk and writes, per channel, the four keys as 8 bytes.
+        {
+            const int dchunk = tid & 15, kg = tid >> 4;
+            h16x8 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = cache_row(page_table, min(t0 + 4 * kg + j, kv_len - 1));
+                v[j] = __builtin_bit_cast(
+                    h16x8, load_chunk(reinterpret_cast<const Chunk*>(Vc + (size_t)row * kv_stride + kvh * kD) + dchunk));
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const h16x4 w = {v[0][i], v[1][i], v[2][i], v[3][i]};
+                *reinterpret_cast<h16x4*>(&sVt[(8 * dchunk + i) * kVtStride + 4 * kg]) = w;
+            }
+        }
+        __syncthreads();
+        if (t0 >= wave_limit) continue;
+
+        // S^T = K Q^T: register 4g + r of tile a is key t0 + 32a + 8g + 4*half + r.
+        f32x16 s[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[a][r] = 0.0f;
+#pragma unroll
+            for (int st = 0; st < kD / 16; ++st) {
+                const int row = 32 * a + col, slot = 2 * st + half;
+                const h16x8 kf = __builtin_bit_cast(h16x8, sK[row * 16 + (slot ^ (row & 15))]);
+                s[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[st], s[a], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
+                const bool seen = key < kv_len && (!causal || key <= q_abs);
+                const float x = seen ? s[a][r] * scale_log2 : -INFINITY;
+                s[a][r] = x;
+                mx = fmaxf(mx, x);
+            }
+        mx = fmaxf(mx, other_half(mx));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2_fast(m_run - m_use);
+        float sum = 0.0f;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = exp2_fast(s[a][r] - m_use);
+                s[a][r] = p;
+                sum += p;
+            }
+        sum += other_half(sum);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+
+        // O^T += V^T P^T over the tile's four 16-key steps. Slot e of this
+        // lane in step (a, sp) is register 8*sp + e of tile a, i.e. key
+        // 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte reads below.
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int a = u >> 1, sp = u & 1;
+            h16x8 pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = (h16)s[a][8 * sp + e];
+#pragma unroll
+            for (int t = 0; t < kD / 32; ++t) {
+                const h16* base = &sVt[(32 * t + col) * kVtStride + 32 * a + 16 * sp + 4 * half];
+                const h16x4 lo = *reinterpret_cast<const h16x4*>(base);
+                const h16x4 hi = *reinterpret_cast<const h16x4*>(base + 8);
+                const h16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[t], 0, 0, 0);
+            }
+        }
+    }
+
+    if (qrow < q_len) {
+        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = to_half(oacc[t][4 * g + r] * inv);
+                *reinterpret_cast<h16x4*>(op + 32 * t + 8 * g + 4 * half) = o;
+            }
+    }
+}
+
+// ── any head_dim <= 256: one wave per (query row, head) ──────────────────
+__global__ __launch_bounds__(kWave) void rows_generic(
+    const h16* Q, const h16* Kc, const h16* Vc, const int* page_table, h16* O, int n_q_heads,
+    int n_kv_heads, int head_dim, int q_len, int q_offset, int kv_len, const int* d_kv_len,
+    int causal, float scale_log2) {
+    const int qrow = (int)blockIdx.x, head = (int)blockIdx.y;
+    const int lane = lane_id();
+    const int kvh = head / (n_q_heads / n_kv_heads);
+    if (d_kv_len) kv_len = *d_kv_len;
+    int limit = kv_len;
+    if (causal) limit = min(kv_len, q_offset + qrow + 1);
+    const h16* qp = Q + ((size_t)qrow * n_q_heads + head) * head_dim;
+    float q[4], acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        q[j] = d < head_dim ? (float)qp[d] * scale_log2 : 0.0f;
+        acc[j] = 0.0f;
+    }
+    float m_run = -INFINITY, l_run = 0.0f;
+    for (int t = 0; t < limit; ++t) {
+        const size_t off = ((size_t)cache_row(page_table, t) * n_kv_heads + kvh) * head_dim;
+        float part = 0.0f, v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + 64 * j;
+            part += d < head_dim ? q[j] * (float)Kc[off + d] : 0.0f;
+            v[j] = d < head_dim ? (float)Vc[off + d] : 0.0f;
+        }
+        const float x = wave_sum(part);
+        const float m_new = fmaxf(m_run, x);
+        const float alpha = exp2_fast(m_run - m_new);
+        const float p = exp2_fast(x - m_new);
+        l_run = l_run * alpha + p;
+        m_run = m_new;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = acc[j] * alpha + p * v[j];
+    }
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    h16* op = O + ((size_t)qrow * n_q_heads + head) * head_dim;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        if (d < head_dim) op[d] = to_half(acc[j] * inv);
+    }
+}
+
+// ── decode, head_dim 128 ─────────────────────────────────────────────────
+constexpr int kHeadsPerPass = 8;     // query heads of one KV head kept in registers
+constexpr int kPartFloats = kD + 2;  // per (head, slice): max, sum, 128 channels
+
+template <int kOp>   // 0: sum, 1: max over the lanes l, l^16, l^32, l^48
+__device__ __forceinline__ float across_rows(float v) {
+    const float a = __shfl_xor(v, 16);
+    v = kOp ? fmaxf(v, a) : v + a;
+    const float b = __shfl_xor(v, 32);
+    return kOp ? fmaxf(v, b) : v + b;
+}
+
+// Sum over the 16 lanes of a DPP row, left in all of them.
+__device__ __forceinline__ float row_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    return v;
+}
+
+__global__ __launch_bounds__(kBlock) void decode_part(
+    const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
+    const int* __restrict__ page_table, h16* __restrict__ O, float* __restrict__ parts,
+    int n_q_heads, int n_kv_heads, int cache_len, const int* __restrict__ d_cache_len,
+    int n_parts, float scale_log2) {
+    __shared__ float sm[kWavesPerBlock][kHeadsPerPass][kPartFloats];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int chunk = lane & 15;          // this lane's 8 channels
+    const int sub = lane >> 4;            // which of the wave's 4 rows per step
+    const int part = (int)blockIdx.x;
+    const int kvh = (int)blockIdx.y;
+    const int group = n_q_heads / n_kv_heads;
+    const int g0 = (int)blockIdx.z * kHeadsPerPass;
+    const int ng = min(kHeadsPerPass, group - g0);
+    const int len = d_cache_len ? *d_cache_len : cache_len;
+    const int per = (((len + n_parts - 1) / n_parts) + 15) & ~15;
+    const int begin = part * per, end = min(len, begin + per);
+    const size_t kv_stride = (size_t)n_kv_heads * kD;
+
+    f32x8 q[kHeadsPerPass], acc[kHeadsPerPass];
+    float m_run[kHeadsPerPass], l_run[kHeadsPerPass];
+#pragma unroll
+    for (int g = 0; g < kHeadsPerPass; ++g) {
+        const int head = kvh * group + g0 + min(g, ng - 1);
+        q[g] = unpack(load_chunk(reinterpret_cast<const Chunk*>(Q + (size_t)head * kD) + chunk));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { q[g][i] *= scale_log2; acc[g][i] = 0.0f; }
+        m_run[g] = -INFINITY;
+        l_run[g] = 0.0f;
+    }
+
+    for (int t = begin + wave * 4 + sub; t < end; t += 16) {
+        const size_t off = (size_t)cache_row(page_table, t) * kv_stride + kvh * kD;
+        const f32x8 k = unpack(load_chunk(reinterpret_cast<const Chunk*>(Kc + off) + chunk));
+        const f32x8 v = unpack(load_chunk(reinterpret_cast<const Chunk*>(Vc + off) + chunk));
+#pragma unroll
+        for (int g = 0; g < kHeadsPerPass; ++g) {
+            if (g < ng) {
+                float d = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], k[i], d);
+                const float x = row_sum(d);
+                const float m_new = fmaxf(m_run[g], x);
+                const float alpha = exp2_fast(m_run[g] - m_new);
+                const float p = exp2_fast(x - m_new);
+                l_run[g] = l_run[g] * alpha + p;
+                m_run[g] = m_new;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(acc[g][i], alpha, p * v[i]);
+            }
+        }
+    }
+
+    // Fold the wave's four row groups, then the four waves through LDS.
+#pragma unroll
+    for (int g = 0; g < kHeadsPerPass; ++g) {
+        const float m_all = across_rows<1>(m_run[g]);
+        const float w = m_run[g] == -INFINITY ? 0.0f : exp2_fast(m_run[g] - m_all);
+        l_run[g] = across_rows<0>(l_run[g] * w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = across_rows<0>(acc[g][i] * w);
+        m_run[g] = m_all;
+        if (sub == 0) {
+            if (chunk == 0) { sm[wave][g][0] = m_run[g]; sm[wave][g][1] = l_run[g]; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sm[wave][g][2 + 8 * chunk + i] = acc[g][i];
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < ng * kD; idx += kBlock) {
+        const int g = idx / kD, d = idx % kD;
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) m_all = fmaxf(m_all, sm[w][g][0]);
+        float l = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) {
+            const float mw = sm[w][g][0];
+            const float f = mw == -INFINITY ? 0.0f : exp2_fast(mw - m_all);
+            l += sm[w][g][1] * f;
+            o += sm[w][g][2 + d] * f;
+        }
+        const int head = kvh * group + g0 + g;
+        if (n_parts == 1) {
+            O[(size_t)head * kD + d] = to_half(l > 0.0f ? o / l : 0.0f);
+        } else {
+            float* dst = parts + ((size_t)head * n_parts + part) * kPartFloats;
+            if (d == 0) { dst[0] = m_all; dst[1] = l; }
+            dst[2 + d] = o;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kD) void decode_merge(const float* __restrict__ parts,
+                                                   h16* __restrict__ O, int n_parts) {
+    const int head = (int)blockIdx.x, d = (int)threadIdx.x;
+    const float* src = parts + (size_t)head * n_parts * kPartFloats;
+    float m_all = -INFINITY;
+    for (int p = 0; p < n_parts; ++p) m_all = fmaxf(m_all, src[p * kPartFloats]);
+    float l = 0.0f, o = 0.0f;
+    for (int p = 0; p < n_parts; ++p) {
+        const float mp = src[p * kPartFloats];
+        const float f = mp == -INFINITY ? 0.0f : exp2_fast(mp - m_all);
+        l += src[p * kPartFloats + 1] * f;
+        o += src[p * kPartFloats + 2 + d] * f;
+    }
+    O[(size_t)head * kD + d] = to_half(l > 0.0f ? o / l : 0.0f);
+}
+
+// ── FP16 cache store ─────────────────────────────────────────────────────
+__global__ __launch_bounds__(kBlock) void kv_store_fp16(
+    const h16* __restrict__ k, const h16* __restrict__ v, h16* __restrict__ k_store,
+    h16* __restrict__ v_store, int row_halves, int pos, const int* __restrict__ d_pos,
+    int n_positions, const int* __restrict__ page_table) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= (size_t)n_positions * row_halves) return;
+    const int p = (int)(i / row_halves), e = (int)(i % row_halves);
+    const int t = (d_pos ? *d_pos : pos) + p;
+    const size_t dst = (size_t)cache_row(page_table, t) * row_halves + e;
+    k_store[dst] = k[i];
+    v_store[dst] = v[i];
+}
+
+struct PageIds { int id[32]; };
+__global__ void page_map(int* table, int first, int n, PageIds ids) {
+    const int i = (int)threadIdx.x;
+    if (i < n) table[first + i] = ids.id[i];
+}
+
+int decode_parts(int cache_len) {
+    int want = (cache_len + 255) / 256, n = 1;
+    while (n < want && n < kMaxParts) n *= 2;
+    return n;
+}
+
+bool shape_ok(int n_q_heads, int n_kv_heads, int head_dim) {
+    return n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0 && head_dim > 0 &&
+           head_dim <= 256;
+}
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+/* One implementation serves every backend name: what differs between fa1,
+ * fa2 and flashinfer on the reference's CUDA side is how the card is used,
+ * not the result. FP16 caches only, contiguous or paged. */
+int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads, int n_kv_heads,
+                    int head_dim) {
+    enum { kAuto = 0, kFa1 = 1, kFa2 = 2, kFlashinfer = 3 };
+    if (kv_format != vv::kFormatFp16 || !vv::shape_ok(n_q_heads, n_kv_heads, head_dim)) return kFa1;
+    if (requested == kFlashinfer) return kFlashinfer;
+    if (requested == kFa1 && !paged) return kFa1;
+    return kFa2;
+}
+
+size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim) {
+    (void)n_kv_heads;
+    if (n_q_heads <= 0 || head_dim <= 0) return 0;
+    return (size_t)n_q_heads * vv::kMaxParts * ((size_t)head_dim + 2) * sizeof(float);
+}
+
+int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len) {
+    (void)backend; (void)n_q_heads; (void)n_kv_heads;
+    return vv::decode_parts(cache_len);
+}
+
+vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, void* out,
+                            int n_q_heads, int q_len, int q_offset, int kv_len, bool causal,
+                            void* scratch, void* stream) {
+    (void)backend; (void)scratch;
+    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
+    if (q_len <= 0 || kv_len <= 0) return VV_OK;
+    if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
+    if (kv->format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
+    if (q_offset < 0) return VV_ERR_INVALID_ARG;
+    hipStream_t st = vv::as_stream(stream);
+    const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
+    const vv::h16* Q = static_cast<const vv::h16*>(q);
+    const vv::h16* K = static_cast<const vv::h16*>(kv->k);
+    const vv::h16* V = static_cast<const vv::h16*>(kv->v);
+    vv::h16* O = static_cast<vv::h16*>(out);
+    if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
+        vv::aligned16(out)) {
+        const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
+        vv::prefill128<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
+                                                    kv->n_kv_heads, q_len, q_offset, kv_len,
+                                                    causal ? 1 : 0, scale_log2);
+    } else {
+        const dim3 grid((unsigned)q_len, (unsigned)n_q_heads);
+        vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
+                                                     kv->n_kv_heads, kv->head_dim, q_len, q_offset,
+                                                     kv_len, nullptr, causal ? 1 : 0, scale_log2);
+    }
+    return vv::launch_status();
+}
+
+vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, void* out,
+                           int n_q_heads, int cache_len, const int* d_cache_len, void* scratch,
+                           void* stream) {
+    (void)backend;
+    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
+    if (cache_len <= 0) return VV_OK;
+    if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
+    if (kv->format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
+    hipStream_t st = vv::as_stream(stream);
+    const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
+    const vv::h16* Q = static_cast<const vv::h16*>(q);
+    const vv::h16* K = static_cast<const vv::h16*>(kv->k);
+    const vv::h16* V = static_cast<const vv::h16*>(kv->v);
+    vv::h16* O = static_cast<vv::h16*>(out);
+    if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v)) {
+        const int n_parts = vv::decode_parts(cache_len);
+        if (n_parts > 1 && !scratch) return VV_ERR_NULL_PTR;
+        const int group = n_q_heads / kv->n_kv_heads;
+        const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads,
+                        (unsigned)((group + vv::kHeadsPerPass - 1) / vv::kHeadsPerPass));
+        vv::decode_part<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O,
+                                                     static_cast<float*>(scratch), n_q_heads,
+                                                     kv->n_kv_heads, cache_len, d_cache_len,
+                                                     n_parts, scale_log2);
+        if (n_parts > 1) {
+            if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
+            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kD, 0, st>>>(
+                static_cast<const float*>(scratch), O, n_parts);
+        }
+    } else {
+        // One row: position cache_len - 1 sees everything, so no mask is needed.
+        const dim3 grid(1u, (unsigned)n_q_heads);
+        vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
+                                                     kv->n_kv_heads, kv->head_dim, 1, 0, cache_len,
+                                                     d_cache_len, 0, scale_log2);
+    }
+    return vv::launch_status();
+}
+
+vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_store, void* v_store,
+                            void* k_meta, void* v_meta, void* k_ref, bool build_ref,
+                            int n_kv_heads, int head_dim, int pos, const int* d_pos,
+                            int n_positions, int kv_format, const int* page_table, void* stream) {
+    (void)k_meta; (void)v_meta; (void)k_ref; (void)build_ref;
+    if (!k_fp16 || !v_fp16 || !k_store || !v_store) return VV_ERR_NULL_PTR;
+    if (kv_format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    if (n_kv_heads <= 0 || head_dim <= 0 || pos < 0) return VV_ERR_INVALID_ARG;
+    if (n_positions <= 0) return VV_OK;
+    const int row = n_kv_heads * head_dim;
+    const size_t n = (size_t)n_positions * row;
+    vv::kv_store_fp16<<<dim3((unsigned)((n + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
+                        vv::as_stream(stream)>>>(
+        static_cast<const vv::h16*>(k_fp16), static_cast<const vv::h16*>(v_fp16),
+        static_cast<vv::h16*>(k_store), static_cast<vv::h16*>(v_store), row, pos, d_pos,
+        n_positions, page_table);
+    return vv::launch_status();
+}
+
+vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages, void* stream) {
+    if (n <= 0) return VV_OK;
+    if (!page_table || !pages) return VV_ERR_NULL_PTR;
+    if (first < 0) return VV_ERR_INVALID_ARG;
+    // The ids travel as kernel arguments, 32 a launch: the host array is read
+    // before this returns and the writes are ordered on the stream.
+    for (int done = 0; done < n; done += 32) {
+        vv::PageIds ids;
+        const int m = n - done < 32 ? n - done : 32;
+        for (int i = 0; i < 32; ++i) ids.id[i] = i < m ? pages[done + i] : 0;
+        vv::page_map<<<1, 32, 0, vv::as_stream(stream)>>>(page_table, first + done, m, ids);
+        if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
+    }
+    return VV_OK;
+}
+
+}  // extern "C"

@@ -25,6 +25,13 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
 
 _vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 
+class KvView(C.Structure):
+    """vv_kv_view_t: one layer of a KV cache as the attention entry points see it."""
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("k_meta", C.c_void_p),
+                ("v_meta", C.c_void_p), ("page_table", C.c_void_p), ("format", C.c_int),
+                ("n_kv_heads", C.c_int), ("head_dim", C.c_int)]
+
+
 # symbol -> (restype, argtypes); the complete export list of include/vibevoice_hip.h
 SIGNATURES = {
     "vv_embedding_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
@@ -42,6 +49,14 @@ SIGNATURES = {
     "vv_col_absmax_dev": (_i, [_vp, _i, _i, _vp, _vp]),
     "vv_gemm_fp16_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _f, _vp]),
     "vv_gemm_fp16_tile_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _f, _vp]),
+    "vv_attn_resolve": (_i, [_i, _i, C.c_bool, _i, _i, _i]),
+    "vv_attn_scratch_bytes": (C.c_size_t, [_i, _i, _i]),
+    "vv_attn_decode_shape": (_i, [_i, _i, _i, _i]),
+    "vv_attn_prefill": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, C.c_bool, _vp, _vp]),
+    "vv_attn_decode": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "vv_kv_store_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_bool, _i, _i, _i, _vp, _i,
+                            _i, _vp, _vp]),
+    "vv_kv_page_map_dev": (_i, [_vp, _i, _i, _vp, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
