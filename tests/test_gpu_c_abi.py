@@ -38,3 +38,26 @@ def test_reference_own_device_memory_test_passes_on_this_backend():
     print(res.stdout[-3000:], res.stderr[-1000:])
     assert res.returncode == 0, res.stdout[-2000:]
     assert "all device memory checks passed" in res.stdout and "FAIL" not in res.stdout
+
+
+LAYER_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_prefill_append_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(LAYER_EXE),
+                    reason="oracle/_ref/test_prefill_append_hip not built (needs the reference tree)")
+def test_reference_layer_runner_passes_on_this_backend():
+    """The reference's tests/test_prefill_append.c with the reference's own
+    decoder and KV cache (compiled unmodified by oracle/Makefile) driving this
+    backend: a 2-layer dense model, one-shot prefill vs prefill + decode step +
+    prefill on top of the cache, and accelerator vs CPU hidden states. Every op
+    of a dense layer goes through libvibevoice_hip.so: RMSNorm, the GEMMs and
+    bias adds, RoPE, the FP16 KV append, prefill and decode attention, the
+    residual adds and SwiGLU."""
+    res = subprocess.run([LAYER_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-5000:], res.stderr[-1000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "SKIP" not in res.stdout.split("GPU:")[1], "the accelerator half did not run"
+    for line in ("GPU: same hidden states", "GPU and CPU agree", "OK (0 failures)"):
+        assert line in res.stdout
+    assert "FAIL" not in res.stdout
