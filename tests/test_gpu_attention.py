@@ -143,8 +143,8 @@ def test_paged_cache_matches_contiguous(rows, nq, nkv, off):
         assert np.array_equal(outs[0], outs[1])
 
 
-@pytest.mark.parametrize("nq,nkv,hd", [(28, 4, 128), (2, 1, 128), (16, 1, 128), (12, 2, 128), (4, 2, 64)])
-@pytest.mark.parametrize("cache_len", [1, 17, 255, 256, 257, 1000, 5000, 14449])
+@pytest.mark.parametrize("nq,nkv,hd", [(28, 4, 128), (2, 1, 128), (40, 1, 128), (12, 2, 128), (4, 2, 64)])
+@pytest.mark.parametrize("cache_len", [1, 17, 64, 65, 255, 257, 1000, 5000, 14449, 40000])
 def test_decode_against_oracle(nq, nkv, hd, cache_len):
     q, k, v = make(1, nq, nkv, hd, cache_len, cache_len + nq)
     ref = oracle.attention_prefill_f32(oracle.widen(q), oracle.widen(k), oracle.widen(v), cache_len - 1,

@@ -18,11 +18,12 @@
 //                laid out as the B operand of O^T = V^T P^T. V is transposed
 //                on its way into LDS (four keys of one channel per 8-byte
 //                slot) so the A operand of that product is two 8-byte reads.
-//   decode_part  one query row: bound by the cache bytes. A workgroup takes
-//                one KV head and one slice of the positions; 16 lanes share a
-//                key row (16 bytes each), all query heads of the group reuse
-//                it from registers. Slices leave (max, sum, unnormalised O)
-//                in the caller's scratch and decode_merge folds them.
+//   decode128    one query row per head: bound by the cache bytes. The same
+//                pieces with the query heads that share a KV head in the
+//                place of the query rows, so a slice of K and V is read once
+//                for the whole group; one wave per (slice, KV head). Slices
+//                leave (max, sum, unnormalised O) in the caller's scratch
+//                and decode_merge folds them.
 //   rows_generic any head_dim <= 256, any alignment: one wave per (row, head).
 #include "vv_common.hpp"
 
@@ -34,7 +35,7 @@ typedef h16 h16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kPage = 64;            // positions per page (include/vibevoice/kv_quant.h:52)
 constexpr int kFormatFp16 = 0;       // VV_KV_FP16
-constexpr int kMaxParts = 64;        // decode slices per KV head
+constexpr int kMaxParts = 128;       // decode slices per KV head
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -44,18 +45,166 @@ __device__ __forceinline__ int cache_row(const int* page_table, int t) {
     return page_table ? page_table[t / kPage] * kPage + t % kPage : t;
 }
 
-// ── prefill, head_dim 128 ────────────────────────────────────────────────
+// ── head_dim 128 on the matrix cores: the pieces both forms share ─────────
 constexpr int kD = 128;
-constexpr int kQTile = 128;          // query rows per workgroup (32 per wave)
+constexpr int kQTile = 128;          // query rows per prefill workgroup (32 per wave)
 constexpr int kKeyTile = 64;         // keys per LDS tile
 constexpr int kVtStride = kKeyTile + 4;   // halves per transposed-V row: 136 B
 
-__global__ __launch_bounds__(kBlock) void prefill128(
+struct KvTile {
+    Chunk k[kKeyTile * (kD / 8)];                 // [key][16 slots], slot ^ (key & 15)
+    __align__(16) h16 vt[kD * kVtStride];         // [channel][key]
+};
+
+// Per-lane state of one query row (lane % 32) over the keys seen so far: O^T
+// register 4g + r of tile t is channel 32t + 8g + 4*(lane / 32) + r.
+struct RowState {
+    f32x16 o[kD / 32];
+    float m, l;                                   // running max (base-2 domain) and sum
+    __device__ __forceinline__ void reset() {
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
+        m = -INFINITY;
+        l = 0.0f;
+    }
+};
+
+// Keys t0 .. t0+63 of KV head kvh, first into registers (fetch: issued a tile
+// ahead, so the loads fly while the previous tile is computed), then into LDS
+// (commit). Rows past last_key repeat it: they are masked, but must hold finite
+// values. K keeps its layout; V is transposed: a thread takes four consecutive
+// keys of one 8-channel chunk and writes, per channel, the four keys as 8 bytes.
+template <int kThreads>
+struct TileRegs {
+    static constexpr int kIter = kKeyTile * (kD / 8) / kThreads;   // chunks per thread, K and V each
+    Chunk k[kIter], v[kIter];
+};
+
+template <int kThreads>
+__device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const h16* __restrict__ Kc,
+                                           const h16* __restrict__ Vc,
+                                           const int* __restrict__ page_table, size_t kv_stride,
+                                           int kvh, int t0, int last_key, int tid) {
+    constexpr int kIter = TileRegs<kThreads>::kIter;
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+        const int q = tid + i * kThreads, r = q >> 4, slot = q & 15;
+        const int row = cache_row(page_table, min(t0 + r, last_key));
+        regs.k[i] = load_chunk(reinterpret_cast<const Chunk*>(Kc + (size_t)row * kv_stride + kvh * kD) + slot);
+    }
+#pragma unroll
+    for (int i = 0; i < kIter / 4; ++i) {
+        const int q = tid + i * kThreads, dchunk = q & 15, kg = q >> 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = cache_row(page_table, min(t0 + 4 * kg + j, last_key));
+            regs.v[4 * i + j] =
+                load_chunk(reinterpret_cast<const Chunk*>(Vc + (size_t)row * kv_stride + kvh * kD) + dchunk);
+        }
+    }
+}
+
+template <int kThreads>
+__device__ __forceinline__ void commit_tile(KvTile& tile, const TileRegs<kThreads>& regs, int tid) {
+    constexpr int kIter = TileRegs<kThreads>::kIter;
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+        const int q = tid + i * kThreads, r = q >> 4, slot = q & 15;
+        tile.k[r * 16 + (slot ^ (r & 15))] = regs.k[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kIter / 4; ++i) {
+        const int q = tid + i * kThreads, dchunk = q & 15, kg = q >> 4;
+        h16x8 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = __builtin_bit_cast(h16x8, regs.v[4 * i + j]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const h16x4 w = {v[0][e], v[1][e], v[2][e], v[3][e]};
+            *reinterpret_cast<h16x4*>(&tile.vt[(8 * dchunk + e) * kVtStride + 4 * kg]) = w;
+        }
+    }
+}
+
+// S^T = K Q^T for the tile: register 4g + r of s[a] is key 32a + 8g + 4*half + r
+// of the tile, for this lane's query row.
+__device__ __forceinline__ void tile_scores(const KvTile& tile, const h16x8 (&qf)[kD / 16],
+                                            int col, int half, f32x16 (&s)[2]) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[a][r] = 0.0f;
+#pragma unroll
+        for (int st = 0; st < kD / 16; ++st) {
+            const int row = 32 * a + col, slot = 2 * st + half;
+            const h16x8 kf = __builtin_bit_cast(h16x8, tile.k[row * 16 + (slot ^ (row & 15))]);
+            s[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[st], s[a], 0, 0, 0);
+        }
+    }
+}
+
+// s holds the masked, scaled scores (-inf where unseen). Online-softmax update
+// of the row state, then O^T += V^T P^T over the tile's four 16-key steps. Slot
+// e of this lane in step (a, sp) is register 8*sp + e of s[a], i.e. key
+// 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte reads of V^T below.
+__device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], RowState& st,
+                                            int col, int half) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
+    mx = fmaxf(mx, other_half(mx));
+    const float m_new = fmaxf(st.m, mx);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+    const float alpha = exp2_fast(st.m - m_use);
+    float sum = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float p = exp2_fast(s[a][r] - m_use);
+            s[a][r] = p;
+            sum += p;
+        }
+    sum += other_half(sum);
+    st.l = st.l * alpha + sum;
+    st.m = m_new;
+#pragma unroll
+    for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int a = u >> 1, sp = u & 1;
+        h16x8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[e] = (h16)s[a][8 * sp + e];
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t) {
+            const h16* base = &tile.vt[(32 * t + col) * kVtStride + 32 * a + 16 * sp + 4 * half];
+            const h16x4 lo = *reinterpret_cast<const h16x4*>(base);
+            const h16x4 hi = *reinterpret_cast<const h16x4*>(base + 8);
+            const h16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, st.o[t], 0, 0, 0);
+        }
+    }
+}
+
+__device__ __forceinline__ void load_query(h16x8 (&qf)[kD / 16], const h16* qp, int half) {
+#pragma unroll
+    for (int s = 0; s < kD / 16; ++s)
+        qf[s] = __builtin_bit_cast(h16x8, load_chunk(reinterpret_cast<const Chunk*>(qp) + 2 * s + half));
+}
+
+// ── prefill ──────────────────────────────────────────────────────────────
+__global__ __launch_bounds__(kBlock, 2) void prefill128(
     const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
     const int* __restrict__ page_table, h16* __restrict__ O, int n_q_heads, int n_kv_heads,
     int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
-    __shared__ Chunk sK[kKeyTile * (kD / 8)];          // [key][16 slots], slot ^ (key & 15)
-    __shared__ __align__(16) h16 sVt[kD * kVtStride];  // [channel][key]
+    __shared__ KvTile tile;
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -64,7 +213,8 @@ __global__ __launch_bounds__(kBlock) void prefill128(
     const int half = lane >> 5;
     const int head = (int)blockIdx.y;
     const int kvh = head / (n_q_heads / n_kv_heads);
-    const int q0 = (int)blockIdx.x * kQTile;
+    // Causal rows late in the prompt see the most keys: launch those first.
+    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kQTile;
     const int qw0 = q0 + wave * 32;
     const int qrow = qw0 + col;
     const int q_abs = q_offset + qrow;
@@ -78,118 +228,34 @@ __global__ __launch_bounds__(kBlock) void prefill128(
     }
 
     h16x8 qf[kD / 16];
-    {
-        const h16* qp = Q + ((size_t)min(qrow, q_len - 1) * n_q_heads + head) * kD;
-#pragma unroll
-        for (int s = 0; s < kD / 16; ++s)
-            qf[s] = __builtin_bit_cast(h16x8,
-                                       load_chunk(reinterpret_cast<const Chunk*>(qp) + 2 * s + half));
-    }
+    load_query(qf, Q + ((size_t)min(qrow, q_len - 1) * n_q_heads + head) * kD, half);
+    RowState st;
+    st.reset();
 
-    f32x16 oacc[kD / 32];
-#pragma unroll
-    for (int t = 0; t < kD / 32; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
-
+    TileRegs<kBlock> regs;
+    if (wg_limit > 0) fetch_tile<kBlock>(regs, Kc, Vc, page_table, kv_stride, kvh, 0, kv_len - 1, tid);
     for (int t0 = 0; t0 < wg_limit; t0 += kKeyTile) {
         __syncthreads();
-        // K tile: four 16-byte slots per thread.
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int q = tid + i * kBlock, r = q >> 4, slot = q & 15;
-            const int row = cache_row(page_table, min(t0 + r, kv_len - 1));
-            sK[r * 16 + (slot ^ (r & 15))] =
-                load_chunk(reinterpret_cast<const Chunk*>(Kc + (size_t)row * kv_stride + kvh * kD) + slot);
-        }
-        // V tile, transposed: a thread takes four consecutive keys of one
-        // 8-channel chunk and writes, per channel, the four keys as 8 bytes.
-        {
-            const int dchunk = tid & 15, kg = tid >> 4;
-            h16x8 v[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int row = cache_row(page_table, min(t0 + 4 * kg + j, kv_len - 1));
-                v[j] = __builtin_bit_cast(
-                    h16x8, load_chunk(reinterpret_cast<const Chunk*>(Vc + (size_t)row * kv_stride + kvh * kD) + dchunk));
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const h16x4 w = {v[0][i], v[1][i], v[2][i], v[3][i]};
-                *reinterpret_cast<h16x4*>(&sVt[(8 * dchunk + i) * kVtStride + 4 * kg]) = w;
-            }
-        }
+        commit_tile<kBlock>(tile, regs, tid);
         __syncthreads();
+        if (t0 + kKeyTile < wg_limit)
+            fetch_tile<kBlock>(regs, Kc, Vc, page_table, kv_stride, kvh, t0 + kKeyTile, kv_len - 1, tid);
         if (t0 >= wave_limit) continue;
-
-        // S^T = K Q^T: register 4g + r of tile a is key t0 + 32a + 8g + 4*half + r.
         f32x16 s[2];
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[a][r] = 0.0f;
-#pragma unroll
-            for (int st = 0; st < kD / 16; ++st) {
-                const int row = 32 * a + col, slot = 2 * st + half;
-                const h16x8 kf = __builtin_bit_cast(h16x8, sK[row * 16 + (slot ^ (row & 15))]);
-                s[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[st], s[a], 0, 0, 0);
-            }
-        }
-        float mx = -INFINITY;
+        tile_scores(tile, qf, col, half, s);
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
                 const bool seen = key < kv_len && (!causal || key <= q_abs);
-                const float x = seen ? s[a][r] * scale_log2 : -INFINITY;
-                s[a][r] = x;
-                mx = fmaxf(mx, x);
+                s[a][r] = seen ? s[a][r] * scale_log2 : -INFINITY;
             }
-        mx = fmaxf(mx, other_half(mx));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2_fast(m_run - m_use);
-        float sum = 0.0f;
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float p = exp2_fast(s[a][r] - m_use);
-                s[a][r] = p;
-                sum += p;
-            }
-        sum += other_half(sum);
-        l_run = l_run * alpha + sum;
-        m_run = m_new;
-#pragma unroll
-        for (int t = 0; t < kD / 32; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
-
-        // O^T += V^T P^T over the tile's four 16-key steps. Slot e of this
-        // lane in step (a, sp) is register 8*sp + e of tile a, i.e. key
-        // 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte reads below.
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int a = u >> 1, sp = u & 1;
-            h16x8 pf;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) pf[e] = (h16)s[a][8 * sp + e];
-#pragma unroll
-            for (int t = 0; t < kD / 32; ++t) {
-                const h16* base = &sVt[(32 * t + col) * kVtStride + 32 * a + 16 * sp + 4 * half];
-                const h16x4 lo = *reinterpret_cast<const h16x4*>(base);
-                const h16x4 hi = *reinterpret_cast<const h16x4*>(base + 8);
-                const h16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[t], 0, 0, 0);
-            }
-        }
+        tile_update(tile, s, st, col, half);
     }
 
     if (qrow < q_len) {
-        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
         h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
@@ -197,7 +263,7 @@ __global__ __launch_bounds__(kBlock) void prefill128(
             for (int g = 0; g < 4; ++g) {
                 h16x4 o;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = to_half(oacc[t][4 * g + r] * inv);
+                for (int r = 0; r < 4; ++r) o[r] = to_half(st.o[t][4 * g + r] * inv);
                 *reinterpret_cast<h16x4*>(op + 32 * t + 8 * g + 4 * half) = o;
             }
     }
@@ -251,136 +317,122 @@ __global__ __launch_bounds__(kWave) void rows_generic(
 }
 
 // ── decode, head_dim 128 ─────────────────────────────────────────────────
-constexpr int kHeadsPerPass = 8;     // query heads of one KV head kept in registers
-constexpr int kPartFloats = kD + 2;  // per (head, slice): max, sum, 128 channels
+// One wave per (slice of the positions, KV head, 32 query heads of its group):
+// the heads sharing a KV head take the place of the prefill's query rows, so
+// the slice's K and V are read once for all of them. n_parts == 1 writes O;
+// otherwise each slice leaves (max, sum, unnormalised O) per head in `parts`.
+constexpr int kPartFloats = kD + 2;
 
-template <int kOp>   // 0: sum, 1: max over the lanes l, l^16, l^32, l^48
-__device__ __forceinline__ float across_rows(float v) {
-    const float a = __shfl_xor(v, 16);
-    v = kOp ? fmaxf(v, a) : v + a;
-    const float b = __shfl_xor(v, 32);
-    return kOp ? fmaxf(v, b) : v + b;
-}
-
-// Sum over the 16 lanes of a DPP row, left in all of them.
-__device__ __forceinline__ float row_sum(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    v += dpp_move<0x140>(v);
-    return v;
-}
-
-__global__ __launch_bounds__(kBlock) void decode_part(
+__global__ __launch_bounds__(kWave) void decode128(
     const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
     const int* __restrict__ page_table, h16* __restrict__ O, float* __restrict__ parts,
     int n_q_heads, int n_kv_heads, int cache_len, const int* __restrict__ d_cache_len,
     int n_parts, float scale_log2) {
-    __shared__ float sm[kWavesPerBlock][kHeadsPerPass][kPartFloats];
+    __shared__ KvTile tile;
 
-    const int tid = (int)threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int chunk = lane & 15;          // this lane's 8 channels
-    const int sub = lane >> 4;            // which of the wave's 4 rows per step
+    const int lane = (int)threadIdx.x;
+    const int col = lane & 31, half = lane >> 5;
     const int part = (int)blockIdx.x;
     const int kvh = (int)blockIdx.y;
     const int group = n_q_heads / n_kv_heads;
-    const int g0 = (int)blockIdx.z * kHeadsPerPass;
-    const int ng = min(kHeadsPerPass, group - g0);
+    const int g = (int)blockIdx.z * 32 + col;                 // this lane's head inside the group
+    const int head = kvh * group + min(g, group - 1);
     const int len = d_cache_len ? *d_cache_len : cache_len;
-    const int per = (((len + n_parts - 1) / n_parts) + 15) & ~15;
+    const int per = (((len + n_parts - 1) / n_parts) + kKeyTile - 1) & ~(kKeyTile - 1);
     const int begin = part * per, end = min(len, begin + per);
     const size_t kv_stride = (size_t)n_kv_heads * kD;
 
-    f32x8 q[kHeadsPerPass], acc[kHeadsPerPass];
-    float m_run[kHeadsPerPass], l_run[kHeadsPerPass];
-#pragma unroll
-    for (int g = 0; g < kHeadsPerPass; ++g) {
-        const int head = kvh * group + g0 + min(g, ng - 1);
-        q[g] = unpack(load_chunk(reinterpret_cast<const Chunk*>(Q + (size_t)head * kD) + chunk));
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { q[g][i] *= scale_log2; acc[g][i] = 0.0f; }
-        m_run[g] = -INFINITY;
-        l_run[g] = 0.0f;
-    }
+    h16x8 qf[kD / 16];
+    load_query(qf, Q + (size_t)head * kD, half);
+    RowState st;
+    st.reset();
 
-    for (int t = begin + wave * 4 + sub; t < end; t += 16) {
-        const size_t off = (size_t)cache_row(page_table, t) * kv_stride + kvh * kD;
-        const f32x8 k = unpack(load_chunk(reinterpret_cast<const Chunk*>(Kc + off) + chunk));
-        const f32x8 v = unpack(load_chunk(reinterpret_cast<const Chunk*>(Vc + off) + chunk));
+    TileRegs<kWave> regs;
+    if (begin < end) fetch_tile<kWave>(regs, Kc, Vc, page_table, kv_stride, kvh, begin, end - 1, lane);
+    for (int t0 = begin; t0 < end; t0 += kKeyTile) {
+        __syncthreads();
+        commit_tile<kWave>(tile, regs, lane);
+        __syncthreads();
+        if (t0 + kKeyTile < end)
+            fetch_tile<kWave>(regs, Kc, Vc, page_table, kv_stride, kvh, t0 + kKeyTile, end - 1, lane);
+        f32x16 s[2];
+        tile_scores(tile, qf, col, half, s);
 #pragma unroll
-        for (int g = 0; g < kHeadsPerPass; ++g) {
-            if (g < ng) {
-                float d = 0.0f;
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], k[i], d);
-                const float x = row_sum(d);
-                const float m_new = fmaxf(m_run[g], x);
-                const float alpha = exp2_fast(m_run[g] - m_new);
-                const float p = exp2_fast(x - m_new);
-                l_run[g] = l_run[g] * alpha + p;
-                m_run[g] = m_new;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(acc[g][i], alpha, p * v[i]);
+            for (int r = 0; r < 16; ++r) {
+                const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
+                s[a][r] = key < end ? s[a][r] * scale_log2 : -INFINITY;
             }
-        }
+        tile_update(tile, s, st, col, half);
     }
 
-    // Fold the wave's four row groups, then the four waves through LDS.
+    if (g >= group) return;
+    if (n_parts == 1) {
+        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+        h16* op = O + (size_t)head * kD;
 #pragma unroll
-    for (int g = 0; g < kHeadsPerPass; ++g) {
-        const float m_all = across_rows<1>(m_run[g]);
-        const float w = m_run[g] == -INFINITY ? 0.0f : exp2_fast(m_run[g] - m_all);
-        l_run[g] = across_rows<0>(l_run[g] * w);
+        for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = across_rows<0>(acc[g][i] * w);
-        m_run[g] = m_all;
-        if (sub == 0) {
-            if (chunk == 0) { sm[wave][g][0] = m_run[g]; sm[wave][g][1] = l_run[g]; }
+            for (int q = 0; q < 4; ++q) {
+                h16x4 o;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sm[wave][g][2 + 8 * chunk + i] = acc[g][i];
-        }
-    }
-    __syncthreads();
-    for (int idx = tid; idx < ng * kD; idx += kBlock) {
-        const int g = idx / kD, d = idx % kD;
-        float m_all = -INFINITY;
+                for (int r = 0; r < 4; ++r) o[r] = to_half(st.o[t][4 * q + r] * inv);
+                *reinterpret_cast<h16x4*>(op + 32 * t + 8 * q + 4 * half) = o;
+            }
+    } else {
+        float* dst = parts + ((size_t)head * n_parts + part) * kPartFloats;
+        if (half == 0) { dst[0] = st.m; dst[1] = st.l; }
 #pragma unroll
-        for (int w = 0; w < kWavesPerBlock; ++w) m_all = fmaxf(m_all, sm[w][g][0]);
-        float l = 0.0f, o = 0.0f;
+        for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
-        for (int w = 0; w < kWavesPerBlock; ++w) {
-            const float mw = sm[w][g][0];
-            const float f = mw == -INFINITY ? 0.0f : exp2_fast(mw - m_all);
-            l += sm[w][g][1] * f;
-            o += sm[w][g][2 + d] * f;
-        }
-        const int head = kvh * group + g0 + g;
-        if (n_parts == 1) {
-            O[(size_t)head * kD + d] = to_half(l > 0.0f ? o / l : 0.0f);
-        } else {
-            float* dst = parts + ((size_t)head * n_parts + part) * kPartFloats;
-            if (d == 0) { dst[0] = m_all; dst[1] = l; }
-            dst[2 + d] = o;
-        }
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    dst[2 + 32 * t + 8 * q + 4 * half + r] = st.o[t][4 * q + r];
     }
 }
 
-__global__ __launch_bounds__(kD) void decode_merge(const float* __restrict__ parts,
-                                                   h16* __restrict__ O, int n_parts) {
-    const int head = (int)blockIdx.x, d = (int)threadIdx.x;
+// Folds the slices of one head: 8 groups of 128 threads take every 8th slice
+// for one channel each, so a thread's loads are few and independent.
+constexpr int kMergeGroups = 8;
+
+__global__ __launch_bounds__(kD * kMergeGroups) void decode_merge(const float* __restrict__ parts,
+                                                                  h16* __restrict__ O,
+                                                                  int n_parts) {
+    __shared__ float s_max[kD * kMergeGroups / kWave];
+    __shared__ float s_o[kMergeGroups][kD];
+    __shared__ float s_l[kMergeGroups];
+    const int head = (int)blockIdx.x, tid = (int)threadIdx.x;
+    const int d = tid % kD, grp = tid / kD;
     const float* src = parts + (size_t)head * n_parts * kPartFloats;
+
+    float m = -INFINITY;
+    for (int p = tid; p < n_parts; p += kD * kMergeGroups) m = fmaxf(m, src[p * kPartFloats]);
+    m = wave_max(m);
+    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    __syncthreads();
     float m_all = -INFINITY;
-    for (int p = 0; p < n_parts; ++p) m_all = fmaxf(m_all, src[p * kPartFloats]);
+#pragma unroll
+    for (int w = 0; w < kD * kMergeGroups / kWave; ++w) m_all = fmaxf(m_all, s_max[w]);
+
     float l = 0.0f, o = 0.0f;
-    for (int p = 0; p < n_parts; ++p) {
+#pragma unroll 4
+    for (int p = grp; p < n_parts; p += kMergeGroups) {
         const float mp = src[p * kPartFloats];
         const float f = mp == -INFINITY ? 0.0f : exp2_fast(mp - m_all);
         l += src[p * kPartFloats + 1] * f;
         o += src[p * kPartFloats + 2 + d] * f;
     }
-    O[(size_t)head * kD + d] = to_half(l > 0.0f ? o / l : 0.0f);
+    s_o[grp][d] = o;
+    if (d == 0) s_l[grp] = l;
+    __syncthreads();
+    if (grp == 0) {
+        float lt = 0.0f, ot = 0.0f;
+#pragma unroll
+        for (int g = 0; g < kMergeGroups; ++g) { lt += s_l[g]; ot += s_o[g][d]; }
+        O[(size_t)head * kD + d] = to_half(lt > 0.0f ? ot / lt : 0.0f);
+    }
 }
 
 // ── FP16 cache store ─────────────────────────────────────────────────────
@@ -404,7 +456,7 @@ __global__ void page_map(int* table, int first, int n, PageIds ids) {
 }
 
 int decode_parts(int cache_len) {
-    int want = (cache_len + 255) / 256, n = 1;
+    int want = (cache_len + kKeyTile - 1) / kKeyTile, n = 1;
     while (n < want && n < kMaxParts) n *= 2;
     return n;
 }
@@ -492,15 +544,14 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
         const int n_parts = vv::decode_parts(cache_len);
         if (n_parts > 1 && !scratch) return VV_ERR_NULL_PTR;
         const int group = n_q_heads / kv->n_kv_heads;
-        const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads,
-                        (unsigned)((group + vv::kHeadsPerPass - 1) / vv::kHeadsPerPass));
-        vv::decode_part<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O,
+        const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads, (unsigned)((group + 31) / 32));
+        vv::decode128<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O,
                                                      static_cast<float*>(scratch), n_q_heads,
                                                      kv->n_kv_heads, cache_len, d_cache_len,
                                                      n_parts, scale_log2);
         if (n_parts > 1) {
             if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
-            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kD, 0, st>>>(
+            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kD * vv::kMergeGroups, 0, st>>>(
                 static_cast<const float*>(scratch), O, n_parts);
         }
     } else {
