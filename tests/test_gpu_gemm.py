@@ -45,7 +45,8 @@ def run(fn, d_a, d_b, d_c, M, N, K, alpha=1.0, beta=0.0):
 
 SHAPES = [(1, 64, 64), (1, 3584, 3584), (3, 512, 3584), (8, 1000, 1536), (9, 64, 64),
           (29, 3584, 3584), (29, 512, 3584), (33, 4608, 1536), (64, 256, 512), (100, 128, 72),
-          (285, 3584, 3584), (130, 101, 200), (257, 37, 8), (48, 512, 256), (70, 3584, 18944)]
+          (285, 3584, 3584), (130, 101, 200), (257, 37, 8), (48, 512, 256), (70, 3584, 18944),
+          (4100, 8200, 72), (4097, 8192, 64)]     # enough 256x256 workgroups for the eight-wave tile
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

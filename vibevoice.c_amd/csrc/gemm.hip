@@ -6,7 +6,7 @@
 // of one row of each operand. Three kernels:
 //
 //   gemm_tile<BM,BN,WM,WN>  workgroup tile BM x BN over WM x WN waves, K in
-//                           slabs of 64 staged through LDS (double-buffered,
+//                           slabs of 64 or 32 staged through LDS (double-buffered,
 //                           16-byte slots XOR-swizzled so that the 32 rows a
 //                           ds_read_b128 touches fall in distinct banks). The
 //                           weight rows are the MFMA's A operand and the
@@ -26,25 +26,33 @@ namespace vv {
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // one 16-byte slot
 
-constexpr int kSlab = 64;                 // K values per LDS slab
-constexpr int kSlabChunks = kSlab / 8;    // 16-byte slots per slab row
-
-// Slot swizzle: rows are 128 B = 32 banks apart, so two rows share a 64-bank
-// line; XOR-ing the slot with (row / 2) % 8 spreads any 16 consecutive rows
-// reading the same logical slot over all 64 banks.
-__device__ __forceinline__ int swz(int row, int slot) { return slot ^ ((row >> 1) & 7); }
+// Slot swizzle for a slab of kSlab K values (kSlab / 8 16-byte slots per row).
+// 64: rows are 128 B = 32 banks apart, two rows share a 64-bank line, and
+// XOR-ing the slot with (row / 2) % 8 spreads any 16 consecutive rows reading
+// the same logical slot over all 64 banks. 32: four rows share a line and the
+// slot is XOR-ed with (row / 4) % 4, to the same effect.
+template <int kSlab>
+__device__ __forceinline__ int swz(int row, int slot) {
+    static_assert(kSlab == 64 || kSlab == 32, "slab widths with a swizzle");
+    return kSlab == 64 ? slot ^ ((row >> 1) & 7) : slot ^ ((row >> 2) & 3);
+}
 
 __device__ __forceinline__ float finish(float acc, float alpha, float beta, h16 old) {
     return alpha * acc + beta * (float)old;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int kValue>
+struct Const { static constexpr int value = kValue; };
+
+template <int BM, int BN, int WM, int WN, int kSlab, bool kFull, int kAhead>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
     const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
     int K, float alpha, float beta, int vec_store) {
     constexpr int NT = WM * WN * kWave;
+    constexpr int kSlabChunks = kSlab / 8;    // 16-byte slots per slab row
+    constexpr int kSteps = kSlab / 16;        // MFMA K steps per slab
     constexpr int TM = BM / WM / 32;          // 32x32 MFMA tiles per wave along M
     constexpr int TN = BN / WN / 32;          // and along N
     constexpr int LA = BM * kSlabChunks / NT; // 16-byte loads per thread per slab, A
@@ -53,8 +61,8 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
     static_assert(LA >= 1 && LB >= 1 && (BM * kSlabChunks) % NT == 0 && (BN * kSlabChunks) % NT == 0,
                   "slab loads must divide evenly over the threads");
 
-    __shared__ Chunk sA[2][BM * kSlabChunks];
-    __shared__ Chunk sB[2][BN * kSlabChunks];
+    constexpr int kASlots = BM * kSlabChunks, kBSlots = BN * kSlabChunks;   // per buffer
+    __shared__ u32x4 lds[2 * (kASlots + kBSlots)];       // [buffer][A rows | B rows][slot]
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -65,40 +73,55 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
     const int kchunks = K / 8;
     const int nslabs = (K + kSlab - 1) / kSlab;
 
-    Chunk ra[LA], rb[LB];
-    const Chunk zero = {{0u, 0u, 0u, 0u}};
+    // Global side: a wave-uniform base per operand (it advances by one slab
+    // per iteration in scalar registers) plus a 32-bit byte offset per load, so
+    // the loop spends no vector instructions on addresses. Thread t's i-th
+    // load is row (t + i*NT) / slots, slot (t + i*NT) % slots of the tile.
+    // Rows past the matrix edge repeat the last row (their results are never
+    // stored).
+    const char* a_base = reinterpret_cast<const char*>(A + (size_t)m_blk * K);
+    const char* b_base = reinterpret_cast<const char*>(B + (size_t)n_blk * K);
+    uint32_t a_off[LA], b_off[LB];
+    const int my_slot = tid % kSlabChunks;               // NT is a multiple of the slots per row
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = min((tid + i * NT) / kSlabChunks, M - 1 - m_blk);
+        a_off[i] = ((uint32_t)row * (uint32_t)K + (uint32_t)my_slot * 8u) * 2u;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = min((tid + i * NT) / kSlabChunks, N - 1 - n_blk);
+        b_off[i] = ((uint32_t)row * (uint32_t)K + (uint32_t)my_slot * 8u) * 2u;
+    }
+    // LDS side: the i-th store of a thread lands NT slots after its first (the
+    // swizzle term depends on row bits 1..3 only and NT / slots is a multiple
+    // of 16 rows).
+    const int w_row = tid / kSlabChunks;
+    const int w_slot = w_row * kSlabChunks + swz<kSlab>(w_row, my_slot);
 
-    auto fetch = [&](int slab) {
+    // Two register sets carry the slabs on their way from global memory to
+    // LDS when kAhead == 2, so a slab is requested two compute phases before
+    // it is needed. kFull (K a multiple of the slab): no predicate on the loads.
+    u32x4 ra[kAhead][LA], rb[kAhead][LB];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    auto fetch = [&](auto set_c, int slab) {
+        constexpr int set = decltype(set_c)::value;
+        const size_t adv = (size_t)slab * (kSlab * 2);
+        const bool live = kFull || slab * kSlabChunks + my_slot < kchunks;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
-            const int gm = min(m_blk + row, M - 1);
-            const int kc = slab * kSlabChunks + slot;
-            ra[i] = kc < kchunks
-                        ? load_chunk(reinterpret_cast<const Chunk*>(A + (size_t)gm * K) + kc)
-                        : zero;
-        }
+        for (int i = 0; i < LA; ++i)
+            ra[set][i] = live ? *reinterpret_cast<const u32x4*>(a_base + adv + a_off[i]) : zero;
 #pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
-            const int gn = min(n_blk + row, N - 1);
-            const int kc = slab * kSlabChunks + slot;
-            rb[i] = kc < kchunks
-                        ? load_chunk(reinterpret_cast<const Chunk*>(B + (size_t)gn * K) + kc)
-                        : zero;
-        }
+        for (int i = 0; i < LB; ++i)
+            rb[set][i] = live ? *reinterpret_cast<const u32x4*>(b_base + adv + b_off[i]) : zero;
     };
-    auto stage = [&](int buf) {
+    auto stage = [&](auto set_c, int buf) {
+        constexpr int set = decltype(set_c)::value;
+        u32x4* dst = lds + buf * (kASlots + kBSlots) + w_slot;
 #pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
-            sA[buf][row * kSlabChunks + swz(row, slot)] = ra[i];
-        }
+        for (int i = 0; i < LA; ++i) dst[i * NT] = ra[set][i];
 #pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            const int q = tid + i * NT, row = q / kSlabChunks, slot = q % kSlabChunks;
-            sB[buf][row * kSlabChunks + swz(row, slot)] = rb[i];
-        }
+        for (int i = 0; i < LB; ++i) dst[kASlots + i * NT] = rb[set][i];
     };
 
     f32x16 acc[TN][TM];
@@ -109,39 +132,78 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
-    fetch(0);
-    stage(0);
-    __syncthreads();
-
     const int frow = lane & 31;       // operand row inside a 32x32 tile
     const int fhalf = lane >> 5;      // which 8 of the step's 16 K values
+    // Fragment reads: one index per K step (the swizzled slot of this lane's
+    // row), the tiles of a wave a constant 32 rows apart.
+    int f_idx[kSteps];
+#pragma unroll
+    for (int step = 0; step < kSteps; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<kSlab>(frow, step * 2 + fhalf);
+    const int fa_base = wm * TM * 32 * kSlabChunks;
+    const int fb_base = kASlots + wn * TN * 32 * kSlabChunks;
 
-    for (int slab = 0; slab < nslabs; ++slab) {
-        const int buf = slab & 1;
-        if (slab + 1 < nslabs) fetch(slab + 1);
+    // One slab: the operand fragments of step s + 1 are read from LDS before
+    // the MFMAs of step s are issued.
+    auto compute = [&](int buf) {
+        const u32x4* src = lds + buf * (kASlots + kBSlots);
+        h16x8 fw[2][TN], fx[2][TM];
+        auto read_frags = [&](auto set_c, int step) {
+            constexpr int set = decltype(set_c)::value;
 #pragma unroll
-        for (int step = 0; step < kSlab / 16; ++step) {
-            const int slot = step * 2 + fhalf;
-            h16x8 fw[TN], fx[TM];
+            for (int a = 0; a < TN; ++a)
+                fw[set][a] = __builtin_bit_cast(h16x8, src[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
 #pragma unroll
-            for (int a = 0; a < TN; ++a) {
-                const int row = (wn * TN + a) * 32 + frow;
-                fw[a] = __builtin_bit_cast(h16x8, sB[buf][row * kSlabChunks + swz(row, slot)]);
+            for (int b = 0; b < TM; ++b)
+                fx[set][b] = __builtin_bit_cast(h16x8, src[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
+        };
+        read_frags(Const<0>{}, 0);
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+            if (step + 1 < kSteps) {
+                if (step & 1) read_frags(Const<0>{}, step + 1);
+                else read_frags(Const<1>{}, step + 1);
             }
-#pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                const int row = (wm * TM + b) * 32 + frow;
-                fx[b] = __builtin_bit_cast(h16x8, sA[buf][row * kSlabChunks + swz(row, slot)]);
-            }
+            // Keep the instruction scheduler from sinking those reads below the
+            // MFMAs that do not need them (it would, to shorten register lifetimes).
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int a = 0; a < TN; ++a)
 #pragma unroll
                 for (int b = 0; b < TM; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[a], fx[b], acc[a][b],
-                                                                       0, 0, 0);
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        fw[step & 1][a], fx[step & 1][b], acc[a][b], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (slab + 1 < nslabs) stage(buf ^ 1);
+    };
+
+    fetch(Const<0>{}, 0);
+    if constexpr (kAhead == 2) {
+        if (nslabs > 1) fetch(Const<1>{}, 1);
+        stage(Const<0>{}, 0);
         __syncthreads();
+        int slab = 0;
+        for (; slab + 2 <= nslabs; slab += 2) {
+            if (slab + 2 < nslabs) fetch(Const<0>{}, slab + 2);
+            compute(0);
+            stage(Const<1>{}, 1);
+            __syncthreads();
+            if (slab + 3 < nslabs) fetch(Const<1>{}, slab + 3);
+            compute(1);
+            if (slab + 2 < nslabs) stage(Const<0>{}, 0);
+            __syncthreads();
+        }
+        if (slab < nslabs) compute(0);
+    } else {
+        stage(Const<0>{}, 0);
+        __syncthreads();
+        for (int slab = 0; slab < nslabs; ++slab) {
+            const int buf = slab & 1;
+            if (slab + 1 < nslabs) fetch(Const<0>{}, slab + 1);
+            compute(buf);
+            if (slab + 1 < nslabs) stage(Const<0>{}, buf ^ 1);
+            __syncthreads();
+        }
     }
 
     // Result register 4g + r of lane l holds column n0 + 8g + 4(l / 32) + r of
@@ -232,17 +294,22 @@ __global__ __launch_bounds__(kBlock) void gemm_naive(const h16* A, const h16* B,
     C[i] = to_half(finish(acc, alpha, beta, old));
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int kSlab, int kAhead = 1>
 void launch_tile(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                  float beta, hipStream_t st) {
     const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
     const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-    gemm_tile<BM, BN, WM, WN><<<grid, WM * WN * kWave, 0, st>>>(
-        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K,
-        alpha, beta, vec);
+    if (K % kSlab == 0)
+        gemm_tile<BM, BN, WM, WN, kSlab, true, kAhead><<<grid, WM * WN * kWave, 0, st>>>(
+            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K,
+            alpha, beta, vec);
+    else
+        gemm_tile<BM, BN, WM, WN, kSlab, false, kAhead><<<grid, WM * WN * kWave, 0, st>>>(
+            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K,
+            alpha, beta, vec);
 }
 
-enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3 };
+enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4 };
 
 vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                  float beta, void* stream, int choice, bool allow_gemv) {
@@ -267,16 +334,18 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         return launch_status();
     }
     if (choice == kAuto) {
-        // The largest tile that still gives every compute unit a workgroup.
+        // The largest tile that still fills the 256 compute units: 256x256
+        // (eight waves, the fewest L1 and LDS bytes per MFMA) from two full
+        // rounds of workgroups on, 128x128 from one round on.
+        const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-        const long wg64 = (long)((M + 63) / 64) * ((N + 63) / 64);
-        choice = (M > 64 && wg128 >= 256) ? k128 : (M > 32 && wg64 >= 128) ? k64
-                 : (M > 32) ? k64 : k32;
+        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128 : (M > 32) ? k64 : k32;
     }
     switch (choice) {
-        case k128: launch_tile<128, 128, 2, 2>(A, B, C, M, N, K, alpha, beta, st); break;
-        case k64:  launch_tile<64, 64, 2, 2>(A, B, C, M, N, K, alpha, beta, st); break;
-        default:   launch_tile<32, 64, 1, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k256: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k64:  launch_tile<64, 64, 2, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
+        default:   launch_tile<32, 64, 1, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
     }
     return launch_status();
 }
@@ -286,7 +355,7 @@ int forced_tile() {
         const char* e = getenv("VV_GEMM_TILE");
         return e ? atoi(e) : 0;
     }();
-    return (v >= 0 && v <= 3) ? v : 0;
+    return (v >= 0 && v <= 4) ? v : 0;
 }
 
 }  // namespace
