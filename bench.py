@@ -224,6 +224,70 @@ def decode_graph_leg(torch, dev, wl1) -> dict:
             "replay_us_per_launch": replay * 1e6 / launches}
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0        # MI355X dense FP16 matrix rate
+
+
+def layer_leg(torch, dev, T: int, st: int) -> dict:
+    """The rest of a dense Qwen2-7B layer at the same prompt length: the four projection shapes of
+    the FP16 GEMM and causal GQA attention at M = T (matrix-core bound: TFLOP/s against the dense
+    FP16 peak), and the decode forms (one row: bound by the weight / cache bytes, GB/s). Not part of
+    the step; the causal FLOP count is 4 * heads * head_dim * T(T+1)/2."""
+    import ctypes as C
+
+    def timed(fn, launches, reps=3):
+        fn()
+        per = []
+        for _ in range(reps):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(launches):
+                fn()
+            e1.record()
+            e1.synchronize()
+            per.append(e0.elapsed_time(e1) * 1e-3 / launches)
+        per.sort()
+        return per[len(per) // 2]
+
+    out = {"gemm": {}, "gemv": {}}
+    shapes = (("q_o_proj", H, H), ("kv_proj", NK * HD, H), ("gate_up_proj", I_FF, H), ("down_proj", H, I_FF))
+    for name, n, k in shapes:
+        w = torch.randn(n, k, dtype=torch.float16, device="cuda") * k ** -0.5
+        for m, key in ((T, "gemm"), (1, "gemv")):
+            a = torch.randn(m, k, dtype=torch.float16, device="cuda")
+            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+            sec = timed(lambda: dev.vv_gemm_fp16_dev(a.data_ptr(), w.data_ptr(), c.data_ptr(), m, n, k,
+                                                     1.0, 0.0, st), 5 if m > 1 else 50)
+            if m > 1:
+                tf = 2.0 * m * n * k / sec / 1e12
+                out[key][name] = {"M": m, "N": n, "K": k, "us": sec * 1e6, "TFLOPs": tf,
+                                  "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+            else:
+                gb = 2.0 * (n * k + k + n) / sec / 1e9
+                out[key][name] = {"N": n, "K": k, "us": sec * 1e6, "GBps": gb,
+                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+            del a, c
+        del w
+    q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
+    k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
+    v_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
+    o = torch.empty_like(q)
+    view = dev.KvView(k=k_.data_ptr(), v=v_.data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                      format=0, n_kv_heads=NK, head_dim=HD)
+    sec = timed(lambda: dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view), o.data_ptr(), NQ, T, 0, T,
+                                            True, None, st), 3)
+    tf = 4.0 * NQ * HD * T * (T + 1) / 2 / sec / 1e12
+    out["attn_prefill"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf,
+                           "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+    scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
+    sec = timed(lambda: dev.vv_attn_decode(2, q.data_ptr(), C.addressof(view), o.data_ptr(), NQ, T, None,
+                                           scratch.data_ptr(), st), 50)
+    gb = 2.0 * T * NK * HD * 2 / sec / 1e9
+    out["attn_decode"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS,
+                          "note": "two launches; the host's launch rate bounds this figure"}
+    return out
+
+
 def cpu_baseline(rows: int) -> dict:
     """The CPU path of the same step on `rows` rows: warm-up, then best of five
     (bench/benchmark.c:197-211). FP32 activations, so its byte count is its own."""
@@ -328,6 +392,9 @@ def main() -> int:
     ap.add_argument("--unfused", action="store_true",
                     help="also time the unfused reference-API calls and the int8-activation fused "
                          "forms (reported under 'unfused'; not part of the step)")
+    ap.add_argument("--layer", action="store_true",
+                    help="also time the dense GEMM and attention entry points at the layer's shapes "
+                         "(reported under 'layer'; not part of the step)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
                          "five times: the known-size reference for rocprofv3 byte counters")
@@ -402,6 +469,20 @@ def main() -> int:
             log(f"  {name:12s} {med * 1e6:9.2f} us  {unfused[name]['GBps']:8.1f} GB/s  "
                 f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (not part of the step)")
 
+    layer = {}
+    if args.layer:
+        layer = layer_leg(torch, dev, T, st)
+        for name, d in layer["gemm"].items():
+            log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+                f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+        for name, d in layer["gemv"].items():
+            log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        d = layer["attn_prefill"]
+        log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+            f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+        d = layer["attn_decode"]
+        log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+
     # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
     decode = {}
     if not args.only:
@@ -443,6 +524,8 @@ def main() -> int:
     }
     if unfused:
         result["unfused"] = unfused
+    if layer:
+        result["layer"] = layer
     if decode:
         result["decode_T1_us"] = decode
     if graph:
