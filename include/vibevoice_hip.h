@@ -124,9 +124,11 @@ vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* str
 /* ── Dense linear layers ───────────────────────────────────────────────── */
 
 /* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32
- * accumulation on the matrix cores. beta == 0 never reads C. M <= 8 streams
- * the weight rows once (one wave per output column); larger M runs 32x64,
- * 64x64 or 128x128 workgroup tiles, all of which add K in the same order and
+ * accumulation on the matrix cores. beta == 0 never reads C. M == 1 streams
+ * the weight rows once (one wave per output column); 2 <= M <= 64 feeds them
+ * from global memory straight into the MFMA operands with K split over a
+ * workgroup's waves; larger M runs 128x128 or 256x256 workgroup tiles (64x64
+ * when there are too few of those), all of which add K in the same order and
  * so give the same bits for an element. K % 8 != 0 or A/B off 16 bytes take a
  * scalar kernel. M <= 0 or N <= 0: VV_OK, nothing launched.
  * replaces device.h:423-425 (src/cuda/gemm.cu). */

@@ -15,10 +15,13 @@
 //                           row: 8-byte stores. Every tile shape adds the K
 //                           slabs in the same order, so all of them produce
 //                           the same bits for the same element.
-//   gemv_rows<MR>           M <= 8 (a decode step): one wave per output
+//   gemm_skinny<kMT>        2 <= M <= 64: the weights go from global memory
+//                           straight into 16x16x32 MFMA operands, K split
+//                           over the eight waves of a workgroup; bound by the
+//                           weight bytes.
+//   gemv_rows               M == 1 (a decode step): one wave per output
 //                           column streams that weight row once with
-//                           non-temporal 16-byte loads and keeps MR dot
-//                           products; bound by the weight bytes.
+//                           non-temporal 16-byte loads.
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
 #include "vv_common.hpp"
 
@@ -281,6 +284,101 @@ __global__ __launch_bounds__(kBlock) void gemv_rows(const h16* __restrict__ A,
     }
 }
 
+// M <= 64 (a streaming chunk, a few decode rows): bound by the weight bytes, so
+// the weights are read exactly once, straight from global memory into MFMA
+// operands, and K is split over the eight waves of a workgroup.
+//
+// A workgroup owns 16 output columns (weight rows) and all M rows. One
+// v_mfma_f32_16x16x32_f16 takes 16 weight rows x 32 K values as its A operand
+// (lane: row lane % 16, K chunk lane / 16) and 16 activation rows as its B
+// operand; kMT such products (M / 16 row tiles) reuse each weight fragment. A
+// wave takes every eighth 64-K "line" (two steps: the whole 128-byte cache line
+// of each weight row), two lines in flight per iteration; the eight partial
+// tiles meet in LDS. The activations (M x K, at most 2.4 MB) come from L1/L2.
+// The K order differs from gemm_tile's, so the bits may too (same bounds).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kSkinnyWaves = 8;
+
+template <int kMT>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
+    const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
+    int K, float alpha, float beta, int vec_store) {
+    __shared__ f32x4 part[kSkinnyWaves][kMT][kWave];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16;
+    const int kchunks = K / 8;
+    const int nlines = (kchunks + 7) / 8;                 // 64 K values = 8 chunks per line
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(B + (size_t)min(n0 + r16, N - 1) * K);
+    const u32x4* arow[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t)
+        arow[t] = reinterpret_cast<const u32x4*>(A + (size_t)min(16 * t + r16, M - 1) * K);
+
+    f32x4 acc[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int line = wave; line < nlines; line += 2 * kSkinnyWaves) {
+        u32x4 w[4], x[kMT][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {                     // (line, step) = (u / 2, u % 2)
+            const int c = (line + (u >> 1) * kSkinnyWaves) * 8 + (u & 1) * 4 + ks;
+            const bool live = c < kchunks;
+            w[u] = live ? wrow[c] : zero;
+#pragma unroll
+            for (int t = 0; t < kMT; ++t) x[t][u] = live ? arow[t][c] : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, w[u]),
+                                                                __builtin_bit_cast(h16x8, x[t][u]),
+                                                                acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    // Register r of lane l is column n0 + 4(l / 16) + r of row 16t + l % 16.
+    if (tid < kMT * kWave) {
+        const int t = tid >> 6;
+        f32x4 sum = part[0][t][lane];
+#pragma unroll
+        for (int w = 1; w < kSkinnyWaves; ++w) {
+            const f32x4 p = part[w][t][lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[r] += p[r];
+        }
+        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        if (m < M && n < N) {
+            h16* crow = C + (size_t)m * N;
+            if (vec_store && n + 3 < N) {
+                typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+                h16x4 old = {0, 0, 0, 0};
+                if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = to_half(finish(sum[r], alpha, beta, old[r]));
+                *reinterpret_cast<h16x4*>(crow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) {
+                        const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                        crow[n + r] = to_half(finish(sum[r], alpha, beta, old));
+                    }
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void gemm_naive(const h16* A, const h16* B, h16* C, int M,
                                                      int N, int K, float alpha, float beta) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -326,11 +424,24 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         gemm_naive<<<dim3((unsigned)blocks), kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
         return launch_status();
     }
-    if (allow_gemv && M <= 8) {
+    if (allow_gemv && M == 1) {
         const dim3 grid((unsigned)((N + kWavesPerBlock - 1) / kWavesPerBlock));
-        if (M == 1) gemv_rows<1><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
-        else if (M <= 4) gemv_rows<4><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
-        else gemv_rows<8><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        gemv_rows<1><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        return launch_status();
+    }
+    // Up to 64 rows: the weight-streaming kernel, unless there are more than 16
+    // rows and enough 64-wide column tiles to fill the chip (then the tile
+    // kernel's LDS reuse of the activations wins: M = 29, N = 18944 is 31 us
+    // tiled against 46 us streamed; N = 3584, K = 18944 is 136 us against 48 us).
+    const bool few_tiles = (long)((N + 63) / 64) < 200;
+    if (allow_gemv && (M <= 16 || (M <= 64 && few_tiles))) {
+        const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+        const dim3 grid((unsigned)((N + 15) / 16));
+        constexpr int kThreads = kSkinnyWaves * kWave;
+        if (M <= 16) gemm_skinny<1><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
+        else if (M <= 32) gemm_skinny<2><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
+        else if (M <= 48) gemm_skinny<3><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
+        else gemm_skinny<4><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
         return launch_status();
     }
     if (choice == kAuto) {
