@@ -288,6 +288,103 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
     return out
 
 
+def decode_token_leg(torch, dev, cache_len: int, layers: int = 28) -> dict:
+    """One decode step of a dense Qwen2-7B-shaped decoder (random weights, 13 GB of them) on this
+    library's entry points alone, in the reference decoder's op order (decoder.c:706-991): per layer
+    norm -> q/k/v GEMV -> bias + RoPE at a device-side position -> KV append at that position ->
+    split decode attention over `cache_len` positions -> o GEMV -> add+norm -> gate/up GEMV ->
+    SwiGLU -> down GEMV -> add+norm. Issued directly, then as one captured graph whose replays
+    advance the position on the device. The floor is the weight bytes over the HBM rate."""
+    import ctypes as C
+    s = C.c_void_p()
+    assert dev.vv_dev_stream_create(C.byref(s)) == 0
+    st = s.value
+    f16 = dict(dtype=torch.float16, device="cuda")
+    QD, KD = NQ * HD, NK * HD
+
+    def w(*shape, std):
+        return torch.randn(*shape, **f16) * std
+
+    wq, wo = w(layers, QD, H, std=H ** -0.5), w(layers, H, QD, std=QD ** -0.5)
+    wk, wv = w(layers, KD, H, std=H ** -0.5), w(layers, KD, H, std=H ** -0.5)
+    wg, wu = w(layers, I_FF, H, std=H ** -0.5), w(layers, I_FF, H, std=H ** -0.5)
+    wd = w(layers, H, I_FF, std=I_FF ** -0.5)
+    bq, bk, bv = w(layers, QD, std=0.1), w(layers, KD, std=0.1), w(layers, KD, std=0.1)
+    n_in, n_post = 1 + w(layers + 1, H, std=0.1), 1 + w(layers, H, std=0.1)
+    room = cache_len + 256
+    kc, vc = w(layers, room, NK, HD, std=1.0), w(layers, room, NK, HD, std=1.0)
+    hidden, normed = w(1, H, std=1.0), torch.empty(1, H, **f16)
+    q, k, v = torch.empty(1, QD, **f16), torch.empty(1, KD, **f16), torch.empty(1, KD, **f16)
+    attn, proj = torch.empty(1, QD, **f16), torch.empty(1, H, **f16)
+    gate, up = torch.empty(1, I_FF, **f16), torch.empty(1, I_FF, **f16)
+    pos = torch.tensor([cache_len - 1], dtype=torch.int32, device="cuda")    # the new token's position
+    nxt = torch.tensor([cache_len], dtype=torch.int32, device="cuda")        # cache length once appended
+    scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
+    views = [dev.KvView(k=kc[l].data_ptr(), v=vc[l].data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                        format=0, n_kv_heads=NK, head_dim=HD) for l in range(layers)]
+    weight_bytes = sum(t.numel() * 2 for t in (wq, wo, wk, wv, wg, wu, wd))
+    P = lambda t: t.data_ptr()
+
+    def gemv(x, wt, y, n, kk):
+        assert dev.vv_gemm_fp16_dev(P(x), P(wt), P(y), 1, n, kk, 1.0, 0.0, st) == 0
+
+    def token():
+        n = 1
+        assert dev.vv_rmsnorm_dev(P(hidden), P(n_in[0]), P(normed), 1, H, EPS, st) == 0
+        for l in range(layers):
+            gemv(normed, wq[l], q, QD, H)
+            gemv(normed, wk[l], k, KD, H)
+            gemv(normed, wv[l], v, KD, H)
+            assert dev.vv_bias_rope_qk_dev(P(q), P(k), P(bq[l]), P(bk[l]), 1, NQ, NK, HD, 0, P(pos), THETA, st) == 0
+            assert dev.vv_bias_add_dev(P(v), P(bv[l]), 1, KD, st) == 0
+            assert dev.vv_dev_memcpy_d2d_at(P(kc[l]), P(k), KD * 2, P(pos), st) == 0
+            assert dev.vv_dev_memcpy_d2d_at(P(vc[l]), P(v), KD * 2, P(pos), st) == 0
+            assert dev.vv_attn_decode(2, P(q), C.addressof(views[l]), P(attn), NQ, cache_len, P(nxt),
+                                      P(scratch), st) == 0
+            gemv(attn, wo[l], proj, H, QD)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_post[l]), P(normed), 1, H, EPS, st) == 0
+            gemv(normed, wg[l], gate, I_FF, H)
+            gemv(normed, wu[l], up, I_FF, H)
+            assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), I_FF, st) == 0
+            gemv(gate, wd[l], proj, H, I_FF)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_in[l + 1]), P(normed), 1, H, EPS, st) == 0
+            n += 16
+        assert dev.vv_pos_add_dev(P(pos), P(pos), 1, st) == 0
+        assert dev.vv_pos_add_dev(P(nxt), P(nxt), 1, st) == 0
+        return n + 2
+
+    torch.cuda.synchronize()
+    launches = token()
+    assert dev.vv_dev_stream_sync(st) == 0
+    reps = 10
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        token()
+    assert dev.vv_dev_stream_sync(st) == 0
+    eager = (time.perf_counter() - t0) / reps
+    assert dev.vv_dev_graph_begin(st) == 0
+    token()
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(st, C.byref(g)) == 0 and g.value
+    for _ in range(2):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    before = int(pos.item())
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    replay = (time.perf_counter() - t0) / reps
+    assert int(pos.item()) == before + reps and int(nxt.item()) == before + reps + 1
+    assert bool(torch.isfinite(normed).all())
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(st)
+    return {"layers": layers, "cache_len": cache_len, "launches": launches, "weight_bytes": weight_bytes,
+            "eager_ms": eager * 1e3, "graph_ms": replay * 1e3, "tokens_per_s": 1.0 / replay,
+            "weight_GBps": weight_bytes / replay / 1e9,
+            "frac_of_hbm_peak": weight_bytes / replay / 1e9 / HBM_PEAK_GBPS}
+
+
 def cpu_baseline(rows: int) -> dict:
     """The CPU path of the same step on `rows` rows: warm-up, then best of five
     (bench/benchmark.c:197-211). FP32 activations, so its byte count is its own."""
@@ -482,6 +579,10 @@ def main() -> int:
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         d = layer["attn_decode"]
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        layer["decode_token"] = d = decode_token_leg(torch, dev, T)
+        log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
 
     # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
     decode = {}
