@@ -46,6 +46,45 @@ __device__ __forceinline__ float finish(float acc, float alpha, float beta, h16 
     return alpha * acc + beta * (float)old;
 }
 
+// A wave's TN x TM accumulator tiles to C. Result register 4g + r of lane l holds
+// column n0 + 8g + 4(l / 32) + r of row m0 + l % 32 of its 32x32 tile.
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile(const f32x16 (&acc)[TN][TM], h16* __restrict__ C, int M,
+                                           int N, int m0, int n0, int frow, int fhalf, float alpha,
+                                           float beta, int vec_store) {
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const int m = m0 + b * 32 + frow;
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+#pragma unroll
+        for (int a = 0; a < TN; ++a) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + a * 32 + 8 * g + 4 * fhalf;
+                if (n >= N) continue;
+                if (vec_store && n + 3 < N) {
+                    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+                    h16x4 old = {0, 0, 0, 0};
+                    if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+                    h16x4 o;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        o[r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old[r]));
+                    *reinterpret_cast<h16x4*>(crow + n) = o;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < N) {
+                            const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                            crow[n + r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old));
+                        }
+                }
+            }
+        }
+    }
+}
+
 template <int kValue>
 struct Const { static constexpr int value = kValue; };
 
@@ -209,39 +248,127 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
         }
     }
 
-    // Result register 4g + r of lane l holds column n0 + 8g + 4(l / 32) + r of
-    // row m0 + l % 32.
+    store_tile<TM, TN>(acc, C, M, N, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf, alpha, beta,
+                       vec_store);
+}
+
+// The 256x256 tile again, with the slabs going from global memory STRAIGHT into
+// LDS (global_load_lds_dwordx4: each lane's 16 bytes land at M0 + lane * 16, no
+// staging registers) and four LDS stages, so a slab is requested three compute
+// phases before it is read: deep enough to hide a last-level-cache miss. The
+// copy is asynchronous and the compiler is not told about it (it would wait for
+// ALL outstanding copies before any LDS read): the wave counts its own copies
+// with s_waitcnt vmcnt, then the workgroup barrier makes every wave's part
+// visible. Since a lane cannot choose where its bytes land, the bank swizzle is
+// applied on the global side: the lane that owns LDS slot (row, p) fetches the
+// row's logical slot p ^ swizzle(row). Needs K % 32 == 0 (no zero fill).
+constexpr int kDmaStages = 4;
+constexpr int kDmaSlab = 32;
+constexpr int kDmaTile = 256;
+constexpr int kDmaWaves = 8;
+constexpr int kDmaStageSlots = 2 * kDmaTile * (kDmaSlab / 8);   // 16-byte slots per stage: A rows, then B rows
+constexpr size_t kDmaLdsBytes = (size_t)kDmaStages * kDmaStageSlots * 16;
+
+// One wave-wide copy: lane l's 16 bytes at gptr go to LDS byte lds_byte_addr + 16 l.
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_byte_addr), "v"(gptr)
+                 : "memory", "m0");
+}
+
+__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
+    const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
+    int K, float alpha, float beta, int vec_store) {
+    constexpr int kSlabChunks = kDmaSlab / 8;             // 4
+    constexpr int WN = 4, TM = 4, TN = 2;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
+    constexpr int kLoads = kDmaStageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 4
+    extern __shared__ u32x4 dma_lds[];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int m_blk = (int)blockIdx.y * kDmaTile;
+    const int n_blk = (int)blockIdx.x * kDmaTile;
+    const int nslabs = K / kDmaSlab;
+    const uint32_t lds0 =
+        (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
+
+    // Copy i of this wave fills slots (wave + 8i) * 64 .. + 63 of a stage: 16
+    // rows x 4 slots. The lane owns (row, physical slot) and fetches the logical
+    // slot that the swizzle maps there.
+    const char* src[kLoads];
+    uint32_t dst[kLoads];
 #pragma unroll
-    for (int b = 0; b < TM; ++b) {
-        const int m = m_blk + (wm * TM + b) * 32 + frow;
-        if (m >= M) continue;
-        h16* crow = C + (size_t)m * N;
-#pragma unroll
-        for (int a = 0; a < TN; ++a) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = n_blk + (wn * TN + a) * 32 + 8 * g + 4 * fhalf;
-                if (n >= N) continue;
-                if (vec_store && n + 3 < N) {
-                    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
-                    h16x4 old = {0, 0, 0, 0};
-                    if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
-                    h16x4 o;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        o[r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old[r]));
-                    *reinterpret_cast<h16x4*>(crow + n) = o;
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (n + r < N) {
-                            const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
-                            crow[n + r] = to_half(finish(acc[a][b][4 * g + r], alpha, beta, old));
-                        }
-                }
-            }
-        }
+    for (int i = 0; i < kLoads; ++i) {
+        const int slot0 = (wave + kDmaWaves * i) * kWave;
+        const int p = slot0 + lane;
+        const int row = p / kSlabChunks, phys = p % kSlabChunks;    // row 0..511: A rows then B rows
+        const int logical = swz<kDmaSlab>(row, phys);
+        const bool is_b = row >= kDmaTile;
+        const int r = is_b ? row - kDmaTile : row;
+        const h16* base = is_b ? B + (size_t)min(n_blk + r, N - 1) * K : A + (size_t)min(m_blk + r, M - 1) * K;
+        src[i] = reinterpret_cast<const char*>(base) + logical * 16;
+        dst[i] = lds0 + (uint32_t)slot0 * 16u;
     }
+    auto request = [&](int slab) {        // slab -> stage slab % 4; past the end: the last slab again
+        const size_t adv = (size_t)min(slab, nslabs - 1) * (kDmaSlab * 2);
+        const uint32_t stage = (uint32_t)(slab % kDmaStages) * (kDmaStageSlots * 16u);
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) lds_dma16(src[i] + adv, dst[i] + stage);
+    };
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    int f_idx[2];
+#pragma unroll
+    for (int step = 0; step < 2; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<kDmaSlab>(frow, step * 2 + fhalf);
+    const int fa_base = wm * TM * 32 * kSlabChunks;
+    const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
+
+    request(0);
+    request(1);
+    request(2);
+    for (int slab = 0; slab < nslabs; ++slab) {
+        // This wave's copies of slabs slab+1 and slab+2 (8 of them) may still fly.
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        __syncthreads();                  // everyone's part of `slab` is in LDS; stage (slab+3)%4 is free
+        request(slab + 3);
+        const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
+        h16x8 fw[2][TN], fx[2][TM];
+#pragma unroll
+        for (int step = 0; step < 2; ++step) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+                fw[step][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                fx[step][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int step = 0; step < 2; ++step)
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[step][a], fx[step][b],
+                                                                       acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
+
+    store_tile<TM, TN>(acc, C, M, N, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf, alpha, beta,
+                       vec_store);
 }
 
 // One wave per output column n; MR rows of A share each weight chunk.
@@ -407,7 +534,30 @@ void launch_tile(const void* A, const void* B, void* C, int M, int N, int K, flo
             alpha, beta, vec);
 }
 
-enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4 };
+bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+                hipStream_t st) {
+    // 128 KB of LDS per workgroup is above the default limit: raised once per thread and device.
+    static thread_local int ready_device = -1;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return false;
+    if (ready_device != device) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kDmaLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        ready_device = device;
+    }
+    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    const dim3 grid((unsigned)((N + kDmaTile - 1) / kDmaTile), (unsigned)((M + kDmaTile - 1) / kDmaTile));
+    gemm_dma<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(
+        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha,
+        beta, vec);
+    return true;
+}
+
+enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4, k256dma = 5 };
 
 vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                  float beta, void* stream, int choice, bool allow_gemv) {
@@ -453,6 +603,9 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128 : (M > 32) ? k64 : k32;
     }
     switch (choice) {
+        case k256dma:
+            if (K % kDmaSlab == 0 && K >= 3 * kDmaSlab && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
+            [[fallthrough]];
         case k256: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k64:  launch_tile<64, 64, 2, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
@@ -466,7 +619,7 @@ int forced_tile() {
         const char* e = getenv("VV_GEMM_TILE");
         return e ? atoi(e) : 0;
     }();
-    return (v >= 0 && v <= 4) ? v : 0;
+    return (v >= 0 && v <= 5) ? v : 0;
 }
 
 }  // namespace
