@@ -335,34 +335,51 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     const int fa_base = wm * TM * 32 * kSlabChunks;
     const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
 
+    // Fragment reads run one MFMA group ahead: while the 8 MFMAs of a K step
+    // execute, the operands of the next step (the next slab's first step, after
+    // the barrier) come in from LDS.
+    h16x8 fw[2][TN], fx[2][TM];
+    auto read_frags = [&](auto set_c, int slab, int step) {
+        constexpr int set = decltype(set_c)::value;
+        const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+            fw[set][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+            fx[set][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
+    };
+    auto mfma_group = [&](auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[set][a], fx[set][b], acc[a][b],
+                                                                   0, 0, 0);
+    };
+
     request(0);
     request(1);
     request(2);
+    request(3);
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __syncthreads();
+    read_frags(Const<0>{}, 0, 0);
     for (int slab = 0; slab < nslabs; ++slab) {
-        // This wave's copies of slabs slab+1 and slab+2 (8 of them) may still fly.
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        __syncthreads();                  // everyone's part of `slab` is in LDS; stage (slab+3)%4 is free
-        request(slab + 3);
-        const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
-        h16x8 fw[2][TN], fx[2][TM];
-#pragma unroll
-        for (int step = 0; step < 2; ++step) {
-#pragma unroll
-            for (int a = 0; a < TN; ++a)
-                fw[step][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
-#pragma unroll
-            for (int b = 0; b < TM; ++b)
-                fx[step][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
-        }
+        read_frags(Const<1>{}, slab, 1);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int step = 0; step < 2; ++step)
-#pragma unroll
-            for (int a = 0; a < TN; ++a)
-#pragma unroll
-                for (int b = 0; b < TM; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[step][a], fx[step][b],
-                                                                       acc[a][b], 0, 0, 0);
+        mfma_group(Const<0>{});
+        __builtin_amdgcn_sched_barrier(0);
+        // Slab + 1 must be in LDS (this wave's copies of slabs + 2 and + 3, 8 of
+        // them, may still fly), and every wave must be done reading this slab
+        // before its stage is handed to slab + 4.
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        request(slab + 4);
+        read_frags(Const<0>{}, slab + 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(Const<1>{});
         __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
@@ -604,7 +621,7 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
     }
     switch (choice) {
         case k256dma:
-            if (K % kDmaSlab == 0 && K >= 3 * kDmaSlab && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
+            if (K % kDmaSlab == 0 && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
             [[fallthrough]];
         case k256: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;
