@@ -3,7 +3,7 @@
 //
 // Both operands are contiguous along K, which is what the CDNA4 matrix core
 // wants: v_mfma_f32_32x32x16_f16 takes, per lane, eight consecutive K values
-// of one row of each operand. Three kernels:
+// of one row of each operand. The kernels:
 //
 //   gemm_tile<BM,BN,WM,WN>  workgroup tile BM x BN over WM x WN waves, K in
 //                           slabs of 64 or 32 staged through LDS (double-buffered,
@@ -15,6 +15,9 @@
 //                           row: 8-byte stores. Every tile shape adds the K
 //                           slabs in the same order, so all of them produce
 //                           the same bits for the same element.
+//   gemm_dma                the 256x256 tile for large problems: slabs copied
+//                           from global memory straight into LDS (no staging
+//                           registers), four LDS stages, same K order.
 //   gemm_skinny<kMT>        2 <= M <= 64: the weights go from global memory
 //                           straight into 16x16x32 MFMA operands, K split
 //                           over the eight waves of a workgroup; bound by the
@@ -574,7 +577,7 @@ bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, floa
     return true;
 }
 
-enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4, k256dma = 5 };
+enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4, k256regs = 5 };
 
 vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                  float beta, void* stream, int choice, bool allow_gemv) {
@@ -613,17 +616,19 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
     }
     if (choice == kAuto) {
         // The largest tile that still fills the 256 compute units: 256x256
-        // (eight waves, the fewest L1 and LDS bytes per MFMA) from two full
-        // rounds of workgroups on, 128x128 from one round on.
+        // (eight waves, the fewest L1 and LDS bytes per MFMA; fed by direct
+        // global-to-LDS copies when K is a multiple of 32, through registers
+        // otherwise) from two full rounds of workgroups on, 128x128 from one
+        // round on.
         const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
         choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128 : (M > 32) ? k64 : k32;
     }
     switch (choice) {
-        case k256dma:
+        case k256:
             if (K % kDmaSlab == 0 && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
             [[fallthrough]];
-        case k256: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k256regs: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k64:  launch_tile<64, 64, 2, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
         default:   launch_tile<32, 64, 1, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
