@@ -145,37 +145,43 @@ __device__ __forceinline__ void tile_scores(const KvTile& tile, const h16x8 (&qf
     }
 }
 
-// s holds the masked, scaled scores (-inf where unseen). Online-softmax update
-// of the row state, then O^T += V^T P^T over the tile's four 16-key steps. Slot
-// e of this lane in step (a, sp) is register 8*sp + e of s[a], i.e. key
-// 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte reads of V^T below.
+// s holds the raw scores (-inf where unseen); scale_log2 = log2(e) / sqrt(d) > 0
+// turns them into base-2 exponents inside one fused multiply-add per value.
+// Online-softmax update of the row state, then O^T += V^T P^T over the tile's
+// four 16-key steps. Slot e of this lane in step (a, sp) is register 8*sp + e
+// of s[a], i.e. key 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte
+// reads of V^T below. O is rescaled only when some row's maximum moved (after
+// the first few tiles it rarely does): the factor is exactly 1 otherwise.
 __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], RowState& st,
-                                            int col, int half) {
+                                            int col, int half, float scale_log2) {
     float mx = -INFINITY;
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
-    mx = fmaxf(mx, other_half(mx));
+    mx = fmaxf(mx, other_half(mx)) * scale_log2;
     const float m_new = fmaxf(st.m, mx);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-    const float alpha = exp2_fast(st.m - m_use);
     float sum = 0.0f;
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float p = exp2_fast(s[a][r] - m_use);
+            const float p = exp2_fast(fmaf(s[a][r], scale_log2, -m_use));
             s[a][r] = p;
             sum += p;
         }
     sum += other_half(sum);
-    st.l = st.l * alpha + sum;
+    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
+        const float alpha = exp2_fast(st.m - m_use);
+        st.l *= alpha;
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+    }
+    st.l += sum;
     st.m = m_new;
-#pragma unroll
-    for (int t = 0; t < kD / 32; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int a = u >> 1, sp = u & 1;
@@ -243,15 +249,19 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
         if (t0 >= wave_limit) continue;
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
+        // Only a tile that reaches past the cache end or past the wave's first
+        // row's position has anything to hide.
+        if (t0 + kKeyTile > kv_len || (causal && t0 + kKeyTile - 1 > q_offset + qw0)) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
-                const bool seen = key < kv_len && (!causal || key <= q_abs);
-                s[a][r] = seen ? s[a][r] * scale_log2 : -INFINITY;
-            }
-        tile_update(tile, s, st, col, half);
+                for (int r = 0; r < 16; ++r) {
+                    const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const bool seen = key < kv_len && (!causal || key <= q_abs);
+                    s[a][r] = seen ? s[a][r] : -INFINITY;
+                }
+        }
+        tile_update(tile, s, st, col, half, scale_log2);
     }
 
     if (qrow < q_len) {
@@ -357,14 +367,16 @@ __global__ __launch_bounds__(kWave) void decode128(
             fetch_tile<kWave>(regs, Kc, Vc, page_table, kv_stride, kvh, t0 + kKeyTile, end - 1, lane);
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
+        if (t0 + kKeyTile > end) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
-                s[a][r] = key < end ? s[a][r] * scale_log2 : -INFINITY;
-            }
-        tile_update(tile, s, st, col, half);
+                for (int r = 0; r < 16; ++r) {
+                    const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
+                    s[a][r] = key < end ? s[a][r] : -INFINITY;
+                }
+        }
+        tile_update(tile, s, st, col, half, scale_log2);
     }
 
     if (g >= group) return;
