@@ -199,6 +199,21 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
 vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages,
                                void* stream);
 
+/* ── LM head ───────────────────────────────────────────────────────────── */
+
+/* logits[V] = W[V,K] x[K]; x, W FP16, FP32 accumulation, FP32 logits. Bound by
+ * the table bytes: one wave per vocabulary row streams it once.
+ * replaces device.h:706-707 (src/cuda/lm_head.cu:139-152). */
+vv_status_t vv_lm_head_gemv_dev(const void* x, const void* W, void* logits, int V,
+                                int K, void* stream);
+/* Greedy argmax over FP32 logits on the device, two launches; scratch_v
+ * (FP32) and scratch_i (int32) hold 256 partial winners each; out_token int32,
+ * out_value FP32 or NULL. The lowest index among equal maxima wins (the CPU
+ * sampler's in-order scan, src/cpu/cpu_kernels.c:1613-1623); a NaN never wins.
+ * replaces device.h:710-712 (lm_head.cu:163-183). */
+vv_status_t vv_argmax_dev(const void* logits, int V, void* scratch_v, void* scratch_i,
+                          void* out_token, void* out_value, void* stream);
+
 /* ── Fused forms (additions) ───────────────────────────────────────────── */
 
 /* addition: vv_residual_add_dev(residual, x) followed by

@@ -75,6 +75,8 @@ def _load():
     lib.vvo_gemm_f16w.argtypes = [_f32p, _u16p, _u16p, _f32p, C.c_int, C.c_int, C.c_int]
     lib.vvo_attention_prefill_f32.restype = C.c_int
     lib.vvo_attention_prefill_f32.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 7
+    lib.vvo_argmax_first.restype = C.c_int
+    lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
     lib.vvo_set_threads.argtypes = [C.c_int]
     for name in ("vvo_rmsnorm_f32", "vvo_rope_f32", "vvo_swiglu_f32", "vvo_residual_add_f32",
@@ -310,3 +312,11 @@ def attention_prefill_f32(q, k, v, q_offset: int, kv_len: int, causal: bool = Tr
                                          n_q, k.shape[1], hd, rows, q_offset, kv_len, int(causal)),
            "attention_prefill_f32")
     return out
+
+
+def argmax_first(logits: np.ndarray):
+    """(token, value): the first maximum of an in-order scan over float32 logits."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    tok, val = C.c_int32(), C.c_float()
+    _check(lib.vvo_argmax_first(_p(logits, _f32p), logits.size, C.byref(tok), C.byref(val)), "argmax_first")
+    return int(tok.value), float(val.value)

@@ -395,6 +395,17 @@ int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
     return VVO_OK;
 }
 
+int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value) {
+    if (!logits || !token) return VVO_ERR_NULL_PTR;
+    int best = 0;
+    float bv = logits[0];
+    for (int i = 1; i < n; i++)
+        if (logits[i] > bv) { bv = logits[i]; best = i; }
+    *token = best;
+    if (value) *value = bv;
+    return VVO_OK;
+}
+
 /* ── seeded inputs ─────────────────────────────────────────────────────── */
 
 static inline uint64_t splitmix64(uint64_t z) {

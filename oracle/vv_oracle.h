@@ -124,6 +124,10 @@ int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
                               int head_dim, int rows, int q_offset, int kv_len,
                               int causal);
 
+/* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
+ * an in-order scan; a NaN never replaces the running best. */
+int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);
+
 /* ── seeded inputs (the same bytes go to the oracle and to the GPU) ────── */
 
 /* N(mean, std) rounded to FP16 (RNE). Counter-based: element i depends only

@@ -76,3 +76,21 @@ def test_attention_closed_form_reference_and_invariants(rows, nq, nkv, hd, off, 
         # the decode form: the last row alone equals the last row of the batch
         last = oracle.attention_prefill_f32(q[-1:], k, v, off + rows - 1, kv_len, True)
         assert np.array_equal(last[0], got[-1])
+
+
+def test_argmax_first_against_numpy_and_reference():
+    """In-order scan, first maximum: numpy's argmax has the same rule; the
+    compiled reference's vv_sample_greedy_cpu is the function restated."""
+    rng = np.random.default_rng(3)
+    cases = [rng.standard_normal(1000).astype(np.float32), np.array([-3.0], np.float32),
+             np.array([1.0, 5.0, 5.0, 2.0, 5.0], np.float32), -np.ones(77, np.float32),
+             np.array([-np.inf, -np.inf, -1e30], np.float32)]
+    for x in cases:
+        tok, val = oracle.argmax_first(x)
+        assert tok == int(np.argmax(x)) and val == float(x.max())
+        if oracle.ref is not None and hasattr(oracle.ref, "vv_sample_greedy_cpu"):
+            t = C.c_int32()
+            assert oracle.ref.vv_sample_greedy_cpu(x.ctypes.data_as(f32p), x.size, C.byref(t)) == 0
+            assert t.value == tok
+    nan_mid = np.array([1.0, np.nan, 3.0, np.nan, 2.0], np.float32)      # a NaN never wins once a number leads
+    assert oracle.argmax_first(nan_mid)[0] == 2

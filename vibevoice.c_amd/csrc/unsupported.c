@@ -9,8 +9,8 @@
  * src/metal/metal_stubs.c:1-30, src/device/device_none.c:129-483).
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
- * HIP library does not define (dense/quantised GEMM and GEMV, attention, KV
- * cache, LM head, VAE, BitNet). It builds into its
+ * HIP library does not define (quantised-weight GEMM and GEMV, the small-M and
+ * NN dense forms, quantised KV formats, VAE, BitNet). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
  * stays exactly what include/vibevoice_hip.h declares.
@@ -53,8 +53,6 @@ VV_DECLINE(vv_gqa_attention_prefill_q_dev)
 VV_DECLINE(vv_kv_quant_store_dev) VV_DECLINE(vv_kv_dequant_dev)
 VV_DECLINE(vv_kv_rotate_dev)      VV_DECLINE(vv_kv_unrotate_dev)
 
-/* LM head (device.h:707-715) */
-VV_DECLINE(vv_lm_head_gemv_dev)  VV_DECLINE(vv_argmax_dev)
 
 /* Conv-VAE speech encoder (device.h:762-870) */
 VV_DECLINE(vv_vae_conv_dev)      VV_DECLINE(vv_vae_tail_dev)      VV_DECLINE(vv_vae_rms_dev)
