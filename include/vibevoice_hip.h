@@ -134,6 +134,24 @@ vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* str
  * replaces device.h:423-425 (src/cuda/gemm.cu). */
 vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N,
                              int K, float alpha, float beta, void* stream);
+/* One projection of a small-M launch: device.h:453-459. */
+typedef struct vv_skinny_proj {
+    const void* w;        /* FP16 [N][K] */
+    const void* scales;   /* quantised formats only: unused here */
+    const void* bias;     /* FP16 [N] or NULL */
+    void*       y;        /* FP16 [M][N] output */
+    int         N;
+} vv_skinny_proj_t;
+/* y_i = alpha * A[M,K] . W_i^T (+ bias_i) for up to three projections of the
+ * same A (q/k/v, gate/up) in one launch, M in 9..64, dense FP16 weights
+ * (format 0). The result equals vv_gemm_fp16_dev followed by vv_bias_add_dev
+ * bit for bit. Other formats, other M, K % 8 != 0, or a projection wide
+ * enough that vv_gemm_fp16_dev would tile it (N >= 12800 above 16 rows):
+ * VV_ERR_UNSUPPORTED, nothing launched; the caller runs that path itself
+ * (src/inference/decoder.c:375-378, 499-505). replaces device.h:472-475. */
+vv_status_t vv_skinny_linear_dev(const void* A, int format,
+                                 const vv_skinny_proj_t* projs, int n_proj,
+                                 int M, int K, float alpha, void* stream);
 /* The 128x128 tile alone, whatever M. replaces device.h:432-434. */
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
                                   int N, int K, float alpha, float beta,

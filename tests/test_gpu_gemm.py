@@ -107,3 +107,60 @@ def test_gemm_edges():
     want = (2.0 * oracle.widen(bits_of(c))).astype(np.float16).view(np.uint16)
     ok(dev.vv_gemm_fp16_dev(p, p, c.data_ptr(), 2, 8, 0, 1.0, 2.0, stream()))
     assert np.array_equal(bits_of(c), want)
+
+
+def skinny(d_a, ws, biases, M, K, alpha=1.0):
+    import ctypes as C
+    outs = [torch.full((M, w.shape[0]), float("nan"), dtype=torch.float16, device="cuda") for w in ws]
+    arr = (dev.SkinnyProj * len(ws))()
+    for i, (w, b, y) in enumerate(zip(ws, biases, outs)):
+        arr[i] = dev.SkinnyProj(w=w.data_ptr(), scales=None, bias=b.data_ptr() if b is not None else None,
+                                y=y.data_ptr(), N=w.shape[0])
+    st = dev.vv_skinny_linear_dev(d_a.data_ptr(), 0, C.addressof(arr), len(ws), M, K, alpha, stream())
+    return st, outs
+
+
+@pytest.mark.parametrize("M", [9, 29, 64])
+@pytest.mark.parametrize("Ns,K,with_bias", [((3584, 512, 512), 3584, True), ((1536, 256), 1536, True),
+                                            ((3584,), 18944, False), ((264, 40, 1000), 520, True)])
+def test_skinny_linear_equals_gemm_then_bias(M, Ns, K, with_bias):
+    """The reference's multi-projection small-M entry point (decoder.c:375, 499):
+    one launch, the same bits as vv_gemm_fp16_dev + vv_bias_add_dev per projection."""
+    d_a = to_dev(oracle.normal_f16((M, K), 31 + M))
+    ws = [to_dev(oracle.normal_f16((n, K), 40 + i, std=K ** -0.5)) for i, n in enumerate(Ns)]
+    bs = [to_dev(oracle.normal_f16((n,), 50 + i, std=0.3)) if with_bias and i != 1 else None for i, n in enumerate(Ns)]
+    st, outs = skinny(d_a, ws, bs, M, K, alpha=0.5)
+    assert st == dev.VV_OK
+    for w, b, y in zip(ws, bs, outs):
+        n = w.shape[0]
+        want = torch.full((M, n), float("nan"), dtype=torch.float16, device="cuda")
+        ok(dev.vv_gemm_fp16_dev(d_a.data_ptr(), w.data_ptr(), want.data_ptr(), M, n, K, 0.5, 0.0, stream()))
+        if b is not None:
+            ok(dev.vv_bias_add_dev(want.data_ptr(), b.data_ptr(), M, n, stream()))
+        assert np.array_equal(bits_of(y), bits_of(want))
+    # and against the oracle: alpha * A W^T + bias exactly, allowing the two FP16 roundings
+    # (product, then sum) and the FP32 accumulation
+    prod, mag = exact(bits_of(d_a), bits_of(ws[0]), None, 0.5, 0.0)
+    ref = prod + (oracle.widen(bits_of(bs[0])) if bs[0] is not None else 0.0)
+    got = oracle.widen(bits_of(outs[0])).astype(np.float64)
+    assert scaled_rel_err(got, ref) <= FP16_TOL
+    ulp = lambda v: np.spacing(np.abs(v).astype(np.float16)).astype(np.float64)
+    bound = 0.5 * ulp(prod) + 0.5 * ulp(ref) + 1e-5 * mag + 2.0 ** -24
+    assert np.max(np.abs(got - ref) / bound) <= 1.0
+
+
+def test_skinny_linear_declines():
+    M, K = 29, 512
+    d_a = to_dev(oracle.normal_f16((M, K), 1))
+    w = to_dev(oracle.normal_f16((256, K), 2))
+    wide = to_dev(oracle.normal_f16((12800, K), 3))
+    U = dev.VV_ERR_UNSUPPORTED
+    assert skinny(d_a, [w], [None], 8, K)[0] == U                       # below 9 rows
+    assert skinny(d_a, [w], [None], 65, K)[0] == U
+    assert skinny(d_a, [w, wide], [None, None], M, K)[0] == U          # vv_gemm_fp16_dev would tile this one
+    assert skinny(d_a, [w] * 3, [None] * 3, M, 500)[0] == U            # K % 8
+    import ctypes as C
+    arr = (dev.SkinnyProj * 1)(dev.SkinnyProj(w=w.data_ptr(), scales=None, bias=None, y=w.data_ptr(), N=256))
+    assert dev.vv_skinny_linear_dev(d_a.data_ptr(), 1, C.addressof(arr), 1, M, K, 1.0, stream()) == U   # INT8 weights
+    assert dev.vv_skinny_linear_dev(None, 0, C.addressof(arr), 1, M, K, 1.0, stream()) == dev.VV_ERR_NULL_PTR
+    torch.cuda.synchronize()

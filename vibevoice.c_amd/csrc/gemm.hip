@@ -446,17 +446,34 @@ __global__ __launch_bounds__(kBlock) void gemv_rows(const h16* __restrict__ A,
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyWaves = 8;
 
+// Up to three projections of the same activations in one launch (q/k/v,
+// gate/up): workgroups [first[p], first[p+1]) serve projection p. A bias, when
+// given, is added to the rounded FP16 product and rounded again, exactly as a
+// bias-add launch after the GEMM would.
+struct SkinnyProjs {
+    const h16* w[3];
+    const h16* bias[3];
+    h16* y[3];
+    int n[3];
+    int first[3];
+    int vec[3];
+};
+
 template <int kMT>
 __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
-    const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
-    int K, float alpha, float beta, int vec_store) {
+    const h16* __restrict__ A, SkinnyProjs projs, int M, int K, float alpha, float beta) {
     __shared__ f32x4 part[kSkinnyWaves][kMT][kWave];
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int r16 = lane & 15, ks = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16;
+    const int which = ((int)blockIdx.x >= projs.first[1]) + ((int)blockIdx.x >= projs.first[2]);
+    const h16* __restrict__ B = projs.w[which];
+    const h16* __restrict__ bias = projs.bias[which];
+    h16* __restrict__ C = projs.y[which];
+    const int N = projs.n[which], vec_store = projs.vec[which];
+    const int n0 = ((int)blockIdx.x - projs.first[which]) * 16;
     const int kchunks = K / 8;
     const int nlines = (kchunks + 7) / 8;                 // 64 K values = 8 chunks per line
     const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -512,18 +529,39 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
                 if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
                 h16x4 o;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = to_half(finish(sum[r], alpha, beta, old[r]));
+                for (int r = 0; r < 4; ++r) {
+                    o[r] = to_half(finish(sum[r], alpha, beta, old[r]));
+                    if (bias) o[r] = to_half((float)o[r] + (float)bias[n + r]);
+                }
                 *reinterpret_cast<h16x4*>(crow + n) = o;
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     if (n + r < N) {
                         const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
-                        crow[n + r] = to_half(finish(sum[r], alpha, beta, old));
+                        h16 o = to_half(finish(sum[r], alpha, beta, old));
+                        if (bias) o = to_half((float)o + (float)bias[n + r]);
+                        crow[n + r] = o;
                     }
             }
         }
     }
+}
+
+// The 64-column tile count below which the weight-streaming kernel beats the
+// tile kernel for 17..64 rows (M = 29, N = 18944 is 31 us tiled against 46 us
+// streamed; N = 3584, K = 18944 is 136 us against 48 us).
+inline bool few_tiles(int N) { return (long)((N + 63) / 64) < 200; }
+inline bool skinny_serves(int M, int N) { return M >= 2 && (M <= 16 || (M <= 64 && few_tiles(N))); }
+
+void launch_skinny(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha,
+                   float beta, hipStream_t st) {
+    constexpr int kThreads = kSkinnyWaves * kWave;
+    const dim3 grid((unsigned)blocks);
+    if (M <= 16) gemm_skinny<1><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else if (M <= 32) gemm_skinny<2><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else if (M <= 48) gemm_skinny<3><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else gemm_skinny<4><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
 }
 
 __global__ __launch_bounds__(kBlock) void gemm_naive(const h16* A, const h16* B, h16* C, int M,
@@ -600,18 +638,16 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         return launch_status();
     }
     // Up to 64 rows: the weight-streaming kernel, unless there are more than 16
-    // rows and enough 64-wide column tiles to fill the chip (then the tile
-    // kernel's LDS reuse of the activations wins: M = 29, N = 18944 is 31 us
-    // tiled against 46 us streamed; N = 3584, K = 18944 is 136 us against 48 us).
-    const bool few_tiles = (long)((N + 63) / 64) < 200;
-    if (allow_gemv && (M <= 16 || (M <= 64 && few_tiles))) {
-        const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
-        const dim3 grid((unsigned)((N + 15) / 16));
-        constexpr int kThreads = kSkinnyWaves * kWave;
-        if (M <= 16) gemm_skinny<1><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
-        else if (M <= 32) gemm_skinny<2><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
-        else if (M <= 48) gemm_skinny<3><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
-        else gemm_skinny<4><<<grid, kThreads, 0, st>>>(a, b, c, M, N, K, alpha, beta, vec);
+    // rows and enough 64-wide column tiles to fill the chip.
+    if (allow_gemv && skinny_serves(M, N)) {
+        SkinnyProjs projs = {};
+        projs.w[0] = b;
+        projs.y[0] = c;
+        projs.n[0] = N;
+        projs.vec[0] = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+        const int blocks = (N + 15) / 16;
+        projs.first[1] = projs.first[2] = blocks;
+        launch_skinny(a, projs, blocks, M, K, alpha, beta, st);
         return launch_status();
     }
     if (choice == kAuto) {
@@ -652,6 +688,34 @@ extern "C" {
 vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N, int K,
                              float alpha, float beta, void* stream) {
     return vv::gemm(A, B, C, M, N, K, alpha, beta, stream, vv::forced_tile(), true);
+}
+
+/* Declines (nothing launched) whatever vv_gemm_fp16_dev would not hand to the
+ * weight-streaming kernel, so that the caller's fallback (vv_gemm_fp16_dev, then
+ * vv_bias_add_dev, per projection) and this entry point always give the same bits. */
+vv_status_t vv_skinny_linear_dev(const void* A, int format, const vv_skinny_proj_t* projs, int n_proj,
+                                 int M, int K, float alpha, void* stream) {
+    if (!A || !projs) return VV_ERR_NULL_PTR;
+    if (format != 0 /* VV_SKINNY_F16 */ || n_proj < 1 || n_proj > 3 || M < 9 || M > 64 || K <= 0 ||
+        K % 8 != 0 || !vv::aligned16(A))
+        return VV_ERR_UNSUPPORTED;
+    vv::SkinnyProjs p = {};
+    int blocks = 0;
+    for (int i = 0; i < 3; ++i) {
+        p.first[i] = blocks;
+        if (i >= n_proj) continue;
+        if (!projs[i].w || !projs[i].y) return VV_ERR_NULL_PTR;
+        if (projs[i].N <= 0 || !vv::skinny_serves(M, projs[i].N) || !vv::aligned16(projs[i].w))
+            return VV_ERR_UNSUPPORTED;
+        p.w[i] = static_cast<const vv::h16*>(projs[i].w);
+        p.bias[i] = static_cast<const vv::h16*>(projs[i].bias);
+        p.y[i] = static_cast<vv::h16*>(projs[i].y);
+        p.n[i] = projs[i].N;
+        p.vec[i] = (projs[i].N % 4 == 0) && ((reinterpret_cast<uintptr_t>(projs[i].y) & 7u) == 0);
+        blocks += (projs[i].N + 15) / 16;
+    }
+    vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, alpha, 0.0f, vv::as_stream(stream));
+    return vv::launch_status();
 }
 
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M, int N, int K,

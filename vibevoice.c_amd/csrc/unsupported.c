@@ -40,8 +40,8 @@ VV_DECLINE(vv_w4a16_gather_dev)  VV_DECLINE(vv_w4a16_gemm_dev)    VV_DECLINE(vv_
 /* W8A8 / W4A8 linears (device.h:362-410); the activation quantisers are implemented */
 VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)   VV_DECLINE(vv_i8_linear_multi_dev)
 
-/* dense FP16 GEMM: the small-M and NN forms (device.h:472-482); NT is implemented */
-VV_DECLINE(vv_skinny_linear_dev)  VV_DECLINE(vv_gemm_fp16_nn_dev)
+/* dense FP16 GEMM: the NN form (device.h:477-479); the NT forms are implemented */
+VV_DECLINE(vv_gemm_fp16_nn_dev)
 void vv_gemm_cleanup() {}
 
 /* the older per-format attention entry points and the quantised KV formats

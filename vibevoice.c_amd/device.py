@@ -32,6 +32,12 @@ class KvView(C.Structure):
                 ("n_kv_heads", C.c_int), ("head_dim", C.c_int)]
 
 
+class SkinnyProj(C.Structure):
+    """vv_skinny_proj_t: one projection of a small-M multi-projection launch."""
+    _fields_ = [("w", C.c_void_p), ("scales", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p),
+                ("N", C.c_int)]
+
+
 # symbol -> (restype, argtypes); the complete export list of include/vibevoice_hip.h
 SIGNATURES = {
     "vv_embedding_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
@@ -59,6 +65,7 @@ SIGNATURES = {
     "vv_kv_page_map_dev": (_i, [_vp, _i, _i, _vp, _vp]),
     "vv_lm_head_gemv_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "vv_argmax_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp]),
+    "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
