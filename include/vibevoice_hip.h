@@ -180,11 +180,11 @@ typedef struct vv_kv_view {
  * replaces device.h:545-546 (src/cuda/attention_fi.cu:554-583). */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
                     int n_kv_heads, int head_dim);
-/* n_q_heads * 128 * (head_dim + 2) floats: the decode slices' partial states.
+/* n_q_heads * 256 * (head_dim + 4) floats: the decode slices' partial states.
  * replaces device.h:554 (attention_fi.cu:585-589). */
 size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim);
 /* The number of slices the decode splits `cache_len` positions into: 1, 2,
- * 4 ... 128, doubling as the length passes 64, 128, 256, ... A captured decode
+ * 4 ... 256, doubling as the length passes 64, 128, 256, ... A captured decode
  * step is valid while this stays equal. replaces device.h:562-563. */
 int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len);
 /* q_len query rows at absolute positions q_offset.. against the first kv_len

@@ -117,10 +117,10 @@ def test_attention_host_queries():
             assert got in (FA1, FA2, FI) and (requested in (AUTO, got) or paged)
             assert dev.vv_attn_resolve(requested, 3, paged, 28, 4, 128) == FA1     # not an FP16 cache
     assert dev.vv_attn_resolve(FA1, 0, True, 28, 4, 128) != FA1                    # fa1 never pages
-    assert dev.vv_attn_scratch_bytes(28, 4, 128) == 28 * 128 * 130 * 4
+    assert dev.vv_attn_scratch_bytes(28, 4, 128) == 28 * 256 * 132 * 4
     shapes = [dev.vv_attn_decode_shape(FA2, 28, 4, n) for n in range(1, 20000, 37)]
-    assert shapes == sorted(shapes) and shapes[0] == 1 and shapes[-1] == 128
-    assert set(shapes) <= {1, 2, 4, 8, 16, 32, 64, 128}
+    assert shapes == sorted(shapes) and shapes[0] == 1 and shapes[-1] == 256
+    assert set(shapes) <= {1, 2, 4, 8, 16, 32, 64, 128, 256}
     assert dev.vv_attn_decode_shape(FA2, 28, 4, 64) == 1 and dev.vv_attn_decode_shape(FA2, 28, 4, 65) == 2
 
 

@@ -32,10 +32,11 @@ namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kPage = 64;            // positions per page (include/vibevoice/kv_quant.h:52)
 constexpr int kFormatFp16 = 0;       // VV_KV_FP16
-constexpr int kMaxParts = 128;       // decode slices per KV head
+constexpr int kMaxParts = 256;       // decode slices per KV head
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(kWave) void rows_generic(
 // the heads sharing a KV head take the place of the prefill's query rows, so
 // the slice's K and V are read once for all of them. n_parts == 1 writes O;
 // otherwise each slice leaves (max, sum, unnormalised O) per head in `parts`.
-constexpr int kPartFloats = kD + 2;
+constexpr int kPartFloats = kD + 4;        // per (head, slice): 128 channels, max, sum, 2 unused (16-byte rows)
 
 __global__ __launch_bounds__(kWave) void decode128(
     const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
@@ -394,56 +395,72 @@ __global__ __launch_bounds__(kWave) void decode128(
             }
     } else {
         float* dst = parts + ((size_t)head * n_parts + part) * kPartFloats;
-        if (half == 0) { dst[0] = st.m; dst[1] = st.l; }
+        if (half == 0) { dst[kD] = st.m; dst[kD + 1] = st.l; }
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    dst[2 + 32 * t + 8 * q + 4 * half + r] = st.o[t][4 * q + r];
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 o = {st.o[t][4 * q], st.o[t][4 * q + 1], st.o[t][4 * q + 2], st.o[t][4 * q + 3]};
+                *reinterpret_cast<f32x4*>(dst + 32 * t + 8 * q + 4 * half) = o;
+            }
     }
 }
 
-// Folds the slices of one head: 8 groups of 128 threads take every 8th slice
-// for one channel each, so a thread's loads are few and independent.
+// Folds the slices of one head. The first n_parts threads turn the slices'
+// maxima into weights 2^(m_p - m_all) (kept in LDS) and sum the weighted
+// denominators; then 8 groups of 128 threads take every 8th slice for one
+// channel each, so a thread's loads are few and independent.
 constexpr int kMergeGroups = 8;
+constexpr int kMergeThreads = kD * kMergeGroups;
 
-__global__ __launch_bounds__(kD * kMergeGroups) void decode_merge(const float* __restrict__ parts,
-                                                                  h16* __restrict__ O,
-                                                                  int n_parts) {
-    __shared__ float s_max[kD * kMergeGroups / kWave];
+__global__ __launch_bounds__(kMergeThreads) void decode_merge(const float* __restrict__ parts,
+                                                              h16* __restrict__ O, int n_parts) {
+    __shared__ float s_f[kMaxParts];
+    __shared__ float s_red[2][kMergeThreads / kWave];
     __shared__ float s_o[kMergeGroups][kD];
-    __shared__ float s_l[kMergeGroups];
     const int head = (int)blockIdx.x, tid = (int)threadIdx.x;
     const int d = tid % kD, grp = tid / kD;
     const float* src = parts + (size_t)head * n_parts * kPartFloats;
 
-    float m = -INFINITY;
-    for (int p = tid; p < n_parts; p += kD * kMergeGroups) m = fmaxf(m, src[p * kPartFloats]);
-    m = wave_max(m);
-    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    const bool mine = tid < n_parts;
+    const float m = mine ? src[tid * kPartFloats + kD] : -INFINITY;
+    const float l = mine ? src[tid * kPartFloats + kD + 1] : 0.0f;
+    const float wm = wave_max(m);
+    if ((tid & 63) == 0) s_red[0][tid >> 6] = wm;
     __syncthreads();
     float m_all = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kD * kMergeGroups / kWave; ++w) m_all = fmaxf(m_all, s_max[w]);
+    for (int w = 0; w < kMergeThreads / kWave; ++w) m_all = fmaxf(m_all, s_red[0][w]);
+    const float f = m == -INFINITY ? 0.0f : exp2_fast(m - m_all);
+    if (mine) s_f[tid] = f;
+    const float wl = wave_sum(l * f);
+    if ((tid & 63) == 0) s_red[1][tid >> 6] = wl;
+    __syncthreads();
+    float l_all = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kMergeThreads / kWave; ++w) l_all += s_red[1][w];
 
-    float l = 0.0f, o = 0.0f;
-#pragma unroll 4
-    for (int p = grp; p < n_parts; p += kMergeGroups) {
-        const float mp = src[p * kPartFloats];
-        const float f = mp == -INFINITY ? 0.0f : exp2_fast(mp - m_all);
-        l += src[p * kPartFloats + 1] * f;
-        o += src[p * kPartFloats + 2 + d] * f;
+    float o = 0.0f;
+    for (int p0 = grp; p0 < n_parts; p0 += 8 * kMergeGroups) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + u * kMergeGroups;
+            v[u] = p < n_parts ? src[p * kPartFloats + d] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + u * kMergeGroups;
+            if (p < n_parts) o = fmaf(v[u], s_f[p], o);
+        }
     }
     s_o[grp][d] = o;
-    if (d == 0) s_l[grp] = l;
     __syncthreads();
     if (grp == 0) {
-        float lt = 0.0f, ot = 0.0f;
+        float total = 0.0f;
 #pragma unroll
-        for (int g = 0; g < kMergeGroups; ++g) { lt += s_l[g]; ot += s_o[g][d]; }
-        O[(size_t)head * kD + d] = to_half(lt > 0.0f ? ot / lt : 0.0f);
+        for (int g = 0; g < kMergeGroups; ++g) total += s_o[g][d];
+        O[(size_t)head * kD + d] = to_half(l_all > 0.0f ? total / l_all : 0.0f);
     }
 }
 
@@ -498,7 +515,7 @@ int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads, int
 size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim) {
     (void)n_kv_heads;
     if (n_q_heads <= 0 || head_dim <= 0) return 0;
-    return (size_t)n_q_heads * vv::kMaxParts * ((size_t)head_dim + 2) * sizeof(float);
+    return (size_t)n_q_heads * vv::kMaxParts * ((size_t)head_dim + 4) * sizeof(float);
 }
 
 int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len) {
@@ -563,7 +580,7 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
                                                      n_parts, scale_log2);
         if (n_parts > 1) {
             if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
-            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kD * vv::kMergeGroups, 0, st>>>(
+            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kMergeThreads, 0, st>>>(
                 static_cast<const float*>(scratch), O, n_parts);
         }
     } else {
