@@ -22,8 +22,8 @@
 //                           straight into 16x16x32 MFMA operands, K split
 //                           over the eight waves of a workgroup; bound by the
 //                           weight bytes.
-//   gemv_rows               M == 1 (a decode step): one wave per output
-//                           column streams that weight row once with
+//   gemv_row<kSplit>        M == 1 (a decode step): one to four waves per
+//                           output column stream that weight row once with
 //                           non-temporal 16-byte loads.
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
 #include "vv_common.hpp"
@@ -391,43 +391,47 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
                        vec_store);
 }
 
-// One wave per output column n; MR rows of A share each weight chunk.
-template <int MR>
-__global__ __launch_bounds__(kBlock) void gemv_rows(const h16* __restrict__ A,
-                                                    const h16* __restrict__ B,
-                                                    h16* __restrict__ C, int M, int N, int K,
-                                                    float alpha, float beta) {
-    const int n = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
-    if (n >= N) return;
-    const int lane = lane_id();
+// M == 1: bound by the weight bytes. kSplit waves share an output column (a
+// weight row), each streaming a contiguous 1/kSplit of it with non-temporal
+// 16-byte loads, four in flight; their sums meet in LDS. Narrow outputs take
+// more waves per row so that the chip always has thousands of waves in flight
+// (N = 3584, K = 18944: 26.4 us with one wave per row).
+template <int kSplit>
+__global__ __launch_bounds__(kBlock) void gemv_row(const h16* __restrict__ A,
+                                                   const h16* __restrict__ B,
+                                                   h16* __restrict__ C, int N, int K, float alpha,
+                                                   float beta) {
+    constexpr int kRows = kWavesPerBlock / kSplit;      // output columns per workgroup
+    __shared__ float part[kWavesPerBlock];
+    const int wave = wave_in_block(), lane = lane_id();
+    const int n = (int)blockIdx.x * kRows + wave / kSplit;
+    const int piece = wave % kSplit;
     const int kchunks = K / 8;
-    const Chunk* w = reinterpret_cast<const Chunk*>(B + (size_t)n * K);
-    float acc[MR];
-#pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+    const int per = (kchunks + kSplit - 1) / kSplit;
+    const int begin = piece * per, end = min(kchunks, begin + per);
+    float acc = 0.0f;
+    if (n < N) {
+        const Chunk* w = reinterpret_cast<const Chunk*>(B + (size_t)n * K);
+        const Chunk* x = reinterpret_cast<const Chunk*>(A);
 #pragma unroll 4
-    for (int c = lane; c < kchunks; c += kWave) {
-        const f32x8 wf = unpack(load_chunk_stream(w + c));
+        for (int c = begin + lane; c < end; c += kWave) {
+            const f32x8 wf = unpack(load_chunk_stream(w + c));
+            const f32x8 xf = unpack(load_chunk(x + c));
 #pragma unroll
-        for (int m = 0; m < MR; ++m) {
-            if (m < M) {
-                const f32x8 xf =
-                    unpack(load_chunk(reinterpret_cast<const Chunk*>(A + (size_t)m * K) + c));
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[m] = fmaf(xf[i], wf[i], acc[m]);
-            }
+            for (int i = 0; i < 8; ++i) acc = fmaf(xf[i], wf[i], acc);
         }
     }
-    float mine = 0.0f;
+    acc = wave_sum(acc);
+    if constexpr (kSplit > 1) {
+        if (lane == 0) part[wave] = acc;
+        __syncthreads();
+        acc = 0.0f;
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-        const float s = wave_sum(acc[m]);
-        if (lane == m) mine = s;
+        for (int p = 0; p < kSplit; ++p) acc += part[(wave / kSplit) * kSplit + p];
     }
-    if (lane < M && lane < MR) {
-        h16* c = C + (size_t)lane * N + n;
-        const h16 old = beta != 0.0f ? *c : (h16)0.0f;
-        *c = to_half(finish(mine, alpha, beta, old));
+    if (n < N && piece == 0 && lane == 0) {
+        const h16 old = beta != 0.0f ? C[n] : (h16)0.0f;
+        C[n] = to_half(finish(acc, alpha, beta, old));
     }
 }
 
@@ -633,8 +637,12 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         return launch_status();
     }
     if (allow_gemv && M == 1) {
-        const dim3 grid((unsigned)((N + kWavesPerBlock - 1) / kWavesPerBlock));
-        gemv_rows<1><<<grid, kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
+        if (N >= 16384)
+            gemv_row<1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
+        else if (N >= 8192)
+            gemv_row<2><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
+        else
+            gemv_row<4><<<dim3((unsigned)N), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
         return launch_status();
     }
     // Up to 64 rows: the weight-streaming kernel, unless there are more than 16
