@@ -288,7 +288,7 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
     return out
 
 
-def decode_token_leg(torch, dev, cache_len: int, layers: int = 28) -> dict:
+def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool = False) -> dict:
     """One decode step of a dense Qwen2-7B-shaped decoder (random weights, 13 GB of them) on this
     library's entry points alone, in the reference decoder's op order (decoder.c:706-991): per layer
     norm -> q/k/v GEMV -> bias + RoPE at a device-side position -> KV append at that position ->
@@ -328,7 +328,38 @@ def decode_token_leg(torch, dev, cache_len: int, layers: int = 28) -> dict:
     def gemv(x, wt, y, n, kk):
         assert dev.vv_gemm_fp16_dev(P(x), P(wt), P(y), 1, n, kk, 1.0, 0.0, st) == 0
 
+    act = torch.empty(1, I_FF, **f16)
+    qkv = []
+    for l in range(layers):
+        arr = (dev.SkinnyProj * 3)()
+        for i, (wt, b, y, n_) in enumerate(((wq, bq, q, QD), (wk, bk, k, KD), (wv, bv, v, KD))):
+            arr[i] = dev.SkinnyProj(w=P(wt[l]), scales=None, bias=P(b[l]), y=P(y), N=n_)
+        qkv.append(arr)
+
+    def token_fused():
+        """The same step on the fused additions: q/k/v with their biases in one launch, gate/up/SwiGLU in one."""
+        n = 1
+        assert dev.vv_rmsnorm_dev(P(hidden), P(n_in[0]), P(normed), 1, H, EPS, st) == 0
+        for l in range(layers):
+            assert dev.vv_gemv_multi_dev(P(normed), C.addressof(qkv[l]), 3, H, st) == 0
+            assert dev.vv_rope_qk_dev(P(q), P(k), 1, NQ, NK, HD, 0, P(pos), THETA, st) == 0
+            assert dev.vv_dev_memcpy_d2d_at(P(kc[l]), P(k), KD * 2, P(pos), st) == 0
+            assert dev.vv_dev_memcpy_d2d_at(P(vc[l]), P(v), KD * 2, P(pos), st) == 0
+            assert dev.vv_attn_decode(2, P(q), C.addressof(views[l]), P(attn), NQ, cache_len, P(nxt),
+                                      P(scratch), st) == 0
+            gemv(attn, wo[l], proj, H, QD)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_post[l]), P(normed), 1, H, EPS, st) == 0
+            assert dev.vv_gemv_swiglu_dev(P(normed), P(wg[l]), P(wu[l]), P(act), I_FF, H, st) == 0
+            gemv(act, wd[l], proj, H, I_FF)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_in[l + 1]), P(normed), 1, H, EPS, st) == 0
+            n += 11
+        assert dev.vv_pos_add_dev(P(pos), P(pos), 1, st) == 0
+        assert dev.vv_pos_add_dev(P(nxt), P(nxt), 1, st) == 0
+        return n + 2
+
     def token():
+        if fused:
+            return token_fused()
         n = 1
         assert dev.vv_rmsnorm_dev(P(hidden), P(n_in[0]), P(normed), 1, H, EPS, st) == 0
         for l in range(layers):
@@ -380,6 +411,7 @@ def decode_token_leg(torch, dev, cache_len: int, layers: int = 28) -> dict:
     dev.vv_dev_graph_destroy(g.value)
     dev.vv_dev_stream_destroy(st)
     return {"layers": layers, "cache_len": cache_len, "launches": launches, "weight_bytes": weight_bytes,
+            "entry_points": "fused additions" if fused else "reference API",
             "eager_ms": eager * 1e3, "graph_ms": replay * 1e3, "tokens_per_s": 1.0 / replay,
             "weight_GBps": weight_bytes / replay / 1e9,
             "frac_of_hbm_peak": weight_bytes / replay / 1e9 / HBM_PEAK_GBPS}
@@ -581,6 +613,10 @@ def main() -> int:
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         layer["decode_token"] = d = decode_token_leg(torch, dev, T)
         log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+        layer["decode_token_fused"] = d = decode_token_leg(torch, dev, T, fused=True)
+        log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
             f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
             f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
 

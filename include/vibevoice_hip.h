@@ -262,6 +262,21 @@ vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias,
                                 int n_kv_heads, int head_dim, int position_offset,
                                 const int* d_position, float theta, void* stream);
 
+/* addition: one activation row through up to three projections in ONE launch
+ * (the decode step's q/k/v): y_i[N_i] = x[K] . W_i^T (+ bias_i). Equals
+ * vv_gemm_fp16_dev(M = 1) followed by vv_bias_add_dev per projection bit for
+ * bit (src/inference/decoder.c:458-464 called three times). All N_i must fall
+ * in the same width class (below 8192, 8192..16383, or from 16384);
+ * otherwise, or when K % 8 != 0: VV_ERR_UNSUPPORTED, nothing launched. */
+vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int n_proj,
+                              int K, void* stream);
+
+/* addition: the decode step's MLP front half in one launch,
+ * y[N] = silu(x . Wg^T) * (x . Wu^T): equals two vv_gemm_fp16_dev(M = 1) and
+ * vv_swiglu_dev bit for bit (decoder.c:966-977) without writing gate and up. */
+vv_status_t vv_gemv_swiglu_dev(const void* x, const void* w_gate, const void* w_up,
+                               void* y, int N, int K, void* stream);
+
 /* addition: vv_embedding_dev(table, ids, hidden) followed by
  * vv_rmsnorm_dev(hidden, weight, normed): the first-layer chain
  * src/inference/pipeline.c:2309 -> decoder.c:810. hidden is bit-exact. */

@@ -167,4 +167,5 @@ def test_the_two_libraries_define_every_symbol_of_the_reference_seam():
     # beyond device.h: the fused entry points, and the two kv_quant.h symbols
     # (kv_quant.h:96-101) the decoder links against, declined
     assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
-                             "vv_embedding_rmsnorm_dev", "vv_kv_rotate_dev", "vv_kv_unrotate_dev"}
+                             "vv_embedding_rmsnorm_dev", "vv_gemv_multi_dev", "vv_gemv_swiglu_dev",
+                             "vv_kv_rotate_dev", "vv_kv_unrotate_dev"}

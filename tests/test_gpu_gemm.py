@@ -164,3 +164,64 @@ def test_skinny_linear_declines():
     assert dev.vv_skinny_linear_dev(d_a.data_ptr(), 1, C.addressof(arr), 1, M, K, 1.0, stream()) == U   # INT8 weights
     assert dev.vv_skinny_linear_dev(None, 0, C.addressof(arr), 1, M, K, 1.0, stream()) == dev.VV_ERR_NULL_PTR
     torch.cuda.synchronize()
+
+
+def gemv_multi(d_x, ws, biases, K):
+    import ctypes as C
+    outs = [torch.full((1, w.shape[0]), float("nan"), dtype=torch.float16, device="cuda") for w in ws]
+    arr = (dev.SkinnyProj * len(ws))()
+    for i, (w, b, y) in enumerate(zip(ws, biases, outs)):
+        arr[i] = dev.SkinnyProj(w=w.data_ptr(), scales=None, bias=b.data_ptr() if b is not None else None,
+                                y=y.data_ptr(), N=w.shape[0])
+    return dev.vv_gemv_multi_dev(d_x.data_ptr(), C.addressof(arr), len(ws), K, stream()), outs
+
+
+@pytest.mark.parametrize("Ns,K", [((3584, 512, 512), 3584), ((1536, 256, 256), 1536), ((18944, 18944), 3584),
+                                  ((9000,), 520), ((37, 5, 101), 72)])
+def test_gemv_multi_equals_gemv_then_bias(Ns, K):
+    """One decode row through several projections in one launch == the separate calls, bit for bit."""
+    d_x = to_dev(oracle.normal_f16((1, K), 61))
+    ws = [to_dev(oracle.normal_f16((n, K), 70 + i, std=K ** -0.5)) for i, n in enumerate(Ns)]
+    bs = [to_dev(oracle.normal_f16((n,), 80 + i, std=0.3)) if i != 1 else None for i, n in enumerate(Ns)]
+    st, outs = gemv_multi(d_x, ws, bs, K)
+    assert st == dev.VV_OK
+    for w, b, y in zip(ws, bs, outs):
+        n = w.shape[0]
+        want = torch.full((1, n), float("nan"), dtype=torch.float16, device="cuda")
+        ok(dev.vv_gemm_fp16_dev(d_x.data_ptr(), w.data_ptr(), want.data_ptr(), 1, n, K, 1.0, 0.0, stream()))
+        if b is not None:
+            ok(dev.vv_bias_add_dev(want.data_ptr(), b.data_ptr(), 1, n, stream()))
+        assert np.array_equal(bits_of(y), bits_of(want))
+    ref, mag = exact(bits_of(d_x), bits_of(ws[1 if len(ws) > 1 else 0]), None, 1.0, 0.0)     # the bias-free one
+    if len(ws) > 1:
+        check(bits_of(outs[1]), ref, mag, "gemv multi")
+
+
+@pytest.mark.parametrize("N,K", [(18944, 3584), (8960, 1536), (100, 64), (9000, 264), (3, 8)])
+def test_gemv_swiglu_equals_two_gemvs_and_swiglu(N, K):
+    d_x = to_dev(oracle.normal_f16((1, K), 91))
+    wg = to_dev(oracle.normal_f16((N, K), 92, std=2.0 * K ** -0.5))
+    wu = to_dev(oracle.normal_f16((N, K), 93, std=2.0 * K ** -0.5))
+    y = torch.full((1, N), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_gemv_swiglu_dev(d_x.data_ptr(), wg.data_ptr(), wu.data_ptr(), y.data_ptr(), N, K, stream()))
+    g = torch.empty((1, N), dtype=torch.float16, device="cuda")
+    u = torch.empty((1, N), dtype=torch.float16, device="cuda")
+    ok(dev.vv_gemm_fp16_dev(d_x.data_ptr(), wg.data_ptr(), g.data_ptr(), 1, N, K, 1.0, 0.0, stream()))
+    ok(dev.vv_gemm_fp16_dev(d_x.data_ptr(), wu.data_ptr(), u.data_ptr(), 1, N, K, 1.0, 0.0, stream()))
+    g_bits, u_bits = bits_of(g), bits_of(u)
+    ok(dev.vv_swiglu_dev(g.data_ptr(), u.data_ptr(), g.data_ptr(), N, stream()))
+    assert np.array_equal(bits_of(y), bits_of(g))
+    # and the oracle's SwiGLU of those FP16 projections
+    ref, rne = oracle.swiglu_f16(g_bits, u_bits)
+    assert scaled_rel_err(oracle.widen(bits_of(y)), ref) <= FP16_TOL
+
+
+def test_gemv_multi_declines():
+    K = 64
+    d_x = to_dev(oracle.normal_f16((1, K), 1))
+    narrow, wide = to_dev(oracle.normal_f16((128, K), 2)), to_dev(oracle.normal_f16((16384, K), 3))
+    assert gemv_multi(d_x, [narrow, wide], [None, None], K)[0] == dev.VV_ERR_UNSUPPORTED     # two width classes
+    assert gemv_multi(d_x, [narrow], [None], 60)[0] == dev.VV_ERR_UNSUPPORTED                 # K % 8
+    assert dev.vv_gemv_swiglu_dev(None, narrow.data_ptr(), narrow.data_ptr(), narrow.data_ptr(), 4, K,
+                                  stream()) == dev.VV_ERR_NULL_PTR
+    torch.cuda.synchronize()

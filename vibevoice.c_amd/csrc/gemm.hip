@@ -26,7 +26,7 @@
 //                           output column stream that weight row once with
 //                           non-temporal 16-byte loads.
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
-#include "vv_common.hpp"
+#include "row_math.hpp"
 
 namespace vv {
 namespace {
@@ -435,6 +435,79 @@ __global__ __launch_bounds__(kBlock) void gemv_row(const h16* __restrict__ A,
     }
 }
 
+// One row of the decode step through two or three projections in one launch.
+// kFuse == 0: y_i = x W_i^T (+ bias_i) for up to three projections (q/k/v);
+// workgroups [first[p], first[p+1]) serve projection p. kFuse == 1: the MLP's
+// gate and up projections and its activation, y = silu(x Wg^T) * (x Wu^T), a
+// wave group taking the same row of both matrices. Either way every product is
+// summed exactly as gemv_row<kSplit> sums it and rounded to FP16 before the
+// bias or the activation is applied, so the result equals the separate launches
+// bit for bit.
+struct GemvProjs {
+    const h16* w[3];
+    const h16* bias[3];
+    h16* y[3];
+    int n[3];
+    int first[3];
+};
+
+template <int kSplit, int kFuse>
+__global__ __launch_bounds__(kBlock) void gemv_multi(const h16* __restrict__ A, GemvProjs projs,
+                                                     int K) {
+    constexpr int kRows = kWavesPerBlock / kSplit;
+    __shared__ float part[2][kWavesPerBlock];
+    const int wave = wave_in_block(), lane = lane_id();
+    const int which = kFuse ? 0 : ((int)blockIdx.x >= projs.first[1]) + ((int)blockIdx.x >= projs.first[2]);
+    const int N = projs.n[which];
+    const int n = ((int)blockIdx.x - projs.first[which]) * kRows + wave / kSplit;
+    const int piece = wave % kSplit;
+    const int kchunks = K / 8;
+    const int per = (kchunks + kSplit - 1) / kSplit;
+    const int begin = piece * per, end = min(kchunks, begin + per);
+    float acc = 0.0f, acc2 = 0.0f;
+    if (n < N) {
+        const Chunk* w = reinterpret_cast<const Chunk*>(projs.w[which] + (size_t)n * K);
+        const Chunk* w2 = reinterpret_cast<const Chunk*>(projs.w[1] + (size_t)n * K);
+        const Chunk* x = reinterpret_cast<const Chunk*>(A);
+#pragma unroll 4
+        for (int c = begin + lane; c < end; c += kWave) {
+            const f32x8 wf = unpack(load_chunk_stream(w + c));
+            const f32x8 xf = unpack(load_chunk(x + c));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = fmaf(xf[i], wf[i], acc);
+            if constexpr (kFuse) {
+                const f32x8 uf = unpack(load_chunk_stream(w2 + c));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc2 = fmaf(xf[i], uf[i], acc2);
+            }
+        }
+    }
+    acc = wave_sum(acc);
+    if constexpr (kFuse) acc2 = wave_sum(acc2);
+    if constexpr (kSplit > 1) {
+        if (lane == 0) { part[0][wave] = acc; part[1][wave] = acc2; }
+        __syncthreads();
+        acc = acc2 = 0.0f;
+#pragma unroll
+        for (int p = 0; p < kSplit; ++p) {
+            acc += part[0][(wave / kSplit) * kSplit + p];
+            acc2 += part[1][(wave / kSplit) * kSplit + p];
+        }
+    }
+    if (n < N && piece == 0 && lane == 0) {
+        h16 o = to_half(acc);
+        if constexpr (kFuse) {
+            o = to_half(swiglu1((float)o, (float)to_half(acc2)));
+        } else if (projs.bias[which]) {
+            o = to_half((float)o + (float)projs.bias[which][n]);
+        }
+        projs.y[which][n] = o;
+    }
+}
+
+// The waves per weight row vv_gemm_fp16_dev gives a one-row product of width N.
+inline int gemv_split(int N) { return N >= 16384 ? 1 : N >= 8192 ? 2 : 4; }
+
 // M <= 64 (a streaming chunk, a few decode rows): bound by the weight bytes, so
 // the weights are read exactly once, straight from global memory into MFMA
 // operands, and K is split over the eight waves of a workgroup.
@@ -637,12 +710,11 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         return launch_status();
     }
     if (allow_gemv && M == 1) {
-        if (N >= 16384)
-            gemv_row<1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
-        else if (N >= 8192)
-            gemv_row<2><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
-        else
-            gemv_row<4><<<dim3((unsigned)N), kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
+        const int split = gemv_split(N);
+        const dim3 grid((unsigned)((N + kWavesPerBlock / split - 1) / (kWavesPerBlock / split)));
+        if (split == 1) gemv_row<1><<<grid, kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
+        else if (split == 2) gemv_row<2><<<grid, kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
+        else gemv_row<4><<<grid, kBlock, 0, st>>>(a, b, c, N, K, alpha, beta);
         return launch_status();
     }
     // Up to 64 rows: the weight-streaming kernel, unless there are more than 16
@@ -723,6 +795,58 @@ vv_status_t vv_skinny_linear_dev(const void* A, int format, const vv_skinny_proj
         blocks += (projs[i].N + 15) / 16;
     }
     vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, alpha, 0.0f, vv::as_stream(stream));
+    return vv::launch_status();
+}
+
+vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int n_proj, int K,
+                              void* stream) {
+    if (!x || !projs) return VV_ERR_NULL_PTR;
+    if (n_proj < 1 || n_proj > 3 || K <= 0 || K % 8 != 0 || !vv::aligned16(x)) return VV_ERR_UNSUPPORTED;
+    vv::GemvProjs p = {};
+    const int split = vv::gemv_split(projs[0].N);
+    const int rows = vv::kWavesPerBlock / split;
+    int blocks = 0;
+    for (int i = 0; i < 3; ++i) {
+        p.first[i] = blocks;
+        if (i >= n_proj) continue;
+        if (!projs[i].w || !projs[i].y) return VV_ERR_NULL_PTR;
+        if (projs[i].N <= 0 || vv::gemv_split(projs[i].N) != split || !vv::aligned16(projs[i].w))
+            return VV_ERR_UNSUPPORTED;
+        p.w[i] = static_cast<const vv::h16*>(projs[i].w);
+        p.bias[i] = static_cast<const vv::h16*>(projs[i].bias);
+        p.y[i] = static_cast<vv::h16*>(projs[i].y);
+        p.n[i] = projs[i].N;
+        blocks += (projs[i].N + rows - 1) / rows;
+    }
+    for (int i = n_proj; i < 3; ++i) p.w[i] = p.w[0];
+    const vv::h16* a = static_cast<const vv::h16*>(x);
+    hipStream_t st = vv::as_stream(stream);
+    if (split == 1) vv::gemv_multi<1, 0><<<dim3((unsigned)blocks), vv::kBlock, 0, st>>>(a, p, K);
+    else if (split == 2) vv::gemv_multi<2, 0><<<dim3((unsigned)blocks), vv::kBlock, 0, st>>>(a, p, K);
+    else vv::gemv_multi<4, 0><<<dim3((unsigned)blocks), vv::kBlock, 0, st>>>(a, p, K);
+    return vv::launch_status();
+}
+
+vv_status_t vv_gemv_swiglu_dev(const void* x, const void* w_gate, const void* w_up, void* y, int N,
+                               int K, void* stream) {
+    if (!x || !w_gate || !w_up || !y) return VV_ERR_NULL_PTR;
+    if (N <= 0) return VV_OK;
+    if (K <= 0 || K % 8 != 0 || !vv::aligned16(x) || !vv::aligned16(w_gate) || !vv::aligned16(w_up))
+        return VV_ERR_UNSUPPORTED;
+    vv::GemvProjs p = {};
+    p.w[0] = static_cast<const vv::h16*>(w_gate);
+    p.w[1] = p.w[2] = static_cast<const vv::h16*>(w_up);
+    p.y[0] = static_cast<vv::h16*>(y);
+    p.n[0] = N;
+    const int split = vv::gemv_split(N);
+    const int rows = vv::kWavesPerBlock / split;
+    const dim3 grid((unsigned)((N + rows - 1) / rows));
+    p.first[1] = p.first[2] = (int)grid.x;
+    const vv::h16* a = static_cast<const vv::h16*>(x);
+    hipStream_t st = vv::as_stream(stream);
+    if (split == 1) vv::gemv_multi<1, 1><<<grid, vv::kBlock, 0, st>>>(a, p, K);
+    else if (split == 2) vv::gemv_multi<2, 1><<<grid, vv::kBlock, 0, st>>>(a, p, K);
+    else vv::gemv_multi<4, 1><<<grid, vv::kBlock, 0, st>>>(a, p, K);
     return vv::launch_status();
 }
 

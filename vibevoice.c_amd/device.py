@@ -66,6 +66,8 @@ SIGNATURES = {
     "vv_lm_head_gemv_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "vv_argmax_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
+    "vv_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vv_gemv_swiglu_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
