@@ -288,6 +288,64 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
     return out
 
 
+def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
+    """One dense decoder layer over the whole T-row prompt, in the reference decoder's op order
+    (decoder.c:706-991) on this library's entry points: norm, q/k/v GEMMs, bias + RoPE, causal
+    attention over the chunk's own K/V, o GEMM, add+norm, gate/up GEMMs, SwiGLU, down GEMM, add+norm.
+    Random weights. Reports the layer time and what 28 such layers make in prompt tokens per second."""
+    import ctypes as C
+    f16 = dict(dtype=torch.float16, device="cuda")
+    QD, KD = NQ * HD, NK * HD
+    w = lambda *shape, std: torch.randn(*shape, **f16) * std
+    wq, wk, wv, wo = w(QD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(H, QD, std=QD ** -0.5)
+    wg, wu, wd = w(I_FF, H, std=H ** -0.5), w(I_FF, H, std=H ** -0.5), w(H, I_FF, std=I_FF ** -0.5)
+    bq, bk, bv = w(QD, std=0.1), w(KD, std=0.1), w(KD, std=0.1)
+    n1, n2 = 1 + w(H, std=0.1), 1 + w(H, std=0.1)
+    hidden, normed, proj = w(T, H, std=1.0), torch.empty(T, H, **f16), torch.empty(T, H, **f16)
+    q, attn = torch.empty(T, QD, **f16), torch.empty(T, QD, **f16)
+    k, v = torch.empty(T, KD, **f16), torch.empty(T, KD, **f16)
+    gate, up = torch.empty(T, I_FF, **f16), torch.empty(T, I_FF, **f16)
+    view = dev.KvView(k=k.data_ptr(), v=v.data_ptr(), k_meta=None, v_meta=None, page_table=None, format=0,
+                      n_kv_heads=NK, head_dim=HD)
+    P = lambda t: t.data_ptr()
+
+    def gemm(x, wt, y, n, kk):
+        assert dev.vv_gemm_fp16_dev(P(x), P(wt), P(y), T, n, kk, 1.0, 0.0, st) == 0
+
+    def layer():
+        assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0
+        gemm(normed, wq, q, QD, H)
+        gemm(normed, wk, k, KD, H)
+        gemm(normed, wv, v, KD, H)
+        assert dev.vv_bias_rope_qk_dev(P(q), P(k), P(bq), P(bk), T, NQ, NK, HD, 0, None, THETA, st) == 0
+        assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
+        assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, T, 0, T, True, None, st) == 0
+        gemm(attn, wo, proj, H, QD)
+        assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n2), P(normed), T, H, EPS, st) == 0
+        gemm(normed, wg, gate, I_FF, H)
+        gemm(normed, wu, up, I_FF, H)
+        assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), T * I_FF, st) == 0
+        gemm(gate, wd, proj, H, I_FF)
+        assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
+
+    layer()
+    torch.cuda.synchronize()
+    per = []
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        layer()
+        e1.record()
+        e1.synchronize()
+        per.append(e0.elapsed_time(e1))
+    per.sort()
+    ms = per[1]
+    assert bool(torch.isfinite(hidden).all())
+    flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
+    return {"rows": T, "ms_per_layer": ms, "TFLOPs": flops / ms / 1e9, "layers_assumed": 28,
+            "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
+
+
 def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool = False) -> dict:
     """One decode step of a dense Qwen2-7B-shaped decoder (random weights, 13 GB of them) on this
     library's entry points alone, in the reference decoder's op order (decoder.c:706-991): per layer
@@ -611,6 +669,9 @@ def main() -> int:
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         d = layer["attn_decode"]
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
+        log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention); "
+            f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
         layer["decode_token"] = d = decode_token_leg(torch, dev, T)
         log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
             f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
