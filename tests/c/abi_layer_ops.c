@@ -13,6 +13,8 @@
  *     M in {1, 7, 285}                                 (test_int8_linear.c:295-354 shapes)
  *   - embedding gather, bit-exact
  *   - capture once, replay many                        (test_device_memory.c:164-212)
+ *   - a linear layer (GEMM + bias, one row and a chunk), the multi-projection small-M form,
+ *     causal attention (prefill, then a decode row on the same cache) and the greedy head
  * The CPU side is the oracle library (test infrastructure, never shipped).
  */
 #include <math.h>
@@ -240,6 +242,96 @@ static void test_graph(void) {
     vv_dev_free(pos); vv_dev_free(rows); vv_dev_free(row);
 }
 
+static uint16_t* rand_f16(size_t n, float scale) {
+    uint16_t* h = (uint16_t*)malloc(n * 2);
+    for (size_t i = 0; i < n; i++) h[i] = vvo_float_to_half_rne(scale * frand());
+    return h;
+}
+
+static float* widen(const uint16_t* h, size_t n) {
+    float* f = (float*)malloc(n * sizeof(float));
+    for (size_t i = 0; i < n; i++) f[i] = vvo_half_to_float(h[i]);
+    return f;
+}
+
+static void test_linear_attention_head(void* st) {
+    printf("linear layers, attention, greedy head:\n");
+    enum { K = 512, N = 384, NQ = 4, NKV = 2, HD = 128, T = 40, V = 1000 };
+    uint16_t* w = rand_f16((size_t)N * K, 0.08f);
+    uint16_t* bias = rand_f16(N, 0.3f);
+    void *d_w = to_dev(w, (size_t)N * K * 2), *d_b = to_dev(bias, N * 2);
+    const int rows[3] = {1, 29, 200};
+    for (int c = 0; c < 3; c++) {
+        const int M = rows[c];
+        uint16_t* x = rand_f16((size_t)M * K, 1.0f);
+        float* xf = widen(x, (size_t)M * K);
+        float* ref = (float*)malloc((size_t)M * N * sizeof(float));
+        vvo_gemm_f16w(xf, w, bias, ref, M, N, K);
+        void *d_x = to_dev(x, (size_t)M * K * 2), *d_y = to_dev(NULL, (size_t)M * N * 2);
+        vv_status_t s = vv_gemm_fp16_dev(d_x, d_w, d_y, M, N, K, 1.0f, 0.0f, st);
+        if (s == VV_OK) s = vv_bias_add_dev(d_y, d_b, M, N, st);
+        uint16_t* y = (uint16_t*)malloc((size_t)M * N * 2);
+        vv_dev_memcpy_d2h(y, d_y, (size_t)M * N * 2, st);
+        vv_dev_stream_sync(st);
+        char what[96];
+        snprintf(what, sizeof what, "GEMM + bias, M=%d: scaled error %.2e", M, scaled_err(y, ref, (size_t)M * N));
+        check(s == VV_OK && scaled_err(y, ref, (size_t)M * N) <= 2e-3, what);
+        if (M == 29) {      /* the reference's small-M entry point: one launch, the same bits */
+            void* d_y2 = to_dev(NULL, (size_t)M * N * 2);
+            vv_skinny_proj_t p = {d_w, NULL, d_b, d_y2, N};
+            s = vv_skinny_linear_dev(d_x, 0, &p, 1, M, K, 1.0f, st);
+            uint16_t* y2 = (uint16_t*)malloc((size_t)M * N * 2);
+            vv_dev_memcpy_d2h(y2, d_y2, (size_t)M * N * 2, st);
+            vv_dev_stream_sync(st);
+            check(s == VV_OK && memcmp(y, y2, (size_t)M * N * 2) == 0, "vv_skinny_linear_dev == GEMM + bias add, bit for bit");
+            free(y2); vv_dev_free(d_y2);
+        }
+        free(x); free(xf); free(ref); free(y); vv_dev_free(d_x); vv_dev_free(d_y);
+    }
+
+    /* attention: T rows over their own K/V, then one more row as a decode step on the same cache */
+    uint16_t *q = rand_f16((size_t)(T + 1) * NQ * HD, 1.5f), *k = rand_f16((size_t)(T + 1) * NKV * HD, 1.0f),
+             *v = rand_f16((size_t)(T + 1) * NKV * HD, 1.0f);
+    float *qf = widen(q, (size_t)(T + 1) * NQ * HD), *kf = widen(k, (size_t)(T + 1) * NKV * HD),
+          *vf = widen(v, (size_t)(T + 1) * NKV * HD);
+    float* aref = (float*)malloc((size_t)(T + 1) * NQ * HD * sizeof(float));
+    vvo_attention_prefill_f32(qf, kf, vf, aref, NQ, NKV, HD, T + 1, 0, T + 1, 1);
+    void *d_q = to_dev(q, (size_t)(T + 1) * NQ * HD * 2), *d_k = to_dev(k, (size_t)(T + 1) * NKV * HD * 2),
+         *d_v = to_dev(v, (size_t)(T + 1) * NKV * HD * 2), *d_o = to_dev(NULL, (size_t)(T + 1) * NQ * HD * 2);
+    const vv_kv_view_t view = {d_k, d_v, NULL, NULL, NULL, 0, NKV, HD};
+    const int backend = vv_attn_resolve(0, 0, false, NQ, NKV, HD);
+    void* scratch = to_dev(NULL, vv_attn_scratch_bytes(NQ, NKV, HD));
+    vv_status_t s = vv_attn_prefill(backend, d_q, &view, d_o, NQ, T, 0, T, true, scratch, st);
+    if (s == VV_OK)
+        s = vv_attn_decode(backend, (char*)d_q + (size_t)T * NQ * HD * 2, &view, (char*)d_o + (size_t)T * NQ * HD * 2,
+                           NQ, T + 1, NULL, scratch, st);
+    uint16_t* o = (uint16_t*)malloc((size_t)(T + 1) * NQ * HD * 2);
+    vv_dev_memcpy_d2h(o, d_o, (size_t)(T + 1) * NQ * HD * 2, st);
+    vv_dev_stream_sync(st);
+    check(backend != 0 && s == VV_OK && scaled_err(o, aref, (size_t)T * NQ * HD) <= 2e-3, "causal prefill attention");
+    check(scaled_err(o + (size_t)T * NQ * HD, aref + (size_t)T * NQ * HD, (size_t)NQ * HD) <= 2e-3,
+          "decode attention on the same cache");
+
+    /* greedy head: logits in FP32, the token the in-order scan picks from them */
+    uint16_t *table = rand_f16((size_t)V * K, 0.05f), *h = rand_f16(K, 1.0f);
+    void *d_t = to_dev(table, (size_t)V * K * 2), *d_h = to_dev(h, K * 2), *d_l = to_dev(NULL, V * 4),
+         *d_sv = to_dev(NULL, 256 * 4), *d_si = to_dev(NULL, 256 * 4);
+    int* d_tok = dev_int(-1);
+    s = vv_lm_head_gemv_dev(d_h, d_t, d_l, V, K, st);
+    if (s == VV_OK) s = vv_argmax_dev(d_l, V, d_sv, d_si, d_tok, NULL, st);
+    float* logits = (float*)malloc(V * sizeof(float));
+    vv_dev_memcpy_d2h(logits, d_l, V * 4, st);
+    vv_dev_stream_sync(st);
+    int32_t want = -2;
+    vvo_argmax_first(logits, V, &want, NULL);
+    check(s == VV_OK && read_dev_int(d_tok) == want, "LM head + on-device argmax");
+
+    free(w); free(bias); free(q); free(k); free(v); free(qf); free(kf); free(vf); free(aref); free(o);
+    free(table); free(h); free(logits);
+    void* frees[] = {d_w, d_b, d_q, d_k, d_v, d_o, scratch, d_t, d_h, d_l, d_sv, d_si, d_tok};
+    for (size_t i = 0; i < sizeof frees / sizeof frees[0]; i++) vv_dev_free(frees[i]);
+}
+
 int main(void) {
     if (vv_dev_device_count() <= 0) {
         printf("SKIP: no device available\n");
@@ -261,6 +353,7 @@ int main(void) {
     test_norm_and_swiglu_shapes(st);
     test_embedding(st);
     test_graph();
+    test_linear_attention_head(st);
     vv_dev_stream_destroy(st);
 
     if (failures) {
