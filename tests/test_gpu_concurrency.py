@@ -67,3 +67,59 @@ def test_four_threads_four_streams():
         want_r, nref, nrne = oracle.add_rmsnorm_f16(r, h, w, 1e-6)
         assert np.array_equal(gr, want_r), f"thread {idx} residual"
         assert_fp16_close(gn, nref, nrne, f"thread {idx} add+norm")
+
+
+def test_threads_run_the_matrix_core_kernels_at_once():
+    """Four threads, four streams: the large-tile GEMM (its one-time LDS-size
+    attribute is set per thread), the small-M form, a one-row GEMV and prefill
+    + decode attention with a scratch of their own. Each thread's results must
+    equal what the same calls give alone on the default stream."""
+    M_BIG, N, K, NQ, NKV, HD, T = 4100, 8192, 256, 4, 2, 128, 300
+    a = to_dev(oracle.normal_f16((M_BIG, K), 1))
+    w = to_dev(oracle.normal_f16((N, K), 2, std=K ** -0.5))
+    q = to_dev(oracle.normal_f16((T, NQ, HD), 3))
+    k = to_dev(oracle.normal_f16((T, NKV, HD), 4))
+    v = to_dev(oracle.normal_f16((T, NKV, HD), 5))
+    view = dev.KvView(k=k.data_ptr(), v=v.data_ptr(), k_meta=None, v_meta=None, page_table=None, format=0,
+                      n_kv_heads=NKV, head_dim=HD)
+
+    def run(st):
+        f16 = dict(dtype=torch.float16, device="cuda")
+        outs = [torch.zeros(M_BIG, N, **f16), torch.zeros(29, N, **f16), torch.zeros(1, N, **f16),
+                torch.zeros(T, NQ, HD, **f16), torch.zeros(1, NQ, HD, **f16)]
+        scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NKV, HD), dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        for m, o in zip((M_BIG, 29, 1), outs[:3]):
+            assert dev.vv_gemm_fp16_dev(a.data_ptr(), w.data_ptr(), o.data_ptr(), m, N, K, 1.0, 0.0, st) == 0
+        assert dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view), outs[3].data_ptr(), NQ, T, 0, T, True,
+                                   None, st) == 0
+        assert dev.vv_attn_decode(2, q.data_ptr() + (T - 1) * NQ * HD * 2, C.addressof(view), outs[4].data_ptr(),
+                                  NQ, T, None, scratch.data_ptr(), st) == 0
+        assert dev.vv_dev_stream_sync(st) == 0
+        return [o.cpu().numpy().view(np.uint16) for o in outs]
+
+    want = run(None)
+    errors, results = [], {}
+    barrier = threading.Barrier(4)
+
+    def work(idx):
+        try:
+            torch.cuda.set_device(0)
+            st = C.c_void_p()
+            assert dev.vv_dev_stream_create(C.byref(st)) == 0
+            barrier.wait()
+            for _ in range(5):
+                results[idx] = run(st.value)
+            dev.vv_dev_stream_destroy(st.value)
+        except Exception as e:                         # noqa: BLE001
+            errors.append((idx, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for idx in range(4):
+        for got, ref in zip(results[idx], want):
+            assert np.array_equal(got, ref), f"thread {idx}"

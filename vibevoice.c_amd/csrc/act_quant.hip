@@ -295,7 +295,8 @@ template <int kSrc>
 vv_status_t launch_quant(const void* a, const void* b, int M, int K, float eps, int layout,
                          int8_t* xq, float* sx, int32_t* xsum, hipStream_t st) {
     const int nchunks = K / 8;
-    if (kSrc == kQNorm && nchunks <= 8 * kWave && !getenv("VV_Q8_LIGHT_NORM")) {
+    static const bool light_norm = getenv("VV_Q8_LIGHT_NORM") != nullptr;   // A/B switch, read once
+    if (kSrc == kQNorm && nchunks <= 8 * kWave && !light_norm) {
         const float inv_k = 1.0f / (float)K;
         const bool nt = use_streaming((size_t)M * (size_t)K * 3u);
         const dim3 g((unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock));
