@@ -338,28 +338,46 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     const int fa_base = wm * TM * 32 * kSlabChunks;
     const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
 
-    // Fragment reads run one MFMA group ahead: while the 8 MFMAs of a K step
-    // execute, the operands of the next step (the next slab's first step, after
-    // the barrier) come in from LDS.
-    h16x8 fw[2][TN], fx[2][TM];
+    // Fragment reads run a whole slab ahead: while the 16 MFMAs of slab s execute
+    // from one register set, the operands of slab s + 1 come in from LDS into the
+    // other (an LDS queue that is two thirds busy answers too late for anything
+    // shorter).
+    h16x8 fw[2][2][TN], fx[2][2][TM];          // [set][K step][tile]
     auto read_frags = [&](auto set_c, int slab, int step) {
         constexpr int set = decltype(set_c)::value;
         const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
 #pragma unroll
         for (int a = 0; a < TN; ++a)
-            fw[set][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
+            fw[set][step][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
 #pragma unroll
         for (int b = 0; b < TM; ++b)
-            fx[set][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
+            fx[set][step][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
     };
-    auto mfma_group = [&](auto set_c) {
+    auto mfma_group = [&](auto set_c, int step) {
         constexpr int set = decltype(set_c)::value;
 #pragma unroll
         for (int a = 0; a < TN; ++a)
 #pragma unroll
             for (int b = 0; b < TM; ++b)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[set][a], fx[set][b], acc[a][b],
-                                                                   0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[set][step][a], fx[set][step][b],
+                                                                   acc[a][b], 0, 0, 0);
+    };
+    // One slab: its operands are (being) loaded in set `cur`; slab + 1 must be in
+    // LDS (this wave's copies of slabs + 2 and + 3, 8 of them, may still fly) and
+    // every wave must have its operands of this slab in registers before the
+    // stage is handed to slab + 4.
+    auto one_slab = [&](auto cur_c, auto nxt_c, int slab) {
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        request(slab + 4);
+        read_frags(nxt_c, slab + 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(cur_c, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(nxt_c, slab + 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(cur_c, 1);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     request(0);
@@ -369,22 +387,13 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     __syncthreads();
     read_frags(Const<0>{}, 0, 0);
-    for (int slab = 0; slab < nslabs; ++slab) {
-        read_frags(Const<1>{}, slab, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_group(Const<0>{});
-        __builtin_amdgcn_sched_barrier(0);
-        // Slab + 1 must be in LDS (this wave's copies of slabs + 2 and + 3, 8 of
-        // them, may still fly), and every wave must be done reading this slab
-        // before its stage is handed to slab + 4.
-        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-        request(slab + 4);
-        read_frags(Const<0>{}, slab + 1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_group(Const<1>{});
-        __builtin_amdgcn_sched_barrier(0);
+    read_frags(Const<0>{}, 0, 1);
+    int slab = 0;
+    for (; slab + 2 <= nslabs; slab += 2) {
+        one_slab(Const<0>{}, Const<1>{}, slab);
+        one_slab(Const<1>{}, Const<0>{}, slab + 1);
     }
+    if (slab < nslabs) one_slab(Const<0>{}, Const<1>{}, slab);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
 
     store_tile<TM, TN>(acc, C, M, N, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf, alpha, beta,
