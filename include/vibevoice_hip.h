@@ -204,6 +204,25 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv,
 vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv,
                            void* out, int n_q_heads, int cache_len,
                            const int* d_cache_len, void* scratch, void* stream);
+/* The older entry points for raw FP16 caches: the cache as two pointers
+ * instead of a view, otherwise vv_attn_scratch_bytes, vv_attn_decode_shape,
+ * vv_attn_decode and vv_attn_prefill. replace device.h:621-655. */
+size_t vv_gqa_decode_scratch_bytes(int n_q_heads, int head_dim);
+int vv_gqa_decode_shape(int cache_len);
+vv_status_t vv_gqa_attention_decode_dev(const void* q, const void* k_cache,
+                                        const void* v_cache, void* output,
+                                        int n_q_heads, int n_kv_heads, int head_dim,
+                                        int cache_len, const int* d_cache_len,
+                                        void* scratch, void* stream);
+vv_status_t vv_gqa_attention_prefill_cached_dev(const void* q, const void* k_cache,
+                                                const void* v_cache, void* output,
+                                                int n_q_heads, int n_kv_heads,
+                                                int head_dim, int q_len, int q_offset,
+                                                int kv_len, bool causal, void* stream);
+vv_status_t vv_gqa_attention_prefill_dev(const void* q, const void* k, const void* v,
+                                         void* output, int n_q_heads, int n_kv_heads,
+                                         int head_dim, int seq_len, bool causal,
+                                         void* stream);
 /* Copy K/V rows [n_positions][n_kv_heads][head_dim] into an FP16 cache layer
  * at positions pos.. (or *d_pos..), through page_table when it is set.
  * Other formats: VV_ERR_UNSUPPORTED. replaces device.h:597-602. */

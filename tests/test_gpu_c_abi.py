@@ -61,3 +61,21 @@ def test_reference_layer_runner_passes_on_this_backend():
     for line in ("GPU: same hidden states", "GPU and CPU agree", "OK (0 failures)"):
         assert line in res.stdout
     assert "FAIL" not in res.stdout
+
+
+ATTN_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_attention_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(ATTN_EXE),
+                    reason="oracle/_ref/test_attention_hip not built (needs the reference tree)")
+def test_reference_own_attention_test_passes_on_this_backend():
+    """The reference's tests/test_attention.c, unmodified: prefill attention at
+    28 query / 4 KV heads of 128 against its FP64 reference, at lengths on and
+    off every tile boundary, with and without the chunked-prefill offset
+    (bars: max |err| < 4e-3, cosine > 0.9999), then its timing loop."""
+    res = subprocess.run([ATTN_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-5000:], res.stderr[-1000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert res.stdout.count("  ok  ") >= 8

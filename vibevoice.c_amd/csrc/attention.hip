@@ -593,6 +593,40 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
     return vv::launch_status();
 }
 
+/* The older entry points for raw FP16 caches (device.h:621-655): the same
+ * kernels, the cache given as two pointers instead of a view. */
+size_t vv_gqa_decode_scratch_bytes(int n_q_heads, int head_dim) {
+    return vv_attn_scratch_bytes(n_q_heads, 1, head_dim);
+}
+
+int vv_gqa_decode_shape(int cache_len) { return vv::decode_parts(cache_len); }
+
+vv_status_t vv_gqa_attention_decode_dev(const void* q, const void* k_cache, const void* v_cache,
+                                        void* output, int n_q_heads, int n_kv_heads, int head_dim,
+                                        int cache_len, const int* d_cache_len, void* scratch,
+                                        void* stream) {
+    const vv_kv_view_t view = {k_cache, v_cache, nullptr, nullptr, nullptr, vv::kFormatFp16, n_kv_heads,
+                               head_dim};
+    return vv_attn_decode(2, q, &view, output, n_q_heads, cache_len, d_cache_len, scratch, stream);
+}
+
+vv_status_t vv_gqa_attention_prefill_cached_dev(const void* q, const void* k_cache, const void* v_cache,
+                                                void* output, int n_q_heads, int n_kv_heads,
+                                                int head_dim, int q_len, int q_offset, int kv_len,
+                                                bool causal, void* stream) {
+    const vv_kv_view_t view = {k_cache, v_cache, nullptr, nullptr, nullptr, vv::kFormatFp16, n_kv_heads,
+                               head_dim};
+    return vv_attn_prefill(2, q, &view, output, n_q_heads, q_len, q_offset, kv_len, causal, nullptr,
+                           stream);
+}
+
+vv_status_t vv_gqa_attention_prefill_dev(const void* q, const void* k, const void* v, void* output,
+                                         int n_q_heads, int n_kv_heads, int head_dim, int seq_len,
+                                         bool causal, void* stream) {
+    return vv_gqa_attention_prefill_cached_dev(q, k, v, output, n_q_heads, n_kv_heads, head_dim, seq_len,
+                                               0, seq_len, causal, stream);
+}
+
 vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_store, void* v_store,
                             void* k_meta, void* v_meta, void* k_ref, bool build_ref,
                             int n_kv_heads, int head_dim, int pos, const int* d_pos,

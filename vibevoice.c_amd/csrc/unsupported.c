@@ -44,12 +44,9 @@ VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)   VV_DECLINE(vv_
 VV_DECLINE(vv_gemm_fp16_nn_dev)
 void vv_gemm_cleanup() {}
 
-/* the older per-format attention entry points and the quantised KV formats
- * (device.h:619-700, kv_quant.h:96-101); vv_attn_* on FP16 caches is implemented */
-VV_ZERO_SIZE(vv_gqa_decode_scratch_bytes) VV_ZERO_INT(vv_gqa_decode_shape)
-VV_DECLINE(vv_gqa_attention_decode_dev)   VV_DECLINE(vv_gqa_attention_prefill_cached_dev)
-VV_DECLINE(vv_gqa_attention_prefill_dev)  VV_DECLINE(vv_gqa_attention_decode_q_dev)
-VV_DECLINE(vv_gqa_attention_prefill_q_dev)
+/* attention over quantised KV formats and their store / unpack / rotations
+ * (device.h:657-700, kv_quant.h:96-101); every FP16-cache entry point is implemented */
+VV_DECLINE(vv_gqa_attention_decode_q_dev) VV_DECLINE(vv_gqa_attention_prefill_q_dev)
 VV_DECLINE(vv_kv_quant_store_dev) VV_DECLINE(vv_kv_dequant_dev)
 VV_DECLINE(vv_kv_rotate_dev)      VV_DECLINE(vv_kv_unrotate_dev)
 

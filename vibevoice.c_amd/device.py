@@ -68,6 +68,11 @@ SIGNATURES = {
     "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
     "vv_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _vp]),
     "vv_gemv_swiglu_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "vv_gqa_decode_scratch_bytes": (C.c_size_t, [_i, _i]),
+    "vv_gqa_decode_shape": (_i, [_i]),
+    "vv_gqa_attention_decode_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "vv_gqa_attention_prefill_cached_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, C.c_bool, _vp]),
+    "vv_gqa_attention_prefill_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_bool, _vp]),
     "vv_add_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_rope_qk_dev": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
