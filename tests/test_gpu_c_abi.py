@@ -79,3 +79,19 @@ def test_reference_own_attention_test_passes_on_this_backend():
     assert res.returncode == 0, res.stdout[-3000:]
     assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
     assert res.stdout.count("  ok  ") >= 8
+
+
+POOL_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_kv_pool_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(POOL_EXE),
+                    reason="oracle/_ref/test_kv_pool_hip not built (needs the reference tree)")
+def test_reference_own_kv_pool_test_passes_on_this_backend():
+    """The reference's tests/test_kv_pool.c with the reference's KV cache code:
+    the paged pool's bookkeeping against the device page table this backend
+    writes (vv_kv_page_map_dev), exhaustion, and four threads contending."""
+    res = subprocess.run([POOL_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "PASS" in res.stdout and "FAIL" not in res.stdout and "SKIP" not in res.stdout
