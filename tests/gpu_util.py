@@ -13,7 +13,7 @@ from __graft_entry__ import load_device
 
 dev = load_device()
 
-FP16_TOL = 2e-3      # BASELINE bar: max|err| / max|ref| for FP16 outputs
+FP16_TOL = 2e-3      # the acceptance bar for FP16 outputs: max|err| / max|ref|
 
 
 def stream() -> int:

@@ -6,7 +6,7 @@ Bars (written where they are applied, in gpu_util.assert_fp16_close):
     fused add+norm, and FP16<->FP32 conversion: BIT-EXACT;
   * RMSNorm, RoPE, SwiGLU outputs (FP16): max|err| / max|ref| <= 2e-3, and on
     top of that at most 1 FP16 ulp from the oracle's correctly rounded value.
-Shapes are BASELINE's configs 2-5 plus the generic widths the reference's own
+Shapes are the benchmark's configurations 2-5 plus the generic widths the reference's own
 tests and callers use (tests/test_int8_linear.c:297, test_prefill_append.c:30).
 """
 import numpy as np
@@ -358,7 +358,7 @@ def test_embedding_any_bit_pattern_other_widths_and_decode_row():
         assert np.array_equal(bits_of(d_o), table[ids]), (hidden, vocab, T)
 
 
-# ── bias add and conversions (next rows) ────────────────────────────────────
+# ── bias add and conversions ─────────────────────────────────────────────────
 
 @pytest.mark.parametrize("M,N", [(285, 3584), (7, 512), (3, 100), (1, 18944)])
 def test_bias_add_bit_exact(M, N):
@@ -390,7 +390,7 @@ def test_fp16_fp32_conversions_bit_exact():
 # ── full prefill size (T = 14449): size-independent properties ──────────────
 
 def test_full_size_properties_T14449():
-    """At BASELINE's full size the oracle is run on sampled rows only; the rest
+    """At the benchmark's full size the oracle is run on sampled rows only; the rest
     is covered by equalities that hold at any size."""
     T = 14449
     gen = torch.Generator(device="cuda").manual_seed(14449)

@@ -184,7 +184,7 @@ def test_reference_recipe_swiglu():
 # ── closed forms, invariants, special cases ─────────────────────────────────
 
 def test_config1_rmsnorm_one_decode_row_seed0():
-    """BASELINE config 1: fp32 x [1,3584] ~N(0,1), w ~N(1,0.1), eps 1e-6, seed 0."""
+    """Benchmark configuration 1: fp32 x [1,3584] ~N(0,1), w ~N(1,0.1), eps 1e-6, seed 0."""
     x = oracle.normal_f32((1, H), seed=0)
     w = oracle.normal_f16((H,), seed=0 + 1000, mean=1.0, std=0.1)
     x64, w64 = x.astype(np.float64), oracle.widen(w).astype(np.float64)
