@@ -121,6 +121,47 @@ vv_status_t vv_swiglu_q8_dev(const void* gate, const void* up, int M, int K,
  * (src/cuda/act_quant.cu:277-313). */
 vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* stream);
 
+/* ── W8A8 linear layers ────────────────────────────────────────────────── */
+
+/* Which kernel family runs an int8 linear layer (device.h:347-352). Here GEMV
+ * is the v_dot4 kernel (M <= 8 only), MMA and SIMT both the MFMA tile kernel. */
+#define VV_I8_PATH_AUTO 0
+#define VV_I8_PATH_GEMV 1
+#define VV_I8_PATH_MMA  2
+#define VV_I8_PATH_SIMT 3
+
+/* y[M,N] = sx[m] * sw[n] * (xq[M,K] . w[N,K]^T) + bias[n] + residual[m,n]:
+ * xq int8 with per-row scales sx (what vv_act_quant_dev writes in layout 0),
+ * w int8 [N][K] with per-output-channel scales sw. bias FP16 [N] or NULL;
+ * residual FP16 [M,N] or NULL, may alias y; y FP16, or FP32 when y_f32. The
+ * int32 sums are exact, and the FP32 value is ((float)t * sx[m]) * sw[n], then
+ * + bias, then + residual, nothing fused: bit-identical to the CPU kernel
+ * (src/cpu/cpu_int8.c:480-483) for every M, N, K and path. K % 16 != 0 or
+ * xq / w not 16-byte aligned: VV_ERR_UNSUPPORTED (the reference asks K % 32).
+ * replaces device.h:363-366 (src/cuda/gemm_i8.cu:584-596). */
+vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* w,
+                               const float* sw, const void* bias, const void* residual,
+                               void* y, int y_f32, int M, int N, int K, int path,
+                               void* stream);
+
+/* One projection of a shared-input int8 launch (device.h:391-398). */
+typedef struct vv_i8_proj {
+    const void* w;     /* int8 [N][K] */
+    const void* sw;    /* FP32 [N] */
+    const void* sz;    /* W4A8 only: unused here */
+    const void* bias;  /* FP16 [N] or NULL */
+    void*       y;     /* FP16 [M][N] */
+    int         N;
+} vv_i8_proj_t;
+
+/* Several projections of one int8 input (q/k/v, gate/up), each computed exactly
+ * as vv_w8a8_linear_dev would. w4 != 0 (W4A8) or x_layout != 0:
+ * VV_ERR_UNSUPPORTED, nothing launched. xsum and group_size are W4A8's and are
+ * ignored. replaces device.h:411-414 (src/cuda/gemm_i8.cu:616-645). */
+vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* sx,
+                                   const int32_t* xsum, int w4, const vv_i8_proj_t* projs,
+                                   int n, int group_size, int M, int K, void* stream);
+
 /* ── Dense linear layers ───────────────────────────────────────────────── */
 
 /* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32

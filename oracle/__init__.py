@@ -75,6 +75,9 @@ def _load():
     lib.vvo_gemm_f16w.argtypes = [_f32p, _u16p, _u16p, _f32p, C.c_int, C.c_int, C.c_int]
     lib.vvo_attention_prefill_f32.restype = C.c_int
     lib.vvo_attention_prefill_f32.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 7
+    lib.vvo_w8a8_linear.restype = C.c_int
+    lib.vvo_w8a8_linear.argtypes = [C.c_void_p, _f32p, C.c_void_p, _f32p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                    C.c_void_p, C.c_int, C.c_int, C.c_int]
     lib.vvo_argmax_first.restype = C.c_int
     lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
@@ -106,6 +109,10 @@ def _load_ref():
     ref.vv_gemm_f16w_cpu.argtypes = [_f32p, vp, vp, _f32p, C.c_int, C.c_int, C.c_int]
     ref.vv_attention_prefill_cpu.restype = C.c_int
     ref.vv_attention_prefill_cpu.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 6 + [C.c_bool]
+    if hasattr(ref, "vv_w8a8_gemm_cpu"):
+        ref.vv_w8a8_gemm_cpu.restype = C.c_int
+        ref.vv_w8a8_gemm_cpu.argtypes = [C.c_void_p, _f32p, C.c_void_p, _f32p, C.c_void_p, _f32p,
+                                         C.c_int, C.c_int, C.c_int]
     if hasattr(ref, "vv_quant_act_q8_cpu"):
         ref.vv_quant_act_q8_cpu.restype = C.c_int
         ref.vv_quant_act_q8_cpu.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8),
@@ -320,3 +327,20 @@ def argmax_first(logits: np.ndarray):
     tok, val = C.c_int32(), C.c_float()
     _check(lib.vvo_argmax_first(_p(logits, _f32p), logits.size, C.byref(tok), C.byref(val)), "argmax_first")
     return int(tok.value), float(val.value)
+
+
+def w8a8_linear(xq, sx, w, sw, bias16=None, res16=None):
+    """int8 [M,K] x int8 [N,K]^T with per-row scales -> (float32 [M,N], FP16 bits [M,N])."""
+    xq, w = np.ascontiguousarray(xq, np.int8), np.ascontiguousarray(w, np.int8)
+    sx, sw = np.ascontiguousarray(sx, np.float32), np.ascontiguousarray(sw, np.float32)
+    M, K = xq.shape
+    N = w.shape[0]
+    f32, f16 = np.empty((M, N), np.float32), np.empty((M, N), np.uint16)
+    ptr = lambda a: a.ctypes.data if a is not None else None
+    if bias16 is not None:
+        bias16 = np.ascontiguousarray(bias16, np.uint16)
+    if res16 is not None:
+        res16 = np.ascontiguousarray(res16, np.uint16)
+    _check(lib.vvo_w8a8_linear(xq.ctypes.data, _p(sx, _f32p), w.ctypes.data, _p(sw, _f32p), ptr(bias16),
+                               ptr(res16), f32.ctypes.data, f16.ctypes.data, M, N, K), "w8a8_linear")
+    return f32, f16

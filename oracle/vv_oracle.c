@@ -395,6 +395,28 @@ int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
     return VVO_OK;
 }
 
+int vvo_w8a8_linear(const int8_t* xq, const float* sx, const int8_t* w, const float* sw,
+                    const uint16_t* bias16, const uint16_t* res16, float* out_f32,
+                    uint16_t* out_f16, int M, int N, int K) {
+    if (!xq || !sx || !w || !sw) return VVO_ERR_NULL_PTR;
+    int n;
+#pragma omp parallel for schedule(static)
+    for (n = 0; n < N; n++) {
+        const int8_t* wr = w + (size_t)n * K;
+        for (int m = 0; m < M; m++) {
+            const int8_t* xr = xq + (size_t)m * K;
+            int32_t t = 0;
+            for (int k = 0; k < K; k++) t += (int32_t)xr[k] * (int32_t)wr[k];
+            float v = (float)t * sx[m] * sw[n];
+            if (bias16) v += vvo_half_to_float(bias16[n]);
+            if (res16) v += vvo_half_to_float(res16[(size_t)m * N + n]);
+            if (out_f32) out_f32[(size_t)m * N + n] = v;
+            if (out_f16) out_f16[(size_t)m * N + n] = vvo_float_to_half_rne(v);
+        }
+    }
+    return VVO_OK;
+}
+
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value) {
     if (!logits || !token) return VVO_ERR_NULL_PTR;
     int best = 0;

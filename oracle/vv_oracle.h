@@ -124,6 +124,16 @@ int vvo_attention_prefill_f32(const float* q, const float* k, const float* v,
                               int head_dim, int rows, int q_offset, int kv_len,
                               int causal);
 
+/* The W8A8 linear layer. src/cpu/cpu_int8.c:455-487 (vv_w8a8_gemm_cpu): exact
+ * int32 dot of the int8 rows, then v = (float)t * sx[m] * sw[n] (+ bias[n]),
+ * products left to right, nothing fused; the device contract
+ * (src/cuda/i8_common.cuh:40-48) then adds a residual [M,N] and writes FP32 or
+ * FP16 (RNE). bias16 / res16 are FP16 bit patterns or NULL; out_f32 / out_f16
+ * either may be NULL. */
+int vvo_w8a8_linear(const int8_t* xq, const float* sx, const int8_t* w, const float* sw,
+                    const uint16_t* bias16, const uint16_t* res16, float* out_f32,
+                    uint16_t* out_f16, int M, int N, int K);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

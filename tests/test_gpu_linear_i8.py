@@ -1,0 +1,231 @@
+"""GPU parity tests of the W8A8 linear layer through the C ABI.
+
+The products are summed in int32 (exact) and the epilogue follows the CPU
+kernel operation for operation, so the bar is bit equality: the FP32 output
+against the oracle's FP32 values, the FP16 output against their
+round-to-nearest-even bits, for every kernel family, tile shape and edge.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import bits_of, dev, ok, stream, to_dev
+
+pytestmark = pytest.mark.gpu
+
+AUTO, GEMV, MMA, SIMT = 0, 1, 2, 3
+
+
+def operands(M, N, K, seed, wide=False):
+    rng = np.random.default_rng(seed)
+    lo = -128 if wide else -127
+    xq = rng.integers(lo, 128, (M, K), dtype=np.int8)
+    w = rng.integers(lo, 128, (N, K), dtype=np.int8)
+    sx = (rng.random(M, dtype=np.float32) * 0.05 + 1e-3).astype(np.float32)
+    sw = (rng.random(N, dtype=np.float32) * 0.01 + 1e-4).astype(np.float32)
+    bias = oracle.normal_f16((N,), seed + 1, std=0.5)
+    res = oracle.normal_f16((M, N), seed + 2, std=2.0)
+    return xq, sx, w, sw, bias, res
+
+
+def i8_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run(xq, sx, w, sw, bias=None, res=None, f32=False, path=AUTO, alias=False):
+    M, K = xq.shape
+    N = w.shape[0]
+    d_xq, d_w, d_sx, d_sw = i8_dev(xq), i8_dev(w), i8_dev(sx), i8_dev(sw)
+    d_b = to_dev(bias) if bias is not None else None
+    d_r = to_dev(res) if res is not None else None
+    if alias:
+        d_y = d_r
+    else:
+        d_y = torch.full((M, N), float("nan"), dtype=torch.float32 if f32 else torch.float16, device="cuda")
+    ok(dev.vv_w8a8_linear_dev(d_xq.data_ptr(), d_sx.data_ptr(), d_w.data_ptr(), d_sw.data_ptr(),
+                              d_b.data_ptr() if d_b is not None else None,
+                              d_r.data_ptr() if d_r is not None else None,
+                              d_y.data_ptr(), 1 if f32 else 0, M, N, K, path, stream()))
+    torch.cuda.synchronize()
+    return d_y.cpu().numpy() if f32 else bits_of(d_y)
+
+
+def same_f32(got, want, what):
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), \
+        f"{what}: {(got.view(np.uint32) != want.view(np.uint32)).sum()} FP32 values differ"
+
+
+SHAPES = [(1, 64, 16), (1, 3584, 3584), (1, 18944, 3584), (1, 8200, 512), (2, 100, 48), (3, 512, 3584), (5, 77, 1040),
+          (8, 1000, 1536), (9, 64, 64), (16, 30, 48), (29, 512, 3584), (33, 77, 528), (64, 256, 512),
+          (65, 3584, 128), (100, 130, 80), (130, 101, 208), (257, 37, 16), (285, 3584, 3584), (300, 4608, 272),
+          (4100, 8200, 64)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_w8a8_bit_exact_against_oracle(M, N, K):
+    xq, sx, w, sw, bias, res = operands(M, N, K, 7 * M + N)
+    want32, want16 = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+    same_f32(run(xq, sx, w, sw, bias, res, f32=True), want32, f"f32 {M}x{N}x{K}")
+    assert np.array_equal(run(xq, sx, w, sw, bias, res), want16), f"f16 {M}x{N}x{K}"
+    plain32, plain16 = oracle.w8a8_linear(xq, sx, w, sw)
+    same_f32(run(xq, sx, w, sw, f32=True), plain32, f"f32 plain {M}x{N}x{K}")
+    assert np.array_equal(run(xq, sx, w, sw), plain16), f"f16 plain {M}x{N}x{K}"
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (4, 260, 128), (8, 3584, 512), (40, 100, 64), (200, 264, 144)])
+@pytest.mark.parametrize("with_bias,with_res", [(True, False), (False, True)])
+def test_w8a8_bias_or_residual_alone(M, N, K, with_bias, with_res):
+    xq, sx, w, sw, bias, res = operands(M, N, K, 31 + M)
+    b, r = (bias if with_bias else None), (res if with_res else None)
+    want32, want16 = oracle.w8a8_linear(xq, sx, w, sw, b, r)
+    same_f32(run(xq, sx, w, sw, b, r, f32=True), want32, "f32")
+    assert np.array_equal(run(xq, sx, w, sw, b, r), want16)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 512, 256), (7, 130, 64), (64, 512, 256), (300, 264, 128)])
+def test_w8a8_residual_may_alias_output(M, N, K):
+    """y += result: the residual buffer is the output buffer."""
+    xq, sx, w, sw, bias, res = operands(M, N, K, 91 + M)
+    _, want16 = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+    assert np.array_equal(run(xq, sx, w, sw, bias, res, alias=True), want16)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 8200, 256), (8, 16400, 64), (8, 77, 48)])
+def test_w8a8_kernel_families_agree(M, N, K):
+    """Up to eight rows both families serve the shape, with the same bits."""
+    xq, sx, w, sw, bias, res = operands(M, N, K, 17 + N)
+    want32, _ = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+    for path in (AUTO, GEMV, MMA, SIMT):
+        same_f32(run(xq, sx, w, sw, bias, res, f32=True, path=path), want32, f"path {path}")
+
+
+def test_w8a8_extreme_values_do_not_saturate():
+    """-128 * -128 over the longest K of the model: 3.1e8, inside int32."""
+    M, N, K = 9, 64, 18944
+    xq = np.full((M, K), -128, np.int8)
+    w = np.full((N, K), -128, np.int8)
+    w[1::2] = 127
+    sx, sw = np.full(M, 2.0 ** -10, np.float32), np.full(N, 2.0 ** -12, np.float32)
+    want32, _ = oracle.w8a8_linear(xq, sx, w, sw)
+    assert want32[0, 0] == np.float32(128 * 128 * K) * np.float32(2.0 ** -22)
+    same_f32(run(xq, sx, w, sw, f32=True), want32, "mfma")
+    same_f32(run(xq[:4], sx[:4], w, sw, f32=True), want32[:4], "gemv")
+
+
+def test_w8a8_unaligned_vectors_and_ragged_n():
+    """bias / scale / output pointers that are only element-aligned, N % 4 != 0."""
+    M, N, K = 37, 103, 96
+    xq, sx, w, sw, bias, res = operands(M, N, K, 5)
+    want32, want16 = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+    same_f32(run(xq, sx, w, sw, bias, res, f32=True), want32, "ragged N")
+    # N % 4 == 0 but every FP16 / FP32 operand one element off a 16-byte boundary
+    N = 104
+    xq, sx, w, sw, bias, res = operands(M, N, K, 6)
+    want32, want16 = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+    d_xq, d_w, d_sx = i8_dev(xq), i8_dev(w), i8_dev(sx)
+    pad = lambda t: torch.cat([torch.zeros(1, dtype=t.dtype, device="cuda"), t.reshape(-1)])[1:]
+    d_sw, d_b, d_r = pad(i8_dev(sw)), pad(to_dev(bias)), pad(to_dev(res))
+    d_y = pad(torch.zeros(M * N, dtype=torch.float16, device="cuda"))
+    assert d_sw.data_ptr() % 16 != 0 and d_b.data_ptr() % 8 != 0 and d_y.data_ptr() % 8 != 0
+    ok(dev.vv_w8a8_linear_dev(d_xq.data_ptr(), d_sx.data_ptr(), d_w.data_ptr(), d_sw.data_ptr(), d_b.data_ptr(),
+                              d_r.data_ptr(), d_y.data_ptr(), 0, M, N, K, AUTO, stream()))
+    assert np.array_equal(bits_of(d_y).reshape(M, N), want16)
+
+
+def test_w8a8_follows_the_device_quantiser():
+    """FP16 activations -> vv_act_quant_dev -> vv_w8a8_linear_dev equals the
+    oracle's quantiser followed by the oracle's linear, and is close to the
+    unquantised product."""
+    M, N, K = 70, 512, 3584
+    x = oracle.normal_f16((M, K), 3)
+    wf = oracle.normal_f32((N, K), 4, std=K ** -0.5)
+    sw = (np.abs(wf).max(axis=1) / 127.0).astype(np.float32)
+    w = np.clip(np.rint(wf / sw[:, None]), -127, 127).astype(np.int8)
+    d_x, d_w, d_sw = to_dev(x), i8_dev(w), i8_dev(sw)
+    d_xq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    d_sx = torch.empty(M, dtype=torch.float32, device="cuda")
+    d_y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    ok(dev.vv_act_quant_dev(d_x.data_ptr(), M, K, 0, d_xq.data_ptr(), d_sx.data_ptr(), None, stream()))
+    ok(dev.vv_w8a8_linear_dev(d_xq.data_ptr(), d_sx.data_ptr(), d_w.data_ptr(), d_sw.data_ptr(), None, None,
+                              d_y.data_ptr(), 1, M, N, K, AUTO, stream()))
+    torch.cuda.synchronize()
+    xq, sx, _ = oracle.quant_act_q8(oracle.widen(x), 0, want_xsum=False)
+    want32, _ = oracle.w8a8_linear(xq, sx, w, sw)
+    same_f32(d_y.cpu().numpy(), want32, "quantise + linear")
+    dense = oracle.widen(x).astype(np.float64) @ wf.astype(np.float64).T
+    assert np.max(np.abs(want32 - dense)) / np.max(np.abs(dense)) < 0.03
+
+
+def test_w8a8_prefill_shape_sampled_rows():
+    """The model's prefill shape (T = 14449 rows through a 3584 x 3584
+    projection): 48 sampled rows against the oracle, and the whole output
+    against the same call split in two row blocks (rows are independent)."""
+    M, N, K = 14449, 3584, 3584
+    xq, sx, w, sw, bias, _ = operands(M, N, K, 11)
+    d_xq, d_w, d_sx, d_sw, d_b = i8_dev(xq), i8_dev(w), i8_dev(sx), i8_dev(sw), to_dev(bias)
+    d_y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    args = lambda r0, rows: (d_xq[r0:].data_ptr(), d_sx[r0:].data_ptr(), d_w.data_ptr(), d_sw.data_ptr(),
+                             d_b.data_ptr(), None)
+    ok(dev.vv_w8a8_linear_dev(*args(0, M), d_y.data_ptr(), 0, M, N, K, AUTO, stream()))
+    got = bits_of(d_y)
+    rows = np.sort(np.random.default_rng(1).choice(M, 48, replace=False))
+    rows[0], rows[-1] = 0, M - 1
+    _, want16 = oracle.w8a8_linear(xq[rows], sx[rows], w, sw, bias)
+    assert np.array_equal(got[rows], want16)
+    d_z = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    cut = 6000
+    ok(dev.vv_w8a8_linear_dev(*args(0, cut), d_z.data_ptr(), 0, cut, N, K, AUTO, stream()))
+    ok(dev.vv_w8a8_linear_dev(*args(cut, M - cut), d_z[cut:].data_ptr(), 0, M - cut, N, K, AUTO, stream()))
+    assert np.array_equal(bits_of(d_z), got)
+
+
+@pytest.mark.parametrize("M", [1, 6, 40])
+def test_i8_linear_multi_equals_single_calls(M):
+    K = 512
+    Ns = [512, 128, 136]
+    xq, sx, *_ = operands(M, 8, K, 50 + M)
+    d_xq, d_sx = i8_dev(xq), i8_dev(sx)
+    keep, projs, wants = [], (dev.I8Proj * 3)(), []
+    for i, N in enumerate(Ns):
+        _, _, w, sw, bias, _ = operands(M, N, K, 60 + i)
+        b = bias if i != 1 else None
+        d_w, d_sw = i8_dev(w), i8_dev(sw)
+        d_b = to_dev(b) if b is not None else None
+        d_y = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        keep.append((d_w, d_sw, d_b, d_y))
+        projs[i] = dev.I8Proj(d_w.data_ptr(), d_sw.data_ptr(), None, d_b.data_ptr() if d_b is not None else None,
+                          d_y.data_ptr(), N)
+        wants.append(oracle.w8a8_linear(xq, sx, w, sw, b)[1])
+    call = lambda layout, w4, n: dev.vv_i8_linear_multi_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), None, w4,
+                                                            C.addressof(projs), n, 0, M, K, stream())
+    ok(call(0, 0, 3))
+    for (_, _, _, d_y), want in zip(keep, wants):
+        assert np.array_equal(bits_of(d_y), want)
+    assert call(0, 1, 3) == dev.VV_ERR_UNSUPPORTED       # W4A8
+    assert call(1, 0, 3) == dev.VV_ERR_UNSUPPORTED       # a layout only W4A8 reads
+    assert call(0, 0, 0) == dev.VV_ERR_INVALID_ARG
+    assert dev.vv_i8_linear_multi_dev(None, 0, d_sx.data_ptr(), None, 0, C.addressof(projs), 3, 0, M, K,
+                                      stream()) == dev.VV_ERR_NULL_PTR
+
+
+def test_w8a8_argument_checks_launch_nothing():
+    M, N, K = 4, 64, 64
+    xq, sx, w, sw, *_ = operands(M, N, K, 1)
+    d_xq, d_w, d_sx, d_sw = i8_dev(xq), i8_dev(w), i8_dev(sx), i8_dev(sw)
+    d_y = torch.full((16, N), 7.0, dtype=torch.float16, device="cuda")
+    X, S, W, SW, Y = d_xq.data_ptr(), d_sx.data_ptr(), d_w.data_ptr(), d_sw.data_ptr(), d_y.data_ptr()
+    f = dev.vv_w8a8_linear_dev
+    for args in [(None, S, W, SW), (X, None, W, SW), (X, S, None, SW), (X, S, W, None)]:
+        assert f(*args, None, None, Y, 0, M, N, K, AUTO, stream()) == dev.VV_ERR_NULL_PTR
+    assert f(X, S, W, SW, None, None, None, 0, M, N, K, AUTO, stream()) == dev.VV_ERR_NULL_PTR
+    for m, n, k in [(0, N, K), (M, 0, K), (M, N, 0), (-1, N, K)]:
+        assert f(X, S, W, SW, None, None, Y, 0, m, n, k, AUTO, stream()) == dev.VV_ERR_INVALID_ARG
+    assert f(X, S, W, SW, None, None, Y, 0, M, N, K, 4, stream()) == dev.VV_ERR_INVALID_ARG
+    assert f(X, S, W, SW, None, None, Y, 0, M, N, 40, AUTO, stream()) == dev.VV_ERR_UNSUPPORTED   # K % 16
+    assert f(X + 4, S, W, SW, None, None, Y, 0, 1, N, 48, AUTO, stream()) == dev.VV_ERR_UNSUPPORTED
+    assert f(X, S, W, SW, None, None, Y, 0, 9, N, K, GEMV, stream()) == dev.VV_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+    assert (d_y == 7.0).all()

@@ -105,3 +105,34 @@ def test_quantiser_argument_checks():
     assert call(x.ctypes.data_as(f32p), 2, 48, 0, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -1
     assert call(x.ctypes.data_as(f32p), 2, 64, 4, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -1
     assert call(None, 2, 64, 0, q.ctypes.data_as(i8p), sx.ctypes.data_as(f32p), None) == -2
+
+
+def test_w8a8_linear_against_integer_closed_form_and_reference():
+    """The int32 dot is exact, so the FP32 output is pinned bit for bit: by the
+    compiled reference (vv_w8a8_gemm_cpu) and by an int64 matmul followed by the
+    same two FP32 products and one addition."""
+    import ctypes as C
+    rng = np.random.default_rng(5)
+    for M, N, K in ((1, 16, 32), (5, 70, 3584), (9, 33, 160)):
+        xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        sx = rng.uniform(0.001, 0.05, M).astype(np.float32)
+        sw = rng.uniform(0.0005, 0.01, N).astype(np.float32)
+        bias = oracle.normal_f16((N,), 3, std=0.5)
+        res = oracle.normal_f16((M, N), 4)
+        t = xq.astype(np.int64) @ w.astype(np.int64).T
+        assert np.abs(t).max() < 2 ** 31
+        want = (t.astype(np.float32) * sx[:, None]) * sw[None, :]
+        plain, _ = oracle.w8a8_linear(xq, sx, w, sw)
+        assert np.array_equal(plain, want)
+        with_b = want + oracle.widen(bias)[None, :]
+        f32, f16 = oracle.w8a8_linear(xq, sx, w, sw, bias, res)
+        assert np.array_equal(f32, with_b + oracle.widen(res))
+        assert np.array_equal(f16, f32.astype(np.float16).view(np.uint16))
+        if oracle.ref is not None and hasattr(oracle.ref, "vv_w8a8_gemm_cpu"):
+            out = np.empty((M, N), np.float32)
+            f32p = C.POINTER(C.c_float)
+            assert oracle.ref.vv_w8a8_gemm_cpu(xq.ctypes.data, sx.ctypes.data_as(f32p), w.ctypes.data,
+                                               sw.ctypes.data_as(f32p), bias.ctypes.data,
+                                               out.ctypes.data_as(f32p), M, N, K) == 0
+            assert np.array_equal(out, with_b)

@@ -1,0 +1,263 @@
+// W8A8 linear layers: y[M,N] = sx[m] * sw[n] * (xq[M,K] . w[N,K]^T) + bias[n]
+// + residual[m,n], int8 activations (per-row scale, from the activation
+// quantisers) times int8 weights (per-output-channel scale).
+//
+// The products are summed in int32, which is exact, so the result does not
+// depend on tile shape or summation order and equals the CPU kernel's bit for
+// bit once the epilogue follows it: (float)t * sx[m] * sw[n], left to right,
+// nothing fused, then the bias, then the residual, one rounding to FP16.
+//
+//   i8_tile   the LDS-tiled loop of the FP16 GEMM with v_mfma_i32_32x32x32_i8:
+//             a lane's 16-byte operand is 16 int8 values, so a K step is 32
+//             wide and a 128-byte slab row carries 128 K values.
+//   i8_gemv   M <= 8: one to four waves per weight row, v_dot4_i32_i8 against
+//             up to eight activation rows that share each weight load.
+#include "mfma_tile.hpp"
+
+namespace vv {
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+
+struct I8Op {
+    typedef i32x16 Acc;
+    static __device__ __forceinline__ Acc mfma(u32x4 w, u32x4 x, Acc c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, w),
+                                                     __builtin_bit_cast(i32x4, x), c, 0, 0, 0);
+    }
+};
+
+struct I8Out {
+    const float* sx;
+    const float* sw;
+    const h16* bias;
+    const h16* res;
+    void* y;
+    int y_f32, M, N, vec;
+};
+
+// One output value from its exact integer sum: the CPU kernel's expression
+// (src/cpu/cpu_int8.c:480-483), then the device contract's residual.
+__device__ __forceinline__ float i8_value(int t, float sxm, float swn, bool has_b, float b, bool has_r,
+                                          float r) {
+#pragma clang fp contract(off)
+    float v = (float)t * sxm * swn;
+    if (has_b) v = v + b;
+    if (has_r) v = v + r;
+    return v;
+}
+
+__device__ __forceinline__ void i8_store1(const I8Out& o, int m, int n, int t) {
+    const size_t idx = (size_t)m * o.N + n;
+    const float v = i8_value(t, o.sx[m], o.sw[n], o.bias != nullptr, o.bias ? (float)o.bias[n] : 0.0f,
+                             o.res != nullptr, o.res ? (float)o.res[idx] : 0.0f);
+    if (o.y_f32) static_cast<float*>(o.y)[idx] = v;
+    else static_cast<h16*>(o.y)[idx] = to_half(v);
+}
+
+// Four consecutive columns of one row.
+__device__ __forceinline__ void i8_store4(const I8Out& o, int m, int n, const int (&t)[4]) {
+    if (o.vec && n + 3 < o.N) {
+        const size_t idx = (size_t)m * o.N + n;
+        const float sxm = o.sx[m];
+        const f32x4 sw = *reinterpret_cast<const f32x4*>(o.sw + n);
+        h16x4 b = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+        if (o.bias) b = *reinterpret_cast<const h16x4*>(o.bias + n);
+        if (o.res) r = *reinterpret_cast<const h16x4*>(o.res + idx);
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = i8_value(t[i], sxm, sw[i], o.bias != nullptr, (float)b[i], o.res != nullptr, (float)r[i]);
+        if (o.y_f32) {
+            *reinterpret_cast<f32x4*>(static_cast<float*>(o.y) + idx) = v;
+        } else {
+            h16x4 h;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[i] = to_half(v[i]);
+            *reinterpret_cast<h16x4*>(static_cast<h16*>(o.y) + idx) = h;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n + i < o.N) i8_store1(o, m, n + i, t[i]);
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int kSlabChunks, bool kFull, int kAhead>
+__global__ __launch_bounds__(WM * WN * kWave) void i8_tile(const int8_t* __restrict__ xq,
+                                                           const int8_t* __restrict__ w, I8Out out,
+                                                           int K) {
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    auto epilogue = [=](const i32x16 (&acc)[TN][TM], int m0, int n0, int frow, int fhalf) {
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int m = m0 + b * 32 + frow;
+            if (m >= out.M) continue;
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + a * 32 + 8 * g + 4 * fhalf;
+                    if (n >= out.N) continue;
+                    const int t[4] = {acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2],
+                                      acc[a][b][4 * g + 3]};
+                    i8_store4(out, m, n, t);
+                }
+        }
+    };
+    mfma_tile<I8Op, BM, BN, WM, WN, kSlabChunks, kFull, kAhead>(xq, w, out.M, out.N, K / 16, epilogue);
+}
+
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);   // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);   // row_mirror
+    return (__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16)) +
+           (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
+}
+
+// M <= MR <= 8 rows: kSplit waves per weight row, each a contiguous 1/kSplit of K.
+template <int MR, int kSplit>
+__global__ __launch_bounds__(kBlock) void i8_gemv(const int8_t* __restrict__ xq,
+                                                  const int8_t* __restrict__ w, I8Out out, int K) {
+    constexpr int kRows = kWavesPerBlock / kSplit;
+    __shared__ int part[kWavesPerBlock][MR];
+    const int wave = wave_in_block(), lane = lane_id();
+    const int n = (int)blockIdx.x * kRows + wave / kSplit;
+    const int piece = wave % kSplit;
+    const int kchunks = K / 16;
+    const int per = (kchunks + kSplit - 1) / kSplit;
+    const int begin = piece * per, end = min(kchunks, begin + per);
+    int acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0;
+    if (n < out.N) {
+        const i32x4* wr = reinterpret_cast<const i32x4*>(w + (size_t)n * K);
+#pragma unroll 2
+        for (int c = begin + lane; c < end; c += kWave) {
+            const i32x4 wv = __builtin_nontemporal_load(wr + c);
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                if (m < out.M) {
+                    const i32x4 xv = *(reinterpret_cast<const i32x4*>(xq + (size_t)m * K) + c);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[m] = __builtin_amdgcn_sdot4(xv[i], wv[i], acc[m], false);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = wave_sum_i32(acc[m]);
+    if constexpr (kSplit > 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MR; ++m) part[wave][m] = acc[m];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            acc[m] = 0;
+#pragma unroll
+            for (int p = 0; p < kSplit; ++p) acc[m] += part[(wave / kSplit) * kSplit + p][m];
+        }
+    }
+    if (n < out.N && piece == 0) {
+        int mine = 0;
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+            if (lane == m) mine = acc[m];
+        if (lane < out.M && lane < MR) i8_store1(out, lane, n, mine);
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int kSlabChunks, int kAhead>
+void launch_i8_tile(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
+    const dim3 grid((unsigned)((out.N + BN - 1) / BN), (unsigned)((out.M + BM - 1) / BM));
+    if ((K / 16) % kSlabChunks == 0)
+        i8_tile<BM, BN, WM, WN, kSlabChunks, true, kAhead><<<grid, WM * WN * kWave, 0, st>>>(xq, w, out, K);
+    else
+        i8_tile<BM, BN, WM, WN, kSlabChunks, false, kAhead><<<grid, WM * WN * kWave, 0, st>>>(xq, w, out, K);
+}
+
+template <int MR>
+void launch_i8_gemv(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
+    const int N = out.N;
+    if (N >= 16384) i8_gemv<MR, 1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(xq, w, out, K);
+    else if (N >= 8192) i8_gemv<MR, 2><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(xq, w, out, K);
+    else i8_gemv<MR, 4><<<dim3((unsigned)N), kBlock, 0, st>>>(xq, w, out, K);
+}
+
+enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* w, const float* sw,
+                               const void* bias, const void* residual, void* y, int y_f32, int M,
+                               int N, int K, int path, void* stream) {
+    if (!xq || !sx || !w || !sw || !y) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0 || path < vv::kPathAuto || path > vv::kPathSimt)
+        return VV_ERR_INVALID_ARG;
+    if (K % 16 != 0 || !vv::aligned16(xq) || !vv::aligned16(w)) return VV_ERR_UNSUPPORTED;
+    if (path == vv::kPathGemv && M > 8) return VV_ERR_UNSUPPORTED;
+    hipStream_t st = vv::as_stream(stream);
+    vv::I8Out out;
+    out.sx = sx;
+    out.sw = sw;
+    out.bias = static_cast<const vv::h16*>(bias);
+    out.res = static_cast<const vv::h16*>(residual);
+    out.y = y;
+    out.y_f32 = y_f32 ? 1 : 0;
+    out.M = M;
+    out.N = N;
+    const auto mis = [](const void* p, unsigned mask) { return p && (reinterpret_cast<uintptr_t>(p) & mask); };
+    out.vec = (N % 4 == 0) && !mis(sw, 15u) && !mis(bias, 7u) && !mis(residual, 7u) &&
+              !mis(y, y_f32 ? 15u : 7u);
+
+    if (M <= 8 && path != vv::kPathMma && path != vv::kPathSimt) {
+        if (M == 1) vv::launch_i8_gemv<1>(xq, w, out, K, st);
+        else if (M == 2) vv::launch_i8_gemv<2>(xq, w, out, K, st);
+        else if (M <= 4) vv::launch_i8_gemv<4>(xq, w, out, K, st);
+        else vv::launch_i8_gemv<8>(xq, w, out, K, st);
+        return vv::launch_status();
+    }
+    // The largest tile that still fills the 256 compute units (as for FP16).
+    const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (wg256 >= 512) vv::launch_i8_tile<256, 256, 2, 4, 4, 2>(xq, w, out, K, st);
+    else if (M > 64 && wg128 >= 256) vv::launch_i8_tile<128, 128, 2, 2, 8, 2>(xq, w, out, K, st);
+    else if (M > 32) vv::launch_i8_tile<64, 64, 2, 2, 8, 1>(xq, w, out, K, st);
+    else vv::launch_i8_tile<32, 64, 1, 2, 8, 1>(xq, w, out, K, st);
+    return vv::launch_status();
+}
+
+/* W8A8 only (w4 == 0), activations in natural column order: one
+ * vv_w8a8_linear_dev per projection, so each is computed exactly as that call
+ * would. W4A8: declined. */
+vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
+                                   int w4, const vv_i8_proj_t* projs, int n, int group_size, int M,
+                                   int K, void* stream) {
+    (void)xsum; (void)group_size;
+    if (!xq || !sx || !projs) return VV_ERR_NULL_PTR;
+    if (n < 1) return VV_ERR_INVALID_ARG;
+    if (w4 != 0 || x_layout != 0) return VV_ERR_UNSUPPORTED;
+    for (int i = 0; i < n; ++i) {
+        if (!projs[i].w || !projs[i].sw || !projs[i].y) return VV_ERR_NULL_PTR;
+        if (K % 16 != 0 || !vv::aligned16(projs[i].w)) return VV_ERR_UNSUPPORTED;
+    }
+    for (int i = 0; i < n; ++i) {
+        const vv_status_t s = vv_w8a8_linear_dev(xq, sx, static_cast<const int8_t*>(projs[i].w),
+                                                 static_cast<const float*>(projs[i].sw), projs[i].bias,
+                                                 nullptr, projs[i].y, 0, M, projs[i].N, K, 0, stream);
+        if (s != VV_OK) return s;
+    }
+    return VV_OK;
+}
+
+}  // extern "C"

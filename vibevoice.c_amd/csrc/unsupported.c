@@ -37,8 +37,8 @@ VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_
 VV_DECLINE(vv_w4a16_gemv_dev)    VV_DECLINE(vv_w4a16_gemv_multi_dev)
 VV_DECLINE(vv_w4a16_gather_dev)  VV_DECLINE(vv_w4a16_gemm_dev)    VV_DECLINE(vv_w4a16_dequant_dev)
 
-/* W8A8 / W4A8 linears (device.h:362-410); the activation quantisers are implemented */
-VV_DECLINE(vv_w8a8_linear_dev)   VV_DECLINE(vv_w4a8_linear_dev)   VV_DECLINE(vv_i8_linear_multi_dev)
+/* W4A8 linear (device.h:385-389); the activation quantisers and W8A8 are implemented */
+VV_DECLINE(vv_w4a8_linear_dev)
 
 /* dense FP16 GEMM: the NN form (device.h:477-479); the NT forms are implemented */
 VV_DECLINE(vv_gemm_fp16_nn_dev)
