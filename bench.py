@@ -225,6 +225,7 @@ def decode_graph_leg(torch, dev, wl1) -> dict:
 
 
 MFMA_F16_PEAK_TFLOPS = 2500.0        # MI355X dense FP16 matrix rate
+MFMA_I8_PEAK_TOPS = 5000.0           # and the dense int8 one
 
 
 def layer_leg(torch, dev, T: int, st: int) -> dict:
@@ -268,6 +269,28 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del a, c
         del w
+    # The same four projections as W8A8 (int8 x int8 on the matrix cores, per-row / per-channel scales).
+    out["w8a8"], out["w8a8_gemv"] = {}, {}
+    for name, n, k in shapes:
+        w8 = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+        sw = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
+        for m, key in ((T, "w8a8"), (1, "w8a8_gemv")):
+            xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+            sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
+            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+            sec = timed(lambda: dev.vv_w8a8_linear_dev(xq.data_ptr(), sx.data_ptr(), w8.data_ptr(), sw.data_ptr(),
+                                                       None, None, c.data_ptr(), 0, m, n, k, 0, st),
+                        5 if m > 1 else 50)
+            if m > 1:
+                tops = 2.0 * m * n * k / sec / 1e12
+                out[key][name] = {"M": m, "N": n, "K": k, "us": sec * 1e6, "TOPs": tops,
+                                  "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
+            else:
+                gb = (n * k + k + 6.0 * n) / sec / 1e9
+                out[key][name] = {"N": n, "K": k, "us": sec * 1e6, "GBps": gb,
+                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+            del xq, sx, c
+        del w8, sw
     q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
     k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
     v_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")

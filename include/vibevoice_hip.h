@@ -121,7 +121,7 @@ vv_status_t vv_swiglu_q8_dev(const void* gate, const void* up, int M, int K,
  * (src/cuda/act_quant.cu:277-313). */
 vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* stream);
 
-/* ── W8A8 linear layers ────────────────────────────────────────────────── */
+/* ── W8A8 / W4A8 linear layers ──────────────────────────────────────────── */
 
 /* Which kernel family runs an int8 linear layer (device.h:347-352). Here GEMV
  * is the v_dot4 kernel (M <= 8 only), MMA and SIMT both the MFMA tile kernel. */
@@ -144,20 +144,40 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
                                void* y, int y_f32, int M, int N, int K, int path,
                                void* stream);
 
+/* y[m,n] = sx[m] * sum_g s[n,g] * sum_{k in g} (q[n,k] - z[n,g]) xq[m,k] + bias[n]
+ * + residual[m,n]: 4-bit weight codes with an FP16 scale and an integer zero
+ * point per group of group_size columns. `packed` [N][K/2] is the accelerator
+ * layout of the INT4 weights (vv_int4g_to_gpu_layout, src/quant/awq_repack.c:
+ * 261-310), `sz` half2 {scale, zero} [N][K/group_size]. x_layout names the
+ * order of xq inside every run of 32 columns: VV_Q8_W4_GEMV (2) for the GEMV
+ * (M <= 8, K <= 20480), VV_Q8_W4_MMA (3) for the matrix-core tiles (any M);
+ * AUTO takes the family the layout belongs to, and a family asked for with the
+ * other layout declines (VV_ERR_UNSUPPORTED), as in the reference. xsum is
+ * accepted and not read (the zero points come off the unpacked codes). Group
+ * sums are exact int32 and the groups are added in order in FP32, nothing
+ * fused, then * sx[m], + bias, + residual: the CPU kernel's scalar form
+ * (src/cpu/cpu_int8.c:212-233, 537-541), the same bits on every path.
+ * K % 32, group_size % 32, K % group_size != 0: VV_ERR_UNSUPPORTED.
+ * replaces device.h:385-389 (src/cuda/gemm_i8.cu:598-614). */
+vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx,
+                               const int32_t* xsum, const void* packed, const void* sz,
+                               int group_size, const void* bias, const void* residual, void* y,
+                               int y_f32, int M, int N, int K, int path, void* stream);
+
 /* One projection of a shared-input int8 launch (device.h:391-398). */
 typedef struct vv_i8_proj {
-    const void* w;     /* int8 [N][K] */
-    const void* sw;    /* FP32 [N] */
-    const void* sz;    /* W4A8 only: unused here */
+    const void* w;     /* W8: int8 [N][K]; W4: accelerator-layout codes [N][K/2] */
+    const void* sw;    /* W8: FP32 [N] */
+    const void* sz;    /* W4: half2 {scale, zero} [N][K/group_size] */
     const void* bias;  /* FP16 [N] or NULL */
     void*       y;     /* FP16 [M][N] */
     int         N;
 } vv_i8_proj_t;
 
 /* Several projections of one int8 input (q/k/v, gate/up), each computed exactly
- * as vv_w8a8_linear_dev would. w4 != 0 (W4A8) or x_layout != 0:
- * VV_ERR_UNSUPPORTED, nothing launched. xsum and group_size are W4A8's and are
- * ignored. replaces device.h:411-414 (src/cuda/gemm_i8.cu:616-645). */
+ * as vv_w8a8_linear_dev (w4 == 0; x_layout must be 0) or vv_w4a8_linear_dev
+ * (w4 != 0, path AUTO) would. replaces device.h:411-414
+ * (src/cuda/gemm_i8.cu:616-645). */
 vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* sx,
                                    const int32_t* xsum, int w4, const vv_i8_proj_t* projs,
                                    int n, int group_size, int M, int K, void* stream);

@@ -78,6 +78,12 @@ def _load():
     lib.vvo_w8a8_linear.restype = C.c_int
     lib.vvo_w8a8_linear.argtypes = [C.c_void_p, _f32p, C.c_void_p, _f32p, C.c_void_p, C.c_void_p, C.c_void_p,
                                     C.c_void_p, C.c_int, C.c_int, C.c_int]
+    lib.vvo_w4a8_linear.restype = C.c_int
+    lib.vvo_w4a8_linear.argtypes = [C.c_void_p, _f32p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]
+    lib.vvo_int4g_to_gpu_layout.restype = C.c_int
+    lib.vvo_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                            C.c_void_p]
     lib.vvo_argmax_first.restype = C.c_int
     lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
@@ -113,6 +119,14 @@ def _load_ref():
         ref.vv_w8a8_gemm_cpu.restype = C.c_int
         ref.vv_w8a8_gemm_cpu.argtypes = [C.c_void_p, _f32p, C.c_void_p, _f32p, C.c_void_p, _f32p,
                                          C.c_int, C.c_int, C.c_int]
+    if hasattr(ref, "vv_w4a8_gemm_cpu"):
+        ref.vv_w4a8_gemm_cpu.restype = C.c_int
+        ref.vv_w4a8_gemm_cpu.argtypes = [C.c_void_p, _f32p, _i32p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                         C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
+    if hasattr(ref, "vv_int4g_to_gpu_layout"):
+        ref.vv_int4g_to_gpu_layout.restype = C.c_int
+        ref.vv_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                               C.c_void_p]
     if hasattr(ref, "vv_quant_act_q8_cpu"):
         ref.vv_quant_act_q8_cpu.restype = C.c_int
         ref.vv_quant_act_q8_cpu.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int8),
@@ -344,3 +358,35 @@ def w8a8_linear(xq, sx, w, sw, bias16=None, res16=None):
     _check(lib.vvo_w8a8_linear(xq.ctypes.data, _p(sx, _f32p), w.ctypes.data, _p(sw, _f32p), ptr(bias16),
                                ptr(res16), f32.ctypes.data, f16.ctypes.data, M, N, K), "w8a8_linear")
     return f32, f16
+
+
+def w4a8_linear(xq, sx, packed, scales16, zeros, G, bias16=None, res16=None):
+    """int8 [M,K] (column order) x INT4G codes [N,K/2] (row-major, high nibble = even column) with FP16
+    group scales [N,K/G] and integer zero points -> (float32 [M,N], FP16 bits [M,N])."""
+    xq = np.ascontiguousarray(xq, np.int8)
+    packed = np.ascontiguousarray(packed, np.uint8)
+    scales16, zeros = np.ascontiguousarray(scales16, np.uint16), np.ascontiguousarray(zeros, np.uint8)
+    sx = np.ascontiguousarray(sx, np.float32)
+    M, K = xq.shape
+    N = packed.shape[0]
+    f32, f16 = np.empty((M, N), np.float32), np.empty((M, N), np.uint16)
+    ptr = lambda a: a.ctypes.data if a is not None else None
+    if bias16 is not None:
+        bias16 = np.ascontiguousarray(bias16, np.uint16)
+    if res16 is not None:
+        res16 = np.ascontiguousarray(res16, np.uint16)
+    _check(lib.vvo_w4a8_linear(xq.ctypes.data, _p(sx, _f32p), packed.ctypes.data, scales16.ctypes.data,
+                               zeros.ctypes.data, G, ptr(bias16), ptr(res16), f32.ctypes.data, f16.ctypes.data,
+                               M, N, K), "w4a8_linear")
+    return f32, f16
+
+
+def int4g_to_gpu_layout(packed, scales16, zeros, G):
+    """Row-major INT4G codes -> (codes in the accelerator layout, half2 {scale, zero} bits [N,K/G,2])."""
+    out = np.array(packed, dtype=np.uint8, order="C", copy=True)
+    scales16, zeros = np.ascontiguousarray(scales16, np.uint16), np.ascontiguousarray(zeros, np.uint8)
+    N, K = out.shape[0], out.shape[1] * 2
+    sz = np.empty((N, K // G, 2), np.uint16)
+    _check(lib.vvo_int4g_to_gpu_layout(out.ctypes.data, scales16.ctypes.data, zeros.ctypes.data, N, K, G,
+                                       sz.ctypes.data), "int4g_to_gpu_layout")
+    return out, sz

@@ -17,7 +17,7 @@
 #include <omp.h>
 #endif
 
-enum { VVO_OK = 0, VVO_ERR_NULL_PTR = -2 };   /* types.h:19,23 */
+enum { VVO_OK = 0, VVO_ERR_INVALID_ARG = -1, VVO_ERR_NULL_PTR = -2 };   /* types.h:19-23 */
 
 /* ── FP16 conversions ─────────────────────────────────────────────────── */
 
@@ -412,6 +412,70 @@ int vvo_w8a8_linear(const int8_t* xq, const float* sx, const int8_t* w, const fl
             if (res16) v += vvo_half_to_float(res16[(size_t)m * N + n]);
             if (out_f32) out_f32[(size_t)m * N + n] = v;
             if (out_f16) out_f16[(size_t)m * N + n] = vvo_float_to_half_rne(v);
+        }
+    }
+    return VVO_OK;
+}
+
+int vvo_w4a8_linear(const int8_t* xq, const float* sx, const uint8_t* packed,
+                    const uint16_t* scales16, const uint8_t* zeros, int G,
+                    const uint16_t* bias16, const uint16_t* res16, float* out_f32,
+                    uint16_t* out_f16, int M, int N, int K) {
+    if (!xq || !sx || !packed || !scales16 || !zeros) return VVO_ERR_NULL_PTR;
+    if (G <= 0 || (G % 32) != 0 || (K % G) != 0) return VVO_ERR_INVALID_ARG;
+    const int ng = K / G;
+    int n;
+#pragma omp parallel for schedule(static)
+    for (n = 0; n < N; n++) {
+        const uint8_t* wr = packed + (size_t)n * (K / 2);
+        for (int m = 0; m < M; m++) {
+            const int8_t* xr = xq + (size_t)m * K;
+            float acc = 0.0f;
+            for (int g = 0; g < ng; g++) {
+                int32_t dot = 0, xs = 0;
+                for (int k = g * G; k < (g + 1) * G; k++) {
+                    const uint8_t b = wr[k / 2];
+                    const int q = (k & 1) ? (b & 15) : (b >> 4);
+                    dot += q * (int32_t)xr[k];
+                    xs += xr[k];
+                }
+                const float s = vvo_half_to_float(scales16[(size_t)n * ng + g]);
+                acc += s * (float)(dot - (int32_t)zeros[(size_t)n * ng + g] * xs);
+            }
+            float v = acc * sx[m];
+            if (bias16) v += vvo_half_to_float(bias16[n]);
+            if (res16) v += vvo_half_to_float(res16[(size_t)m * N + n]);
+            if (out_f32) out_f32[(size_t)m * N + n] = v;
+            if (out_f16) out_f16[(size_t)m * N + n] = vvo_float_to_half_rne(v);
+        }
+    }
+    return VVO_OK;
+}
+
+int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
+                            int N, int K, int G, uint16_t* out_sz) {
+    if (!packed || !scales16 || !zeros || !out_sz) return VVO_ERR_NULL_PTR;
+    if (N <= 0 || K <= 0 || (K % 32) != 0 || G < 32 || (G % 32) != 0 || (K % G) != 0)
+        return VVO_ERR_INVALID_ARG;
+    const int ng = K / G;
+    for (int n = 0; n < N; n++) {
+        for (int c = 0; c < K / 32; c++) {
+            uint8_t* chunk = packed + (size_t)n * (K / 2) + (size_t)c * 16;
+            uint8_t code[32];                       /* code[j]: column 32c + j */
+            for (int j = 0; j < 32; j++)
+                code[j] = (j & 1) ? (uint8_t)(chunk[j / 2] & 15) : (uint8_t)(chunk[j / 2] >> 4);
+            for (int t = 0; t < 4; t++) {
+                uint32_t word = 0;
+                /* slot s of word t: column 2 (t + 4 (s % 4)) + s / 4 */
+                for (int slot = 0; slot < 8; slot++)
+                    word |= (uint32_t)code[2 * (t + 4 * (slot & 3)) + (slot >> 2)] << (4 * slot);
+                for (int b = 0; b < 4; b++) chunk[4 * t + b] = (uint8_t)(word >> (8 * b));
+            }
+        }
+        for (int g = 0; g < ng; g++) {
+            out_sz[((size_t)n * ng + g) * 2] = scales16[(size_t)n * ng + g];
+            out_sz[((size_t)n * ng + g) * 2 + 1] =
+                vvo_float_to_half_rne((float)zeros[(size_t)n * ng + g]);
         }
     }
     return VVO_OK;

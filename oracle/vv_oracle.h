@@ -134,6 +134,29 @@ int vvo_w8a8_linear(const int8_t* xq, const float* sx, const int8_t* w, const fl
                     const uint16_t* bias16, const uint16_t* res16, float* out_f32,
                     uint16_t* out_f16, int M, int N, int K);
 
+/* The W4A8 linear layer. src/cpu/cpu_int8.c:212-233 (w4_dot_scalar) inside
+ * 489-545 (vv_w4a8_gemm_cpu): per group of G columns an exact int32
+ * sum_k q x - z * sum_k x, then acc += s_g * (float)that, groups in order,
+ * nothing fused; v = acc * sx[m] (+ bias[n]); the device contract then adds a
+ * residual and writes FP32 or FP16 (RNE) as for W8A8. `packed` is the
+ * row-major INT4G form ([N][K/2], high nibble = even column), `xq` in column
+ * order (the CPU kernel reads VV_Q8_NIBBLE order; an exact integer sum does
+ * not depend on the order). The reference's vectorised variants add the
+ * groups in another order, so its own FP32 results differ between instruction
+ * sets in the last bits: against the compiled reference this function is
+ * pinned exactly for unit scales and to 1e-6 otherwise. */
+int vvo_w4a8_linear(const int8_t* xq, const float* sx, const uint8_t* packed,
+                    const uint16_t* scales16, const uint8_t* zeros, int G,
+                    const uint16_t* bias16, const uint16_t* res16, float* out_f32,
+                    uint16_t* out_f16, int M, int N, int K);
+
+/* src/quant/awq_repack.c:261-310 (vv_int4g_to_gpu_layout): row-major INT4G
+ * codes to the layout the accelerator kernels read, in place: inside every
+ * 16-byte chunk (32 columns), nibble slot s of 32-bit word t holds column
+ * 2 (t + 4 (s % 4)) + s / 4; out_sz[n][g] = half2 {scale, (half)zero}. */
+int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
+                            int N, int K, int G, uint16_t* out_sz);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

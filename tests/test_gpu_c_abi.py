@@ -95,3 +95,25 @@ def test_reference_own_kv_pool_test_passes_on_this_backend():
     print(res.stdout[-3000:], res.stderr[-2000:])
     assert res.returncode == 0, res.stdout[-3000:]
     assert "PASS" in res.stdout and "FAIL" not in res.stdout and "SKIP" not in res.stdout
+
+
+INT8_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_int8_linear_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(INT8_EXE),
+                    reason="oracle/_ref/test_int8_linear_hip not built (needs the reference tree)")
+def test_reference_own_int8_linear_test_passes_on_this_backend():
+    """The reference's tests/test_int8_linear.c: its CPU quantiser and linear
+    kernels, then this backend's activation quantisers (plain and fused, four
+    orders, bit for bit against the CPU quantiser), column absmax, and the W8A8
+    / W4A8 linear layers on every kernel family (exact integers with unit
+    scales, FP16 outputs with bias and an aliased residual, shared-input
+    launches)."""
+    res = subprocess.run([INT8_EXE], capture_output=True, text=True, timeout=280)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "FAIL" not in res.stdout and "SKIPPED" not in res.stdout
+    last = res.stdout.strip().splitlines()[-1]
+    done, total = last.strip("= ").split()[0].split("/")
+    assert done == total and int(total) >= 1600, last

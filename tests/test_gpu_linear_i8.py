@@ -204,8 +204,7 @@ def test_i8_linear_multi_equals_single_calls(M):
     ok(call(0, 0, 3))
     for (_, _, _, d_y), want in zip(keep, wants):
         assert np.array_equal(bits_of(d_y), want)
-    assert call(0, 1, 3) == dev.VV_ERR_UNSUPPORTED       # W4A8
-    assert call(1, 0, 3) == dev.VV_ERR_UNSUPPORTED       # a layout only W4A8 reads
+    assert call(1, 0, 3) == dev.VV_ERR_UNSUPPORTED       # W8A8 reads column order only
     assert call(0, 0, 0) == dev.VV_ERR_INVALID_ARG
     assert dev.vv_i8_linear_multi_dev(None, 0, d_sx.data_ptr(), None, 0, C.addressof(projs), 3, 0, M, K,
                                       stream()) == dev.VV_ERR_NULL_PTR
@@ -229,3 +228,161 @@ def test_w8a8_argument_checks_launch_nothing():
     assert f(X, S, W, SW, None, None, Y, 0, 9, N, K, GEMV, stream()) == dev.VV_ERR_UNSUPPORTED
     torch.cuda.synchronize()
     assert (d_y == 7.0).all()
+
+
+# ── W4A8 ────────────────────────────────────────────────────────────────────
+
+L_GEMV, L_MMA = 2, 3        # VV_Q8_W4_GEMV, VV_Q8_W4_MMA
+
+
+def w4_problem(M, N, K, G, seed, unit=False):
+    """Activations quantised by the oracle in column order and in both
+    accelerator orders; codes, FP16 group scales and zero points; the codes in
+    the accelerator layout with their half2 {scale, zero} table."""
+    rng = np.random.default_rng(seed)
+    x = rng.normal(size=(M, K)).astype(np.float32) * 3
+    xq, sx, _ = oracle.quant_act_q8(x, 0, want_xsum=False)
+    orders = {lay: oracle.quant_act_q8(x, lay, want_xsum=False)[0] for lay in (L_GEMV, L_MMA)}
+    packed = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    zeros = rng.integers(0, 16, (N, K // G), dtype=np.uint8)
+    if unit:
+        scales = np.full((N, K // G), 0x3C00, np.uint16)
+        sx = np.ones(M, np.float32)
+    else:
+        scales = rng.uniform(0.002, 0.022, (N, K // G)).astype(np.float16).view(np.uint16)
+    gpu, sz = oracle.int4g_to_gpu_layout(packed, scales, zeros, G)
+    bias = oracle.normal_f16((N,), seed + 1, std=0.5)
+    res = oracle.normal_f16((M, N), seed + 2, std=2.0)
+    return dict(xq=xq, sx=sx, orders=orders, packed=packed, scales=scales, zeros=zeros, gpu=gpu, sz=sz,
+                bias=bias, res=res, G=G)
+
+
+def run_w4(p, layout, bias=False, res=False, f32=False, path=AUTO, alias=False, expect=None):
+    M, K = p["xq"].shape
+    N = p["packed"].shape[0]
+    d_xq, d_sx = i8_dev(p["orders"].get(layout, p["xq"])), i8_dev(p["sx"])
+    d_w, d_sz = i8_dev(p["gpu"]), i8_dev(p["sz"])
+    d_b = to_dev(p["bias"]) if bias else None
+    d_r = to_dev(p["res"]) if res else None
+    if alias:
+        d_y = d_r
+    else:
+        d_y = torch.full((M, N), float("nan"), dtype=torch.float32 if f32 else torch.float16, device="cuda")
+    st = dev.vv_w4a8_linear_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), None, d_w.data_ptr(), d_sz.data_ptr(),
+                                p["G"], d_b.data_ptr() if bias else None, d_r.data_ptr() if res else None,
+                                d_y.data_ptr(), 1 if f32 else 0, M, N, K, path, stream())
+    if expect is not None:
+        assert st == expect, st
+        return None
+    ok(st)
+    torch.cuda.synchronize()
+    return d_y.cpu().numpy() if f32 else bits_of(d_y)
+
+
+def want_w4(p, bias=False, res=False):
+    return oracle.w4a8_linear(p["xq"], p["sx"], p["packed"], p["scales"], p["zeros"], p["G"],
+                              p["bias"] if bias else None, p["res"] if res else None)
+
+
+W4_SHAPES = [(1, 64, 32, 32), (1, 3584, 3584, 128), (1, 512, 18944, 128), (2, 77, 256, 256), (5, 136, 640, 32),
+             (8, 300, 640, 64), (8, 64, 1024, 512), (9, 64, 64, 32), (16, 30, 96, 32), (17, 77, 256, 256),
+             (33, 136, 640, 32), (64, 300, 640, 64), (65, 64, 1024, 512), (100, 130, 160, 32), (130, 101, 224, 32),
+             (285, 3584, 3584, 128), (300, 4608, 1536, 128), (921, 512, 3584, 128)]
+
+
+@pytest.mark.parametrize("M,N,K,G", W4_SHAPES)
+def test_w4a8_bit_exact_against_oracle(M, N, K, G):
+    """Both kernel families (the GEMV where it serves the shape) give the
+    oracle's FP32 bits and their correctly rounded FP16."""
+    p = w4_problem(M, N, K, G, 3 * M + N)
+    want32, want16 = want_w4(p, True, True)
+    plain32, _ = want_w4(p)
+    layouts = (L_GEMV, L_MMA) if M <= 8 else (L_MMA,)
+    for lay in layouts:
+        same_f32(run_w4(p, lay, True, True, f32=True), want32, f"f32 layout {lay}")
+        assert np.array_equal(run_w4(p, lay, True, True), want16), f"f16 layout {lay}"
+        same_f32(run_w4(p, lay, f32=True), plain32, f"f32 plain layout {lay}")
+
+
+@pytest.mark.parametrize("M,N,K,G", [(1, 256, 3584, 128), (7, 300, 640, 64), (40, 136, 640, 32), (300, 264, 1024, 512)])
+def test_w4a8_unit_scales_give_the_exact_integer(M, N, K, G):
+    """With every scale 1 the FP32 output is sum_k (q - z) x itself."""
+    p = w4_problem(M, N, K, G, 70 + M, unit=True)
+    codes = np.empty((N, K), np.int64)
+    codes[:, 0::2], codes[:, 1::2] = p["packed"] >> 4, p["packed"] & 15
+    codes -= np.repeat(p["zeros"].astype(np.int64), G, axis=1)
+    exact = p["xq"].astype(np.int64) @ codes.T
+    assert np.abs(exact).max() < 2 ** 24
+    for lay in ((L_GEMV, L_MMA) if M <= 8 else (L_MMA,)):
+        assert np.array_equal(run_w4(p, lay, f32=True).astype(np.int64), exact)
+
+
+@pytest.mark.parametrize("M,layout", [(3, L_GEMV), (3, L_MMA), (200, L_MMA)])
+def test_w4a8_residual_may_alias_output(M, layout):
+    p = w4_problem(M, 264, 512, 128, 40 + M)
+    _, want16 = want_w4(p, True, True)
+    assert np.array_equal(run_w4(p, layout, True, True, alias=True), want16)
+
+
+def test_w4a8_paths_and_layouts():
+    """AUTO follows the layout; a family asked for with the other family's
+    layout, or the GEMV beyond eight rows, declines."""
+    p = w4_problem(4, 96, 256, 64, 9)
+    want32, _ = want_w4(p)
+    same_f32(run_w4(p, L_GEMV, f32=True, path=GEMV), want32, "gemv")
+    for path in (MMA, SIMT):
+        same_f32(run_w4(p, L_MMA, f32=True, path=path), want32, f"path {path}")
+        run_w4(p, L_GEMV, path=path, expect=dev.VV_ERR_UNSUPPORTED)
+    run_w4(p, L_MMA, path=GEMV, expect=dev.VV_ERR_UNSUPPORTED)
+    run_w4(p, 0, expect=dev.VV_ERR_INVALID_ARG)
+    run_w4(p, 1, expect=dev.VV_ERR_INVALID_ARG)
+    run_w4(p, L_MMA, path=4, expect=dev.VV_ERR_INVALID_ARG)
+    big = w4_problem(9, 64, 64, 32, 10)
+    run_w4(big, L_GEMV, expect=dev.VV_ERR_UNSUPPORTED)
+    bad_group = dict(p, G=48)
+    run_w4(bad_group, L_MMA, expect=dev.VV_ERR_UNSUPPORTED)
+    assert dev.vv_w4a8_linear_dev(None, L_MMA, None, None, None, None, 64, None, None, None, 0, 4, 96, 256, 0,
+                                  stream()) == dev.VV_ERR_NULL_PTR
+
+
+def test_w4a8_follows_the_device_quantiser():
+    """vv_act_quant_dev in each accelerator order feeds the kernel that reads it."""
+    M, N, K, G = 6, 512, 3584, 128
+    p = w4_problem(M, N, K, G, 21)
+    x = oracle.normal_f16((M, K), 5, std=2.0)
+    xq, sx, _ = oracle.quant_act_q8(oracle.widen(x), 0, want_xsum=False)
+    want32, _ = oracle.w4a8_linear(xq, sx, p["packed"], p["scales"], p["zeros"], G)
+    d_x, d_w, d_sz = to_dev(x), i8_dev(p["gpu"]), i8_dev(p["sz"])
+    for lay in (L_GEMV, L_MMA):
+        d_xq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+        d_sx = torch.empty(M, dtype=torch.float32, device="cuda")
+        d_xs = torch.empty((M, K // 32), dtype=torch.int32, device="cuda")
+        d_y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        ok(dev.vv_act_quant_dev(d_x.data_ptr(), M, K, lay, d_xq.data_ptr(), d_sx.data_ptr(), d_xs.data_ptr(),
+                                stream()))
+        ok(dev.vv_w4a8_linear_dev(d_xq.data_ptr(), lay, d_sx.data_ptr(), d_xs.data_ptr(), d_w.data_ptr(),
+                                  d_sz.data_ptr(), G, None, None, d_y.data_ptr(), 1, M, N, K, AUTO, stream()))
+        torch.cuda.synchronize()
+        same_f32(d_y.cpu().numpy(), want32, f"layout {lay}")
+
+
+@pytest.mark.parametrize("M,layout", [(2, L_GEMV), (40, L_MMA)])
+def test_i8_linear_multi_w4(M, layout):
+    K, G = 512, 128
+    base = w4_problem(M, 8, K, G, 80 + M)
+    d_xq, d_sx = i8_dev(base["orders"][layout]), i8_dev(base["sx"])
+    keep, projs, wants = [], (dev.I8Proj * 3)(), []
+    for i, N in enumerate((512, 128, 136)):
+        p = w4_problem(M, N, K, G, 90 + i)
+        d_w, d_sz = i8_dev(p["gpu"]), i8_dev(p["sz"])
+        d_b = to_dev(p["bias"]) if i != 1 else None
+        d_y = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        keep.append((d_w, d_sz, d_b, d_y))
+        projs[i] = dev.I8Proj(d_w.data_ptr(), None, d_sz.data_ptr(), d_b.data_ptr() if d_b is not None else None,
+                              d_y.data_ptr(), N)
+        wants.append(oracle.w4a8_linear(base["xq"], base["sx"], p["packed"], p["scales"], p["zeros"], G,
+                                        p["bias"] if i != 1 else None)[1])
+    ok(dev.vv_i8_linear_multi_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), None, 1, C.addressof(projs), 3, G,
+                                  M, K, stream()))
+    for (_, _, _, d_y), want in zip(keep, wants):
+        assert np.array_equal(bits_of(d_y), want)

@@ -136,3 +136,107 @@ def test_w8a8_linear_against_integer_closed_form_and_reference():
                                                sw.ctypes.data_as(f32p), bias.ctypes.data,
                                                out.ctypes.data_as(f32p), M, N, K) == 0
             assert np.array_equal(out, with_b)
+
+
+def int4_problem(N, K, G, seed, unit=False):
+    rng = np.random.default_rng(seed)
+    packed = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    zeros = rng.integers(0, 16, (N, K // G), dtype=np.uint8)
+    if unit:
+        scales = np.full((N, K // G), 0x3C00, np.uint16)
+    else:
+        scales = rng.uniform(0.002, 0.022, (N, K // G)).astype(np.float16).view(np.uint16)
+    return packed, scales, zeros
+
+
+def int4_codes(packed):
+    """[N,K/2] row-major INT4G bytes -> [N,K] codes (high nibble = even column)."""
+    out = np.empty((packed.shape[0], packed.shape[1] * 2), np.int64)
+    out[:, 0::2], out[:, 1::2] = packed >> 4, packed & 15
+    return out
+
+
+def test_w4a8_linear_against_closed_form_and_reference():
+    """Integer part: an int64 matmul of (q - z) per group. With unit scales the
+    FP32 output is that integer exactly (and so is the compiled reference's,
+    whichever instruction set it picked); with real scales the groups are
+    added in order in FP32, checked against float64 to the worst case of that
+    many roundings ((groups + 2) * 2^-24 of the sum of magnitudes). The
+    compiled reference's vector kernels scale partial sums of q x and z x
+    separately, so they agree to the same count of roundings of THOSE
+    magnitudes (sum_k s (q + z) |x|), no closer."""
+    import ctypes as C
+    rng = np.random.default_rng(8)
+    f32p, i32p = C.POINTER(C.c_float), C.POINTER(C.c_int32)
+    for M, N, K, G in ((1, 16, 64, 32), (5, 40, 3584, 128), (9, 33, 1024, 512), (4, 24, 256, 256)):
+        x = rng.normal(size=(M, K)).astype(np.float32) * 3
+        xq, sx, xs = oracle.quant_act_q8(x, 0)
+        xq_nib, _, _ = oracle.quant_act_q8(x, 1)
+        ng = K // G
+        for unit in (True, False):
+            packed, scales, zeros = int4_problem(N, K, G, 11 + N, unit)
+            d = int4_codes(packed).reshape(N, ng, G) - zeros[:, :, None].astype(np.int64)
+            per_group = np.einsum("mgk,ngk->mng", xq.astype(np.int64).reshape(M, ng, G), d)
+            s = oracle.widen(scales).astype(np.float64)
+            one = np.ones(M, np.float32)
+            got, _ = oracle.w4a8_linear(xq, one if unit else sx, packed, scales, zeros, G)
+            exact = (per_group * s[None]).sum(-1) * (1.0 if unit else sx[:, None].astype(np.float64))
+            mag = (np.abs(per_group) * s[None]).sum(-1) * (1.0 if unit else sx[:, None])
+            bar = (ng + 2) * 2.0 ** -24 * mag + 1e-30
+            if unit:
+                assert np.abs(exact).max() < 2 ** 24 and np.array_equal(got.astype(np.float64), exact)
+            else:
+                assert np.max(np.abs(got - exact) / bar) <= 1.0
+            if oracle.ref is not None and hasattr(oracle.ref, "vv_w4a8_gemm_cpu"):
+                out = np.empty((M, N), np.float32)
+                sxu = one if unit else sx
+                assert oracle.ref.vv_w4a8_gemm_cpu(xq_nib.ctypes.data, sxu.ctypes.data_as(f32p),
+                                                   xs.ctypes.data_as(i32p), packed.ctypes.data, scales.ctypes.data,
+                                                   zeros.ctypes.data, G, None, out.ctypes.data_as(f32p),
+                                                   M, N, K) == 0
+                if unit:
+                    assert np.array_equal(out, got)
+                else:
+                    qz = int4_codes(packed).reshape(N, ng, G) + zeros[:, :, None].astype(np.int64)
+                    loose = np.einsum("mgk,ngk->mng", np.abs(xq.astype(np.int64)).reshape(M, ng, G), qz)
+                    loose = (loose * s[None]).sum(-1) * sx[:, None]
+                    assert np.max(np.abs(out - got) / ((ng + 2) * 2.0 ** -24 * loose)) <= 1.0
+        bias = oracle.normal_f16((N,), 3, std=0.5)
+        res = oracle.normal_f16((M, N), 4)
+        plain, _ = oracle.w4a8_linear(xq, sx, packed, scales, zeros, G)
+        f32, f16 = oracle.w4a8_linear(xq, sx, packed, scales, zeros, G, bias, res)
+        assert np.array_equal(f32, (plain + oracle.widen(bias)[None, :]) + oracle.widen(res))
+        assert np.array_equal(f16, f32.astype(np.float16).view(np.uint16))
+
+
+def test_int4_gpu_layout_against_reference_and_the_activation_orders():
+    """The converter against the compiled reference byte for byte, and against
+    what the layout is for: reading word t of a chunk as `w & 0x0F0F0F0F` /
+    `(w >> 4) & 0x0F0F0F0F` next to activations in VV_Q8_W4_GEMV order, or as
+    its low / high 16 bits next to VV_Q8_W4_MMA order, gives the same integer
+    dot as codes and activations both in column order."""
+    N, K, G = 12, 256, 64
+    packed, scales, zeros = int4_problem(N, K, G, 2)
+    gpu, sz = oracle.int4g_to_gpu_layout(packed, scales, zeros, G)
+    assert np.array_equal(sz[:, :, 0], scales)
+    assert np.array_equal(oracle.widen(sz[:, :, 1]), zeros.astype(np.float32))
+    if oracle.ref is not None and hasattr(oracle.ref, "vv_int4g_to_gpu_layout"):
+        theirs, their_sz = packed.copy(), np.empty_like(sz)
+        assert oracle.ref.vv_int4g_to_gpu_layout(theirs.ctypes.data, scales.ctypes.data, zeros.ctypes.data,
+                                                 N, K, G, their_sz.ctypes.data) == 0
+        assert np.array_equal(theirs, gpu) and np.array_equal(their_sz, sz)
+    x = np.random.default_rng(3).normal(size=(3, K)).astype(np.float32)
+    nat, _, _ = oracle.quant_act_q8(x, 0)
+    gemv, _, _ = oracle.quant_act_q8(x, 2)
+    mma, _, _ = oracle.quant_act_q8(x, 3)
+    want = nat.astype(np.int64) @ int4_codes(packed).T
+    words = gpu.reshape(N, K // 32, 4, 4).astype(np.uint32)
+    words = words[..., 0] | words[..., 1] << 8 | words[..., 2] << 16 | words[..., 3] << 24      # [N, chunk, t]
+    nib = np.stack([(words >> (4 * s)) & 15 for s in range(8)], axis=-1).astype(np.int64)    # [N, chunk, t, slot]
+    # GEMV order: positions 8t..8t+3 meet slots 0,2,4,6 and 8t+4..8t+7 slots 1,3,5,7
+    by_gemv = np.concatenate([nib[..., 0::2], nib[..., 1::2]], axis=-1).reshape(N, K)
+    assert np.array_equal(gemv.astype(np.int64) @ by_gemv.T, want)
+    # MMA order: positions 4t..4t+3 meet slots 0..3, positions 16+4t.. slots 4..7
+    by_mma = np.concatenate([nib[..., :4].reshape(N, K // 32, 16), nib[..., 4:].reshape(N, K // 32, 16)],
+                            axis=-1).reshape(N, K)
+    assert np.array_equal(mma.astype(np.int64) @ by_mma.T, want)

@@ -237,24 +237,21 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
     return vv::launch_status();
 }
 
-/* W8A8 only (w4 == 0), activations in natural column order: one
- * vv_w8a8_linear_dev per projection, so each is computed exactly as that call
- * would. W4A8: declined. */
+/* One linear call per projection, so each is computed exactly as
+ * vv_w8a8_linear_dev / vv_w4a8_linear_dev would. */
 vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
                                    int w4, const vv_i8_proj_t* projs, int n, int group_size, int M,
                                    int K, void* stream) {
-    (void)xsum; (void)group_size;
     if (!xq || !sx || !projs) return VV_ERR_NULL_PTR;
     if (n < 1) return VV_ERR_INVALID_ARG;
-    if (w4 != 0 || x_layout != 0) return VV_ERR_UNSUPPORTED;
+    if (!w4 && x_layout != 0) return VV_ERR_UNSUPPORTED;   // W8A8 reads column order
     for (int i = 0; i < n; ++i) {
-        if (!projs[i].w || !projs[i].sw || !projs[i].y) return VV_ERR_NULL_PTR;
-        if (K % 16 != 0 || !vv::aligned16(projs[i].w)) return VV_ERR_UNSUPPORTED;
-    }
-    for (int i = 0; i < n; ++i) {
-        const vv_status_t s = vv_w8a8_linear_dev(xq, sx, static_cast<const int8_t*>(projs[i].w),
-                                                 static_cast<const float*>(projs[i].sw), projs[i].bias,
-                                                 nullptr, projs[i].y, 0, M, projs[i].N, K, 0, stream);
+        const vv_i8_proj_t& q = projs[i];
+        const vv_status_t s =
+            w4 ? vv_w4a8_linear_dev(xq, x_layout, sx, xsum, q.w, q.sz, group_size, q.bias, nullptr, q.y, 0,
+                                    M, q.N, K, 0, stream)
+               : vv_w8a8_linear_dev(xq, sx, static_cast<const int8_t*>(q.w), static_cast<const float*>(q.sw),
+                                    q.bias, nullptr, q.y, 0, M, q.N, K, 0, stream);
         if (s != VV_OK) return s;
     }
     return VV_OK;

@@ -1,0 +1,394 @@
+// W4A8 linear layers: y[m,n] = sx[m] * sum_g s[n,g] * sum_{k in g} (q[n,k] - z[n,g]) xq[m,k]
+// + bias[n] + residual[m,n]: int8 activations with per-row scales, 4-bit weight
+// codes with an FP16 scale and an integer zero point per group of G columns.
+//
+// The codes arrive in the accelerator layout of the INT4 weights: every 16-byte
+// chunk holds 32 consecutive columns, nibble slot s of 32-bit word t being
+// column 2 (t + 4 (s % 4)) + s / 4. The activations arrive permuted inside
+// every run of 32 columns so that the codes unpack with masks alone:
+//   VV_Q8_W4_GEMV  bytes 8t..8t+3 meet slots 0,2,4,6 (w & 0x0F0F0F0F), bytes
+//                  8t+4..8t+7 slots 1,3,5,7 ((w >> 4) & 0x0F0F0F0F)
+//   VV_Q8_W4_MMA   bytes 4t..4t+3 meet slots 0..3, bytes 16+4t.. slots 4..7, so
+//                  a chunk unpacks into the two 16-byte operands of one
+//                  v_mfma_i32_32x32x32_i8 step
+// Either way the zero point is taken off the unpacked bytes (q - z fits int8),
+// the per-group sums are exact int32, and the groups are added in order in
+// FP32 with nothing fused: acc += s_g * (float)sum_g, then acc * sx[m], + bias,
+// + residual. That is the CPU kernel's scalar form (src/cpu/cpu_int8.c:212-233,
+// 537-541), so every path and tile shape gives the same bits.
+#include "mfma_tile.hpp"
+
+namespace vv {
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kLayoutGemv = 2, kLayoutMma = 3;   // VV_Q8_W4_GEMV, VV_Q8_W4_MMA (q8.h:31-43)
+
+struct W4Args {
+    const int8_t* xq;
+    const float* sx;
+    const uint32_t* packed;   // [N][K/8] words
+    const uint32_t* sz;       // [N][K/G] half2 {scale, zero}
+    const h16* bias;
+    const h16* res;
+    void* y;
+    int y_f32, M, N, K, G, vec;
+};
+
+__device__ __forceinline__ float sz_scale(uint32_t sz) {
+    return (float)__builtin_bit_cast(h16, (uint16_t)(sz & 0xFFFFu));
+}
+// The zero point replicated into four bytes.
+__device__ __forceinline__ uint32_t sz_zero4(uint32_t sz) {
+    return (uint32_t)(int)(float)__builtin_bit_cast(h16, (uint16_t)(sz >> 16)) * 0x01010101u;
+}
+// Four codes 0..15 in the bytes of `codes`, minus the zero point, as int8:
+// 0x80 + q - z never borrows from the next byte, and flipping the top bit of
+// 0x80 + d is d in two's complement for -15 <= d <= 15.
+__device__ __forceinline__ uint32_t minus_zero(uint32_t codes, uint32_t z4) {
+    return ((codes | 0x80808080u) - z4) ^ 0x80808080u;
+}
+
+__device__ __forceinline__ float w4_value(float acc, float sxm, bool has_b, float b, bool has_r, float r) {
+#pragma clang fp contract(off)
+    float v = acc * sxm;
+    if (has_b) v = v + b;
+    if (has_r) v = v + r;
+    return v;
+}
+
+__device__ __forceinline__ void w4_store1(const W4Args& o, int m, int n, float acc) {
+    const size_t idx = (size_t)m * o.N + n;
+    const float v = w4_value(acc, o.sx[m], o.bias != nullptr, o.bias ? (float)o.bias[n] : 0.0f,
+                             o.res != nullptr, o.res ? (float)o.res[idx] : 0.0f);
+    if (o.y_f32) static_cast<float*>(o.y)[idx] = v;
+    else static_cast<h16*>(o.y)[idx] = to_half(v);
+}
+
+__device__ __forceinline__ void w4_store4(const W4Args& o, int m, int n, const float (&acc)[4]) {
+    if (o.vec && n + 3 < o.N) {
+        const size_t idx = (size_t)m * o.N + n;
+        const float sxm = o.sx[m];
+        h16x4 b = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+        if (o.bias) b = *reinterpret_cast<const h16x4*>(o.bias + n);
+        if (o.res) r = *reinterpret_cast<const h16x4*>(o.res + idx);
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = w4_value(acc[i], sxm, o.bias != nullptr, (float)b[i], o.res != nullptr, (float)r[i]);
+        if (o.y_f32) {
+            *reinterpret_cast<f32x4*>(static_cast<float*>(o.y) + idx) = v;
+        } else {
+            h16x4 h;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[i] = to_half(v[i]);
+            *reinterpret_cast<h16x4*>(static_cast<h16*>(o.y) + idx) = h;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n + i < o.N) w4_store1(o, m, n + i, acc[i]);
+    }
+}
+
+// ── M <= 8: one workgroup per weight row ───────────────────────────────────
+// Every thread takes whole 32-column chunks (16 bytes of codes against 32
+// bytes of each activation row) and leaves the chunk's exact sums in LDS; the
+// group sums are scaled in parallel, and one thread per activation row adds
+// the groups in order.
+constexpr int kGemvMaxChunks = 640;    // K <= 20480
+
+template <int MR>
+__global__ __launch_bounds__(kBlock) void w4a8_gemv(W4Args a) {
+    __shared__ int chunk_sum[MR][kGemvMaxChunks];
+    __shared__ float group_term[MR][kGemvMaxChunks];
+    const int tid = (int)threadIdx.x;
+    const int n = (int)blockIdx.x;
+    const int nchunks = a.K / 32, ng = a.K / a.G, per_group = a.G / 32;
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(a.packed + (size_t)n * (a.K / 8));
+    const uint32_t* szrow = a.sz + (size_t)n * ng;
+    for (int c = tid; c < nchunks; c += kBlock) {
+        const u32x4 w = __builtin_nontemporal_load(wrow + c);
+        const uint32_t z4 = sz_zero4(szrow[c / per_group]);
+        int wq[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            wq[2 * t] = (int)minus_zero(w[t] & 0x0F0F0F0Fu, z4);
+            wq[2 * t + 1] = (int)minus_zero((w[t] >> 4) & 0x0F0F0F0Fu, z4);
+        }
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            if (m < a.M) {
+                const i32x4* xr = reinterpret_cast<const i32x4*>(a.xq + (size_t)m * a.K) + 2 * c;
+                const i32x4 x0 = xr[0], x1 = xr[1];
+                int d = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    d = __builtin_amdgcn_sdot4(x0[i], wq[i], d, false);
+                    d = __builtin_amdgcn_sdot4(x1[i], wq[4 + i], d, false);
+                }
+                chunk_sum[m][c] = d;
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < a.M * ng; idx += kBlock) {
+        const int m = idx / ng, g = idx - m * ng;
+        int d = 0;
+        for (int j = 0; j < per_group; ++j) d += chunk_sum[m][g * per_group + j];
+        group_term[m][g] = sz_scale(szrow[g]) * (float)d;
+    }
+    __syncthreads();
+    if (tid < a.M) {
+        float acc = 0.0f;
+        for (int g = 0; g < ng; ++g) acc = acc + group_term[tid][g];
+        w4_store1(a, tid, n, acc);
+    }
+}
+
+// ── larger M: LDS-tiled int8 MFMA over codes unpacked on their way into LDS ─
+// Slabs of 64 columns (two MFMA steps = two chunks of codes), double-buffered
+// through registers. A thread that stages chunk p of weight row n also leaves
+// that chunk's group scale in LDS; when a step ends a group, every int32
+// accumulator is scaled into its FP32 partner and cleared.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
+    constexpr int NT = WM * WN * kWave;
+    constexpr int kSlots = 4;                     // 16-byte slots per slab row
+    constexpr int kSteps = 2;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int LA = BM * kSlots / NT;          // activation loads per thread per slab
+    constexpr int kBLoads = BN * kSteps;          // code chunks per slab
+    constexpr int LB = (kBLoads + NT - 1) / NT;
+    static_assert(LA >= 1 && (BM * kSlots) % NT == 0, "activation loads divide over the threads");
+    static_assert(kBLoads % NT == 0 || LB == 1, "code loads: whole rounds, or one partial round");
+    constexpr int kASlots = BM * kSlots, kBSlots = BN * kSlots;
+    __shared__ u32x4 lds[2 * (kASlots + kBSlots)];
+    __shared__ float scales[2][kSteps][BN];
+
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int m_blk = (int)blockIdx.y * BM, n_blk = (int)blockIdx.x * BN;
+    const int nsteps = a.K / 32, nslabs = (nsteps + kSteps - 1) / kSteps;
+    const int per_group = a.G / 32, ng = a.K / a.G;
+
+    // activations: thread t's i-th load is row (t + i NT) / 4, slot t % 4
+    const int a_slot = tid % kSlots;
+    const int8_t* a_ptr[LA];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = min((tid + i * NT) / kSlots, a.M - 1 - m_blk);
+        a_ptr[i] = a.xq + (size_t)(m_blk + row) * a.K + a_slot * 16;
+    }
+    const int aw_row = tid / kSlots;
+    const int aw_idx = aw_row * kSlots + swz<32>(aw_row, a_slot);
+    // codes: load j is row (t + j NT) / 2, chunk (t % 2) of the slab
+    const int b_step = tid % kSteps;
+    const uint32_t* b_ptr[LB];
+    const uint32_t* z_ptr[LB];
+    int b_row[LB];
+#pragma unroll
+    for (int j = 0; j < LB; ++j) {
+        b_row[j] = (tid + j * NT) / kSteps;
+        const int row = min(b_row[j], a.N - 1 - n_blk);
+        b_ptr[j] = a.packed + (size_t)(n_blk + row) * (a.K / 8) + b_step * 4;
+        z_ptr[j] = a.sz + (size_t)(n_blk + row) * ng;
+    }
+    const bool b_active = kBLoads % NT == 0 || tid < kBLoads;
+
+    u32x4 ra[LA], rb[LB];
+    uint32_t rz[LB];
+    auto fetch = [&](int slab) {
+        const bool a_live = slab * kSlots + a_slot < a.K / 16;
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            if (a_live) ra[i] = *reinterpret_cast<const u32x4*>(a_ptr[i] + (size_t)slab * (kSlots * 16));
+        const int step = slab * kSteps + b_step;
+        if (b_active && step < nsteps) {
+#pragma unroll
+            for (int j = 0; j < LB; ++j) {
+                rb[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(b_ptr[j] + (size_t)slab * (kSteps * 4)));
+                rz[j] = z_ptr[j][step / per_group];
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+        u32x4* dst = lds + buf * (kASlots + kBSlots);
+#pragma unroll
+        for (int i = 0; i < LA; ++i) dst[aw_idx + i * NT] = ra[i];
+        if (b_active) {
+#pragma unroll
+            for (int j = 0; j < LB; ++j) {
+                const uint32_t z4 = sz_zero4(rz[j]);
+                u32x4 lo, hi;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint32_t even = rb[j][t] & 0x0F0F0F0Fu;           // slots 0,2,4,6
+                    const uint32_t odd = (rb[j][t] >> 4) & 0x0F0F0F0Fu;     // slots 1,3,5,7
+                    // v_perm_b32 picks bytes from {odd : even} (even = bytes 0..3): slots 0,1,2,3 / 4,5,6,7
+                    lo[t] = minus_zero(__builtin_amdgcn_perm(odd, even, 0x05010400u), z4);
+                    hi[t] = minus_zero(__builtin_amdgcn_perm(odd, even, 0x07030602u), z4);
+                }
+                const int row = b_row[j];
+                dst[kASlots + row * kSlots + swz<32>(row, 2 * b_step)] = lo;
+                dst[kASlots + row * kSlots + swz<32>(row, 2 * b_step + 1)] = hi;
+                scales[buf][b_step][row] = sz_scale(rz[j]);
+            }
+        }
+    };
+
+    i32x16 acc[TN][TM];
+    f32x16 facc[TN][TM];
+#pragma unroll
+    for (int x = 0; x < TN; ++x)
+#pragma unroll
+        for (int y = 0; y < TM; ++y)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { acc[x][y][r] = 0; facc[x][y][r] = 0.0f; }
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    int f_idx[kSteps];
+#pragma unroll
+    for (int step = 0; step < kSteps; ++step)
+        f_idx[step] = frow * kSlots + swz<32>(frow, step * 2 + fhalf);
+    const int fa_base = wm * TM * 32 * kSlots;
+    const int fb_base = kASlots + wn * TN * 32 * kSlots;
+    int until_flush = per_group;
+
+    auto compute = [&](int buf, int slab) {
+        const u32x4* src = lds + buf * (kASlots + kBSlots);
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+            if (slab * kSteps + step >= nsteps) break;
+            u32x4 fw[TN], fx[TM];
+#pragma unroll
+            for (int x = 0; x < TN; ++x) fw[x] = src[fb_base + x * 32 * kSlots + f_idx[step]];
+#pragma unroll
+            for (int y = 0; y < TM; ++y) fx[y] = src[fa_base + y * 32 * kSlots + f_idx[step]];
+#pragma unroll
+            for (int x = 0; x < TN; ++x)
+#pragma unroll
+                for (int y = 0; y < TM; ++y)
+                    acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fw[x]),
+                                                                      __builtin_bit_cast(i32x4, fx[y]),
+                                                                      acc[x][y], 0, 0, 0);
+            if (--until_flush == 0) {
+                until_flush = per_group;
+                const float* sc = &scales[buf][step][wn * TN * 32 + 4 * fhalf];
+#pragma unroll
+                for (int x = 0; x < TN; ++x)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 s = *reinterpret_cast<const f32x4*>(sc + x * 32 + 8 * g);
+#pragma unroll
+                        for (int y = 0; y < TM; ++y)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+#pragma clang fp contract(off)
+                                const float term = s[r] * (float)acc[x][y][4 * g + r];
+                                facc[x][y][4 * g + r] = facc[x][y][4 * g + r] + term;
+                                acc[x][y][4 * g + r] = 0;
+                            }
+                    }
+            }
+        }
+    };
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (int slab = 0; slab < nslabs; ++slab) {
+        const int buf = slab & 1;
+        if (slab + 1 < nslabs) fetch(slab + 1);
+        compute(buf, slab);
+        if (slab + 1 < nslabs) stage(buf ^ 1);
+        __syncthreads();
+    }
+
+    const int m0 = m_blk + wm * TM * 32, n0 = n_blk + wn * TN * 32;
+#pragma unroll
+    for (int y = 0; y < TM; ++y) {
+        const int m = m0 + y * 32 + frow;
+        if (m >= a.M) continue;
+#pragma unroll
+        for (int x = 0; x < TN; ++x)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + x * 32 + 8 * g + 4 * fhalf;
+                if (n >= a.N) continue;
+                const float t[4] = {facc[x][y][4 * g], facc[x][y][4 * g + 1], facc[x][y][4 * g + 2],
+                                    facc[x][y][4 * g + 3]};
+                w4_store4(a, m, n, t);
+            }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+void launch_w4_tile(const W4Args& a, hipStream_t st) {
+    const dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM));
+    w4a8_tile<BM, BN, WM, WN><<<grid, WM * WN * kWave, 0, st>>>(a);
+}
+
+enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
+                               const void* packed, const void* sz, int group_size, const void* bias,
+                               const void* residual, void* y, int y_f32, int M, int N, int K, int path,
+                               void* stream) {
+    (void)xsum;   // the zero points are taken off the unpacked codes, so the per-32 sums are not needed
+    if (!xq || !sx || !packed || !sz || !y) return VV_ERR_NULL_PTR;
+    if (x_layout != vv::kLayoutGemv && x_layout != vv::kLayoutMma) return VV_ERR_INVALID_ARG;
+    if (M <= 0 || N <= 0 || K <= 0 || path < vv::kPathAuto || path > vv::kPathSimt)
+        return VV_ERR_INVALID_ARG;
+    if (K % 32 != 0 || group_size <= 0 || group_size % 32 != 0 || K % group_size != 0)
+        return VV_ERR_UNSUPPORTED;
+    if (!vv::aligned16(xq) || !vv::aligned16(packed) || (reinterpret_cast<uintptr_t>(sz) & 3u))
+        return VV_ERR_UNSUPPORTED;
+    if (path == vv::kPathAuto) path = x_layout == vv::kLayoutGemv ? vv::kPathGemv : vv::kPathMma;
+    // Each kernel family reads one order of the activations.
+    if ((path == vv::kPathGemv) != (x_layout == vv::kLayoutGemv)) return VV_ERR_UNSUPPORTED;
+    if (path == vv::kPathGemv && (M > 8 || K / 32 > vv::kGemvMaxChunks)) return VV_ERR_UNSUPPORTED;
+
+    hipStream_t st = vv::as_stream(stream);
+    vv::W4Args a;
+    a.xq = xq;
+    a.sx = sx;
+    a.packed = static_cast<const uint32_t*>(packed);
+    a.sz = static_cast<const uint32_t*>(sz);
+    a.bias = static_cast<const vv::h16*>(bias);
+    a.res = static_cast<const vv::h16*>(residual);
+    a.y = y;
+    a.y_f32 = y_f32 ? 1 : 0;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = group_size;
+    const auto mis = [](const void* p, unsigned mask) { return p && (reinterpret_cast<uintptr_t>(p) & mask); };
+    a.vec = (N % 4 == 0) && !mis(bias, 7u) && !mis(residual, 7u) && !mis(y, y_f32 ? 15u : 7u);
+
+    if (path == vv::kPathGemv) {
+        const dim3 grid((unsigned)N);
+        if (M == 1) vv::w4a8_gemv<1><<<grid, vv::kBlock, 0, st>>>(a);
+        else if (M == 2) vv::w4a8_gemv<2><<<grid, vv::kBlock, 0, st>>>(a);
+        else if (M <= 4) vv::w4a8_gemv<4><<<grid, vv::kBlock, 0, st>>>(a);
+        else vv::w4a8_gemv<8><<<grid, vv::kBlock, 0, st>>>(a);
+        return vv::launch_status();
+    }
+    const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (M > 64 && wg128 >= 256) vv::launch_w4_tile<128, 128, 2, 2>(a, st);
+    else if (M > 32) vv::launch_w4_tile<64, 64, 2, 2>(a, st);
+    else vv::launch_w4_tile<32, 64, 1, 2>(a, st);
+    return vv::launch_status();
+}
+
+}  // extern "C"

@@ -9,7 +9,7 @@
  * src/metal/metal_stubs.c:1-30, src/device/device_none.c:129-483).
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
- * HIP library does not define (quantised-weight GEMM and GEMV, the small-M and
+ * HIP library does not define (weight-only quantised GEMM and GEMV, the small-M and
  * NN dense forms, quantised KV formats, VAE, BitNet). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
@@ -36,9 +36,6 @@ VV_DECLINE(vv_awq_gemv_dev)      VV_DECLINE(vv_awq_gemm_dev)      VV_DECLINE(vv_
 VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_dequant_int8_dev)
 VV_DECLINE(vv_w4a16_gemv_dev)    VV_DECLINE(vv_w4a16_gemv_multi_dev)
 VV_DECLINE(vv_w4a16_gather_dev)  VV_DECLINE(vv_w4a16_gemm_dev)    VV_DECLINE(vv_w4a16_dequant_dev)
-
-/* W4A8 linear (device.h:385-389); the activation quantisers and W8A8 are implemented */
-VV_DECLINE(vv_w4a8_linear_dev)
 
 /* dense FP16 GEMM: the NN form (device.h:477-479); the NT forms are implemented */
 VV_DECLINE(vv_gemm_fp16_nn_dev)

@@ -74,6 +74,7 @@ SIGNATURES = {
     "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
     "vv_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _vp]),
     "vv_w8a8_linear_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "vv_w4a8_linear_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_i8_linear_multi_dev": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "vv_gemv_swiglu_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "vv_gqa_decode_scratch_bytes": (C.c_size_t, [_i, _i]),
