@@ -291,6 +291,31 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del xq, sx, c
         del w8, sw
+    # And as W4A8: 4-bit codes with a scale and a zero point per 128 columns (any bytes are valid codes).
+    out["w4a8"], out["w4a8_gemv"] = {}, {}
+    G = 128
+    for name, n, k in shapes:
+        w4 = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
+        sz = torch.stack([torch.rand(n, k // G, device="cuda") * 0.02 + 0.002,
+                          torch.randint(0, 16, (n, k // G), device="cuda").float()], dim=-1).half().contiguous()
+        for m, key, layout in ((T, "w4a8", 3), (1, "w4a8_gemv", 2)):
+            xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+            sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
+            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+            xs = xq.view(m, k // 32, 32).sum(-1, dtype=torch.int32).contiguous()     # what the quantiser writes
+            sec = timed(lambda: dev.vv_w4a8_linear_dev(xq.data_ptr(), layout, sx.data_ptr(), xs.data_ptr(), w4.data_ptr(),
+                                                       sz.data_ptr(), G, None, None, c.data_ptr(), 0, m, n, k, 0,
+                                                       st), 5 if m > 1 else 50)
+            if m > 1:
+                tops = 2.0 * m * n * k / sec / 1e12
+                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TOPs": tops,
+                                  "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
+            else:
+                gb = (n * k / 2 + n * (k // G) * 4 + k + 2.0 * n) / sec / 1e9
+                out[key][name] = {"N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+            del xq, sx, c
+        del w4, sz
     q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
     k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
     v_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")

@@ -241,7 +241,7 @@ def w4_problem(M, N, K, G, seed, unit=False):
     the accelerator layout with their half2 {scale, zero} table."""
     rng = np.random.default_rng(seed)
     x = rng.normal(size=(M, K)).astype(np.float32) * 3
-    xq, sx, _ = oracle.quant_act_q8(x, 0, want_xsum=False)
+    xq, sx, xs = oracle.quant_act_q8(x, 0)
     orders = {lay: oracle.quant_act_q8(x, lay, want_xsum=False)[0] for lay in (L_GEMV, L_MMA)}
     packed = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
     zeros = rng.integers(0, 16, (N, K // G), dtype=np.uint8)
@@ -253,22 +253,24 @@ def w4_problem(M, N, K, G, seed, unit=False):
     gpu, sz = oracle.int4g_to_gpu_layout(packed, scales, zeros, G)
     bias = oracle.normal_f16((N,), seed + 1, std=0.5)
     res = oracle.normal_f16((M, N), seed + 2, std=2.0)
-    return dict(xq=xq, sx=sx, orders=orders, packed=packed, scales=scales, zeros=zeros, gpu=gpu, sz=sz,
+    return dict(xq=xq, sx=sx, xs=xs, orders=orders, packed=packed, scales=scales, zeros=zeros, gpu=gpu, sz=sz,
                 bias=bias, res=res, G=G)
 
 
-def run_w4(p, layout, bias=False, res=False, f32=False, path=AUTO, alias=False, expect=None):
+def run_w4(p, layout, bias=False, res=False, f32=False, path=AUTO, alias=False, expect=None, xsum=False):
     M, K = p["xq"].shape
     N = p["packed"].shape[0]
     d_xq, d_sx = i8_dev(p["orders"].get(layout, p["xq"])), i8_dev(p["sx"])
     d_w, d_sz = i8_dev(p["gpu"]), i8_dev(p["sz"])
     d_b = to_dev(p["bias"]) if bias else None
     d_r = to_dev(p["res"]) if res else None
+    d_xs = i8_dev(p["xs"]) if xsum else None
     if alias:
         d_y = d_r
     else:
         d_y = torch.full((M, N), float("nan"), dtype=torch.float32 if f32 else torch.float16, device="cuda")
-    st = dev.vv_w4a8_linear_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), None, d_w.data_ptr(), d_sz.data_ptr(),
+    st = dev.vv_w4a8_linear_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), d_xs.data_ptr() if xsum else None,
+                                d_w.data_ptr(), d_sz.data_ptr(),
                                 p["G"], d_b.data_ptr() if bias else None, d_r.data_ptr() if res else None,
                                 d_y.data_ptr(), 1 if f32 else 0, M, N, K, path, stream())
     if expect is not None:
@@ -284,7 +286,7 @@ def want_w4(p, bias=False, res=False):
                               p["bias"] if bias else None, p["res"] if res else None)
 
 
-W4_SHAPES = [(1, 64, 32, 32), (1, 3584, 3584, 128), (1, 512, 18944, 128), (2, 77, 256, 256), (5, 136, 640, 32),
+W4_SHAPES = [(1, 64, 32, 32), (3, 50, 192, 96), (1, 40, 8192, 4096), (8, 37, 18944, 32), (1, 18944, 3584, 128), (1, 3584, 3584, 128), (1, 512, 18944, 128), (2, 77, 256, 256), (5, 136, 640, 32),
              (8, 300, 640, 64), (8, 64, 1024, 512), (9, 64, 64, 32), (16, 30, 96, 32), (17, 77, 256, 256),
              (33, 136, 640, 32), (64, 300, 640, 64), (65, 64, 1024, 512), (100, 130, 160, 32), (130, 101, 224, 32),
              (285, 3584, 3584, 128), (300, 4608, 1536, 128), (921, 512, 3584, 128)]
@@ -302,6 +304,7 @@ def test_w4a8_bit_exact_against_oracle(M, N, K, G):
         same_f32(run_w4(p, lay, True, True, f32=True), want32, f"f32 layout {lay}")
         assert np.array_equal(run_w4(p, lay, True, True), want16), f"f16 layout {lay}"
         same_f32(run_w4(p, lay, f32=True), plain32, f"f32 plain layout {lay}")
+        same_f32(run_w4(p, lay, True, True, f32=True, xsum=True), want32, f"f32 layout {lay} with xsum")
 
 
 @pytest.mark.parametrize("M,N,K,G", [(1, 256, 3584, 128), (7, 300, 640, 64), (40, 136, 640, 32), (300, 264, 1024, 512)])

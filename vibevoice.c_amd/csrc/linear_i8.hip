@@ -120,57 +120,79 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
            (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
 }
 
-// M <= MR <= 8 rows: kSplit waves per weight row, each a contiguous 1/kSplit of K.
-template <int MR, int kSplit>
+// M <= MR <= 8 rows: kSplit waves per RW weight rows, each wave a contiguous
+// 1/kSplit of K. RW = 2 where a wave owns whole short rows: twice the bytes in
+// flight per wave, and the activation loads shared by both rows.
+template <int MR, int kSplit, int RW>
 __global__ __launch_bounds__(kBlock) void i8_gemv(const int8_t* __restrict__ xq,
                                                   const int8_t* __restrict__ w, I8Out out, int K) {
-    constexpr int kRows = kWavesPerBlock / kSplit;
-    __shared__ int part[kWavesPerBlock][MR];
+    constexpr int kSets = kWavesPerBlock / kSplit;
+    __shared__ int part[kWavesPerBlock][RW][MR];
     const int wave = wave_in_block(), lane = lane_id();
-    const int n = (int)blockIdx.x * kRows + wave / kSplit;
+    const int n0 = ((int)blockIdx.x * kSets + wave / kSplit) * RW;
     const int piece = wave % kSplit;
     const int kchunks = K / 16;
     const int per = (kchunks + kSplit - 1) / kSplit;
     const int begin = piece * per, end = min(kchunks, begin + per);
-    int acc[MR];
+    int acc[RW][MR];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = 0;
-    if (n < out.N) {
-        const i32x4* wr = reinterpret_cast<const i32x4*>(w + (size_t)n * K);
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0;
+    const i32x4* wr[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+        wr[r] = reinterpret_cast<const i32x4*>(w + (size_t)min(n0 + r, out.N - 1) * K);
+    if (n0 < out.N) {
 #pragma unroll 2
         for (int c = begin + lane; c < end; c += kWave) {
-            const i32x4 wv = __builtin_nontemporal_load(wr + c);
+            i32x4 wv[RW];
+#pragma unroll
+            for (int r = 0; r < RW; ++r) wv[r] = __builtin_nontemporal_load(wr[r] + c);
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
                 if (m < out.M) {
                     const i32x4 xv = *(reinterpret_cast<const i32x4*>(xq + (size_t)m * K) + c);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[m] = __builtin_amdgcn_sdot4(xv[i], wv[i], acc[m], false);
+                    for (int r = 0; r < RW; ++r)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[r][m] = __builtin_amdgcn_sdot4(xv[i], wv[r][i], acc[r][m], false);
                 }
             }
         }
     }
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = wave_sum_i32(acc[m]);
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = wave_sum_i32(acc[r][m]);
     if constexpr (kSplit > 1) {
         if (lane == 0) {
 #pragma unroll
-            for (int m = 0; m < MR; ++m) part[wave][m] = acc[m];
+            for (int r = 0; r < RW; ++r)
+#pragma unroll
+                for (int m = 0; m < MR; ++m) part[wave][r][m] = acc[r][m];
         }
         __syncthreads();
 #pragma unroll
-        for (int m = 0; m < MR; ++m) {
-            acc[m] = 0;
+        for (int r = 0; r < RW; ++r)
 #pragma unroll
-            for (int p = 0; p < kSplit; ++p) acc[m] += part[(wave / kSplit) * kSplit + p][m];
-        }
+            for (int m = 0; m < MR; ++m) {
+                acc[r][m] = 0;
+#pragma unroll
+                for (int p = 0; p < kSplit; ++p) acc[r][m] += part[(wave / kSplit) * kSplit + p][r][m];
+            }
     }
-    if (n < out.N && piece == 0) {
+    if (piece == 0) {
+        // lane r * MR + m stores row m of weight row n0 + r
         int mine = 0;
 #pragma unroll
-        for (int m = 0; m < MR; ++m)
-            if (lane == m) mine = acc[m];
-        if (lane < out.M && lane < MR) i8_store1(out, lane, n, mine);
+        for (int r = 0; r < RW; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (lane == r * MR + m) mine = acc[r][m];
+        const int r = lane / MR, m = lane % MR;
+        if (lane < RW * MR && m < out.M && n0 + r < out.N) i8_store1(out, m, n0 + r, mine);
     }
 }
 
@@ -186,9 +208,10 @@ void launch_i8_tile(const int8_t* xq, const int8_t* w, const I8Out& out, int K, 
 template <int MR>
 void launch_i8_gemv(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
     const int N = out.N;
-    if (N >= 16384) i8_gemv<MR, 1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(xq, w, out, K);
-    else if (N >= 8192) i8_gemv<MR, 2><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(xq, w, out, K);
-    else i8_gemv<MR, 4><<<dim3((unsigned)N), kBlock, 0, st>>>(xq, w, out, K);
+    if (N >= 16384 && K <= 8192) i8_gemv<MR, 1, 2><<<dim3((unsigned)((N + 7) / 8)), kBlock, 0, st>>>(xq, w, out, K);
+    else if (N >= 16384) i8_gemv<MR, 1, 1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(xq, w, out, K);
+    else if (N >= 8192) i8_gemv<MR, 2, 1><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(xq, w, out, K);
+    else i8_gemv<MR, 4, 1><<<dim3((unsigned)N), kBlock, 0, st>>>(xq, w, out, K);
 }
 
 enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };

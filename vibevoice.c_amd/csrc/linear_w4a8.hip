@@ -11,8 +11,9 @@
 //   VV_Q8_W4_MMA   bytes 4t..4t+3 meet slots 0..3, bytes 16+4t.. slots 4..7, so
 //                  a chunk unpacks into the two 16-byte operands of one
 //                  v_mfma_i32_32x32x32_i8 step
-// Either way the zero point is taken off the unpacked bytes (q - z fits int8),
-// the per-group sums are exact int32, and the groups are added in order in
+// The zero point is taken off the unpacked bytes (q - z fits int8) or, in the
+// GEMV when the quantiser's per-chunk sums of x are passed, through those; the
+// per-group sums are exact int32 either way, and the groups are added in order in
 // FP32 with nothing fused: acc += s_g * (float)sum_g, then acc * sx[m], + bias,
 // + residual. That is the CPU kernel's scalar form (src/cpu/cpu_int8.c:212-233,
 // 537-541), so every path and tile shape gives the same bits.
@@ -96,7 +97,7 @@ __device__ __forceinline__ void w4_store4(const W4Args& o, int m, int n, const f
     }
 }
 
-// ── M <= 8: one workgroup per weight row ───────────────────────────────────
+// ── M <= 8, any group size: one workgroup per weight row ───────────────────
 // Every thread takes whole 32-column chunks (16 bytes of codes against 32
 // bytes of each activation row) and leaves the chunk's exact sums in LDS; the
 // group sums are scaled in parallel, and one thread per activation row adds
@@ -149,6 +150,125 @@ __global__ __launch_bounds__(kBlock) void w4a8_gemv(W4Args a) {
         for (int g = 0; g < ng; ++g) acc = acc + group_term[tid][g];
         w4_store1(a, tid, n, acc);
     }
+}
+
+// The same for group sizes of 32 * 2^j columns (j <= 6), without the chunk sums
+// in LDS. kSplit waves share RW weight rows: wave p of them takes the rounds of
+// 64 chunks p, p + kSplit, ... (a round holds whole groups), lane l chunk l of
+// the round; the lanes of a group add their chunk sums with shuffles, and only
+// the scaled group terms go to LDS for the in-order addition. kSplit > 1 keeps
+// the chip busy when there are few rows, RW > 1 keeps more bytes in flight per
+// wave when rows are many and short, and shares the activation loads. kXsum:
+// the zero point goes through the quantiser's per-chunk sums of x
+// (sum q x - z sum x) instead of being taken off every code.
+constexpr int kBlockTerms = 8192;      // FP32 group terms per workgroup (32 KB)
+
+template <int MR, int kSplit, int RW, bool kXsum>
+__global__ __launch_bounds__(kBlock) void w4a8_gemv_rows(W4Args a, const int32_t* __restrict__ xsum,
+                                                         int log2_per_group) {
+    constexpr int kRows = kWavesPerBlock / kSplit * RW;    // weight rows per workgroup
+    extern __shared__ float terms[];                       // [kRows][MR][groups]
+    const int wave = wave_in_block(), lane = lane_id();
+    const int nchunks = a.K / 32, ng = a.K / a.G;
+    const int per_group = 1 << log2_per_group;
+    const int set = wave / kSplit, piece = wave % kSplit;
+    const int n_blk = (int)blockIdx.x * kRows;
+    const u32x4* wrow[RW];
+    const uint32_t* szrow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const int row = min(n_blk + set * RW + r, a.N - 1);
+        wrow[r] = reinterpret_cast<const u32x4*>(a.packed + (size_t)row * (a.K / 8));
+        szrow[r] = a.sz + (size_t)row * ng;
+    }
+#pragma unroll 2
+    for (int base = piece * kWave; base < nchunks; base += kSplit * kWave) {
+        const bool live = base + lane < nchunks;
+        const int c = live ? base + lane : nchunks - 1;
+        const int g = c >> log2_per_group;
+        i32x4 x0[MR], x1[MR];
+        int xs[MR];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            if (m < a.M) {
+                const i32x4* xr = reinterpret_cast<const i32x4*>(a.xq + (size_t)m * a.K) + 2 * c;
+                x0[m] = xr[0];
+                x1[m] = xr[1];
+                if (kXsum) xs[m] = xsum[(size_t)m * nchunks + c];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            const u32x4 w = __builtin_nontemporal_load(wrow[r] + c);
+            const uint32_t szw = szrow[r][g];
+            const uint32_t z4 = sz_zero4(szw);
+            const int z = (int)(z4 & 0xFFu);
+            const float scale = sz_scale(szw);
+            int wq[8];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t even = w[t] & 0x0F0F0F0Fu, odd = (w[t] >> 4) & 0x0F0F0F0Fu;
+                wq[2 * t] = (int)(kXsum ? even : minus_zero(even, z4));
+                wq[2 * t + 1] = (int)(kXsum ? odd : minus_zero(odd, z4));
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                if (m < a.M) {
+                    int d = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        d = __builtin_amdgcn_sdot4(x0[m][i], wq[i], d, false);
+                        d = __builtin_amdgcn_sdot4(x1[m][i], wq[4 + i], d, false);
+                    }
+                    if (kXsum) d -= z * xs[m];
+                    if (!live) d = 0;
+                    for (int o = 1; o < per_group; o <<= 1) d += __shfl_xor(d, o);
+                    if (live && (lane & (per_group - 1)) == 0)
+                        terms[((set * RW + r) * MR + m) * ng + g] = scale * (float)d;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int tid = (int)threadIdx.x;
+    if (tid < kRows * MR) {
+        const int row = tid / MR, m = tid % MR;
+        if (m < a.M && n_blk + row < a.N) {
+            const float* t = terms + (row * MR + m) * ng;
+            float acc = 0.0f;
+            for (int g = 0; g < ng; ++g) acc = acc + t[g];
+            w4_store1(a, m, n_blk + row, acc);
+        }
+    }
+}
+
+template <int MR, int kSplit, int RW>
+void launch_gemv_rows(const W4Args& a, const int32_t* xsum, int log2_pg, hipStream_t st) {
+    constexpr int kRows = kWavesPerBlock / kSplit * RW;
+    const dim3 grid((unsigned)((a.N + kRows - 1) / kRows));
+    const size_t lds = (size_t)kRows * MR * (a.K / a.G) * sizeof(float);     // at most kBlockTerms floats
+    if (xsum) w4a8_gemv_rows<MR, kSplit, RW, true><<<grid, kBlock, lds, st>>>(a, xsum, log2_pg);
+    else w4a8_gemv_rows<MR, kSplit, RW, false><<<grid, kBlock, lds, st>>>(a, xsum, log2_pg);
+}
+
+template <int MR>
+bool launch_gemv_fast(const W4Args& a, const int32_t* xsum, hipStream_t st) {
+    const int per_group = a.G / 32, ng = a.K / a.G, nchunks = a.K / 32;
+    if (per_group > kWave || (per_group & (per_group - 1)) != 0) return false;
+    int log2_pg = 0;
+    while ((1 << log2_pg) < per_group) ++log2_pg;
+    // Thousands of waves in flight, and no wave with less than half a round of chunks.
+    int split = 1, rw = 1;
+    while (split < 4 && (long)a.N * split < 4096 && nchunks / (2 * split) >= kWave / 2) split *= 2;
+    while (split == 1 && rw < 4 && a.N / (2 * rw) >= 8192 && a.K * rw <= 8192) rw *= 2;
+    while (rw > 1 && kWavesPerBlock * rw * MR * ng > kBlockTerms) rw >>= 1;
+    if (kWavesPerBlock / split * rw * MR * ng > kBlockTerms) return false;
+    if (rw == 4) launch_gemv_rows<MR, 1, 4>(a, xsum, log2_pg, st);
+    else if (rw == 2) launch_gemv_rows<MR, 1, 2>(a, xsum, log2_pg, st);
+    else if (split == 1) launch_gemv_rows<MR, 1, 1>(a, xsum, log2_pg, st);
+    else if (split == 2) launch_gemv_rows<MR, 2, 1>(a, xsum, log2_pg, st);
+    else launch_gemv_rows<MR, 4, 1>(a, xsum, log2_pg, st);
+    return true;
 }
 
 // ── larger M: LDS-tiled int8 MFMA over codes unpacked on their way into LDS ─
@@ -345,7 +465,6 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
                                const void* packed, const void* sz, int group_size, const void* bias,
                                const void* residual, void* y, int y_f32, int M, int N, int K, int path,
                                void* stream) {
-    (void)xsum;   // the zero points are taken off the unpacked codes, so the per-32 sums are not needed
     if (!xq || !sx || !packed || !sz || !y) return VV_ERR_NULL_PTR;
     if (x_layout != vv::kLayoutGemv && x_layout != vv::kLayoutMma) return VV_ERR_INVALID_ARG;
     if (M <= 0 || N <= 0 || K <= 0 || path < vv::kPathAuto || path > vv::kPathSimt)
@@ -357,7 +476,8 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
     if (path == vv::kPathAuto) path = x_layout == vv::kLayoutGemv ? vv::kPathGemv : vv::kPathMma;
     // Each kernel family reads one order of the activations.
     if ((path == vv::kPathGemv) != (x_layout == vv::kLayoutGemv)) return VV_ERR_UNSUPPORTED;
-    if (path == vv::kPathGemv && (M > 8 || K / 32 > vv::kGemvMaxChunks)) return VV_ERR_UNSUPPORTED;
+    if (path == vv::kPathGemv && M > 8) return VV_ERR_UNSUPPORTED;
+    if (xsum && (reinterpret_cast<uintptr_t>(xsum) & 3u)) return VV_ERR_UNSUPPORTED;
 
     hipStream_t st = vv::as_stream(stream);
     vv::W4Args a;
@@ -377,10 +497,18 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
     a.vec = (N % 4 == 0) && !mis(bias, 7u) && !mis(residual, 7u) && !mis(y, y_f32 ? 15u : 7u);
 
     if (path == vv::kPathGemv) {
+        // xsum (may be NULL) is only read here: the other kernels take the zero point off the codes
+        const int mr = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : 8;
+        const bool fast = mr == 1 ? vv::launch_gemv_fast<1>(a, xsum, st)
+                        : mr == 2 ? vv::launch_gemv_fast<2>(a, xsum, st)
+                        : mr == 4 ? vv::launch_gemv_fast<4>(a, xsum, st)
+                                  : vv::launch_gemv_fast<8>(a, xsum, st);
+        if (fast) return vv::launch_status();
+        if (K / 32 > vv::kGemvMaxChunks) return VV_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)N);
-        if (M == 1) vv::w4a8_gemv<1><<<grid, vv::kBlock, 0, st>>>(a);
-        else if (M == 2) vv::w4a8_gemv<2><<<grid, vv::kBlock, 0, st>>>(a);
-        else if (M <= 4) vv::w4a8_gemv<4><<<grid, vv::kBlock, 0, st>>>(a);
+        if (mr == 1) vv::w4a8_gemv<1><<<grid, vv::kBlock, 0, st>>>(a);
+        else if (mr == 2) vv::w4a8_gemv<2><<<grid, vv::kBlock, 0, st>>>(a);
+        else if (mr == 4) vv::w4a8_gemv<4><<<grid, vv::kBlock, 0, st>>>(a);
         else vv::w4a8_gemv<8><<<grid, vv::kBlock, 0, st>>>(a);
         return vv::launch_status();
     }
