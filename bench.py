@@ -712,6 +712,12 @@ def main() -> int:
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         for name, d in layer["gemv"].items():
             log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        for kind in ("w8a8", "w4a8"):
+            for name, d in layer[kind].items():
+                log(f"  {kind} {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TOPs']:7.1f} TOP/s "
+                    f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
+            for name, d in layer[kind + "_gemv"].items():
+                log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         d = layer["attn_prefill"]
         log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")

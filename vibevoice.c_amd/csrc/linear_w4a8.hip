@@ -272,15 +272,14 @@ bool launch_gemv_fast(const W4Args& a, const int32_t* xsum, hipStream_t st) {
 }
 
 // ── larger M: LDS-tiled int8 MFMA over codes unpacked on their way into LDS ─
-// Slabs of 64 columns (two MFMA steps = two chunks of codes), double-buffered
+// Slabs of 128 columns (four MFMA steps = four chunks of codes), double-buffered
 // through registers. A thread that stages chunk p of weight row n also leaves
 // that chunk's group scale in LDS; when a step ends a group, every int32
 // accumulator is scaled into its FP32 partner and cleared.
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int kSteps>
 __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
     constexpr int NT = WM * WN * kWave;
-    constexpr int kSlots = 4;                     // 16-byte slots per slab row
-    constexpr int kSteps = 2;
+    constexpr int kSlots = 2 * kSteps;            // 16-byte slots per slab row
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int LA = BM * kSlots / NT;          // activation loads per thread per slab
     constexpr int kBLoads = BN * kSteps;          // code chunks per slab
@@ -288,8 +287,8 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
     static_assert(LA >= 1 && (BM * kSlots) % NT == 0, "activation loads divide over the threads");
     static_assert(kBLoads % NT == 0 || LB == 1, "code loads: whole rounds, or one partial round");
     constexpr int kASlots = BM * kSlots, kBSlots = BN * kSlots;
-    __shared__ u32x4 lds[2 * (kASlots + kBSlots)];
-    __shared__ float scales[2][kSteps][BN];
+    extern __shared__ u32x4 lds[];                // [2][A rows | B rows][slot], then the scales
+    float (*scales)[kSteps][BN] = reinterpret_cast<float (*)[kSteps][BN]>(lds + 2 * (kASlots + kBSlots));
 
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -297,7 +296,7 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
     const int nsteps = a.K / 32, nslabs = (nsteps + kSteps - 1) / kSteps;
     const int per_group = a.G / 32, ng = a.K / a.G;
 
-    // activations: thread t's i-th load is row (t + i NT) / 4, slot t % 4
+    // activations: thread t's i-th load is row (t + i NT) / kSlots, slot t % kSlots
     const int a_slot = tid % kSlots;
     const int8_t* a_ptr[LA];
 #pragma unroll
@@ -306,8 +305,8 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
         a_ptr[i] = a.xq + (size_t)(m_blk + row) * a.K + a_slot * 16;
     }
     const int aw_row = tid / kSlots;
-    const int aw_idx = aw_row * kSlots + swz<32>(aw_row, a_slot);
-    // codes: load j is row (t + j NT) / 2, chunk (t % 2) of the slab
+    const int aw_idx = aw_row * kSlots + swz<kSlots * 8>(aw_row, a_slot);
+    // codes: load j is row (t + j NT) / kSteps, chunk t % kSteps of the slab
     const int b_step = tid % kSteps;
     const uint32_t* b_ptr[LB];
     const uint32_t* z_ptr[LB];
@@ -355,8 +354,8 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
                     hi[t] = minus_zero(__builtin_amdgcn_perm(odd, even, 0x07030602u), z4);
                 }
                 const int row = b_row[j];
-                dst[kASlots + row * kSlots + swz<32>(row, 2 * b_step)] = lo;
-                dst[kASlots + row * kSlots + swz<32>(row, 2 * b_step + 1)] = hi;
+                dst[kASlots + row * kSlots + swz<kSlots * 8>(row, 2 * b_step)] = lo;
+                dst[kASlots + row * kSlots + swz<kSlots * 8>(row, 2 * b_step + 1)] = hi;
                 scales[buf][b_step][row] = sz_scale(rz[j]);
             }
         }
@@ -369,16 +368,17 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
 #pragma unroll
         for (int y = 0; y < TM; ++y)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { acc[x][y][r] = 0; facc[x][y][r] = 0.0f; }
+            for (int r = 0; r < 16; ++r) facc[x][y][r] = 0.0f;
 
     const int frow = lane & 31, fhalf = lane >> 5;
     int f_idx[kSteps];
 #pragma unroll
     for (int step = 0; step < kSteps; ++step)
-        f_idx[step] = frow * kSlots + swz<32>(frow, step * 2 + fhalf);
+        f_idx[step] = frow * kSlots + swz<kSlots * 8>(frow, step * 2 + fhalf);
     const int fa_base = wm * TM * 32 * kSlots;
     const int fb_base = kASlots + wn * TN * 32 * kSlots;
     int until_flush = per_group;
+    bool fresh = true;
 
     auto compute = [&](int buf, int slab) {
         const u32x4* src = lds + buf * (kASlots + kBSlots);
@@ -390,15 +390,29 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
             for (int x = 0; x < TN; ++x) fw[x] = src[fb_base + x * 32 * kSlots + f_idx[step]];
 #pragma unroll
             for (int y = 0; y < TM; ++y) fx[y] = src[fa_base + y * 32 * kSlots + f_idx[step]];
+            // The first step of a group starts from a literal zero, so a flush need not clear anything.
+            if (fresh) {
+                const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int x = 0; x < TN; ++x)
+                for (int x = 0; x < TN; ++x)
 #pragma unroll
-                for (int y = 0; y < TM; ++y)
-                    acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fw[x]),
-                                                                      __builtin_bit_cast(i32x4, fx[y]),
-                                                                      acc[x][y], 0, 0, 0);
+                    for (int y = 0; y < TM; ++y)
+                        acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fw[x]),
+                                                                          __builtin_bit_cast(i32x4, fx[y]),
+                                                                          zero, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int x = 0; x < TN; ++x)
+#pragma unroll
+                    for (int y = 0; y < TM; ++y)
+                        acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fw[x]),
+                                                                          __builtin_bit_cast(i32x4, fx[y]),
+                                                                          acc[x][y], 0, 0, 0);
+            }
+            fresh = false;
             if (--until_flush == 0) {
                 until_flush = per_group;
+                fresh = true;
                 const float* sc = &scales[buf][step][wn * TN * 32 + 4 * fhalf];
 #pragma unroll
                 for (int x = 0; x < TN; ++x)
@@ -412,7 +426,6 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
 #pragma clang fp contract(off)
                                 const float term = s[r] * (float)acc[x][y][4 * g + r];
                                 facc[x][y][4 * g + r] = facc[x][y][4 * g + r] + term;
-                                acc[x][y][4 * g + r] = 0;
                             }
                     }
             }
@@ -448,10 +461,26 @@ __global__ __launch_bounds__(WM * WN * kWave, 2) void w4a8_tile(W4Args a) {
     }
 }
 
-template <int BM, int BN, int WM, int WN>
-void launch_w4_tile(const W4Args& a, hipStream_t st) {
+template <int BM, int BN, int WM, int WN, int kSteps>
+bool launch_w4_tile(const W4Args& a, hipStream_t st) {
+    constexpr size_t kLds = (size_t)2 * (BM + BN) * 2 * kSteps * 16 + (size_t)2 * kSteps * BN * sizeof(float);
+    if constexpr (kLds > 64 * 1024) {
+        // above the default limit of dynamic LDS: raised once per thread and device
+        static thread_local int ready_device = -1;
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess) return false;
+        if (ready_device != device) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(w4a8_tile<BM, BN, WM, WN, kSteps>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+                (void)hipGetLastError();
+                return false;
+            }
+            ready_device = device;
+        }
+    }
     const dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)((a.M + BM - 1) / BM));
-    w4a8_tile<BM, BN, WM, WN><<<grid, WM * WN * kWave, 0, st>>>(a);
+    w4a8_tile<BM, BN, WM, WN, kSteps><<<grid, WM * WN * kWave, kLds, st>>>(a);
+    return true;
 }
 
 enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
@@ -513,9 +542,13 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
         return vv::launch_status();
     }
     const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (M > 64 && wg128 >= 256) vv::launch_w4_tile<128, 128, 2, 2>(a, st);
-    else if (M > 32) vv::launch_w4_tile<64, 64, 2, 2>(a, st);
-    else vv::launch_w4_tile<32, 64, 1, 2>(a, st);
+    if (M > 64 && wg128 >= 256) {
+        if (!vv::launch_w4_tile<128, 128, 2, 2, 4>(a, st)) return VV_ERR_CUDA_LAUNCH;
+    } else if (M > 32) {
+        vv::launch_w4_tile<64, 64, 2, 2, 4>(a, st);
+    } else {
+        vv::launch_w4_tile<32, 64, 1, 2, 4>(a, st);
+    }
     return vv::launch_status();
 }
 
