@@ -183,6 +183,50 @@ vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* 
                                    const int32_t* xsum, int w4, const vv_i8_proj_t* projs,
                                    int n, int group_size, int M, int K, void* stream);
 
+/* ── W4A16 linear layers ───────────────────────────────────────────────── */
+
+/* INT4 group-affine weights in the accelerator layout (vv_int4g_to_gpu_layout,
+ * src/quant/awq_repack.c:261-310): packed [N][K/2], sz half2 {scale, zero}
+ * [N][K/group_size], group_size one of 32, 64, 128, 256, K % 32 == 0 (the
+ * reference asks K % 64 for its tensor-core path and N % 8; neither is needed
+ * here). Every kernel dequantises with w = (q - z) * s rounded once to FP16
+ * (device.h:233) and accumulates in FP32; the bias is added in FP32 before the
+ * one rounding of the output. Other shapes or unaligned pointers:
+ * VV_ERR_UNSUPPORTED. */
+
+/* y[N] = W . x (+ bias) for one token; no allocation, no per-token host
+ * arguments. replaces device.h:247-249 (src/cuda/w4a16.cu:848-856). */
+vv_status_t vv_w4a16_gemv_dev(const void* x, const void* packed, const void* sz,
+                              const void* bias, void* y, int N, int K, int group_size,
+                              void* stream);
+/* One projection of a fused GEMV (device.h:252-258). */
+typedef struct vv_w4a16_proj {
+    const void* packed;
+    const void* sz;
+    const void* bias;   /* FP16 [N] or NULL */
+    void*       y;      /* FP16 [N] */
+    int         N;
+} vv_w4a16_proj_t;
+/* Up to three GEMVs of the same x in ONE launch (q/k/v, gate/up); each row
+ * exactly as vv_w4a16_gemv_dev over the combined row count would compute it.
+ * replaces device.h:266-268 (src/cuda/w4a16.cu:858-879). */
+vv_status_t vv_w4a16_gemv_multi_dev(const void* x, const vv_w4a16_proj_t* projs, int n_proj,
+                                    int K, int group_size, void* stream);
+/* out[m][j] = x[m][perm[j]] (FP16, K % 8 == 0, perm 16-byte aligned): the
+ * column order of an act-order checkpoint. replaces device.h:275-277. */
+vv_status_t vv_w4a16_gather_dev(const void* x, const int32_t* perm, void* out, int M, int K,
+                                void* stream);
+/* C[M,N] = A[M,K] . W^T (+ bias). M <= 8: the GEMV kernel; larger M: LDS-tiled
+ * FP16 MFMA with the codes dequantised on their way into LDS. `scratch` is
+ * never touched (no split-K partials, no dequantised copy) and may be NULL.
+ * replaces device.h:288-291 (src/cuda/w4a16.cu:894-932). */
+vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
+                              const void* bias, void* C, void* scratch, size_t scratch_bytes,
+                              int M, int N, int K, int group_size, void* stream);
+/* Accelerator-layout INT4 -> dense FP16 [N,K]. replaces device.h:294-296. */
+vv_status_t vv_w4a16_dequant_dev(const void* packed, const void* sz, void* out_fp16, int N,
+                                 int K, int group_size, void* stream);
+
 /* ── Dense linear layers ───────────────────────────────────────────────── */
 
 /* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32

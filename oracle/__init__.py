@@ -84,6 +84,8 @@ def _load():
     lib.vvo_int4g_to_gpu_layout.restype = C.c_int
     lib.vvo_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
                                             C.c_void_p]
+    lib.vvo_int4g_dequant_f16.restype = C.c_int
+    lib.vvo_int4g_dequant_f16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
     lib.vvo_argmax_first.restype = C.c_int
     lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
@@ -123,6 +125,10 @@ def _load_ref():
         ref.vv_w4a8_gemm_cpu.restype = C.c_int
         ref.vv_w4a8_gemm_cpu.argtypes = [C.c_void_p, _f32p, _i32p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                          C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
+    if hasattr(ref, "vv_int4g_gemm_cpu"):
+        ref.vv_int4g_gemm_cpu.restype = C.c_int
+        ref.vv_int4g_gemm_cpu.argtypes = [_f32p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _f32p,
+                                          C.c_int, C.c_int, C.c_int, C.c_int]
     if hasattr(ref, "vv_int4g_to_gpu_layout"):
         ref.vv_int4g_to_gpu_layout.restype = C.c_int
         ref.vv_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
@@ -390,3 +396,14 @@ def int4g_to_gpu_layout(packed, scales16, zeros, G):
     _check(lib.vvo_int4g_to_gpu_layout(out.ctypes.data, scales16.ctypes.data, zeros.ctypes.data, N, K, G,
                                        sz.ctypes.data), "int4g_to_gpu_layout")
     return out, sz
+
+
+def int4g_dequant_f16(packed, scales16, zeros, G):
+    """Row-major INT4G codes [N,K/2] -> FP16 bits [N,K] of (q - z) * s, rounded once."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    scales16, zeros = np.ascontiguousarray(scales16, np.uint16), np.ascontiguousarray(zeros, np.uint8)
+    N, K = packed.shape[0], packed.shape[1] * 2
+    out = np.empty((N, K), np.uint16)
+    _check(lib.vvo_int4g_dequant_f16(packed.ctypes.data, scales16.ctypes.data, zeros.ctypes.data, N, K, G,
+                                     out.ctypes.data), "int4g_dequant_f16")
+    return out

@@ -452,6 +452,24 @@ int vvo_w4a8_linear(const int8_t* xq, const float* sx, const uint8_t* packed,
     return VVO_OK;
 }
 
+int vvo_int4g_dequant_f16(const uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
+                          int N, int K, int G, uint16_t* out16) {
+    if (!packed || !scales16 || !zeros || !out16) return VVO_ERR_NULL_PTR;
+    if (N <= 0 || K <= 0 || G <= 0 || (K % G) != 0 || (K % 2) != 0) return VVO_ERR_INVALID_ARG;
+    const int ng = K / G;
+    for (int n = 0; n < N; n++)
+        for (int k = 0; k < K; k++) {
+            const uint8_t b = packed[(size_t)n * (K / 2) + k / 2];
+            const int q = (k & 1) ? (b & 15) : (b >> 4);
+            const size_t g = (size_t)n * ng + k / G;
+            /* q - z is an exact small integer, the scale an FP16 value: the FP32 product is exact,
+               so this is one rounding of the true product to FP16 */
+            const float w = (float)(q - (int)zeros[g]) * vvo_half_to_float(scales16[g]);
+            out16[(size_t)n * K + k] = vvo_float_to_half_rne(w);
+        }
+    return VVO_OK;
+}
+
 int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
                             int N, int K, int G, uint16_t* out_sz) {
     if (!packed || !scales16 || !zeros || !out_sz) return VVO_ERR_NULL_PTR;

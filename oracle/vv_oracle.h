@@ -150,6 +150,13 @@ int vvo_w4a8_linear(const int8_t* xq, const float* sx, const uint8_t* packed,
                     const uint16_t* bias16, const uint16_t* res16, float* out_f32,
                     uint16_t* out_f16, int M, int N, int K);
 
+/* INT4 group-affine weights to dense FP16 [N,K]: w = (q - z) * s rounded once to
+ * FP16, the formula include/vibevoice/device.h:233 and src/cuda/w4a16.cu:24-27
+ * state for every W4A16 kernel. `packed` is the row-major INT4G form. The
+ * W4A16 linear layer is then vvo_gemm_f16w over these weights. */
+int vvo_int4g_dequant_f16(const uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
+                          int N, int K, int G, uint16_t* out16);
+
 /* src/quant/awq_repack.c:261-310 (vv_int4g_to_gpu_layout): row-major INT4G
  * codes to the layout the accelerator kernels read, in place: inside every
  * 16-byte chunk (32 columns), nibble slot s of 32-bit word t holds column

@@ -117,3 +117,21 @@ def test_reference_own_int8_linear_test_passes_on_this_backend():
     last = res.stdout.strip().splitlines()[-1]
     done, total = last.strip("= ").split()[0].split("/")
     assert done == total and int(total) >= 1600, last
+
+
+W4A16_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_w4a16_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(W4A16_EXE),
+                    reason="oracle/_ref/test_w4a16_hip not built (needs the reference tree)")
+def test_reference_own_w4a16_test_passes_on_this_backend():
+    """The reference's tests/test_w4a16.c: AWQ, GPTQ (symmetric, act-order) and
+    load-time INT4 weights made and repacked by the reference's host code, then
+    this backend's GEMV, fused GEMV, gather and GEMM at ten row counts against
+    the reference's CPU kernel and an FP64 product of the exact FP16 weights."""
+    res = subprocess.run([W4A16_EXE], capture_output=True, text=True, timeout=580)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert "all W4A16 checks match the reference" in res.stdout

@@ -240,3 +240,27 @@ def test_int4_gpu_layout_against_reference_and_the_activation_orders():
     by_mma = np.concatenate([nib[..., :4].reshape(N, K // 32, 16), nib[..., 4:].reshape(N, K // 32, 16)],
                             axis=-1).reshape(N, K)
     assert np.array_equal(mma.astype(np.int64) @ by_mma.T, want)
+
+
+def test_int4_dequant_against_closed_form_and_reference_gemm():
+    """(q - z) * s: the FP64 product is exact, so its direct rounding to FP16
+    pins every bit. The compiled reference's CPU GEMM dequantises as
+    q * s + fp16(-z * s) (one more rounding per weight), so a product of these
+    weights agrees with it to FP16 weight precision, not bit for bit."""
+    import ctypes as C
+    N, K, G, M = 24, 256, 64, 5
+    packed, scales, zeros = int4_problem(N, K, G, 4)
+    w16 = oracle.int4g_dequant_f16(packed, scales, zeros, G)
+    d = int4_codes(packed) - np.repeat(zeros.astype(np.int64), G, axis=1)
+    s = np.repeat(oracle.widen(scales).astype(np.float64), G, axis=1)
+    assert np.array_equal(w16, (d * s).astype(np.float16).view(np.uint16))
+    if oracle.ref is not None and hasattr(oracle.ref, "vv_int4g_gemm_cpu"):
+        x = np.random.default_rng(6).normal(size=(M, K)).astype(np.float32)
+        mins = (-(zeros.astype(np.float32)) * oracle.widen(scales)).astype(np.float16).view(np.uint16)
+        out = np.empty((M, N), np.float32)
+        f32p = C.POINTER(C.c_float)
+        assert oracle.ref.vv_int4g_gemm_cpu(x.ctypes.data_as(f32p), packed.ctypes.data, scales.ctypes.data,
+                                            mins.ctypes.data, None, out.ctypes.data_as(f32p), M, N, K, G) == 0
+        ours = oracle.gemm_f16w(x, w16)
+        mag = np.abs(x).astype(np.float64) @ np.abs(oracle.widen(w16)).astype(np.float64).T
+        assert np.max(np.abs(out - ours) / mag) < 2e-3

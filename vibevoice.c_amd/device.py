@@ -38,6 +38,12 @@ class SkinnyProj(C.Structure):
                 ("N", C.c_int)]
 
 
+class W4A16Proj(C.Structure):
+    """vv_w4a16_proj_t: one projection of a fused W4A16 GEMV."""
+    _fields_ = [("packed", C.c_void_p), ("sz", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p),
+                ("N", C.c_int)]
+
+
 class I8Proj(C.Structure):
     """vv_i8_proj_t: one projection of a shared-input int8 launch."""
     _fields_ = [("w", C.c_void_p), ("sw", C.c_void_p), ("sz", C.c_void_p), ("bias", C.c_void_p),
@@ -73,6 +79,11 @@ SIGNATURES = {
     "vv_argmax_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
     "vv_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vv_w4a16_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_w4a16_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _i, _vp]),
+    "vv_w4a16_gather_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "vv_w4a16_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _i, _i, _i, _i, _vp]),
+    "vv_w4a16_dequant_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "vv_w8a8_linear_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_w4a8_linear_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_i8_linear_multi_dev": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
