@@ -315,6 +315,24 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                 out[key][name] = {"N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del xq, sx, c
+        # the same codes against FP16 activations (W4A16)
+        for m, key in ((T, "w4a16"), (1, "w4a16_gemv")):
+            out.setdefault(key, {})
+            a = torch.randn(m, k, dtype=torch.float16, device="cuda")
+            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+            dense = torch.empty(n * k, dtype=torch.float16, device="cuda")     # the decoder's dequant scratch
+            sec = timed(lambda: dev.vv_w4a16_gemm_dev(a.data_ptr(), w4.data_ptr(), sz.data_ptr(), None, c.data_ptr(),
+                                                      dense.data_ptr(), n * k * 2, m, n, k, G, st),
+                        5 if m > 1 else 50)
+            if m > 1:
+                tf = 2.0 * m * n * k / sec / 1e12
+                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TFLOPs": tf,
+                                  "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+            else:
+                gb = (n * k / 2 + n * (k // G) * 4 + 2.0 * k + 2.0 * n) / sec / 1e9
+                out[key][name] = {"N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+            del a, c, dense
         del w4, sz
     q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
     k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
@@ -718,6 +736,11 @@ def main() -> int:
                     f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
             for name, d in layer[kind + "_gemv"].items():
                 log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        for name, d in layer["w4a16"].items():
+            log(f"  w4a16 {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+                f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+        for name, d in layer["w4a16_gemv"].items():
+            log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         d = layer["attn_prefill"]
         log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")

@@ -217,9 +217,11 @@ vv_status_t vv_w4a16_gemv_multi_dev(const void* x, const vv_w4a16_proj_t* projs,
 vv_status_t vv_w4a16_gather_dev(const void* x, const int32_t* perm, void* out, int M, int K,
                                 void* stream);
 /* C[M,N] = A[M,K] . W^T (+ bias). M <= 8: the GEMV kernel; larger M: LDS-tiled
- * FP16 MFMA with the codes dequantised on their way into LDS. `scratch` is
- * never touched (no split-K partials, no dequantised copy) and may be NULL.
- * replaces device.h:288-291 (src/cuda/w4a16.cu:894-932). */
+ * FP16 MFMA with the codes dequantised on their way into LDS; from 1024 rows,
+ * when `scratch` holds N * K * 2 bytes: the weight dequantised there once, then
+ * vv_gemm_fp16_dev started from the bias. `scratch` may be NULL (no split-K
+ * partials are ever needed). replaces device.h:288-291
+ * (src/cuda/w4a16.cu:894-932). */
 vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
                               const void* bias, void* C, void* scratch, size_t scratch_bytes,
                               int M, int N, int K, int group_size, void* stream);

@@ -47,13 +47,15 @@ def check(got_bits, x, w, bias, what):
     assert worst <= 1.0, f"{what}: {worst:.3f}x the elementwise bound"
 
 
-def gemm(x, w, bias=None):
+def gemm(x, w, bias=None, scratch=False):
     M = x.shape[0]
     d_x = to_dev(x)
     d_b = to_dev(bias) if bias is not None else None
     d_y = torch.full((M, w["N"]), float("nan"), dtype=torch.float16, device="cuda")
+    d_s = torch.empty(w["N"] * w["K"], dtype=torch.float16, device="cuda") if scratch else None
     ok(dev.vv_w4a16_gemm_dev(d_x.data_ptr(), w["d_w"].data_ptr(), w["d_sz"].data_ptr(),
-                             d_b.data_ptr() if d_b is not None else None, d_y.data_ptr(), None, 0, M, w["N"],
+                             d_b.data_ptr() if d_b is not None else None, d_y.data_ptr(),
+                             d_s.data_ptr() if scratch else None, d_s.numel() * 2 if scratch else 0, M, w["N"],
                              w["K"], w["G"], stream()))
     return bits_of(d_y)
 
@@ -113,12 +115,26 @@ def test_gemm_large(M, N, K, G):
     check(gemm(x, w), x, w, None, f"gemm M={M} {N}x{K} g{G}")
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gemm_through_the_scratch(with_bias):
+    """From 1024 rows a scratch that holds the dense weight is used; the bias
+    still joins the FP32 sum before the only rounding, so the bars are the same
+    and, the K order being the same, so are the bits."""
+    M, N, K, G = 1100, 512, 3584, 128
+    w = weight(N, K, G, 33)
+    bias = oracle.normal_f16((N,), 8, std=0.5) if with_bias else None
+    x = activations(M, K, 34)
+    through = gemm(x, w, bias, scratch=True)
+    check(through, x, w, bias, "dequantise + FP16 GEMM")
+    assert np.array_equal(through, gemm(x, w, bias)), "scratch or not, the same bits"
+
+
 def test_gemm_prefill_shape_sampled_rows():
     M, N, K, G = 14449, 3584, 3584, 128
     w = weight(N, K, G, 41)
     bias = oracle.normal_f16((N,), 7, std=0.5)
     x = activations(M, K, 42)
-    got = gemm(x, w, bias)
+    got = gemm(x, w, bias, scratch=True)
     rows = np.sort(np.random.default_rng(2).choice(M, 40, replace=False))
     rows[0], rows[-1] = 0, M - 1
     check(got[rows], x[rows], w, bias, "sampled rows at T = 14449")

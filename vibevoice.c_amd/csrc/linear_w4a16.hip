@@ -84,6 +84,16 @@ __global__ __launch_bounds__(kBlock) void w4a16_gather(const h16* __restrict__ x
     *reinterpret_cast<h16x8*>(out + m * K + j) = v;
 }
 
+// c[m][n] = bias[n]: the starting value of a GEMM that adds into C, so that the bias
+// joins the FP32 sum before the one rounding of the output.
+__global__ __launch_bounds__(kBlock) void bias_rows(const h16* __restrict__ bias, h16* __restrict__ c, int M, int N) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;       // one run of 8 outputs (N % 8 == 0)
+    const int per_row = N / 8;
+    if (i >= (size_t)M * per_row) return;
+    const int j = (int)(i % (size_t)per_row) * 8;
+    *reinterpret_cast<h16x8*>(c + (i / (size_t)per_row) * N + j) = *reinterpret_cast<const h16x8*>(bias + j);
+}
+
 // ── M <= 8 ─────────────────────────────────────────────────────────────────
 constexpr int kMaxSegs = 3;
 
@@ -486,11 +496,13 @@ vv_status_t vv_w4a16_gemv_dev(const void* x, const void* packed, const void* sz,
     return vv_w4a16_gemv_multi_dev(x, &p, 1, K, group_size, stream);
 }
 
-/* scratch is never needed: the weights stay packed until they are in LDS. */
+/* Many rows and a scratch that holds the dense weight: dequantise once, then the FP16 GEMM (its
+ * 256 x 256 direct-to-LDS kernel is faster than any tile that unpacks codes on the way in, and the
+ * dequantiser costs a percent of it). Otherwise the weights stay packed until they are in LDS and
+ * the scratch is not touched. */
 vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz, const void* bias, void* C,
                               void* scratch, size_t scratch_bytes, int M, int N, int K, int group_size,
                               void* stream) {
-    (void)scratch; (void)scratch_bytes;
     if (!A || !packed || !sz || !C) return VV_ERR_NULL_PTR;
     const int gs = vv::group_shift(group_size);
     if (gs < 0 || K <= 0 || K % 32 != 0 || K % group_size != 0 || M <= 0 || N <= 0) return VV_ERR_UNSUPPORTED;
@@ -506,6 +518,18 @@ vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
         segs.n[0] = N;
         vv::launch_gemv_rows(static_cast<const vv::h16*>(A), segs, 1, M, K, gs, st);
         return vv::launch_status();
+    }
+    const bool bias_ok = !bias || (N % 8 == 0 && vv::aligned16(bias) && vv::aligned16(C));
+    if (M >= 1024 && scratch && vv::aligned16(scratch) && scratch_bytes >= (size_t)N * K * 2 && bias_ok) {
+        vv_status_t s = vv_w4a16_dequant_dev(packed, sz, scratch, N, K, group_size, stream);
+        if (s != VV_OK) return s;
+        if (bias) {
+            const size_t total = (size_t)M * (N / 8);
+            vv::bias_rows<<<dim3((unsigned)((total + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0, st>>>(
+                static_cast<const vv::h16*>(bias), static_cast<vv::h16*>(C), M, N);
+            if (vv::launch_status() != VV_OK) return VV_ERR_CUDA_LAUNCH;
+        }
+        return vv_gemm_fp16_dev(A, scratch, C, M, N, K, 1.0f, bias ? 1.0f : 0.0f, stream);
     }
     vv::TileArgs a;
     a.a = static_cast<const vv::h16*>(A);
