@@ -124,7 +124,10 @@ vv_status_t vv_col_absmax_dev(const void* x, int M, int K, float* acc, void* str
 /* ── W8A8 / W4A8 linear layers ──────────────────────────────────────────── */
 
 /* Which kernel family runs an int8 linear layer (device.h:347-352). Here GEMV
- * is the v_dot4 kernel (M <= 8 only), MMA and SIMT both the MFMA tile kernel. */
+ * is the v_dot4 kernel (M <= 8 only), MMA and SIMT both the MFMA kernels (tiles,
+ * or weights straight into MFMA operands up to 64 rows). AUTO: GEMV for one or
+ * two rows, MFMA beyond. Integer sums are exact, so the choice never shows in
+ * the result. */
 #define VV_I8_PATH_AUTO 0
 #define VV_I8_PATH_GEMV 1
 #define VV_I8_PATH_MMA  2
@@ -216,8 +219,10 @@ vv_status_t vv_w4a16_gemv_multi_dev(const void* x, const vv_w4a16_proj_t* projs,
  * column order of an act-order checkpoint. replaces device.h:275-277. */
 vv_status_t vv_w4a16_gather_dev(const void* x, const int32_t* perm, void* out, int M, int K,
                                 void* stream);
-/* C[M,N] = A[M,K] . W^T (+ bias). M <= 8: the GEMV kernel; larger M: LDS-tiled
- * FP16 MFMA with the codes dequantised on their way into LDS; from 1024 rows,
+/* C[M,N] = A[M,K] . W^T (+ bias). M <= 4: the GEMV kernel; to 64 rows: codes
+ * straight into 16x16x32 MFMA operands, K split over a workgroup's waves;
+ * larger M (or wide layers beyond 16 rows): LDS-tiled FP16 MFMA with the
+ * codes dequantised on their way into LDS; from 1024 rows,
  * when `scratch` holds N * K * 2 bytes: the weight dequantised there once, then
  * vv_gemm_fp16_dev started from the bias. `scratch` may be NULL (no split-K
  * partials are ever needed). replaces device.h:288-291

@@ -10,6 +10,8 @@
 //   i8_tile   the LDS-tiled loop of the FP16 GEMM with v_mfma_i32_32x32x32_i8:
 //             a lane's 16-byte operand is 16 int8 values, so a K step is 32
 //             wide and a 128-byte slab row carries 128 K values.
+//   i8_skinny up to 64 rows: weights straight from global memory into 16x16x64
+//             MFMA operands, K split over the eight waves of a workgroup.
 //   i8_gemv   M <= 8: one to four waves per weight row, v_dot4_i32_i8 against
 //             up to eight activation rows that share each weight load.
 #include "mfma_tile.hpp"
@@ -196,6 +198,66 @@ __global__ __launch_bounds__(kBlock) void i8_gemv(const int8_t* __restrict__ xq,
     }
 }
 
+// 9 <= M <= 64: sixteen weight rows per workgroup, K split over its eight waves,
+// weights and activations from global memory straight into 16x16x64 int8 MFMA
+// operands (a lane's 16 bytes are 16 of a step's 64 columns). Bound by the
+// weight bytes; the int32 partial tiles of the waves are added through LDS,
+// and integer addition being exact the result is the tile kernel's, bit for bit.
+constexpr int kSkinnyWaves = 8;
+
+template <int kMT>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void i8_skinny(const int8_t* __restrict__ xq,
+                                                                  const int8_t* __restrict__ w, I8Out out,
+                                                                  int K) {
+    __shared__ i32x4 part[kSkinnyWaves][kMT][kWave];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16;
+    const int kchunks = K / 16, nsteps = (kchunks + 3) / 4;
+    const i32x4* wrow = reinterpret_cast<const i32x4*>(w + (size_t)min(n0 + r16, out.N - 1) * K);
+    const i32x4* xrow[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t)
+        xrow[t] = reinterpret_cast<const i32x4*>(xq + (size_t)min(16 * t + r16, out.M - 1) * K);
+    const i32x4 zero = {0, 0, 0, 0};
+    i32x4 acc[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) acc[t] = zero;
+
+    for (int s0 = wave * 4; s0 < nsteps; s0 += kSkinnyWaves * 4) {
+        i32x4 wv[4], xv[kMT][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = (s0 + u) * 4 + ks;
+            const bool live = c < kchunks;
+            wv[u] = live ? __builtin_nontemporal_load(wrow + c) : zero;
+#pragma unroll
+            for (int t = 0; t < kMT; ++t) xv[t][u] = live ? xrow[t][c] : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u], xv[t][u], acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    // register r of lane l: column n0 + 4(l / 16) + r of row 16t + l % 16
+    if (tid < kMT * kWave) {
+        const int t = tid >> 6;
+        i32x4 sum = part[0][t][lane];
+#pragma unroll
+        for (int p = 1; p < kSkinnyWaves; ++p) sum += part[p][t][lane];
+        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        if (m < out.M && n < out.N) {
+            const int v[4] = {sum.x, sum.y, sum.z, sum.w};
+            i8_store4(out, m, n, v);
+        }
+    }
+}
+
 template <int BM, int BN, int WM, int WN, int kSlabChunks, int kAhead>
 void launch_i8_tile(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
     const dim3 grid((unsigned)((out.N + BN - 1) / BN), (unsigned)((out.M + BM - 1) / BM));
@@ -243,11 +305,22 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
     out.vec = (N % 4 == 0) && !mis(sw, 15u) && !mis(bias, 7u) && !mis(residual, 7u) &&
               !mis(y, y_f32 ? 15u : 7u);
 
-    if (M <= 8 && path != vv::kPathMma && path != vv::kPathSimt) {
+    // AUTO keeps the dot-product kernel for one or two rows; from three the MFMA kernels are faster.
+    if (path == vv::kPathGemv || (path == vv::kPathAuto && M <= 2)) {
         if (M == 1) vv::launch_i8_gemv<1>(xq, w, out, K, st);
         else if (M == 2) vv::launch_i8_gemv<2>(xq, w, out, K, st);
         else if (M <= 4) vv::launch_i8_gemv<4>(xq, w, out, K, st);
         else vv::launch_i8_gemv<8>(xq, w, out, K, st);
+        return vv::launch_status();
+    }
+    // Beyond 16 rows a wide layer re-reads the activations once per 16 columns: tiles serve it better.
+    if (M <= 16 || (M <= 64 && (N + 63) / 64 < 200)) {
+        const dim3 grid((unsigned)((N + 15) / 16));
+        constexpr int kThreads = vv::kSkinnyWaves * vv::kWave;
+        if (M <= 16) vv::i8_skinny<1><<<grid, kThreads, 0, st>>>(xq, w, out, K);
+        else if (M <= 32) vv::i8_skinny<2><<<grid, kThreads, 0, st>>>(xq, w, out, K);
+        else if (M <= 48) vv::i8_skinny<3><<<grid, kThreads, 0, st>>>(xq, w, out, K);
+        else vv::i8_skinny<4><<<grid, kThreads, 0, st>>>(xq, w, out, K);
         return vv::launch_status();
     }
     // The largest tile that still fills the 256 compute units (as for FP16).

@@ -10,9 +10,11 @@
 // column pair t + 4j; subtracting 1024 + z is exact, and the multiply by the
 // scale is the rounding. Accumulation is FP32.
 //   w4a16_dequant   codes -> dense FP16 [N][K]
-//   w4a16_gemv      M <= 8: lanes take whole chunks, v_dot2_f32_f16 against the
+//   w4a16_gemv      M <= 4: lanes take whole chunks, v_dot2_f32_f16 against the
 //                   natural half2 pairs of x; K split over waves or several
 //                   rows per wave by shape; up to three projections per launch
+//   w4a16_skinny    5 <= M <= 64: codes straight into 16x16x32 MFMA operands, K
+//                   split over the eight waves of a workgroup
 //   w4a16_tile      larger M: the LDS-tiled 32x32x16 FP16 MFMA loop with the
 //                   codes dequantised on their way into LDS
 //   w4a16_gather    out[m][j] = x[m][perm[j]] (act-order checkpoints)
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void bias_rows(const h16* __restrict__ bias
     *reinterpret_cast<h16x8*>(c + (i / (size_t)per_row) * N + j) = *reinterpret_cast<const h16x8*>(bias + j);
 }
 
-// ── M <= 8 ─────────────────────────────────────────────────────────────────
+// ── M <= 4 (and the fused single-row launches) ─────────────────────────────────────────────────────────────────
 constexpr int kMaxSegs = 3;
 
 struct GemvSegs {
@@ -249,7 +251,6 @@ void launch_gemv_rows(const h16* x, const GemvSegs& segs, int n_segs, int M, int
     else launch_gemv<8>(x, segs, n_segs, M, K, gshift, st);
 }
 
-// ── larger M ───────────────────────────────────────────────────────────────
 struct TileArgs {
     const h16* a;            // [M][K]
     const u32x4* packed;     // [N][K/32] chunks
@@ -258,6 +259,95 @@ struct TileArgs {
     h16* c;                  // [M][N]
     int M, N, K, gshift, vec;
 };
+
+// ── 5 <= M <= 64 ───────────────────────────────────────────────────────────
+// Sixteen weight rows per workgroup, K split over its eight waves, the codes
+// going from global memory straight into 16x16x32 MFMA operands: one chunk of
+// codes is one K step, lane (row, q) dequantises the chunk's q-th run of eight
+// columns (four half2 from the four words) and meets the same eight columns of
+// up to 64 activation rows. Bound by the code bytes; no LDS until the waves'
+// partial tiles are added.
+constexpr int kSkinnyWaves = 8;
+
+template <int kMT>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void w4a16_skinny(TileArgs a) {
+    __shared__ f32x4 part[kSkinnyWaves][kMT][kWave];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16;
+    const int ncodes = a.K / 32, ng = a.K >> a.gshift;
+    const int row = min(n0 + r16, a.N - 1);
+    const u32x4* wrow = a.packed + (size_t)row * ncodes;
+    const uint32_t* szrow = a.sz + (size_t)row * ng;
+    const u32x4* arow[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t)
+        arow[t] = reinterpret_cast<const u32x4*>(a.a + (size_t)min(16 * t + r16, a.M - 1) * a.K);
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    f32x4 acc[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int c0 = wave * 4; c0 < ncodes; c0 += kSkinnyWaves * 4) {
+        u32x4 codes[4], x[kMT][4];
+        uint32_t gsz[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool live = c0 + u < ncodes;
+            const int c = live ? c0 + u : ncodes - 1;
+            codes[u] = __builtin_nontemporal_load(wrow + c);
+            gsz[u] = szrow[(c * 32) >> a.gshift];
+#pragma unroll
+            for (int t = 0; t < kMT; ++t) x[t][u] = live ? arow[t][c * 4 + ks] : zero;   // a dead step adds zero
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const GroupConst gc = group_const(gsz[u]);
+            u32x4 w;
+            w.x = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].x, ks, gc));
+            w.y = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].y, ks, gc));
+            w.z = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].z, ks, gc));
+            w.w = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].w, ks, gc));
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, w),
+                                                                __builtin_bit_cast(h16x8, x[t][u]), acc[t], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    // register r of lane l: column n0 + 4(l / 16) + r of row 16t + l % 16
+    if (tid < kMT * kWave) {
+        const int t = tid >> 6;
+        f32x4 sum = part[0][t][lane];
+#pragma unroll
+        for (int w = 1; w < kSkinnyWaves; ++w) {
+            const f32x4 p = part[w][t][lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[r] += p[r];
+        }
+        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        if (m < a.M && n < a.N) {
+            h16* crow = a.c + (size_t)m * a.N;
+            if (a.vec && n + 3 < a.N) {
+                h16x4 b = {0, 0, 0, 0};
+                if (a.bias) b = *reinterpret_cast<const h16x4*>(a.bias + n);
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = to_half(sum[r] + (float)b[r]);
+                *reinterpret_cast<h16x4*>(crow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < a.N) crow[n + r] = to_half(sum[r] + (a.bias ? (float)a.bias[n + r] : 0.0f));
+            }
+        }
+    }
+}
+
+// ── larger M ───────────────────────────────────────────────────────────────
 
 // Slabs of kSlots 16-byte FP16 slots per row (8 columns each), double-buffered
 // through registers; a chunk of codes becomes four consecutive slots of its row.
@@ -509,7 +599,7 @@ vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
     if (!vv::aligned16(A) || !vv::aligned16(packed) || (reinterpret_cast<uintptr_t>(sz) & 3u))
         return VV_ERR_UNSUPPORTED;
     hipStream_t st = vv::as_stream(stream);
-    if (M <= 8) {
+    if (M <= 4) {
         vv::GemvSegs segs = {};
         segs.w[0] = static_cast<const vv::u32x4*>(packed);
         segs.sz[0] = static_cast<const uint32_t*>(sz);
@@ -542,6 +632,16 @@ vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
     a.K = K;
     a.gshift = gs;
     a.vec = (N % 4 == 0) && !(reinterpret_cast<uintptr_t>(C) & 7u) && !(bias && (reinterpret_cast<uintptr_t>(bias) & 7u));
+    // Beyond 16 rows a wide layer re-reads the activations once per 16 columns: tiles serve it better.
+    if (M <= 16 || (M <= 64 && (N + 63) / 64 < 200)) {
+        const dim3 grid((unsigned)((N + 15) / 16));
+        constexpr int kThreads = vv::kSkinnyWaves * vv::kWave;
+        if (M <= 16) vv::w4a16_skinny<1><<<grid, kThreads, 0, st>>>(a);
+        else if (M <= 32) vv::w4a16_skinny<2><<<grid, kThreads, 0, st>>>(a);
+        else if (M <= 48) vv::w4a16_skinny<3><<<grid, kThreads, 0, st>>>(a);
+        else vv::w4a16_skinny<4><<<grid, kThreads, 0, st>>>(a);
+        return vv::launch_status();
+    }
     const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     if (wg256 >= 512) vv::launch_tile<256, 256, 2, 4, 4>(a, st);
