@@ -541,6 +541,151 @@ def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool =
             "frac_of_hbm_peak": weight_bytes / replay / 1e9 / HBM_PEAK_GBPS}
 
 
+def decode_token_quant_leg(torch, dev, cache_len: int, kind: str, layers: int = 28) -> dict:
+    """The decode step of decode_token_leg with quantised projections, in the reference decoder's op
+    order for them. kind "w4a16": INT4 codes against FP16 activations (decoder.c:412-422, 512-520:
+    fused q/k/v and gate/up GEMVs with their biases). kind "w8a8" / "w4a8": int8 activations written
+    by the producing op (RMSNorm, attention output, SwiGLU), o and down adding into the hidden state
+    through the linear's residual (decoder.c:575-640, 795-932). Random weights and codes."""
+    import ctypes as C
+    s = C.c_void_p()
+    assert dev.vv_dev_stream_create(C.byref(s)) == 0
+    st = s.value
+    f16 = dict(dtype=torch.float16, device="cuda")
+    QD, KD, G = NQ * HD, NK * HD, 128
+    P = lambda t: t.data_ptr() if t is not None else None
+    a8, w4 = kind in ("w8a8", "w4a8"), kind in ("w4a16", "w4a8")
+    lay = 2 if kind == "w4a8" else 0                        # VV_Q8_W4_GEMV for one row, else column order
+
+    def w(*shape, std):
+        return torch.randn(*shape, **f16) * std
+
+    shapes = {"q": (QD, H), "k": (KD, H), "v": (KD, H), "o": (H, QD), "g": (I_FF, H), "u": (I_FF, H), "d": (H, I_FF)}
+    wt, sc, weight_bytes = {}, {}, 0
+    for name, (n, k) in shapes.items():
+        if w4:
+            wt[name] = torch.randint(0, 256, (layers, n, k // 2), dtype=torch.uint8, device="cuda")
+            sc[name] = torch.stack([torch.rand(layers, n, k // G, device="cuda") * 0.004 + 0.002,
+                                    torch.randint(0, 16, (layers, n, k // G), device="cuda").float()],
+                                   dim=-1).half().contiguous()
+        else:
+            wt[name] = torch.randint(-127, 128, (layers, n, k), dtype=torch.int8, device="cuda")
+            sc[name] = torch.rand(layers, n, dtype=torch.float32, device="cuda") * 2e-4 + 1e-4
+        weight_bytes += wt[name].numel() * wt[name].element_size() + sc[name].numel() * sc[name].element_size()
+    bq, bk, bv = w(layers, QD, std=0.1), w(layers, KD, std=0.1), w(layers, KD, std=0.1)
+    n_in, n_post = 1 + w(layers + 1, H, std=0.1), 1 + w(layers, H, std=0.1)
+    room = cache_len + 256
+    kc, vc = w(layers, room, NK, HD, std=1.0), w(layers, room, NK, HD, std=1.0)
+    hidden, normed = w(1, H, std=1.0), torch.empty(1, H, **f16)
+    q, k, v = torch.empty(1, QD, **f16), torch.empty(1, KD, **f16), torch.empty(1, KD, **f16)
+    attn, proj = torch.empty(1, QD, **f16), torch.empty(1, H, **f16)
+    gate, up, act = torch.empty(1, I_FF, **f16), torch.empty(1, I_FF, **f16), torch.empty(1, I_FF, **f16)
+    xq = torch.empty(1, I_FF, dtype=torch.int8, device="cuda")
+    sx = torch.empty(1, dtype=torch.float32, device="cuda")
+    xs = torch.empty(1, I_FF // 32, dtype=torch.int32, device="cuda")
+    pos = torch.tensor([cache_len - 1], dtype=torch.int32, device="cuda")
+    nxt = torch.tensor([cache_len], dtype=torch.int32, device="cuda")
+    scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
+    views = [dev.KvView(k=kc[l].data_ptr(), v=vc[l].data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                        format=0, n_kv_heads=NK, head_dim=HD) for l in range(layers)]
+
+    qkv, gu = [], []
+    for l in range(layers):
+        if a8:
+            a3, a2 = (dev.I8Proj * 3)(), (dev.I8Proj * 2)()
+            for i, (nm, b, y, n_) in enumerate((("q", bq, q, QD), ("k", bk, k, KD), ("v", bv, v, KD))):
+                a3[i] = dev.I8Proj(P(wt[nm][l]), P(sc[nm][l]), P(sc[nm][l]), P(b[l]), P(y), n_)
+            for i, (nm, y) in enumerate((("g", gate), ("u", up))):
+                a2[i] = dev.I8Proj(P(wt[nm][l]), P(sc[nm][l]), P(sc[nm][l]), None, P(y), I_FF)
+        else:
+            a3, a2 = (dev.W4A16Proj * 3)(), (dev.W4A16Proj * 2)()
+            for i, (nm, b, y, n_) in enumerate((("q", bq, q, QD), ("k", bk, k, KD), ("v", bv, v, KD))):
+                a3[i] = dev.W4A16Proj(P(wt[nm][l]), P(sc[nm][l]), P(b[l]), P(y), n_)
+            for i, (nm, y) in enumerate((("g", gate), ("u", up))):
+                a2[i] = dev.W4A16Proj(P(wt[nm][l]), P(sc[nm][l]), None, P(y), I_FF)
+        qkv.append(a3)
+        gu.append(a2)
+
+    def a8_linear(nm, l, n, kk, residual, y):
+        if w4:
+            assert dev.vv_w4a8_linear_dev(P(xq), lay, P(sx), P(xs), P(wt[nm][l]), P(sc[nm][l]), G, None, P(residual),
+                                          P(y), 0, 1, n, kk, 0, st) == 0
+        else:
+            assert dev.vv_w8a8_linear_dev(P(xq), P(sx), P(wt[nm][l]), P(sc[nm][l]), None, P(residual), P(y), 0, 1, n,
+                                          kk, 0, st) == 0
+
+    def common_attention(l):
+        assert dev.vv_rope_qk_dev(P(q), P(k), 1, NQ, NK, HD, 0, P(pos), THETA, st) == 0
+        assert dev.vv_dev_memcpy_d2d_at(P(kc[l]), P(k), KD * 2, P(pos), st) == 0
+        assert dev.vv_dev_memcpy_d2d_at(P(vc[l]), P(v), KD * 2, P(pos), st) == 0
+        assert dev.vv_attn_decode(2, P(q), C.addressof(views[l]), P(attn), NQ, cache_len, P(nxt), P(scratch), st) == 0
+        return 4
+
+    def token():
+        n = 1
+        if a8:
+            assert dev.vv_rmsnorm_q8_dev(P(hidden), P(n_in[0]), 1, H, EPS, lay, P(xq), P(sx), P(xs), st) == 0
+            for l in range(layers):
+                assert dev.vv_i8_linear_multi_dev(P(xq), lay, P(sx), P(xs), 1 if w4 else 0, C.addressof(qkv[l]), 3, G,
+                                                  1, H, st) == 0
+                n += 1 + common_attention(l)
+                assert dev.vv_act_quant_dev(P(attn), 1, QD, lay, P(xq), P(sx), P(xs), st) == 0
+                a8_linear("o", l, H, QD, hidden, hidden)
+                assert dev.vv_rmsnorm_q8_dev(P(hidden), P(n_post[l]), 1, H, EPS, lay, P(xq), P(sx), P(xs), st) == 0
+                assert dev.vv_i8_linear_multi_dev(P(xq), lay, P(sx), P(xs), 1 if w4 else 0, C.addressof(gu[l]), 2, G,
+                                                  1, H, st) == 0
+                assert dev.vv_swiglu_q8_dev(P(gate), P(up), 1, I_FF, lay, P(xq), P(sx), P(xs), st) == 0
+                a8_linear("d", l, H, I_FF, hidden, hidden)
+                assert dev.vv_rmsnorm_q8_dev(P(hidden), P(n_in[l + 1]), 1, H, EPS, lay, P(xq), P(sx), P(xs), st) == 0
+                n += 7
+        else:
+            assert dev.vv_rmsnorm_dev(P(hidden), P(n_in[0]), P(normed), 1, H, EPS, st) == 0
+            for l in range(layers):
+                assert dev.vv_w4a16_gemv_multi_dev(P(normed), C.addressof(qkv[l]), 3, H, G, st) == 0
+                n += 1 + common_attention(l)
+                assert dev.vv_w4a16_gemv_dev(P(attn), P(wt["o"][l]), P(sc["o"][l]), None, P(proj), H, QD, G, st) == 0
+                assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_post[l]), P(normed), 1, H, EPS, st) == 0
+                assert dev.vv_w4a16_gemv_multi_dev(P(normed), C.addressof(gu[l]), 2, H, G, st) == 0
+                assert dev.vv_swiglu_dev(P(gate), P(up), P(act), I_FF, st) == 0
+                assert dev.vv_w4a16_gemv_dev(P(act), P(wt["d"][l]), P(sc["d"][l]), None, P(proj), H, I_FF, G, st) == 0
+                assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_in[l + 1]), P(normed), 1, H, EPS, st) == 0
+                n += 6
+        assert dev.vv_pos_add_dev(P(pos), P(pos), 1, st) == 0
+        assert dev.vv_pos_add_dev(P(nxt), P(nxt), 1, st) == 0
+        return n + 2
+
+    torch.cuda.synchronize()
+    calls = token()
+    assert dev.vv_dev_stream_sync(st) == 0
+    reps = 10
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        token()
+    assert dev.vv_dev_stream_sync(st) == 0
+    eager = (time.perf_counter() - t0) / reps
+    assert dev.vv_dev_graph_begin(st) == 0
+    token()
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(st, C.byref(g)) == 0 and g.value
+    for _ in range(2):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    before = int(pos.item())
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        assert dev.vv_dev_graph_launch(g.value, st) == 0
+    assert dev.vv_dev_stream_sync(st) == 0
+    replay = (time.perf_counter() - t0) / reps
+    assert int(pos.item()) == before + reps
+    assert bool(torch.isfinite(hidden).all())
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(st)
+    return {"weights": kind, "layers": layers, "cache_len": cache_len, "calls": calls, "weight_bytes": weight_bytes,
+            "eager_ms": eager * 1e3, "graph_ms": replay * 1e3, "tokens_per_s": 1.0 / replay,
+            "weight_GBps": weight_bytes / replay / 1e9,
+            "frac_of_hbm_peak": weight_bytes / replay / 1e9 / HBM_PEAK_GBPS}
+
+
 def cpu_baseline(rows: int) -> dict:
     """The CPU path of the same step on `rows` rows: warm-up, then best of five
     (bench/benchmark.c:197-211). FP32 activations, so its byte count is its own."""
@@ -757,6 +902,13 @@ def main() -> int:
         log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
             f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
             f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+
+        for kind in ("w4a16", "w8a8", "w4a8"):
+            torch.cuda.empty_cache()
+            layer["decode_token_" + kind] = d = decode_token_quant_leg(torch, dev, T, kind)
+            log(f"  decode token, {kind} projections: {d['calls']} calls, eager {d['eager_ms']:.3f} ms, "
+                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at "
+                f"{d['weight_GBps']:.0f} GB/s ({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
 
     # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
     decode = {}

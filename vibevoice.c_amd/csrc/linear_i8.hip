@@ -125,13 +125,25 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
 // M <= MR <= 8 rows: kSplit waves per RW weight rows, each wave a contiguous
 // 1/kSplit of K. RW = 2 where a wave owns whole short rows: twice the bytes in
 // flight per wave, and the activation loads shared by both rows.
+// Up to three projections of the same activations in one launch: workgroups
+// [first[p], first[p + 1]) serve projection p and never straddle two.
+constexpr int kMaxSegs = 3;
+struct I8Segs {
+    const int8_t* w[kMaxSegs];
+    I8Out out[kMaxSegs];
+    int first[kMaxSegs + 1];
+};
+
 template <int MR, int kSplit, int RW>
-__global__ __launch_bounds__(kBlock) void i8_gemv(const int8_t* __restrict__ xq,
-                                                  const int8_t* __restrict__ w, I8Out out, int K) {
+__global__ __launch_bounds__(kBlock) void i8_gemv(const int8_t* __restrict__ xq, I8Segs segs, int K) {
     constexpr int kSets = kWavesPerBlock / kSplit;
     __shared__ int part[kWavesPerBlock][RW][MR];
     const int wave = wave_in_block(), lane = lane_id();
-    const int n0 = ((int)blockIdx.x * kSets + wave / kSplit) * RW;
+    const int b = (int)blockIdx.x;
+    const int seg = (b >= segs.first[1] ? 1 : 0) + (b >= segs.first[2] ? 1 : 0);
+    const I8Out out = segs.out[seg];
+    const int8_t* __restrict__ w = segs.w[seg];
+    const int n0 = ((b - segs.first[seg]) * kSets + wave / kSplit) * RW;
     const int piece = wave % kSplit;
     const int kchunks = K / 16;
     const int per = (kchunks + kSplit - 1) / kSplit;
@@ -267,19 +279,62 @@ void launch_i8_tile(const int8_t* xq, const int8_t* w, const I8Out& out, int K, 
         i8_tile<BM, BN, WM, WN, kSlabChunks, false, kAhead><<<grid, WM * WN * kWave, 0, st>>>(xq, w, out, K);
 }
 
+template <int MR, int kSplit, int RW>
+void launch_i8_gemv_cfg(const int8_t* xq, I8Segs segs, int n_segs, int K, hipStream_t st) {
+    constexpr int kRows = kWavesPerBlock / kSplit * RW;
+    int blocks = 0;
+    for (int i = 0; i <= kMaxSegs; ++i) {
+        segs.first[i] = i <= n_segs ? blocks : 0x7FFFFFFF;
+        if (i < n_segs) blocks += (segs.out[i].N + kRows - 1) / kRows;
+    }
+    for (int i = n_segs; i < kMaxSegs; ++i) { segs.w[i] = segs.w[0]; segs.out[i] = segs.out[0]; }
+    i8_gemv<MR, kSplit, RW><<<dim3((unsigned)blocks), kBlock, 0, st>>>(xq, segs, K);
+}
+
+// The configuration follows the rows of all projections together.
 template <int MR>
-void launch_i8_gemv(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
-    const int N = out.N;
-    if (N >= 16384 && K <= 8192) i8_gemv<MR, 1, 2><<<dim3((unsigned)((N + 7) / 8)), kBlock, 0, st>>>(xq, w, out, K);
-    else if (N >= 16384) i8_gemv<MR, 1, 1><<<dim3((unsigned)((N + 3) / 4)), kBlock, 0, st>>>(xq, w, out, K);
-    else if (N >= 8192) i8_gemv<MR, 2, 1><<<dim3((unsigned)((N + 1) / 2)), kBlock, 0, st>>>(xq, w, out, K);
-    else i8_gemv<MR, 4, 1><<<dim3((unsigned)N), kBlock, 0, st>>>(xq, w, out, K);
+void launch_i8_gemv(const int8_t* xq, const I8Segs& segs, int n_segs, int K, hipStream_t st) {
+    long N = 0;
+    for (int i = 0; i < n_segs; ++i) N += segs.out[i].N;
+    if (N >= 16384 && K <= 8192) launch_i8_gemv_cfg<MR, 1, 2>(xq, segs, n_segs, K, st);
+    else if (N >= 16384) launch_i8_gemv_cfg<MR, 1, 1>(xq, segs, n_segs, K, st);
+    else if (N >= 8192) launch_i8_gemv_cfg<MR, 2, 1>(xq, segs, n_segs, K, st);
+    else launch_i8_gemv_cfg<MR, 4, 1>(xq, segs, n_segs, K, st);
+}
+
+void launch_i8_gemv_rows(const int8_t* xq, const I8Segs& segs, int n_segs, int M, int K, hipStream_t st) {
+    if (M == 1) launch_i8_gemv<1>(xq, segs, n_segs, K, st);
+    else if (M == 2) launch_i8_gemv<2>(xq, segs, n_segs, K, st);
+    else if (M <= 4) launch_i8_gemv<4>(xq, segs, n_segs, K, st);
+    else launch_i8_gemv<8>(xq, segs, n_segs, K, st);
+}
+
+// The output descriptor of one W8A8 projection.
+I8Out make_out(const float* sx, const float* sw, const void* bias, const void* residual, void* y, int y_f32,
+               int M, int N) {
+    I8Out out;
+    out.sx = sx;
+    out.sw = sw;
+    out.bias = static_cast<const h16*>(bias);
+    out.res = static_cast<const h16*>(residual);
+    out.y = y;
+    out.y_f32 = y_f32 ? 1 : 0;
+    out.M = M;
+    out.N = N;
+    const auto mis = [](const void* p, unsigned mask) { return p && (reinterpret_cast<uintptr_t>(p) & mask); };
+    out.vec = (N % 4 == 0) && !mis(sw, 15u) && !mis(bias, 7u) && !mis(residual, 7u) && !mis(y, y_f32 ? 15u : 7u);
+    return out;
 }
 
 enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
 
 }  // namespace
 }  // namespace vv
+
+// linear_w4a8.hip: every projection of a W4A8 GEMV in one launch, or VV_ERR_UNSUPPORTED.
+__attribute__((visibility("hidden")))
+vv_status_t vv_w4a8_gemv_multi(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
+                               const vv_i8_proj_t* projs, int n, int group_size, int M, int K, void* stream);
 
 extern "C" {
 
@@ -292,25 +347,14 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
     if (K % 16 != 0 || !vv::aligned16(xq) || !vv::aligned16(w)) return VV_ERR_UNSUPPORTED;
     if (path == vv::kPathGemv && M > 8) return VV_ERR_UNSUPPORTED;
     hipStream_t st = vv::as_stream(stream);
-    vv::I8Out out;
-    out.sx = sx;
-    out.sw = sw;
-    out.bias = static_cast<const vv::h16*>(bias);
-    out.res = static_cast<const vv::h16*>(residual);
-    out.y = y;
-    out.y_f32 = y_f32 ? 1 : 0;
-    out.M = M;
-    out.N = N;
-    const auto mis = [](const void* p, unsigned mask) { return p && (reinterpret_cast<uintptr_t>(p) & mask); };
-    out.vec = (N % 4 == 0) && !mis(sw, 15u) && !mis(bias, 7u) && !mis(residual, 7u) &&
-              !mis(y, y_f32 ? 15u : 7u);
+    const vv::I8Out out = vv::make_out(sx, sw, bias, residual, y, y_f32, M, N);
 
     // AUTO keeps the dot-product kernel for one or two rows; from three the MFMA kernels are faster.
     if (path == vv::kPathGemv || (path == vv::kPathAuto && M <= 2)) {
-        if (M == 1) vv::launch_i8_gemv<1>(xq, w, out, K, st);
-        else if (M == 2) vv::launch_i8_gemv<2>(xq, w, out, K, st);
-        else if (M <= 4) vv::launch_i8_gemv<4>(xq, w, out, K, st);
-        else vv::launch_i8_gemv<8>(xq, w, out, K, st);
+        vv::I8Segs segs = {};
+        segs.w[0] = w;
+        segs.out[0] = out;
+        vv::launch_i8_gemv_rows(xq, segs, 1, M, K, st);
         return vv::launch_status();
     }
     // Beyond 16 rows a wide layer re-reads the activations once per 16 columns: tiles serve it better.
@@ -341,6 +385,25 @@ vv_status_t vv_i8_linear_multi_dev(const int8_t* xq, int x_layout, const float* 
     if (!xq || !sx || !projs) return VV_ERR_NULL_PTR;
     if (n < 1) return VV_ERR_INVALID_ARG;
     if (!w4 && x_layout != 0) return VV_ERR_UNSUPPORTED;   // W8A8 reads column order
+    if (w4) {
+        const vv_status_t s = vv_w4a8_gemv_multi(xq, x_layout, sx, xsum, projs, n, group_size, M, K, stream);
+        if (s != VV_ERR_UNSUPPORTED) return s;              // else: one call per projection
+    } else if (M <= 2 && n <= vv::kMaxSegs && K > 0 && K % 16 == 0 && vv::aligned16(xq)) {
+        // one or two rows: the dot-product kernel, every projection in ONE launch
+        vv::I8Segs segs = {};
+        bool ok = true;
+        for (int i = 0; i < n && ok; ++i) {
+            const vv_i8_proj_t& q = projs[i];
+            if (!q.w || !q.sw || !q.y) return VV_ERR_NULL_PTR;
+            ok = q.N > 0 && vv::aligned16(q.w);
+            segs.w[i] = static_cast<const int8_t*>(q.w);
+            segs.out[i] = vv::make_out(sx, static_cast<const float*>(q.sw), q.bias, nullptr, q.y, 0, M, q.N);
+        }
+        if (ok) {
+            vv::launch_i8_gemv_rows(xq, segs, n, M, K, vv::as_stream(stream));
+            return vv::launch_status();
+        }
+    }
     for (int i = 0; i < n; ++i) {
         const vv_i8_proj_t& q = projs[i];
         const vv_status_t s =

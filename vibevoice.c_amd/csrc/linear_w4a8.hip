@@ -163,16 +163,35 @@ __global__ __launch_bounds__(kBlock) void w4a8_gemv(W4Args a) {
 // (sum q x - z sum x) instead of being taken off every code.
 constexpr int kBlockTerms = 8192;      // FP32 group terms per workgroup (32 KB)
 
+// Up to three projections of the same activations in one launch: workgroups
+// [first[p], first[p + 1]) serve projection p and never straddle two.
+constexpr int kMaxSegs = 3;
+struct W4Segs {
+    const uint32_t* packed[kMaxSegs];
+    const uint32_t* sz[kMaxSegs];
+    const h16* bias[kMaxSegs];
+    void* y[kMaxSegs];
+    int n[kMaxSegs];
+    int first[kMaxSegs + 1];
+};
+
 template <int MR, int kSplit, int RW, bool kXsum>
-__global__ __launch_bounds__(kBlock) void w4a8_gemv_rows(W4Args a, const int32_t* __restrict__ xsum,
+__global__ __launch_bounds__(kBlock) void w4a8_gemv_rows(W4Args a, W4Segs segs, const int32_t* __restrict__ xsum,
                                                          int log2_per_group) {
     constexpr int kRows = kWavesPerBlock / kSplit * RW;    // weight rows per workgroup
     extern __shared__ float terms[];                       // [kRows][MR][groups]
     const int wave = wave_in_block(), lane = lane_id();
+    const int b = (int)blockIdx.x;
+    const int seg = (b >= segs.first[1] ? 1 : 0) + (b >= segs.first[2] ? 1 : 0);
+    a.packed = segs.packed[seg];
+    a.sz = segs.sz[seg];
+    a.bias = segs.bias[seg];
+    a.y = segs.y[seg];
+    a.N = segs.n[seg];
     const int nchunks = a.K / 32, ng = a.K / a.G;
     const int per_group = 1 << log2_per_group;
     const int set = wave / kSplit, piece = wave % kSplit;
-    const int n_blk = (int)blockIdx.x * kRows;
+    const int n_blk = (b - segs.first[seg]) * kRows;
     const u32x4* wrow[RW];
     const uint32_t* szrow[RW];
 #pragma unroll
@@ -243,32 +262,55 @@ __global__ __launch_bounds__(kBlock) void w4a8_gemv_rows(W4Args a, const int32_t
 }
 
 template <int MR, int kSplit, int RW>
-void launch_gemv_rows(const W4Args& a, const int32_t* xsum, int log2_pg, hipStream_t st) {
+void launch_gemv_rows(const W4Args& a, W4Segs segs, int n_segs, const int32_t* xsum, int log2_pg, hipStream_t st) {
     constexpr int kRows = kWavesPerBlock / kSplit * RW;
-    const dim3 grid((unsigned)((a.N + kRows - 1) / kRows));
+    int blocks = 0;
+    for (int i = 0; i <= kMaxSegs; ++i) {
+        segs.first[i] = i <= n_segs ? blocks : 0x7FFFFFFF;
+        if (i < n_segs) blocks += (segs.n[i] + kRows - 1) / kRows;
+    }
+    for (int i = n_segs; i < kMaxSegs; ++i) {
+        segs.packed[i] = segs.packed[0];
+        segs.sz[i] = segs.sz[0];
+        segs.bias[i] = nullptr;
+        segs.y[i] = segs.y[0];
+        segs.n[i] = 1;
+    }
+    const dim3 grid((unsigned)blocks);
     const size_t lds = (size_t)kRows * MR * (a.K / a.G) * sizeof(float);     // at most kBlockTerms floats
-    if (xsum) w4a8_gemv_rows<MR, kSplit, RW, true><<<grid, kBlock, lds, st>>>(a, xsum, log2_pg);
-    else w4a8_gemv_rows<MR, kSplit, RW, false><<<grid, kBlock, lds, st>>>(a, xsum, log2_pg);
+    if (xsum) w4a8_gemv_rows<MR, kSplit, RW, true><<<grid, kBlock, lds, st>>>(a, segs, xsum, log2_pg);
+    else w4a8_gemv_rows<MR, kSplit, RW, false><<<grid, kBlock, lds, st>>>(a, segs, xsum, log2_pg);
 }
 
+// The configuration follows the rows of all projections together.
 template <int MR>
-bool launch_gemv_fast(const W4Args& a, const int32_t* xsum, hipStream_t st) {
+bool launch_gemv_fast(const W4Args& a, const W4Segs& segs, int n_segs, const int32_t* xsum, hipStream_t st) {
     const int per_group = a.G / 32, ng = a.K / a.G, nchunks = a.K / 32;
     if (per_group > kWave || (per_group & (per_group - 1)) != 0) return false;
     int log2_pg = 0;
     while ((1 << log2_pg) < per_group) ++log2_pg;
+    long rows = 0;
+    for (int i = 0; i < n_segs; ++i) rows += segs.n[i];
     // Thousands of waves in flight, and no wave with less than half a round of chunks.
     int split = 1, rw = 1;
-    while (split < 4 && (long)a.N * split < 4096 && nchunks / (2 * split) >= kWave / 2) split *= 2;
-    while (split == 1 && rw < 4 && a.N / (2 * rw) >= 8192 && a.K * rw <= 8192) rw *= 2;
+    while (split < 4 && rows * split < 4096 && nchunks / (2 * split) >= kWave / 2) split *= 2;
+    while (split == 1 && rw < 4 && rows / (2 * rw) >= 8192 && a.K * rw <= 8192) rw *= 2;
     while (rw > 1 && kWavesPerBlock * rw * MR * ng > kBlockTerms) rw >>= 1;
     if (kWavesPerBlock / split * rw * MR * ng > kBlockTerms) return false;
-    if (rw == 4) launch_gemv_rows<MR, 1, 4>(a, xsum, log2_pg, st);
-    else if (rw == 2) launch_gemv_rows<MR, 1, 2>(a, xsum, log2_pg, st);
-    else if (split == 1) launch_gemv_rows<MR, 1, 1>(a, xsum, log2_pg, st);
-    else if (split == 2) launch_gemv_rows<MR, 2, 1>(a, xsum, log2_pg, st);
-    else launch_gemv_rows<MR, 4, 1>(a, xsum, log2_pg, st);
+    if (rw == 4) launch_gemv_rows<MR, 1, 4>(a, segs, n_segs, xsum, log2_pg, st);
+    else if (rw == 2) launch_gemv_rows<MR, 1, 2>(a, segs, n_segs, xsum, log2_pg, st);
+    else if (split == 1) launch_gemv_rows<MR, 1, 1>(a, segs, n_segs, xsum, log2_pg, st);
+    else if (split == 2) launch_gemv_rows<MR, 2, 1>(a, segs, n_segs, xsum, log2_pg, st);
+    else launch_gemv_rows<MR, 4, 1>(a, segs, n_segs, xsum, log2_pg, st);
     return true;
+}
+
+bool launch_gemv_fast_rows(const W4Args& a, const W4Segs& segs, int n_segs, const int32_t* xsum, hipStream_t st) {
+    const int mr = a.M == 1 ? 1 : a.M == 2 ? 2 : a.M <= 4 ? 4 : 8;
+    return mr == 1 ? launch_gemv_fast<1>(a, segs, n_segs, xsum, st)
+         : mr == 2 ? launch_gemv_fast<2>(a, segs, n_segs, xsum, st)
+         : mr == 4 ? launch_gemv_fast<4>(a, segs, n_segs, xsum, st)
+                   : launch_gemv_fast<8>(a, segs, n_segs, xsum, st);
 }
 
 // ── larger M: LDS-tiled int8 MFMA over codes unpacked on their way into LDS ─
@@ -488,6 +530,37 @@ enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
 }  // namespace
 }  // namespace vv
 
+// Every projection of a W4A8 GEMV (FP16 outputs, no residual) in ONE launch, each row computed
+// exactly as vv_w4a8_linear_dev would; VV_ERR_UNSUPPORTED (nothing launched) when the shape is not
+// the shuffle GEMV's, so that the caller runs one call per projection instead.
+__attribute__((visibility("hidden")))
+vv_status_t vv_w4a8_gemv_multi(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
+                               const vv_i8_proj_t* projs, int n, int group_size, int M, int K, void* stream) {
+    if (x_layout != vv::kLayoutGemv || M < 1 || M > 8 || n < 1 || n > vv::kMaxSegs) return VV_ERR_UNSUPPORTED;
+    if (K <= 0 || K % 32 != 0 || group_size <= 0 || group_size % 32 != 0 || K % group_size != 0)
+        return VV_ERR_UNSUPPORTED;
+    if (!vv::aligned16(xq) || (xsum && (reinterpret_cast<uintptr_t>(xsum) & 3u))) return VV_ERR_UNSUPPORTED;
+    vv::W4Args a = {};
+    a.xq = xq;
+    a.sx = sx;
+    a.M = M;
+    a.K = K;
+    a.G = group_size;
+    vv::W4Segs segs = {};
+    for (int i = 0; i < n; ++i) {
+        const vv_i8_proj_t& q = projs[i];
+        if (!q.w || !q.sz || !q.y) return VV_ERR_NULL_PTR;
+        if (q.N <= 0 || !vv::aligned16(q.w) || (reinterpret_cast<uintptr_t>(q.sz) & 3u)) return VV_ERR_UNSUPPORTED;
+        segs.packed[i] = static_cast<const uint32_t*>(q.w);
+        segs.sz[i] = static_cast<const uint32_t*>(q.sz);
+        segs.bias[i] = static_cast<const vv::h16*>(q.bias);
+        segs.y[i] = q.y;
+        segs.n[i] = q.N;
+    }
+    if (!vv::launch_gemv_fast_rows(a, segs, n, xsum, vv::as_stream(stream))) return VV_ERR_UNSUPPORTED;
+    return vv::launch_status();
+}
+
 extern "C" {
 
 vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, const int32_t* xsum,
@@ -528,10 +601,13 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
     if (path == vv::kPathGemv) {
         // xsum (may be NULL) is only read here: the other kernels take the zero point off the codes
         const int mr = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : 8;
-        const bool fast = mr == 1 ? vv::launch_gemv_fast<1>(a, xsum, st)
-                        : mr == 2 ? vv::launch_gemv_fast<2>(a, xsum, st)
-                        : mr == 4 ? vv::launch_gemv_fast<4>(a, xsum, st)
-                                  : vv::launch_gemv_fast<8>(a, xsum, st);
+        vv::W4Segs segs = {};
+        segs.packed[0] = a.packed;
+        segs.sz[0] = a.sz;
+        segs.bias[0] = a.bias;
+        segs.y[0] = a.y;
+        segs.n[0] = N;
+        const bool fast = vv::launch_gemv_fast_rows(a, segs, 1, xsum, st);
         if (fast) return vv::launch_status();
         if (K / 32 > vv::kGemvMaxChunks) return VV_ERR_UNSUPPORTED;
         const dim3 grid((unsigned)N);
