@@ -461,14 +461,15 @@ def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool =
         qkv.append(arr)
 
     def token_fused():
-        """The same step on the fused additions: q/k/v with their biases in one launch, gate/up/SwiGLU in one."""
+        """The same step on the fused additions: q/k/v with their biases in one launch, gate/up/SwiGLU in one,
+        K and V appended by one vv_kv_store_dev."""
         n = 1
         assert dev.vv_rmsnorm_dev(P(hidden), P(n_in[0]), P(normed), 1, H, EPS, st) == 0
         for l in range(layers):
             assert dev.vv_gemv_multi_dev(P(normed), C.addressof(qkv[l]), 3, H, st) == 0
             assert dev.vv_rope_qk_dev(P(q), P(k), 1, NQ, NK, HD, 0, P(pos), THETA, st) == 0
-            assert dev.vv_dev_memcpy_d2d_at(P(kc[l]), P(k), KD * 2, P(pos), st) == 0
-            assert dev.vv_dev_memcpy_d2d_at(P(vc[l]), P(v), KD * 2, P(pos), st) == 0
+            assert dev.vv_kv_store_dev(P(k), P(v), P(kc[l]), P(vc[l]), None, None, None, False, NK, HD, 0, P(pos), 1,
+                                       0, None, st) == 0
             assert dev.vv_attn_decode(2, P(q), C.addressof(views[l]), P(attn), NQ, cache_len, P(nxt),
                                       P(scratch), st) == 0
             gemv(attn, wo[l], proj, H, QD)
@@ -476,7 +477,7 @@ def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool =
             assert dev.vv_gemv_swiglu_dev(P(normed), P(wg[l]), P(wu[l]), P(act), I_FF, H, st) == 0
             gemv(act, wd[l], proj, H, I_FF)
             assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n_in[l + 1]), P(normed), 1, H, EPS, st) == 0
-            n += 11
+            n += 10
         assert dev.vv_pos_add_dev(P(pos), P(pos), 1, st) == 0
         assert dev.vv_pos_add_dev(P(nxt), P(nxt), 1, st) == 0
         return n + 2
@@ -616,10 +617,10 @@ def decode_token_quant_leg(torch, dev, cache_len: int, kind: str, layers: int = 
 
     def common_attention(l):
         assert dev.vv_rope_qk_dev(P(q), P(k), 1, NQ, NK, HD, 0, P(pos), THETA, st) == 0
-        assert dev.vv_dev_memcpy_d2d_at(P(kc[l]), P(k), KD * 2, P(pos), st) == 0
-        assert dev.vv_dev_memcpy_d2d_at(P(vc[l]), P(v), KD * 2, P(pos), st) == 0
+        assert dev.vv_kv_store_dev(P(k), P(v), P(kc[l]), P(vc[l]), None, None, None, False, NK, HD, 0, P(pos), 1, 0,
+                                   None, st) == 0
         assert dev.vv_attn_decode(2, P(q), C.addressof(views[l]), P(attn), NQ, cache_len, P(nxt), P(scratch), st) == 0
-        return 4
+        return 3
 
     def token():
         n = 1
