@@ -412,6 +412,98 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
             "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
 
 
+def prefill_layer_quant_leg(torch, dev, T: int, st: int, kind: str) -> dict:
+    """prefill_layer_leg with quantised projections. kind "w8a8" / "w4a8": int8 activations written by
+    the producing op (fused RMSNorm, attention output, fused SwiGLU), biases inside the linears, o and
+    down adding into the hidden state through the linear's residual (decoder.c:575-640, 795-932).
+    kind "w4a16": INT4 codes against FP16 activations with the decoder's dequant scratch."""
+    import ctypes as C
+    f16 = dict(dtype=torch.float16, device="cuda")
+    QD, KD, G = NQ * HD, NK * HD, 128
+    P = lambda t: t.data_ptr() if t is not None else None
+    a8, w4 = kind in ("w8a8", "w4a8"), kind in ("w4a16", "w4a8")
+    lay = 3 if kind == "w4a8" else 0                        # VV_Q8_W4_MMA for the tiles, else column order
+    w = lambda *shape, std: torch.randn(*shape, **f16) * std
+    shapes = {"q": (QD, H), "k": (KD, H), "v": (KD, H), "o": (H, QD), "g": (I_FF, H), "u": (I_FF, H), "d": (H, I_FF)}
+    wt, sc = {}, {}
+    for name, (n, k) in shapes.items():
+        if w4:
+            wt[name] = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
+            sc[name] = torch.stack([torch.rand(n, k // G, device="cuda") * 0.004 + 0.002,
+                                    torch.randint(0, 16, (n, k // G), device="cuda").float()], dim=-1).half().contiguous()
+        else:
+            wt[name] = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+            sc[name] = torch.rand(n, dtype=torch.float32, device="cuda") * 2e-4 + 1e-4
+    bias = {"q": w(QD, std=0.1), "k": w(KD, std=0.1), "v": w(KD, std=0.1)}
+    n1, n2 = 1 + w(H, std=0.1), 1 + w(H, std=0.1)
+    hidden, normed, proj = w(T, H, std=1.0), torch.empty(T, H, **f16), torch.empty(T, H, **f16)
+    q, attn = torch.empty(T, QD, **f16), torch.empty(T, QD, **f16)
+    k, v = torch.empty(T, KD, **f16), torch.empty(T, KD, **f16)
+    gate, up = torch.empty(T, I_FF, **f16), torch.empty(T, I_FF, **f16)
+    xq = torch.empty(T, I_FF, dtype=torch.int8, device="cuda")
+    sx = torch.empty(T, dtype=torch.float32, device="cuda")
+    xs = torch.empty(T, I_FF // 32, dtype=torch.int32, device="cuda")
+    dense = torch.empty(I_FF * H, **f16) if kind == "w4a16" else None
+    view = dev.KvView(k=k.data_ptr(), v=v.data_ptr(), k_meta=None, v_meta=None, page_table=None, format=0,
+                      n_kv_heads=NK, head_dim=HD)
+
+    def linear(nm, x, y, n, kk, residual=None):
+        if kind == "w4a16":
+            assert dev.vv_w4a16_gemm_dev(P(x), P(wt[nm]), P(sc[nm]), P(bias.get(nm)), P(y), P(dense), dense.numel() * 2,
+                                         T, n, kk, G, st) == 0
+        elif kind == "w4a8":
+            assert dev.vv_w4a8_linear_dev(P(xq), lay, P(sx), P(xs), P(wt[nm]), P(sc[nm]), G, P(bias.get(nm)),
+                                          P(residual), P(y), 0, T, n, kk, 0, st) == 0
+        else:
+            assert dev.vv_w8a8_linear_dev(P(xq), P(sx), P(wt[nm]), P(sc[nm]), P(bias.get(nm)), P(residual), P(y), 0,
+                                          T, n, kk, 0, st) == 0
+
+    def layer():
+        if a8:
+            assert dev.vv_rmsnorm_q8_dev(P(hidden), P(n1), T, H, EPS, lay, P(xq), P(sx), P(xs), st) == 0
+        else:
+            assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0
+        linear("q", normed, q, QD, H)
+        linear("k", normed, k, KD, H)
+        linear("v", normed, v, KD, H)
+        assert dev.vv_rope_qk_dev(P(q), P(k), T, NQ, NK, HD, 0, None, THETA, st) == 0
+        assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, T, 0, T, True, None, st) == 0
+        if a8:
+            assert dev.vv_act_quant_dev(P(attn), T, QD, lay, P(xq), P(sx), P(xs), st) == 0
+            linear("o", attn, hidden, H, QD, residual=hidden)
+            assert dev.vv_rmsnorm_q8_dev(P(hidden), P(n2), T, H, EPS, lay, P(xq), P(sx), P(xs), st) == 0
+        else:
+            linear("o", attn, proj, H, QD)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n2), P(normed), T, H, EPS, st) == 0
+        linear("g", normed, gate, I_FF, H)
+        linear("u", normed, up, I_FF, H)
+        if a8:
+            assert dev.vv_swiglu_q8_dev(P(gate), P(up), T, I_FF, lay, P(xq), P(sx), P(xs), st) == 0
+            linear("d", gate, hidden, H, I_FF, residual=hidden)
+        else:
+            assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), T * I_FF, st) == 0
+            linear("d", gate, proj, H, I_FF)
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
+
+    layer()
+    torch.cuda.synchronize()
+    per = []
+    for _ in range(3):
+        hidden.normal_()                                   # the residual path of the a8 forms grows otherwise
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        layer()
+        e1.record()
+        e1.synchronize()
+        per.append(e0.elapsed_time(e1))
+    per.sort()
+    ms = per[1]
+    assert bool(torch.isfinite(hidden).all())
+    ops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
+    return {"weights": kind, "rows": T, "ms_per_layer": ms, "Tops": ops / ms / 1e9, "layers_assumed": 28,
+            "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
+
+
 def decode_token_leg(torch, dev, cache_len: int, layers: int = 28, fused: bool = False) -> dict:
     """One decode step of a dense Qwen2-7B-shaped decoder (random weights, 13 GB of them) on this
     library's entry points alone, in the reference decoder's op order (decoder.c:706-991): per layer
@@ -895,6 +987,11 @@ def main() -> int:
         layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
         log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention); "
             f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
+        for kind in ("w8a8", "w4a8", "w4a16"):
+            torch.cuda.empty_cache()
+            layer["prefill_layer_" + kind] = d = prefill_layer_quant_leg(torch, dev, T, st, kind)
+            log(f"  prefill layer, {kind} projections: {d['ms_per_layer']:.2f} ms ({d['Tops']:.0f} TOP/s over linears + "
+                f"attention); 28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
         layer["decode_token"] = d = decode_token_leg(torch, dev, T)
         log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
             f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "

@@ -26,7 +26,7 @@
 //                           output column stream that weight row once with
 //                           non-temporal 16-byte loads.
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
-#include "mfma_tile.hpp"
+#include "mfma_dma.hpp"
 #include "row_math.hpp"
 
 namespace vv {
@@ -96,149 +96,15 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
     mfma_tile<F16Op, BM, BN, WM, WN, kSlab / 8, kFull, kAhead>(A, B, M, N, K / 8, epilogue);
 }
 
-// The 256x256 tile again, with the slabs going from global memory STRAIGHT into
-// LDS (global_load_lds_dwordx4: each lane's 16 bytes land at M0 + lane * 16, no
-// staging registers) and four LDS stages, so a slab is requested three compute
-// phases before it is read: deep enough to hide a last-level-cache miss. The
-// copy is asynchronous and the compiler is not told about it (it would wait for
-// ALL outstanding copies before any LDS read): the wave counts its own copies
-// with s_waitcnt vmcnt, then the workgroup barrier makes every wave's part
-// visible. Since a lane cannot choose where its bytes land, the bank swizzle is
-// applied on the global side: the lane that owns LDS slot (row, p) fetches the
-// row's logical slot p ^ swizzle(row). Needs K % 32 == 0 (no zero fill).
-constexpr int kDmaStages = 4;
-constexpr int kDmaSlab = 32;
-constexpr int kDmaTile = 256;
-constexpr int kDmaWaves = 8;
-constexpr int kDmaStageSlots = 2 * kDmaTile * (kDmaSlab / 8);   // 16-byte slots per stage: A rows, then B rows
-constexpr size_t kDmaLdsBytes = (size_t)kDmaStages * kDmaStageSlots * 16;
-
-// One wave-wide copy: lane l's 16 bytes at gptr go to LDS byte lds_byte_addr + 16 l.
-__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :
-                 : "s"(lds_byte_addr), "v"(gptr)
-                 : "memory", "m0");
-}
-
+// The 256x256 tile with the slabs copied from global memory straight into LDS
+// (mfma_dma.hpp). Needs K % 32 == 0.
 __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
     int K, float alpha, float beta, int vec_store) {
-    constexpr int kSlabChunks = kDmaSlab / 8;             // 4
-    constexpr int WN = 4, TM = 4, TN = 2;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
-    constexpr int kLoads = kDmaStageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 4
-    extern __shared__ u32x4 dma_lds[];
-
-    const int tid = (int)threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WN, wn = wave % WN;
-    const int m_blk = (int)blockIdx.y * kDmaTile;
-    const int n_blk = (int)blockIdx.x * kDmaTile;
-    const int nslabs = K / kDmaSlab;
-    const uint32_t lds0 =
-        (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
-
-    // Copy i of this wave fills slots (wave + 8i) * 64 .. + 63 of a stage: 16
-    // rows x 4 slots. The lane owns (row, physical slot) and fetches the logical
-    // slot that the swizzle maps there.
-    const char* src[kLoads];
-    uint32_t dst[kLoads];
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-        const int slot0 = (wave + kDmaWaves * i) * kWave;
-        const int p = slot0 + lane;
-        const int row = p / kSlabChunks, phys = p % kSlabChunks;    // row 0..511: A rows then B rows
-        const int logical = swz<kDmaSlab>(row, phys);
-        const bool is_b = row >= kDmaTile;
-        const int r = is_b ? row - kDmaTile : row;
-        const h16* base = is_b ? B + (size_t)min(n_blk + r, N - 1) * K : A + (size_t)min(m_blk + r, M - 1) * K;
-        src[i] = reinterpret_cast<const char*>(base) + logical * 16;
-        dst[i] = lds0 + (uint32_t)slot0 * 16u;
-    }
-    auto request = [&](int slab) {        // slab -> stage slab % 4; past the end: the last slab again
-        const size_t adv = (size_t)min(slab, nslabs - 1) * (kDmaSlab * 2);
-        const uint32_t stage = (uint32_t)(slab % kDmaStages) * (kDmaStageSlots * 16u);
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) lds_dma16(src[i] + adv, dst[i] + stage);
+    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
+        store_tile<4, 2>(acc, C, M, N, m0, n0, frow, fhalf, alpha, beta, vec_store);
     };
-
-    f32x16 acc[TN][TM];
-#pragma unroll
-    for (int a = 0; a < TN; ++a)
-#pragma unroll
-        for (int b = 0; b < TM; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
-
-    const int frow = lane & 31, fhalf = lane >> 5;
-    int f_idx[2];
-#pragma unroll
-    for (int step = 0; step < 2; ++step)
-        f_idx[step] = frow * kSlabChunks + swz<kDmaSlab>(frow, step * 2 + fhalf);
-    const int fa_base = wm * TM * 32 * kSlabChunks;
-    const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
-
-    // Fragment reads run a whole slab ahead: while the 16 MFMAs of slab s execute
-    // from one register set, the operands of slab s + 1 come in from LDS into the
-    // other (an LDS queue that is two thirds busy answers too late for anything
-    // shorter).
-    h16x8 fw[2][2][TN], fx[2][2][TM];          // [set][K step][tile]
-    auto read_frags = [&](auto set_c, int slab, int step) {
-        constexpr int set = decltype(set_c)::value;
-        const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
-#pragma unroll
-        for (int a = 0; a < TN; ++a)
-            fw[set][step][a] = __builtin_bit_cast(h16x8, st[fb_base + a * 32 * kSlabChunks + f_idx[step]]);
-#pragma unroll
-        for (int b = 0; b < TM; ++b)
-            fx[set][step][b] = __builtin_bit_cast(h16x8, st[fa_base + b * 32 * kSlabChunks + f_idx[step]]);
-    };
-    auto mfma_group = [&](auto set_c, int step) {
-        constexpr int set = decltype(set_c)::value;
-#pragma unroll
-        for (int a = 0; a < TN; ++a)
-#pragma unroll
-            for (int b = 0; b < TM; ++b)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[set][step][a], fx[set][step][b],
-                                                                   acc[a][b], 0, 0, 0);
-    };
-    // One slab: its operands are (being) loaded in set `cur`; slab + 1 must be in
-    // LDS (this wave's copies of slabs + 2 and + 3, 8 of them, may still fly) and
-    // every wave must have its operands of this slab in registers before the
-    // stage is handed to slab + 4.
-    auto one_slab = [&](auto cur_c, auto nxt_c, int slab) {
-        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-        request(slab + 4);
-        read_frags(nxt_c, slab + 1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_group(cur_c, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(nxt_c, slab + 1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_group(cur_c, 1);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    request(0);
-    request(1);
-    request(2);
-    request(3);
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    __syncthreads();
-    read_frags(Const<0>{}, 0, 0);
-    read_frags(Const<0>{}, 0, 1);
-    int slab = 0;
-    for (; slab + 2 <= nslabs; slab += 2) {
-        one_slab(Const<0>{}, Const<1>{}, slab);
-        one_slab(Const<1>{}, Const<0>{}, slab + 1);
-    }
-    if (slab < nslabs) one_slab(Const<0>{}, Const<1>{}, slab);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
-
-    store_tile<TM, TN>(acc, C, M, N, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf, alpha, beta,
-                       vec_store);
+    mfma_dma<F16Op>(A, B, M, N, K * 2, epilogue);
 }
 
 // M == 1: bound by the weight bytes. kSplit waves share an output column (a
@@ -592,7 +458,7 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
     }
     switch (choice) {
         case k256:
-            if (K % kDmaSlab == 0 && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
+            if (K % (kDmaSlabBytes / 2) == 0 && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
             [[fallthrough]];
         case k256regs: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;

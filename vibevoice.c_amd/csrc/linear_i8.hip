@@ -14,7 +14,7 @@
 //             MFMA operands, K split over the eight waves of a workgroup.
 //   i8_gemv   M <= 8: one to four waves per weight row, v_dot4_i32_i8 against
 //             up to eight activation rows that share each weight load.
-#include "mfma_tile.hpp"
+#include "mfma_dma.hpp"
 
 namespace vv {
 namespace {
@@ -88,29 +88,47 @@ __device__ __forceinline__ void i8_store4(const I8Out& o, int m, int n, const in
     }
 }
 
+// A wave's TN x TM accumulator tiles through the epilogue: register 4g + r of
+// lane l holds column n0 + 32a + 8g + 4(l / 32) + r of row m0 + 32b + l % 32.
+template <int TM, int TN>
+__device__ __forceinline__ void i8_epilogue(const i32x16 (&acc)[TN][TM], const I8Out& out, int m0, int n0,
+                                            int frow, int fhalf) {
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const int m = m0 + b * 32 + frow;
+        if (m >= out.M) continue;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + a * 32 + 8 * g + 4 * fhalf;
+                if (n >= out.N) continue;
+                const int t[4] = {acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2],
+                                  acc[a][b][4 * g + 3]};
+                i8_store4(out, m, n, t);
+            }
+    }
+}
+
 template <int BM, int BN, int WM, int WN, int kSlabChunks, bool kFull, int kAhead>
 __global__ __launch_bounds__(WM * WN * kWave) void i8_tile(const int8_t* __restrict__ xq,
                                                            const int8_t* __restrict__ w, I8Out out,
                                                            int K) {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     auto epilogue = [=](const i32x16 (&acc)[TN][TM], int m0, int n0, int frow, int fhalf) {
-#pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const int m = m0 + b * 32 + frow;
-            if (m >= out.M) continue;
-#pragma unroll
-            for (int a = 0; a < TN; ++a)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + a * 32 + 8 * g + 4 * fhalf;
-                    if (n >= out.N) continue;
-                    const int t[4] = {acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2],
-                                      acc[a][b][4 * g + 3]};
-                    i8_store4(out, m, n, t);
-                }
-        }
+        i8_epilogue<TM, TN>(acc, out, m0, n0, frow, fhalf);
     };
     mfma_tile<I8Op, BM, BN, WM, WN, kSlabChunks, kFull, kAhead>(xq, w, out.M, out.N, K / 16, epilogue);
+}
+
+// The 256 x 256 tile with the slabs copied from global memory straight into LDS
+// (mfma_dma.hpp): K % 64 == 0.
+__global__ __launch_bounds__(kDmaWaves * kWave) void i8_dma(const int8_t* __restrict__ xq,
+                                                            const int8_t* __restrict__ w, I8Out out, int K) {
+    auto epilogue = [=](const i32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
+        i8_epilogue<4, 2>(acc, out, m0, n0, frow, fhalf);
+    };
+    mfma_dma<I8Op>(xq, w, out.M, out.N, K, epilogue);
 }
 
 __device__ __forceinline__ int wave_sum_i32(int v) {
@@ -279,6 +297,24 @@ void launch_i8_tile(const int8_t* xq, const int8_t* w, const I8Out& out, int K, 
         i8_tile<BM, BN, WM, WN, kSlabChunks, false, kAhead><<<grid, WM * WN * kWave, 0, st>>>(xq, w, out, K);
 }
 
+bool launch_i8_dma(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
+    // 128 KB of LDS per workgroup is above the default limit: raised once per thread and device.
+    static thread_local int ready_device = -1;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return false;
+    if (ready_device != device) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(i8_dma), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kDmaLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        ready_device = device;
+    }
+    const dim3 grid((unsigned)((out.N + kDmaTile - 1) / kDmaTile), (unsigned)((out.M + kDmaTile - 1) / kDmaTile));
+    i8_dma<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(xq, w, out, K);
+    return true;
+}
+
 template <int MR, int kSplit, int RW>
 void launch_i8_gemv_cfg(const int8_t* xq, I8Segs segs, int n_segs, int K, hipStream_t st) {
     constexpr int kRows = kWavesPerBlock / kSplit * RW;
@@ -370,7 +406,9 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
     // The largest tile that still fills the 256 compute units (as for FP16).
     const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (wg256 >= 512) vv::launch_i8_tile<256, 256, 2, 4, 4, 2>(xq, w, out, K, st);
+    static const bool no_dma = [] { const char* e = getenv("VV_I8_NO_DMA"); return e && e[0] == '1'; }();
+    if (wg256 >= 512 && K % vv::kDmaSlabBytes == 0 && !no_dma && vv::launch_i8_dma(xq, w, out, K, st)) {}
+    else if (wg256 >= 512) vv::launch_i8_tile<256, 256, 2, 4, 4, 2>(xq, w, out, K, st);
     else if (M > 64 && wg128 >= 256) vv::launch_i8_tile<128, 128, 2, 2, 8, 2>(xq, w, out, K, st);
     else if (M > 32) vv::launch_i8_tile<64, 64, 2, 2, 8, 1>(xq, w, out, K, st);
     else vv::launch_i8_tile<32, 64, 1, 2, 8, 1>(xq, w, out, K, st);

@@ -1,0 +1,156 @@
+// The 256x256 tile with direct global-to-LDS copies, shared by the FP16 GEMM and
+// the W8A8 linear layer (both operands K-contiguous, rows of `row_bytes`).
+#pragma once
+
+#include "mfma_tile.hpp"
+
+namespace vv {
+
+// The slabs go from global memory STRAIGHT into
+// LDS (global_load_lds_dwordx4: each lane's 16 bytes land at M0 + lane * 16, no
+// staging registers) and four LDS stages, so a slab is requested three compute
+// phases before it is read: deep enough to hide a last-level-cache miss. The
+// copy is asynchronous and the compiler is not told about it (it would wait for
+// ALL outstanding copies before any LDS read): the wave counts its own copies
+// with s_waitcnt vmcnt, then the workgroup barrier makes every wave's part
+// visible. Since a lane cannot choose where its bytes land, the bank swizzle is
+// applied on the global side: the lane that owns LDS slot (row, p) fetches the
+// row's logical slot p ^ swizzle(row). Rows must be whole slabs (no zero fill):
+// K % 32 == 0 for FP16, K % 64 == 0 for int8. Op and the epilogue are those of
+// mfma_tile; the wave tile is TN x TM = 2 x 4 products of 32 x 32.
+constexpr int kDmaStages = 4;
+constexpr int kDmaSlabBytes = 64;       // one slab: 64 bytes of every row (32 halves, 64 int8)
+constexpr int kDmaTile = 256;
+constexpr int kDmaWaves = 8;
+constexpr int kDmaStageSlots = 2 * kDmaTile * (kDmaSlabBytes / 16);   // 16-byte slots per stage: A rows, then B rows
+constexpr size_t kDmaLdsBytes = (size_t)kDmaStages * kDmaStageSlots * 16;
+
+// One wave-wide copy: lane l's 16 bytes at gptr go to LDS byte lds_byte_addr + 16 l.
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_byte_addr), "v"(gptr)
+                 : "memory", "m0");
+}
+
+template <typename Op, typename Epi>
+__device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
+                                         int row_bytes, const Epi& epi) {
+    typedef typename Op::Acc Acc;
+    constexpr int kSlabChunks = kDmaSlabBytes / 16;       // 4
+    constexpr int WN = 4, TM = 4, TN = 2;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
+    constexpr int kLoads = kDmaStageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 4
+    extern __shared__ u32x4 dma_lds[];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int m_blk = (int)blockIdx.y * kDmaTile;
+    const int n_blk = (int)blockIdx.x * kDmaTile;
+    const int nslabs = row_bytes / kDmaSlabBytes;
+    const uint32_t lds0 =
+        (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
+
+    // Copy i of this wave fills slots (wave + 8i) * 64 .. + 63 of a stage: 16
+    // rows x 4 slots. The lane owns (row, physical slot) and fetches the logical
+    // slot that the swizzle maps there.
+    const char* src[kLoads];
+    uint32_t dst[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const int slot0 = (wave + kDmaWaves * i) * kWave;
+        const int p = slot0 + lane;
+        const int row = p / kSlabChunks, phys = p % kSlabChunks;    // row 0..511: A rows then B rows
+        const int logical = swz<32>(row, phys);
+        const bool is_b = row >= kDmaTile;
+        const int r = is_b ? row - kDmaTile : row;
+        const char* base = is_b ? static_cast<const char*>(B) + (size_t)min(n_blk + r, N - 1) * row_bytes
+                                : static_cast<const char*>(A) + (size_t)min(m_blk + r, M - 1) * row_bytes;
+        src[i] = base + logical * 16;
+        dst[i] = lds0 + (uint32_t)slot0 * 16u;
+    }
+    auto request = [&](int slab) {        // slab -> stage slab % 4; past the end: the last slab again
+        const size_t adv = (size_t)min(slab, nslabs - 1) * kDmaSlabBytes;
+        const uint32_t stage = (uint32_t)(slab % kDmaStages) * (kDmaStageSlots * 16u);
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) lds_dma16(src[i] + adv, dst[i] + stage);
+    };
+
+    Acc acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    int f_idx[2];
+#pragma unroll
+    for (int step = 0; step < 2; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<32>(frow, step * 2 + fhalf);
+    const int fa_base = wm * TM * 32 * kSlabChunks;
+    const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
+
+    // Fragment reads run a whole slab ahead: while the 16 MFMAs of slab s execute
+    // from one register set, the operands of slab s + 1 come in from LDS into the
+    // other (an LDS queue that is two thirds busy answers too late for anything
+    // shorter).
+    u32x4 fw[2][2][TN], fx[2][2][TM];          // [set][K step][tile]
+    auto read_frags = [&](auto set_c, int slab, int step) {
+        constexpr int set = decltype(set_c)::value;
+        const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+            fw[set][step][a] = st[fb_base + a * 32 * kSlabChunks + f_idx[step]];
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+            fx[set][step][b] = st[fa_base + b * 32 * kSlabChunks + f_idx[step]];
+    };
+    auto mfma_group = [&](auto set_c, int step) {
+        constexpr int set = decltype(set_c)::value;
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                acc[a][b] = Op::mfma(fw[set][step][a], fx[set][step][b], acc[a][b]);
+    };
+    // One slab: its operands are (being) loaded in set `cur`; slab + 1 must be in
+    // LDS (this wave's copies of slabs + 2 and + 3, 8 of them, may still fly) and
+    // every wave must have its operands of this slab in registers before the
+    // stage is handed to slab + 4.
+    auto one_slab = [&](auto cur_c, auto nxt_c, int slab) {
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        request(slab + 4);
+        read_frags(nxt_c, slab + 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(cur_c, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(nxt_c, slab + 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(cur_c, 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    request(0);
+    request(1);
+    request(2);
+    request(3);
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __syncthreads();
+    read_frags(Const<0>{}, 0, 0);
+    read_frags(Const<0>{}, 0, 1);
+    int slab = 0;
+    for (; slab + 2 <= nslabs; slab += 2) {
+        one_slab(Const<0>{}, Const<1>{}, slab);
+        one_slab(Const<1>{}, Const<0>{}, slab + 1);
+    }
+    if (slab < nslabs) one_slab(Const<0>{}, Const<1>{}, slab);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
+
+    epi(acc, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf);
+}
+
+}  // namespace vv
