@@ -279,17 +279,17 @@ vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
 typedef struct vv_kv_view {
     const void* k;
     const void* v;
-    const void* k_meta;       /* quantised formats only: unused here */
+    const void* k_meta;       /* TurboQuant formats only: unused here */
     const void* v_meta;
     const int*  page_table;   /* device memory, or NULL */
-    int         format;       /* vv_kv_format_t; only VV_KV_FP16 (0) is served */
+    int         format;       /* vv_kv_format_t: VV_KV_FP16 (0), VV_KV_FP8_E4M3 (1), VV_KV_FP8_E5M2 (2) */
     int         n_kv_heads;
     int         head_dim;
 } vv_kv_view_t;
 
 /* The backend a context should name (never VV_ATTN_AUTO = 0). All backend
- * names run the same kernels here; a format other than FP16 answers
- * VV_ATTN_FA1 (1) and the attention calls then decline.
+ * names run the same kernels here; a TurboQuant format (or FP8 at a head_dim
+ * other than 128) answers VV_ATTN_FA1 (1) and the attention calls then decline.
  * replaces device.h:545-546 (src/cuda/attention_fi.cu:554-583). */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
                     int n_kv_heads, int head_dim);
@@ -336,14 +336,45 @@ vv_status_t vv_gqa_attention_prefill_dev(const void* q, const void* k, const voi
                                          void* output, int n_q_heads, int n_kv_heads,
                                          int head_dim, int seq_len, bool causal,
                                          void* stream);
-/* Copy K/V rows [n_positions][n_kv_heads][head_dim] into an FP16 cache layer
- * at positions pos.. (or *d_pos..), through page_table when it is set.
- * Other formats: VV_ERR_UNSUPPORTED. replaces device.h:597-602. */
+/* Write K/V rows [n_positions][n_kv_heads][head_dim] into a cache layer at
+ * positions pos.. (or *d_pos..), through page_table when it is set. FP16: a
+ * copy. FP8 (E4M3 / E5M2, head_dim 128): each value encoded in integer
+ * arithmetic exactly as src/cuda/kv_codec.cuh:66-128 (round to nearest even,
+ * saturating, NaN -> 0); when k_ref is set the head's reference key is
+ * subtracted from K first (softmax does not see a shift common to all keys),
+ * and with build_ref it is first computed as this run's mean key. TurboQuant
+ * formats: VV_ERR_UNSUPPORTED. replaces device.h:597-602
+ * (src/cuda/kv_quant.cu:507-552). */
 vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_store,
                             void* v_store, void* k_meta, void* v_meta, void* k_ref,
                             bool build_ref, int n_kv_heads, int head_dim, int pos,
                             const int* d_pos, int n_positions, int kv_format,
                             const int* page_table, void* stream);
+/* The same without a page table, quantised formats only (FP16:
+ * VV_ERR_UNSUPPORTED). replaces device.h:689-694 (kv_quant.cu:554-567). */
+vv_status_t vv_kv_quant_store_dev(const void* k_fp16, const void* v_fp16, void* k_store,
+                                  void* v_store, void* k_meta, void* v_meta, void* k_ref,
+                                  bool build_ref, int n_kv_heads, int head_dim, int pos,
+                                  const int* d_pos, int n_positions, int kv_format, void* stream);
+/* An FP8 store [n_pos][n_kv_heads][128] back to FP16, plus `ref` [n_kv_heads][128]
+ * when given. replaces device.h:697-699 (kv_quant.cu:586-603). */
+vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* ref,
+                              void* out_fp16, int n_kv_heads, int head_dim, int n_pos,
+                              int kv_format, void* stream);
+/* Attention over a quantised cache given as pointers: vv_attn_decode /
+ * vv_attn_prefill with the format in the view. Every FP8 value is an FP16
+ * value, so the result is, bit for bit, that of an FP16 cache holding the
+ * decoded values. replace device.h:662-675 (kv_quant.cu:605-673). */
+vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, const void* v_store,
+                                          const void* k_meta, const void* v_meta, void* output,
+                                          int n_q_heads, int n_kv_heads, int head_dim,
+                                          int cache_len, const int* d_cache_len, int kv_format,
+                                          void* scratch, void* stream);
+vv_status_t vv_gqa_attention_prefill_q_dev(const void* q, const void* k_store, const void* v_store,
+                                           const void* k_meta, const void* v_meta, void* output,
+                                           int n_q_heads, int n_kv_heads, int head_dim, int q_len,
+                                           int q_offset, int kv_len, bool causal, int kv_format,
+                                           void* stream);
 /* page_table[first + i] = pages[i], i < n, ordered on the stream; `pages` is
  * host memory, consumed before the call returns. replaces device.h:610-611. */
 vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages,

@@ -86,6 +86,12 @@ def _load():
                                             C.c_void_p]
     lib.vvo_int4g_dequant_f16.restype = C.c_int
     lib.vvo_int4g_dequant_f16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    for name, args in (("vvo_fp8_encode", [_f32p, C.c_int, C.c_int, C.c_void_p]),
+                       ("vvo_fp8_decode", [C.c_void_p, C.c_int, C.c_int, _f32p]),
+                       ("vvo_kv_build_ref", [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+                       ("vvo_kv_store_fp8", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p])):
+        getattr(lib, name).restype = C.c_int
+        getattr(lib, name).argtypes = args
     lib.vvo_argmax_first.restype = C.c_int
     lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
@@ -406,4 +412,41 @@ def int4g_dequant_f16(packed, scales16, zeros, G):
     out = np.empty((N, K), np.uint16)
     _check(lib.vvo_int4g_dequant_f16(packed.ctypes.data, scales16.ctypes.data, zeros.ctypes.data, N, K, G,
                                      out.ctypes.data), "int4g_dequant_f16")
+    return out
+
+
+def fp8_encode(x, e5m2: bool) -> np.ndarray:
+    """float32 values -> FP8 codes (uint8, same shape)."""
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(x.shape, np.uint8)
+    _check(lib.vvo_fp8_encode(_p(x, _f32p), x.size, int(e5m2), out.ctypes.data), "fp8_encode")
+    return out
+
+
+def fp8_decode(codes, e5m2: bool) -> np.ndarray:
+    """FP8 codes -> float32 values (same shape)."""
+    codes = np.ascontiguousarray(codes, np.uint8)
+    out = np.empty(codes.shape, np.float32)
+    _check(lib.vvo_fp8_decode(codes.ctypes.data, codes.size, int(e5m2), _p(out, _f32p)), "fp8_decode")
+    return out
+
+
+def kv_build_ref(k16) -> np.ndarray:
+    """FP16 keys [n_pos, n_kv_heads, head_dim] -> their per-head mean, FP16 bits [n_kv_heads, head_dim]."""
+    k16 = np.ascontiguousarray(k16, np.uint16)
+    n_pos, nkv, hd = k16.shape
+    ref = np.empty((nkv, hd), np.uint16)
+    _check(lib.vvo_kv_build_ref(k16.ctypes.data, n_pos, nkv, hd, ref.ctypes.data), "kv_build_ref")
+    return ref
+
+
+def kv_store_fp8(src16, ref16, e5m2: bool) -> np.ndarray:
+    """FP16 vectors [n_pos, n_kv_heads, head_dim] (minus ref16 [n_kv_heads, head_dim] when given) -> FP8 codes."""
+    src16 = np.ascontiguousarray(src16, np.uint16)
+    n_pos, nkv, hd = src16.shape
+    if ref16 is not None:
+        ref16 = np.ascontiguousarray(ref16, np.uint16)
+    out = np.empty((n_pos, nkv, hd), np.uint8)
+    _check(lib.vvo_kv_store_fp8(src16.ctypes.data, ref16.ctypes.data if ref16 is not None else None, n_pos, nkv, hd,
+                                int(e5m2), out.ctypes.data), "kv_store_fp8")
     return out

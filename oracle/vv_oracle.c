@@ -499,6 +499,94 @@ int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uin
     return VVO_OK;
 }
 
+/* ── FP8 KV-cache codec (src/cuda/kv_codec.cuh:66-128, emulated in integer arithmetic) ── */
+
+static uint32_t f32_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
+static float bits_f32(uint32_t b) { float f; memcpy(&f, &b, 4); return f; }
+
+/* One value to E4M3 (bias 7, 3 mantissa bits, no infinities, largest finite
+ * 448 = 0x7E) or E5M2 (bias 15, 2 mantissa bits, largest finite 57344 = 0x7B):
+ * zero and NaN give a signed zero; magnitudes from the half-way point above the
+ * largest finite value saturate to it; below the smallest normal the value is
+ * a count of subnormal steps rounded half up; else round to nearest even on
+ * the FP32 mantissa with the carry going into the exponent. */
+static uint8_t fp8_encode_one(float f, int e5m2) {
+    const int mant_bits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7, drop = 23 - mant_bits;
+    const int min_exp = 1 - bias;                       /* exponent of the smallest normal */
+    const uint32_t max_code = e5m2 ? 0x7Bu : 0x7Eu;
+    const float saturate_from = e5m2 ? 61440.0f : 464.0f;
+    const int max_exp = e5m2 ? 15 : 8;
+    const uint32_t b = f32_bits(f);
+    const uint32_t sign = (b >> 24) & 0x80u;
+    const float a = fabsf(f);
+    if (!(a > 0.0f)) return (uint8_t)sign;
+    if (a >= saturate_from) return (uint8_t)(sign | max_code);
+    int e = (int)((b >> 23) & 0xFFu) - 127;
+    if (e < min_exp) {
+        const float steps = e5m2 ? 65536.0f : 512.0f;   /* 1 / (subnormal step) */
+        int q = (int)(a * steps + 0.5f);
+        const int top = 1 << mant_bits;                 /* rolls into the smallest normal */
+        if (q > top) q = top;
+        return (uint8_t)(sign | (uint32_t)q);
+    }
+    const uint32_t m = b & 0x7FFFFFu;
+    uint32_t mm = m >> drop;
+    const uint32_t rem = m & ((1u << drop) - 1u), half_way = 1u << (drop - 1);
+    if (rem > half_way || (rem == half_way && (mm & 1u))) {
+        if (++mm == (1u << mant_bits)) { mm = 0; ++e; }
+    }
+    if (e > max_exp) return (uint8_t)(sign | max_code);
+    return (uint8_t)(sign | ((uint32_t)(e + bias) << mant_bits) | mm);
+}
+
+static float fp8_decode_one(uint8_t v, int e5m2) {
+    const int mant_bits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7;
+    const uint32_t e = (v >> mant_bits) & (e5m2 ? 0x1Fu : 0xFu);
+    const uint32_t m = v & ((1u << mant_bits) - 1u);
+    const float r = e == 0u ? (float)m * (e5m2 ? 1.52587890625e-05f : 0.001953125f)
+                            : bits_f32(((e + 127u - (uint32_t)bias) << 23) | (m << (23 - mant_bits)));
+    return (v & 0x80u) ? -r : r;
+}
+
+int vvo_fp8_encode(const float* x, int n, int e5m2, uint8_t* out) {
+    if (!x || !out) return VVO_ERR_NULL_PTR;
+    for (int i = 0; i < n; i++) out[i] = fp8_encode_one(x[i], e5m2);
+    return VVO_OK;
+}
+
+int vvo_fp8_decode(const uint8_t* codes, int n, int e5m2, float* out) {
+    if (!codes || !out) return VVO_ERR_NULL_PTR;
+    for (int i = 0; i < n; i++) out[i] = fp8_decode_one(codes[i], e5m2);
+    return VVO_OK;
+}
+
+int vvo_kv_build_ref(const uint16_t* k16, int n_pos, int n_kv_heads, int head_dim, uint16_t* ref16) {
+    if (!k16 || !ref16) return VVO_ERR_NULL_PTR;
+    if (n_pos <= 0) return VVO_ERR_INVALID_ARG;
+    for (int h = 0; h < n_kv_heads; h++)
+        for (int d = 0; d < head_dim; d++) {
+            float acc = 0.0f;
+            for (int p = 0; p < n_pos; p++)
+                acc += vvo_half_to_float(k16[((size_t)p * n_kv_heads + h) * head_dim + d]);
+            ref16[(size_t)h * head_dim + d] = vvo_float_to_half_rne(acc / (float)n_pos);
+        }
+    return VVO_OK;
+}
+
+int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads,
+                     int head_dim, int e5m2, uint8_t* store) {
+    if (!src16 || !store) return VVO_ERR_NULL_PTR;
+    for (int p = 0; p < n_pos; p++)
+        for (int h = 0; h < n_kv_heads; h++)
+            for (int d = 0; d < head_dim; d++) {
+                const size_t i = ((size_t)p * n_kv_heads + h) * head_dim + d;
+                float v = vvo_half_to_float(src16[i]);
+                if (ref16) v -= vvo_half_to_float(ref16[(size_t)h * head_dim + d]);
+                store[i] = fp8_encode_one(v, e5m2);
+            }
+    return VVO_OK;
+}
+
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value) {
     if (!logits || !token) return VVO_ERR_NULL_PTR;
     int best = 0;

@@ -164,6 +164,22 @@ int vvo_int4g_dequant_f16(const uint8_t* packed, const uint16_t* scales16, const
 int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
                             int N, int K, int G, uint16_t* out_sz);
 
+/* The FP8 KV-cache codec, src/cuda/kv_codec.cuh:66-128 (the reference has no
+ * CPU form of it; this restates the accelerator's integer arithmetic, and the
+ * tests pin it to what the formats themselves fix: every code decodes to its
+ * closed-form value, and every FP16 input encodes to a nearest representable
+ * value). e5m2 == 0: E4M3 (largest finite 448), else E5M2 (57344); zero and NaN
+ * encode as a signed zero, out-of-range magnitudes saturate. */
+int vvo_fp8_encode(const float* x, int n, int e5m2, uint8_t* out);
+int vvo_fp8_decode(const uint8_t* codes, int n, int e5m2, float* out);
+/* src/cuda/kv_quant.cu:157-169 (kv_build_ref_kernel): per head and channel the
+ * FP32 mean of the run's keys, positions added in order, rounded to FP16. */
+int vvo_kv_build_ref(const uint16_t* k16, int n_pos, int n_kv_heads, int head_dim, uint16_t* ref16);
+/* src/cuda/kv_quant.cu:57-84 (kv_store_kernel, FP8 formats): FP16 -> FP32, minus
+ * the head's reference key when there is one, then the codec. */
+int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads,
+                     int head_dim, int e5m2, uint8_t* store);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

@@ -83,17 +83,59 @@ struct TileRegs {
     Chunk k[kIter], v[kIter];
 };
 
-template <int kThreads>
-__device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const h16* __restrict__ Kc,
-                                           const h16* __restrict__ Vc,
-                                           const int* __restrict__ page_table, size_t kv_stride,
+// Cache formats the matrix-core kernels read (include/vibevoice/kv_quant.h:34-36).
+// The FP8 ones are widened to FP16 on their way into the registers: every
+// E4M3 / E5M2 value is an FP16 value, so from there on the tile is the tile of
+// an FP16 cache that holds the decoded values.
+constexpr int kFmtFp16 = 0, kFmtE4M3 = 1, kFmtE5M2 = 2;
+
+// Four FP8 codes (the bytes of `codes`) as two half2 words, lanes in byte order.
+template <int kFmt>
+__device__ __forceinline__ void widen4(uint32_t codes, uint32_t& lo, uint32_t& hi) {
+    // byte b -> 16-bit lane b << 8: an E5M2 code IS the top byte of the FP16 value
+    lo = __builtin_amdgcn_perm(0u, codes, 0x010C000Cu);
+    hi = __builtin_amdgcn_perm(0u, codes, 0x030C020Cu);
+    if constexpr (kFmt == kFmtE4M3) {
+        // sign stays, exponent and mantissa move down one bit (FP16 has five exponent bits):
+        // that reads 2^-8 too small (bias 15 against 7), subnormals included, so scale by 256
+        typedef h16 h16x2v __attribute__((ext_vector_type(2)));
+        const h16x2v k256 = {(h16)256.0f, (h16)256.0f};
+        const uint32_t l = ((lo >> 1) & 0x3F803F80u) | (lo & 0x80008000u);
+        const uint32_t h = ((hi >> 1) & 0x3F803F80u) | (hi & 0x80008000u);
+        lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2v, l) * k256);
+        hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2v, h) * k256);
+    }
+}
+
+// Slot `slot` (eight channels) of vector `vec` (= cache row * n_kv_heads + KV head) as FP16.
+template <int kFmt>
+__device__ __forceinline__ Chunk load_slot(const void* __restrict__ cache, size_t vec, int slot) {
+    if constexpr (kFmt == kFmtFp16) {
+        return load_chunk(static_cast<const Chunk*>(cache) + vec * (kD / 8) + slot);
+    } else {
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+        const u32x2 codes = *(static_cast<const u32x2*>(cache) + vec * (kD / 8) + slot);
+        u32x4v w;
+        uint32_t a, b, c, d;
+        widen4<kFmt>(codes.x, a, b);
+        widen4<kFmt>(codes.y, c, d);
+        w.x = a; w.y = b; w.z = c; w.w = d;
+        return __builtin_bit_cast(Chunk, w);
+    }
+}
+
+template <int kThreads, int kFmt>
+__device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const void* __restrict__ Kc,
+                                           const void* __restrict__ Vc,
+                                           const int* __restrict__ page_table, int n_kv_heads,
                                            int kvh, int t0, int last_key, int tid) {
     constexpr int kIter = TileRegs<kThreads>::kIter;
 #pragma unroll
     for (int i = 0; i < kIter; ++i) {
         const int q = tid + i * kThreads, r = q >> 4, slot = q & 15;
         const int row = cache_row(page_table, min(t0 + r, last_key));
-        regs.k[i] = load_chunk(reinterpret_cast<const Chunk*>(Kc + (size_t)row * kv_stride + kvh * kD) + slot);
+        regs.k[i] = load_slot<kFmt>(Kc, (size_t)row * n_kv_heads + kvh, slot);
     }
 #pragma unroll
     for (int i = 0; i < kIter / 4; ++i) {
@@ -101,8 +143,7 @@ __device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const h16* 
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int row = cache_row(page_table, min(t0 + 4 * kg + j, last_key));
-            regs.v[4 * i + j] =
-                load_chunk(reinterpret_cast<const Chunk*>(Vc + (size_t)row * kv_stride + kvh * kD) + dchunk);
+            regs.v[4 * i + j] = load_slot<kFmt>(Vc, (size_t)row * n_kv_heads + kvh, dchunk);
         }
     }
 }
@@ -207,8 +248,9 @@ __device__ __forceinline__ void load_query(h16x8 (&qf)[kD / 16], const h16* qp, 
 }
 
 // ── prefill ──────────────────────────────────────────────────────────────
+template <int kFmt>
 __global__ __launch_bounds__(kBlock, 2) void prefill128(
-    const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
+    const h16* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
     const int* __restrict__ page_table, h16* __restrict__ O, int n_q_heads, int n_kv_heads,
     int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
     __shared__ KvTile tile;
@@ -225,7 +267,6 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
     const int qw0 = q0 + wave * 32;
     const int qrow = qw0 + col;
     const int q_abs = q_offset + qrow;
-    const size_t kv_stride = (size_t)n_kv_heads * kD;
 
     // Keys any row of the workgroup / of this wave may see.
     int wg_limit = kv_len, wave_limit = qw0 < q_len ? kv_len : 0;
@@ -240,13 +281,13 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
     st.reset();
 
     TileRegs<kBlock> regs;
-    if (wg_limit > 0) fetch_tile<kBlock>(regs, Kc, Vc, page_table, kv_stride, kvh, 0, kv_len - 1, tid);
+    if (wg_limit > 0) fetch_tile<kBlock, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, 0, kv_len - 1, tid);
     for (int t0 = 0; t0 < wg_limit; t0 += kKeyTile) {
         __syncthreads();
         commit_tile<kBlock>(tile, regs, tid);
         __syncthreads();
         if (t0 + kKeyTile < wg_limit)
-            fetch_tile<kBlock>(regs, Kc, Vc, page_table, kv_stride, kvh, t0 + kKeyTile, kv_len - 1, tid);
+            fetch_tile<kBlock, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, t0 + kKeyTile, kv_len - 1, tid);
         if (t0 >= wave_limit) continue;
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
@@ -334,8 +375,9 @@ __global__ __launch_bounds__(kWave) void rows_generic(
 // otherwise each slice leaves (max, sum, unnormalised O) per head in `parts`.
 constexpr int kPartFloats = kD + 4;        // per (head, slice): 128 channels, max, sum, 2 unused (16-byte rows)
 
+template <int kFmt>
 __global__ __launch_bounds__(kWave) void decode128(
-    const h16* __restrict__ Q, const h16* __restrict__ Kc, const h16* __restrict__ Vc,
+    const h16* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
     const int* __restrict__ page_table, h16* __restrict__ O, float* __restrict__ parts,
     int n_q_heads, int n_kv_heads, int cache_len, const int* __restrict__ d_cache_len,
     int n_parts, float scale_log2) {
@@ -351,7 +393,6 @@ __global__ __launch_bounds__(kWave) void decode128(
     const int len = d_cache_len ? *d_cache_len : cache_len;
     const int per = (((len + n_parts - 1) / n_parts) + kKeyTile - 1) & ~(kKeyTile - 1);
     const int begin = part * per, end = min(len, begin + per);
-    const size_t kv_stride = (size_t)n_kv_heads * kD;
 
     h16x8 qf[kD / 16];
     load_query(qf, Q + (size_t)head * kD, half);
@@ -359,13 +400,13 @@ __global__ __launch_bounds__(kWave) void decode128(
     st.reset();
 
     TileRegs<kWave> regs;
-    if (begin < end) fetch_tile<kWave>(regs, Kc, Vc, page_table, kv_stride, kvh, begin, end - 1, lane);
+    if (begin < end) fetch_tile<kWave, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, begin, end - 1, lane);
     for (int t0 = begin; t0 < end; t0 += kKeyTile) {
         __syncthreads();
         commit_tile<kWave>(tile, regs, lane);
         __syncthreads();
         if (t0 + kKeyTile < end)
-            fetch_tile<kWave>(regs, Kc, Vc, page_table, kv_stride, kvh, t0 + kKeyTile, end - 1, lane);
+            fetch_tile<kWave, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, t0 + kKeyTile, end - 1, lane);
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
         if (t0 + kKeyTile > end) {
@@ -478,6 +519,93 @@ __global__ __launch_bounds__(kBlock) void kv_store_fp16(
     v_store[dst] = v[i];
 }
 
+// ── FP8 cache store (src/cuda/kv_quant.cu:57-84, kv_codec.cuh:66-128) ──────
+// One value to E4M3 (bias 7, largest finite 448 = 0x7E) or E5M2 (bias 15,
+// largest finite 57344 = 0x7B) in integer arithmetic: zero and NaN give a signed
+// zero, magnitudes from half a step above the largest finite value saturate to
+// it, below the smallest normal the value is a count of subnormal steps rounded
+// half up, else round to nearest even on the FP32 mantissa with the carry going
+// into the exponent.
+template <bool kE5M2>
+__device__ __forceinline__ uint32_t fp8_encode(float f) {
+    constexpr int kMant = kE5M2 ? 2 : 3, kBias = kE5M2 ? 15 : 7, kDrop = 23 - kMant;
+    constexpr uint32_t kMaxCode = kE5M2 ? 0x7Bu : 0x7Eu;
+    const uint32_t b = __builtin_bit_cast(uint32_t, f);
+    const uint32_t sign = (b >> 24) & 0x80u;
+    const float a = fabsf(f);
+    if (!(a > 0.0f)) return sign;
+    if (a >= (kE5M2 ? 61440.0f : 464.0f)) return sign | kMaxCode;
+    int e = (int)((b >> 23) & 0xFFu) - 127;
+    if (e < 1 - kBias) {
+        int q = (int)(a * (kE5M2 ? 65536.0f : 512.0f) + 0.5f);
+        q = min(q, 1 << kMant);                       // rolls into the smallest normal
+        return sign | (uint32_t)q;
+    }
+    const uint32_t m = b & 0x7FFFFFu;
+    uint32_t mm = m >> kDrop;
+    const uint32_t rem = m & ((1u << kDrop) - 1u), half_way = 1u << (kDrop - 1);
+    if (rem > half_way || (rem == half_way && (mm & 1u))) {
+        if (++mm == (1u << kMant)) { mm = 0; ++e; }
+    }
+    if (e > (kE5M2 ? 15 : 8)) return sign | kMaxCode;
+    return sign | ((uint32_t)(e + kBias) << kMant) | mm;
+}
+
+// Per head and channel the FP32 mean of the run's keys, positions in order.
+__global__ void kv_build_ref(const h16* __restrict__ k, h16* __restrict__ ref, int n_kv_heads, int n_pos) {
+    const int h = (int)blockIdx.x, d = (int)threadIdx.x;
+    float acc = 0.0f;
+    for (int p = 0; p < n_pos; ++p) acc += (float)k[((size_t)p * n_kv_heads + h) * kD + d];
+    ref[(size_t)h * kD + d] = to_half(acc / (float)n_pos);
+}
+
+// blockIdx.y = 0: keys (minus the head's reference key when there is one), 1: values.
+// A thread encodes eight channels.
+template <bool kE5M2>
+__global__ __launch_bounds__(kBlock) void kv_store_fp8(
+    const h16* __restrict__ k, const h16* __restrict__ v, uint8_t* __restrict__ k_store,
+    uint8_t* __restrict__ v_store, const h16* __restrict__ k_ref, int n_kv_heads, int pos,
+    const int* __restrict__ d_pos, int n_positions, const int* __restrict__ page_table) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;         // (position, head, slot)
+    const int slots_per_pos = n_kv_heads * (kD / 8);
+    if (i >= (size_t)n_positions * slots_per_pos) return;
+    const bool keys = blockIdx.y == 0;
+    const int p = (int)(i / slots_per_pos), e = (int)(i % slots_per_pos);
+    const int head = e / (kD / 8), slot = e % (kD / 8);
+    const h16x8 src = *(reinterpret_cast<const h16x8*>(keys ? k : v) + i);
+    h16x8 ref = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool centred = keys && k_ref != nullptr;
+    if (centred) ref = *(reinterpret_cast<const h16x8*>(k_ref) + head * (kD / 8) + slot);
+    uint32_t w[2] = {0u, 0u};
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        float val = (float)src[c];
+        if (centred) val -= (float)ref[c];
+        w[c >> 2] |= fp8_encode<kE5M2>(val) << (8 * (c & 3));
+    }
+    const int t = (d_pos ? *d_pos : pos) + p;
+    const size_t dst = (size_t)cache_row(page_table, t) * slots_per_pos + e;
+    *(reinterpret_cast<u32x2*>(keys ? k_store : v_store) + dst) = u32x2{w[0], w[1]};
+}
+
+// FP8 codes back to FP16 (plus the reference key when given): tests, offload.
+template <int kFmt>
+__global__ __launch_bounds__(kBlock) void kv_dequant_fp8(const void* __restrict__ store,
+                                                         const h16* __restrict__ ref, h16* __restrict__ out,
+                                                         int n_kv_heads, size_t n_slots) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_slots) return;
+    h16x8 val = __builtin_bit_cast(h16x8, load_slot<kFmt>(store, i / (kD / 8), (int)(i % (kD / 8))));
+    if (ref) {
+        const int head = (int)((i / (kD / 8)) % n_kv_heads), slot = (int)(i % (kD / 8));
+        const h16x8 r = *(reinterpret_cast<const h16x8*>(ref) + head * (kD / 8) + slot);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) val[c] = to_half((float)val[c] + (float)r[c]);
+    }
+    *(reinterpret_cast<h16x8*>(out) + i) = val;
+}
+
 struct PageIds { int id[32]; };
 __global__ void page_map(int* table, int first, int n, PageIds ids) {
     const int i = (int)threadIdx.x;
@@ -489,6 +617,8 @@ int decode_parts(int cache_len) {
     while (n < want && n < kMaxParts) n *= 2;
     return n;
 }
+
+bool fp8_format(int kv_format) { return kv_format == kFmtE4M3 || kv_format == kFmtE5M2; }
 
 bool shape_ok(int n_q_heads, int n_kv_heads, int head_dim) {
     return n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0 && head_dim > 0 &&
@@ -502,11 +632,13 @@ extern "C" {
 
 /* One implementation serves every backend name: what differs between fa1,
  * fa2 and flashinfer on the reference's CUDA side is how the card is used,
- * not the result. FP16 caches only, contiguous or paged. */
+ * not the result. FP16 caches, and FP8 (E4M3 / E5M2) ones at head_dim 128,
+ * contiguous or paged. */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads, int n_kv_heads,
                     int head_dim) {
     enum { kAuto = 0, kFa1 = 1, kFa2 = 2, kFlashinfer = 3 };
-    if (kv_format != vv::kFormatFp16 || !vv::shape_ok(n_q_heads, n_kv_heads, head_dim)) return kFa1;
+    const bool served = kv_format == vv::kFormatFp16 || (vv::fp8_format(kv_format) && head_dim == vv::kD);
+    if (!served || !vv::shape_ok(n_q_heads, n_kv_heads, head_dim)) return kFa1;
     if (requested == kFlashinfer) return kFlashinfer;
     if (requested == kFa1 && !paged) return kFa1;
     return kFa2;
@@ -530,8 +662,12 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     if (!q || !kv || !out) return VV_ERR_NULL_PTR;
     if (q_len <= 0 || kv_len <= 0) return VV_OK;
     if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
-    if (kv->format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    const bool fp8 = vv::fp8_format(kv->format);
+    if (kv->format != vv::kFormatFp16 && !fp8) return VV_ERR_UNSUPPORTED;
     if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
+    if (fp8 && (kv->head_dim != vv::kD || !vv::aligned16(q) || !vv::aligned16(out) ||
+                ((reinterpret_cast<uintptr_t>(kv->k) | reinterpret_cast<uintptr_t>(kv->v)) & 7u)))
+        return VV_ERR_UNSUPPORTED;
     if (q_offset < 0) return VV_ERR_INVALID_ARG;
     hipStream_t st = vv::as_stream(stream);
     const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
@@ -539,12 +675,22 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     const vv::h16* K = static_cast<const vv::h16*>(kv->k);
     const vv::h16* V = static_cast<const vv::h16*>(kv->v);
     vv::h16* O = static_cast<vv::h16*>(out);
-    if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
-        vv::aligned16(out)) {
+    if (fp8) {
         const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
-        vv::prefill128<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
-                                                    kv->n_kv_heads, q_len, q_offset, kv_len,
-                                                    causal ? 1 : 0, scale_log2);
+        if (kv->format == vv::kFmtE4M3)
+            vv::prefill128<vv::kFmtE4M3><<<grid, vv::kBlock, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, n_q_heads,
+                                                                      kv->n_kv_heads, q_len, q_offset, kv_len,
+                                                                      causal ? 1 : 0, scale_log2);
+        else
+            vv::prefill128<vv::kFmtE5M2><<<grid, vv::kBlock, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, n_q_heads,
+                                                                      kv->n_kv_heads, q_len, q_offset, kv_len,
+                                                                      causal ? 1 : 0, scale_log2);
+    } else if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
+               vv::aligned16(out)) {
+        const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
+        vv::prefill128<vv::kFmtFp16><<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
+                                                                  kv->n_kv_heads, q_len, q_offset, kv_len,
+                                                                  causal ? 1 : 0, scale_log2);
     } else {
         const dim3 grid((unsigned)q_len, (unsigned)n_q_heads);
         vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
@@ -561,23 +707,36 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
     if (!q || !kv || !out) return VV_ERR_NULL_PTR;
     if (cache_len <= 0) return VV_OK;
     if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
-    if (kv->format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    const bool fp8 = vv::fp8_format(kv->format);
+    if (kv->format != vv::kFormatFp16 && !fp8) return VV_ERR_UNSUPPORTED;
     if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
+    if (fp8 && (kv->head_dim != vv::kD || !vv::aligned16(q) ||
+                ((reinterpret_cast<uintptr_t>(kv->k) | reinterpret_cast<uintptr_t>(kv->v)) & 7u)))
+        return VV_ERR_UNSUPPORTED;
     hipStream_t st = vv::as_stream(stream);
     const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
     const vv::h16* Q = static_cast<const vv::h16*>(q);
     const vv::h16* K = static_cast<const vv::h16*>(kv->k);
     const vv::h16* V = static_cast<const vv::h16*>(kv->v);
     vv::h16* O = static_cast<vv::h16*>(out);
-    if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v)) {
+    if (fp8 || (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v))) {
         const int n_parts = vv::decode_parts(cache_len);
         if (n_parts > 1 && !scratch) return VV_ERR_NULL_PTR;
         const int group = n_q_heads / kv->n_kv_heads;
         const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads, (unsigned)((group + 31) / 32));
-        vv::decode128<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O,
-                                                     static_cast<float*>(scratch), n_q_heads,
-                                                     kv->n_kv_heads, cache_len, d_cache_len,
-                                                     n_parts, scale_log2);
+        float* parts = static_cast<float*>(scratch);
+        if (kv->format == vv::kFmtE4M3)
+            vv::decode128<vv::kFmtE4M3><<<grid, vv::kWave, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, parts, n_q_heads,
+                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
+                                                                    scale_log2);
+        else if (kv->format == vv::kFmtE5M2)
+            vv::decode128<vv::kFmtE5M2><<<grid, vv::kWave, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, parts, n_q_heads,
+                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
+                                                                    scale_log2);
+        else
+            vv::decode128<vv::kFmtFp16><<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, parts, n_q_heads,
+                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
+                                                                    scale_log2);
         if (n_parts > 1) {
             if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
             vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kMergeThreads, 0, st>>>(
@@ -631,11 +790,37 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
                             void* k_meta, void* v_meta, void* k_ref, bool build_ref,
                             int n_kv_heads, int head_dim, int pos, const int* d_pos,
                             int n_positions, int kv_format, const int* page_table, void* stream) {
-    (void)k_meta; (void)v_meta; (void)k_ref; (void)build_ref;
+    (void)k_meta; (void)v_meta;     // the formats with a per-vector scale are not served
     if (!k_fp16 || !v_fp16 || !k_store || !v_store) return VV_ERR_NULL_PTR;
-    if (kv_format != vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    if (kv_format != vv::kFormatFp16 && !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
     if (n_kv_heads <= 0 || head_dim <= 0 || pos < 0) return VV_ERR_INVALID_ARG;
     if (n_positions <= 0) return VV_OK;
+    if (vv::fp8_format(kv_format)) {
+        if (head_dim != vv::kD || !vv::aligned16(k_fp16) || !vv::aligned16(v_fp16) || (k_ref && !vv::aligned16(k_ref)) ||
+            ((reinterpret_cast<uintptr_t>(k_store) | reinterpret_cast<uintptr_t>(v_store)) & 7u))
+            return VV_ERR_UNSUPPORTED;
+        hipStream_t st = vv::as_stream(stream);
+        if (k_ref && build_ref) {
+            vv::kv_build_ref<<<dim3((unsigned)n_kv_heads), vv::kD, 0, st>>>(static_cast<const vv::h16*>(k_fp16),
+                                                                           static_cast<vv::h16*>(k_ref), n_kv_heads,
+                                                                           n_positions);
+            if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
+        }
+        const size_t slots = (size_t)n_positions * n_kv_heads * (vv::kD / 8);
+        const dim3 grid((unsigned)((slots + vv::kBlock - 1) / vv::kBlock), 2u);
+        const vv::h16* K = static_cast<const vv::h16*>(k_fp16);
+        const vv::h16* V = static_cast<const vv::h16*>(v_fp16);
+        uint8_t* KS = static_cast<uint8_t*>(k_store);
+        uint8_t* VS = static_cast<uint8_t*>(v_store);
+        const vv::h16* R = static_cast<const vv::h16*>(k_ref);
+        if (kv_format == vv::kFmtE5M2)
+            vv::kv_store_fp8<true><<<grid, vv::kBlock, 0, st>>>(K, V, KS, VS, R, n_kv_heads, pos, d_pos, n_positions,
+                                                                page_table);
+        else
+            vv::kv_store_fp8<false><<<grid, vv::kBlock, 0, st>>>(K, V, KS, VS, R, n_kv_heads, pos, d_pos, n_positions,
+                                                                 page_table);
+        return vv::launch_status();
+    }
     const int row = n_kv_heads * head_dim;
     const size_t n = (size_t)n_positions * row;
     vv::kv_store_fp16<<<dim3((unsigned)((n + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
@@ -644,6 +829,55 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
         static_cast<vv::h16*>(k_store), static_cast<vv::h16*>(v_store), row, pos, d_pos,
         n_positions, page_table);
     return vv::launch_status();
+}
+
+vv_status_t vv_kv_quant_store_dev(const void* k_fp16, const void* v_fp16, void* k_store, void* v_store,
+                                  void* k_meta, void* v_meta, void* k_ref, bool build_ref, int n_kv_heads,
+                                  int head_dim, int pos, const int* d_pos, int n_positions, int kv_format,
+                                  void* stream) {
+    if (kv_format == vv::kFormatFp16) return VV_ERR_UNSUPPORTED;
+    return vv_kv_store_dev(k_fp16, v_fp16, k_store, v_store, k_meta, v_meta, k_ref, build_ref, n_kv_heads,
+                           head_dim, pos, d_pos, n_positions, kv_format, nullptr, stream);
+}
+
+vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* ref, void* out_fp16,
+                              int n_kv_heads, int head_dim, int n_pos, int kv_format, void* stream) {
+    (void)meta;
+    if (!store || !out_fp16) return VV_ERR_NULL_PTR;
+    if (head_dim != vv::kD || !vv::fp8_format(kv_format) || n_kv_heads <= 0) return VV_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(store) & 7u) || !vv::aligned16(out_fp16) || (ref && !vv::aligned16(ref)))
+        return VV_ERR_UNSUPPORTED;
+    if (n_pos <= 0) return VV_OK;
+    const size_t slots = (size_t)n_pos * n_kv_heads * (vv::kD / 8);
+    const dim3 grid((unsigned)((slots + vv::kBlock - 1) / vv::kBlock));
+    hipStream_t st = vv::as_stream(stream);
+    const vv::h16* R = static_cast<const vv::h16*>(ref);
+    vv::h16* O = static_cast<vv::h16*>(out_fp16);
+    if (kv_format == vv::kFmtE4M3) vv::kv_dequant_fp8<vv::kFmtE4M3><<<grid, vv::kBlock, 0, st>>>(store, R, O, n_kv_heads, slots);
+    else vv::kv_dequant_fp8<vv::kFmtE5M2><<<grid, vv::kBlock, 0, st>>>(store, R, O, n_kv_heads, slots);
+    return vv::launch_status();
+}
+
+vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, const void* v_store,
+                                          const void* k_meta, const void* v_meta, void* output,
+                                          int n_q_heads, int n_kv_heads, int head_dim, int cache_len,
+                                          const int* d_cache_len, int kv_format, void* scratch, void* stream) {
+    if (!q || !k_store || !v_store || !output || !scratch) return VV_ERR_NULL_PTR;
+    if (cache_len == 0) return VV_OK;
+    if (head_dim != vv::kD || !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
+    const vv_kv_view_t view = {k_store, v_store, k_meta, v_meta, nullptr, kv_format, n_kv_heads, head_dim};
+    return vv_attn_decode(2, q, &view, output, n_q_heads, cache_len, d_cache_len, scratch, stream);
+}
+
+vv_status_t vv_gqa_attention_prefill_q_dev(const void* q, const void* k_store, const void* v_store,
+                                           const void* k_meta, const void* v_meta, void* output,
+                                           int n_q_heads, int n_kv_heads, int head_dim, int q_len,
+                                           int q_offset, int kv_len, bool causal, int kv_format, void* stream) {
+    if (!q || !k_store || !v_store || !output) return VV_ERR_NULL_PTR;
+    if (q_len == 0 || kv_len == 0) return VV_OK;
+    if (head_dim != vv::kD || !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
+    const vv_kv_view_t view = {k_store, v_store, k_meta, v_meta, nullptr, kv_format, n_kv_heads, head_dim};
+    return vv_attn_prefill(2, q, &view, output, n_q_heads, q_len, q_offset, kv_len, causal, nullptr, stream);
 }
 
 vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages, void* stream) {

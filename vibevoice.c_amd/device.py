@@ -72,6 +72,10 @@ SIGNATURES = {
     "vv_attn_decode_shape": (_i, [_i, _i, _i, _i]),
     "vv_attn_prefill": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, C.c_bool, _vp, _vp]),
     "vv_attn_decode": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "vv_kv_quant_store_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_bool, _i, _i, _i, _vp, _i, _i, _vp]),
+    "vv_kv_dequant_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "vv_gqa_attention_decode_q_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
+    "vv_gqa_attention_prefill_q_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, C.c_bool, _i, _vp]),
     "vv_kv_store_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_bool, _i, _i, _i, _vp, _i,
                             _i, _vp, _vp]),
     "vv_kv_page_map_dev": (_i, [_vp, _i, _i, _vp, _vp]),
