@@ -351,6 +351,19 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
     gb = 2.0 * T * NK * HD * 2 / sec / 1e9
     out["attn_decode"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS,
                           "note": "two launches; the host's launch rate bounds this figure"}
+    # The same two over an FP8 (E4M3) cache: half the cache bytes, widened on their way into the tile.
+    k8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
+    v8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
+    view8 = dev.KvView(k=k8.data_ptr(), v=v8.data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                       format=1, n_kv_heads=NK, head_dim=HD)
+    sec = timed(lambda: dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, 0, T,
+                                            True, None, st), 3)
+    tf = 4.0 * NQ * HD * T * (T + 1) / 2 / sec / 1e12
+    out["attn_prefill_fp8"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf, "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+    sec = timed(lambda: dev.vv_attn_decode(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, None,
+                                           scratch.data_ptr(), st), 50)
+    gb = 2.0 * T * NK * HD / sec / 1e9
+    out["attn_decode_fp8"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
     return out
 
 
@@ -984,6 +997,10 @@ def main() -> int:
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         d = layer["attn_decode"]
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        d = layer["attn_prefill_fp8"]
+        log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
+        d = layer["attn_decode_fp8"]
+        log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
         log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention); "
             f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
