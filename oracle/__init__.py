@@ -92,6 +92,12 @@ def _load():
                        ("vvo_kv_store_fp8", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p])):
         getattr(lib, name).restype = C.c_int
         getattr(lib, name).argtypes = args
+    for name, args in (("vvo_kv_bytes_per_vec", [C.c_int]),
+                       ("vvo_kv_rotate", [C.c_void_p, C.c_int, C.c_int]),
+                       ("vvo_kv_store_tq", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+                       ("vvo_kv_dequant", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p])):
+        getattr(lib, name).restype = C.c_int
+        getattr(lib, name).argtypes = args
     lib.vvo_argmax_first.restype = C.c_int
     lib.vvo_argmax_first.argtypes = [_f32p, C.c_int, C.POINTER(C.c_int32), _f32p]
     lib.vvo_threads.restype = C.c_int
@@ -449,4 +455,44 @@ def kv_store_fp8(src16, ref16, e5m2: bool) -> np.ndarray:
     out = np.empty((n_pos, nkv, hd), np.uint8)
     _check(lib.vvo_kv_store_fp8(src16.ctypes.data, ref16.ctypes.data if ref16 is not None else None, n_pos, nkv, hd,
                                 int(e5m2), out.ctypes.data), "kv_store_fp8")
+    return out
+
+
+def kv_bytes_per_vec(fmt: int) -> int:
+    return lib.vvo_kv_bytes_per_vec(fmt)
+
+
+def kv_rotate(x16, inverse: bool = False) -> np.ndarray:
+    """FP16 bits [..., 128] -> the randomised Hadamard transform (or its inverse) of every vector."""
+    out = np.array(x16, dtype=np.uint16, order="C", copy=True)
+    _check(lib.vvo_kv_rotate(out.ctypes.data, out.size // 128, int(inverse)), "kv_rotate")
+    return out
+
+
+def kv_store_tq(src16, ref16, fmt: int):
+    """FP16 vectors [n_pos, n_kv_heads, 128] -> (codes uint8 [n_pos, n_kv_heads, bytes], RMS FP16 bits [n_pos, n_kv_heads])."""
+    src16 = np.ascontiguousarray(src16, np.uint16)
+    n_pos, nkv, hd = src16.shape
+    assert hd == 128
+    if ref16 is not None:
+        ref16 = np.ascontiguousarray(ref16, np.uint16)
+    store = np.empty((n_pos, nkv, kv_bytes_per_vec(fmt)), np.uint8)
+    meta = np.empty((n_pos, nkv), np.uint16)
+    _check(lib.vvo_kv_store_tq(src16.ctypes.data, ref16.ctypes.data if ref16 is not None else None, n_pos, nkv, fmt,
+                               store.ctypes.data, meta.ctypes.data), "kv_store_tq")
+    return store, meta
+
+
+def kv_dequant(store, meta16, ref16, fmt: int) -> np.ndarray:
+    """Codes [n_pos, n_kv_heads, bytes] (+ RMS for TurboQuant) -> FP16 bits [n_pos, n_kv_heads, 128] in the stored space."""
+    store = np.ascontiguousarray(store, np.uint8)
+    n_pos, nkv = store.shape[:2]
+    if meta16 is not None:
+        meta16 = np.ascontiguousarray(meta16, np.uint16)
+    if ref16 is not None:
+        ref16 = np.ascontiguousarray(ref16, np.uint16)
+    out = np.empty((n_pos, nkv, 128), np.uint16)
+    _check(lib.vvo_kv_dequant(store.ctypes.data, meta16.ctypes.data if meta16 is not None else None,
+                              ref16.ctypes.data if ref16 is not None else None, n_pos, nkv, fmt, out.ctypes.data),
+           "kv_dequant")
     return out

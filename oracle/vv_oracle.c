@@ -10,6 +10,7 @@
  */
 #include "vv_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -584,6 +585,218 @@ int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, in
                 if (ref16) v -= vvo_half_to_float(ref16[(size_t)h * head_dim + d]);
                 store[i] = fp8_encode_one(v, e5m2);
             }
+    return VVO_OK;
+}
+
+/* ── TurboQuant KV-cache codec (src/cuda/kv_codec.cuh:38-62, 130-165, 180-285; kv_quant.cu:86-119) ── */
+
+/* Lloyd-Max levels of a unit Gaussian (kv_codec.cuh:43-62). */
+static const float kLev4[16] = {-2.725112f, -2.065280f, -1.613787f, -1.251845f, -0.938657f, -0.654379f,
+                                -0.386970f, -0.127960f, +0.127960f, +0.386970f, +0.654379f, +0.938657f,
+                                +1.251845f, +1.613787f, +2.065280f, +2.725112f};
+static const float kLev3[8] = {-2.150300f, -1.343258f, -0.755588f, -0.244756f,
+                               +0.244756f, +0.755588f, +1.343258f, +2.150300f};
+static const float kLev2[4] = {-1.511418f, -0.452456f, +0.452456f, +1.511418f};
+static const float kVq15[16] = {-1.500251f, +0.674678f, -1.127883f, -0.787015f, -0.283251f, +0.390133f,
+                                -0.103102f, +1.624620f, +0.100120f, -1.618563f, +0.286482f, -0.379555f,
+                                +1.134227f, +0.790368f, +1.496572f, -0.666578f};
+#define VVO_WHT_NORM 0.0883883476f      /* 1 / sqrt(128) */
+
+enum { VVO_KV_TQ4 = 3, VVO_KV_TQ3 = 4, VVO_KV_TQ2 = 5, VVO_KV_TQ1_5 = 6 };
+
+static int tq_lane_bits(int fmt) { return fmt == VVO_KV_TQ4 ? 16 : fmt == VVO_KV_TQ3 ? 12 : fmt == VVO_KV_TQ2 ? 8 : 6; }
+int vvo_kv_bytes_per_vec(int fmt) {      /* head_dim 128 (kv_quant.h:63-76) */
+    switch (fmt) {
+        case 1: case 2: return 128;
+        case VVO_KV_TQ4: return 64;
+        case VVO_KV_TQ3: return 48;
+        case VVO_KV_TQ2: return 32;
+        case VVO_KV_TQ1_5: return 24;
+        default: return 256;
+    }
+}
+
+/* The fixed +-1 pattern of the randomised transform (kv_codec.cuh:132-136). */
+static float kv_sign(int d) {
+    uint32_t h = (uint32_t)d * 2654435761u + 0x9E3779B9u;
+    h ^= h >> 15; h *= 0x85EBCA6Bu; h ^= h >> 13;
+    return (h & 1u) ? -1.0f : 1.0f;
+}
+
+/* Walsh-Hadamard transform of 128 values in the order the accelerator adds
+ * them: value 4 L + i lives in lane L; strides 1 and 2 inside a lane, then
+ * lane strides 1 .. 16, the upper partner taking (other - own). */
+static void wht128(float v[32][4]) {
+    for (int L = 0; L < 32; L++) {
+        float* x = v[L];
+        float a;
+        a = x[0] + x[1]; x[1] = x[0] - x[1]; x[0] = a;
+        a = x[2] + x[3]; x[3] = x[2] - x[3]; x[2] = a;
+        a = x[0] + x[2]; x[2] = x[0] - x[2]; x[0] = a;
+        a = x[1] + x[3]; x[3] = x[1] - x[3]; x[1] = a;
+    }
+    for (int m = 1; m < 32; m <<= 1) {
+        float n[32][4];
+        for (int L = 0; L < 32; L++)
+            for (int i = 0; i < 4; i++) {
+                const float o = v[L ^ m][i];
+                n[L][i] = (L & m) ? o - v[L][i] : v[L][i] + o;
+            }
+        memcpy(v, n, sizeof(n));
+    }
+}
+
+static void rotate128(float v[32][4], int inverse) {
+    if (!inverse) {
+        for (int L = 0; L < 32; L++)
+            for (int i = 0; i < 4; i++) v[L][i] *= kv_sign(4 * L + i);
+        wht128(v);
+        for (int L = 0; L < 32; L++)
+            for (int i = 0; i < 4; i++) v[L][i] *= VVO_WHT_NORM;
+    } else {
+        wht128(v);
+        for (int L = 0; L < 32; L++)
+            for (int i = 0; i < 4; i++) v[L][i] *= VVO_WHT_NORM * kv_sign(4 * L + i);
+    }
+}
+
+int vvo_kv_rotate(uint16_t* x16, int n_vectors, int inverse) {
+    if (!x16) return VVO_ERR_NULL_PTR;
+    for (int n = 0; n < n_vectors; n++) {
+        float v[32][4];
+        for (int d = 0; d < 128; d++) v[d / 4][d % 4] = vvo_half_to_float(x16[(size_t)n * 128 + d]);
+        rotate128(v, inverse);
+        for (int d = 0; d < 128; d++) x16[(size_t)n * 128 + d] = vvo_float_to_half_rne(v[d / 4][d % 4]);
+    }
+    return VVO_OK;
+}
+
+/* The packed code of a lane's four values (kv_codec.cuh:228-285): per value the
+ * number of mid-points between neighbouring levels that it exceeds; for the
+ * 1.5-bit form the nearest of eight 2-D code words per pair, first wins ties. */
+static uint32_t tq_pack4(int fmt, const float y[4], float inv_sigma) {
+    uint32_t bits = 0;
+    if (fmt == VVO_KV_TQ1_5) {
+        for (int p = 0; p < 2; p++) {
+            const float a = y[2 * p] * inv_sigma, b = y[2 * p + 1] * inv_sigma;
+            uint32_t best = 0;
+            float bd = FLT_MAX;
+            for (int c = 0; c < 8; c++) {
+                const float da = a - kVq15[2 * c], db = b - kVq15[2 * c + 1];
+                const float d = da * da + db * db;
+                if (d < bd) { bd = d; best = (uint32_t)c; }
+            }
+            bits |= best << (3 * p);
+        }
+        return bits;
+    }
+    const float* lev = fmt == VVO_KV_TQ4 ? kLev4 : fmt == VVO_KV_TQ3 ? kLev3 : kLev2;
+    const int nb = fmt == VVO_KV_TQ4 ? 4 : fmt == VVO_KV_TQ3 ? 3 : 2;
+    for (int i = 0; i < 4; i++) {
+        const float t = y[i] * inv_sigma;
+        uint32_t c = 0;
+        for (int j = 0; j + 1 < (1 << nb); j++) c += (t > 0.5f * (lev[j] + lev[j + 1])) ? 1u : 0u;
+        bits |= c << (nb * i);
+    }
+    return bits;
+}
+
+static void tq_unpack4(int fmt, uint32_t bits, float sigma, float out[4]) {
+    if (fmt == VVO_KV_TQ1_5) {
+        for (int p = 0; p < 2; p++) {
+            const uint32_t c = (bits >> (3 * p)) & 7u;
+            out[2 * p] = sigma * kVq15[2 * c];
+            out[2 * p + 1] = sigma * kVq15[2 * c + 1];
+        }
+        return;
+    }
+    const float* lev = fmt == VVO_KV_TQ4 ? kLev4 : fmt == VVO_KV_TQ3 ? kLev3 : kLev2;
+    const int nb = fmt == VVO_KV_TQ4 ? 4 : fmt == VVO_KV_TQ3 ? 3 : 2;
+    for (int i = 0; i < 4; i++) out[i] = sigma * lev[(bits >> (nb * i)) & ((1u << nb) - 1u)];
+}
+
+/* One vector: minus the reference, rotated, scaled by its own RMS, coded. The
+ * sum of squares is an FMA chain per lane and a butterfly over lane strides
+ * 16 .. 1 (kv_codec.cuh:167-171): every lane ends with the same bits. */
+static void tq_store_one(int fmt, const uint16_t* src16, const uint16_t* ref16, uint8_t* dst, uint16_t* meta) {
+    float v[32][4], ss[32];
+    for (int d = 0; d < 128; d++) {
+        float x = vvo_half_to_float(src16[d]);
+        if (ref16) x -= vvo_half_to_float(ref16[d]);
+        v[d / 4][d % 4] = x;
+    }
+    rotate128(v, 0);
+    for (int L = 0; L < 32; L++) {
+        float a = 0.0f;
+        for (int i = 0; i < 4; i++) a = fmaf(v[L][i], v[L][i], a);
+        ss[L] = a;
+    }
+    for (int o = 16; o > 0; o >>= 1) {
+        float n[32];
+        for (int L = 0; L < 32; L++) n[L] = ss[L] + ss[L ^ o];
+        memcpy(ss, n, sizeof(n));
+    }
+    const float sigma = sqrtf(fmaxf(ss[0] / 128.0f, 1e-12f));
+    const int nb = tq_lane_bits(fmt), bpv = vvo_kv_bytes_per_vec(fmt);
+    uint32_t words[16] = {0};
+    for (int L = 0; L < 32; L++) {
+        const uint32_t bits = tq_pack4(fmt, v[L], 1.0f / sigma);
+        const int bit = nb * L;
+        words[bit >> 5] |= bits << (bit & 31);
+        if ((bit & 31) + nb > 32) words[(bit >> 5) + 1] |= bits >> (32 - (bit & 31));
+    }
+    memcpy(dst, words, (size_t)bpv);
+    *meta = vvo_float_to_half_rne(sigma);
+}
+
+int vvo_kv_store_tq(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads, int fmt,
+                    uint8_t* store, uint16_t* meta16) {
+    if (!src16 || !store || !meta16) return VVO_ERR_NULL_PTR;
+    if (fmt < VVO_KV_TQ4 || fmt > VVO_KV_TQ1_5) return VVO_ERR_INVALID_ARG;
+    const int bpv = vvo_kv_bytes_per_vec(fmt);
+    for (int p = 0; p < n_pos; p++)
+        for (int h = 0; h < n_kv_heads; h++) {
+            const size_t vec = (size_t)p * n_kv_heads + h;
+            tq_store_one(fmt, src16 + vec * 128, ref16 ? ref16 + (size_t)h * 128 : NULL, store + vec * bpv,
+                         meta16 + vec);
+        }
+    return VVO_OK;
+}
+
+/* Stored vectors back to FP16, in the space they were stored in (rotated for
+ * TurboQuant), plus the reference when given (kv_quant.cu: kv_dequant_kernel). */
+int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t* ref16, int n_pos,
+                   int n_kv_heads, int fmt, uint16_t* out16) {
+    if (!store || !out16) return VVO_ERR_NULL_PTR;
+    const int bpv = vvo_kv_bytes_per_vec(fmt);
+    for (int p = 0; p < n_pos; p++)
+        for (int h = 0; h < n_kv_heads; h++) {
+            const size_t vec = (size_t)p * n_kv_heads + h;
+            const uint8_t* src = store + vec * bpv;
+            float val[128];
+            if (fmt == 1 || fmt == 2) {
+                for (int d = 0; d < 128; d++) val[d] = fp8_decode_one(src[d], fmt == 2);
+            } else if (fmt >= VVO_KV_TQ4 && fmt <= VVO_KV_TQ1_5) {
+                if (!meta16) return VVO_ERR_NULL_PTR;
+                uint32_t words[17] = {0};
+                memcpy(words, src, (size_t)bpv);
+                const int nb = tq_lane_bits(fmt);
+                const float sigma = vvo_half_to_float(meta16[vec]);
+                for (int L = 0; L < 32; L++) {
+                    const int bit = nb * L, sh = bit & 31;
+                    const uint32_t lo = words[bit >> 5], hi = words[(bit >> 5) + 1];
+                    const uint32_t bits = (sh ? ((lo >> sh) | (hi << (32 - sh))) : lo) & ((1u << nb) - 1u);
+                    tq_unpack4(fmt, bits, sigma, val + 4 * L);
+                }
+            } else {
+                return VVO_ERR_INVALID_ARG;
+            }
+            for (int d = 0; d < 128; d++) {
+                float x = val[d];
+                if (ref16) x += vvo_half_to_float(ref16[(size_t)h * 128 + d]);
+                out16[vec * 128 + d] = vvo_float_to_half_rne(x);
+            }
+        }
     return VVO_OK;
 }
 

@@ -180,6 +180,29 @@ int vvo_kv_build_ref(const uint16_t* k16, int n_pos, int n_kv_heads, int head_di
 int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads,
                      int head_dim, int e5m2, uint8_t* store);
 
+/* The TurboQuant KV-cache codec (formats 3..6 of include/vibevoice/kv_quant.h:
+ * 4, 3, 2 and 1.5 bits per value, plus an FP16 RMS per vector). Like the FP8
+ * codec the reference holds it only as accelerator code (src/cuda/kv_codec.cuh:
+ * 38-62, 130-165, 180-285; kv_quant.cu:86-119, 171-199); this restates it with
+ * the accelerator's order of FP32 additions. Pinned by what the method fixes:
+ * the transform is the 128-point Hadamard matrix times a +-1 diagonal, scaled
+ * to be orthogonal; the level tables are the Lloyd-Max fixed points of a unit
+ * Gaussian and reach the signal-to-noise ratios the reference quotes for them;
+ * a code is the nearest level (code word). The particular +-1 pattern (a hash
+ * of the channel index) is restated only: parity unpinned for that one table,
+ * which no result depends on as long as store and reader agree.
+ *   vvo_kv_rotate   in-place transform (or its inverse) of n_vectors x 128 FP16
+ *   vvo_kv_store_tq FP16 [n_pos][n_kv_heads][128] (minus ref16 [n_kv_heads][128]
+ *                   when given) -> codes [..][bytes_per_vec] and meta16 [..]
+ *   vvo_kv_dequant  any quantised format (FP8 too) back to FP16 in the stored
+ *                   space, plus ref16 when given */
+int vvo_kv_bytes_per_vec(int fmt);
+int vvo_kv_rotate(uint16_t* x16, int n_vectors, int inverse);
+int vvo_kv_store_tq(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads, int fmt,
+                    uint8_t* store, uint16_t* meta16);
+int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t* ref16, int n_pos,
+                   int n_kv_heads, int fmt, uint16_t* out16);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

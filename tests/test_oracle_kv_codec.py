@@ -73,3 +73,108 @@ def test_reference_key_and_store():
         want = oracle.fp8_encode(oracle.widen(k) - oracle.widen(ref)[None], e5m2)
         assert np.array_equal(store, want)
         assert np.array_equal(oracle.kv_store_fp8(k, None, e5m2), oracle.fp8_encode(oracle.widen(k), e5m2))
+
+
+# ── TurboQuant ──────────────────────────────────────────────────────────────
+TQ = {3: dict(bits=4, snr_db=20.2), 4: dict(bits=3, snr_db=14.6), 5: dict(bits=2, snr_db=9.3), 6: dict(bits=1.5, snr_db=7.0)}
+
+
+def test_rotation_is_the_scaled_hadamard_matrix_times_signs():
+    """Against the explicit 128 x 128 matrix H[i][j] = (-1)^popcount(i & j) / sqrt(128)
+    in FP64: rotate(x) = H (s * x) for ONE +-1 diagonal s (read off by rotating
+    nothing but its inverse), the inverse undoes it, and norms are kept."""
+    idx = np.arange(128)
+    H = np.array([[(-1.0) ** bin(i & j).count("1") for j in idx] for i in idx]) / np.sqrt(128.0)
+    x = oracle.normal_f16((40, 128), 1, std=2.0)
+    xf = oracle.widen(x).astype(np.float64)
+    y = oracle.widen(oracle.kv_rotate(x)).astype(np.float64)
+    # the sign diagonal: rotate a vector of ones, undo the Hadamard part
+    ones = oracle.narrow(np.ones((1, 128), np.float32))
+    s = np.rint(H.T @ oracle.widen(oracle.kv_rotate(ones)).astype(np.float64)[0] * 1.0)
+    s = np.sign(H @ oracle.widen(oracle.kv_rotate(ones)).astype(np.float64)[0])
+    assert set(np.unique(s)) <= {-1.0, 1.0} and 20 < (s < 0).sum() < 108
+    want = (xf * s[None]) @ H.T
+    assert np.max(np.abs(y - want)) <= 2.0 ** -10 * np.max(np.abs(want)) + 1e-6
+    back = oracle.widen(oracle.kv_rotate(oracle.kv_rotate(x), inverse=True)).astype(np.float64)
+    assert np.max(np.abs(back - xf)) <= 3 * 2.0 ** -10 * np.max(np.abs(xf))
+    assert np.allclose((y ** 2).sum(1), (xf ** 2).sum(1), rtol=3e-3)
+
+
+def gaussian_cell_means(levels):
+    """Centroids of N(0,1) over the cells bounded by the mid-points of `levels`."""
+    from scipy.stats import norm
+    edges = np.concatenate([[-np.inf], (levels[1:] + levels[:-1]) / 2, [np.inf]])
+    lo, hi = edges[:-1], edges[1:]
+    return (norm.pdf(lo) - norm.pdf(hi)) / (norm.cdf(hi) - norm.cdf(lo))
+
+
+@pytest.mark.parametrize("fmt", [3, 4, 5])
+def test_scalar_levels_are_the_lloyd_max_fixed_point(fmt):
+    """Store a vector whose RMS is 1 and read the levels back through the codec;
+    each must be the mean of a unit Gaussian over its own cell."""
+    nb = TQ[fmt]["bits"]
+    # every code value appears when the stored values are the cell centres; read the table off the dequantiser
+    store = np.zeros((1, 1, oracle.kv_bytes_per_vec(fmt)), np.uint8)
+    n_levels = 1 << nb
+    codes = np.arange(128) % n_levels
+    stream = 0
+    for d, c in enumerate(codes):
+        stream |= int(c) << (d * nb)
+    store[0, 0] = np.frombuffer(stream.to_bytes(oracle.kv_bytes_per_vec(fmt), "little"), np.uint8)
+    one = oracle.narrow(np.ones((1, 1), np.float32))
+    levels = oracle.widen(oracle.kv_dequant(store, one, None, fmt))[0, 0, :n_levels].astype(np.float64)
+    assert np.all(np.diff(levels) > 0) and np.allclose(levels, -levels[::-1], atol=1e-3)
+    assert np.max(np.abs(levels - gaussian_cell_means(levels))) < 4e-3        # FP16 read-back of 6-digit tables
+
+
+@pytest.mark.parametrize("fmt", [3, 4, 5, 6])
+def test_codes_are_nearest_and_reach_the_quoted_signal_to_noise(fmt):
+    """On Gaussian vectors: dequant(store(x)) is, per value (per pair for 1.5
+    bits), the nearest entry of the scaled table, and the signal-to-noise ratio
+    is the one the reference quotes for the format (kv_codec.cuh:40-41)."""
+    n = 64
+    x = oracle.normal_f16((n, 1, 128), 7 + fmt, std=1.7)
+    store, meta = oracle.kv_store_tq(x, None, fmt)
+    assert store.shape[-1] == oracle.kv_bytes_per_vec(fmt)
+    y = oracle.widen(oracle.kv_rotate(x)).astype(np.float64)[:, 0]              # what was quantised (to FP16 rounding)
+    got = oracle.widen(oracle.kv_dequant(store, meta, None, fmt)).astype(np.float64)[:, 0]
+    sigma = oracle.widen(meta).astype(np.float64)[:, 0]
+    assert np.allclose(sigma, np.sqrt((y ** 2).mean(1)), rtol=2e-3)
+    err = ((got - y) ** 2).sum() / (y ** 2).sum()
+    snr = -10 * np.log10(err)
+    assert abs(snr - TQ[fmt]["snr_db"]) < 0.5, snr
+    # nearest: no other table entry is closer (up to the FP16 rounding of the rotated input)
+    if fmt != 6:
+        vals = np.sort((got / sigma[:, None]).ravel())
+        table = np.array([c.mean() for c in np.split(vals, np.nonzero(np.diff(vals) > 0.05)[0] + 1)])
+        assert len(table) == 1 << TQ[fmt]["bits"]
+        d_best = np.abs(y[:, :, None] / sigma[:, None, None] - table[None, None, :]).min(-1)
+        d_got = np.abs(y / sigma[:, None] - got / sigma[:, None])
+        assert np.max(d_got - d_best) < 5e-3
+    else:
+        pairs = (got / sigma[:, None]).reshape(n, 64, 2)
+        flat = pairs.reshape(-1, 2)
+        table = []
+        for p in flat:                                   # cluster the read-back pairs (FP16 noise apart)
+            if not any(np.abs(p - t).max() < 0.05 for t in table):
+                table.append(p)
+        table = np.array(table)
+        assert len(table) == 8
+        yp = (y / sigma[:, None]).reshape(n, 64, 2)
+        d_best = ((yp[:, :, None, :] - table[None, None]) ** 2).sum(-1).min(-1)
+        d_got = ((yp - pairs) ** 2).sum(-1)
+        assert np.max(d_got - d_best) < 1e-2
+
+
+def test_turboquant_reference_key_and_fp8_dequant_agree_with_the_codec():
+    k = oracle.normal_f16((9, 4, 128), 3, mean=2.0, std=1.0)
+    ref = oracle.kv_build_ref(k)
+    centred = oracle.narrow(oracle.widen(k) - oracle.widen(ref)[None])
+    for fmt in (3, 6):
+        a, ma = oracle.kv_store_tq(k, ref, fmt)
+        # subtracting in FP32 before the transform is not subtracting FP16-rounded differences, but nearly
+        b, mb = oracle.kv_store_tq(centred, None, fmt)
+        assert (a != b).mean() < 0.02 and np.abs(oracle.widen(ma) - oracle.widen(mb)).max() < 1e-2
+    for fmt, e5m2 in ((1, False), (2, True)):
+        codes = oracle.kv_store_fp8(k, None, e5m2)
+        assert np.array_equal(oracle.widen(oracle.kv_dequant(codes, None, None, fmt)), oracle.fp8_decode(codes, e5m2))
