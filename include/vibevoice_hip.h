@@ -279,17 +279,17 @@ vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
 typedef struct vv_kv_view {
     const void* k;
     const void* v;
-    const void* k_meta;       /* TurboQuant formats only: unused here */
+    const void* k_meta;       /* TurboQuant formats: FP16 RMS per stored vector [rows][n_kv_heads] */
     const void* v_meta;
     const int*  page_table;   /* device memory, or NULL */
-    int         format;       /* vv_kv_format_t: VV_KV_FP16 (0), VV_KV_FP8_E4M3 (1), VV_KV_FP8_E5M2 (2) */
+    int         format;       /* vv_kv_format_t 0..6: FP16, FP8 E4M3 / E5M2, TurboQuant 4 / 3 / 2 / 1.5 bits */
     int         n_kv_heads;
     int         head_dim;
 } vv_kv_view_t;
 
 /* The backend a context should name (never VV_ATTN_AUTO = 0). All backend
- * names run the same kernels here; a TurboQuant format (or FP8 at a head_dim
- * other than 128) answers VV_ATTN_FA1 (1) and the attention calls then decline.
+ * names run the same kernels here; a packed format at a head_dim other than
+ * 128 answers VV_ATTN_FA1 (1) and the attention calls then decline.
  * replaces device.h:545-546 (src/cuda/attention_fi.cu:554-583). */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
                     int n_kv_heads, int head_dim);
@@ -343,7 +343,11 @@ vv_status_t vv_gqa_attention_prefill_dev(const void* q, const void* k, const voi
  * saturating, NaN -> 0); when k_ref is set the head's reference key is
  * subtracted from K first (softmax does not see a shift common to all keys),
  * and with build_ref it is first computed as this run's mean key. TurboQuant
- * formats: VV_ERR_UNSUPPORTED. replaces device.h:597-602
+ * (4 / 3 / 2 / 1.5 bits, head_dim 128): the vector, minus the reference key,
+ * goes through the randomised Hadamard transform, its RMS goes to k_meta /
+ * v_meta [rows][n_kv_heads] as FP16, and each value (pair) takes the code of
+ * the nearest Lloyd-Max level (code word) of value / RMS
+ * (src/cuda/kv_quant.cu:86-119). replaces device.h:597-602
  * (src/cuda/kv_quant.cu:507-552). */
 vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_store,
                             void* v_store, void* k_meta, void* v_meta, void* k_ref,
@@ -356,15 +360,18 @@ vv_status_t vv_kv_quant_store_dev(const void* k_fp16, const void* v_fp16, void* 
                                   void* v_store, void* k_meta, void* v_meta, void* k_ref,
                                   bool build_ref, int n_kv_heads, int head_dim, int pos,
                                   const int* d_pos, int n_positions, int kv_format, void* stream);
-/* An FP8 store [n_pos][n_kv_heads][128] back to FP16, plus `ref` [n_kv_heads][128]
+/* A packed store [n_pos][n_kv_heads][bytes per vector] back to FP16 in the
+ * space it was stored in (rotated for TurboQuant), plus `ref` [n_kv_heads][128]
  * when given. replaces device.h:697-699 (kv_quant.cu:586-603). */
 vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* ref,
                               void* out_fp16, int n_kv_heads, int head_dim, int n_pos,
                               int kv_format, void* stream);
 /* Attention over a quantised cache given as pointers: vv_attn_decode /
- * vv_attn_prefill with the format in the view. Every FP8 value is an FP16
- * value, so the result is, bit for bit, that of an FP16 cache holding the
- * decoded values. replace device.h:662-675 (kv_quant.cu:605-673). */
+ * vv_attn_prefill with the format in the view. The codes are widened to FP16
+ * on their way into the tile, so the result is, bit for bit, that of an FP16
+ * cache holding what vv_kv_dequant_dev returns. A TurboQuant cache holds
+ * rotated vectors: rotate Q before and un-rotate the output after.
+ * replace device.h:662-675 (kv_quant.cu:605-673). */
 vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, const void* v_store,
                                           const void* k_meta, const void* v_meta, void* output,
                                           int n_q_heads, int n_kv_heads, int head_dim,
@@ -375,6 +382,11 @@ vv_status_t vv_gqa_attention_prefill_q_dev(const void* q, const void* k_store, c
                                            int n_q_heads, int n_kv_heads, int head_dim, int q_len,
                                            int q_offset, int kv_len, bool causal, int kv_format,
                                            void* stream);
+/* In-place randomised Hadamard transform of [rows][n_heads][128] FP16 (the
+ * orthogonal map TurboQuant stores K and V under: dot(Hq, Hk) == dot(q, k)) and
+ * its inverse. replace kv_quant.h:96-101 (kv_quant.cu:171-199, 569-584). */
+vv_status_t vv_kv_rotate_dev(void* x_fp16, int n_heads, int head_dim, int rows, void* stream);
+vv_status_t vv_kv_unrotate_dev(void* x_fp16, int n_heads, int head_dim, int rows, void* stream);
 /* page_table[first + i] = pages[i], i < n, ordered on the stream; `pages` is
  * host memory, consumed before the call returns. replaces device.h:610-611. */
 vv_status_t vv_kv_page_map_dev(int* page_table, int first, int n, const int* pages,

@@ -115,7 +115,10 @@ def test_attention_host_queries():
         for paged in (False, True):
             got = dev.vv_attn_resolve(requested, 0, paged, 28, 4, 128)
             assert got in (FA1, FA2, FI) and (requested in (AUTO, got) or paged)
-            assert dev.vv_attn_resolve(requested, 3, paged, 28, 4, 128) == FA1     # not an FP16 cache
+            for fmt in (1, 3, 6):                                                  # FP8 and TurboQuant caches are served ...
+                assert dev.vv_attn_resolve(requested, fmt, paged, 28, 4, 128) == got
+                assert dev.vv_attn_resolve(requested, fmt, paged, 28, 4, 64) == FA1   # ... at head_dim 128 only
+            assert dev.vv_attn_resolve(requested, 9, paged, 28, 4, 128) == FA1     # no such format
     assert dev.vv_attn_resolve(FA1, 0, True, 28, 4, 128) != FA1                    # fa1 never pages
     assert dev.vv_attn_scratch_bytes(28, 4, 128) == 28 * 256 * 132 * 4
     shapes = [dev.vv_attn_decode_shape(FA2, 28, 4, n) for n in range(1, 20000, 37)]
@@ -133,7 +136,7 @@ def test_unsupported_library_declines_everything_and_overlaps_nothing():
     import ctypes as C
     out = subprocess.check_output(["nm", "-D", "--defined-only", STUB_PATH], text=True)
     stubs = sorted(l.split()[-1] for l in out.splitlines() if " T vv_" in l)
-    assert len(stubs) == 28
+    assert len(stubs) == 26
     assert not set(stubs) & set(dev.SIGNATURES)          # no symbol defined twice
     lib = C.CDLL(STUB_PATH)
     zero = {"vv_i8_head_argmax_scratch_bytes"}

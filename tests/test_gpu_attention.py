@@ -183,13 +183,13 @@ def test_declines_and_edges():
     assert dev.vv_attn_prefill(FA2, None, C.addressof(vw), p, nq, 4, 0, 4, True, None, stream()) == dev.VV_ERR_NULL_PTR
     assert dev.vv_attn_prefill(FA2, p, C.addressof(vw), p, nq, 0, 0, 4, True, None, stream()) == dev.VV_OK
     assert dev.vv_attn_decode(FA2, p, C.addressof(vw), p, nq, 0, None, None, stream()) == dev.VV_OK
-    tq = view_of(d, d, nkv, hd, fmt=3)             # a TurboQuant cache: not served
+    tq = view_of(d, d, nkv, hd, fmt=3)             # a TurboQuant cache without its per-vector scales
     assert dev.vv_attn_prefill(FA2, p, C.addressof(tq), p, nq, 4, 0, 4, True, None, stream()) == dev.VV_ERR_UNSUPPORTED
     assert dev.vv_attn_decode(FA2, p, C.addressof(tq), p, nq, 4, None, None, stream()) == dev.VV_ERR_UNSUPPORTED
     odd = view_of(d, d, 3, hd)                     # 2 query heads over 3 KV heads
     assert dev.vv_attn_prefill(FA2, p, C.addressof(odd), p, nq, 4, 0, 4, True, None, stream()) == dev.VV_ERR_UNSUPPORTED
     big = view_of(d, d, nkv, hd)                   # more than one slice needs the scratch
     assert dev.vv_attn_decode(FA2, p, C.addressof(big), p, nq, 4000, None, None, stream()) == dev.VV_ERR_NULL_PTR
-    assert dev.vv_kv_store_dev(p, p, p, p, None, None, None, False, nkv, hd, 0, None, 1, 3, None,
-                               stream()) == dev.VV_ERR_UNSUPPORTED
+    assert dev.vv_kv_store_dev(p, p, p, p, None, None, None, False, nkv, hd, 0, None, 1, 7, None,
+                               stream()) == dev.VV_ERR_UNSUPPORTED       # FP32 caches are the CPU path's
     torch.cuda.synchronize()

@@ -183,7 +183,7 @@ def test_decode_equals_fp16_cache_of_decoded_values(fmt, cache_len, paged):
 
 def test_formats_and_shapes_not_served():
     P = torch.zeros(4096, dtype=torch.float16, device="cuda").data_ptr()
-    for fmt in (3, 4, 5, 6):          # TurboQuant
+    for fmt in (7, 9):                # FP32 (the CPU path's), no such format
         assert dev.vv_kv_quant_store_dev(P, P, P, P, P, P, None, False, NKV, HD, 0, None, 1, fmt, stream()) == dev.VV_ERR_UNSUPPORTED
         assert dev.vv_kv_dequant_dev(P, P, None, P, NKV, HD, 1, fmt, stream()) == dev.VV_ERR_UNSUPPORTED
         assert dev.vv_gqa_attention_decode_q_dev(P, P, P, P, P, P, 28, NKV, HD, 10, None, fmt, P, stream()) == dev.VV_ERR_UNSUPPORTED
@@ -194,3 +194,6 @@ def test_formats_and_shapes_not_served():
     assert dev.vv_kv_quant_store_dev(None, P, P, P, None, None, None, False, NKV, HD, 0, None, 1, E4M3, stream()) == dev.VV_ERR_NULL_PTR
     assert dev.vv_attn_resolve(FA2, E4M3, True, 28, NKV, HD) == FA2 and dev.vv_attn_resolve(FA2, E5M2, False, 28, NKV, 64) == 1
     assert dev.vv_gqa_attention_decode_q_dev(P, P, P, None, None, P, 28, NKV, HD, 0, None, E4M3, P, stream()) == dev.VV_OK
+    # TurboQuant needs the per-vector scales
+    assert dev.vv_gqa_attention_decode_q_dev(P, P, P, None, None, P, 28, NKV, HD, 10, None, 3, P, stream()) == dev.VV_ERR_UNSUPPORTED
+    assert dev.vv_kv_dequant_dev(P, None, None, P, NKV, HD, 1, 3, stream()) == dev.VV_ERR_NULL_PTR

@@ -55,6 +55,7 @@ constexpr int kVtStride = kKeyTile + 4;   // halves per transposed-V row: 136 B
 struct KvTile {
     Chunk k[kKeyTile * (kD / 8)];                 // [key][16 slots], slot ^ (key & 15)
     __align__(16) h16 vt[kD * kVtStride];         // [channel][key]
+    float lev[16];                                // TurboQuant caches: the format's level table
 };
 
 // Per-lane state of one query row (lane % 32) over the keys seen so far: O^T
@@ -88,6 +89,31 @@ struct TileRegs {
 // E4M3 / E5M2 value is an FP16 value, so from there on the tile is the tile of
 // an FP16 cache that holds the decoded values.
 constexpr int kFmtFp16 = 0, kFmtE4M3 = 1, kFmtE5M2 = 2;
+// TurboQuant (kv_quant.h:37-40): 4, 3, 2 or 1.5 bits per value as one little-endian
+// bit stream per vector, value d at bit d * bits (pair P at bit 3 P for 1.5 bits),
+// each code an index into a table of Lloyd-Max levels of a unit Gaussian, times
+// the vector's own RMS (FP16, one per vector, beside the store). The vectors are
+// stored rotated; the caller rotates Q and un-rotates O (vv_kv_rotate_dev).
+constexpr int kFmtTq4 = 3, kFmtTq3 = 4, kFmtTq2 = 5, kFmtTq15 = 6;
+
+__device__ const float kTqLevels[4][16] = {
+    {-2.725112f, -2.065280f, -1.613787f, -1.251845f, -0.938657f, -0.654379f, -0.386970f, -0.127960f,
+     +0.127960f, +0.386970f, +0.654379f, +0.938657f, +1.251845f, +1.613787f, +2.065280f, +2.725112f},
+    {-2.150300f, -1.343258f, -0.755588f, -0.244756f, +0.244756f, +0.755588f, +1.343258f, +2.150300f},
+    {-1.511418f, -0.452456f, +0.452456f, +1.511418f},
+    // 1.5 bits: eight 2-D code words, a pair of values shares one 3-bit index
+    {-1.500251f, +0.674678f, -1.127883f, -0.787015f, -0.283251f, +0.390133f, -0.103102f, +1.624620f,
+     +0.100120f, -1.618563f, +0.286482f, -0.379555f, +1.134227f, +0.790368f, +1.496572f, -0.666578f}};
+
+template <int kFmt> struct KvFormat {
+    static constexpr bool kTq = kFmt >= kFmtTq4;
+    // bytes per 128-value vector; bits one 8-channel slot takes; bits per code; values per code
+    static constexpr int kBytes = kFmt == kFmtFp16 ? 256 : kFmt <= kFmtE5M2 ? 128
+                                : kFmt == kFmtTq4 ? 64 : kFmt == kFmtTq3 ? 48 : kFmt == kFmtTq2 ? 32 : 24;
+    static constexpr int kCodeBits = kFmt == kFmtTq4 ? 4 : kFmt == kFmtTq2 ? 2 : 3;
+    static constexpr int kPerCode = kFmt == kFmtTq15 ? 2 : 1;
+    static constexpr int kSlotBits = 8 / kPerCode * kCodeBits;
+};
 
 // Four FP8 codes (the bytes of `codes`) as two half2 words, lanes in byte order.
 template <int kFmt>
@@ -107,11 +133,49 @@ __device__ __forceinline__ void widen4(uint32_t codes, uint32_t& lo, uint32_t& h
     }
 }
 
-// Slot `slot` (eight channels) of vector `vec` (= cache row * n_kv_heads + KV head) as FP16.
+// `count` bits at bit `offset` of a vector of `nwords` 32-bit words.
+__device__ __forceinline__ uint32_t stream_bits(const uint32_t* __restrict__ words, int nwords, int offset,
+                                                int count) {
+    const int wi = offset >> 5, sh = offset & 31;
+    const uint32_t lo = words[wi], hi = words[min(wi + 1, nwords - 1)];
+    const uint32_t v = sh ? ((lo >> sh) | (hi << (32 - sh))) : lo;
+    return count == 32 ? v : v & ((1u << count) - 1u);
+}
+
+// The eight channels of slot `slot` of a TurboQuant vector in FP32: RMS times level.
 template <int kFmt>
-__device__ __forceinline__ Chunk load_slot(const void* __restrict__ cache, size_t vec, int slot) {
+__device__ __forceinline__ void tq_slot_values(const void* __restrict__ cache, const h16* __restrict__ meta,
+                                               const float* lev, size_t vec, int slot, float (&val)[8]) {
+    typedef KvFormat<kFmt> F;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(cache) + vec * F::kBytes);
+    const uint32_t bits = stream_bits(words, F::kBytes / 4, slot * F::kSlotBits, F::kSlotBits);
+    const float sigma = (float)meta[vec];
+#pragma unroll
+    for (int c = 0; c < 8 / F::kPerCode; ++c) {
+        const uint32_t code = (bits >> (F::kCodeBits * c)) & ((1u << F::kCodeBits) - 1u);
+        if constexpr (F::kPerCode == 1) {
+            val[c] = sigma * lev[code];
+        } else {
+            val[2 * c] = sigma * lev[2 * code];
+            val[2 * c + 1] = sigma * lev[2 * code + 1];
+        }
+    }
+}
+
+// Slot `slot` (eight channels) of vector `vec` (= cache row * n_kv_heads + KV head) as FP16.
+// `meta` (per-vector RMS) and `lev` (the level table, in LDS) serve the TurboQuant formats.
+template <int kFmt>
+__device__ __forceinline__ Chunk load_slot(const void* __restrict__ cache, const h16* __restrict__ meta,
+                                           const float* lev, size_t vec, int slot) {
     if constexpr (kFmt == kFmtFp16) {
         return load_chunk(static_cast<const Chunk*>(cache) + vec * (kD / 8) + slot);
+    } else if constexpr (KvFormat<kFmt>::kTq) {
+        float val[8];
+        tq_slot_values<kFmt>(cache, meta, lev, vec, slot, val);
+        h16x8 out;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) out[c] = to_half(val[c]);
+        return __builtin_bit_cast(Chunk, out);
     } else {
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
@@ -125,17 +189,35 @@ __device__ __forceinline__ Chunk load_slot(const void* __restrict__ cache, size_
     }
 }
 
+struct KvSource {
+    const void* k;
+    const void* v;
+    const h16* k_meta;
+    const h16* v_meta;
+    const int* page_table;
+};
+
+// The format's level table into the tile (TurboQuant only); every thread of the workgroup calls it.
+template <int kFmt>
+__device__ __forceinline__ void load_levels(KvTile& tile, int tid) {
+    if constexpr (KvFormat<kFmt>::kTq) {
+        if (tid < 16) tile.lev[tid] = kTqLevels[kFmt - kFmtTq4][tid];
+        __syncthreads();
+    }
+}
+
 template <int kThreads, int kFmt>
-__device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const void* __restrict__ Kc,
-                                           const void* __restrict__ Vc,
-                                           const int* __restrict__ page_table, int n_kv_heads,
-                                           int kvh, int t0, int last_key, int tid) {
+__device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const KvSource& src, const float* lev,
+                                           int n_kv_heads, int kvh, int t0, int last_key, int tid) {
+    const void* __restrict__ Kc = src.k;
+    const void* __restrict__ Vc = src.v;
+    const int* __restrict__ page_table = src.page_table;
     constexpr int kIter = TileRegs<kThreads>::kIter;
 #pragma unroll
     for (int i = 0; i < kIter; ++i) {
         const int q = tid + i * kThreads, r = q >> 4, slot = q & 15;
         const int row = cache_row(page_table, min(t0 + r, last_key));
-        regs.k[i] = load_slot<kFmt>(Kc, (size_t)row * n_kv_heads + kvh, slot);
+        regs.k[i] = load_slot<kFmt>(Kc, src.k_meta, lev, (size_t)row * n_kv_heads + kvh, slot);
     }
 #pragma unroll
     for (int i = 0; i < kIter / 4; ++i) {
@@ -143,7 +225,7 @@ __device__ __forceinline__ void fetch_tile(TileRegs<kThreads>& regs, const void*
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int row = cache_row(page_table, min(t0 + 4 * kg + j, last_key));
-            regs.v[4 * i + j] = load_slot<kFmt>(Vc, (size_t)row * n_kv_heads + kvh, dchunk);
+            regs.v[4 * i + j] = load_slot<kFmt>(Vc, src.v_meta, lev, (size_t)row * n_kv_heads + kvh, dchunk);
         }
     }
 }
@@ -250,12 +332,12 @@ __device__ __forceinline__ void load_query(h16x8 (&qf)[kD / 16], const h16* qp, 
 // ── prefill ──────────────────────────────────────────────────────────────
 template <int kFmt>
 __global__ __launch_bounds__(kBlock, 2) void prefill128(
-    const h16* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
-    const int* __restrict__ page_table, h16* __restrict__ O, int n_q_heads, int n_kv_heads,
+    const h16* __restrict__ Q, KvSource src, h16* __restrict__ O, int n_q_heads, int n_kv_heads,
     int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
     __shared__ KvTile tile;
 
     const int tid = (int)threadIdx.x;
+    load_levels<kFmt>(tile, tid);
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int col = lane & 31;        // this lane's query row inside the wave's 32
@@ -281,13 +363,13 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
     st.reset();
 
     TileRegs<kBlock> regs;
-    if (wg_limit > 0) fetch_tile<kBlock, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, 0, kv_len - 1, tid);
+    if (wg_limit > 0) fetch_tile<kBlock, kFmt>(regs, src, tile.lev, n_kv_heads, kvh, 0, kv_len - 1, tid);
     for (int t0 = 0; t0 < wg_limit; t0 += kKeyTile) {
         __syncthreads();
         commit_tile<kBlock>(tile, regs, tid);
         __syncthreads();
         if (t0 + kKeyTile < wg_limit)
-            fetch_tile<kBlock, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, t0 + kKeyTile, kv_len - 1, tid);
+            fetch_tile<kBlock, kFmt>(regs, src, tile.lev, n_kv_heads, kvh, t0 + kKeyTile, kv_len - 1, tid);
         if (t0 >= wave_limit) continue;
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
@@ -377,13 +459,13 @@ constexpr int kPartFloats = kD + 4;        // per (head, slice): 128 channels, m
 
 template <int kFmt>
 __global__ __launch_bounds__(kWave) void decode128(
-    const h16* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
-    const int* __restrict__ page_table, h16* __restrict__ O, float* __restrict__ parts,
+    const h16* __restrict__ Q, KvSource src, h16* __restrict__ O, float* __restrict__ parts,
     int n_q_heads, int n_kv_heads, int cache_len, const int* __restrict__ d_cache_len,
     int n_parts, float scale_log2) {
     __shared__ KvTile tile;
 
     const int lane = (int)threadIdx.x;
+    load_levels<kFmt>(tile, lane);
     const int col = lane & 31, half = lane >> 5;
     const int part = (int)blockIdx.x;
     const int kvh = (int)blockIdx.y;
@@ -400,13 +482,13 @@ __global__ __launch_bounds__(kWave) void decode128(
     st.reset();
 
     TileRegs<kWave> regs;
-    if (begin < end) fetch_tile<kWave, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, begin, end - 1, lane);
+    if (begin < end) fetch_tile<kWave, kFmt>(regs, src, tile.lev, n_kv_heads, kvh, begin, end - 1, lane);
     for (int t0 = begin; t0 < end; t0 += kKeyTile) {
         __syncthreads();
         commit_tile<kWave>(tile, regs, lane);
         __syncthreads();
         if (t0 + kKeyTile < end)
-            fetch_tile<kWave, kFmt>(regs, Kc, Vc, page_table, n_kv_heads, kvh, t0 + kKeyTile, end - 1, lane);
+            fetch_tile<kWave, kFmt>(regs, src, tile.lev, n_kv_heads, kvh, t0 + kKeyTile, end - 1, lane);
         f32x16 s[2];
         tile_scores(tile, qf, col, half, s);
         if (t0 + kKeyTile > end) {
@@ -589,20 +671,174 @@ __global__ __launch_bounds__(kBlock) void kv_store_fp8(
     *(reinterpret_cast<u32x2*>(keys ? k_store : v_store) + dst) = u32x2{w[0], w[1]};
 }
 
-// FP8 codes back to FP16 (plus the reference key when given): tests, offload.
+// ── TurboQuant store, unpack and rotation (src/cuda/kv_quant.cu:86-119, 171-199;
+//    kv_codec.cuh:130-165, 228-285) ──────────────────────────────────────────
+// 32 lanes per vector (two vectors per wave), four consecutive channels per lane,
+// FP32 additions in exactly this order: strides 1 and 2 inside a lane, then lane
+// strides 1 .. 16, the upper partner taking (other - own).
+constexpr float kWhtNorm = 0.0883883476f;      // 1 / sqrt(128)
+
+__device__ __forceinline__ float tq_sign(int d) {     // the fixed +-1 pattern of the transform
+    uint32_t h = (uint32_t)d * 2654435761u + 0x9E3779B9u;
+    h ^= h >> 15; h *= 0x85EBCA6Bu; h ^= h >> 13;
+    return (h & 1u) ? -1.0f : 1.0f;
+}
+
+__device__ __forceinline__ void wht128(float (&v)[4], int lane32) {
+    float a;
+    a = v[0] + v[1]; v[1] = v[0] - v[1]; v[0] = a;
+    a = v[2] + v[3]; v[3] = v[2] - v[3]; v[2] = a;
+    a = v[0] + v[2]; v[2] = v[0] - v[2]; v[0] = a;
+    a = v[1] + v[3]; v[3] = v[1] - v[3]; v[1] = a;
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float o = __shfl_xor(v[i], m);
+            v[i] = (lane32 & m) ? o - v[i] : v[i] + o;
+        }
+    }
+}
+
+__device__ __forceinline__ void tq_rotate(float (&v)[4], int lane32, bool inverse) {
+    if (!inverse) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= tq_sign(4 * lane32 + i);
+        wht128(v, lane32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= kWhtNorm;
+    } else {
+        wht128(v, lane32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= kWhtNorm * tq_sign(4 * lane32 + i);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void kv_rotate(h16* __restrict__ x, int n_vectors, int inverse) {
+    const int vec = (int)blockIdx.x * (kBlock / 32) + (int)threadIdx.x / 32;
+    const int lane32 = (int)threadIdx.x & 31;
+    h16* p = x + (size_t)min(vec, n_vectors - 1) * kD + 4 * lane32;
+    const h16x4 in = *reinterpret_cast<const h16x4*>(p);
+    float v[4] = {(float)in[0], (float)in[1], (float)in[2], (float)in[3]};
+    tq_rotate(v, lane32, inverse != 0);
+    if (vec < n_vectors) *reinterpret_cast<h16x4*>(p) = h16x4{to_half(v[0]), to_half(v[1]), to_half(v[2]), to_half(v[3])};
+}
+
+// The packed code of a lane's four values: per value the number of mid-points
+// between neighbouring levels it exceeds; 1.5 bits: the nearest of eight 2-D
+// code words per pair, the first winning ties.
 template <int kFmt>
-__global__ __launch_bounds__(kBlock) void kv_dequant_fp8(const void* __restrict__ store,
-                                                         const h16* __restrict__ ref, h16* __restrict__ out,
-                                                         int n_kv_heads, size_t n_slots) {
+__device__ __forceinline__ uint32_t tq_pack4(const float (&y)[4], float inv_sigma) {
+#pragma clang fp contract(off)
+    typedef KvFormat<kFmt> F;
+    const float* lev = kTqLevels[kFmt - kFmtTq4];
+    uint32_t bits = 0;
+    if constexpr (kFmt == kFmtTq15) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const float a = y[2 * p] * inv_sigma, b = y[2 * p + 1] * inv_sigma;
+            uint32_t best = 0;
+            float bd = 3.402823466e+38f;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const float da = a - lev[2 * c], db = b - lev[2 * c + 1];
+                const float d = da * da + db * db;
+                if (d < bd) { bd = d; best = (uint32_t)c; }
+            }
+            bits |= best << (3 * p);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float t = y[i] * inv_sigma;
+            uint32_t c = 0;
+#pragma unroll
+            for (int j = 0; j + 1 < (1 << F::kCodeBits); ++j) c += (t > 0.5f * (lev[j] + lev[j + 1])) ? 1u : 0u;
+            bits |= c << (F::kCodeBits * i);
+        }
+    }
+    return bits;
+}
+
+// blockIdx.y = 0: keys (minus the head's reference key when there is one), 1: values.
+template <int kFmt>
+__global__ __launch_bounds__(kBlock) void kv_store_tq(
+    const h16* __restrict__ k, const h16* __restrict__ v, uint8_t* __restrict__ k_store,
+    uint8_t* __restrict__ v_store, h16* __restrict__ k_meta, h16* __restrict__ v_meta,
+    const h16* __restrict__ k_ref, int n_kv_heads, int pos, const int* __restrict__ d_pos, int n_positions,
+    const int* __restrict__ page_table) {
+    typedef KvFormat<kFmt> F;
+    constexpr int kLaneBits = 4 / F::kPerCode * F::kCodeBits;      // 16, 12, 8, 6
+    __shared__ uint32_t pack[kBlock / 32][16];
+    const int slot = (int)threadIdx.x / 32, lane32 = (int)threadIdx.x & 31;
+    const int total = n_positions * n_kv_heads;
+    const int idx = (int)blockIdx.x * (kBlock / 32) + slot;
+    const int vec = min(idx, total - 1);
+    const bool keys = blockIdx.y == 0;
+    const int p = vec / n_kv_heads, head = vec % n_kv_heads;
+    const h16x4 in = *reinterpret_cast<const h16x4*>((keys ? k : v) + (size_t)vec * kD + 4 * lane32);
+    float val[4] = {(float)in[0], (float)in[1], (float)in[2], (float)in[3]};
+    if (keys && k_ref) {
+        const h16x4 r = *reinterpret_cast<const h16x4*>(k_ref + (size_t)head * kD + 4 * lane32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) val[i] -= (float)r[i];
+    }
+    tq_rotate(val, lane32, false);
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss = fmaf(val[i], val[i], ss);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    const float sigma = sqrtf(fmaxf(ss / (float)kD, 1e-12f));
+    const uint32_t bits = tq_pack4<kFmt>(val, 1.0f / sigma);
+
+    // lanes own overlapping words: assemble the vector's bit stream in LDS
+    if (lane32 < 16) pack[slot][lane32] = 0u;
+    __syncthreads();
+    const int bit = kLaneBits * lane32;
+    atomicOr(&pack[slot][bit >> 5], bits << (bit & 31));
+    if ((bit & 31) + kLaneBits > 32) atomicOr(&pack[slot][(bit >> 5) + 1], bits >> (32 - (bit & 31)));
+    __syncthreads();
+    if (idx >= total) return;
+    const int t = (d_pos ? *d_pos : pos) + p;
+    const size_t row_vec = (size_t)cache_row(page_table, t) * n_kv_heads + head;
+    uint32_t* dst = reinterpret_cast<uint32_t*>((keys ? k_store : v_store) + row_vec * F::kBytes);
+    if (lane32 < F::kBytes / 4) dst[lane32] = pack[slot][lane32];
+    h16* meta = keys ? k_meta : v_meta;
+    if (lane32 == 0 && meta) meta[row_vec] = to_half(sigma);
+}
+
+// Any quantised store back to FP16, in the space it was stored in (rotated for
+// TurboQuant), plus the reference key when given. A thread unpacks eight channels.
+template <int kFmt>
+__global__ __launch_bounds__(kBlock) void kv_dequant(const void* __restrict__ store, const h16* __restrict__ meta,
+                                                     const h16* __restrict__ ref, h16* __restrict__ out,
+                                                     int n_kv_heads, size_t n_slots) {
+    __shared__ float lev[16];
+    if constexpr (KvFormat<kFmt>::kTq) {
+        if (threadIdx.x < 16) lev[threadIdx.x] = kTqLevels[kFmt - kFmtTq4][threadIdx.x];
+        __syncthreads();
+    }
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n_slots) return;
-    h16x8 val = __builtin_bit_cast(h16x8, load_slot<kFmt>(store, i / (kD / 8), (int)(i % (kD / 8))));
+    // FP32 until the one rounding of the output (an FP8 value is exact in FP16 either way)
+    float f[8];
+    if constexpr (KvFormat<kFmt>::kTq) {
+        tq_slot_values<kFmt>(store, meta, lev, i / (kD / 8), (int)(i % (kD / 8)), f);
+    } else {
+        const h16x8 h = __builtin_bit_cast(h16x8, load_slot<kFmt>(store, meta, lev, i / (kD / 8), (int)(i % (kD / 8))));
+#pragma unroll
+        for (int c = 0; c < 8; ++c) f[c] = (float)h[c];
+    }
     if (ref) {
         const int head = (int)((i / (kD / 8)) % n_kv_heads), slot = (int)(i % (kD / 8));
         const h16x8 r = *(reinterpret_cast<const h16x8*>(ref) + head * (kD / 8) + slot);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) val[c] = to_half((float)val[c] + (float)r[c]);
+        for (int c = 0; c < 8; ++c) f[c] += (float)r[c];
     }
+    h16x8 val;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) val[c] = to_half(f[c]);
     *(reinterpret_cast<h16x8*>(out) + i) = val;
 }
 
@@ -619,6 +855,30 @@ int decode_parts(int cache_len) {
 }
 
 bool fp8_format(int kv_format) { return kv_format == kFmtE4M3 || kv_format == kFmtE5M2; }
+bool tq_format(int kv_format) { return kv_format >= kFmtTq4 && kv_format <= kFmtTq15; }
+bool packed_format(int kv_format) { return fp8_format(kv_format) || tq_format(kv_format); }
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+
+// One kernel instance per packed cache format.
+#define VV_FOR_PACKED_FORMAT(fmt, CALL)                 \
+    switch (fmt) {                                      \
+        case kFmtE4M3: CALL(kFmtE4M3); break;           \
+        case kFmtE5M2: CALL(kFmtE5M2); break;           \
+        case kFmtTq4: CALL(kFmtTq4); break;             \
+        case kFmtTq3: CALL(kFmtTq3); break;             \
+        case kFmtTq2: CALL(kFmtTq2); break;             \
+        default: CALL(kFmtTq15); break;                 \
+    }
+
+// What a packed format needs of a view: head_dim 128, 16-byte aligned Q / O, stores aligned to
+// their unit (8 bytes of FP8 codes per slot, 32-bit words of TurboQuant codes) and, for
+// TurboQuant, the per-vector RMS arrays.
+bool packed_view_ok(const vv_kv_view_t* kv) {
+    if (kv->head_dim != kD) return false;
+    if (fp8_format(kv->format)) return aligned8(kv->k) && aligned8(kv->v);
+    return aligned4(kv->k) && aligned4(kv->v) && kv->k_meta && kv->v_meta;
+}
 
 bool shape_ok(int n_q_heads, int n_kv_heads, int head_dim) {
     return n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0 && head_dim > 0 &&
@@ -632,12 +892,12 @@ extern "C" {
 
 /* One implementation serves every backend name: what differs between fa1,
  * fa2 and flashinfer on the reference's CUDA side is how the card is used,
- * not the result. FP16 caches, and FP8 (E4M3 / E5M2) ones at head_dim 128,
+ * not the result. FP16 caches, and FP8 / TurboQuant ones at head_dim 128,
  * contiguous or paged. */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads, int n_kv_heads,
                     int head_dim) {
     enum { kAuto = 0, kFa1 = 1, kFa2 = 2, kFlashinfer = 3 };
-    const bool served = kv_format == vv::kFormatFp16 || (vv::fp8_format(kv_format) && head_dim == vv::kD);
+    const bool served = kv_format == vv::kFormatFp16 || (vv::packed_format(kv_format) && head_dim == vv::kD);
     if (!served || !vv::shape_ok(n_q_heads, n_kv_heads, head_dim)) return kFa1;
     if (requested == kFlashinfer) return kFlashinfer;
     if (requested == kFa1 && !paged) return kFa1;
@@ -662,12 +922,10 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     if (!q || !kv || !out) return VV_ERR_NULL_PTR;
     if (q_len <= 0 || kv_len <= 0) return VV_OK;
     if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
-    const bool fp8 = vv::fp8_format(kv->format);
-    if (kv->format != vv::kFormatFp16 && !fp8) return VV_ERR_UNSUPPORTED;
+    const bool packed = vv::packed_format(kv->format);
+    if (kv->format != vv::kFormatFp16 && !packed) return VV_ERR_UNSUPPORTED;
     if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
-    if (fp8 && (kv->head_dim != vv::kD || !vv::aligned16(q) || !vv::aligned16(out) ||
-                ((reinterpret_cast<uintptr_t>(kv->k) | reinterpret_cast<uintptr_t>(kv->v)) & 7u)))
-        return VV_ERR_UNSUPPORTED;
+    if (packed && (!vv::packed_view_ok(kv) || !vv::aligned16(q) || !vv::aligned16(out))) return VV_ERR_UNSUPPORTED;
     if (q_offset < 0) return VV_ERR_INVALID_ARG;
     hipStream_t st = vv::as_stream(stream);
     const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
@@ -675,22 +933,21 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     const vv::h16* K = static_cast<const vv::h16*>(kv->k);
     const vv::h16* V = static_cast<const vv::h16*>(kv->v);
     vv::h16* O = static_cast<vv::h16*>(out);
-    if (fp8) {
+    const vv::KvSource src = {kv->k, kv->v, static_cast<const vv::h16*>(kv->k_meta),
+                              static_cast<const vv::h16*>(kv->v_meta), kv->page_table};
+    if (packed) {
         const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
-        if (kv->format == vv::kFmtE4M3)
-            vv::prefill128<vv::kFmtE4M3><<<grid, vv::kBlock, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, n_q_heads,
-                                                                      kv->n_kv_heads, q_len, q_offset, kv_len,
-                                                                      causal ? 1 : 0, scale_log2);
-        else
-            vv::prefill128<vv::kFmtE5M2><<<grid, vv::kBlock, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, n_q_heads,
-                                                                      kv->n_kv_heads, q_len, q_offset, kv_len,
-                                                                      causal ? 1 : 0, scale_log2);
+#define VV_PREFILL(F)                                                                                          \
+    vv::prefill128<vv::F><<<grid, vv::kBlock, 0, st>>>(Q, src, O, n_q_heads, kv->n_kv_heads, q_len, q_offset, \
+                                                       kv_len, causal ? 1 : 0, scale_log2)
+        using namespace vv;
+        VV_FOR_PACKED_FORMAT(kv->format, VV_PREFILL)
+#undef VV_PREFILL
     } else if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
                vv::aligned16(out)) {
         const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
-        vv::prefill128<vv::kFmtFp16><<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
-                                                                  kv->n_kv_heads, q_len, q_offset, kv_len,
-                                                                  causal ? 1 : 0, scale_log2);
+        vv::prefill128<vv::kFmtFp16><<<grid, vv::kBlock, 0, st>>>(Q, src, O, n_q_heads, kv->n_kv_heads, q_len,
+                                                                  q_offset, kv_len, causal ? 1 : 0, scale_log2);
     } else {
         const dim3 grid((unsigned)q_len, (unsigned)n_q_heads);
         vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
@@ -707,36 +964,34 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
     if (!q || !kv || !out) return VV_ERR_NULL_PTR;
     if (cache_len <= 0) return VV_OK;
     if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
-    const bool fp8 = vv::fp8_format(kv->format);
-    if (kv->format != vv::kFormatFp16 && !fp8) return VV_ERR_UNSUPPORTED;
+    const bool packed = vv::packed_format(kv->format);
+    if (kv->format != vv::kFormatFp16 && !packed) return VV_ERR_UNSUPPORTED;
     if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
-    if (fp8 && (kv->head_dim != vv::kD || !vv::aligned16(q) ||
-                ((reinterpret_cast<uintptr_t>(kv->k) | reinterpret_cast<uintptr_t>(kv->v)) & 7u)))
-        return VV_ERR_UNSUPPORTED;
+    if (packed && (!vv::packed_view_ok(kv) || !vv::aligned16(q))) return VV_ERR_UNSUPPORTED;
     hipStream_t st = vv::as_stream(stream);
     const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
     const vv::h16* Q = static_cast<const vv::h16*>(q);
     const vv::h16* K = static_cast<const vv::h16*>(kv->k);
     const vv::h16* V = static_cast<const vv::h16*>(kv->v);
     vv::h16* O = static_cast<vv::h16*>(out);
-    if (fp8 || (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v))) {
+    const vv::KvSource src = {kv->k, kv->v, static_cast<const vv::h16*>(kv->k_meta),
+                              static_cast<const vv::h16*>(kv->v_meta), kv->page_table};
+    if (packed || (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v))) {
         const int n_parts = vv::decode_parts(cache_len);
         if (n_parts > 1 && !scratch) return VV_ERR_NULL_PTR;
         const int group = n_q_heads / kv->n_kv_heads;
         const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads, (unsigned)((group + 31) / 32));
         float* parts = static_cast<float*>(scratch);
-        if (kv->format == vv::kFmtE4M3)
-            vv::decode128<vv::kFmtE4M3><<<grid, vv::kWave, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, parts, n_q_heads,
-                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
-                                                                    scale_log2);
-        else if (kv->format == vv::kFmtE5M2)
-            vv::decode128<vv::kFmtE5M2><<<grid, vv::kWave, 0, st>>>(Q, kv->k, kv->v, kv->page_table, O, parts, n_q_heads,
-                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
-                                                                    scale_log2);
-        else
-            vv::decode128<vv::kFmtFp16><<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, parts, n_q_heads,
-                                                                    kv->n_kv_heads, cache_len, d_cache_len, n_parts,
-                                                                    scale_log2);
+#define VV_DECODE(F)                                                                                       \
+    vv::decode128<vv::F><<<grid, vv::kWave, 0, st>>>(Q, src, O, parts, n_q_heads, kv->n_kv_heads, cache_len, \
+                                                     d_cache_len, n_parts, scale_log2)
+        if (packed) {
+            using namespace vv;
+            VV_FOR_PACKED_FORMAT(kv->format, VV_DECODE)
+        } else {
+            VV_DECODE(kFmtFp16);
+        }
+#undef VV_DECODE
         if (n_parts > 1) {
             if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
             vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kMergeThreads, 0, st>>>(
@@ -790,14 +1045,15 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
                             void* k_meta, void* v_meta, void* k_ref, bool build_ref,
                             int n_kv_heads, int head_dim, int pos, const int* d_pos,
                             int n_positions, int kv_format, const int* page_table, void* stream) {
-    (void)k_meta; (void)v_meta;     // the formats with a per-vector scale are not served
     if (!k_fp16 || !v_fp16 || !k_store || !v_store) return VV_ERR_NULL_PTR;
-    if (kv_format != vv::kFormatFp16 && !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
+    if (kv_format != vv::kFormatFp16 && !vv::packed_format(kv_format)) return VV_ERR_UNSUPPORTED;
     if (n_kv_heads <= 0 || head_dim <= 0 || pos < 0) return VV_ERR_INVALID_ARG;
     if (n_positions <= 0) return VV_OK;
-    if (vv::fp8_format(kv_format)) {
-        if (head_dim != vv::kD || !vv::aligned16(k_fp16) || !vv::aligned16(v_fp16) || (k_ref && !vv::aligned16(k_ref)) ||
-            ((reinterpret_cast<uintptr_t>(k_store) | reinterpret_cast<uintptr_t>(v_store)) & 7u))
+    if (vv::packed_format(kv_format)) {
+        if (head_dim != vv::kD || !vv::aligned16(k_fp16) || !vv::aligned16(v_fp16) || (k_ref && !vv::aligned16(k_ref)))
+            return VV_ERR_UNSUPPORTED;
+        if (vv::fp8_format(kv_format) ? !(vv::aligned8(k_store) && vv::aligned8(v_store))
+                                      : !(vv::aligned4(k_store) && vv::aligned4(v_store)))
             return VV_ERR_UNSUPPORTED;
         hipStream_t st = vv::as_stream(stream);
         if (k_ref && build_ref) {
@@ -813,6 +1069,23 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
         uint8_t* KS = static_cast<uint8_t*>(k_store);
         uint8_t* VS = static_cast<uint8_t*>(v_store);
         const vv::h16* R = static_cast<const vv::h16*>(k_ref);
+        if (vv::tq_format(kv_format)) {
+            constexpr int kPerBlock = vv::kBlock / 32;
+            const dim3 tq_grid((unsigned)((n_positions * n_kv_heads + kPerBlock - 1) / kPerBlock), 2u);
+            vv::h16* KM = static_cast<vv::h16*>(k_meta);
+            vv::h16* VM = static_cast<vv::h16*>(v_meta);
+#define VV_STORE(F)                                                                                            \
+    vv::kv_store_tq<vv::F><<<tq_grid, vv::kBlock, 0, st>>>(K, V, KS, VS, KM, VM, R, n_kv_heads, pos, d_pos,     \
+                                                           n_positions, page_table)
+            switch (kv_format) {
+                case vv::kFmtTq4: VV_STORE(kFmtTq4); break;
+                case vv::kFmtTq3: VV_STORE(kFmtTq3); break;
+                case vv::kFmtTq2: VV_STORE(kFmtTq2); break;
+                default: VV_STORE(kFmtTq15); break;
+            }
+#undef VV_STORE
+            return vv::launch_status();
+        }
         if (kv_format == vv::kFmtE5M2)
             vv::kv_store_fp8<true><<<grid, vv::kBlock, 0, st>>>(K, V, KS, VS, R, n_kv_heads, pos, d_pos, n_positions,
                                                                 page_table);
@@ -842,20 +1115,47 @@ vv_status_t vv_kv_quant_store_dev(const void* k_fp16, const void* v_fp16, void* 
 
 vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* ref, void* out_fp16,
                               int n_kv_heads, int head_dim, int n_pos, int kv_format, void* stream) {
-    (void)meta;
     if (!store || !out_fp16) return VV_ERR_NULL_PTR;
-    if (head_dim != vv::kD || !vv::fp8_format(kv_format) || n_kv_heads <= 0) return VV_ERR_UNSUPPORTED;
-    if ((reinterpret_cast<uintptr_t>(store) & 7u) || !vv::aligned16(out_fp16) || (ref && !vv::aligned16(ref)))
+    if (head_dim != vv::kD || !vv::packed_format(kv_format) || n_kv_heads <= 0) return VV_ERR_UNSUPPORTED;
+    if (vv::tq_format(kv_format) && !meta) return VV_ERR_NULL_PTR;
+    if (!(vv::fp8_format(kv_format) ? vv::aligned8(store) : vv::aligned4(store)) || !vv::aligned16(out_fp16) ||
+        (ref && !vv::aligned16(ref)))
         return VV_ERR_UNSUPPORTED;
     if (n_pos <= 0) return VV_OK;
     const size_t slots = (size_t)n_pos * n_kv_heads * (vv::kD / 8);
     const dim3 grid((unsigned)((slots + vv::kBlock - 1) / vv::kBlock));
     hipStream_t st = vv::as_stream(stream);
+    const vv::h16* M = static_cast<const vv::h16*>(meta);
     const vv::h16* R = static_cast<const vv::h16*>(ref);
     vv::h16* O = static_cast<vv::h16*>(out_fp16);
-    if (kv_format == vv::kFmtE4M3) vv::kv_dequant_fp8<vv::kFmtE4M3><<<grid, vv::kBlock, 0, st>>>(store, R, O, n_kv_heads, slots);
-    else vv::kv_dequant_fp8<vv::kFmtE5M2><<<grid, vv::kBlock, 0, st>>>(store, R, O, n_kv_heads, slots);
+#define VV_DEQUANT(F) vv::kv_dequant<vv::F><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, slots)
+    {
+        using namespace vv;
+        VV_FOR_PACKED_FORMAT(kv_format, VV_DEQUANT)
+    }
+#undef VV_DEQUANT
     return vv::launch_status();
+}
+
+/* In-place randomised Hadamard transform of [rows][n_heads][128] FP16 (Q before attention over
+ * a TurboQuant cache) and its inverse (O after it). */
+static vv_status_t kv_rotate_entry(void* x_fp16, int n_heads, int head_dim, int rows, int inverse, void* stream) {
+    if (!x_fp16) return VV_ERR_NULL_PTR;
+    if (head_dim != vv::kD || !vv::aligned8(x_fp16)) return VV_ERR_UNSUPPORTED;
+    if (n_heads <= 0 || rows <= 0) return VV_OK;
+    const int n = rows * n_heads;
+    constexpr int kPerBlock = vv::kBlock / 32;
+    vv::kv_rotate<<<dim3((unsigned)((n + kPerBlock - 1) / kPerBlock)), vv::kBlock, 0, vv::as_stream(stream)>>>(
+        static_cast<vv::h16*>(x_fp16), n, inverse);
+    return vv::launch_status();
+}
+
+vv_status_t vv_kv_rotate_dev(void* x_fp16, int n_heads, int head_dim, int rows, void* stream) {
+    return kv_rotate_entry(x_fp16, n_heads, head_dim, rows, 0, stream);
+}
+
+vv_status_t vv_kv_unrotate_dev(void* x_fp16, int n_heads, int head_dim, int rows, void* stream) {
+    return kv_rotate_entry(x_fp16, n_heads, head_dim, rows, 1, stream);
 }
 
 vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, const void* v_store,
@@ -864,7 +1164,7 @@ vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, co
                                           const int* d_cache_len, int kv_format, void* scratch, void* stream) {
     if (!q || !k_store || !v_store || !output || !scratch) return VV_ERR_NULL_PTR;
     if (cache_len == 0) return VV_OK;
-    if (head_dim != vv::kD || !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
+    if (head_dim != vv::kD || !vv::packed_format(kv_format)) return VV_ERR_UNSUPPORTED;
     const vv_kv_view_t view = {k_store, v_store, k_meta, v_meta, nullptr, kv_format, n_kv_heads, head_dim};
     return vv_attn_decode(2, q, &view, output, n_q_heads, cache_len, d_cache_len, scratch, stream);
 }
@@ -875,7 +1175,7 @@ vv_status_t vv_gqa_attention_prefill_q_dev(const void* q, const void* k_store, c
                                            int q_offset, int kv_len, bool causal, int kv_format, void* stream) {
     if (!q || !k_store || !v_store || !output) return VV_ERR_NULL_PTR;
     if (q_len == 0 || kv_len == 0) return VV_OK;
-    if (head_dim != vv::kD || !vv::fp8_format(kv_format)) return VV_ERR_UNSUPPORTED;
+    if (head_dim != vv::kD || !vv::packed_format(kv_format)) return VV_ERR_UNSUPPORTED;
     const vv_kv_view_t view = {k_store, v_store, k_meta, v_meta, nullptr, kv_format, n_kv_heads, head_dim};
     return vv_attn_prefill(2, q, &view, output, n_q_heads, q_len, q_offset, kv_len, causal, nullptr, stream);
 }

@@ -10,7 +10,7 @@
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
  * HIP library does not define (NF4, AWQ and INT8 weight-only GEMM and GEMV, the small-M and
- * NN dense forms, the TurboQuant rotations, VAE, BitNet). It builds into its
+ * NN dense forms, VAE, BitNet). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
  * stays exactly what include/vibevoice_hip.h declares.
@@ -39,9 +39,6 @@ VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_
 VV_DECLINE(vv_gemm_fp16_nn_dev)
 void vv_gemm_cleanup() {}
 
-/* the TurboQuant rotations (kv_quant.h:96-101); the FP16 and FP8 caches are implemented, and the
- * quantised-cache entry points decline the TurboQuant formats themselves */
-VV_DECLINE(vv_kv_rotate_dev)      VV_DECLINE(vv_kv_unrotate_dev)
 
 
 /* Conv-VAE speech encoder (device.h:762-870) */

@@ -76,6 +76,8 @@ SIGNATURES = {
     "vv_kv_dequant_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "vv_gqa_attention_decode_q_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
     "vv_gqa_attention_prefill_q_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, C.c_bool, _i, _vp]),
+    "vv_kv_rotate_dev": (_i, [_vp, _i, _i, _i, _vp]),
+    "vv_kv_unrotate_dev": (_i, [_vp, _i, _i, _i, _vp]),
     "vv_kv_store_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_bool, _i, _i, _i, _vp, _i,
                             _i, _vp, _vp]),
     "vv_kv_page_map_dev": (_i, [_vp, _i, _i, _vp, _vp]),
