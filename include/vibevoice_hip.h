@@ -296,9 +296,10 @@ int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
 /* n_q_heads * 256 * (head_dim + 4) floats: the decode slices' partial states.
  * replaces device.h:554 (attention_fi.cu:585-589). */
 size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim);
-/* The number of slices the decode splits `cache_len` positions into: 1, 2,
- * 4 ... 256, doubling as the length passes 64, 128, 256, ... A captured decode
- * step is valid while this stays equal. replaces device.h:562-563. */
+/* The number of slices the decode splits `cache_len` positions into: 16 up to
+ * 1024 positions, then 32, 64, 128, 256, doubling as the length passes 1024,
+ * 2048, 4096, 8192. A captured decode step is valid while this stays equal.
+ * replaces device.h:562-563. */
 int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len);
 /* q_len query rows at absolute positions q_offset.. against the first kv_len
  * positions of the cache; Q, O [q_len][n_q_heads][head_dim] FP16; causal:
@@ -312,7 +313,7 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv,
 /* One query row per head against the whole cache. cache_len sizes the launch;
  * d_cache_len (device int, or NULL) holds the exact length and need only be in
  * the same vv_attn_decode_shape() bucket. scratch: vv_attn_scratch_bytes()
- * of device memory owned by the caller (may be NULL while the shape is 1).
+ * of device memory owned by the caller.
  * replaces device.h:586-589 (attention_fi.cu:634-660). */
 vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv,
                            void* out, int n_q_heads, int cache_len,

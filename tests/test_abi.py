@@ -122,9 +122,12 @@ def test_attention_host_queries():
     assert dev.vv_attn_resolve(FA1, 0, True, 28, 4, 128) != FA1                    # fa1 never pages
     assert dev.vv_attn_scratch_bytes(28, 4, 128) == 28 * 256 * 132 * 4
     shapes = [dev.vv_attn_decode_shape(FA2, 28, 4, n) for n in range(1, 20000, 37)]
-    assert shapes == sorted(shapes) and shapes[0] == 1 and shapes[-1] == 256
-    assert set(shapes) <= {1, 2, 4, 8, 16, 32, 64, 128, 256}
-    assert dev.vv_attn_decode_shape(FA2, 28, 4, 64) == 1 and dev.vv_attn_decode_shape(FA2, 28, 4, 65) == 2
+    assert shapes == sorted(shapes) and shapes[0] == 16 and shapes[-1] == 256
+    assert set(shapes) <= {16, 32, 64, 128, 256}
+    # still over the first 1024 positions, moving at 1025 (what the reference's own test asks of a backend)
+    assert dev.vv_attn_decode_shape(FA2, 28, 4, 1) == dev.vv_attn_decode_shape(FA2, 28, 4, 1024) == 16
+    assert dev.vv_attn_decode_shape(FA2, 28, 4, 1025) == dev.vv_attn_decode_shape(FA2, 28, 4, 2048) == 32
+    assert dev.vv_gqa_decode_shape(1024) != dev.vv_gqa_decode_shape(1025)
 
 
 # ── the declined remainder of the seam ──────────────────────────────────────

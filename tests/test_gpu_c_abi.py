@@ -135,3 +135,37 @@ def test_reference_own_w4a16_test_passes_on_this_backend():
     assert res.returncode == 0, res.stdout[-3000:]
     assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
     assert "all W4A16 checks match the reference" in res.stdout
+
+
+KVQ_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_kv_quant_hip")
+POS_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_decode_position_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(KVQ_EXE),
+                    reason="oracle/_ref/test_kv_quant_hip not built (needs the reference tree)")
+def test_reference_own_kv_quant_test_passes_on_this_backend():
+    """The reference's tests/test_kv_quant.c: a cache shaped like Qwen2's keys
+    stored in both FP8 and all four TurboQuant formats, unpacked, attended to
+    (rotating Q and un-rotating the output where the format asks), and compared
+    with FP16 attention by cosine against the reference's own bars."""
+    res = subprocess.run([KVQ_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "PASSED" in res.stdout and "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert res.stdout.count(" ok") >= 7
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(POS_EXE),
+                    reason="oracle/_ref/test_decode_position_hip not built (needs the reference tree)")
+def test_reference_own_decode_position_test_passes_on_this_backend():
+    """The reference's tests/test_decode_position.c: everything a captured decode
+    step reads from a device int (position add, the row copy, FP16 and
+    TurboQuant decode and store, RoPE) must give the bytes the host value gives,
+    and the decode launch shape must hold across a 1024-position bucket."""
+    res = subprocess.run([POS_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert res.stdout.count("  ok  ") >= 14

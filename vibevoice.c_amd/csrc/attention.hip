@@ -848,8 +848,13 @@ __global__ void page_map(int* table, int first, int n, PageIds ids) {
     if (i < n) table[first + i] = ids.id[i];
 }
 
+// Slices of the decode: one per 64 keys, rounded up to a power of two between 16 and 256. The
+// floor of 16 keeps the launch shape still over the first 1024 positions (a captured decode step
+// is re-made when the shape moves; the reference's shape moves every 1024 positions too, and its
+// own test of the device-side length holds a backend to that, tests/test_decode_position.c:213-218).
+constexpr int kMinParts = 16;
 int decode_parts(int cache_len) {
-    int want = (cache_len + kKeyTile - 1) / kKeyTile, n = 1;
+    int want = (cache_len + kKeyTile - 1) / kKeyTile, n = kMinParts;
     while (n < want && n < kMaxParts) n *= 2;
     return n;
 }
