@@ -362,15 +362,17 @@ vv_status_t vv_kv_quant_store_dev(const void* k_fp16, const void* v_fp16, void* 
                                   bool build_ref, int n_kv_heads, int head_dim, int pos,
                                   const int* d_pos, int n_positions, int kv_format, void* stream);
 /* A packed store [n_pos][n_kv_heads][bytes per vector] back to FP16 in the
- * space it was stored in (rotated for TurboQuant), plus `ref` [n_kv_heads][128]
- * when given. replaces device.h:697-699 (kv_quant.cu:586-603). */
+ * ORIGINAL space: unpacked, for TurboQuant un-rotated, plus `ref`
+ * [n_kv_heads][128] when given, rounded once. For inspection and offload, not
+ * the hot path. replaces device.h:697-699 (kv_quant.cu:311-338, 586-603). */
 vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* ref,
                               void* out_fp16, int n_kv_heads, int head_dim, int n_pos,
                               int kv_format, void* stream);
 /* Attention over a quantised cache given as pointers: vv_attn_decode /
  * vv_attn_prefill with the format in the view. The codes are widened to FP16
  * on their way into the tile, so the result is, bit for bit, that of an FP16
- * cache holding what vv_kv_dequant_dev returns. A TurboQuant cache holds
+ * cache holding the unpacked vectors (FP8: what vv_kv_dequant_dev returns;
+ * TurboQuant: RMS times level, still rotated). A TurboQuant cache holds
  * rotated vectors: rotate Q before and un-rotate the output after.
  * replace device.h:662-675 (kv_quant.cu:605-673). */
 vv_status_t vv_gqa_attention_decode_q_dev(const void* q, const void* k_store, const void* v_store,

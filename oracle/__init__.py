@@ -95,6 +95,7 @@ def _load():
     for name, args in (("vvo_kv_bytes_per_vec", [C.c_int]),
                        ("vvo_kv_rotate", [C.c_void_p, C.c_int, C.c_int]),
                        ("vvo_kv_store_tq", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+                       ("vvo_kv_unpack", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
                        ("vvo_kv_dequant", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p])):
         getattr(lib, name).restype = C.c_int
         getattr(lib, name).argtypes = args
@@ -483,8 +484,22 @@ def kv_store_tq(src16, ref16, fmt: int):
     return store, meta
 
 
+def kv_unpack(store, meta16, fmt: int) -> np.ndarray:
+    """Codes [n_pos, n_kv_heads, bytes] (+ RMS for TurboQuant) -> FP16 bits [n_pos, n_kv_heads, 128] in the space
+    they were stored in (TurboQuant: rotated): the values attention over the cache multiplies with."""
+    store = np.ascontiguousarray(store, np.uint8)
+    n_pos, nkv = store.shape[:2]
+    if meta16 is not None:
+        meta16 = np.ascontiguousarray(meta16, np.uint16)
+    out = np.empty((n_pos, nkv, 128), np.uint16)
+    _check(lib.vvo_kv_unpack(store.ctypes.data, meta16.ctypes.data if meta16 is not None else None, n_pos * nkv, fmt,
+                             out.ctypes.data), "kv_unpack")
+    return out
+
+
 def kv_dequant(store, meta16, ref16, fmt: int) -> np.ndarray:
-    """Codes [n_pos, n_kv_heads, bytes] (+ RMS for TurboQuant) -> FP16 bits [n_pos, n_kv_heads, 128] in the stored space."""
+    """Codes [n_pos, n_kv_heads, bytes] (+ RMS for TurboQuant) -> FP16 bits [n_pos, n_kv_heads, 128] in the original
+    space (TurboQuant: un-rotated), plus the reference key when given."""
     store = np.ascontiguousarray(store, np.uint8)
     n_pos, nkv = store.shape[:2]
     if meta16 is not None:

@@ -763,8 +763,45 @@ int vvo_kv_store_tq(const uint16_t* src16, const uint16_t* ref16, int n_pos, int
     return VVO_OK;
 }
 
-/* Stored vectors back to FP16, in the space they were stored in (rotated for
- * TurboQuant), plus the reference when given (kv_quant.cu: kv_dequant_kernel). */
+/* One stored vector as FP32 in the space it was stored in: an FP8 value, or
+ * RMS times level for TurboQuant (still rotated). */
+static int kv_unpack_one(const uint8_t* src, const uint16_t* meta, int fmt, float val[128]) {
+    if (fmt == 1 || fmt == 2) {
+        for (int d = 0; d < 128; d++) val[d] = fp8_decode_one(src[d], fmt == 2);
+        return VVO_OK;
+    }
+    if (fmt < VVO_KV_TQ4 || fmt > VVO_KV_TQ1_5) return VVO_ERR_INVALID_ARG;
+    if (!meta) return VVO_ERR_NULL_PTR;
+    uint32_t words[17] = {0};
+    memcpy(words, src, (size_t)vvo_kv_bytes_per_vec(fmt));
+    const int nb = tq_lane_bits(fmt);
+    const float sigma = vvo_half_to_float(*meta);
+    for (int L = 0; L < 32; L++) {
+        const int bit = nb * L, sh = bit & 31;
+        const uint32_t lo = words[bit >> 5], hi = words[(bit >> 5) + 1];
+        const uint32_t bits = (sh ? ((lo >> sh) | (hi << (32 - sh))) : lo) & ((1u << nb) - 1u);
+        tq_unpack4(fmt, bits, sigma, val + 4 * L);
+    }
+    return VVO_OK;
+}
+
+/* What attention over a quantised cache multiplies with: the stored vectors as
+ * FP16 in the space they were stored in (TurboQuant: rotated, no reference). */
+int vvo_kv_unpack(const uint8_t* store, const uint16_t* meta16, int n_vectors, int fmt, uint16_t* out16) {
+    if (!store || !out16) return VVO_ERR_NULL_PTR;
+    const int bpv = vvo_kv_bytes_per_vec(fmt);
+    for (size_t vec = 0; vec < (size_t)n_vectors; vec++) {
+        float val[128];
+        const int rc = kv_unpack_one(store + vec * bpv, meta16 ? meta16 + vec : NULL, fmt, val);
+        if (rc != VVO_OK) return rc;
+        for (int d = 0; d < 128; d++) out16[vec * 128 + d] = vvo_float_to_half_rne(val[d]);
+    }
+    return VVO_OK;
+}
+
+/* Stored vectors back to FP16 in the ORIGINAL space (kv_quant.cu:311-338): the
+ * unpacked values, for TurboQuant the inverse rotation, plus the reference when
+ * given; FP32 throughout, one rounding at the end. */
 int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t* ref16, int n_pos,
                    int n_kv_heads, int fmt, uint16_t* out16) {
     if (!store || !out16) return VVO_ERR_NULL_PTR;
@@ -772,27 +809,12 @@ int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t*
     for (int p = 0; p < n_pos; p++)
         for (int h = 0; h < n_kv_heads; h++) {
             const size_t vec = (size_t)p * n_kv_heads + h;
-            const uint8_t* src = store + vec * bpv;
-            float val[128];
-            if (fmt == 1 || fmt == 2) {
-                for (int d = 0; d < 128; d++) val[d] = fp8_decode_one(src[d], fmt == 2);
-            } else if (fmt >= VVO_KV_TQ4 && fmt <= VVO_KV_TQ1_5) {
-                if (!meta16) return VVO_ERR_NULL_PTR;
-                uint32_t words[17] = {0};
-                memcpy(words, src, (size_t)bpv);
-                const int nb = tq_lane_bits(fmt);
-                const float sigma = vvo_half_to_float(meta16[vec]);
-                for (int L = 0; L < 32; L++) {
-                    const int bit = nb * L, sh = bit & 31;
-                    const uint32_t lo = words[bit >> 5], hi = words[(bit >> 5) + 1];
-                    const uint32_t bits = (sh ? ((lo >> sh) | (hi << (32 - sh))) : lo) & ((1u << nb) - 1u);
-                    tq_unpack4(fmt, bits, sigma, val + 4 * L);
-                }
-            } else {
-                return VVO_ERR_INVALID_ARG;
-            }
+            float v[32][4];
+            const int rc = kv_unpack_one(store + vec * bpv, meta16 ? meta16 + vec : NULL, fmt, &v[0][0]);
+            if (rc != VVO_OK) return rc;
+            if (fmt >= VVO_KV_TQ4) rotate128(v, 1);
             for (int d = 0; d < 128; d++) {
-                float x = val[d];
+                float x = v[d / 4][d % 4];
                 if (ref16) x += vvo_half_to_float(ref16[(size_t)h * 128 + d]);
                 out16[vec * 128 + d] = vvo_float_to_half_rne(x);
             }

@@ -194,12 +194,16 @@ int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, in
  *   vvo_kv_rotate   in-place transform (or its inverse) of n_vectors x 128 FP16
  *   vvo_kv_store_tq FP16 [n_pos][n_kv_heads][128] (minus ref16 [n_kv_heads][128]
  *                   when given) -> codes [..][bytes_per_vec] and meta16 [..]
- *   vvo_kv_dequant  any quantised format (FP8 too) back to FP16 in the stored
- *                   space, plus ref16 when given */
+ *   vvo_kv_unpack   any quantised format (FP8 too) as FP16 in the space it was
+ *                   stored in (TurboQuant: rotated): what attention reads
+ *   vvo_kv_dequant  any quantised format back to FP16 in the ORIGINAL space:
+ *                   unpacked, un-rotated (TurboQuant), plus ref16 when given,
+ *                   one rounding (kv_quant.cu:311-338) */
 int vvo_kv_bytes_per_vec(int fmt);
 int vvo_kv_rotate(uint16_t* x16, int n_vectors, int inverse);
 int vvo_kv_store_tq(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads, int fmt,
                     uint8_t* store, uint16_t* meta16);
+int vvo_kv_unpack(const uint8_t* store, const uint16_t* meta16, int n_vectors, int fmt, uint16_t* out16);
 int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t* ref16, int n_pos,
                    int n_kv_heads, int fmt, uint16_t* out16);
 

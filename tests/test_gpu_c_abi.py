@@ -169,3 +169,37 @@ def test_reference_own_decode_position_test_passes_on_this_backend():
     assert res.returncode == 0, res.stdout[-3000:]
     assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
     assert res.stdout.count("  ok  ") >= 14
+
+
+ATTN_BACKENDS_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_attn_backends_hip")
+CONCURRENT_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_concurrent_decode_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(ATTN_BACKENDS_EXE),
+                    reason="oracle/_ref/test_attn_backends_hip not built (needs the reference tree)")
+def test_reference_own_attention_interface_test_passes_on_this_backend():
+    """The reference's tests/test_attn_backends.c: every backend name over slab
+    and paged caches in FP16, FP8 and TurboQuant, prefill and decode at two head
+    layouts, against a CPU attention over the cache as vv_kv_dequant_dev returns
+    it (so that call must hand back original-space vectors), and paged against
+    contiguous on shuffled pages."""
+    res = subprocess.run([ATTN_BACKENDS_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "every backend matches the reference" in res.stdout
+    assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert res.stdout.count("  ok ") >= 300
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(CONCURRENT_EXE),
+                    reason="oracle/_ref/test_concurrent_decode_hip not built (needs the reference tree)")
+def test_reference_own_concurrent_decode_test_passes_on_this_backend():
+    """The reference's tests/test_concurrent_decode.c: four threads, each with
+    its own stream and scratch, decode over slab caches and over pages of one
+    shared pool; every answer must equal the single-threaded one."""
+    res = subprocess.run([CONCURRENT_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "PASS" in res.stdout and "FAIL" not in res.stdout and "SKIP" not in res.stdout

@@ -3,7 +3,8 @@
 Rotation, store (codes and per-vector RMS) and unpack are held to bit equality
 with the oracle, which adds in the accelerator's order. Attention over a
 TurboQuant cache must equal, bit for bit, attention over an FP16 cache holding
-the unpacked (still rotated) vectors; and the whole recipe (rotate Q, attend,
+the unpacked (still rotated) vectors; the dequantiser returns to the original
+space as the reference's does; and the whole recipe (rotate Q, attend,
 un-rotate the output) must track FP16 attention over the original vectors to
 the format's accuracy.
 """
@@ -83,7 +84,7 @@ def test_store_and_unpack_bit_exact(fmt):
     assert np.array_equal(st["ks"].cpu().numpy()[:n], want_k) and np.array_equal(bits_of(st["km"])[:n], want_km)
     assert np.array_equal(st["vs"].cpu().numpy()[:n], want_v) and np.array_equal(bits_of(st["vm"])[:n], want_vm)
     assert (st["ks"].cpu().numpy()[n:] == 0xAA).all() and (bits_of(st["km"])[n:] == bits_of(st["km"])[-1, -1]).all()
-    # unpack: in the rotated space, with and without the reference key
+    # back to FP16 in the original space, with and without the reference key
     d_out = torch.zeros((n, NKV, HD), dtype=torch.float16, device="cuda")
     ok(dev.vv_kv_dequant_dev(st["ks"].data_ptr(), st["km"].data_ptr(), None, d_out.data_ptr(), NKV, HD, n, fmt, stream()))
     assert np.array_equal(bits_of(d_out), oracle.kv_dequant(want_k, want_km, None, fmt))
@@ -119,7 +120,7 @@ def test_decode_equals_fp16_cache_of_unpacked_vectors_and_tracks_fp16_attention(
     ref = oracle.kv_build_ref(k)
     ks, km = oracle.kv_store_tq(k, ref, fmt)
     vs, vm = oracle.kv_store_tq(v, None, fmt)
-    k16, v16 = oracle.kv_dequant(ks, km, None, fmt), oracle.kv_dequant(vs, vm, None, fmt)
+    k16, v16 = oracle.kv_unpack(ks, km, fmt), oracle.kv_unpack(vs, vm, fmt)
     q = oracle.normal_f16((1, nq, HD), 7, std=0.6)
     qr = oracle.kv_rotate(q)
     d_q = to_dev(qr)
@@ -157,7 +158,7 @@ def test_prefill_equals_fp16_cache_of_unpacked_vectors(fmt):
     k, v = qwen_like(kv_len, 11)
     ks, km = oracle.kv_store_tq(k, None, fmt)
     vs, vm = oracle.kv_store_tq(v, None, fmt)
-    k16, v16 = oracle.kv_dequant(ks, km, None, fmt), oracle.kv_dequant(vs, vm, None, fmt)
+    k16, v16 = oracle.kv_unpack(ks, km, fmt), oracle.kv_unpack(vs, vm, fmt)
     d_q = to_dev(oracle.kv_rotate(oracle.normal_f16((q_len, nq, HD), 12, std=0.6)))
     outs = []
     for vw in (view(u8(ks), u8(vs), to_dev(km), to_dev(vm), fmt), view(to_dev(k16), to_dev(v16), None, None, 0)):

@@ -122,14 +122,14 @@ def test_scalar_levels_are_the_lloyd_max_fixed_point(fmt):
         stream |= int(c) << (d * nb)
     store[0, 0] = np.frombuffer(stream.to_bytes(oracle.kv_bytes_per_vec(fmt), "little"), np.uint8)
     one = oracle.narrow(np.ones((1, 1), np.float32))
-    levels = oracle.widen(oracle.kv_dequant(store, one, None, fmt))[0, 0, :n_levels].astype(np.float64)
+    levels = oracle.widen(oracle.kv_unpack(store, one, fmt))[0, 0, :n_levels].astype(np.float64)
     assert np.all(np.diff(levels) > 0) and np.allclose(levels, -levels[::-1], atol=1e-3)
     assert np.max(np.abs(levels - gaussian_cell_means(levels))) < 4e-3        # FP16 read-back of 6-digit tables
 
 
 @pytest.mark.parametrize("fmt", [3, 4, 5, 6])
 def test_codes_are_nearest_and_reach_the_quoted_signal_to_noise(fmt):
-    """On Gaussian vectors: dequant(store(x)) is, per value (per pair for 1.5
+    """On Gaussian vectors: unpack(store(x)) is, per value (per pair for 1.5
     bits), the nearest entry of the scaled table, and the signal-to-noise ratio
     is the one the reference quotes for the format (kv_codec.cuh:40-41)."""
     n = 64
@@ -137,7 +137,7 @@ def test_codes_are_nearest_and_reach_the_quoted_signal_to_noise(fmt):
     store, meta = oracle.kv_store_tq(x, None, fmt)
     assert store.shape[-1] == oracle.kv_bytes_per_vec(fmt)
     y = oracle.widen(oracle.kv_rotate(x)).astype(np.float64)[:, 0]              # what was quantised (to FP16 rounding)
-    got = oracle.widen(oracle.kv_dequant(store, meta, None, fmt)).astype(np.float64)[:, 0]
+    got = oracle.widen(oracle.kv_unpack(store, meta, fmt)).astype(np.float64)[:, 0]
     sigma = oracle.widen(meta).astype(np.float64)[:, 0]
     assert np.allclose(sigma, np.sqrt((y ** 2).mean(1)), rtol=2e-3)
     err = ((got - y) ** 2).sum() / (y ** 2).sum()
@@ -178,3 +178,27 @@ def test_turboquant_reference_key_and_fp8_dequant_agree_with_the_codec():
     for fmt, e5m2 in ((1, False), (2, True)):
         codes = oracle.kv_store_fp8(k, None, e5m2)
         assert np.array_equal(oracle.widen(oracle.kv_dequant(codes, None, None, fmt)), oracle.fp8_decode(codes, e5m2))
+        assert np.array_equal(oracle.kv_dequant(codes, None, None, fmt), oracle.kv_unpack(codes, None, fmt))
+
+
+@pytest.mark.parametrize("fmt", [3, 4, 5, 6])
+def test_dequant_returns_to_the_original_space(fmt):
+    """The seam's dequantiser undoes the rotation and adds the reference key back
+    (kv_quant.cu:325-334): it is the inverse transform of the unpacked vector to
+    FP16 rounding, and, the transform being orthogonal, lands as close to the
+    original vector as the unpacked one is to the rotated one."""
+    k = oracle.normal_f16((33, 4, 128), 21, mean=1.5, std=1.0)
+    ref = oracle.kv_build_ref(k)
+    store, meta = oracle.kv_store_tq(k, ref, fmt)
+    plain = oracle.widen(oracle.kv_dequant(store, meta, None, fmt)).astype(np.float64)
+    by_hand = oracle.widen(oracle.kv_rotate(oracle.kv_unpack(store, meta, fmt), inverse=True)).astype(np.float64)
+    assert np.max(np.abs(plain - by_hand)) < 6e-3                 # one rounding against two
+    with_ref = oracle.widen(oracle.kv_dequant(store, meta, ref, fmt)).astype(np.float64)
+    assert np.max(np.abs(with_ref - (plain + oracle.widen(ref)[None]))) < 6e-3
+    x = oracle.widen(k).astype(np.float64)
+    centred = x - oracle.widen(ref)[None]
+    err_orig = ((with_ref - x) ** 2).sum() / (centred ** 2).sum()
+    y = oracle.widen(oracle.kv_rotate(oracle.narrow(centred.astype(np.float32)))).astype(np.float64)
+    err_rot = ((oracle.widen(oracle.kv_unpack(store, meta, fmt)) - y) ** 2).sum() / (y ** 2).sum()
+    assert abs(-10 * np.log10(err_orig) - TQ[fmt]["snr_db"]) < 0.6
+    assert abs(err_orig - err_rot) < 0.05 * err_rot

@@ -808,28 +808,19 @@ __global__ __launch_bounds__(kBlock) void kv_store_tq(
     if (lane32 == 0 && meta) meta[row_vec] = to_half(sigma);
 }
 
-// Any quantised store back to FP16, in the space it was stored in (rotated for
-// TurboQuant), plus the reference key when given. A thread unpacks eight channels.
+// An FP8 store back to FP16, plus the reference key when given. A thread unpacks eight channels.
 template <int kFmt>
 __global__ __launch_bounds__(kBlock) void kv_dequant(const void* __restrict__ store, const h16* __restrict__ meta,
                                                      const h16* __restrict__ ref, h16* __restrict__ out,
                                                      int n_kv_heads, size_t n_slots) {
-    __shared__ float lev[16];
-    if constexpr (KvFormat<kFmt>::kTq) {
-        if (threadIdx.x < 16) lev[threadIdx.x] = kTqLevels[kFmt - kFmtTq4][threadIdx.x];
-        __syncthreads();
-    }
+    static_assert(!KvFormat<kFmt>::kTq, "TurboQuant stores unpack through kv_dequant_tq");
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n_slots) return;
     // FP32 until the one rounding of the output (an FP8 value is exact in FP16 either way)
     float f[8];
-    if constexpr (KvFormat<kFmt>::kTq) {
-        tq_slot_values<kFmt>(store, meta, lev, i / (kD / 8), (int)(i % (kD / 8)), f);
-    } else {
-        const h16x8 h = __builtin_bit_cast(h16x8, load_slot<kFmt>(store, meta, lev, i / (kD / 8), (int)(i % (kD / 8))));
+    const h16x8 h = __builtin_bit_cast(h16x8, load_slot<kFmt>(store, meta, nullptr, i / (kD / 8), (int)(i % (kD / 8))));
 #pragma unroll
-        for (int c = 0; c < 8; ++c) f[c] = (float)h[c];
-    }
+    for (int c = 0; c < 8; ++c) f[c] = (float)h[c];
     if (ref) {
         const int head = (int)((i / (kD / 8)) % n_kv_heads), slot = (int)(i % (kD / 8));
         const h16x8 r = *(reinterpret_cast<const h16x8*>(ref) + head * (kD / 8) + slot);
@@ -840,6 +831,47 @@ __global__ __launch_bounds__(kBlock) void kv_dequant(const void* __restrict__ st
 #pragma unroll
     for (int c = 0; c < 8; ++c) val[c] = to_half(f[c]);
     *(reinterpret_cast<h16x8*>(out) + i) = val;
+}
+
+// A TurboQuant store back to FP16 in the ORIGINAL space: RMS times level, the
+// inverse rotation, plus the reference key when given, one rounding at the end
+// (kv_quant.cu:311-338). 32 lanes share a vector, four channels each, as in the store.
+template <int kFmt>
+__global__ __launch_bounds__(kBlock) void kv_dequant_tq(const void* __restrict__ store, const h16* __restrict__ meta,
+                                                        const h16* __restrict__ ref, h16* __restrict__ out,
+                                                        int n_kv_heads, size_t n_vectors) {
+    typedef KvFormat<kFmt> F;
+    __shared__ float lev[16];
+    if (threadIdx.x < 16) lev[threadIdx.x] = kTqLevels[kFmt - kFmtTq4][threadIdx.x];
+    __syncthreads();
+    const size_t at = (size_t)blockIdx.x * (kBlock / 32) + threadIdx.x / 32;
+    const size_t vec = at < n_vectors ? at : n_vectors - 1;          // every lane takes part in the exchange
+    const int lane32 = (int)threadIdx.x & 31;
+    constexpr int kLaneBits = F::kSlotBits / 2;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(store) + vec * F::kBytes);
+    const uint32_t bits = stream_bits(words, F::kBytes / 4, lane32 * kLaneBits, kLaneBits);
+    const float sigma = (float)meta[vec];
+    float v[4];
+#pragma unroll
+    for (int c = 0; c < 4 / F::kPerCode; ++c) {
+#pragma clang fp contract(off)       // rounded products: the butterfly's first additions must not fuse with them
+        const uint32_t code = (bits >> (F::kCodeBits * c)) & ((1u << F::kCodeBits) - 1u);
+        if constexpr (F::kPerCode == 1) {
+            v[c] = sigma * lev[code];
+        } else {
+            v[2 * c] = sigma * lev[2 * code];
+            v[2 * c + 1] = sigma * lev[2 * code + 1];
+        }
+    }
+    tq_rotate(v, lane32, true);
+    if (ref) {
+        const h16x4 r = *reinterpret_cast<const h16x4*>(ref + (vec % n_kv_heads) * kD + 4 * lane32);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] += (float)r[c];
+    }
+    if (at < n_vectors)
+        *reinterpret_cast<h16x4*>(out + vec * kD + 4 * lane32) =
+            h16x4{to_half(v[0]), to_half(v[1]), to_half(v[2]), to_half(v[3])};
 }
 
 struct PageIds { int id[32]; };
@@ -1127,18 +1159,24 @@ vv_status_t vv_kv_dequant_dev(const void* store, const void* meta, const void* r
         (ref && !vv::aligned16(ref)))
         return VV_ERR_UNSUPPORTED;
     if (n_pos <= 0) return VV_OK;
-    const size_t slots = (size_t)n_pos * n_kv_heads * (vv::kD / 8);
-    const dim3 grid((unsigned)((slots + vv::kBlock - 1) / vv::kBlock));
     hipStream_t st = vv::as_stream(stream);
     const vv::h16* M = static_cast<const vv::h16*>(meta);
     const vv::h16* R = static_cast<const vv::h16*>(ref);
     vv::h16* O = static_cast<vv::h16*>(out_fp16);
-#define VV_DEQUANT(F) vv::kv_dequant<vv::F><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, slots)
-    {
-        using namespace vv;
-        VV_FOR_PACKED_FORMAT(kv_format, VV_DEQUANT)
+    const size_t vectors = (size_t)n_pos * n_kv_heads, slots = vectors * (vv::kD / 8);
+    if (vv::tq_format(kv_format)) {
+        const dim3 grid((unsigned)((vectors + vv::kBlock / 32 - 1) / (vv::kBlock / 32)));
+        switch (kv_format) {
+            case vv::kFmtTq4: vv::kv_dequant_tq<vv::kFmtTq4><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, vectors); break;
+            case vv::kFmtTq3: vv::kv_dequant_tq<vv::kFmtTq3><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, vectors); break;
+            case vv::kFmtTq2: vv::kv_dequant_tq<vv::kFmtTq2><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, vectors); break;
+            default: vv::kv_dequant_tq<vv::kFmtTq15><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, vectors); break;
+        }
+    } else {
+        const dim3 grid((unsigned)((slots + vv::kBlock - 1) / vv::kBlock));
+        if (kv_format == vv::kFmtE4M3) vv::kv_dequant<vv::kFmtE4M3><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, slots);
+        else vv::kv_dequant<vv::kFmtE5M2><<<grid, vv::kBlock, 0, st>>>(store, M, R, O, n_kv_heads, slots);
     }
-#undef VV_DEQUANT
     return vv::launch_status();
 }
 
