@@ -234,6 +234,64 @@ vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
 vv_status_t vv_w4a16_dequant_dev(const void* packed, const void* sz, void* out_fp16, int N,
                                  int K, int group_size, void* stream);
 
+/* ── The older weight-only formats on FP16 activations ─────────────────── */
+
+/* NF4 (bitsandbytes): codes [N*K/2], the high nibble of a byte the even
+ * element; FP16 absmax per 64 flat elements [N*K/64]; w = book[code] * absmax
+ * rounded once to FP16 wherever a kernel needs the FP16 weight. */
+/* y[N] = W x (+ bias), one row. K % 32 == 0 (the reference asks K % 256 == 0).
+ * The code book is met in FP16 and the block's absmax applied to the FP32
+ * partial sum. replaces device.h:168-170 (nf4_gemv.cu:44-90). */
+vv_status_t vv_nf4_gemv_dev(const void* x, const uint8_t* packed, const void* scales,
+                            const void* bias, void* y, int N, int K, void* stream);
+/* M <= 8 (K % 32 == 0): the one-row kernel over up to eight rows, no scratch.
+ * 9..64 rows: the small-M MFMA kernel where vv_skinny_linear_dev serves the
+ * shape, no scratch. Otherwise the weight is dequantised into temp_weight_fp16
+ * [N][K] (NULL there: VV_ERR_NULL_PTR) and vv_gemm_fp16_dev runs; the last two
+ * give the same bits. block_size must be 64. replaces device.h:174-178
+ * (gemm.cu:468-500). */
+vv_status_t vv_nf4_gemm_dev(const void* input_fp16, const uint8_t* weight_packed,
+                            const void* weight_scales_fp16, void* output_fp16,
+                            void* temp_weight_fp16, int M, int N, int K, int block_size,
+                            void* stream);
+/* n_elements % 8 == 0, block_size 64. replaces device.h:181-183
+ * (dequant_nf4.cu:40-66, 117-147). */
+vv_status_t vv_dequant_nf4_dev(const uint8_t* packed, const void* scales_fp16, void* output_fp16,
+                               int n_elements, int block_size, void* stream);
+
+/* INT4 group-affine in the row-major form (vv_awq_repack): codes [N][K/2], high
+ * nibble = even column; FP16 scales and mins [N][K/G], G in {32, 64, 128, 256};
+ * w = q * scale + min. `packed` and `mins` are typed as the reference types
+ * them; they are byte and FP16 arrays. */
+/* One row; K % 32 == 0. replaces device.h:193-196 (awq_gemv.cu:33-72). */
+vv_status_t vv_awq_gemv_dev(const void* x, const uint32_t* packed, const uint32_t* mins,
+                            const void* scales, const void* bias, void* y, int N, int K,
+                            int group_size, void* stream);
+/* M <= 8 and K % 32 == 0: the one-row kernel; else dequantise into
+ * temp_weight_fp16 + vv_gemm_fp16_dev. replaces device.h:199-202
+ * (awq_gemv.cu:213-238). */
+vv_status_t vv_awq_gemm_dev(const void* input_fp16, const uint32_t* packed, const uint32_t* mins,
+                            const void* scales, void* output_fp16, void* temp_weight_fp16,
+                            int M, int N, int K, int group_size, void* stream);
+/* replaces device.h:205-207 (awq_gemv.cu:125-153). */
+vv_status_t vv_dequant_awq_dev(const uint32_t* packed, const uint32_t* mins, const void* scales,
+                               void* output_fp16, int N, int K, int group_size, void* stream);
+
+/* Per-channel INT8: q [N][K], FP32 scale per row, w = q * scale; K % 16 == 0. */
+/* One row: sum q x in FP32 (the codes as exact FP16 integers), scale and bias
+ * once per output. replaces device.h:216-218 (int8_gemv.cu:72-101). */
+vv_status_t vv_int8_gemv_dev(const void* x, const int8_t* q, const float* scales,
+                             const void* bias, void* y, int N, int K, void* stream);
+/* M <= 8 the one-row kernel, 9..64 the small-M MFMA kernel where it serves (no
+ * scratch), else dequantise + vv_gemm_fp16_dev; the last two give the same
+ * bits. No bias. replaces device.h:223-226 (int8_gemv.cu:194-223). */
+vv_status_t vv_int8_gemm_dev(const void* input_fp16, const int8_t* q, const float* scales,
+                             void* output_fp16, void* temp_weight_fp16, int M, int N, int K,
+                             void* stream);
+/* replaces device.h:229-231 (int8_gemv.cu:139-160, 179-192). */
+vv_status_t vv_dequant_int8_dev(const int8_t* q, const float* scales, void* output_fp16, int N,
+                                int K, void* stream);
+
 /* ── Dense linear layers ───────────────────────────────────────────────── */
 
 /* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32
@@ -249,23 +307,29 @@ vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N
                              int K, float alpha, float beta, void* stream);
 /* One projection of a small-M launch: device.h:453-459. */
 typedef struct vv_skinny_proj {
-    const void* w;        /* FP16 [N][K] */
-    const void* scales;   /* quantised formats only: unused here */
+    const void* w;        /* format 0: FP16 [N][K]; 1: int8 [N][K]; 2: NF4 codes [N][K/2] */
+    const void* scales;   /* 1: FP32 [N]; 2: FP16 absmax [N*K/64]; 0: unused */
     const void* bias;     /* FP16 [N] or NULL */
     void*       y;        /* FP16 [M][N] output */
     int         N;
 } vv_skinny_proj_t;
 /* y_i = alpha * A[M,K] . W_i^T (+ bias_i) for up to three projections of the
- * same A (q/k/v, gate/up) in one launch, M in 9..64, dense FP16 weights
- * (format 0). The result equals vv_gemm_fp16_dev followed by vv_bias_add_dev
- * bit for bit. Other formats, other M, K % 8 != 0, or a projection wide
+ * same A (q/k/v, gate/up) in one launch, M in 9..64; dense FP16 (format 0),
+ * per-channel INT8 (1) or NF4 (2) weights, the quantised ones dequantised in
+ * registers to the bits vv_dequant_int8_dev / vv_dequant_nf4_dev write. The
+ * result equals dequantising, vv_gemm_fp16_dev (or vv_gemm_fp16_tile_dev) and
+ * vv_bias_add_dev bit for bit. Other formats, other M, K % 8 != 0, or a projection wide
  * enough that vv_gemm_fp16_dev would tile it (N >= 12800 above 16 rows):
  * VV_ERR_UNSUPPORTED, nothing launched; the caller runs that path itself
  * (src/inference/decoder.c:375-378, 499-505). replaces device.h:472-475. */
 vv_status_t vv_skinny_linear_dev(const void* A, int format,
                                  const vv_skinny_proj_t* projs, int n_proj,
                                  int M, int K, float alpha, void* stream);
-/* The 128x128 tile alone, whatever M. replaces device.h:432-434. */
+/* The LDS-tiled kernel alone (128x128 tile), whatever M — except for 9..64
+ * rows, where it runs what vv_gemm_fp16_dev runs: the reference holds its
+ * small-M entry point to this one bit for bit (device.h:464-468), and the
+ * weight-streaming kernel that serves those rows here adds K in its own order.
+ * replaces device.h:432-434. */
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M,
                                   int N, int K, float alpha, float beta,
                                   void* stream);

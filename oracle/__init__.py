@@ -92,6 +92,12 @@ def _load():
                        ("vvo_kv_store_fp8", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p])):
         getattr(lib, name).restype = C.c_int
         getattr(lib, name).argtypes = args
+    for name, args in (("vvo_nf4_dequant", [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
+                       ("vvo_awq_dequant", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                            C.c_void_p]),
+                       ("vvo_int8_dequant", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p])):
+        getattr(lib, name).restype = C.c_int
+        getattr(lib, name).argtypes = args
     for name, args in (("vvo_kv_bytes_per_vec", [C.c_int]),
                        ("vvo_kv_rotate", [C.c_void_p, C.c_int, C.c_int]),
                        ("vvo_kv_store_tq", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
@@ -142,6 +148,12 @@ def _load_ref():
         ref.vv_int4g_gemm_cpu.restype = C.c_int
         ref.vv_int4g_gemm_cpu.argtypes = [_f32p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _f32p,
                                           C.c_int, C.c_int, C.c_int, C.c_int]
+    if hasattr(ref, "vv_nf4_gemm_cpu"):
+        ref.vv_nf4_gemm_cpu.restype = C.c_int
+        ref.vv_nf4_gemm_cpu.argtypes = [_f32p, C.c_void_p, C.c_void_p, C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
+    if hasattr(ref, "vv_int8_gemm_cpu"):
+        ref.vv_int8_gemm_cpu.restype = C.c_int
+        ref.vv_int8_gemm_cpu.argtypes = [_f32p, C.c_void_p, C.c_void_p, C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
     if hasattr(ref, "vv_int4g_to_gpu_layout"):
         ref.vv_int4g_to_gpu_layout.restype = C.c_int
         ref.vv_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
@@ -420,6 +432,40 @@ def int4g_dequant_f16(packed, scales16, zeros, G):
     _check(lib.vvo_int4g_dequant_f16(packed.ctypes.data, scales16.ctypes.data, zeros.ctypes.data, N, K, G,
                                      out.ctypes.data), "int4g_dequant_f16")
     return out
+
+
+def nf4_dequant(packed, scales16):
+    """NF4 codes [N, K/2] and FP16 absmax bits per 64 flat elements -> (FP16 bits, FP32 values), both [N, K]."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    scales16 = np.ascontiguousarray(scales16, np.uint16)
+    N, K = packed.shape[0], packed.shape[1] * 2
+    assert scales16.size * 64 == N * K
+    o16, o32 = np.empty((N, K), np.uint16), np.empty((N, K), np.float32)
+    _check(lib.vvo_nf4_dequant(packed.ctypes.data, scales16.ctypes.data, N * K, o16.ctypes.data, o32.ctypes.data),
+           "nf4_dequant")
+    return o16, o32
+
+
+def awq_dequant(packed, scales16, mins16, G: int):
+    """INT4 codes [N, K/2] with FP16 scale and min bits [N, K/G] -> (FP16 bits, FP32 values) of q * scale + min."""
+    packed = np.ascontiguousarray(packed, np.uint8)
+    scales16, mins16 = np.ascontiguousarray(scales16, np.uint16), np.ascontiguousarray(mins16, np.uint16)
+    N, K = packed.shape[0], packed.shape[1] * 2
+    o16, o32 = np.empty((N, K), np.uint16), np.empty((N, K), np.float32)
+    _check(lib.vvo_awq_dequant(packed.ctypes.data, scales16.ctypes.data, mins16.ctypes.data, N, K, G, o16.ctypes.data,
+                               o32.ctypes.data), "awq_dequant")
+    return o16, o32
+
+
+def int8_dequant(q, scales):
+    """int8 codes [N, K] with an FP32 scale per row -> (FP16 bits, FP32 values) of q * scale."""
+    q = np.ascontiguousarray(q, np.int8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    N, K = q.shape
+    o16, o32 = np.empty((N, K), np.uint16), np.empty((N, K), np.float32)
+    _check(lib.vvo_int8_dequant(q.ctypes.data, scales.ctypes.data, N, K, o16.ctypes.data, o32.ctypes.data),
+           "int8_dequant")
+    return o16, o32
 
 
 def fp8_encode(x, e5m2: bool) -> np.ndarray:

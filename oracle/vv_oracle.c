@@ -471,6 +471,62 @@ int vvo_int4g_dequant_f16(const uint8_t* packed, const uint16_t* scales16, const
     return VVO_OK;
 }
 
+/* ── the older weight-only formats on FP16 activations ───────────────────── */
+
+/* bitsandbytes' NF4 code book (dequant_nf4.cu:17-22, cpu_kernels.c:61-66). */
+static const float kNf4[16] = {
+    -1.0f,                 -0.6961928009986877f,  -0.5250730514526367f,  -0.39491748809814453f,
+    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+    0.07958029955625534f,  0.16093020141124725f,  0.24611230194568634f,  0.33791524171829224f,
+    0.44070982933044434f,  0.5626170039176941f,   0.7229568362236023f,   1.0f};
+
+/* dequant_nf4.cu:40-66: element e of the flat weight is code book[nibble] times the
+ * FP16 absmax of its block of 64, the high nibble of a byte being the even element. */
+int vvo_nf4_dequant(const uint8_t* packed, const uint16_t* scales16, size_t n_elements, uint16_t* out16,
+                    float* out32) {
+    if (!packed || !scales16) return VVO_ERR_NULL_PTR;
+    if ((n_elements & 7) != 0) return VVO_ERR_INVALID_ARG;
+    for (size_t e = 0; e < n_elements; e++) {
+        const uint8_t b = packed[e / 2];
+        const float w = kNf4[(e & 1) ? (b & 15) : (b >> 4)] * vvo_half_to_float(scales16[e >> 6]);
+        if (out32) out32[e] = w;
+        if (out16) out16[e] = vvo_float_to_half_rne(w);
+    }
+    return VVO_OK;
+}
+
+/* awq_gemv.cu:125-153: w = q * scale + min per group of G along K, one rounding
+ * in FP32 (q * scale is exact there), then one to FP16. */
+int vvo_awq_dequant(const uint8_t* packed, const uint16_t* scales16, const uint16_t* mins16, int N, int K,
+                    int G, uint16_t* out16, float* out32) {
+    if (!packed || !scales16 || !mins16) return VVO_ERR_NULL_PTR;
+    if (N <= 0 || K <= 0 || G <= 0 || (K % G) != 0 || (K % 8) != 0) return VVO_ERR_INVALID_ARG;
+    const int ng = K / G;
+    for (int n = 0; n < N; n++)
+        for (int k = 0; k < K; k++) {
+            const uint8_t b = packed[(size_t)n * (K / 2) + k / 2];
+            const float q = (float)((k & 1) ? (b & 15) : (b >> 4));
+            const size_t g = (size_t)n * ng + k / G;
+            const float w = fmaf(q, vvo_half_to_float(scales16[g]), vvo_half_to_float(mins16[g]));
+            if (out32) out32[(size_t)n * K + k] = w;
+            if (out16) out16[(size_t)n * K + k] = vvo_float_to_half_rne(w);
+        }
+    return VVO_OK;
+}
+
+/* int8_gemv.cu:139-160: w = q * scale[row], the FP32 product rounded to FP16. */
+int vvo_int8_dequant(const int8_t* q, const float* scales, int N, int K, uint16_t* out16, float* out32) {
+    if (!q || !scales) return VVO_ERR_NULL_PTR;
+    if (N <= 0 || K <= 0) return VVO_ERR_INVALID_ARG;
+    for (int n = 0; n < N; n++)
+        for (int k = 0; k < K; k++) {
+            const float w = (float)q[(size_t)n * K + k] * scales[n];
+            if (out32) out32[(size_t)n * K + k] = w;
+            if (out16) out16[(size_t)n * K + k] = vvo_float_to_half_rne(w);
+        }
+    return VVO_OK;
+}
+
 int vvo_int4g_to_gpu_layout(uint8_t* packed, const uint16_t* scales16, const uint8_t* zeros,
                             int N, int K, int G, uint16_t* out_sz) {
     if (!packed || !scales16 || !zeros || !out_sz) return VVO_ERR_NULL_PTR;
@@ -809,9 +865,10 @@ int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t*
     for (int p = 0; p < n_pos; p++)
         for (int h = 0; h < n_kv_heads; h++) {
             const size_t vec = (size_t)p * n_kv_heads + h;
-            float v[32][4];
-            const int rc = kv_unpack_one(store + vec * bpv, meta16 ? meta16 + vec : NULL, fmt, &v[0][0]);
+            float flat[128], v[32][4];
+            const int rc = kv_unpack_one(store + vec * bpv, meta16 ? meta16 + vec : NULL, fmt, flat);
             if (rc != VVO_OK) return rc;
+            memcpy(v, flat, sizeof(flat));
             if (fmt >= VVO_KV_TQ4) rotate128(v, 1);
             for (int d = 0; d < 128; d++) {
                 float x = v[d / 4][d % 4];

@@ -180,6 +180,19 @@ int vvo_kv_build_ref(const uint16_t* k16, int n_pos, int n_kv_heads, int head_di
 int vvo_kv_store_fp8(const uint16_t* src16, const uint16_t* ref16, int n_pos, int n_kv_heads,
                      int head_dim, int e5m2, uint8_t* store);
 
+/* The older weight-only formats, run on FP16 activations. Each writes the
+ * weight as FP16 bits (what a GEMM multiplies after dequantisation) and/or as
+ * the FP32 value before that rounding (what the one-row kernels multiply):
+ *   vvo_nf4_dequant   dequant_nf4.cu:40-66 — code book[nibble] x FP16 absmax per
+ *                     64 flat elements, high nibble = even element
+ *   vvo_awq_dequant   awq_gemv.cu:125-153 — q x scale + min per group of G
+ *   vvo_int8_dequant  int8_gemv.cu:139-160 — q x FP32 scale of the row */
+int vvo_nf4_dequant(const uint8_t* packed, const uint16_t* scales16, size_t n_elements, uint16_t* out16,
+                    float* out32);
+int vvo_awq_dequant(const uint8_t* packed, const uint16_t* scales16, const uint16_t* mins16, int N, int K,
+                    int G, uint16_t* out16, float* out32);
+int vvo_int8_dequant(const int8_t* q, const float* scales, int N, int K, uint16_t* out16, float* out32);
+
 /* The TurboQuant KV-cache codec (formats 3..6 of include/vibevoice/kv_quant.h:
  * 4, 3, 2 and 1.5 bits per value, plus an FP16 RMS per vector). Like the FP8
  * codec the reference holds it only as accelerator code (src/cuda/kv_codec.cuh:

@@ -203,3 +203,24 @@ def test_reference_own_concurrent_decode_test_passes_on_this_backend():
     print(res.stdout[-3000:], res.stderr[-2000:])
     assert res.returncode == 0, res.stdout[-3000:]
     assert "PASS" in res.stdout and "FAIL" not in res.stdout and "SKIP" not in res.stdout
+
+
+SKINNY_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_skinny_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(SKINNY_EXE),
+                    reason="oracle/_ref/test_skinny_hip not built (needs the reference tree)")
+def test_reference_own_small_m_test_passes_on_this_backend():
+    """The reference's tests/test_skinny.c: dense FP16, per-channel INT8 and NF4
+    linear layers at every row count where a tiling changes between 9 and 64,
+    the small-M entry point against dequantise + vv_gemm_fp16_tile_dev +
+    vv_bias_add_dev byte for byte, the public GEMM entry points likewise, all
+    against its CPU kernels and an FP64 bound; q/k/v and gate/up in one launch
+    against separate launches; the shapes a backend must decline."""
+    res = subprocess.run([SKINNY_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "match the tile path byte for byte" in res.stdout
+    assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
+    assert res.stdout.count("  ok  ") >= 250

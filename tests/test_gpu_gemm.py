@@ -161,7 +161,8 @@ def test_skinny_linear_declines():
     assert skinny(d_a, [w] * 3, [None] * 3, M, 500)[0] == U            # K % 8
     import ctypes as C
     arr = (dev.SkinnyProj * 1)(dev.SkinnyProj(w=w.data_ptr(), scales=None, bias=None, y=w.data_ptr(), N=256))
-    assert dev.vv_skinny_linear_dev(d_a.data_ptr(), 1, C.addressof(arr), 1, M, K, 1.0, stream()) == U   # INT8 weights
+    assert dev.vv_skinny_linear_dev(d_a.data_ptr(), 3, C.addressof(arr), 1, M, K, 1.0, stream()) == U   # no such format
+    assert dev.vv_skinny_linear_dev(d_a.data_ptr(), 1, C.addressof(arr), 1, M, K, 1.0, stream()) == dev.VV_ERR_NULL_PTR  # INT8 without scales
     assert dev.vv_skinny_linear_dev(None, 0, C.addressof(arr), 1, M, K, 1.0, stream()) == dev.VV_ERR_NULL_PTR
     torch.cuda.synchronize()
 

@@ -28,6 +28,7 @@
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
 #include "mfma_dma.hpp"
 #include "row_math.hpp"
+#include "wonly.hpp"
 
 namespace vv {
 namespace {
@@ -244,7 +245,8 @@ constexpr int kSkinnyWaves = 8;
 // given, is added to the rounded FP16 product and rounded again, exactly as a
 // bias-add launch after the GEMM would.
 struct SkinnyProjs {
-    const h16* w[3];
+    const void* w[3];
+    const void* scales[3];      // INT8: FP32 per weight row; NF4: FP16 absmax per 64 elements; FP16: unused
     const h16* bias[3];
     h16* y[3];
     int n[3];
@@ -252,17 +254,22 @@ struct SkinnyProjs {
     int vec[3];
 };
 
-template <int kMT>
+template <int kMT, int kFmt>
 __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
     const h16* __restrict__ A, SkinnyProjs projs, int M, int K, float alpha, float beta) {
     __shared__ f32x4 part[kSkinnyWaves][kMT][kWave];
+    __shared__ float book[16];
+    if constexpr (kFmt == kWoNf4) {
+        if (threadIdx.x < 16) book[threadIdx.x] = kNf4Book[threadIdx.x];
+        __syncthreads();
+    }
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int r16 = lane & 15, ks = lane >> 4;
     const int which = ((int)blockIdx.x >= projs.first[1]) + ((int)blockIdx.x >= projs.first[2]);
-    const h16* __restrict__ B = projs.w[which];
+    const WoSource B = {projs.w[which], projs.scales[which], nullptr, 0};
     const h16* __restrict__ bias = projs.bias[which];
     h16* __restrict__ C = projs.y[which];
     const int N = projs.n[which], vec_store = projs.vec[which];
@@ -271,7 +278,7 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
     const int nlines = (kchunks + 7) / 8;                 // 64 K values = 8 chunks per line
     const u32x4 zero = {0u, 0u, 0u, 0u};
 
-    const u32x4* wrow = reinterpret_cast<const u32x4*>(B + (size_t)min(n0 + r16, N - 1) * K);
+    const size_t wrow = (size_t)min(n0 + r16, N - 1);
     const u32x4* arow[kMT];
 #pragma unroll
     for (int t = 0; t < kMT; ++t)
@@ -287,7 +294,7 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
         for (int u = 0; u < 4; ++u) {                     // (line, step) = (u / 2, u % 2)
             const int c = (line + (u >> 1) * kSkinnyWaves) * 8 + (u & 1) * 4 + ks;
             const bool live = c < kchunks;
-            w[u] = live ? wrow[c] : zero;
+            w[u] = live ? wo_slot<kFmt>(B, book, wrow, K, c) : zero;      // FP16: the 16 bytes as stored
 #pragma unroll
             for (int t = 0; t < kMT; ++t) x[t][u] = live ? arow[t][c] : zero;
         }
@@ -347,14 +354,22 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
 inline bool few_tiles(int N) { return (long)((N + 63) / 64) < 200; }
 inline bool skinny_serves(int M, int N) { return M >= 2 && (M <= 16 || (M <= 64 && few_tiles(N))); }
 
-void launch_skinny(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha,
-                   float beta, hipStream_t st) {
+template <int kFmt>
+void launch_skinny_as(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha,
+                      float beta, hipStream_t st) {
     constexpr int kThreads = kSkinnyWaves * kWave;
     const dim3 grid((unsigned)blocks);
-    if (M <= 16) gemm_skinny<1><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
-    else if (M <= 32) gemm_skinny<2><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
-    else if (M <= 48) gemm_skinny<3><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
-    else gemm_skinny<4><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    if (M <= 16) gemm_skinny<1, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else if (M <= 32) gemm_skinny<2, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else if (M <= 48) gemm_skinny<3, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+    else gemm_skinny<4, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
+}
+
+void launch_skinny(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha,
+                   float beta, hipStream_t st, int format = kWoF16) {
+    if (format == kWoInt8) launch_skinny_as<kWoInt8>(A, projs, blocks, M, K, alpha, beta, st);
+    else if (format == kWoNf4) launch_skinny_as<kWoNf4>(A, projs, blocks, M, K, alpha, beta, st);
+    else launch_skinny_as<kWoF16>(A, projs, blocks, M, K, alpha, beta, st);
 }
 
 __global__ __launch_bounds__(kBlock) void gemm_naive(const h16* A, const h16* B, h16* C, int M,
@@ -492,25 +507,30 @@ vv_status_t vv_gemm_fp16_dev(const void* A, const void* B, void* C, int M, int N
 vv_status_t vv_skinny_linear_dev(const void* A, int format, const vv_skinny_proj_t* projs, int n_proj,
                                  int M, int K, float alpha, void* stream) {
     if (!A || !projs) return VV_ERR_NULL_PTR;
-    if (format != 0 /* VV_SKINNY_F16 */ || n_proj < 1 || n_proj > 3 || M < 9 || M > 64 || K <= 0 ||
-        K % 8 != 0 || !vv::aligned16(A))
+    if ((format != vv::kWoF16 && format != vv::kWoInt8 && format != vv::kWoNf4) || n_proj < 1 || n_proj > 3 ||
+        M < 9 || M > 64 || K <= 0 || K % 8 != 0 || !vv::aligned16(A))
         return VV_ERR_UNSUPPORTED;
     vv::SkinnyProjs p = {};
     int blocks = 0;
     for (int i = 0; i < 3; ++i) {
         p.first[i] = blocks;
         if (i >= n_proj) continue;
-        if (!projs[i].w || !projs[i].y) return VV_ERR_NULL_PTR;
-        if (projs[i].N <= 0 || !vv::skinny_serves(M, projs[i].N) || !vv::aligned16(projs[i].w))
+        if (!projs[i].w || !projs[i].y || (format != vv::kWoF16 && !projs[i].scales)) return VV_ERR_NULL_PTR;
+        // the widest load per weight row: 16 bytes of FP16, 8 of int8, 4 of NF4 codes
+        const uintptr_t at = reinterpret_cast<uintptr_t>(projs[i].w);
+        const bool placed = format == vv::kWoF16 ? (at & 15u) == 0 : format == vv::kWoInt8 ? (at & 7u) == 0 : (at & 3u) == 0;
+        if (projs[i].N <= 0 || !vv::skinny_serves(M, projs[i].N) || !placed ||
+            (format != vv::kWoF16 && (reinterpret_cast<uintptr_t>(projs[i].scales) & (format == vv::kWoInt8 ? 3u : 1u))))
             return VV_ERR_UNSUPPORTED;
-        p.w[i] = static_cast<const vv::h16*>(projs[i].w);
+        p.w[i] = projs[i].w;
+        p.scales[i] = projs[i].scales;
         p.bias[i] = static_cast<const vv::h16*>(projs[i].bias);
         p.y[i] = static_cast<vv::h16*>(projs[i].y);
         p.n[i] = projs[i].N;
         p.vec[i] = (projs[i].N % 4 == 0) && ((reinterpret_cast<uintptr_t>(projs[i].y) & 7u) == 0);
         blocks += (projs[i].N + 15) / 16;
     }
-    vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, alpha, 0.0f, vv::as_stream(stream));
+    vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, alpha, 0.0f, vv::as_stream(stream), format);
     return vv::launch_status();
 }
 
@@ -568,6 +588,9 @@ vv_status_t vv_gemv_swiglu_dev(const void* x, const void* w_gate, const void* w_
 
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M, int N, int K,
                                   float alpha, float beta, void* stream) {
+    // 9..64 rows: whatever vv_gemm_fp16_dev runs there. The small-M entry point is held to this
+    // one bit for bit (device.h:464-468), and the weight-streaming kernel adds K in its own order.
+    if (M >= 9 && M <= 64) return vv::gemm(A, B, C, M, N, K, alpha, beta, stream, vv::forced_tile(), true);
     return vv::gemm(A, B, C, M, N, K, alpha, beta, stream, vv::k128, false);
 }
 

@@ -9,8 +9,7 @@
  * src/metal/metal_stubs.c:1-30, src/device/device_none.c:129-483).
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
- * HIP library does not define (NF4, AWQ and INT8 weight-only GEMM and GEMV, the small-M and
- * NN dense forms, VAE, BitNet). It builds into its
+ * HIP library does not define (the NN dense GEMM, VAE, BitNet). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
  * stays exactly what include/vibevoice_hip.h declares.
@@ -29,11 +28,6 @@
 #define VV_DECLINE(name) int name() { return VV_ERR_UNSUPPORTED; }
 #define VV_ZERO_INT(name) int name() { return 0; }
 #define VV_ZERO_SIZE(name) size_t name() { return 0; }
-
-/* weight-only quantised linear layers other than W4A16 (device.h:168-230) */
-VV_DECLINE(vv_nf4_gemv_dev)      VV_DECLINE(vv_nf4_gemm_dev)      VV_DECLINE(vv_dequant_nf4_dev)
-VV_DECLINE(vv_awq_gemv_dev)      VV_DECLINE(vv_awq_gemm_dev)      VV_DECLINE(vv_dequant_awq_dev)
-VV_DECLINE(vv_int8_gemv_dev)     VV_DECLINE(vv_int8_gemm_dev)     VV_DECLINE(vv_dequant_int8_dev)
 
 /* dense FP16 GEMM: the NN form (device.h:477-479); the NT forms are implemented */
 VV_DECLINE(vv_gemm_fp16_nn_dev)

@@ -90,6 +90,15 @@ SIGNATURES = {
     "vv_w4a16_gather_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "vv_w4a16_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_size_t, _i, _i, _i, _i, _vp]),
     "vv_w4a16_dequant_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_nf4_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "vv_nf4_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "vv_dequant_nf4_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "vv_awq_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_awq_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "vv_dequant_awq_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_int8_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "vv_int8_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_dequant_int8_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "vv_w8a8_linear_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_w4a8_linear_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_i8_linear_multi_dev": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
