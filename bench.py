@@ -334,6 +334,55 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del a, c, dense
         del w4, sz
+    # The older weight-only formats on FP16 activations: one row (decode), 29 rows (a streaming
+    # chunk, the small-M kernel where it serves) and the dequantiser that feeds the FP16 GEMM.
+    out["weight_only"] = {}
+    for fmt in ("int8", "nf4", "int4"):
+        for name, n, k in shapes:
+            if fmt == "int8":
+                wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+                sc = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
+                mn, wbytes = None, n * k + 4.0 * n
+            else:
+                wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
+                per = 64 if fmt == "nf4" else G
+                sc = (torch.rand(n * k // per, device="cuda") * 0.02 + 0.002).half()
+                mn = (-torch.rand(n * k // per, device="cuda") * 0.1).half() if fmt == "int4" else None
+                wbytes = n * k / 2 + (2.0 if fmt == "nf4" else 4.0) * n * k / per
+            dense = torch.empty(n * k, dtype=torch.float16, device="cuda")
+            P = lambda t: t.data_ptr() if t is not None else None
+
+            def run(m, a, c):
+                if fmt == "int8":
+                    return dev.vv_int8_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, st)
+                if fmt == "nf4":
+                    return dev.vv_nf4_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, 64, st)
+                return dev.vv_awq_gemm_dev(P(a), P(wq), P(mn), P(sc), P(c), P(dense), m, n, k, G, st)
+
+            def run_dequant():
+                if fmt == "int8":
+                    return dev.vv_dequant_int8_dev(P(wq), P(sc), P(dense), n, k, st)
+                if fmt == "nf4":
+                    return dev.vv_dequant_nf4_dev(P(wq), P(sc), P(dense), n * k, 64, st)
+                return dev.vv_dequant_awq_dev(P(wq), P(mn), P(sc), P(dense), n, k, G, st)
+
+            d = {"N": n, "K": k}
+            for m in (1, 29):
+                a = torch.randn(m, k, dtype=torch.float16, device="cuda")
+                c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                assert run(m, a, c) == 0
+                sec = timed(lambda: run(m, a, c), 50)
+                d[f"M{m}_us"] = sec * 1e6
+                if m == 1:
+                    d["M1_GBps"] = (wbytes + 2.0 * k + 2.0 * n) / sec / 1e9
+                    d["M1_frac_of_hbm_peak"] = d["M1_GBps"] / HBM_PEAK_GBPS
+                del a, c
+            assert run_dequant() == 0
+            sec = timed(run_dequant, 20)
+            d["dequant_us"] = sec * 1e6
+            d["dequant_GBps"] = (wbytes + 2.0 * n * k) / sec / 1e9
+            out["weight_only"][f"{fmt} {name}"] = d
+            del wq, sc, mn, dense
     q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
     k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
     v_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
@@ -992,6 +1041,9 @@ def main() -> int:
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         for name, d in layer["w4a16_gemv"].items():
             log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        for name, d in layer["weight_only"].items():
+            log(f"  weight-only {name:18s} N={d['N']} K={d['K']}: one row {d['M1_us']:7.2f} us {d['M1_GBps']:7.1f} GB/s, "
+                f"29 rows {d['M29_us']:7.2f} us, dequantise {d['dequant_us']:7.2f} us {d['dequant_GBps']:7.1f} GB/s")
         d = layer["attn_prefill"]
         log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")

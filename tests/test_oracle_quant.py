@@ -264,3 +264,74 @@ def test_int4_dequant_against_closed_form_and_reference_gemm():
         ours = oracle.gemm_f16w(x, w16)
         mag = np.abs(x).astype(np.float64) @ np.abs(oracle.widen(w16)).astype(np.float64).T
         assert np.max(np.abs(out - ours) / mag) < 2e-3
+
+
+# ── the older weight-only formats ───────────────────────────────────────────
+
+def _identity_through(fn, K, N, *weights):
+    """Push the identity through a CPU GEMM of the compiled reference: row m of the
+    output is column m of the weight it multiplies, with nothing added to it."""
+    eye = np.eye(K, dtype=np.float32)
+    out = np.empty((K, N), np.float32)
+    fp = C.POINTER(C.c_float)
+    rc = fn(eye.ctypes.data_as(fp), *weights, None, out.ctypes.data_as(fp), K, N, K)
+    assert rc == 0
+    return out.T
+
+
+def test_weight_only_dequantisers_against_closed_forms():
+    rng = np.random.default_rng(5)
+    N, K = 12, 256
+    # NF4: every code against the published code book, high nibble first, one absmax per 64 flat elements
+    book = np.array([-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+                     -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+                     0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+                     0.7229568362236023, 1.0], np.float32)
+    assert np.all(np.diff(book) > 0) and book[7] == 0.0
+    p = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    s = oracle.narrow(rng.uniform(0.01, 0.3, N * K // 64).astype(np.float32))
+    w16, w32 = oracle.nf4_dequant(p, s)
+    codes = np.stack([p >> 4, p & 15], -1).reshape(N, K)
+    want = book[codes] * np.repeat(oracle.widen(s), 64).reshape(N, K)
+    assert np.array_equal(w32, want.astype(np.float32))
+    assert np.array_equal(w16, want.astype(np.float32).astype(np.float16).view(np.uint16))
+    # INT4 {scale, min}: q * s + m is exact in FP64, one rounding to FP32 and one to FP16
+    G = 64
+    sc = oracle.narrow(rng.uniform(0.01, 0.05, (N, K // G)).astype(np.float32))
+    mn = oracle.narrow(-rng.uniform(0.05, 0.4, (N, K // G)).astype(np.float32))
+    w16, w32 = oracle.awq_dequant(p, sc, mn, G)
+    exact = codes.astype(np.float64) * np.repeat(oracle.widen(sc).astype(np.float64), G, 1) \
+        + np.repeat(oracle.widen(mn).astype(np.float64), G, 1)
+    assert np.array_equal(w32, exact.astype(np.float32))
+    assert np.array_equal(w16, exact.astype(np.float32).astype(np.float16).view(np.uint16))
+    # INT8: the FP32 product, then FP16
+    q = rng.integers(-128, 128, (N, K), dtype=np.int8)
+    s8 = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    w16, w32 = oracle.int8_dequant(q, s8)
+    want = q.astype(np.float32) * s8[:, None]
+    assert np.array_equal(w32, want) and np.array_equal(w16, want.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.skipif(oracle.ref is None or not hasattr(oracle.ref, "vv_nf4_gemm_cpu"),
+                    reason="oracle/_ref not built (needs the reference tree)")
+def test_weight_only_dequantisers_against_the_compiled_reference():
+    """The reference's CPU kernels multiply the FP32 weight: the identity pushed
+    through them must return the oracle's FP32 weights exactly."""
+    rng = np.random.default_rng(6)
+    N, K, G = 24, 256, 64
+    p = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    s = oracle.narrow(rng.uniform(0.01, 0.3, N * K // 64).astype(np.float32))
+    assert np.array_equal(_identity_through(oracle.ref.vv_nf4_gemm_cpu, K, N, p.ctypes.data, s.ctypes.data),
+                          oracle.nf4_dequant(p, s)[1])
+    q = rng.integers(-128, 128, (N, K), dtype=np.int8)
+    s8 = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    assert np.array_equal(_identity_through(oracle.ref.vv_int8_gemm_cpu, K, N, q.ctypes.data, s8.ctypes.data),
+                          oracle.int8_dequant(q, s8)[1])
+    sc = oracle.narrow(rng.uniform(0.01, 0.05, (N, K // G)).astype(np.float32))
+    mn = oracle.narrow(-rng.uniform(0.05, 0.4, (N, K // G)).astype(np.float32))
+    eye = np.eye(K, dtype=np.float32)
+    out = np.empty((K, N), np.float32)
+    fp = C.POINTER(C.c_float)
+    assert oracle.ref.vv_int4g_gemm_cpu(eye.ctypes.data_as(fp), p.ctypes.data, sc.ctypes.data, mn.ctypes.data, None,
+                                        out.ctypes.data_as(fp), K, N, K, G) == 0
+    assert np.array_equal(out.T, oracle.awq_dequant(p, sc, mn, G)[1])
