@@ -292,6 +292,44 @@ vv_status_t vv_int8_gemm_dev(const void* input_fp16, const int8_t* q, const floa
 vv_status_t vv_dequant_int8_dev(const int8_t* q, const float* scales, void* output_fp16, int N,
                                 int K, void* stream);
 
+/* ── BitNet integer layers (include/vibevoice/bitnet.h numerics) ───────── */
+
+/* Per-token int8: s = (float)(127 / max(max|x|, 1e-5)) in double, q = the
+ * integer fma(x, s, 1.5 * 2^23) carries (the product is never rounded on its
+ * own), clamped to [-128, 127]. x FP16 (x_f16 != 0) or FP32 [M][K]; scale [M];
+ * sum [M] = row sums of q, or NULL. Bit-identical to vv_act_quant_i8_cpu.
+ * replaces device.h:898-900 (bitnet.cu:44-93). */
+vv_status_t vv_act_quant_i8_dev(const void* x, int x_f16, int M, int K, int8_t* q,
+                                float* scale, int32_t* sum, void* stream);
+/* Ternary (I2_S codes [N][K/4], K % 128 == 0) x int8: acc = sum_k (c - 1) q
+ * exactly, and y = ((float)acc / x_scale[m]) * w_scale (+ bias[n]), each step
+ * rounded on its own; y FP16 (y_f16) or FP32; acc and y may each be NULL. All
+ * row counts run one MFMA kernel. replaces device.h:916-920 (bitnet.cu:138-178,
+ * 470-497). */
+vv_status_t vv_ternary_gemm_dev(const int8_t* q, const int32_t* xsum, const float* x_scale,
+                                const uint8_t* codes, float w_scale, const float* bias,
+                                int32_t* acc, void* y, int y_f16, int M, int N, int K,
+                                void* stream);
+/* int8 x int8: acc = sum_k w a exactly, and y = (float)acc * (w_scale /
+ * *a_scale) (+ bias[n]) with max |y| folded into *absmax (device float that
+ * must start at 0). Any K; K % 16 != 0 or operands off 16 bytes take a scalar
+ * kernel. replaces device.h:928-931 (bitnet.cu:180-222, 499-530). */
+vv_status_t vv_i8_gemm_dev(const int8_t* a, const float* a_scale, const int8_t* w, float w_scale,
+                           const float* bias, int32_t* acc, float* y, float* absmax, int M,
+                           int N, int K, void* stream);
+/* q = rne(clamp(y * (127 / *absmax), relu ? 0 : -127, 127)); *out_scale = 127 /
+ * *absmax (0 when *absmax is 0). replaces device.h:938-940 (bitnet.cu:369-382). */
+vv_status_t vv_i8s_requant_dev(const float* y, int64_t n, const float* absmax, int relu,
+                               int8_t* q, float* out_scale, void* stream);
+/* Scratch for vv_i8_head_argmax_dev. replaces device.h:943 (bitnet.cu:545-548). */
+size_t vv_i8_head_argmax_scratch_bytes(int V);
+/* logit_n = ((float)(w_n . q) * w_scale[n]) / *scale; the largest wins, ties to
+ * the lowest index. K % 4 == 0. replaces device.h:952-955 (bitnet.cu:384-455,
+ * 549-563). */
+vv_status_t vv_i8_head_argmax_dev(const int8_t* q, const float* scale, const int8_t* w,
+                                  const float* w_scale, int V, int K, int32_t* token,
+                                  float* value, void* scratch, void* stream);
+
 /* ── Dense linear layers ───────────────────────────────────────────────── */
 
 /* C[M,N] = alpha * A[M,K] * B[N,K]^T + beta * C; A, B, C FP16 row-major, FP32

@@ -98,6 +98,17 @@ def _load():
                        ("vvo_int8_dequant", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p])):
         getattr(lib, name).restype = C.c_int
         getattr(lib, name).argtypes = args
+    for name, args in (("vvo_ternary_pack", [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]),
+                       ("vvo_bn_act_quant", [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+                       ("vvo_ternary_linear", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int, C.c_int,
+                                               C.c_int, C.c_void_p, C.c_void_p]),
+                       ("vvo_i8_linear", [C.c_void_p, C.c_float, C.c_void_p, C.c_float, C.c_void_p, C.c_int, C.c_int,
+                                          C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+                       ("vvo_i8s_requant", [C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_void_p, C.c_void_p]),
+                       ("vvo_i8_head_argmax", [C.c_void_p, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                               C.c_void_p, C.c_void_p])):
+        getattr(lib, name).restype = C.c_int
+        getattr(lib, name).argtypes = args
     for name, args in (("vvo_kv_bytes_per_vec", [C.c_int]),
                        ("vvo_kv_rotate", [C.c_void_p, C.c_int, C.c_int]),
                        ("vvo_kv_store_tq", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
@@ -154,6 +165,20 @@ def _load_ref():
     if hasattr(ref, "vv_int8_gemm_cpu"):
         ref.vv_int8_gemm_cpu.restype = C.c_int
         ref.vv_int8_gemm_cpu.argtypes = [_f32p, C.c_void_p, C.c_void_p, C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
+    for name, args in (("vv_ternary_pack", [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]),
+                       ("vv_act_quant_i8_cpu", [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+                       ("vv_ternary_gemm_i32_cpu", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]),
+                       ("vv_ternary_linear_cpu", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
+                                                  C.c_int, C.c_int, C.c_int]),
+                       ("vv_i8_gemm_i32_cpu", [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]),
+                       ("vv_i8_linear_cpu", [C.c_void_p, C.c_float, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.c_int, C.c_int, C.c_int]),
+                       ("vv_i8s_requant_cpu", [C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_void_p, C.c_void_p]),
+                       ("vv_i8_head_argmax_cpu", [C.c_void_p, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                                  C.c_void_p, C.c_void_p])):
+        if hasattr(ref, name):
+            getattr(ref, name).restype = C.c_int
+            getattr(ref, name).argtypes = args
     if hasattr(ref, "vv_int4g_to_gpu_layout"):
         ref.vv_int4g_to_gpu_layout.restype = C.c_int
         ref.vv_int4g_to_gpu_layout.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
@@ -466,6 +491,71 @@ def int8_dequant(q, scales):
     _check(lib.vvo_int8_dequant(q.ctypes.data, scales.ctypes.data, N, K, o16.ctypes.data, o32.ctypes.data),
            "int8_dequant")
     return o16, o32
+
+
+def ternary_pack(t) -> np.ndarray:
+    """Ternary values {-1, 0, 1} [N, K] (K % 128 == 0) -> the I2_S bytes [N, K/4]."""
+    t = np.ascontiguousarray(t, np.int8)
+    N, K = t.shape
+    codes = np.empty((N, K // 4), np.uint8)
+    _check(lib.vvo_ternary_pack(t.ctypes.data, N, K, codes.ctypes.data), "ternary_pack")
+    return codes
+
+
+def bn_act_quant(x):
+    """FP32 rows [M, K] -> (int8 codes [M, K], multiplier [M], row sums of the codes [M])."""
+    x = np.ascontiguousarray(x, np.float32)
+    M, K = x.shape
+    q, s, sm = np.empty((M, K), np.int8), np.empty(M, np.float32), np.empty(M, np.int32)
+    _check(lib.vvo_bn_act_quant(x.ctypes.data, M, K, q.ctypes.data, s.ctypes.data, sm.ctypes.data), "bn_act_quant")
+    return q, s, sm
+
+
+def ternary_linear(q, x_scale, codes, w_scale: float, bias=None):
+    """int8 rows [M, K] against I2_S codes [N, K/4] -> (int32 sums [M, N], FP32 y [M, N])."""
+    q, codes = np.ascontiguousarray(q, np.int8), np.ascontiguousarray(codes, np.uint8)
+    x_scale = np.ascontiguousarray(x_scale, np.float32)
+    M, K = q.shape
+    N = codes.shape[0]
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, np.float32)
+    acc, y = np.empty((M, N), np.int32), np.empty((M, N), np.float32)
+    _check(lib.vvo_ternary_linear(q.ctypes.data, x_scale.ctypes.data, codes.ctypes.data, w_scale,
+                                  bias.ctypes.data if bias is not None else None, M, N, K, acc.ctypes.data,
+                                  y.ctypes.data), "ternary_linear")
+    return acc, y
+
+
+def i8_linear(a, a_scale: float, w, w_scale: float, bias=None):
+    """int8 rows [M, K] against int8 weights [N, K] -> (int32 sums, FP32 y, max |y|)."""
+    a, w = np.ascontiguousarray(a, np.int8), np.ascontiguousarray(w, np.int8)
+    M, K = a.shape
+    N = w.shape[0]
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, np.float32)
+    acc, y, am = np.empty((M, N), np.int32), np.empty((M, N), np.float32), np.zeros(1, np.float32)
+    _check(lib.vvo_i8_linear(a.ctypes.data, a_scale, w.ctypes.data, w_scale, bias.ctypes.data if bias is not None else None,
+                             M, N, K, acc.ctypes.data, y.ctypes.data, am.ctypes.data), "i8_linear")
+    return acc, y, float(am[0])
+
+
+def i8s_requant(y, absmax: float, relu: bool):
+    """FP32 values -> (int8 codes of the same shape, the multiplier 127 / absmax)."""
+    y = np.ascontiguousarray(y, np.float32)
+    q, inv = np.empty(y.shape, np.int8), np.zeros(1, np.float32)
+    _check(lib.vvo_i8s_requant(y.ctypes.data, y.size, absmax, int(relu), q.ctypes.data, inv.ctypes.data), "i8s_requant")
+    return q, float(inv[0])
+
+
+def i8_head_argmax(q, scale: float, w, w_scale):
+    """int8 activation [K] against int8 rows [V, K] with a scale per row -> (token, its logit)."""
+    q, w = np.ascontiguousarray(q, np.int8), np.ascontiguousarray(w, np.int8)
+    w_scale = np.ascontiguousarray(w_scale, np.float32)
+    V, K = w.shape
+    tok, val = np.zeros(1, np.int32), np.zeros(1, np.float32)
+    _check(lib.vvo_i8_head_argmax(q.ctypes.data, scale, w.ctypes.data, w_scale.ctypes.data, V, K, tok.ctypes.data,
+                                  val.ctypes.data), "i8_head_argmax")
+    return int(tok[0]), float(val[0])
 
 
 def fp8_encode(x, e5m2: bool) -> np.ndarray:

@@ -879,6 +879,151 @@ int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t*
     return VVO_OK;
 }
 
+/* ── BitNet: ternary and int8 integer layers (include/vibevoice/bitnet.h) ──── */
+
+/* bitnet.h:13-24, bitnet_cpu.c:222-235: value t in {-1, 0, 1} is stored as code
+ * t + 1; byte j of a 32-byte block holds k = j (bits 7:6), j + 32 (5:4),
+ * j + 64 (3:2), j + 96 (1:0) of the block's 128 columns. */
+int vvo_ternary_pack(const int8_t* t, int64_t N, int64_t K, uint8_t* codes) {
+    if (!t || !codes) return VVO_ERR_NULL_PTR;
+    if (N <= 0 || K <= 0 || (K % 128) != 0) return VVO_ERR_INVALID_ARG;
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t b = 0; b < K / 128; b++)
+            for (int j = 0; j < 32; j++) {
+                uint8_t byte = 0;
+                for (int p = 0; p < 4; p++) {
+                    const int v = t[n * K + b * 128 + 32 * p + j];
+                    if (v < -1 || v > 1) return VVO_ERR_INVALID_ARG;
+                    byte |= (uint8_t)((v + 1) << (6 - 2 * p));
+                }
+                codes[n * (K / 4) + b * 32 + j] = byte;
+            }
+    return VVO_OK;
+}
+
+static int ternary_code(const uint8_t* row, int64_t k) {
+    const int64_t b = k / 128, r = k % 128;
+    return (row[b * 32 + r % 32] >> (6 - 2 * (int)(r / 32))) & 3;
+}
+
+/* bitnet_cpu.c:352-358, 396-441: per row s = (float)(127 / max(amax, 1e-5)) in
+ * double; q = the integer that x * s + 1.5 * 2^23, rounded ONCE as a fused
+ * multiply-add, carries in its mantissa; clamped to [-128, 127]. */
+int vvo_bn_act_quant(const float* x, int M, int K, int8_t* q, float* scale, int32_t* sum) {
+    if (!x || !q || !scale) return VVO_ERR_NULL_PTR;
+    if (M <= 0 || K <= 0) return VVO_ERR_INVALID_ARG;
+    for (int m = 0; m < M; m++) {
+        const float* xr = x + (size_t)m * K;
+        float amax = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const float a = fabsf(xr[k]);
+            if (a > amax) amax = a;
+        }
+        const double dmax = amax > 0.00001 ? (double)amax : 0.00001;
+        const float s = (float)(127.0 / dmax);
+        int32_t acc = 0;
+        for (int k = 0; k < K; k++) {
+            const float v = fmaf(xr[k], s, 12582912.0f);
+            int32_t bits;
+            memcpy(&bits, &v, 4);
+            int i = (bits & 0x007fffff) - 0x00400000;
+            if (i > 127) i = 127;
+            if (i < -128) i = -128;
+            q[(size_t)m * K + k] = (int8_t)i;
+            acc += i;
+        }
+        scale[m] = s;
+        if (sum) sum[m] = acc;
+    }
+    return VVO_OK;
+}
+
+/* bitnet_cpu.c:741-790: acc = sum_k (code - 1) * q, exactly; y = ((float)acc /
+ * x_scale[m]) * w_scale (+ bias[n]), each operation rounded on its own. */
+int vvo_ternary_linear(const int8_t* q, const float* x_scale, const uint8_t* codes, float w_scale,
+                       const float* bias, int M, int N, int K, int32_t* acc_out, float* y) {
+    if (!q || !codes) return VVO_ERR_NULL_PTR;
+    if (y && !x_scale) return VVO_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0 || (K % 128) != 0) return VVO_ERR_INVALID_ARG;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; n++) {
+        const uint8_t* row = codes + (size_t)n * (K / 4);
+        for (int m = 0; m < M; m++) {
+            int32_t acc = 0;
+            for (int k = 0; k < K; k++) acc += (ternary_code(row, k) - 1) * (int32_t)q[(size_t)m * K + k];
+            const size_t o = (size_t)m * N + n;
+            if (acc_out) acc_out[o] = acc;
+            if (y) {
+                float v = (float)acc / x_scale[m];
+                v = v * w_scale;
+                if (bias) v = v + bias[n];
+                y[o] = v;
+            }
+        }
+    }
+    return VVO_OK;
+}
+
+/* bitnet_cpu.c:1048-1131: acc = sum_k w * a; y = (float)acc * (w_scale / a_scale)
+ * (+ bias[n]); absmax = max |y|. */
+int vvo_i8_linear(const int8_t* a, float a_scale, const int8_t* w, float w_scale, const float* bias,
+                  int M, int N, int K, int32_t* acc_out, float* y, float* absmax) {
+    if (!a || !w) return VVO_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0) return VVO_ERR_INVALID_ARG;
+    const float d = y ? w_scale / a_scale : 0.0f;
+    float amax = 0.0f;
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < N; n++) {
+            int32_t acc = 0;
+            for (int k = 0; k < K; k++) acc += (int32_t)w[(size_t)n * K + k] * (int32_t)a[(size_t)m * K + k];
+            const size_t o = (size_t)m * N + n;
+            if (acc_out) acc_out[o] = acc;
+            if (y) {
+                float v = (float)acc * d;
+                if (bias) v = v + bias[n];
+                y[o] = v;
+                if (fabsf(v) > amax) amax = fabsf(v);
+            }
+        }
+    if (absmax) *absmax = amax;
+    return VVO_OK;
+}
+
+/* bitnet_cpu.c:1133-1151: inv = 127 / absmax (0 when absmax is 0);
+ * q = round_half_even(clamp(y * inv, relu ? 0 : -127, 127)). */
+int vvo_i8s_requant(const float* y, int64_t n, float absmax, int relu, int8_t* q, float* out_scale) {
+    if (!y || !q) return VVO_ERR_NULL_PTR;
+    const float inv = absmax != 0.0f ? 127.0f / absmax : 0.0f;
+    const float lo = relu ? 0.0f : -127.0f;
+    for (int64_t i = 0; i < n; i++) {
+        float v = y[i] * inv;
+        v = v < lo ? lo : (v > 127.0f ? 127.0f : v);
+        q[i] = (int8_t)nearbyintf(v);
+    }
+    if (out_scale) *out_scale = inv;
+    return VVO_OK;
+}
+
+/* bitnet_cpu.c:1153-1213: logit_n = ((float)(w_n . q) * w_scale[n]) / scale; the
+ * largest wins, ties to the lowest index. */
+int vvo_i8_head_argmax(const int8_t* q, float scale, const int8_t* w, const float* w_scale, int V, int K,
+                       int32_t* token, float* value) {
+    if (!q || !w || !w_scale || !token) return VVO_ERR_NULL_PTR;
+    if (V <= 0 || K <= 0 || !(scale > 0.0f)) return VVO_ERR_INVALID_ARG;
+    float bv = -FLT_MAX;
+    int32_t bi = 0;
+    for (int n = 0; n < V; n++) {
+        int32_t acc = 0;
+        for (int k = 0; k < K; k++) acc += (int32_t)w[(size_t)n * K + k] * (int32_t)q[k];
+        float v = (float)acc * w_scale[n];
+        v = v / scale;
+        if (n == 0 || v > bv) { bv = v; bi = n; }
+    }
+    *token = bi;
+    if (value) *value = bv;
+    return VVO_OK;
+}
+
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value) {
     if (!logits || !token) return VVO_ERR_NULL_PTR;
     int best = 0;

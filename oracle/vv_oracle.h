@@ -220,6 +220,26 @@ int vvo_kv_unpack(const uint8_t* store, const uint16_t* meta16, int n_vectors, i
 int vvo_kv_dequant(const uint8_t* store, const uint16_t* meta16, const uint16_t* ref16, int n_pos,
                    int n_kv_heads, int fmt, uint16_t* out16);
 
+/* BitNet's integer layers (include/vibevoice/bitnet.h, src/cpu/bitnet_cpu.c),
+ * written the slow way: integer sums exact, every FP32 operation rounded on
+ * its own in the order the reference states.
+ *   vvo_ternary_pack    {-1,0,1} [N][K] -> the I2_S bytes (bitnet_cpu.c:222-235)
+ *   vvo_bn_act_quant    per-token int8 with the fused-multiply-add rounding of
+ *                       ggml's quantiser (bitnet_cpu.c:352-358, 396-441)
+ *   vvo_ternary_linear  acc and y = acc / x_scale * w_scale + bias (:741-790)
+ *   vvo_i8_linear       acc, y = acc * (w_scale / a_scale) + bias, max|y| (:1048-1131)
+ *   vvo_i8s_requant     one-scale requantisation (:1133-1151)
+ *   vvo_i8_head_argmax  int8 tied-head argmax, ties to the lowest index (:1153-1213) */
+int vvo_ternary_pack(const int8_t* t, int64_t N, int64_t K, uint8_t* codes);
+int vvo_bn_act_quant(const float* x, int M, int K, int8_t* q, float* scale, int32_t* sum);
+int vvo_ternary_linear(const int8_t* q, const float* x_scale, const uint8_t* codes, float w_scale,
+                       const float* bias, int M, int N, int K, int32_t* acc_out, float* y);
+int vvo_i8_linear(const int8_t* a, float a_scale, const int8_t* w, float w_scale, const float* bias,
+                  int M, int N, int K, int32_t* acc_out, float* y, float* absmax);
+int vvo_i8s_requant(const float* y, int64_t n, float absmax, int relu, int8_t* q, float* out_scale);
+int vvo_i8_head_argmax(const int8_t* q, float scale, const int8_t* w, const float* w_scale, int V, int K,
+                       int32_t* token, float* value);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

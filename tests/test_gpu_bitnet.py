@@ -1,0 +1,157 @@
+"""GPU parity tests of BitNet's integer layers through the C ABI: everything is
+an exact integer sum followed by a fixed sequence of FP32 operations, so every
+comparison with the oracle is bit for bit (the reference's own bar,
+tests/test_bitnet.c:1-12)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, ok, stream
+
+pytestmark = pytest.mark.gpu
+
+
+def D(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def P(t):
+    return t.data_ptr() if t is not None else None
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def activations(M, K, seed):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((M, K)) * 2.5).astype(np.float32)
+    x.reshape(-1)[::97] *= 30.0
+    if M > 2:
+        x[1] = 0.0                       # the 1e-5 floor
+    return x
+
+
+@pytest.mark.parametrize("M,K", [(1, 128), (5, 1536), (3, 8960), (33, 2048), (2, 250)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_activation_quantiser_bit_exact(M, K, f16):
+    x = activations(M, K, M + K)
+    if f16:
+        x = x.astype(np.float16).astype(np.float32)
+    d_x = D(x.astype(np.float16) if f16 else x)
+    d_q = torch.full((M, K), 99, dtype=torch.int8, device="cuda")
+    d_s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    d_sum = torch.zeros(M, dtype=torch.int32, device="cuda")
+    ok(dev.vv_act_quant_i8_dev(P(d_x), int(f16), M, K, P(d_q), P(d_s), P(d_sum), stream()))
+    q, s, sm = oracle.bn_act_quant(x)
+    assert np.array_equal(host(d_q), q) and np.array_equal(host(d_s), s) and np.array_equal(host(d_sum), sm)
+    ok(dev.vv_act_quant_i8_dev(P(d_x), int(f16), M, K, P(d_q), P(d_s), None, stream()))      # the sums are optional
+    assert np.array_equal(host(d_q), q)
+
+
+@pytest.mark.parametrize("M", [1, 2, 7, 8, 9, 16, 17, 33, 64, 65, 150])
+@pytest.mark.parametrize("N,K", [(40, 128), (1536, 1536), (520, 2048), (256, 8960)])
+def test_ternary_product_bit_exact(M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    t = rng.integers(-1, 2, (N, K)).astype(np.int8)
+    codes = oracle.ternary_pack(t)
+    q, s, sm = oracle.bn_act_quant(activations(M, K, 3 + M))
+    bias = rng.standard_normal(N).astype(np.float32)
+    acc, y = oracle.ternary_linear(q, s, codes, 0.0123, bias)
+    d_q, d_s, d_sum, d_c, d_b = D(q), D(s), D(sm), D(codes), D(bias)
+    d_acc = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    d_y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ok(dev.vv_ternary_gemm_dev(P(d_q), P(d_sum), P(d_s), P(d_c), 0.0123, P(d_b), P(d_acc), P(d_y), 0, M, N, K, stream()))
+    assert np.array_equal(host(d_acc), acc)
+    assert np.array_equal(host(d_y).view(np.uint32), y.view(np.uint32))
+    # FP16 output, no bias, no accumulators
+    _, y0 = oracle.ternary_linear(q, s, codes, 0.0123, None)
+    d_h = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_ternary_gemm_dev(P(d_q), P(d_sum), P(d_s), P(d_c), 0.0123, None, None, P(d_h), 1, M, N, K, stream()))
+    assert np.array_equal(host(d_h).view(np.uint16), y0.astype(np.float16).view(np.uint16))
+    # accumulators only
+    d_acc.fill_(-7)
+    ok(dev.vv_ternary_gemm_dev(P(d_q), P(d_sum), None, P(d_c), 0.0123, None, P(d_acc), None, 0, M, N, K, stream()))
+    assert np.array_equal(host(d_acc), acc)
+
+
+@pytest.mark.parametrize("M", [1, 8, 9, 29, 64, 100])
+@pytest.mark.parametrize("N,K", [(33, 64), (512, 1536), (130, 1000), (64, 37), (257, 4096)])
+def test_int8_product_bit_exact(M, N, K):
+    rng = np.random.default_rng(M + 2 * N + K)
+    a = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    acc, y, am = oracle.i8_linear(a, 7.25, w, 0.004, bias)
+    d_a, d_w, d_b = D(a), D(w), D(bias)
+    d_as = D(np.array([7.25], np.float32))
+    d_acc = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    d_y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    d_am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    ok(dev.vv_i8_gemm_dev(P(d_a), P(d_as), P(d_w), 0.004, P(d_b), P(d_acc), P(d_y), P(d_am), M, N, K, stream()))
+    assert np.array_equal(host(d_acc), acc)
+    assert np.array_equal(host(d_y).view(np.uint32), y.view(np.uint32))
+    assert float(host(d_am)[0]) == am
+    # then the requantisation that follows it in the encoder, reading the folded maximum from device memory
+    for relu in (False, True):
+        want_q, want_inv = oracle.i8s_requant(y, am, relu)
+        d_rq = torch.full((M, N), 99, dtype=torch.int8, device="cuda")
+        d_inv = torch.zeros(1, dtype=torch.float32, device="cuda")
+        ok(dev.vv_i8s_requant_dev(P(d_y), M * N, P(d_am), int(relu), P(d_rq), P(d_inv), stream()))
+        assert np.array_equal(host(d_rq), want_q) and float(host(d_inv)[0]) == want_inv
+    # accumulators only
+    d_acc.fill_(-7)
+    ok(dev.vv_i8_gemm_dev(P(d_a), None, P(d_w), 0.004, None, P(d_acc), None, None, M, N, K, stream()))
+    assert np.array_equal(host(d_acc), acc)
+
+
+def test_requant_of_all_zero_tensor():
+    d_y = torch.zeros(1000, dtype=torch.float32, device="cuda")
+    d_am = torch.zeros(1, dtype=torch.float32, device="cuda")
+    d_q = torch.full((1000,), 5, dtype=torch.int8, device="cuda")
+    d_inv = torch.ones(1, dtype=torch.float32, device="cuda")
+    ok(dev.vv_i8s_requant_dev(P(d_y), 1000, P(d_am), 0, P(d_q), P(d_inv), stream()))
+    assert host(d_q).max() == 0 and host(d_q).min() == 0 and float(host(d_inv)[0]) == 0.0
+
+
+@pytest.mark.parametrize("V,K", [(40, 64), (1000, 1536), (151936, 1536), (777, 100)])
+def test_int8_head_argmax(V, K):
+    rng = np.random.default_rng(V + K)
+    w = rng.integers(-127, 128, (V, K), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.01, V).astype(np.float32)
+    q = rng.integers(-128, 128, K, dtype=np.int8)
+    if V > 100:                                             # a tie: the lowest index must win
+        tok0, _ = oracle.i8_head_argmax(q, 9.5, w, ws)
+        dup = (tok0 + 37) % V
+        w[dup], ws[dup] = w[tok0], ws[tok0]
+    tok, val = oracle.i8_head_argmax(q, 9.5, w, ws)
+    d_q, d_w, d_ws = D(q), D(w), D(ws)
+    d_s = D(np.array([9.5], np.float32))
+    d_tok = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    d_val = torch.zeros(1, dtype=torch.float32, device="cuda")
+    nbytes = dev.vv_i8_head_argmax_scratch_bytes(V)
+    assert nbytes >= 8
+    d_scr = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    ok(dev.vv_i8_head_argmax_dev(P(d_q), P(d_s), P(d_w), P(d_ws), V, K, P(d_tok), P(d_val), P(d_scr), stream()))
+    assert int(host(d_tok)[0]) == tok and float(host(d_val)[0]) == val
+    ok(dev.vv_i8_head_argmax_dev(P(d_q), P(d_s), P(d_w), P(d_ws), V, K, P(d_tok), None, P(d_scr), stream()))
+    assert int(host(d_tok)[0]) == tok
+
+
+def test_argument_checks():
+    p = torch.zeros(4096, dtype=torch.float32, device="cuda").data_ptr()
+    s = stream()
+    N, I = dev.VV_ERR_NULL_PTR, dev.VV_ERR_INVALID_ARG
+    assert dev.vv_act_quant_i8_dev(None, 0, 1, 128, p, p, p, s) == N
+    assert dev.vv_act_quant_i8_dev(p, 0, 0, 128, p, p, p, s) == I
+    assert dev.vv_ternary_gemm_dev(p, None, p, p, 1.0, None, p, None, 0, 1, 8, 128, s) == N
+    assert dev.vv_ternary_gemm_dev(p, p, None, p, 1.0, None, None, p, 0, 1, 8, 128, s) == N      # y without x_scale
+    assert dev.vv_ternary_gemm_dev(p, p, p, p, 1.0, None, p, None, 0, 1, 8, 64, s) == I           # K % 128
+    assert dev.vv_i8_gemm_dev(p, None, p, 1.0, None, None, p, None, 1, 8, 64, s) == N             # y without a_scale
+    assert dev.vv_i8_gemm_dev(p, p, p, 1.0, None, p, None, None, 0, 8, 64, s) == I
+    assert dev.vv_i8s_requant_dev(p, 0, p, 0, p, None, s) == I
+    assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 6, p, None, p, s) == I                        # K % 4
+    assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 64, p, None, None, s) == N
+    assert dev.vv_i8_head_argmax_scratch_bytes(0) == 0

@@ -224,3 +224,20 @@ def test_reference_own_small_m_test_passes_on_this_backend():
     assert "match the tile path byte for byte" in res.stdout
     assert "FAIL" not in res.stdout and "SKIP" not in res.stdout
     assert res.stdout.count("  ok  ") >= 250
+
+
+BITNET_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_bitnet_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(BITNET_EXE),
+                    reason="oracle/_ref/test_bitnet_hip not built (needs the reference tree)")
+def test_reference_own_bitnet_test_passes_on_this_backend():
+    """The reference's tests/test_bitnet.c: its CPU integer kernels on every ISA
+    the host offers against scalar references, then the accelerator's quantiser,
+    ternary and int8 products, requantisation and int8 head against the CPU,
+    all with ==."""
+    res = subprocess.run([BITNET_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:]
+    assert "FAIL" not in res.stdout

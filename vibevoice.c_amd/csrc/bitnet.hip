@@ -1,0 +1,433 @@
+// BitNet's integer layers: ternary (I2_S codes, one FP32 scale per tensor) and
+// int8 weights against per-token int8 activations. Integer sums are exact, so
+// the int32 accumulators equal the CPU's whatever the order they are added in;
+// the FP32 steps after them are taken one rounding at a time, in the order the
+// interface states, so the FP32 bits equal the CPU's too.
+//
+//   bn_act_quant  one workgroup per row: max |x|, s = (float)(127 / max(amax,
+//                 1e-5)) in double, q = the integer that fma(x, s, 1.5 * 2^23)
+//                 carries in its mantissa (the product is never rounded on its
+//                 own), clamped to [-128, 127]; the row sum of q beside it
+//   bn_gemm       sixteen weight rows per workgroup against up to 64 activation
+//                 rows (grid.y walks M), K split over the eight waves, operands
+//                 from global memory straight into v_mfma_i32_16x16x64_i8. A
+//                 32-bit word of I2_S codes IS a lane's operand of one step:
+//                 its four 2-bit planes are the codes of columns j, j + 32,
+//                 j + 64, j + 96 (j = 4 bytes of the 32-byte block), met with
+//                 the four activation words at those columns — the order of
+//                 the 64 columns inside a step is free in integer arithmetic.
+//                 Codes stay 0..2; the row sum of the activations is subtracted
+//                 once at the end: sum (c - 1) q = sum c q - sum q.
+//   bn_naive      int8 x int8 when K is not a multiple of 16 or an operand is
+//                 off 16 bytes: one thread per output
+//   bn_requant    one scale for a whole tensor, read from device memory
+//   bn_head       int8 tied-head argmax in two stages; ties to the lowest index
+#include <float.h>
+
+#include "vv_common.hpp"
+
+namespace vv {
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int wave_sum_int(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// ── activation quantiser ────────────────────────────────────────────────────
+
+template <bool kF16>
+__device__ __forceinline__ float bn_load(const void* x, size_t i) {
+    if constexpr (kF16) return (float)static_cast<const h16*>(x)[i];
+    else return static_cast<const float*>(x)[i];
+}
+
+template <bool kF16>
+__global__ __launch_bounds__(kBlock) void bn_act_quant(const void* __restrict__ x, int K, int8_t* __restrict__ q,
+                                                       float* __restrict__ scale, int32_t* __restrict__ sum) {
+    __shared__ float wave_amax[kWavesPerBlock];
+    __shared__ int wave_total[kWavesPerBlock];
+    __shared__ float row_scale;
+    const size_t base = (size_t)blockIdx.x * K;
+    const int wave = wave_in_block(), lane = lane_id();
+    float amax = 0.0f;
+    for (int k = (int)threadIdx.x; k < K; k += kBlock) amax = fmaxf(amax, fabsf(bn_load<kF16>(x, base + k)));
+    amax = wave_max(amax);
+    if (lane == 0) wave_amax[wave] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float mx = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) mx = fmaxf(mx, wave_amax[w]);
+        const double d = mx > 0.00001 ? (double)mx : 0.00001;
+        row_scale = (float)(127.0 / d);
+    }
+    __syncthreads();
+    const float s = row_scale;
+    int total = 0;
+    for (int k = (int)threadIdx.x; k < K; k += kBlock) {
+        const float t = __builtin_fmaf(bn_load<kF16>(x, base + k), s, 12582912.0f);
+        int v = (__builtin_bit_cast(int, t) & 0x007fffff) - 0x00400000;
+        v = v > 127 ? 127 : (v < -128 ? -128 : v);
+        q[base + k] = (int8_t)v;
+        total += v;
+    }
+    total = wave_sum_int(total);
+    if (lane == 0) wave_total[wave] = total;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) t += wave_total[w];
+        scale[blockIdx.x] = s;
+        if (sum) sum[blockIdx.x] = t;
+    }
+}
+
+// ── the shared epilogue ─────────────────────────────────────────────────────
+
+struct BnOut {
+    const int32_t* xsum;     // ternary: row sums of the activations, subtracted
+    const float* x_scale;    // ternary: per-row multiplier
+    const float* a_scale;    // int8: one multiplier, in device memory
+    float w_scale;
+    const float* bias;
+    int32_t* acc;
+    void* y;
+    float* absmax;           // int8: max |y| folded in (must start at 0)
+    int y_f16, tern;
+    int M, N;
+};
+
+// One output: returns |y| (0 when no y is asked for). Every FP32 operation
+// rounds on its own.
+__device__ __forceinline__ float bn_finish(const BnOut& o, int m, int n, int v) {
+#pragma clang fp contract(off)
+    if (o.tern) v -= o.xsum[m];
+    const size_t at = (size_t)m * o.N + n;
+    if (o.acc) o.acc[at] = v;
+    if (!o.y) return 0.0f;
+    float r;
+    if (o.tern) {
+        r = (float)v / o.x_scale[m];
+        r = r * o.w_scale;
+    } else {
+        const float d = o.w_scale / *o.a_scale;
+        r = (float)v * d;
+    }
+    if (o.bias) r = r + o.bias[n];
+    if (o.y_f16) static_cast<h16*>(o.y)[at] = to_half(r);
+    else static_cast<float*>(o.y)[at] = r;
+    return fabsf(r);
+}
+
+// Non-negative floats order like their bit patterns.
+__device__ __forceinline__ void bn_fold_absmax(float* absmax, float v) {
+    v = wave_max(v);
+    if (lane_id() == 0 && v > 0.0f) atomicMax(reinterpret_cast<int*>(absmax), __builtin_bit_cast(int, v));
+}
+
+// ── the product ─────────────────────────────────────────────────────────────
+
+constexpr int kBnWaves = 8;
+
+template <bool kTern, int kMT>
+__global__ __launch_bounds__(kBnWaves * kWave) void bn_gemm(const int8_t* __restrict__ a, const void* __restrict__ w,
+                                                            BnOut out, int K) {
+    __shared__ i32x4 part[kBnWaves][kMT][kWave];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16, m0 = (int)blockIdx.y * (16 * kMT);
+    const int kchunks = K / 16, nsteps = (kchunks + 3) / 4;       // a step: 64 columns, four lanes' 16 each
+    const size_t wrow = (size_t)min(n0 + r16, out.N - 1);
+    const int8_t* xrow[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) xrow[t] = a + (size_t)min(m0 + 16 * t + r16, out.M - 1) * K;
+    const i32x4 zero = {0, 0, 0, 0};
+    i32x4 acc[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) acc[t] = zero;
+
+    for (int s0 = wave * 2; s0 < nsteps; s0 += kBnWaves * 2) {
+        i32x4 wv[2], xv[kMT][2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int s = s0 + u;
+            if constexpr (kTern) {
+                // step s = half (s & 1) of block s / 2; this lane's word of codes: 4 (s & 1) + ks of the block's eight
+                const bool live = s < nsteps;                       // K % 128 == 0: whole steps only
+                const int word = min(s, nsteps - 1) * 4 + ks;       // (s / 2) * 8 + 4 (s & 1) + ks
+                const uint32_t codes = static_cast<const uint32_t*>(w)[wrow * (size_t)(K / 16) + word];
+                wv[u] = live ? i32x4{(int)((codes >> 6) & 0x03030303u), (int)((codes >> 4) & 0x03030303u),
+                                     (int)((codes >> 2) & 0x03030303u), (int)(codes & 0x03030303u)}
+                             : zero;
+                // the four activation words at columns j, j + 32, j + 64, j + 96 of the block, j = 4 (word % 8)
+                const int first = (word >> 3) * 32 + (word & 7);    // in 32-bit words of the row
+#pragma unroll
+                for (int t = 0; t < kMT; ++t) {
+                    const int* xr = reinterpret_cast<const int*>(xrow[t]) + first;
+                    xv[t][u] = i32x4{xr[0], xr[8], xr[16], xr[24]};
+                }
+            } else {
+                const int c = s * 4 + ks;
+                const bool live = c < kchunks;
+                const int cc = live ? c : 0;
+                wv[u] = live ? __builtin_nontemporal_load(
+                                   reinterpret_cast<const i32x4*>(static_cast<const int8_t*>(w) + wrow * K) + cc)
+                             : zero;
+#pragma unroll
+                for (int t = 0; t < kMT; ++t) xv[t][u] = live ? reinterpret_cast<const i32x4*>(xrow[t])[cc] : zero;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u], xv[t][u], acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    __syncthreads();
+
+    // register r of lane l: column n0 + 4 (l / 16) + r of row m0 + 16 t + l % 16
+    float amax = 0.0f;
+    if (tid < kMT * kWave) {
+        const int t = tid >> 6;
+        i32x4 sum = part[0][t][lane];
+#pragma unroll
+        for (int p = 1; p < kBnWaves; ++p) sum += part[p][t][lane];
+        const int m = m0 + 16 * t + r16, n = n0 + 4 * ks;
+        if (m < out.M) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < out.N) amax = fmaxf(amax, bn_finish(out, m, n + r, sum[r]));
+        }
+    }
+    if (!kTern && out.absmax && out.y && tid < kMT * kWave) bn_fold_absmax(out.absmax, amax);
+}
+
+__global__ __launch_bounds__(kBlock) void bn_naive(const int8_t* __restrict__ a, const int8_t* __restrict__ w, BnOut out,
+                                                   int K) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const bool live = i < (size_t)out.M * out.N;
+    float amax = 0.0f;
+    if (live) {
+        const int m = (int)(i / out.N), n = (int)(i % out.N);
+        const int8_t* ar = a + (size_t)m * K;
+        const int8_t* wr = w + (size_t)n * K;
+        int s = 0;
+        for (int k = 0; k < K; ++k) s += (int)wr[k] * (int)ar[k];
+        amax = bn_finish(out, m, n, s);
+    }
+    if (out.absmax && out.y) bn_fold_absmax(out.absmax, amax);
+}
+
+template <bool kTern>
+void launch_bn_gemm(const int8_t* a, const void* w, const BnOut& out, int K, hipStream_t st) {
+    const int mt = out.M <= 16 ? 1 : out.M <= 32 ? 2 : out.M <= 48 ? 3 : 4;
+    const dim3 grid((unsigned)((out.N + 15) / 16), (unsigned)((out.M + 16 * mt - 1) / (16 * mt)));
+    constexpr int kThreads = kBnWaves * kWave;
+    if (mt == 1) bn_gemm<kTern, 1><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    else if (mt == 2) bn_gemm<kTern, 2><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    else if (mt == 3) bn_gemm<kTern, 3><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    else bn_gemm<kTern, 4><<<grid, kThreads, 0, st>>>(a, w, out, K);
+}
+
+// ── requantisation ──────────────────────────────────────────────────────────
+
+__global__ __launch_bounds__(kBlock) void bn_requant(const float* __restrict__ y, int64_t n,
+                                                     const float* __restrict__ absmax, int relu,
+                                                     int8_t* __restrict__ q, float* __restrict__ out_scale) {
+    const float am = *absmax;
+    const float inv = am != 0.0f ? 127.0f / am : 0.0f;
+    const float lo = relu ? 0.0f : -127.0f;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+        float v = y[i] * inv;
+        v = v < lo ? lo : (v > 127.0f ? 127.0f : v);        // a NaN falls through both, as on the CPU
+        q[i] = (int8_t)(int)__builtin_rintf(v);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0 && out_scale) *out_scale = inv;
+}
+
+// ── int8 head + argmax ──────────────────────────────────────────────────────
+
+constexpr int kHeadRowsPerWave = 8;
+constexpr int kHeadRows = kWavesPerBlock * kHeadRowsPerWave;
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+template <bool kWide>
+__global__ __launch_bounds__(kBlock) void bn_head(const int8_t* __restrict__ q, const float* __restrict__ scale,
+                                                  const int8_t* __restrict__ w, const float* __restrict__ w_scale,
+                                                  int V, int K, float* __restrict__ pv, int* __restrict__ pi) {
+#pragma clang fp contract(off)
+    __shared__ float best_v[kWavesPerBlock];
+    __shared__ int best_i[kWavesPerBlock];
+    const int wave = wave_in_block(), lane = lane_id();
+    const float s = *scale;
+    float bv = -FLT_MAX;
+    int bi = 0x7fffffff;
+    const int r0 = (int)blockIdx.x * kHeadRows + wave * kHeadRowsPerWave;
+    for (int r = 0; r < kHeadRowsPerWave; ++r) {
+        const int n = r0 + r;
+        if (n >= V) break;
+        const int8_t* wr = w + (size_t)n * K;
+        int acc = 0;
+        if constexpr (kWide) {
+            const i32x4* w4 = reinterpret_cast<const i32x4*>(wr);
+            const i32x4* x4 = reinterpret_cast<const i32x4*>(q);
+            for (int i = lane; i < K / 16; i += kWave) {
+                const i32x4 a = __builtin_nontemporal_load(w4 + i), b = x4[i];
+                acc = __builtin_amdgcn_sdot4(a.x, b.x, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.z, b.z, acc, false);
+                acc = __builtin_amdgcn_sdot4(a.w, b.w, acc, false);
+            }
+        } else {
+            const int* w1 = reinterpret_cast<const int*>(wr);
+            const int* x1 = reinterpret_cast<const int*>(q);
+            for (int i = lane; i < K / 4; i += kWave) acc = __builtin_amdgcn_sdot4(w1[i], x1[i], acc, false);
+        }
+        acc = wave_sum_int(acc);
+        float v = (float)acc * w_scale[n];
+        v = v / s;
+        if (better(v, n, bv, bi)) { bv = v; bi = n; }
+    }
+    if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float v = best_v[0];
+        int i = best_i[0];
+#pragma unroll
+        for (int k = 1; k < kWavesPerBlock; ++k)
+            if (better(best_v[k], best_i[k], v, i)) { v = best_v[k]; i = best_i[k]; }
+        pv[blockIdx.x] = v;
+        pi[blockIdx.x] = i;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bn_head_final(const float* __restrict__ pv, const int* __restrict__ pi, int n,
+                                                        int32_t* __restrict__ token, float* __restrict__ value) {
+    __shared__ float sv[kBlock];
+    __shared__ int si[kBlock];
+    float bv = -FLT_MAX;
+    int bi = 0x7fffffff;
+    for (int i = (int)threadIdx.x; i < n; i += kBlock)
+        if (better(pv[i], pi[i], bv, bi)) { bv = pv[i]; bi = pi[i]; }
+    sv[threadIdx.x] = bv;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int st = kBlock / 2; st > 0; st >>= 1) {
+        if ((int)threadIdx.x < st && better(sv[threadIdx.x + st], si[threadIdx.x + st], sv[threadIdx.x], si[threadIdx.x])) {
+            sv[threadIdx.x] = sv[threadIdx.x + st];
+            si[threadIdx.x] = si[threadIdx.x + st];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        *token = si[0];
+        if (value) *value = sv[0];
+    }
+}
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_act_quant_i8_dev(const void* x, int x_f16, int M, int K, int8_t* q, float* scale, int32_t* sum,
+                                void* stream) {
+    if (!x || !q || !scale) return VV_ERR_NULL_PTR;
+    if (M <= 0 || K <= 0) return VV_ERR_INVALID_ARG;
+    hipStream_t st = vv::as_stream(stream);
+    if (x_f16) vv::bn_act_quant<true><<<dim3((unsigned)M), vv::kBlock, 0, st>>>(x, K, q, scale, sum);
+    else vv::bn_act_quant<false><<<dim3((unsigned)M), vv::kBlock, 0, st>>>(x, K, q, scale, sum);
+    return vv::launch_status();
+}
+
+vv_status_t vv_ternary_gemm_dev(const int8_t* q, const int32_t* xsum, const float* x_scale, const uint8_t* codes,
+                                float w_scale, const float* bias, int32_t* acc, void* y, int y_f16, int M, int N,
+                                int K, void* stream) {
+    if (!q || !xsum || !codes) return VV_ERR_NULL_PTR;
+    if (y && !x_scale) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0 || K % 128) return VV_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(q) & 3u) || (reinterpret_cast<uintptr_t>(codes) & 3u)) return VV_ERR_UNSUPPORTED;
+    vv::BnOut out = {};
+    out.xsum = xsum;
+    out.x_scale = x_scale;
+    out.w_scale = w_scale;
+    out.bias = bias;
+    out.acc = acc;
+    out.y = y;
+    out.y_f16 = y_f16;
+    out.tern = 1;
+    out.M = M;
+    out.N = N;
+    vv::launch_bn_gemm<true>(q, codes, out, K, vv::as_stream(stream));
+    return vv::launch_status();
+}
+
+vv_status_t vv_i8_gemm_dev(const int8_t* a, const float* a_scale, const int8_t* w, float w_scale, const float* bias,
+                           int32_t* acc, float* y, float* absmax, int M, int N, int K, void* stream) {
+    if (!a || !w) return VV_ERR_NULL_PTR;
+    if (y && !a_scale) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0) return VV_ERR_INVALID_ARG;
+    vv::BnOut out = {};
+    out.a_scale = a_scale;
+    out.w_scale = w_scale;
+    out.bias = bias;
+    out.acc = acc;
+    out.y = y;
+    out.absmax = y ? absmax : nullptr;
+    out.M = M;
+    out.N = N;
+    hipStream_t st = vv::as_stream(stream);
+    if (K % 16 == 0 && vv::aligned16(a) && vv::aligned16(w)) {
+        vv::launch_bn_gemm<false>(a, w, out, K, st);
+    } else {
+        const size_t blocks = ((size_t)M * N + vv::kBlock - 1) / vv::kBlock;
+        if (blocks > 0x7FFFFFFFu) return VV_ERR_UNSUPPORTED;
+        vv::bn_naive<<<dim3((unsigned)blocks), vv::kBlock, 0, st>>>(a, w, out, K);
+    }
+    return vv::launch_status();
+}
+
+vv_status_t vv_i8s_requant_dev(const float* y, int64_t n, const float* absmax, int relu, int8_t* q, float* out_scale,
+                               void* stream) {
+    if (!y || !absmax || !q) return VV_ERR_NULL_PTR;
+    if (n <= 0) return VV_ERR_INVALID_ARG;
+    int64_t blocks = (n + vv::kBlock - 1) / vv::kBlock;
+    if (blocks > 8192) blocks = 8192;
+    vv::bn_requant<<<dim3((unsigned)blocks), vv::kBlock, 0, vv::as_stream(stream)>>>(y, n, absmax, relu, q, out_scale);
+    return vv::launch_status();
+}
+
+size_t vv_i8_head_argmax_scratch_bytes(int V) {
+    if (V <= 0) return 0;
+    const size_t nb = ((size_t)V + vv::kHeadRows - 1) / vv::kHeadRows;
+    return nb * (sizeof(float) + sizeof(int));
+}
+
+vv_status_t vv_i8_head_argmax_dev(const int8_t* q, const float* scale, const int8_t* w, const float* w_scale, int V,
+                                  int K, int32_t* token, float* value, void* scratch, void* stream) {
+    if (!q || !scale || !w || !w_scale || !token || !scratch) return VV_ERR_NULL_PTR;
+    if (V <= 0 || K <= 0 || K % 4) return VV_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(q) & 3u) || (reinterpret_cast<uintptr_t>(w) & 3u) ||
+        (reinterpret_cast<uintptr_t>(scratch) & 3u))
+        return VV_ERR_UNSUPPORTED;
+    const int nb = (V + vv::kHeadRows - 1) / vv::kHeadRows;
+    float* pv = static_cast<float*>(scratch);
+    int* pi = reinterpret_cast<int*>(pv + nb);
+    hipStream_t st = vv::as_stream(stream);
+    if (K % 16 == 0 && vv::aligned16(q) && vv::aligned16(w))
+        vv::bn_head<true><<<dim3((unsigned)nb), vv::kBlock, 0, st>>>(q, scale, w, w_scale, V, K, pv, pi);
+    else
+        vv::bn_head<false><<<dim3((unsigned)nb), vv::kBlock, 0, st>>>(q, scale, w, w_scale, V, K, pv, pi);
+    vv::bn_head_final<<<dim3(1), vv::kBlock, 0, st>>>(pv, pi, nb, token, value);
+    return vv::launch_status();
+}
+
+}  // extern "C"

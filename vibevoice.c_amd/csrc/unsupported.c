@@ -9,7 +9,7 @@
  * src/metal/metal_stubs.c:1-30, src/device/device_none.c:129-483).
  *
  * This file is that remainder for libvibevoice_hip: every device.h symbol the
- * HIP library does not define (the NN dense GEMM, VAE, BitNet). It builds into its
+ * HIP library does not define (the NN dense GEMM and the Conv-VAE kernels). It builds into its
  * own small library, libvibevoice_hip_unsupported.so, which a full engine link
  * adds next to libvibevoice_hip.so; the layer-op library's own export list
  * stays exactly what include/vibevoice_hip.h declares.
@@ -39,8 +39,3 @@ void vv_gemm_cleanup() {}
 VV_DECLINE(vv_vae_conv_dev)      VV_DECLINE(vv_vae_tail_dev)      VV_DECLINE(vv_vae_rms_dev)
 VV_DECLINE(vv_vae_mixer_dev)     VV_DECLINE(vv_vae_im2col_dev)    VV_DECLINE(vv_vae_conv_gemm_dev)
 VV_DECLINE(vv_vae_gemm_nn_dev)   VV_DECLINE(vv_vae_gemm_tn_dev)   VV_DECLINE(vv_vae_f32_to_f16_dev)
-
-/* BitNet (device.h:888-942) */
-VV_DECLINE(vv_act_quant_i8_dev)  VV_DECLINE(vv_ternary_gemm_dev)  VV_DECLINE(vv_i8_gemm_dev)
-VV_DECLINE(vv_i8s_requant_dev)
-VV_ZERO_SIZE(vv_i8_head_argmax_scratch_bytes) VV_DECLINE(vv_i8_head_argmax_dev)

@@ -99,6 +99,12 @@ SIGNATURES = {
     "vv_int8_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "vv_int8_gemm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "vv_dequant_int8_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "vv_act_quant_i8_dev": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "vv_ternary_gemm_dev": (_i, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "vv_i8_gemm_dev": (_i, [_vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "vv_i8s_requant_dev": (_i, [_vp, C.c_int64, _vp, _i, _vp, _vp, _vp]),
+    "vv_i8_head_argmax_scratch_bytes": (C.c_size_t, [_i]),
+    "vv_i8_head_argmax_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "vv_w8a8_linear_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_w4a8_linear_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_i8_linear_multi_dev": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
