@@ -292,6 +292,117 @@ vv_status_t vv_int8_gemm_dev(const void* input_fp16, const int8_t* q, const floa
 vv_status_t vv_dequant_int8_dev(const int8_t* q, const float* scales, void* output_fp16, int N,
                                 int K, void* stream);
 
+/* ── Batched, streaming Conv-VAE encoder ops ────────────────────────────── */
+
+/* Activations are FP16, channel-first and packed along time: the items of one
+ * launch sit side by side in one [C][ld] buffer. Only convolutions look back
+ * in time; they take the item boundaries and each item's streaming context
+ * from a descriptor passed by value. No result depends on where an item sits
+ * in the packed axis or on how a stream was cut into chunks: every output adds
+ * its products in one fixed order. device.h:722-755. */
+#define VV_VAE_MAX_ITEMS 32
+typedef struct vv_vae_conv_item {
+    int64_t     in_off;    /* first input column in the packed input */
+    int64_t     out_off;   /* first output column in the packed output */
+    const void* in_ptr;    /* the item's own input, overriding in_off */
+    const void* tail_in;   /* [in_ch][cap] left context; NULL = zeros */
+    void*       tail_out;  /* [in_ch][cap] receives the next context */
+    void*       out_ptr;   /* transposed output: rows [frame][out_ld] */
+    int         in_len;    /* input columns this chunk */
+    int         out_len;   /* output columns this chunk */
+    int         have;      /* context columns in front of the input */
+    int         keep;      /* context columns to leave for the next chunk */
+    int         out_ld;    /* transposed output row stride, elements */
+    int         skip;      /* leading output frames not written */
+} vv_vae_conv_item_t;
+typedef struct vv_vae_conv_desc {
+    int                n;
+    int                cap;   /* context stride per channel, columns */
+    vv_vae_conv_item_t it[VV_VAE_MAX_ITEMS];
+} vv_vae_conv_desc_t;
+
+/* Causal conv (groups = 1) over every item: y[oc][t] = sum over (in channel,
+ * tap) in that order of w[oc][ic][kk] * in[ic][t * stride + kk], an FP32 fused
+ * multiply-add chain from zero, plus the bias, rounded once to FP16. Position p
+ * of an item's input is column p of [context ++ input]; past the end is zero.
+ * `transposed`: rows [frame][out_ch] at each item's out_ptr instead of packed.
+ * replaces device.h:762-765 (vae_kernels.cu:50-89, 736-755). */
+vv_status_t vv_vae_conv_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in,
+                            const void* w, const void* b, void* y, int64_t ld_out,
+                            int in_ch, int out_ch, int k, int stride, bool transposed,
+                            void* stream);
+/* The last `keep` columns of [context ++ input] of every item into its
+ * tail_out. replaces device.h:768-769 (vae_kernels.cu:95-116, 756-765). */
+vv_status_t vv_vae_tail_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in,
+                            int in_ch, void* stream);
+/* 1 / rms over the channels of every packed column into rinv[0..T), and of
+ * every context column of the items in d (may be NULL) into
+ * rinv[T + item * cap + j]. replaces device.h:775-777 (vae_kernels.cu:286-318,
+ * 766-781). */
+vv_status_t vv_vae_rms_dev(const void* x, int64_t ld, int64_t T, int C, float eps, float* rinv,
+                           const vv_vae_conv_desc_t* d, void* stream);
+/* xout = xin + gamma * (depthwise conv(rmsnorm(xin)) + bias), with an FP16
+ * rounding wherever separate kernels would have stored one. k <= 16.
+ * replaces device.h:783-787 (vae_kernels.cu:320-392, 782-800). */
+vv_status_t vv_vae_mixer_dev(const vv_vae_conv_desc_t* d, const void* xin, void* xout,
+                             int64_t ld, const float* rinv, int64_t T_total,
+                             const void* norm_w, const void* conv_w, const void* conv_b,
+                             const void* gamma, int C, int k, void* stream);
+#define VV_VAE_EPI_BIAS_GELU  0  /* C = gelu(half(half(A B) + bias)) */
+#define VV_VAE_EPI_BIAS_RESID 1  /* C = half(C + half(half(A B) + bias) * gamma), in place */
+#define VV_VAE_EPI_BIAS       2  /* C = half(A B + bias), one rounding */
+/* col[ic * k + kk][q] = what tap kk of input channel ic sees for packed output
+ * column p0 + q. replaces device.h:802-805 (vae_kernels.cu:118-147, 934-946). */
+vv_status_t vv_vae_im2col_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in,
+                              int in_ch, int k, int stride, int64_t p0, int pc, void* col,
+                              int64_t ldcol, void* stream);
+/* y = w [out_ch][K] x col + b in FP32 fused multiply-adds in K order from
+ * zero: bit-identical to vv_vae_conv_dev. y NULL writes the transposed rows of
+ * the items in d. `tile` (0, 16, 32, 64) is accepted and changes no bit.
+ * replaces device.h:819-822 (vae_kernels.cu:149-284, 906-933). */
+vv_status_t vv_vae_conv_gemm_dev(const vv_vae_conv_desc_t* d, const void* w, const void* col,
+                                 int64_t ldcol, const void* b, void* y, int64_t ld_out,
+                                 int out_ch, int K, int64_t p0, int pc, int tile,
+                                 void* stream);
+/* C[M,P] (stride ldc) from A[M,K] x B[K,P] (stride ldb) on the matrix cores,
+ * FP32 accumulation in K order; rinv and norm_w (both or neither) normalise B
+ * on its way in: half(B[k][p] * rinv[p] * norm_w[k]). `tile` (0, 64, 128)
+ * changes no bit. replaces device.h:835-839 (vae_kernels.cu:394-607, 868-905). */
+vv_status_t vv_vae_gemm_nn_dev(int epilogue, const void* A, const void* B, int64_t ldb, void* C,
+                               int64_t ldc, int M, int K, int P, const void* bias,
+                               const void* gamma, const float* rinv, const void* norm_w,
+                               int tile, void* stream);
+#define VV_VAE_ROWS_PLAIN        0  /* C[r][c], stride ldc */
+#define VV_VAE_ROWS_STORE        1  /* segment rows, as computed */
+#define VV_VAE_ROWS_STORE_TRUNC  2  /* segment rows, FP16 by truncation, subnormals flushed */
+#define VV_VAE_ROWS_ACC_TRUNC    3  /* segment rows += value, truncated */
+typedef struct vv_vae_row_seg {
+    int   row0;   /* first packed row of this segment */
+    int   ld;     /* destination row stride, elements */
+    void* dst;
+} vv_vae_row_seg_t;
+typedef struct vv_vae_rows {
+    int              mode;
+    int              n;
+    vv_vae_row_seg_t seg[VV_VAE_MAX_ITEMS];
+} vv_vae_rows_t;
+/* C[M,N] = half(half(A[M,K] (stride lda) x B[N,K]^T) + bias), rows scattered per
+ * `rows` (NULL = plain). replaces device.h:863-866 (vae_kernels.cu:609-712,
+ * 947-970). */
+vv_status_t vv_vae_gemm_tn_dev(const void* A, int64_t lda, const void* B, void* C, int64_t ldc,
+                               int M, int N, int K, const void* bias,
+                               const vv_vae_rows_t* rows, void* stream);
+/* FP32 -> FP16 with a 64-bit count. replaces device.h:869-870. */
+vv_status_t vv_vae_f32_to_f16_dev(const float* in, void* out, int64_t n, void* stream);
+
+/* C[M,P] = alpha * A[M,K] x B[K,P] + beta * C, all row-major FP16, FP32
+ * accumulation on the matrix cores; beta == 0 never reads C.
+ * replaces device.h:477-479 (gemm.cu:441-460). */
+vv_status_t vv_gemm_fp16_nn_dev(const void* A, const void* B, void* C, int M, int K, int P,
+                                float alpha, float beta, void* stream);
+/* No handle to release. replaces device.h:482. */
+void vv_gemm_cleanup(void);
+
 /* ── BitNet integer layers (include/vibevoice/bitnet.h numerics) ───────── */
 
 /* Per-token int8: s = (float)(127 / max(max|x|, 1e-5)) in double, q = the

@@ -130,47 +130,22 @@ def test_attention_host_queries():
     assert dev.vv_gqa_decode_shape(1024) != dev.vv_gqa_decode_shape(1025)
 
 
-# ── the declined remainder of the seam ──────────────────────────────────────
-
-STUB_PATH = os.path.join(os.path.dirname(dev.LIB_PATH), "libvibevoice_hip_unsupported.so")
-
-
-def test_unsupported_library_declines_everything_and_overlaps_nothing():
-    import ctypes as C
-    out = subprocess.check_output(["nm", "-D", "--defined-only", STUB_PATH], text=True)
-    stubs = sorted(l.split()[-1] for l in out.splitlines() if " T vv_" in l)
-    assert len(stubs) == 11
-    assert not set(stubs) & set(dev.SIGNATURES)          # no symbol defined twice
-    lib = C.CDLL(STUB_PATH)
-    zero = set()
-    for name in stubs:
-        fn = getattr(lib, name)
-        if name == "vv_gemm_cleanup":
-            fn.restype = None
-            fn()
-        elif name in zero:
-            fn.restype = C.c_size_t
-            assert fn(1, 2, 3) == 0
-        else:
-            fn.restype = C.c_int
-            assert fn(None, None, None, 4, 5, None) == dev.VV_ERR_UNSUPPORTED, name
-
+# ── the whole seam ──────────────────────────────────────────────────────────
 
 REF_HEADER = "/root/reference/include/vibevoice/device.h"
 
 
 @pytest.mark.skipif(not os.path.exists(REF_HEADER), reason="reference tree not present")
-def test_the_two_libraries_define_every_symbol_of_the_reference_seam():
+def test_the_library_defines_every_symbol_of_the_reference_seam():
     text = re.sub(r"/\*.*?\*/", "", open(REF_HEADER).read(), flags=re.S)
     wanted = set(re.findall(r"^\s*(?:vv_status_t|int|size_t|void|bool|const char\*)\s+(vv_[a-z0-9_]+)\s*\(",
                             text, flags=re.M))
-    have = set()
-    for path in (dev.LIB_PATH, STUB_PATH):
-        out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
-        have |= {l.split()[-1] for l in out.splitlines() if " T vv_" in l}
+    out = subprocess.check_output(["nm", "-D", "--defined-only", dev.LIB_PATH], text=True)
+    have = {l.split()[-1] for l in out.splitlines() if " T vv_" in l}
+    assert not os.path.exists(os.path.join(os.path.dirname(dev.LIB_PATH), "libvibevoice_hip_unsupported.so"))
     assert len(wanted) >= 100 and not (wanted - have), sorted(wanted - have)
     # beyond device.h: the fused entry points, and the two kv_quant.h symbols
-    # (kv_quant.h:96-101) the decoder links against, declined
+    # (kv_quant.h:96-101) the decoder links against
     assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
                              "vv_embedding_rmsnorm_dev", "vv_gemv_multi_dev", "vv_gemv_swiglu_dev",
                              "vv_kv_rotate_dev", "vv_kv_unrotate_dev"}

@@ -241,3 +241,23 @@ def test_reference_own_bitnet_test_passes_on_this_backend():
     print(res.stdout[-3000:], res.stderr[-2000:])
     assert res.returncode == 0, res.stdout[-3000:]
     assert "FAIL" not in res.stdout
+
+
+VAE_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_vae_stream_hip")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(VAE_EXE),
+                    reason="oracle/_ref/test_vae_stream_hip not built (needs the reference tree)")
+def test_reference_own_vae_stream_test_passes_on_this_backend():
+    """The reference's tests/test_vae_stream.c: its whole Conv-VAE host pipeline
+    (encoder plan, streaming state, front end, speech connectors) on a tiny
+    random-weight model, driving this backend's kernels: against its FP32 and
+    CPU encoders, batched == one by one, any chunking == the whole signal,
+    conv-as-GEMM == direct conv and every GEMM tile == every other, bit for bit,
+    four threads at once == alone."""
+    res = subprocess.run([VAE_EXE], capture_output=True, text=True, timeout=110)
+    print(res.stdout[-3000:], res.stderr[-2000:])
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-2000:]
+    assert "FAIL" not in res.stdout and "FAIL" not in res.stderr and "SKIP" not in res.stdout
+    assert "43/43 passed" in res.stdout

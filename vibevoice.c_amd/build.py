@@ -19,7 +19,6 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libvibevoice_hip.so")
-STUB_LIB = os.path.join(LIBDIR, "libvibevoice_hip_unsupported.so")
 ARCH = "gfx950"
 
 # -packed-fp32-ops off: scalar FP32 arithmetic is never fused into v_pk_*_f32.
@@ -59,12 +58,11 @@ def build(verbose: bool = True) -> str:
         objs = list(pool.map(_compile, sources))
     cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB, *objs]
     subprocess.check_call(cmd)
-    # The remainder of device.h, declined: plain C, no device code.
-    subprocess.check_call([shutil.which("cc") or "gcc", "-O2", "-std=gnu11", "-fPIC", "-shared",
-                           "-Wno-deprecated-non-prototype", "-o", STUB_LIB,
-                           os.path.join(CSRC, "unsupported.c")])
+    stale = os.path.join(LIBDIR, "libvibevoice_hip_unsupported.so")      # an older build's second library
+    if os.path.exists(stale):
+        os.remove(stale)
     if verbose:
-        print(f"built {LIB} from {len(sources)} sources for {ARCH}, and {os.path.basename(STUB_LIB)}")
+        print(f"built {LIB} from {len(sources)} sources for {ARCH}")
     return LIB
 
 

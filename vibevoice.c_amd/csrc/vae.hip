@@ -1,0 +1,608 @@
+// The batched, streaming Conv-VAE encoder ops. FP16 activations, channel-first
+// and packed along time; the items of a launch sit side by side in one
+// [C][ld] buffer and only the convolutions know where one ends (a descriptor
+// passed by value). No output's arithmetic depends on where its item sits, on
+// how a stream was cut into chunks, or on which workgroup computes it: every
+// sum runs in one fixed order, and an FP16 rounding happens wherever a chain of
+// separate kernels would have stored an intermediate. So batching, chunking
+// and fusing change no bit.
+//
+//   vae_conv       one output per thread, an FP32 fused multiply-add chain over
+//                  (in channel, tap) from zero
+//   vae_tail       the next chunk's left context
+//   vae_im2col     the inputs of a strided conv as GEMM columns
+//   vae_conv_gemm  the conv over those columns: FP32 FMAs in K order per output
+//                  (the bits of vae_conv), 64x64 tile, 4x4 outputs per thread
+//   vae_rms        1 / rms over channels per column (packed and context)
+//   vae_mixer      RMSNorm -> depthwise conv -> gamma residual, fused
+//   vae_gemm       the FFN (A x B, B K-major) and connector (A x B^T) GEMMs on
+//                  v_mfma_f32_16x16x32_f16: 64x64 tile, four waves of 32x32,
+//                  64 K per LDS stage; a K-major B is transposed on its way
+//                  into LDS (and RMS-normalised there when asked); epilogues
+//                  bias+GELU, bias+gamma-residual, bias, bias+row scatter
+#include "vv_common.hpp"
+
+namespace vv {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+typedef vv_vae_conv_desc_t Desc;
+typedef vv_vae_conv_item_t Item;
+
+// Column `pos` of [context ++ input] of an item, channel ic; zero past either end.
+__device__ __forceinline__ h16 item_value(const Desc& d, const Item& it, const h16* __restrict__ x, int64_t ld_in,
+                                          int ic, int pos) {
+    if (pos >= it.have + it.in_len) return (h16)0.0f;
+    if (pos < it.have) {
+        const h16* tl = static_cast<const h16*>(it.tail_in);
+        return tl ? tl[(size_t)ic * d.cap + pos] : (h16)0.0f;
+    }
+    const h16* xb = it.in_ptr ? static_cast<const h16*>(it.in_ptr) : x + it.in_off;
+    return xb[(size_t)ic * ld_in + (pos - it.have)];
+}
+
+template <bool kTransposed>
+__global__ __launch_bounds__(kBlock) void vae_conv(Desc d, const h16* __restrict__ x, int64_t ld_in,
+                                                   const h16* __restrict__ w, const h16* __restrict__ b,
+                                                   h16* __restrict__ y, int64_t ld_out, int in_ch, int k,
+                                                   int stride) {
+    const Item& it = d.it[blockIdx.z];
+    const int oc = (int)blockIdx.y;
+    const int t = (int)blockIdx.x * kBlock + (int)threadIdx.x;
+    if (t >= it.out_len) return;
+    const int total = it.have + it.in_len;
+    const h16* wr = w + (size_t)oc * in_ch * k;
+    float sum = 0.0f;
+    for (int ic = 0; ic < in_ch; ++ic)
+        for (int kk = 0; kk < k; ++kk) {
+            const int p = t * stride + kk;
+            if (p < total) sum = __builtin_fmaf((float)wr[ic * k + kk], (float)item_value(d, it, x, ld_in, ic, p), sum);
+        }
+    if (b) sum += (float)b[oc];
+    if constexpr (kTransposed) {
+        if (t >= it.skip) static_cast<h16*>(it.out_ptr)[(size_t)(t - it.skip) * it.out_ld + oc] = to_half(sum);
+    } else {
+        y[(size_t)oc * ld_out + it.out_off + t] = to_half(sum);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void vae_tail(Desc d, const h16* __restrict__ x, int64_t ld_in, int in_ch) {
+    const Item& it = d.it[blockIdx.y];
+    if (!it.tail_out || it.keep <= 0) return;
+    const int idx = (int)blockIdx.x * kBlock + (int)threadIdx.x;
+    if (idx >= in_ch * it.keep) return;
+    const int c = idx / it.keep, j = idx - c * it.keep;
+    const int p = it.have + it.in_len - it.keep + j;
+    static_cast<h16*>(it.tail_out)[(size_t)c * d.cap + j] = p < 0 ? (h16)0.0f : item_value(d, it, x, ld_in, c, p);
+}
+
+// The item that owns packed output column p.
+__device__ __forceinline__ int item_of(const Desc& d, int64_t p) {
+    int i = 0;
+    while (i + 1 < d.n && p >= d.it[i + 1].out_off) ++i;
+    return i;
+}
+
+__global__ __launch_bounds__(kBlock) void vae_im2col(Desc d, const h16* __restrict__ x, int64_t ld_in, int k,
+                                                     int stride, int64_t p0, int pc, h16* __restrict__ col,
+                                                     int64_t ldcol) {
+    const int q = (int)blockIdx.x * kBlock + (int)threadIdx.x;
+    if (q >= pc) return;
+    const int kr = (int)blockIdx.y;
+    const int ic = kr / k, kk = kr - ic * k;
+    const int64_t p = p0 + q;
+    const Item& it = d.it[item_of(d, p)];
+    const int t = (int)(p - it.out_off);
+    h16 v = (h16)0.0f;
+    if (t < it.out_len) v = item_value(d, it, x, ld_in, ic, t * stride + kk);
+    col[(size_t)kr * ldcol + q] = v;
+}
+
+// y = A [M][K] x B [K][ldb] + bias in FP32, every output a fused multiply-add
+// chain over K from zero. 64x64 outputs per workgroup, 4x4 per thread, 16 K per stage.
+template <bool kTransposed>
+__global__ __launch_bounds__(kBlock) void vae_conv_gemm(const h16* __restrict__ A, const h16* __restrict__ B,
+                                                        int64_t ldb, h16* __restrict__ C, int64_t ldc, int M, int K,
+                                                        int P, const h16* __restrict__ bias, Desc d, int64_t p0) {
+    constexpr int T = 64, TBK = 16;
+    __shared__ float As[TBK][T + 4];
+    __shared__ float Bs[TBK][T + 4];
+    const int tid = (int)threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    const int row_base = (int)blockIdx.y * T, col_base = (int)blockIdx.x * T;
+    const int ar = tid / 4, ac = (tid % 4) * 4;         // A: row ar, K columns ac .. ac + 3 of the stage
+    const int br = tid / 16, bc = (tid % 16) * 4;       // B: K row br, columns bc .. bc + 3
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += TBK) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int gr = row_base + ar, gk = k0 + ac + t;
+            As[ac + t][ar] = (gr < M && gk < K) ? (float)A[(size_t)gr * K + gk] : 0.0f;
+            const int bk = k0 + br, gc = col_base + bc + t;
+            Bs[br][bc + t] = (bk < K && gc < P) ? (float)B[(size_t)bk * ldb + gc] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TBK; ++kk) {
+            float av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = col_base + tx * 4 + j;
+        if (c >= P) continue;
+        h16* dst;
+        int64_t step;
+        if constexpr (kTransposed) {
+            const int64_t p = p0 + c;
+            const Item& it = d.it[item_of(d, p)];
+            const int t = (int)(p - it.out_off);
+            if (t >= it.out_len || t < it.skip) continue;
+            dst = static_cast<h16*>(it.out_ptr) + (size_t)(t - it.skip) * it.out_ld;
+            step = 1;
+        } else {
+            dst = C + c;
+            step = ldc;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = row_base + ty * 4 + i;
+            if (r >= M) continue;
+            float v = acc[i][j];
+            if (bias) v += (float)bias[r];
+            dst[(size_t)r * step] = to_half(v);
+        }
+    }
+}
+
+__global__ __launch_bounds__(128) void vae_rms(const h16* __restrict__ x, int64_t ld, int64_t T, int C, float eps,
+                                               float* __restrict__ rinv, Desc d) {
+    const int64_t i = (int64_t)blockIdx.x * 128 + threadIdx.x;
+    const h16* col;
+    int64_t stride;
+    if (i < T) {
+        col = x + i;
+        stride = ld;
+    } else {
+        const int64_t j = i - T;
+        if (d.cap <= 0) return;
+        const int item = (int)(j / d.cap), q = (int)(j - (int64_t)item * d.cap);
+        if (item >= d.n) return;
+        const Item& it = d.it[item];
+        if (!it.tail_in || q >= it.have) return;
+        col = static_cast<const h16*>(it.tail_in) + q;
+        stride = d.cap;
+    }
+    float sum_sq = 0.0f;
+    for (int c = 0; c < C; ++c) {
+        const float v = (float)col[(size_t)c * stride];
+        sum_sq = __builtin_fmaf(v, v, sum_sq);
+    }
+    rinv[i] = __builtin_amdgcn_rsqf(sum_sq / (float)C + eps);
+}
+
+constexpr int kMixT = 64, kMixC = 32, kMixMaxK = 16;
+
+__global__ __launch_bounds__(kBlock) void vae_mixer(Desc d, const h16* __restrict__ xin, h16* __restrict__ xout,
+                                                    int64_t ld, const float* __restrict__ rinv, int64_t T_total,
+                                                    const h16* __restrict__ nw, const h16* __restrict__ cw,
+                                                    const h16* __restrict__ cb, const h16* __restrict__ gamma, int C,
+                                                    int k) {
+    const int item = (int)blockIdx.z;
+    const Item& it = d.it[item];
+    const int t0 = (int)blockIdx.x * kMixT;
+    if (t0 >= it.in_len) return;
+    const int c0 = (int)blockIdx.y * kMixC;
+    const int H = k - 1, W = kMixT + H;
+    __shared__ h16 nv[kMixC][kMixT + kMixMaxK];
+    const h16* tl = static_cast<const h16*>(it.tail_in);
+    for (int e = (int)threadIdx.x; e < kMixC * W; e += kBlock) {
+        const int cl = e / W, q = e - cl * W;
+        const int c = c0 + cl;
+        h16 out = (h16)0.0f;
+        if (c < C) {
+            const int p = t0 - H + q;
+            if (p >= 0) {
+                if (p < it.in_len) {
+                    const int64_t col = it.in_off + p;
+                    out = to_half(((float)xin[(size_t)c * ld + col] * rinv[col]) * (float)nw[c]);
+                }
+            } else {
+                const int tp = it.have + p;
+                if (tl && tp >= 0)
+                    out = to_half(((float)tl[(size_t)c * d.cap + tp] * rinv[T_total + (int64_t)item * d.cap + tp]) *
+                                  (float)nw[c]);
+            }
+        }
+        nv[cl][q] = out;
+    }
+    __syncthreads();
+    for (int e = (int)threadIdx.x; e < kMixC * kMixT; e += kBlock) {
+        const int cl = e / kMixT, tt = e - cl * kMixT;
+        const int c = c0 + cl, t = t0 + tt;
+        if (c >= C || t >= it.in_len) continue;
+        float sum = 0.0f;
+        for (int kk = 0; kk < k; ++kk) sum = __builtin_fmaf((float)cw[c * k + kk], (float)nv[cl][tt + kk], sum);
+        if (cb) sum += (float)cb[c];
+        const float yv = (float)to_half(sum);
+        const size_t off = (size_t)c * ld + it.in_off + t;
+        const float xv = (float)xin[off];
+        xout[off] = gamma ? to_half(__builtin_fmaf(yv, (float)gamma[c], xv)) : to_half(xv + yv);
+    }
+}
+
+// ── GEMMs on the matrix cores ───────────────────────────────────────────────
+
+enum { kEpiBiasGelu = 0, kEpiBiasResid = 1, kEpiBias = 2, kEpiRows = 3, kEpiAlphaBeta = 4 };
+
+struct GemmOut {
+    h16* c;
+    int64_t ldc;
+    const h16* bias;       // per row (NN epilogues) or per column (rows epilogue)
+    const h16* gamma;
+    float alpha, beta;
+    vv_vae_rows_t rows;
+};
+
+__device__ __forceinline__ float vae_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+
+// FP32 -> FP16 by truncation of the mantissa, subnormal results flushed to a
+// signed zero, overflow to infinity.
+__device__ __forceinline__ h16 trunc_half(float f) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int e = (int)((u >> 23) & 0xFF) - 127 + 15;
+    const uint32_t frac = (u >> 13) & 0x3FFu;
+    uint16_t h;
+    if (e <= 0) h = (uint16_t)sign;
+    else if (e >= 31) h = (uint16_t)(sign | 0x7C00u);
+    else h = (uint16_t)(sign | ((uint32_t)e << 10) | frac);
+    return __builtin_bit_cast(h16, h);
+}
+
+template <int kEpi>
+__device__ __forceinline__ void gemm_finish(const GemmOut& o, float acc, int r, int c) {
+    if constexpr (kEpi == kEpiRows) {
+        h16 y = to_half(acc);
+        if (o.bias) y = to_half((float)y + (float)o.bias[c]);
+        if (o.rows.mode == VV_VAE_ROWS_PLAIN) {
+            o.c[(size_t)r * o.ldc + c] = y;
+            return;
+        }
+        int s = 0;
+        while (s + 1 < o.rows.n && r >= o.rows.seg[s + 1].row0) ++s;
+        h16* dst = static_cast<h16*>(o.rows.seg[s].dst) + (size_t)(r - o.rows.seg[s].row0) * o.rows.seg[s].ld + c;
+        if (o.rows.mode == VV_VAE_ROWS_STORE) *dst = y;
+        else if (o.rows.mode == VV_VAE_ROWS_STORE_TRUNC) *dst = trunc_half((float)y);
+        else *dst = trunc_half((float)*dst + (float)y);
+        return;
+    }
+    const size_t off = (size_t)r * o.ldc + c;
+    if constexpr (kEpi == kEpiAlphaBeta) {
+        float v = o.alpha * acc;
+        if (o.beta != 0.0f) v = __builtin_fmaf(o.beta, (float)o.c[off], v);
+        o.c[off] = to_half(v);
+    } else if constexpr (kEpi == kEpiBias) {
+        o.c[off] = to_half(acc + (o.bias ? (float)o.bias[r] : 0.0f));
+    } else {
+        float v = (float)to_half(acc);
+        if (o.bias) v = (float)to_half(v + (float)o.bias[r]);
+        if constexpr (kEpi == kEpiBiasGelu) {
+            o.c[off] = to_half(vae_gelu(v));
+        } else {
+            const float xv = (float)o.c[off];
+            o.c[off] = o.gamma ? to_half(__builtin_fmaf(v, (float)o.gamma[r], xv)) : to_half(xv + v);
+        }
+    }
+}
+
+constexpr int kGT = 64;          // output tile edge
+constexpr int kGK = 64;          // K per LDS stage: two MFMA steps
+constexpr int kGLd = kGK + 8;    // LDS row stride in halves: 144 bytes, 16-byte aligned, rows on different banks
+
+// C[M][P] = A[M][K] (row stride lda) x B, B either [P][K] (kNN false, row stride
+// ldb) or [K][P] (kNN true, row stride ldb; optionally RMS-normalised while staged).
+template <bool kNN, int kEpi>
+__global__ __launch_bounds__(kBlock) void vae_gemm(const h16* __restrict__ A, int64_t lda, const h16* __restrict__ B,
+                                                   int64_t ldb, int M, int K, int P, const float* __restrict__ rinv,
+                                                   const h16* __restrict__ nw, GemmOut out) {
+    __shared__ __attribute__((aligned(16))) h16 As[kGT][kGLd];
+    __shared__ __attribute__((aligned(16))) h16 Bs[kGT][kGLd];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int row_base = (int)blockIdx.y * kGT, col_base = (int)blockIdx.x * kGT;
+    const bool a_vec = (lda & 7) == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0;
+    const bool b_vec = (ldb & 7) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+
+    f32x4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // K-contiguous rows of `src` (row stride ld) into dst[row][k]: 64 rows x 8 chunks of 8, two per thread.
+    auto stage_rows = [&](const h16* src, int64_t ld, bool vec, int base, int limit, int k0, h16 (*dst)[kGLd]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = tid + u * kBlock;
+            const int r = e >> 3, c = (e & 7) * 8;
+            const int gr = base + r;
+            h16x8 v;
+            if (vec && gr < limit && k0 + c + 8 <= K) {
+                v = *reinterpret_cast<const h16x8*>(src + (size_t)gr * ld + k0 + c);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    v[t] = (gr < limit && k0 + c + t < K) ? src[(size_t)gr * ld + k0 + c + t] : (h16)0.0f;
+            }
+            *reinterpret_cast<h16x8*>(&dst[r][c]) = v;
+        }
+    };
+    // K-major B: 64 K rows x 8 chunks of 8 columns, two per thread, transposed into Bs[column][k].
+    auto stage_kmajor = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = tid + u * kBlock;
+            const int kr = e >> 3, c = (e & 7) * 8;
+            const int gk = k0 + kr, gc = col_base + c;
+            h16x8 v;
+            if (b_vec && gk < K && gc + 8 <= P) {
+                v = *reinterpret_cast<const h16x8*>(B + (size_t)gk * ldb + gc);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = (gk < K && gc + t < P) ? B[(size_t)gk * ldb + gc + t] : (h16)0.0f;
+            }
+            if (nw) {
+                const float wn_k = gk < K ? (float)nw[gk] : 0.0f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    if (gk < K && gc + t < P) v[t] = to_half(((float)v[t] * rinv[gc + t]) * wn_k);
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) Bs[c + t][kr] = v[t];
+        }
+    };
+
+    for (int k0 = 0; k0 < K; k0 += kGK) {
+        stage_rows(A, lda, a_vec, row_base, M, k0, As);
+        if constexpr (kNN) stage_kmajor(k0);
+        else stage_rows(B, ldb, b_vec, col_base, P, k0, Bs);
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < kGK / 32; ++ks) {
+            h16x8 af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                af[i] = *reinterpret_cast<const h16x8*>(&As[wm * 32 + i * 16 + r16][ks * 32 + kq * 8]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                bf[j] = *reinterpret_cast<const h16x8*>(&Bs[wn * 32 + j * 16 + r16][ks * 32 + kq * 8]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    // register r of lane l: row 4 (l / 16) + r of the A tile, column l % 16 of the B tile
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = row_base + wm * 32 + i * 16 + 4 * kq + r;
+                const int col = col_base + wn * 32 + j * 16 + r16;
+                if (row < M && col < P) gemm_finish<kEpi>(out, acc[i][j][r], row, col);
+            }
+}
+
+__global__ __launch_bounds__(kBlock) void vae_f32_to_f16(const float* __restrict__ in, h16* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = to_half(in[i]);
+}
+
+int desc_max(const Desc* d, bool out) {
+    int m = 0;
+    for (int i = 0; i < d->n; ++i) {
+        const int v = out ? d->it[i].out_len : d->it[i].in_len;
+        if (v > m) m = v;
+    }
+    return m;
+}
+
+inline dim3 gemm_grid(int M, int P) { return dim3((unsigned)((P + kGT - 1) / kGT), (unsigned)((M + kGT - 1) / kGT)); }
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_vae_conv_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, const void* w, const void* b,
+                            void* y, int64_t ld_out, int in_ch, int out_ch, int k, int stride, bool transposed,
+                            void* stream) {
+    if (!d || !w) return VV_ERR_NULL_PTR;
+    if (d->n <= 0 || d->n > VV_VAE_MAX_ITEMS || in_ch <= 0 || out_ch <= 0 || out_ch > 65535 || k <= 0 || stride <= 0)
+        return VV_ERR_INVALID_ARG;
+    if (!transposed && !y) return VV_ERR_NULL_PTR;
+    const int m = vv::desc_max(d, true);
+    if (m <= 0) return VV_OK;
+    const dim3 grid((unsigned)((m + vv::kBlock - 1) / vv::kBlock), (unsigned)out_ch, (unsigned)d->n);
+    hipStream_t st = vv::as_stream(stream);
+    const vv::h16 *X = static_cast<const vv::h16*>(x), *W = static_cast<const vv::h16*>(w),
+                  *Bv = static_cast<const vv::h16*>(b);
+    if (transposed)
+        vv::vae_conv<true><<<grid, vv::kBlock, 0, st>>>(*d, X, ld_in, W, Bv, static_cast<vv::h16*>(y), ld_out, in_ch, k,
+                                                       stride);
+    else
+        vv::vae_conv<false><<<grid, vv::kBlock, 0, st>>>(*d, X, ld_in, W, Bv, static_cast<vv::h16*>(y), ld_out, in_ch, k,
+                                                        stride);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_tail_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, int in_ch, void* stream) {
+    if (!d) return VV_ERR_NULL_PTR;
+    if (d->n > VV_VAE_MAX_ITEMS || in_ch < 0) return VV_ERR_INVALID_ARG;
+    if (d->n <= 0 || d->cap <= 0 || in_ch == 0) return VV_OK;
+    const int n = in_ch * d->cap;
+    const dim3 grid((unsigned)((n + vv::kBlock - 1) / vv::kBlock), (unsigned)d->n);
+    vv::vae_tail<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(*d, static_cast<const vv::h16*>(x), ld_in, in_ch);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_rms_dev(const void* x, int64_t ld, int64_t T, int C, float eps, float* rinv,
+                           const vv_vae_conv_desc_t* d, void* stream) {
+    if (!x || !rinv) return VV_ERR_NULL_PTR;
+    if (C <= 0 || (d && d->n > VV_VAE_MAX_ITEMS)) return VV_ERR_INVALID_ARG;
+    vv_vae_conv_desc_t none = {};
+    const vv_vae_conv_desc_t* dd = d ? d : &none;
+    const int64_t n = (T > 0 ? T : 0) + (int64_t)(dd->n > 0 ? dd->n : 0) * (dd->cap > 0 ? dd->cap : 0);
+    if (n <= 0) return VV_OK;
+    const int64_t blocks = (n + 127) / 128;
+    if (blocks > 0x7FFFFFFF) return VV_ERR_UNSUPPORTED;
+    vv::vae_rms<<<dim3((unsigned)blocks), 128, 0, vv::as_stream(stream)>>>(static_cast<const vv::h16*>(x), ld,
+                                                                          T > 0 ? T : 0, C, eps, rinv, *dd);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_mixer_dev(const vv_vae_conv_desc_t* d, const void* xin, void* xout, int64_t ld, const float* rinv,
+                             int64_t T_total, const void* norm_w, const void* conv_w, const void* conv_b,
+                             const void* gamma, int C, int k, void* stream) {
+    if (!d || !xin || !xout || !rinv || !norm_w || !conv_w) return VV_ERR_NULL_PTR;
+    if (k < 1 || k > vv::kMixMaxK || d->n <= 0 || d->n > VV_VAE_MAX_ITEMS || C <= 0) return VV_ERR_INVALID_ARG;
+    const int m = vv::desc_max(d, false);
+    if (m <= 0) return VV_OK;
+    const dim3 grid((unsigned)((m + vv::kMixT - 1) / vv::kMixT), (unsigned)((C + vv::kMixC - 1) / vv::kMixC),
+                    (unsigned)d->n);
+    typedef const vv::h16* H;
+    vv::vae_mixer<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(*d, static_cast<H>(xin), static_cast<vv::h16*>(xout), ld,
+                                                                 rinv, T_total, static_cast<H>(norm_w),
+                                                                 static_cast<H>(conv_w), static_cast<H>(conv_b),
+                                                                 static_cast<H>(gamma), C, k);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_im2col_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, int in_ch, int k, int stride,
+                              int64_t p0, int pc, void* col, int64_t ldcol, void* stream) {
+    if (!d || !col) return VV_ERR_NULL_PTR;
+    if (d->n <= 0 || d->n > VV_VAE_MAX_ITEMS || in_ch <= 0 || k <= 0 || in_ch * k > 65535) return VV_ERR_INVALID_ARG;
+    if (pc <= 0) return VV_OK;
+    const dim3 grid((unsigned)((pc + vv::kBlock - 1) / vv::kBlock), (unsigned)(in_ch * k));
+    vv::vae_im2col<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(*d, static_cast<const vv::h16*>(x), ld_in, k, stride,
+                                                                  p0, pc, static_cast<vv::h16*>(col), ldcol);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_conv_gemm_dev(const vv_vae_conv_desc_t* d, const void* w, const void* col, int64_t ldcol,
+                                 const void* b, void* y, int64_t ld_out, int out_ch, int K, int64_t p0, int pc, int tile,
+                                 void* stream) {
+    if (!w || !col) return VV_ERR_NULL_PTR;
+    if (out_ch <= 0 || K <= 0) return VV_ERR_INVALID_ARG;
+    if (tile != 0 && tile != 16 && tile != 32 && tile != 64) return VV_ERR_INVALID_ARG;
+    if (!y && (!d || d->n <= 0 || d->n > VV_VAE_MAX_ITEMS)) return VV_ERR_INVALID_ARG;
+    if (pc <= 0) return VV_OK;
+    vv_vae_conv_desc_t none = {};
+    const dim3 grid((unsigned)((pc + 63) / 64), (unsigned)((out_ch + 63) / 64));
+    hipStream_t st = vv::as_stream(stream);
+    typedef const vv::h16* H;
+    if (y)
+        vv::vae_conv_gemm<false><<<grid, vv::kBlock, 0, st>>>(static_cast<H>(w), static_cast<H>(col), ldcol,
+                                                             static_cast<vv::h16*>(y), ld_out, out_ch, K, pc,
+                                                             static_cast<H>(b), none, p0);
+    else
+        vv::vae_conv_gemm<true><<<grid, vv::kBlock, 0, st>>>(static_cast<H>(w), static_cast<H>(col), ldcol, nullptr, 0,
+                                                            out_ch, K, pc, static_cast<H>(b), *d, p0);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_gemm_nn_dev(int epilogue, const void* A, const void* B, int64_t ldb, void* C, int64_t ldc, int M,
+                               int K, int P, const void* bias, const void* gamma, const float* rinv, const void* norm_w,
+                               int tile, void* stream) {
+    if (!A || !B || !C) return VV_ERR_NULL_PTR;
+    if (M <= 0 || K <= 0 || P <= 0) return VV_ERR_INVALID_ARG;
+    if ((norm_w != nullptr) != (rinv != nullptr)) return VV_ERR_INVALID_ARG;
+    if (tile != 0 && tile != 64 && tile != 128) return VV_ERR_INVALID_ARG;
+    typedef const vv::h16* H;
+    vv::GemmOut out = {};
+    out.c = static_cast<vv::h16*>(C);
+    out.ldc = ldc;
+    out.bias = static_cast<H>(bias);
+    out.gamma = static_cast<H>(gamma);
+    hipStream_t st = vv::as_stream(stream);
+    const dim3 grid = vv::gemm_grid(M, P);
+    H a = static_cast<H>(A), b = static_cast<H>(B), nw = static_cast<H>(norm_w);
+    if (epilogue == VV_VAE_EPI_BIAS_GELU)
+        vv::vae_gemm<true, vv::kEpiBiasGelu><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+    else if (epilogue == VV_VAE_EPI_BIAS_RESID)
+        vv::vae_gemm<true, vv::kEpiBiasResid><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+    else if (epilogue == VV_VAE_EPI_BIAS)
+        vv::vae_gemm<true, vv::kEpiBias><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+    else
+        return VV_ERR_INVALID_ARG;
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_gemm_tn_dev(const void* A, int64_t lda, const void* B, void* C, int64_t ldc, int M, int N, int K,
+                               const void* bias, const vv_vae_rows_t* rows, void* stream) {
+    if (!A || !B) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0 || K <= 0) return VV_ERR_INVALID_ARG;
+    vv::GemmOut out = {};
+    out.rows.mode = VV_VAE_ROWS_PLAIN;
+    if (rows) out.rows = *rows;
+    if (out.rows.mode == VV_VAE_ROWS_PLAIN && !C) return VV_ERR_NULL_PTR;
+    if (out.rows.mode != VV_VAE_ROWS_PLAIN &&
+        (out.rows.mode < 0 || out.rows.mode > VV_VAE_ROWS_ACC_TRUNC || out.rows.n <= 0 || out.rows.n > VV_VAE_MAX_ITEMS ||
+         out.rows.seg[0].row0 != 0))
+        return VV_ERR_INVALID_ARG;
+    out.c = static_cast<vv::h16*>(C);
+    out.ldc = ldc;
+    out.bias = static_cast<const vv::h16*>(bias);
+    vv::vae_gemm<false, vv::kEpiRows><<<vv::gemm_grid(M, N), vv::kBlock, 0, vv::as_stream(stream)>>>(
+        static_cast<const vv::h16*>(A), lda, static_cast<const vv::h16*>(B), K, M, K, N, nullptr, nullptr, out);
+    return vv::launch_status();
+}
+
+vv_status_t vv_vae_f32_to_f16_dev(const float* in, void* out, int64_t n, void* stream) {
+    if (!in || !out) return VV_ERR_NULL_PTR;
+    if (n <= 0) return VV_OK;
+    const int64_t blocks = (n + vv::kBlock - 1) / vv::kBlock;
+    if (blocks > 0x7FFFFFFF) return VV_ERR_UNSUPPORTED;
+    vv::vae_f32_to_f16<<<dim3((unsigned)blocks), vv::kBlock, 0, vv::as_stream(stream)>>>(in, static_cast<vv::h16*>(out), n);
+    return vv::launch_status();
+}
+
+vv_status_t vv_gemm_fp16_nn_dev(const void* A, const void* B, void* C, int M, int K, int P, float alpha, float beta,
+                                void* stream) {
+    if (!A || !B || !C) return VV_ERR_NULL_PTR;
+    if (M <= 0 || P <= 0) return VV_OK;
+    if (K < 0) return VV_ERR_INVALID_ARG;
+    vv::GemmOut out = {};
+    out.c = static_cast<vv::h16*>(C);
+    out.ldc = P;
+    out.alpha = alpha;
+    out.beta = beta;
+    vv::vae_gemm<true, vv::kEpiAlphaBeta><<<vv::gemm_grid(M, P), vv::kBlock, 0, vv::as_stream(stream)>>>(
+        static_cast<const vv::h16*>(A), K, static_cast<const vv::h16*>(B), P, M, K, P, nullptr, nullptr, out);
+    return vv::launch_status();
+}
+
+void vv_gemm_cleanup(void) {}
+
+}  // extern "C"

@@ -50,6 +50,30 @@ class I8Proj(C.Structure):
                 ("y", C.c_void_p), ("N", C.c_int)]
 
 
+VAE_MAX_ITEMS = 32
+
+
+class VaeConvItem(C.Structure):
+    """vv_vae_conv_item_t: one item's view of one convolution layer."""
+    _fields_ = [("in_off", C.c_int64), ("out_off", C.c_int64), ("in_ptr", C.c_void_p), ("tail_in", C.c_void_p),
+                ("tail_out", C.c_void_p), ("out_ptr", C.c_void_p), ("in_len", C.c_int), ("out_len", C.c_int),
+                ("have", C.c_int), ("keep", C.c_int), ("out_ld", C.c_int), ("skip", C.c_int)]
+
+
+class VaeConvDesc(C.Structure):
+    """vv_vae_conv_desc_t: the items of a launch, passed by value to the kernels."""
+    _fields_ = [("n", C.c_int), ("cap", C.c_int), ("it", VaeConvItem * VAE_MAX_ITEMS)]
+
+
+class VaeRowSeg(C.Structure):
+    _fields_ = [("row0", C.c_int), ("ld", C.c_int), ("dst", C.c_void_p)]
+
+
+class VaeRows(C.Structure):
+    """vv_vae_rows_t: where the rows of a connector GEMM go."""
+    _fields_ = [("mode", C.c_int), ("n", C.c_int), ("seg", VaeRowSeg * VAE_MAX_ITEMS)]
+
+
 # symbol -> (restype, argtypes); the complete export list of include/vibevoice_hip.h
 SIGNATURES = {
     "vv_embedding_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
@@ -105,6 +129,17 @@ SIGNATURES = {
     "vv_i8s_requant_dev": (_i, [_vp, C.c_int64, _vp, _i, _vp, _vp, _vp]),
     "vv_i8_head_argmax_scratch_bytes": (C.c_size_t, [_i]),
     "vv_i8_head_argmax_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
+    "vv_vae_conv_dev": (_i, [_vp, _vp, C.c_int64, _vp, _vp, _vp, C.c_int64, _i, _i, _i, _i, C.c_bool, _vp]),
+    "vv_vae_tail_dev": (_i, [_vp, _vp, C.c_int64, _i, _vp]),
+    "vv_vae_rms_dev": (_i, [_vp, C.c_int64, C.c_int64, _i, C.c_float, _vp, _vp, _vp]),
+    "vv_vae_mixer_dev": (_i, [_vp, _vp, _vp, C.c_int64, _vp, C.c_int64, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "vv_vae_im2col_dev": (_i, [_vp, _vp, C.c_int64, _i, _i, _i, C.c_int64, _i, _vp, C.c_int64, _vp]),
+    "vv_vae_conv_gemm_dev": (_i, [_vp, _vp, _vp, C.c_int64, _vp, _vp, C.c_int64, _i, _i, C.c_int64, _i, _i, _vp]),
+    "vv_vae_gemm_nn_dev": (_i, [_i, _vp, _vp, C.c_int64, _vp, C.c_int64, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "vv_vae_gemm_tn_dev": (_i, [_vp, C.c_int64, _vp, _vp, C.c_int64, _i, _i, _i, _vp, _vp, _vp]),
+    "vv_vae_f32_to_f16_dev": (_i, [_vp, _vp, C.c_int64, _vp]),
+    "vv_gemm_fp16_nn_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, C.c_float, C.c_float, _vp]),
+    "vv_gemm_cleanup": (None, []),
     "vv_w8a8_linear_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_w4a8_linear_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "vv_i8_linear_multi_dev": (_i, [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
