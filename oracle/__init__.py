@@ -109,6 +109,19 @@ def _load():
                                                C.c_void_p, C.c_void_p])):
         getattr(lib, name).restype = C.c_int
         getattr(lib, name).argtypes = args
+    V, I64 = C.c_void_p, C.c_int64
+    for name, args in (("vvo_vae_conv", [V, V, I64, V, V, V, I64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+                       ("vvo_vae_tail", [V, V, I64, C.c_int]),
+                       ("vvo_vae_im2col", [V, V, I64, C.c_int, C.c_int, C.c_int, I64, C.c_int, V, I64]),
+                       ("vvo_vae_conv_gemm", [V, V, I64, V, V, I64, C.c_int, C.c_int, C.c_int]),
+                       ("vvo_vae_rms", [V, I64, I64, C.c_int, C.c_float, V, V]),
+                       ("vvo_vae_mixer", [V, V, V, I64, V, I64, V, V, V, V, C.c_int, C.c_int]),
+                       ("vvo_vae_gemm_nn", [C.c_int, V, V, I64, V, I64, C.c_int, C.c_int, C.c_int, V, V, V, V]),
+                       ("vvo_vae_gemm_tn", [V, I64, V, V, I64, C.c_int, C.c_int, C.c_int, V, V])):
+        getattr(lib, name).restype = C.c_int
+        getattr(lib, name).argtypes = args
+    lib.vvo_trunc_half.restype = C.c_uint16
+    lib.vvo_trunc_half.argtypes = [C.c_float]
     for name, args in (("vvo_kv_bytes_per_vec", [C.c_int]),
                        ("vvo_kv_rotate", [C.c_void_p, C.c_int, C.c_int]),
                        ("vvo_kv_store_tq", [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
@@ -491,6 +504,76 @@ def int8_dequant(q, scales):
     _check(lib.vvo_int8_dequant(q.ctypes.data, scales.ctypes.data, N, K, o16.ctypes.data, o32.ctypes.data),
            "int8_dequant")
     return o16, o32
+
+
+# ── Conv-VAE encoder ops: thin views of the C functions ─────────────────────
+# The descriptor mirrors include/vibevoice/device.h:733-755 field for field, so
+# one ctypes layout serves the oracle (host pointers) and the device library.
+
+VAE_MAX_ITEMS = 32
+
+
+class VaeConvItem(C.Structure):
+    _fields_ = [("in_off", C.c_int64), ("out_off", C.c_int64), ("in_ptr", C.c_void_p), ("tail_in", C.c_void_p),
+                ("tail_out", C.c_void_p), ("out_ptr", C.c_void_p), ("in_len", C.c_int), ("out_len", C.c_int),
+                ("have", C.c_int), ("keep", C.c_int), ("out_ld", C.c_int), ("skip", C.c_int)]
+
+
+class VaeConvDesc(C.Structure):
+    _fields_ = [("n", C.c_int), ("cap", C.c_int), ("it", VaeConvItem * VAE_MAX_ITEMS)]
+
+
+class VaeRowSeg(C.Structure):
+    _fields_ = [("row0", C.c_int), ("ld", C.c_int), ("dst", C.c_void_p)]
+
+
+class VaeRows(C.Structure):
+    _fields_ = [("mode", C.c_int), ("n", C.c_int), ("seg", VaeRowSeg * VAE_MAX_ITEMS)]
+
+
+def _hp(a):
+    """Host address of a numpy array (or None)."""
+    return a.ctypes.data if a is not None else None
+
+
+def vae_conv(desc, x, ld_in, w, b, y, ld_out, in_ch, out_ch, k, stride, transposed=False):
+    _check(lib.vvo_vae_conv(C.addressof(desc), _hp(x), ld_in, _hp(w), _hp(b), _hp(y), ld_out, in_ch, out_ch, k, stride,
+                            int(transposed)), "vae_conv")
+
+
+def vae_tail(desc, x, ld_in, in_ch):
+    _check(lib.vvo_vae_tail(C.addressof(desc), _hp(x), ld_in, in_ch), "vae_tail")
+
+
+def vae_im2col(desc, x, ld_in, in_ch, k, stride, p0, pc, col, ldcol):
+    _check(lib.vvo_vae_im2col(C.addressof(desc), _hp(x), ld_in, in_ch, k, stride, p0, pc, _hp(col), ldcol), "vae_im2col")
+
+
+def vae_conv_gemm(w, col, ldcol, b, y, ld_out, out_ch, K, pc):
+    _check(lib.vvo_vae_conv_gemm(_hp(w), _hp(col), ldcol, _hp(b), _hp(y), ld_out, out_ch, K, pc), "vae_conv_gemm")
+
+
+def vae_rms(x, ld, T, Cn, eps, rinv, desc=None):
+    _check(lib.vvo_vae_rms(_hp(x), ld, T, Cn, eps, _hp(rinv), C.addressof(desc) if desc is not None else None), "vae_rms")
+
+
+def vae_mixer(desc, xin, xout, ld, rinv, T_total, nw, cw, cb, gamma, Cn, k):
+    _check(lib.vvo_vae_mixer(C.addressof(desc), _hp(xin), _hp(xout), ld, _hp(rinv), T_total, _hp(nw), _hp(cw), _hp(cb),
+                             _hp(gamma), Cn, k), "vae_mixer")
+
+
+def vae_gemm_nn(epilogue, A, B, ldb, Cm, ldc, M, K, P, bias=None, gamma=None, rinv=None, nw=None):
+    _check(lib.vvo_vae_gemm_nn(epilogue, _hp(A), _hp(B), ldb, _hp(Cm), ldc, M, K, P, _hp(bias), _hp(gamma), _hp(rinv),
+                               _hp(nw)), "vae_gemm_nn")
+
+
+def vae_gemm_tn(A, lda, B, Cm, ldc, M, N, K, bias=None, rows=None):
+    _check(lib.vvo_vae_gemm_tn(_hp(A), lda, _hp(B), _hp(Cm), ldc, M, N, K, _hp(bias),
+                               C.addressof(rows) if rows is not None else None), "vae_gemm_tn")
+
+
+def trunc_half(f: float) -> int:
+    return int(lib.vvo_trunc_half(float(f)))
 
 
 def ternary_pack(t) -> np.ndarray:

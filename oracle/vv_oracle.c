@@ -1024,6 +1024,232 @@ int vvo_i8_head_argmax(const int8_t* q, float scale, const int8_t* w, const floa
     return VVO_OK;
 }
 
+/* ── Conv-VAE encoder ops (src/cuda/vae_kernels.cu) ───────────────────────── */
+
+/* Column pos of [context ++ input] of an item, channel ic: context from the
+ * state (zeros when there is none), then the item's input, then zeros. */
+static float vae_item_value(const vvo_vae_conv_desc_t* d, const vvo_vae_conv_item_t* it, const uint16_t* x,
+                            int64_t ld_in, int ic, int pos, uint16_t* bits) {
+    uint16_t v = 0;
+    if (pos >= 0 && pos < it->have + it->in_len) {
+        if (pos < it->have) {
+            const uint16_t* tl = (const uint16_t*)it->tail_in;
+            v = tl ? tl[(size_t)ic * d->cap + pos] : 0;
+        } else {
+            const uint16_t* xb = it->in_ptr ? (const uint16_t*)it->in_ptr : x + it->in_off;
+            v = xb[(size_t)ic * ld_in + (pos - it->have)];
+        }
+    }
+    if (bits) *bits = v;
+    return vvo_half_to_float(v);
+}
+
+int vvo_vae_conv(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, const uint16_t* w,
+                 const uint16_t* b, uint16_t* y, int64_t ld_out, int in_ch, int out_ch, int k, int stride,
+                 int transposed) {
+    if (!d || !w) return VVO_ERR_NULL_PTR;
+    if (d->n <= 0 || d->n > VVO_VAE_MAX_ITEMS) return VVO_ERR_INVALID_ARG;
+    for (int i = 0; i < d->n; i++) {
+        const vvo_vae_conv_item_t* it = &d->it[i];
+        for (int oc = 0; oc < out_ch; oc++)
+            for (int t = 0; t < it->out_len; t++) {
+                float sum = 0.0f;
+                for (int ic = 0; ic < in_ch; ic++)
+                    for (int kk = 0; kk < k; kk++) {
+                        const int p = t * stride + kk;
+                        if (p < it->have + it->in_len)
+                            sum = fmaf(vvo_half_to_float(w[((size_t)oc * in_ch + ic) * k + kk]),
+                                       vae_item_value(d, it, x, ld_in, ic, p, NULL), sum);
+                    }
+                if (b) sum += vvo_half_to_float(b[oc]);
+                if (transposed) {
+                    if (t >= it->skip)
+                        ((uint16_t*)it->out_ptr)[(size_t)(t - it->skip) * it->out_ld + oc] = vvo_float_to_half_rne(sum);
+                } else {
+                    y[(size_t)oc * ld_out + it->out_off + t] = vvo_float_to_half_rne(sum);
+                }
+            }
+    }
+    return VVO_OK;
+}
+
+int vvo_vae_tail(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, int in_ch) {
+    if (!d) return VVO_ERR_NULL_PTR;
+    for (int i = 0; i < d->n; i++) {
+        const vvo_vae_conv_item_t* it = &d->it[i];
+        if (!it->tail_out || it->keep <= 0) continue;
+        for (int c = 0; c < in_ch; c++)
+            for (int j = 0; j < it->keep; j++) {
+                uint16_t v;
+                vae_item_value(d, it, x, ld_in, c, it->have + it->in_len - it->keep + j, &v);
+                ((uint16_t*)it->tail_out)[(size_t)c * d->cap + j] = v;
+            }
+    }
+    return VVO_OK;
+}
+
+static const vvo_vae_conv_item_t* vae_item_of(const vvo_vae_conv_desc_t* d, int64_t p) {
+    int i = 0;
+    while (i + 1 < d->n && p >= d->it[i + 1].out_off) i++;
+    return &d->it[i];
+}
+
+int vvo_vae_im2col(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, int in_ch, int k, int stride,
+                   int64_t p0, int pc, uint16_t* col, int64_t ldcol) {
+    if (!d || !col) return VVO_ERR_NULL_PTR;
+    for (int kr = 0; kr < in_ch * k; kr++)
+        for (int q = 0; q < pc; q++) {
+            const vvo_vae_conv_item_t* it = vae_item_of(d, p0 + q);
+            const int t = (int)(p0 + q - it->out_off);
+            uint16_t v = 0;
+            if (t < it->out_len) vae_item_value(d, it, x, ld_in, kr / k, t * stride + kr % k, &v);
+            col[(size_t)kr * ldcol + q] = v;
+        }
+    return VVO_OK;
+}
+
+int vvo_vae_conv_gemm(const uint16_t* w, const uint16_t* col, int64_t ldcol, const uint16_t* b, uint16_t* y,
+                      int64_t ld_out, int out_ch, int K, int pc) {
+    if (!w || !col || !y) return VVO_ERR_NULL_PTR;
+    for (int oc = 0; oc < out_ch; oc++)
+        for (int q = 0; q < pc; q++) {
+            float sum = 0.0f;
+            for (int kr = 0; kr < K; kr++)
+                sum = fmaf(vvo_half_to_float(w[(size_t)oc * K + kr]), vvo_half_to_float(col[(size_t)kr * ldcol + q]), sum);
+            if (b) sum += vvo_half_to_float(b[oc]);
+            y[(size_t)oc * ld_out + q] = vvo_float_to_half_rne(sum);
+        }
+    return VVO_OK;
+}
+
+static float vae_rms_col(const uint16_t* col, int64_t stride, int C, float eps) {
+    float ss = 0.0f;
+    for (int c = 0; c < C; c++) {
+        const float v = vvo_half_to_float(col[(size_t)c * stride]);
+        ss = fmaf(v, v, ss);
+    }
+    return 1.0f / sqrtf(ss / (float)C + eps);
+}
+
+int vvo_vae_rms(const uint16_t* x, int64_t ld, int64_t T, int C, float eps, float* rinv,
+                const vvo_vae_conv_desc_t* d) {
+    if (!x || !rinv) return VVO_ERR_NULL_PTR;
+    for (int64_t i = 0; i < T; i++) rinv[i] = vae_rms_col(x + i, ld, C, eps);
+    if (d && d->cap > 0)
+        for (int item = 0; item < d->n; item++) {
+            const vvo_vae_conv_item_t* it = &d->it[item];
+            if (!it->tail_in) continue;
+            for (int q = 0; q < it->have; q++)
+                rinv[T + (int64_t)item * d->cap + q] = vae_rms_col((const uint16_t*)it->tail_in + q, d->cap, C, eps);
+        }
+    return VVO_OK;
+}
+
+int vvo_vae_mixer(const vvo_vae_conv_desc_t* d, const uint16_t* xin, uint16_t* xout, int64_t ld, const float* rinv,
+                  int64_t T_total, const uint16_t* nw, const uint16_t* cw, const uint16_t* cb,
+                  const uint16_t* gamma, int C, int k) {
+    if (!d || !xin || !xout || !rinv || !nw || !cw) return VVO_ERR_NULL_PTR;
+    if (k < 1 || k > 16) return VVO_ERR_INVALID_ARG;
+    for (int item = 0; item < d->n; item++) {
+        const vvo_vae_conv_item_t* it = &d->it[item];
+        const uint16_t* tl = (const uint16_t*)it->tail_in;
+        for (int c = 0; c < C; c++)
+            for (int t = 0; t < it->in_len; t++) {
+                float sum = 0.0f;
+                for (int kk = 0; kk < k; kk++) {
+                    const int p = t - (k - 1) + kk;             /* position in the item's input; negative = context */
+                    uint16_t nv = 0;
+                    if (p >= 0) {
+                        const int64_t col = it->in_off + p;
+                        nv = vvo_float_to_half_rne((vvo_half_to_float(xin[(size_t)c * ld + col]) * rinv[col]) *
+                                                   vvo_half_to_float(nw[c]));
+                    } else {
+                        const int tp = it->have + p;
+                        if (tl && tp >= 0)
+                            nv = vvo_float_to_half_rne((vvo_half_to_float(tl[(size_t)c * d->cap + tp]) *
+                                                        rinv[T_total + (int64_t)item * d->cap + tp]) *
+                                                       vvo_half_to_float(nw[c]));
+                    }
+                    sum = fmaf(vvo_half_to_float(cw[c * k + kk]), vvo_half_to_float(nv), sum);
+                }
+                if (cb) sum += vvo_half_to_float(cb[c]);
+                const float yv = vvo_half_to_float(vvo_float_to_half_rne(sum));
+                const size_t off = (size_t)c * ld + it->in_off + t;
+                const float xv = vvo_half_to_float(xin[off]);
+                xout[off] = vvo_float_to_half_rne(gamma ? fmaf(yv, vvo_half_to_float(gamma[c]), xv) : xv + yv);
+            }
+    }
+    return VVO_OK;
+}
+
+int vvo_vae_gemm_nn(int epilogue, const uint16_t* A, const uint16_t* B, int64_t ldb, uint16_t* C, int64_t ldc,
+                    int M, int K, int P, const uint16_t* bias, const uint16_t* gamma, const float* rinv,
+                    const uint16_t* nw) {
+    if (!A || !B || !C) return VVO_ERR_NULL_PTR;
+    if (epilogue < 0 || epilogue > 2 || ((nw != NULL) != (rinv != NULL))) return VVO_ERR_INVALID_ARG;
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < M; r++)
+        for (int c = 0; c < P; c++) {
+            double acc = 0.0;
+            for (int kk = 0; kk < K; kk++) {
+                float bv = vvo_half_to_float(B[(size_t)kk * ldb + c]);
+                if (nw) bv = vvo_half_to_float(vvo_float_to_half_rne((bv * rinv[c]) * vvo_half_to_float(nw[kk])));
+                acc += (double)vvo_half_to_float(A[(size_t)r * K + kk]) * (double)bv;
+            }
+            const size_t off = (size_t)r * ldc + c;
+            if (epilogue == 2) {
+                C[off] = vvo_float_to_half_rne((float)acc + (bias ? vvo_half_to_float(bias[r]) : 0.0f));
+                continue;
+            }
+            float v = vvo_half_to_float(vvo_float_to_half_rne((float)acc));
+            if (bias) v = vvo_half_to_float(vvo_float_to_half_rne(v + vvo_half_to_float(bias[r])));
+            if (epilogue == 0) {
+                C[off] = vvo_float_to_half_rne(0.5f * v * (1.0f + erff(v * 0.7071067811865476f)));
+            } else {
+                const float xv = vvo_half_to_float(C[off]);
+                C[off] = vvo_float_to_half_rne(gamma ? fmaf(v, vvo_half_to_float(gamma[r]), xv) : xv + v);
+            }
+        }
+    return VVO_OK;
+}
+
+uint16_t vvo_trunc_half(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int e = (int)((u >> 23) & 0xFF) - 127 + 15;
+    const uint32_t frac = (u >> 13) & 0x3FFu;
+    if (e <= 0) return (uint16_t)sign;
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+    return (uint16_t)(sign | ((uint32_t)e << 10) | frac);
+}
+
+int vvo_vae_gemm_tn(const uint16_t* A, int64_t lda, const uint16_t* B, uint16_t* C, int64_t ldc, int M, int N,
+                    int K, const uint16_t* bias, const vvo_vae_rows_t* rows) {
+    if (!A || !B) return VVO_ERR_NULL_PTR;
+    const int mode = rows ? rows->mode : 0;
+    if (mode == 0 && !C) return VVO_ERR_NULL_PTR;
+    for (int r = 0; r < M; r++)
+        for (int c = 0; c < N; c++) {
+            double acc = 0.0;
+            for (int kk = 0; kk < K; kk++)
+                acc += (double)vvo_half_to_float(A[(size_t)r * lda + kk]) * (double)vvo_half_to_float(B[(size_t)c * K + kk]);
+            uint16_t y = vvo_float_to_half_rne((float)acc);
+            if (bias) y = vvo_float_to_half_rne(vvo_half_to_float(y) + vvo_half_to_float(bias[c]));
+            if (mode == 0) {
+                C[(size_t)r * ldc + c] = y;
+                continue;
+            }
+            int s = 0;
+            while (s + 1 < rows->n && r >= rows->seg[s + 1].row0) s++;
+            uint16_t* dst = (uint16_t*)rows->seg[s].dst + (size_t)(r - rows->seg[s].row0) * rows->seg[s].ld + c;
+            if (mode == 1) *dst = y;
+            else if (mode == 2) *dst = vvo_trunc_half(vvo_half_to_float(y));
+            else *dst = vvo_trunc_half(vvo_half_to_float(*dst) + vvo_half_to_float(y));
+        }
+    return VVO_OK;
+}
+
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value) {
     if (!logits || !token) return VVO_ERR_NULL_PTR;
     int best = 0;

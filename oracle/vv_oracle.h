@@ -240,6 +240,57 @@ int vvo_i8s_requant(const float* y, int64_t n, float absmax, int relu, int8_t* q
 int vvo_i8_head_argmax(const int8_t* q, float scale, const int8_t* w, const float* w_scale, int V, int K,
                        int32_t* token, float* value);
 
+/* The batched, streaming Conv-VAE encoder ops (src/cuda/vae_kernels.cu; the
+ * reference's CPU encoder works in FP32 with other roundings, so these restate
+ * the accelerator's arithmetic). Host pointers throughout; FP16 as uint16 bits.
+ * The descriptor is include/vibevoice/device.h:733-755, field for field.
+ *   vvo_vae_conv      vae_kernels.cu:50-89   FP32 fused multiply-add chain over
+ *                     (in channel, tap) from zero, + bias, one FP16 rounding
+ *   vvo_vae_tail      :95-116    the last `keep` columns of [context ++ input]
+ *   vvo_vae_im2col    :118-147
+ *   vvo_vae_conv_gemm :149-284   the same chain over K of the im2col columns
+ *   vvo_vae_rms       :286-318   1 / sqrt(sum of squares (FMA chain) / C + eps)
+ *   vvo_vae_mixer     :320-392   half((x * rinv) * w) -> depthwise FMA chain ->
+ *                     half -> half(x + y * gamma)
+ *   vvo_vae_gemm_nn   :394-607   A[M,K] x B[K,P] (double accumulation here), B
+ *                     optionally normalised on its way in, three epilogues
+ *   vvo_vae_gemm_tn   :609-712   A x B^T + bias, rows scattered, truncating modes
+ *   vvo_trunc_half    :614-625 */
+#define VVO_VAE_MAX_ITEMS 32
+typedef struct vvo_vae_conv_item {
+    int64_t in_off, out_off;
+    const void* in_ptr;
+    const void* tail_in;
+    void* tail_out;
+    void* out_ptr;
+    int in_len, out_len, have, keep, out_ld, skip;
+} vvo_vae_conv_item_t;
+typedef struct vvo_vae_conv_desc {
+    int n, cap;
+    vvo_vae_conv_item_t it[VVO_VAE_MAX_ITEMS];
+} vvo_vae_conv_desc_t;
+typedef struct vvo_vae_row_seg { int row0, ld; void* dst; } vvo_vae_row_seg_t;
+typedef struct vvo_vae_rows { int mode, n; vvo_vae_row_seg_t seg[VVO_VAE_MAX_ITEMS]; } vvo_vae_rows_t;
+int vvo_vae_conv(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, const uint16_t* w,
+                 const uint16_t* b, uint16_t* y, int64_t ld_out, int in_ch, int out_ch, int k, int stride,
+                 int transposed);
+int vvo_vae_tail(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, int in_ch);
+int vvo_vae_im2col(const vvo_vae_conv_desc_t* d, const uint16_t* x, int64_t ld_in, int in_ch, int k, int stride,
+                   int64_t p0, int pc, uint16_t* col, int64_t ldcol);
+int vvo_vae_conv_gemm(const uint16_t* w, const uint16_t* col, int64_t ldcol, const uint16_t* b, uint16_t* y,
+                      int64_t ld_out, int out_ch, int K, int pc);
+int vvo_vae_rms(const uint16_t* x, int64_t ld, int64_t T, int C, float eps, float* rinv,
+                const vvo_vae_conv_desc_t* d);
+int vvo_vae_mixer(const vvo_vae_conv_desc_t* d, const uint16_t* xin, uint16_t* xout, int64_t ld, const float* rinv,
+                  int64_t T_total, const uint16_t* nw, const uint16_t* cw, const uint16_t* cb,
+                  const uint16_t* gamma, int C, int k);
+int vvo_vae_gemm_nn(int epilogue, const uint16_t* A, const uint16_t* B, int64_t ldb, uint16_t* C, int64_t ldc,
+                    int M, int K, int P, const uint16_t* bias, const uint16_t* gamma, const float* rinv,
+                    const uint16_t* nw);
+int vvo_vae_gemm_tn(const uint16_t* A, int64_t lda, const uint16_t* B, uint16_t* C, int64_t ldc, int M, int N,
+                    int K, const uint16_t* bias, const vvo_vae_rows_t* rows);
+uint16_t vvo_trunc_half(float f);
+
 /* src/cpu/cpu_kernels.c:1613-1623 (vv_sample_greedy_cpu): the first maximum of
  * an in-order scan; a NaN never replaces the running best. */
 int vvo_argmax_first(const float* logits, int n, int32_t* token, float* value);

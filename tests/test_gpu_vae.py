@@ -1,0 +1,312 @@
+"""GPU parity tests of the Conv-VAE encoder ops through the C ABI. Everything
+whose arithmetic the interface fixes operation by operation (the convolutions
+and their GEMM form, the context copy, im2col, the fused mixer given the same
+1/rms, the conversions) is held to bit equality with the oracle; the 1/rms
+itself to 2 FP32 ulps (hardware reciprocal square root); the matrix-core GEMMs,
+whose FP32 sums run in the hardware's order, to the FP16 bar (scaled error
+<= 2e-3) with at most a stray FP16 step against the oracle's double sums."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import VaeConvDesc, VaeRows
+from gpu_util import FP16_TOL, bits_of, dev, ok, stream, to_dev
+from conftest import scaled_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def P(t):
+    return t.data_ptr() if t is not None else None
+
+
+def f16(shape, seed, std=1.0):
+    return oracle.normal_f16(shape, seed, std=std)
+
+
+class Batch:
+    """Three items packed side by side: a fresh one, one with a carried state, one given by its own pointer."""
+
+    def __init__(self, in_ch, k, stride, seed, own_pointer=True):
+        rng = np.random.default_rng(seed)
+        self.in_ch, self.k, self.stride = in_ch, k, stride
+        self.cap = max(k - stride, 1)
+        in_lens = [int(rng.integers(3, 40)) * stride, int(rng.integers(50, 300)) * stride + (stride > 1), 7 * stride]
+        self.items = []
+        in_off = out_off = 0
+        for i, n_in in enumerate(in_lens):
+            have = 0 if i == 0 else self.cap
+            own = own_pointer and i == 2
+            it = dict(in_len=n_in, out_len=-(-n_in // stride), have=have, keep=self.cap, in_off=0 if own else in_off,
+                      out_off=out_off, tail_in=f16((in_ch, self.cap), seed + 10 + i) if have else None,
+                      tail_out=np.full((in_ch, self.cap), 0x7E00, np.uint16),
+                      own=f16((in_ch, n_in + 5), seed + 20) if own else None)
+            self.items.append(it)
+            if not own:
+                in_off += n_in
+            out_off += it["out_len"]
+        self.T_in, self.T_out = in_off, out_off
+        self.x = f16((in_ch, self.T_in), seed + 1)
+
+    def desc(self, device, out_t=None, out_ld=0, skip=0):
+        """(descriptor, keep-alive list). device: pointers into device copies; else host arrays."""
+        d = VaeConvDesc()
+        d.n, d.cap = len(self.items), self.cap
+        alive = []
+        for i, it in enumerate(self.items):
+            e = d.it[i]
+            for f in ("in_len", "out_len", "have", "keep", "in_off", "out_off"):
+                setattr(e, f, it[f])
+            for f, src in (("tail_in", it["tail_in"]), ("tail_out", it["tail_out"]), ("in_ptr", it["own"])):
+                if src is None:
+                    continue
+                if device:
+                    t = to_dev(src)
+                    alive.append((f, i, t))
+                    setattr(e, f, t.data_ptr())
+                else:
+                    setattr(e, f, src.ctypes.data)
+            if out_t is not None:
+                e.out_ptr = (out_t[i].data_ptr() if device else out_t[i].ctypes.data)
+                e.out_ld, e.skip = out_ld, (skip if i == 1 else 0)
+        return d, alive
+
+    def ld_own(self):
+        return self.items[2]["in_len"] + 5
+
+
+@pytest.mark.parametrize("in_ch,out_ch,k,stride", [(1, 32, 7, 1), (32, 64, 4, 2), (64, 48, 10, 5), (24, 70, 3, 1)])
+def test_conv_tail_im2col_and_gemm_form_bit_exact(in_ch, out_ch, k, stride):
+    b = Batch(in_ch, k, stride, 100 + k, own_pointer=False)
+    w, bias = f16((out_ch, in_ch, k), 3, std=(in_ch * k) ** -0.5), f16((out_ch,), 4, std=0.2)
+    # oracle
+    hd, _ = b.desc(False)
+    want = np.full((out_ch, b.T_out), 0x7E00, np.uint16)
+    oracle.vae_conv(hd, b.x, b.T_in, w, bias, want, b.T_out, in_ch, out_ch, k, stride)
+    oracle.vae_tail(hd, b.x, b.T_in, in_ch)
+    want_tails = [it["tail_out"].copy() for it in b.items]
+    # device
+    dd, alive = b.desc(True)
+    d_x, d_w, d_b = to_dev(b.x), to_dev(w), to_dev(bias)
+    d_y = torch.full((out_ch, b.T_out), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_vae_conv_dev(C.addressof(dd), P(d_x), b.T_in, P(d_w), P(d_b), P(d_y), b.T_out, in_ch, out_ch, k, stride,
+                           False, stream()))
+    assert np.array_equal(bits_of(d_y), want)
+    ok(dev.vv_vae_tail_dev(C.addressof(dd), P(d_x), b.T_in, in_ch, stream()))
+    for f, i, t in alive:
+        if f == "tail_out":
+            assert np.array_equal(bits_of(t), want_tails[i])
+    # im2col over a window that starts inside the second item, then the GEMM over it, every tile
+    p0, pc = b.items[1]["out_off"] + 3, b.T_out - b.items[1]["out_off"] - 3
+    ldcol = pc + 6
+    col = np.zeros((in_ch * k, ldcol), np.uint16)
+    oracle.vae_im2col(hd, b.x, b.T_in, in_ch, k, stride, p0, pc, col, ldcol)
+    d_col = torch.zeros((in_ch * k, ldcol), dtype=torch.float16, device="cuda")
+    ok(dev.vv_vae_im2col_dev(C.addressof(dd), P(d_x), b.T_in, in_ch, k, stride, p0, pc, P(d_col), ldcol, stream()))
+    assert np.array_equal(bits_of(d_col), col)
+    for tile in (0, 16, 32, 64):
+        d_g = torch.full((out_ch, b.T_out), float("nan"), dtype=torch.float16, device="cuda")
+        ok(dev.vv_vae_conv_gemm_dev(None, P(d_w), P(d_col), ldcol, P(d_b), d_g.data_ptr() + 2 * p0, b.T_out, out_ch,
+                                    in_ch * k, p0, pc, tile, stream()))
+        assert np.array_equal(bits_of(d_g)[:, p0:], want[:, p0:])
+        assert np.isnan(oracle.widen(bits_of(d_g)[:, :p0])).all()
+    # transposed output (the head): rows [frame][out_ld] per item, the second item skipping two frames
+    out_ld = out_ch + 4
+    host_t = [np.zeros((it["out_len"], out_ld), np.uint16) for it in b.items]
+    hd_t, _ = b.desc(False, host_t, out_ld, 2)
+    oracle.vae_conv(hd_t, b.x, b.T_in, w, bias, None, 0, in_ch, out_ch, k, stride, transposed=True)
+    dev_t = [torch.zeros((it["out_len"], out_ld), dtype=torch.float16, device="cuda") for it in b.items]
+    dd_t, alive_t = b.desc(True, dev_t, out_ld, 2)
+    ok(dev.vv_vae_conv_dev(C.addressof(dd_t), P(d_x), b.T_in, P(d_w), P(d_b), None, 0, in_ch, out_ch, k, stride, True,
+                           stream()))
+    for h, t in zip(host_t, dev_t):
+        assert np.array_equal(bits_of(t), h)
+    for t in dev_t:
+        t.zero_()
+    full_col = torch.zeros((in_ch * k, b.T_out), dtype=torch.float16, device="cuda")
+    ok(dev.vv_vae_im2col_dev(C.addressof(dd_t), P(d_x), b.T_in, in_ch, k, stride, 0, b.T_out, P(full_col), b.T_out,
+                             stream()))
+    ok(dev.vv_vae_conv_gemm_dev(C.addressof(dd_t), P(d_w), P(full_col), b.T_out, P(d_b), None, 0, out_ch, in_ch * k, 0,
+                                b.T_out, 0, stream()))
+    for h, t in zip(host_t, dev_t):
+        assert np.array_equal(bits_of(t), h)
+
+
+def test_conv_reads_an_item_through_its_own_pointer():
+    b = Batch(8, 4, 2, 7, own_pointer=True)
+    w = f16((16, 8, 4), 3, std=0.2)
+    hd, _ = b.desc(False)
+    want = np.zeros((16, b.T_out), np.uint16)
+    oracle.vae_conv(hd, b.x, b.ld_own(), w, None, want, b.T_out, 8, 16, 4, 2)
+    dd, alive = b.desc(True)
+    d_x, d_w = to_dev(b.x), to_dev(w)
+    d_y = torch.zeros((16, b.T_out), dtype=torch.float16, device="cuda")
+    ok(dev.vv_vae_conv_dev(C.addressof(dd), P(d_x), b.ld_own(), P(d_w), None, P(d_y), b.T_out, 8, 16, 4, 2, False,
+                           stream()))
+    own_cols = slice(b.items[2]["out_off"], b.T_out)
+    assert np.array_equal(bits_of(d_y)[:, own_cols], want[:, own_cols])
+
+
+@pytest.mark.parametrize("C_,k", [(32, 7), (70, 7), (128, 16), (8, 1)])
+def test_rms_then_mixer(C_, k):
+    b = Batch(C_, k, 1, 300 + C_, own_pointer=False)
+    T = b.T_in
+    hd, _ = b.desc(False)
+    dd, alive = b.desc(True)
+    d_x = to_dev(b.x)
+    n_r = T + len(b.items) * b.cap
+    d_r = torch.full((n_r,), float("nan"), dtype=torch.float32, device="cuda")
+    ok(dev.vv_vae_rms_dev(P(d_x), T, T, C_, 1e-5, P(d_r), C.addressof(dd), stream()))
+    torch.cuda.synchronize()
+    got_r = d_r.cpu().numpy()
+    want_r = np.full(n_r, np.nan, np.float32)
+    oracle.vae_rms(b.x, T, T, C_, 1e-5, want_r, hd)
+    live = ~np.isnan(want_r)
+    assert np.array_equal(np.isnan(got_r), ~live)                           # slots of absent context stay untouched
+    ulps = np.abs(got_r[live].view(np.int32).astype(np.int64) - want_r[live].view(np.int32).astype(np.int64))
+    assert ulps.max() <= 2
+    # the mixer on the device's own 1/rms: every later step is fixed, so the bits must agree
+    nw, cw, cb, g = f16((C_,), 7, std=0.5), f16((C_, k), 8, std=0.4), f16((C_,), 9, std=0.1), f16((C_,), 10, std=0.3)
+    for gamma, bias in ((g, cb), (None, None)):
+        want = np.zeros_like(b.x)
+        oracle.vae_mixer(hd, b.x, want, T, np.nan_to_num(got_r), T, nw, cw, bias, gamma, C_, k)
+        d_o = torch.zeros((C_, T), dtype=torch.float16, device="cuda")
+        d_nw, d_cw = to_dev(nw), to_dev(cw)                # held: a freed temporary's memory is handed out again
+        d_cb = to_dev(bias) if bias is not None else None
+        d_g = to_dev(gamma) if gamma is not None else None
+        ok(dev.vv_vae_mixer_dev(C.addressof(dd), P(d_x), P(d_o), T, P(d_r), T, P(d_nw), P(d_cw), P(d_cb), P(d_g), C_,
+                                k, stream()))
+        assert np.array_equal(bits_of(d_o), want)
+
+
+def close_to(got_bits, want_bits, what, operands=None, slack=0.0):
+    """`operands`: magnitudes the result was formed from (a sum's terms), when it can be much smaller than they are."""
+    got, want = oracle.widen(got_bits).astype(np.float64), oracle.widen(want_bits).astype(np.float64)
+    assert scaled_rel_err(got, want) <= FP16_TOL, what
+    size = np.maximum(np.abs(want), 2.0 ** -14) if operands is None else np.maximum(np.abs(want), operands)
+    step = np.spacing(size.astype(np.float16)).astype(np.float64)
+    off = np.maximum(np.abs(got - want) - slack, 0.0) / step
+    assert off.max() <= 2.0 and (off > 0).mean() < 0.05, f"{what}: {off.max()} steps, {(off > 0).mean():.4f} differ"
+
+
+@pytest.mark.parametrize("epi", [0, 1, 2])
+@pytest.mark.parametrize("M,K,P_", [(64, 64, 128), (256, 64, 300), (70, 200, 77), (16, 8, 5), (512, 2048, 130)])
+@pytest.mark.parametrize("normalise", [False, True])
+def test_gemm_nn(epi, M, K, P_, normalise):
+    ldb, ldc = P_ + 8, P_ + 3
+    A, B = f16((M, K), 11, std=K ** -0.5), f16((K, ldb), 12)
+    bias, gamma = f16((M,), 13, std=0.3), f16((M,), 14, std=0.5)
+    Cm = f16((M, ldc), 15)
+    rinv = np.random.default_rng(16).uniform(0.5, 1.5, ldb).astype(np.float32) if normalise else None
+    nw = f16((K,), 17, std=0.7) if normalise else None
+    want = Cm.copy()
+    oracle.vae_gemm_nn(epi, A, B, ldb, want, ldc, M, K, P_, bias, gamma, rinv, nw)
+    outs = []
+    d_a, d_b, d_bias, d_g = to_dev(A), to_dev(B), to_dev(bias), to_dev(gamma)
+    d_r = torch.from_numpy(rinv).cuda() if normalise else None
+    d_nw = to_dev(nw) if normalise else None
+    for tile in (0, 64, 128):
+        d_c = to_dev(Cm)
+        ok(dev.vv_vae_gemm_nn_dev(epi, P(d_a), P(d_b), ldb, P(d_c), ldc, M, K, P_, P(d_bias), P(d_g), P(d_r), P(d_nw),
+                                  tile, stream()))
+        outs.append(bits_of(d_c))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    assert np.array_equal(outs[0][:, P_:], Cm[:, P_:])
+    # The unit of error is an FP16 step of the largest value a result was formed from (the sum before the bias, the
+    # bias, for the residual form the old C and v * gamma; gelu(v) itself can be far smaller than v), plus the FP32
+    # accumulation's own error, 1e-5 of sum |a||b|.
+    Af, Bf = oracle.widen(A).astype(np.float64), oracle.widen(B).astype(np.float64)[:, :P_]
+    if normalise:
+        Bf = (Bf * rinv[None, :P_] * oracle.widen(nw).astype(np.float64)[:, None]).astype(np.float16).astype(np.float64)
+    terms = np.maximum(np.abs(Af @ Bf), np.abs(oracle.widen(bias).astype(np.float64))[:, None])
+    if epi == 1:
+        g = np.maximum(1.0, np.abs(oracle.widen(gamma).astype(np.float64)))[:, None]
+        terms = np.maximum(terms * g, np.abs(oracle.widen(Cm[:, :P_]).astype(np.float64)))
+    slack = 1e-5 * (np.abs(Af) @ np.abs(Bf)) * (g if epi == 1 else 1.0)
+    close_to(outs[0][:, :P_], want[:, :P_], f"gemm_nn epilogue {epi}", terms, slack)
+    # one call == two narrower calls, bit for bit
+    if P_ > 40:
+        d_c = to_dev(Cm)
+        cut = 33
+        for c0, pc in ((0, cut), (cut, P_ - cut)):
+            ok(dev.vv_vae_gemm_nn_dev(epi, P(d_a), d_b.data_ptr() + 2 * c0, ldb, d_c.data_ptr() + 2 * c0, ldc, M, K, pc,
+                                      P(d_bias), P(d_g), (d_r.data_ptr() + 4 * c0) if normalise else None, P(d_nw), 0,
+                                      stream()))
+        assert np.array_equal(bits_of(d_c), outs[0])
+
+
+@pytest.mark.parametrize("M,N,K,lda", [(100, 64, 64, 64), (37, 130, 72, 80), (5, 8, 3, 3), (300, 1536, 64, 64)])
+def test_gemm_tn_and_row_scatter(M, N, K, lda):
+    A, B, bias = f16((M, lda), 21, std=K ** -0.5), f16((N, K), 22), f16((N,), 23, std=0.2)
+    want = np.zeros((M, N), np.uint16)
+    oracle.vae_gemm_tn(A, lda, B, want, N, M, N, K, bias)
+    d_a, d_b, d_bias = to_dev(A), to_dev(B), to_dev(bias)
+    d_c = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    ok(dev.vv_vae_gemm_tn_dev(P(d_a), lda, P(d_b), P(d_c), N, M, N, K, P(d_bias), None, stream()))
+    plain = bits_of(d_c)
+    Af, Bf = oracle.widen(A).astype(np.float64)[:, :K], oracle.widen(B).astype(np.float64)
+    terms = np.maximum(np.abs(Af @ Bf.T), np.abs(oracle.widen(bias).astype(np.float64))[None, :])
+    close_to(plain, want, "gemm_tn", terms, 1e-5 * (np.abs(Af) @ np.abs(Bf).T))
+    if M < 20:
+        return
+    # two segments: rows [0, 11) and [11, M), stored, stored truncated, accumulated truncated
+    cut = 11
+    for mode in (1, 2, 3):
+        seg = [torch.full((cut, N + 2), 0.5, dtype=torch.float16, device="cuda"),
+               torch.full((M - cut, N), 0.5, dtype=torch.float16, device="cuda")]
+        rows = VaeRows()
+        rows.mode, rows.n = mode, 2
+        rows.seg[0].row0, rows.seg[0].ld, rows.seg[0].dst = 0, N + 2, seg[0].data_ptr()
+        rows.seg[1].row0, rows.seg[1].ld, rows.seg[1].dst = cut, N, seg[1].data_ptr()
+        ok(dev.vv_vae_gemm_tn_dev(P(d_a), lda, P(d_b), None, 0, M, N, K, P(d_bias), C.addressof(rows), stream()))
+        got = np.concatenate([bits_of(seg[0])[:, :N], bits_of(seg[1])])
+        vals = oracle.widen(plain)
+        if mode == 1:
+            exp = plain
+        elif mode == 2:
+            exp = np.array([oracle.trunc_half(v) for v in vals.ravel()], np.uint16).reshape(M, N)
+        else:
+            exp = np.array([oracle.trunc_half(np.float32(0.5) + v) for v in vals.ravel()], np.uint16).reshape(M, N)
+        assert np.array_equal(got, exp)
+        assert (bits_of(seg[0])[:, N:] == 0x3800).all()              # nothing written past a row's N columns
+
+
+def test_f32_to_f16_and_nn_gemm():
+    x = (np.random.default_rng(1).standard_normal(100003) * 100).astype(np.float32)
+    x[:4] = [1e-8, 65519.9, 65520.0, -1e6]
+    d_o = torch.zeros(100003, dtype=torch.float16, device="cuda")
+    d_x = torch.from_numpy(x).cuda()
+    ok(dev.vv_vae_f32_to_f16_dev(P(d_x), P(d_o), 100003, stream()))
+    assert np.array_equal(bits_of(d_o), oracle.narrow(x))
+    M, K, P_ = 70, 136, 200
+    A, B, Cm = f16((M, K), 2, std=K ** -0.5), f16((K, P_), 3), f16((M, P_), 4)
+    for alpha, beta in ((1.0, 0.0), (0.5, -2.0)):
+        d_c = to_dev(Cm) if beta else torch.full((M, P_), float("nan"), dtype=torch.float16, device="cuda")
+        d_a, d_b = to_dev(A), to_dev(B)
+        ok(dev.vv_gemm_fp16_nn_dev(P(d_a), P(d_b), P(d_c), M, K, P_, alpha, beta, stream()))
+        ref = alpha * (oracle.widen(A).astype(np.float64) @ oracle.widen(B).astype(np.float64)) \
+            + beta * oracle.widen(Cm).astype(np.float64)
+        assert scaled_rel_err(oracle.widen(bits_of(d_c)).astype(np.float64), ref) <= FP16_TOL
+    dev.vv_gemm_cleanup()
+
+
+def test_argument_checks():
+    p = torch.zeros(4096, dtype=torch.float16, device="cuda").data_ptr()
+    d = VaeConvDesc()
+    s = stream()
+    N, I = dev.VV_ERR_NULL_PTR, dev.VV_ERR_INVALID_ARG
+    assert dev.vv_vae_conv_dev(None, p, 8, p, None, p, 8, 1, 1, 1, 1, False, s) == N
+    assert dev.vv_vae_conv_dev(C.addressof(d), p, 8, p, None, p, 8, 1, 1, 1, 1, False, s) == I        # no items
+    d.n = 1
+    assert dev.vv_vae_conv_dev(C.addressof(d), p, 8, p, None, p, 8, 1, 1, 1, 1, False, s) == dev.VV_OK  # empty items
+    assert dev.vv_vae_mixer_dev(C.addressof(d), p, p, 8, p, 8, p, p, None, None, 4, 17, s) == I         # k > 16
+    assert dev.vv_vae_gemm_nn_dev(5, p, p, 8, p, 8, 4, 4, 4, None, None, None, None, 0, s) == I
+    assert dev.vv_vae_gemm_nn_dev(0, p, p, 8, p, 8, 4, 4, 4, None, None, p, None, 0, s) == I            # rinv without norm_w
+    assert dev.vv_vae_gemm_nn_dev(0, p, p, 8, p, 8, 4, 4, 4, None, None, None, None, 32, s) == I        # tile
+    assert dev.vv_vae_conv_gemm_dev(None, p, p, 8, None, None, 8, 4, 4, 0, 4, 0, s) == I                # transposed needs items
+    assert dev.vv_vae_gemm_tn_dev(p, 8, p, None, 8, 4, 4, 4, None, None, s) == N
+    assert dev.vv_vae_f32_to_f16_dev(p, p, 0, s) == dev.VV_OK
+    assert dev.vv_vae_im2col_dev(C.addressof(d), p, 8, 70000, 1, 1, 0, 4, p, 8, s) == I
