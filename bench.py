@@ -413,6 +413,58 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                            scratch.data_ptr(), st), 50)
     gb = 2.0 * T * NK * HD / sec / 1e9
     out["attn_decode_fp8"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+    del q, k_, v_, o, k8, v8
+    # BitNet's integer layers at the 1.5B shape (hidden 1536, FFN 8960, vocabulary 151936): quantise, one decode row
+    # and a 512-row prefill through the ternary gate projection, the int8 tied head.
+    Hb, Fb, Vb, Mb = 1536, 8960, 151936, 512
+    bn = {}
+    xb = torch.randn(Mb, Hb, dtype=torch.float16, device="cuda")
+    qb = torch.empty(Mb, Hb, dtype=torch.int8, device="cuda")
+    sb = torch.empty(Mb, dtype=torch.float32, device="cuda")
+    smb = torch.empty(Mb, dtype=torch.int32, device="cuda")
+    sec = timed(lambda: dev.vv_act_quant_i8_dev(xb.data_ptr(), 1, Mb, Hb, qb.data_ptr(), sb.data_ptr(), smb.data_ptr(), st), 50)
+    bn["act_quant_512x1536_us"] = sec * 1e6
+    codes = torch.randint(0, 3, (Fb, Hb // 4, 4), dtype=torch.uint8, device="cuda")
+    codes = (codes[..., 0] << 6 | codes[..., 1] << 4 | codes[..., 2] << 2 | codes[..., 3]).contiguous()
+    yb = torch.empty(Mb, Fb, dtype=torch.float16, device="cuda")
+    for m in (1, Mb):
+        sec = timed(lambda: dev.vv_ternary_gemm_dev(qb.data_ptr(), smb.data_ptr(), sb.data_ptr(), codes.data_ptr(), 0.02,
+                                                    None, None, yb.data_ptr(), 1, m, Fb, Hb, st), 50)
+        bn[f"ternary_{Fb}x{Hb}_M{m}_us"] = sec * 1e6
+    wh = torch.randint(-127, 128, (Vb, Hb), dtype=torch.int8, device="cuda")
+    wsh = torch.rand(Vb, dtype=torch.float32, device="cuda") * 1e-2
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    scr = torch.empty(dev.vv_i8_head_argmax_scratch_bytes(Vb), dtype=torch.uint8, device="cuda")
+    sec = timed(lambda: dev.vv_i8_head_argmax_dev(qb.data_ptr(), sb.data_ptr(), wh.data_ptr(), wsh.data_ptr(), Vb, Hb,
+                                                  tok.data_ptr(), None, scr.data_ptr(), st), 50)
+    bn["i8_head_argmax_us"] = sec * 1e6
+    bn["i8_head_argmax_GBps"] = (Vb * Hb + 4.0 * Vb) / sec / 1e9
+    out["bitnet"] = bn
+    del xb, qb, sb, smb, codes, yb, wh, wsh, tok, scr
+    # Conv-VAE encoder ops at a deep stage's shape: 512 channels, 24000 packed columns in one item.
+    Cv, Tv, kv = 512, 24000, 7
+    d = dev.VaeConvDesc()
+    d.n, d.cap = 1, kv - 1
+    d.it[0].in_len = d.it[0].out_len = Tv
+    xv = torch.randn(Cv, Tv, dtype=torch.float16, device="cuda")
+    xo = torch.empty_like(xv)
+    rv = torch.empty(Tv, dtype=torch.float32, device="cuda")
+    nwv = torch.randn(Cv, dtype=torch.float16, device="cuda")
+    cwv = torch.randn(Cv, kv, dtype=torch.float16, device="cuda") * 0.3
+    vae = {}
+    sec = timed(lambda: dev.vv_vae_rms_dev(xv.data_ptr(), Tv, Tv, Cv, 1e-5, rv.data_ptr(), None, st), 50)
+    vae["rms_us"] = sec * 1e6
+    sec = timed(lambda: dev.vv_vae_mixer_dev(C.addressof(d), xv.data_ptr(), xo.data_ptr(), Tv, rv.data_ptr(), Tv,
+                                             nwv.data_ptr(), cwv.data_ptr(), None, nwv.data_ptr(), Cv, kv, st), 50)
+    vae["mixer_us"] = sec * 1e6
+    vae["mixer_GBps"] = 4.0 * Cv * Tv / sec / 1e9
+    w1 = torch.randn(4 * Cv, Cv, dtype=torch.float16, device="cuda") * Cv ** -0.5
+    hv = torch.empty(4 * Cv, Tv, dtype=torch.float16, device="cuda")
+    sec = timed(lambda: dev.vv_vae_gemm_nn_dev(0, w1.data_ptr(), xv.data_ptr(), Tv, hv.data_ptr(), Tv, 4 * Cv, Cv, Tv,
+                                               None, None, rv.data_ptr(), nwv.data_ptr(), 0, st), 20)
+    vae["ffn_up_gelu_us"] = sec * 1e6
+    vae["ffn_up_gelu_TFLOPs"] = 2.0 * 4 * Cv * Cv * Tv / sec / 1e12
+    out["vae"] = vae
     return out
 
 
@@ -1053,6 +1105,10 @@ def main() -> int:
         log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
         d = layer["attn_decode_fp8"]
         log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        d = layer["bitnet"]
+        log("  BitNet (1536 / 8960 / 151936): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
+        d = layer["vae"]
+        log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
         layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
         log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention); "
             f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")

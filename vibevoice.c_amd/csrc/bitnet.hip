@@ -8,16 +8,15 @@
 //                 1e-5)) in double, q = the integer that fma(x, s, 1.5 * 2^23)
 //                 carries in its mantissa (the product is never rounded on its
 //                 own), clamped to [-128, 127]; the row sum of q beside it
-//   bn_gemm       sixteen weight rows per workgroup against up to 64 activation
+//   bn_gemm       16 or 32 weight rows per workgroup against 16 or 32 activation
 //                 rows (grid.y walks M), K split over the eight waves, operands
-//                 from global memory straight into v_mfma_i32_16x16x64_i8. A
-//                 32-bit word of I2_S codes IS a lane's operand of one step:
-//                 its four 2-bit planes are the codes of columns j, j + 32,
-//                 j + 64, j + 96 (j = 4 bytes of the 32-byte block), met with
-//                 the four activation words at those columns — the order of
-//                 the 64 columns inside a step is free in integer arithmetic.
-//                 Codes stay 0..2; the row sum of the activations is subtracted
-//                 once at the end: sum (c - 1) q = sum c q - sum q.
+//                 from global memory straight into v_mfma_i32_16x16x64_i8 with
+//                 16-byte loads. Sixteen consecutive columns of a 128-block are
+//                 one bit plane of sixteen consecutive code bytes, so a lane's
+//                 16-byte load of codes gives its operands of both 64-column
+//                 steps of the block by a shift and a mask. Codes stay 0..2; the
+//                 row sum of the activations is subtracted once at the end:
+//                 sum (c - 1) q = sum c q - sum q.
 //   bn_naive      int8 x int8 when K is not a multiple of 16 or an operand is
 //                 off 16 bytes: one thread per output
 //   bn_requant    one scale for a whole tensor, read from device memory
@@ -134,79 +133,98 @@ __device__ __forceinline__ void bn_fold_absmax(float* absmax, float v) {
 
 constexpr int kBnWaves = 8;
 
-template <bool kTern, int kMT>
+// kRG groups of sixteen weight rows against kMT tiles of sixteen activation rows per workgroup; a wave takes every
+// eighth 128-column block (two MFMA steps of 64 columns, a lane's share of a step being 16 consecutive columns).
+template <bool kTern, int kMT, int kRG>
 __global__ __launch_bounds__(kBnWaves * kWave) void bn_gemm(const int8_t* __restrict__ a, const void* __restrict__ w,
                                                             BnOut out, int K) {
-    __shared__ i32x4 part[kBnWaves][kMT][kWave];
+    __shared__ i32x4 part[kBnWaves][kMT * kRG][kWave];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, ks = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16, m0 = (int)blockIdx.y * (16 * kMT);
-    const int kchunks = K / 16, nsteps = (kchunks + 3) / 4;       // a step: 64 columns, four lanes' 16 each
-    const size_t wrow = (size_t)min(n0 + r16, out.N - 1);
-    const int8_t* xrow[kMT];
+    const int n0 = (int)blockIdx.x * (16 * kRG), m0 = (int)blockIdx.y * (16 * kMT);
+    const int kchunks = K / 16, nblocks = (kchunks + 7) / 8;
+    size_t wrow[kRG];
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) xrow[t] = a + (size_t)min(m0 + 16 * t + r16, out.M - 1) * K;
+    for (int g = 0; g < kRG; ++g) wrow[g] = (size_t)min(n0 + 16 * g + r16, out.N - 1);
+    const i32x4* xrow[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; ++t)
+        xrow[t] = reinterpret_cast<const i32x4*>(a + (size_t)min(m0 + 16 * t + r16, out.M - 1) * K);
     const i32x4 zero = {0, 0, 0, 0};
-    i32x4 acc[kMT];
+    i32x4 acc[kMT][kRG];
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) acc[t] = zero;
+    for (int t = 0; t < kMT; ++t)
+#pragma unroll
+        for (int g = 0; g < kRG; ++g) acc[t][g] = zero;
 
-    for (int s0 = wave * 2; s0 < nsteps; s0 += kBnWaves * 2) {
-        i32x4 wv[2], xv[kMT][2];
+    for (int b = wave; b < nblocks; b += kBnWaves) {
+        i32x4 wv[kRG][2], xv[kMT][2];
+        // activations: step s of the block is chunks 4 s .. 4 s + 3, this lane's being 4 s + ks
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int s = s0 + u;
-            if constexpr (kTern) {
-                // step s = half (s & 1) of block s / 2; this lane's word of codes: 4 (s & 1) + ks of the block's eight
-                const bool live = s < nsteps;                       // K % 128 == 0: whole steps only
-                const int word = min(s, nsteps - 1) * 4 + ks;       // (s / 2) * 8 + 4 (s & 1) + ks
-                const uint32_t codes = static_cast<const uint32_t*>(w)[wrow * (size_t)(K / 16) + word];
-                wv[u] = live ? i32x4{(int)((codes >> 6) & 0x03030303u), (int)((codes >> 4) & 0x03030303u),
-                                     (int)((codes >> 2) & 0x03030303u), (int)(codes & 0x03030303u)}
-                             : zero;
-                // the four activation words at columns j, j + 32, j + 64, j + 96 of the block, j = 4 (word % 8)
-                const int first = (word >> 3) * 32 + (word & 7);    // in 32-bit words of the row
+        for (int s = 0; s < 2; ++s) {
+            const int c = b * 8 + 4 * s + ks;
+            const bool live = c < kchunks;
 #pragma unroll
-                for (int t = 0; t < kMT; ++t) {
-                    const int* xr = reinterpret_cast<const int*>(xrow[t]) + first;
-                    xv[t][u] = i32x4{xr[0], xr[8], xr[16], xr[24]};
+            for (int t = 0; t < kMT; ++t) xv[t][s] = live ? xrow[t][live ? c : 0] : zero;
+        }
+        if constexpr (kTern) {
+            // Columns 16 j .. 16 j + 15 of a block (j = 4 s + ks) are bit plane j / 2 = 2 s + ks / 2 of code bytes
+            // 16 (j % 2) .. + 15 = 16 (ks % 2) ..: one 16-byte load of codes serves both steps (K % 128 == 0).
+#pragma unroll
+            for (int g = 0; g < kRG; ++g) {
+                const i32x4 codes = __builtin_nontemporal_load(
+                    reinterpret_cast<const i32x4*>(static_cast<const uint8_t*>(w) + wrow[g] * (size_t)(K / 4)) + b * 2 +
+                    (ks & 1));
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int shift = 6 - 2 * (2 * s + (ks >> 1));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) wv[g][s][e] = (int)(((uint32_t)codes[e] >> shift) & 0x03030303u);
                 }
-            } else {
-                const int c = s * 4 + ks;
-                const bool live = c < kchunks;
-                const int cc = live ? c : 0;
-                wv[u] = live ? __builtin_nontemporal_load(
-                                   reinterpret_cast<const i32x4*>(static_cast<const int8_t*>(w) + wrow * K) + cc)
-                             : zero;
-#pragma unroll
-                for (int t = 0; t < kMT; ++t) xv[t][u] = live ? reinterpret_cast<const i32x4*>(xrow[t])[cc] : zero;
             }
+        } else {
+#pragma unroll
+            for (int g = 0; g < kRG; ++g)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int c = b * 8 + 4 * s + ks;
+                    const bool live = c < kchunks;
+                    wv[g][s] = live ? __builtin_nontemporal_load(
+                                          reinterpret_cast<const i32x4*>(static_cast<const int8_t*>(w) + wrow[g] * K) +
+                                          (live ? c : 0))
+                                    : zero;
+                }
         }
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
             for (int t = 0; t < kMT; ++t)
-                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u], xv[t][u], acc[t], 0, 0, 0);
+#pragma unroll
+                for (int g = 0; g < kRG; ++g)
+                    acc[t][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[g][s], xv[t][s], acc[t][g], 0, 0, 0);
     }
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    for (int t = 0; t < kMT; ++t)
+#pragma unroll
+        for (int g = 0; g < kRG; ++g) part[wave][t * kRG + g][lane] = acc[t][g];
     __syncthreads();
 
-    // register r of lane l: column n0 + 4 (l / 16) + r of row m0 + 16 t + l % 16
+    // register r of lane l: column n0 + 16 g + 4 (l / 16) + r of row m0 + 16 t + l % 16
     float amax = 0.0f;
-    if (tid < kMT * kWave) {
-        const int t = tid >> 6;
-        i32x4 sum = part[0][t][lane];
+    constexpr int kTiles = kMT * kRG;
+    for (int tile = wave; tile < kTiles; tile += kBnWaves) {
+        i32x4 sum = part[0][tile][lane];
 #pragma unroll
-        for (int p = 1; p < kBnWaves; ++p) sum += part[p][t][lane];
-        const int m = m0 + 16 * t + r16, n = n0 + 4 * ks;
+        for (int p = 1; p < kBnWaves; ++p) sum += part[p][tile][lane];
+        const int t = tile / kRG, g = tile % kRG;
+        const int m = m0 + 16 * t + r16, n = n0 + 16 * g + 4 * ks;
         if (m < out.M) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 if (n + r < out.N) amax = fmaxf(amax, bn_finish(out, m, n + r, sum[r]));
         }
     }
-    if (!kTern && out.absmax && out.y && tid < kMT * kWave) bn_fold_absmax(out.absmax, amax);
+    if (!kTern && out.absmax && out.y && wave < kTiles) bn_fold_absmax(out.absmax, amax);
 }
 
 __global__ __launch_bounds__(kBlock) void bn_naive(const int8_t* __restrict__ a, const int8_t* __restrict__ w, BnOut out,
@@ -227,13 +245,14 @@ __global__ __launch_bounds__(kBlock) void bn_naive(const int8_t* __restrict__ a,
 
 template <bool kTern>
 void launch_bn_gemm(const int8_t* a, const void* w, const BnOut& out, int K, hipStream_t st) {
-    const int mt = out.M <= 16 ? 1 : out.M <= 32 ? 2 : out.M <= 48 ? 3 : 4;
-    const dim3 grid((unsigned)((out.N + 15) / 16), (unsigned)((out.M + 16 * mt - 1) / (16 * mt)));
     constexpr int kThreads = kBnWaves * kWave;
-    if (mt == 1) bn_gemm<kTern, 1><<<grid, kThreads, 0, st>>>(a, w, out, K);
-    else if (mt == 2) bn_gemm<kTern, 2><<<grid, kThreads, 0, st>>>(a, w, out, K);
-    else if (mt == 3) bn_gemm<kTern, 3><<<grid, kThreads, 0, st>>>(a, w, out, K);
-    else bn_gemm<kTern, 4><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    if (out.M <= 16) {          // decode and a few rows: sixteen weight rows per workgroup, the most workgroups
+        const dim3 grid((unsigned)((out.N + 15) / 16), 1);
+        bn_gemm<kTern, 1, 1><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    } else {                    // 32 x 32 outputs per workgroup: each operand register feeds two products
+        const dim3 grid((unsigned)((out.N + 31) / 32), (unsigned)((out.M + 31) / 32));
+        bn_gemm<kTern, 2, 2><<<grid, kThreads, 0, st>>>(a, w, out, K);
+    }
 }
 
 // ── requantisation ──────────────────────────────────────────────────────────
@@ -354,7 +373,7 @@ vv_status_t vv_ternary_gemm_dev(const int8_t* q, const int32_t* xsum, const floa
     if (!q || !xsum || !codes) return VV_ERR_NULL_PTR;
     if (y && !x_scale) return VV_ERR_NULL_PTR;
     if (M <= 0 || N <= 0 || K <= 0 || K % 128) return VV_ERR_INVALID_ARG;
-    if ((reinterpret_cast<uintptr_t>(q) & 3u) || (reinterpret_cast<uintptr_t>(codes) & 3u)) return VV_ERR_UNSUPPORTED;
+    if (!vv::aligned16(q) || !vv::aligned16(codes)) return VV_ERR_UNSUPPORTED;      // 16-byte operand loads
     vv::BnOut out = {};
     out.xsum = xsum;
     out.x_scale = x_scale;
