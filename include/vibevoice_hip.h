@@ -366,8 +366,8 @@ vv_status_t vv_vae_conv_gemm_dev(const vv_vae_conv_desc_t* d, const void* w, con
                                  void* stream);
 /* C[M,P] (stride ldc) from A[M,K] x B[K,P] (stride ldb) on the matrix cores,
  * FP32 accumulation in K order; rinv and norm_w (both or neither) normalise B
- * on its way in: half(B[k][p] * rinv[p] * norm_w[k]). `tile` (0, 64, 128)
- * changes no bit. replaces device.h:835-839 (vae_kernels.cu:394-607, 868-905). */
+ * on its way in: half(B[k][p] * rinv[p] * norm_w[k]). `tile`: 64 or 128 (the
+ * workgroup's output tile edge) or 0 to choose by the grid; it changes no bit. replaces device.h:835-839 (vae_kernels.cu:394-607, 868-905). */
 vv_status_t vv_vae_gemm_nn_dev(int epilogue, const void* A, const void* B, int64_t ldb, void* C,
                                int64_t ldc, int M, int K, int P, const void* bias,
                                const void* gamma, const float* rinv, const void* norm_w,

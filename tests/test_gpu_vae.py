@@ -2,7 +2,7 @@
 whose arithmetic the interface fixes operation by operation (the convolutions
 and their GEMM form, the context copy, im2col, the fused mixer given the same
 1/rms, the conversions) is held to bit equality with the oracle; the 1/rms
-itself to 2 FP32 ulps (hardware reciprocal square root); the matrix-core GEMMs,
+itself to 16 FP32 ulps (eight partial sums, hardware reciprocal square root); the matrix-core GEMMs,
 whose FP32 sums run in the hardware's order, to the FP16 bar (scaled error
 <= 2e-3) with at most a stray FP16 step against the oracle's double sums."""
 import ctypes as C
@@ -167,7 +167,7 @@ def test_rms_then_mixer(C_, k):
     live = ~np.isnan(want_r)
     assert np.array_equal(np.isnan(got_r), ~live)                           # slots of absent context stay untouched
     ulps = np.abs(got_r[live].view(np.int32).astype(np.int64) - want_r[live].view(np.int32).astype(np.int64))
-    assert ulps.max() <= 2
+    assert ulps.max() <= 16            # eight partial sums and a hardware reciprocal square root against one chain
     # the mixer on the device's own 1/rms: every later step is fixed, so the bits must agree
     nw, cw, cb, g = f16((C_,), 7, std=0.5), f16((C_, k), 8, std=0.4), f16((C_,), 9, std=0.1), f16((C_,), 10, std=0.3)
     for gamma, bias in ((g, cb), (None, None)):
@@ -194,9 +194,10 @@ def close_to(got_bits, want_bits, what, operands=None, slack=0.0):
 
 @pytest.mark.parametrize("epi", [0, 1, 2])
 @pytest.mark.parametrize("M,K,P_", [(64, 64, 128), (256, 64, 300), (70, 200, 77), (16, 8, 5), (512, 2048, 130)])
-@pytest.mark.parametrize("normalise", [False, True])
-def test_gemm_nn(epi, M, K, P_, normalise):
-    ldb, ldc = P_ + 8, P_ + 3
+@pytest.mark.parametrize("normalise,aligned_c", [(False, False), (True, False), (True, True)])
+def test_gemm_nn(epi, M, K, P_, normalise, aligned_c):
+    # rows of C on 16-byte boundaries let whole tiles leave through LDS as 16-byte stores; others store element-wise
+    ldb, ldc = P_ + 8, ((P_ + 15) // 8 * 8 if aligned_c else P_ + 3)
     A, B = f16((M, K), 11, std=K ** -0.5), f16((K, ldb), 12)
     bias, gamma = f16((M,), 13, std=0.3), f16((M,), 14, std=0.5)
     Cm = f16((M, ldc), 15)
@@ -283,7 +284,7 @@ def test_f32_to_f16_and_nn_gemm():
     assert np.array_equal(bits_of(d_o), oracle.narrow(x))
     M, K, P_ = 70, 136, 200
     A, B, Cm = f16((M, K), 2, std=K ** -0.5), f16((K, P_), 3), f16((M, P_), 4)
-    for alpha, beta in ((1.0, 0.0), (0.5, -2.0)):
+    for alpha, beta in ((1.0, 0.0), (0.5, -2.0)):             # P_ = 200: three whole tiles and a ragged one per row
         d_c = to_dev(Cm) if beta else torch.full((M, P_), float("nan"), dtype=torch.float16, device="cuda")
         d_a, d_b = to_dev(A), to_dev(B)
         ok(dev.vv_gemm_fp16_nn_dev(P(d_a), P(d_b), P(d_c), M, K, P_, alpha, beta, stream()))

@@ -16,10 +16,11 @@
 //   vae_rms        1 / rms over channels per column (packed and context)
 //   vae_mixer      RMSNorm -> depthwise conv -> gamma residual, fused
 //   vae_gemm       the FFN (A x B, B K-major) and connector (A x B^T) GEMMs on
-//                  v_mfma_f32_16x16x32_f16: 64x64 tile, four waves of 32x32,
+//                  v_mfma_f32_16x16x32_f16: 128x128 or 64x64 tile, four waves,
 //                  64 K per LDS stage; a K-major B is transposed on its way
 //                  into LDS (and RMS-normalised there when asked); epilogues
-//                  bias+GELU, bias+gamma-residual, bias, bias+row scatter
+//                  bias+GELU, bias+gamma-residual, bias, bias+row scatter; whole
+//                  tiles leave through LDS as 16-byte stores
 #include "vv_common.hpp"
 
 namespace vv {
@@ -170,30 +171,48 @@ __global__ __launch_bounds__(kBlock) void vae_conv_gemm(const h16* __restrict__ 
     }
 }
 
-__global__ __launch_bounds__(128) void vae_rms(const h16* __restrict__ x, int64_t ld, int64_t T, int C, float eps,
-                                               float* __restrict__ rinv, Desc d) {
-    const int64_t i = (int64_t)blockIdx.x * 128 + threadIdx.x;
-    const h16* col;
-    int64_t stride;
+// 32 columns x 8 channel ranges per workgroup: a thread adds the squares of its range in channel order, the eight
+// partial sums are added in one fixed tree, so a column's value does not depend on where it sits.
+constexpr int kRmsCols = 32, kRmsSplit = 8;
+
+__global__ __launch_bounds__(kRmsCols * kRmsSplit) void vae_rms(const h16* __restrict__ x, int64_t ld, int64_t T, int C,
+                                                                float eps, float* __restrict__ rinv, Desc d) {
+    __shared__ float part[kRmsSplit][kRmsCols];
+    const int lane_col = (int)threadIdx.x % kRmsCols, range = (int)threadIdx.x / kRmsCols;
+    const int64_t i = (int64_t)blockIdx.x * kRmsCols + lane_col;
+    const h16* col = nullptr;
+    int64_t stride = 0;
     if (i < T) {
         col = x + i;
         stride = ld;
-    } else {
+    } else if (d.cap > 0) {
         const int64_t j = i - T;
-        if (d.cap <= 0) return;
         const int item = (int)(j / d.cap), q = (int)(j - (int64_t)item * d.cap);
-        if (item >= d.n) return;
-        const Item& it = d.it[item];
-        if (!it.tail_in || q >= it.have) return;
-        col = static_cast<const h16*>(it.tail_in) + q;
-        stride = d.cap;
+        if (item < d.n) {
+            const Item& it = d.it[item];
+            if (it.tail_in && q < it.have) {
+                col = static_cast<const h16*>(it.tail_in) + q;
+                stride = d.cap;
+            }
+        }
     }
+    const int per = (C + kRmsSplit - 1) / kRmsSplit;
+    const int c0 = range * per, c1 = min(C, c0 + per);
     float sum_sq = 0.0f;
-    for (int c = 0; c < C; ++c) {
-        const float v = (float)col[(size_t)c * stride];
-        sum_sq = __builtin_fmaf(v, v, sum_sq);
+    if (col) {
+#pragma unroll 8
+        for (int c = c0; c < c1; ++c) {
+            const float v = (float)col[(size_t)c * stride];
+            sum_sq = __builtin_fmaf(v, v, sum_sq);
+        }
     }
-    rinv[i] = __builtin_amdgcn_rsqf(sum_sq / (float)C + eps);
+    part[range][lane_col] = sum_sq;
+    __syncthreads();
+    if (range == 0 && col) {
+        const float total = ((part[0][lane_col] + part[1][lane_col]) + (part[2][lane_col] + part[3][lane_col])) +
+                            ((part[4][lane_col] + part[5][lane_col]) + (part[6][lane_col] + part[7][lane_col]));
+        rinv[i] = __builtin_amdgcn_rsqf(total / (float)C + eps);
+    }
 }
 
 constexpr int kMixT = 64, kMixC = 32, kMixMaxK = 16;
@@ -275,6 +294,24 @@ __device__ __forceinline__ h16 trunc_half(float f) {
     return __builtin_bit_cast(h16, h);
 }
 
+// The value of C[r][.] from its accumulated product and, for the forms that add to C, its old value.
+template <int kEpi>
+__device__ __forceinline__ h16 gemm_value(const GemmOut& o, float acc, int r, h16 old) {
+    if constexpr (kEpi == kEpiAlphaBeta) {
+        float v = o.alpha * acc;
+        if (o.beta != 0.0f) v = __builtin_fmaf(o.beta, (float)old, v);
+        return to_half(v);
+    } else if constexpr (kEpi == kEpiBias) {
+        return to_half(acc + (o.bias ? (float)o.bias[r] : 0.0f));
+    } else {
+        float v = (float)to_half(acc);
+        if (o.bias) v = (float)to_half(v + (float)o.bias[r]);
+        if constexpr (kEpi == kEpiBiasGelu) return to_half(vae_gelu(v));
+        const float xv = (float)old;
+        return o.gamma ? to_half(__builtin_fmaf(v, (float)o.gamma[r], xv)) : to_half(xv + v);
+    }
+}
+
 template <int kEpi>
 __device__ __forceinline__ void gemm_finish(const GemmOut& o, float acc, int r, int c) {
     if constexpr (kEpi == kEpiRows) {
@@ -293,125 +330,219 @@ __device__ __forceinline__ void gemm_finish(const GemmOut& o, float acc, int r, 
         return;
     }
     const size_t off = (size_t)r * o.ldc + c;
-    if constexpr (kEpi == kEpiAlphaBeta) {
-        float v = o.alpha * acc;
-        if (o.beta != 0.0f) v = __builtin_fmaf(o.beta, (float)o.c[off], v);
-        o.c[off] = to_half(v);
-    } else if constexpr (kEpi == kEpiBias) {
-        o.c[off] = to_half(acc + (o.bias ? (float)o.bias[r] : 0.0f));
-    } else {
-        float v = (float)to_half(acc);
-        if (o.bias) v = (float)to_half(v + (float)o.bias[r]);
-        if constexpr (kEpi == kEpiBiasGelu) {
-            o.c[off] = to_half(vae_gelu(v));
-        } else {
-            const float xv = (float)o.c[off];
-            o.c[off] = o.gamma ? to_half(__builtin_fmaf(v, (float)o.gamma[r], xv)) : to_half(xv + v);
-        }
-    }
+    const bool reads = kEpi == kEpiBiasResid || (kEpi == kEpiAlphaBeta && o.beta != 0.0f);
+    o.c[off] = gemm_value<kEpi>(o, acc, r, reads ? o.c[off] : (h16)0.0f);
 }
 
-constexpr int kGT = 64;          // output tile edge
 constexpr int kGK = 64;          // K per LDS stage: two MFMA steps
 constexpr int kGLd = kGK + 8;    // LDS row stride in halves: 144 bytes, 16-byte aligned, rows on different banks
 
-// C[M][P] = A[M][K] (row stride lda) x B, B either [P][K] (kNN false, row stride
-// ldb) or [K][P] (kNN true, row stride ldb; optionally RMS-normalised while staged).
-template <bool kNN, int kEpi>
+// C[M][P] = A[M][K] (row stride lda) x B, B either [P][K] (kNN false, row stride ldb) or [K][P] (kNN true, row
+// stride ldb; optionally RMS-normalised while staged). kT x kT outputs per workgroup (64 or 128), four waves of
+// kT/2 x kT/2. Every output adds its K products 32 at a time in K order whatever the tile, so the tile changes no bit.
+template <bool kNN, int kEpi, int kT>
 __global__ __launch_bounds__(kBlock) void vae_gemm(const h16* __restrict__ A, int64_t lda, const h16* __restrict__ B,
                                                    int64_t ldb, int M, int K, int P, const float* __restrict__ rinv,
                                                    const h16* __restrict__ nw, GemmOut out) {
-    __shared__ __attribute__((aligned(16))) h16 As[kGT][kGLd];
-    __shared__ __attribute__((aligned(16))) h16 Bs[kGT][kGLd];
+    constexpr int kF = kT / 32;                 // 16x16 MFMA tiles per wave along each side
+    constexpr int kCLd = kT + 8;                // row stride of the result tile
+    static_assert(2 * kT * kGLd >= kT * kCLd, "the result tile fits over the operand stages");
+    __shared__ __attribute__((aligned(16))) h16 lds[2 * kT * kGLd];
+    h16 (*As)[kGLd] = reinterpret_cast<h16 (*)[kGLd]>(lds);
+    h16 (*Bs)[kGLd] = reinterpret_cast<h16 (*)[kGLd]>(lds + kT * kGLd);
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int row_base = (int)blockIdx.y * kGT, col_base = (int)blockIdx.x * kGT;
+    const int row_base = (int)blockIdx.y * kT, col_base = (int)blockIdx.x * kT;
     const bool a_vec = (lda & 7) == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0;
     const bool b_vec = (ldb & 7) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
 
-    f32x4 acc[2][2];
+    f32x4 acc[kF][kF];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < kF; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // K-contiguous rows of `src` (row stride ld) into dst[row][k]: 64 rows x 8 chunks of 8, two per thread.
-    auto stage_rows = [&](const h16* src, int64_t ld, bool vec, int base, int limit, int k0, h16 (*dst)[kGLd]) {
+    // Staging is split in two so that the next stage's global loads are in flight while this stage multiplies:
+    // fetch_* bring a stage's chunks into registers, put_* write them to LDS after the products of the stage before.
+    constexpr int kRowChunks = kT * 8 / kBlock;          // chunks per thread of a K-contiguous operand's stage
+    constexpr int kHalves = kT / 64;
+    // K-contiguous rows of `src` (row stride ld): kT rows x 8 chunks of 8.
+    auto fetch_rows = [&](const h16* src, int64_t ld, bool vec, int base, int limit, int k0, h16x8 (&reg)[kRowChunks]) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < kRowChunks; ++u) {
             const int e = tid + u * kBlock;
             const int r = e >> 3, c = (e & 7) * 8;
             const int gr = base + r;
-            h16x8 v;
             if (vec && gr < limit && k0 + c + 8 <= K) {
-                v = *reinterpret_cast<const h16x8*>(src + (size_t)gr * ld + k0 + c);
+                reg[u] = *reinterpret_cast<const h16x8*>(src + (size_t)gr * ld + k0 + c);
             } else {
 #pragma unroll
                 for (int t = 0; t < 8; ++t)
-                    v[t] = (gr < limit && k0 + c + t < K) ? src[(size_t)gr * ld + k0 + c + t] : (h16)0.0f;
+                    reg[u][t] = (gr < limit && k0 + c + t < K) ? src[(size_t)gr * ld + k0 + c + t] : (h16)0.0f;
             }
-            *reinterpret_cast<h16x8*>(&dst[r][c]) = v;
         }
     };
-    // K-major B: 64 K rows x 8 chunks of 8 columns, two per thread, transposed into Bs[column][k].
-    auto stage_kmajor = [&](int k0) {
+    auto put_rows = [&](const h16x8 (&reg)[kRowChunks], h16 (*dst)[kGLd]) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < kRowChunks; ++u) {
             const int e = tid + u * kBlock;
-            const int kr = e >> 3, c = (e & 7) * 8;
-            const int gk = k0 + kr, gc = col_base + c;
-            h16x8 v;
-            if (b_vec && gk < K && gc + 8 <= P) {
-                v = *reinterpret_cast<const h16x8*>(B + (size_t)gk * ldb + gc);
-            } else {
+            *reinterpret_cast<h16x8*>(&dst[e >> 3][(e & 7) * 8]) = reg[u];
+        }
+    };
+    // K-major B: thread (kg, c) takes K rows 2 kg, 2 kg + 1 of the stage and columns 8 c .. 8 c + 7 (of every 64),
+    // and writes the eight (k, k + 1) pairs into Bs[column][k]. The 16-byte K groups of a Bs row are XOR-ed with
+    // the column's (column / 8) % 8, which spreads a wave's 64 pair writes over all 64 banks.
+    const int kg = tid >> 3;
+    float col_rinv[kHalves][8];                          // 1 / rms of this thread's columns: the same for every stage
+    if constexpr (kNN) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = (gk < K && gc + t < P) ? B[(size_t)gk * ldb + gc + t] : (h16)0.0f;
+        for (int half = 0; half < kHalves; ++half)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int gc = col_base + half * 64 + (tid & 7) * 8 + t;
+                col_rinv[half][t] = (nw && gc < P) ? rinv[gc] : 0.0f;
             }
+    }
+    auto fetch_kmajor = [&](int k0, h16x8 (&reg)[kHalves][2]) {
+#pragma unroll
+        for (int half = 0; half < kHalves; ++half) {
+            const int gc = col_base + half * 64 + (tid & 7) * 8;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int gk = k0 + 2 * kg + u;
+                if (b_vec && gk < K && gc + 8 <= P) {
+                    reg[half][u] = *reinterpret_cast<const h16x8*>(B + (size_t)gk * ldb + gc);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        reg[half][u][t] = (gk < K && gc + t < P) ? B[(size_t)gk * ldb + gc + t] : (h16)0.0f;
+                }
+            }
+        }
+    };
+    auto put_kmajor = [&](int k0, h16x8 (&reg)[kHalves][2]) {
+        const int at = (((kg >> 2) ^ (tid & 7)) << 3) + 2 * (kg & 3);       // (column / 8) % 8 == tid & 7 for all of them
+#pragma unroll
+        for (int half = 0; half < kHalves; ++half) {
+            const int c = half * 64 + (tid & 7) * 8;
             if (nw) {
-                const float wn_k = gk < K ? (float)nw[gk] : 0.0f;
 #pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    if (gk < K && gc + t < P) v[t] = to_half(((float)v[t] * rinv[gc + t]) * wn_k);
+                for (int u = 0; u < 2; ++u) {
+                    const int gk = k0 + 2 * kg + u;
+                    const float wn_k = gk < K ? (float)nw[gk] : 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)        // zero operands (past K or P) stay zero: 0 * x * 0
+                        reg[half][u][t] = to_half(((float)reg[half][u][t] * col_rinv[half][t]) * wn_k);
+                }
             }
 #pragma unroll
-            for (int t = 0; t < 8; ++t) Bs[c + t][kr] = v[t];
+            for (int t = 0; t < 8; ++t) {
+                const h16x2 pair = {reg[half][0][t], reg[half][1][t]};
+                *reinterpret_cast<h16x2*>(&Bs[c + t][at]) = pair;
+            }
         }
     };
 
+    h16x8 ra[kRowChunks], rb_rows[kNN ? 1 : kRowChunks], rb_k[kNN ? kHalves : 1][2];
+    fetch_rows(A, lda, a_vec, row_base, M, 0, ra);
+    if constexpr (kNN) fetch_kmajor(0, rb_k);
+    else fetch_rows(B, ldb, b_vec, col_base, P, 0, rb_rows);
     for (int k0 = 0; k0 < K; k0 += kGK) {
-        stage_rows(A, lda, a_vec, row_base, M, k0, As);
-        if constexpr (kNN) stage_kmajor(k0);
-        else stage_rows(B, ldb, b_vec, col_base, P, k0, Bs);
+        put_rows(ra, As);
+        if constexpr (kNN) put_kmajor(k0, rb_k);
+        else put_rows(rb_rows, Bs);
         __syncthreads();
+        if (k0 + kGK < K) {
+            fetch_rows(A, lda, a_vec, row_base, M, k0 + kGK, ra);
+            if constexpr (kNN) fetch_kmajor(k0 + kGK, rb_k);
+            else fetch_rows(B, ldb, b_vec, col_base, P, k0 + kGK, rb_rows);
+        }
 #pragma unroll
         for (int ks = 0; ks < kGK / 32; ++ks) {
-            h16x8 af[2], bf[2];
+            h16x8 af[kF], bf[kF];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                af[i] = *reinterpret_cast<const h16x8*>(&As[wm * 32 + i * 16 + r16][ks * 32 + kq * 8]);
+            for (int i = 0; i < kF; ++i)
+                af[i] = *reinterpret_cast<const h16x8*>(&As[wm * (kT / 2) + i * 16 + r16][ks * 32 + kq * 8]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                bf[j] = *reinterpret_cast<const h16x8*>(&Bs[wn * 32 + j * 16 + r16][ks * 32 + kq * 8]);
+            for (int j = 0; j < kF; ++j) {
+                const int col = wn * (kT / 2) + j * 16 + r16;
+                const int group = kNN ? ((ks * 4 + kq) ^ ((col >> 3) & 7)) : ks * 4 + kq;
+                bf[j] = *reinterpret_cast<const h16x8*>(&Bs[col][group * 8]);
+            }
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < kF; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < kF; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
     // register r of lane l: row 4 (l / 16) + r of the A tile, column l % 16 of the B tile
+    bool through_lds = false;
+    if constexpr (kEpi != kEpiRows)
+        through_lds = row_base + kT <= M && col_base + kT <= P && (out.ldc & 7) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out.c) & 15u) == 0;
+    if (through_lds) {
+        // A whole tile whose rows are 16-byte aligned: the results meet in LDS (over the operand stages, free after
+        // the loop's last barrier) and leave as 16-byte stores; the forms that add to C bring the old tile in the same way.
+        h16 (*Ct)[kCLd] = reinterpret_cast<h16 (*)[kCLd]>(lds);
+        h16* cbase = out.c + (size_t)row_base * out.ldc + col_base;
+        const bool reads = kEpi == kEpiBiasResid || (kEpi == kEpiAlphaBeta && out.beta != 0.0f);
+        constexpr int kChunksPerRow = kT / 8;
+        if (reads) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+            for (int u = 0; u < kT * kChunksPerRow / kBlock; ++u) {
+                const int e = tid + u * kBlock;
+                const int r = e / kChunksPerRow, c = (e % kChunksPerRow) * 8;
+                *reinterpret_cast<h16x8*>(&Ct[r][c]) = *reinterpret_cast<const h16x8*>(cbase + (size_t)r * out.ldc + c);
+            }
+            __syncthreads();
+        }
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int i = 0; i < kF; ++i)
+#pragma unroll
+            for (int j = 0; j < kF; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int lr = wm * (kT / 2) + i * 16 + 4 * kq + r, lc = wn * (kT / 2) + j * 16 + r16;
+                    if constexpr (kEpi != kEpiRows)
+                        Ct[lr][lc] = gemm_value<kEpi>(out, acc[i][j][r], row_base + lr, reads ? Ct[lr][lc] : (h16)0.0f);
+                }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kT * kChunksPerRow / kBlock; ++u) {
+            const int e = tid + u * kBlock;
+            const int r = e / kChunksPerRow, c = (e % kChunksPerRow) * 8;
+            *reinterpret_cast<h16x8*>(cbase + (size_t)r * out.ldc + c) = *reinterpret_cast<const h16x8*>(&Ct[r][c]);
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < kF; ++i)
+#pragma unroll
+        for (int j = 0; j < kF; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int row = row_base + wm * 32 + i * 16 + 4 * kq + r;
-                const int col = col_base + wn * 32 + j * 16 + r16;
+                const int row = row_base + wm * (kT / 2) + i * 16 + 4 * kq + r;
+                const int col = col_base + wn * (kT / 2) + j * 16 + r16;
                 if (row < M && col < P) gemm_finish<kEpi>(out, acc[i][j][r], row, col);
             }
+}
+
+// The 128 tile halves the operand bytes a product pulls through L2; the 64 tile keeps small problems on enough
+// workgroups. Either gives the same bits.
+template <bool kNN, int kEpi>
+void launch_vae_gemm(const h16* A, int64_t lda, const h16* B, int64_t ldb, int M, int K, int P, const float* rinv,
+                     const h16* nw, const GemmOut& out, hipStream_t st, int tile = 0) {
+    const long big = (long)((M + 127) / 128) * ((P + 127) / 128);
+    if (tile == 128 || (tile == 0 && M >= 128 && P >= 128 && big >= 512)) {
+        const dim3 grid((unsigned)((P + 127) / 128), (unsigned)((M + 127) / 128));
+        vae_gemm<kNN, kEpi, 128><<<grid, kBlock, 0, st>>>(A, lda, B, ldb, M, K, P, rinv, nw, out);
+    } else {
+        const dim3 grid((unsigned)((P + 63) / 64), (unsigned)((M + 63) / 64));
+        vae_gemm<kNN, kEpi, 64><<<grid, kBlock, 0, st>>>(A, lda, B, ldb, M, K, P, rinv, nw, out);
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void vae_f32_to_f16(const float* __restrict__ in, h16* __restrict__ out, int64_t n) {
@@ -427,8 +558,6 @@ int desc_max(const Desc* d, bool out) {
     }
     return m;
 }
-
-inline dim3 gemm_grid(int M, int P) { return dim3((unsigned)((P + kGT - 1) / kGT), (unsigned)((M + kGT - 1) / kGT)); }
 
 }  // namespace
 }  // namespace vv
@@ -475,9 +604,9 @@ vv_status_t vv_vae_rms_dev(const void* x, int64_t ld, int64_t T, int C, float ep
     const vv_vae_conv_desc_t* dd = d ? d : &none;
     const int64_t n = (T > 0 ? T : 0) + (int64_t)(dd->n > 0 ? dd->n : 0) * (dd->cap > 0 ? dd->cap : 0);
     if (n <= 0) return VV_OK;
-    const int64_t blocks = (n + 127) / 128;
+    const int64_t blocks = (n + vv::kRmsCols - 1) / vv::kRmsCols;
     if (blocks > 0x7FFFFFFF) return VV_ERR_UNSUPPORTED;
-    vv::vae_rms<<<dim3((unsigned)blocks), 128, 0, vv::as_stream(stream)>>>(static_cast<const vv::h16*>(x), ld,
+    vv::vae_rms<<<dim3((unsigned)blocks), vv::kRmsCols * vv::kRmsSplit, 0, vv::as_stream(stream)>>>(static_cast<const vv::h16*>(x), ld,
                                                                           T > 0 ? T : 0, C, eps, rinv, *dd);
     return vv::launch_status();
 }
@@ -546,14 +675,13 @@ vv_status_t vv_vae_gemm_nn_dev(int epilogue, const void* A, const void* B, int64
     out.bias = static_cast<H>(bias);
     out.gamma = static_cast<H>(gamma);
     hipStream_t st = vv::as_stream(stream);
-    const dim3 grid = vv::gemm_grid(M, P);
     H a = static_cast<H>(A), b = static_cast<H>(B), nw = static_cast<H>(norm_w);
     if (epilogue == VV_VAE_EPI_BIAS_GELU)
-        vv::vae_gemm<true, vv::kEpiBiasGelu><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+        vv::launch_vae_gemm<true, vv::kEpiBiasGelu>(a, K, b, ldb, M, K, P, rinv, nw, out, st, tile);
     else if (epilogue == VV_VAE_EPI_BIAS_RESID)
-        vv::vae_gemm<true, vv::kEpiBiasResid><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+        vv::launch_vae_gemm<true, vv::kEpiBiasResid>(a, K, b, ldb, M, K, P, rinv, nw, out, st, tile);
     else if (epilogue == VV_VAE_EPI_BIAS)
-        vv::vae_gemm<true, vv::kEpiBias><<<grid, vv::kBlock, 0, st>>>(a, K, b, ldb, M, K, P, rinv, nw, out);
+        vv::launch_vae_gemm<true, vv::kEpiBias>(a, K, b, ldb, M, K, P, rinv, nw, out, st, tile);
     else
         return VV_ERR_INVALID_ARG;
     return vv::launch_status();
@@ -574,8 +702,8 @@ vv_status_t vv_vae_gemm_tn_dev(const void* A, int64_t lda, const void* B, void* 
     out.c = static_cast<vv::h16*>(C);
     out.ldc = ldc;
     out.bias = static_cast<const vv::h16*>(bias);
-    vv::vae_gemm<false, vv::kEpiRows><<<vv::gemm_grid(M, N), vv::kBlock, 0, vv::as_stream(stream)>>>(
-        static_cast<const vv::h16*>(A), lda, static_cast<const vv::h16*>(B), K, M, K, N, nullptr, nullptr, out);
+    vv::launch_vae_gemm<false, vv::kEpiRows>(static_cast<const vv::h16*>(A), lda, static_cast<const vv::h16*>(B), K, M, K,
+                                            N, nullptr, nullptr, out, vv::as_stream(stream));
     return vv::launch_status();
 }
 
@@ -598,8 +726,8 @@ vv_status_t vv_gemm_fp16_nn_dev(const void* A, const void* B, void* C, int M, in
     out.ldc = P;
     out.alpha = alpha;
     out.beta = beta;
-    vv::vae_gemm<true, vv::kEpiAlphaBeta><<<vv::gemm_grid(M, P), vv::kBlock, 0, vv::as_stream(stream)>>>(
-        static_cast<const vv::h16*>(A), K, static_cast<const vv::h16*>(B), P, M, K, P, nullptr, nullptr, out);
+    vv::launch_vae_gemm<true, vv::kEpiAlphaBeta>(static_cast<const vv::h16*>(A), K, static_cast<const vv::h16*>(B), P, M,
+                                                 K, P, nullptr, nullptr, out, vv::as_stream(stream));
     return vv::launch_status();
 }
 
