@@ -30,11 +30,13 @@ def f16(shape, seed, std=1.0):
 class Batch:
     """Three items packed side by side: a fresh one, one with a carried state, one given by its own pointer."""
 
-    def __init__(self, in_ch, k, stride, seed, own_pointer=True):
+    def __init__(self, in_ch, k, stride, seed, own_pointer=True, round8=False):
         rng = np.random.default_rng(seed)
         self.in_ch, self.k, self.stride = in_ch, k, stride
         self.cap = max(k - stride, 1)
         in_lens = [int(rng.integers(3, 40)) * stride, int(rng.integers(50, 300)) * stride + (stride > 1), 7 * stride]
+        if round8:          # every item starts on a 16-byte boundary (the last may still end off one)
+            in_lens = [8 * int(rng.integers(1, 6)), 8 * int(rng.integers(9, 40)), 8 * int(rng.integers(1, 4)) + 5]
         self.items = []
         in_off = out_off = 0
         for i, n_in in enumerate(in_lens):
@@ -151,8 +153,14 @@ def test_conv_reads_an_item_through_its_own_pointer():
 
 
 @pytest.mark.parametrize("C_,k", [(32, 7), (70, 7), (128, 16), (8, 1)])
-def test_rms_then_mixer(C_, k):
-    b = Batch(C_, k, 1, 300 + C_, own_pointer=False)
+@pytest.mark.parametrize("aligned", [False, True])
+def test_rms_then_mixer(C_, k, aligned):
+    """aligned: items on 16-byte boundaries and a row stride that keeps them there (the 16-byte-access kernel)."""
+    b = Batch(C_, k, 1, 300 + C_, own_pointer=False, round8=aligned)
+    if aligned:             # pad the packed axis to a multiple of 8 columns: the padding belongs to no item
+        pad = (-b.T_in) % 8
+        b.x = np.concatenate([b.x, np.full((C_, pad), 0x7E00, np.uint16)], 1) if pad else b.x
+        b.T_in += pad
     T = b.T_in
     hd, _ = b.desc(False)
     dd, alive = b.desc(True)
