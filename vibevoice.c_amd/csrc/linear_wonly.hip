@@ -57,54 +57,68 @@ __device__ __forceinline__ uint32_t byte_table_entry(int b) {
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// kSplit waves share a weight row: wave p takes the rounds of 64 chunks p,
-// p + kSplit, ...; lane l chunk l of the round.
-template <int kFmt, int MR, int kSplit>
+// kSplit waves share RW weight rows: wave p takes the rounds of 64 chunks p,
+// p + kSplit, ...; lane l chunk l of the round, of each of its RW rows (the
+// activation chunk is loaded once for all of them).
+template <int kFmt, int MR, int kSplit, int RW>
 __global__ __launch_bounds__(kBlock) void wo_gemv(const h16* __restrict__ x, WoGemv a, int M) {
     constexpr int kCols = kFmt == kWoInt8 ? 16 : 32;       // weights per 16-byte chunk
-    constexpr int kRows = kWavesPerBlock / kSplit;
+    constexpr int kRows = kWavesPerBlock / kSplit * RW;
     __shared__ uint32_t table[256];
-    __shared__ float part[kWavesPerBlock][MR];
+    __shared__ float part[kWavesPerBlock][RW][MR];
     if constexpr (kFmt != kWoInt8) {
         table[threadIdx.x] = byte_table_entry<kFmt>((int)threadIdx.x);
         __syncthreads();
     }
     const int wave = wave_in_block(), lane = lane_id();
     const int set = wave / kSplit, piece = wave % kSplit;
-    const int n = (int)blockIdx.x * kRows + set;
-    const size_t row = (size_t)min(n, a.N - 1);
+    const int n0 = (int)blockIdx.x * kRows + set * RW;
     const int K = a.K, nchunks = K / kCols;
-    const u32x4* wrow = a.w + row * nchunks;
-
-    float acc[MR];
+    size_t row[RW];
+    const u32x4* wrow[RW];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+    for (int r = 0; r < RW; ++r) {
+        row[r] = (size_t)min(n0 + r, a.N - 1);
+        wrow[r] = a.w + row[r] * nchunks;
+    }
+
+    float acc[RW][MR];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0.0f;
 
 #pragma unroll 2
     for (int base = piece * kWave; base < nchunks; base += kSplit * kWave) {
         const bool live = base + lane < nchunks;
         const int c = live ? base + lane : nchunks - 1;
-        const u32x4 codes = __builtin_nontemporal_load(wrow + c);
-        float sc = 1.0f, mn = 0.0f;
-        if constexpr (kFmt == kWoNf4) {
-            sc = (float)static_cast<const h16*>(a.scales)[(row * K + (size_t)c * kCols) >> 6];
-        } else if constexpr (kFmt == kWoAwq) {
-            const size_t g = row * (size_t)(K >> a.gshift) + (size_t)((c * kCols) >> a.gshift);
-            sc = (float)static_cast<const h16*>(a.scales)[g];
-            mn = (float)a.mins[g];
-        }
-        h16x2 wv[kCols / 2];                       // wv[p]: columns 2p, 2p + 1 of the chunk
+        float sc[RW], mn[RW];
+        h16x2 wv[RW][kCols / 2];                   // wv[r][p]: columns 2p, 2p + 1 of the chunk
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if constexpr (kFmt == kWoInt8) {
-                // byte -> 0x6400 | (q + 128) = 1152 + q as FP16; minus 1152 is exact
-                const uint32_t u = codes[t] ^ 0x80808080u;
-                const h16x2 off = {(h16)1152.0f, (h16)1152.0f};
-                wv[2 * t] = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - off;
-                wv[2 * t + 1] = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - off;
-            } else {
+        for (int r = 0; r < RW; ++r) {
+            const u32x4 codes = __builtin_nontemporal_load(wrow[r] + c);
+            sc[r] = 1.0f;
+            mn[r] = 0.0f;
+            if constexpr (kFmt == kWoNf4) {
+                sc[r] = (float)static_cast<const h16*>(a.scales)[(row[r] * K + (size_t)c * kCols) >> 6];
+            } else if constexpr (kFmt == kWoAwq) {
+                const size_t g = row[r] * (size_t)(K >> a.gshift) + (size_t)((c * kCols) >> a.gshift);
+                sc[r] = (float)static_cast<const h16*>(a.scales)[g];
+                mn[r] = (float)a.mins[g];
+            }
 #pragma unroll
-                for (int b = 0; b < 4; ++b) wv[4 * t + b] = __builtin_bit_cast(h16x2, table[(codes[t] >> (8 * b)) & 0xFFu]);
+            for (int t = 0; t < 4; ++t) {
+                if constexpr (kFmt == kWoInt8) {
+                    // byte -> 0x6400 | (q + 128) = 1152 + q as FP16; minus 1152 is exact
+                    const uint32_t u = codes[t] ^ 0x80808080u;
+                    const h16x2 off = {(h16)1152.0f, (h16)1152.0f};
+                    wv[r][2 * t] = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - off;
+                    wv[r][2 * t + 1] = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - off;
+                } else {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b)
+                        wv[r][4 * t + b] = __builtin_bit_cast(h16x2, table[(codes[t] >> (8 * b)) & 0xFFu]);
+                }
             }
         }
 #pragma unroll
@@ -120,66 +134,89 @@ __global__ __launch_bounds__(kBlock) void wo_gemv(const h16* __restrict__ x, WoG
                     xw[4 * q + 2] = v.z;
                     xw[4 * q + 3] = v.w;
                 }
-                float dot = kFmt == kWoInt8 ? acc[m] : 0.0f;
-#pragma unroll
-                for (int p = 0; p < kCols / 2; ++p)
-                    dot = __builtin_amdgcn_fdot2(wv[p], __builtin_bit_cast(h16x2, xw[p]), dot, false);
-                if constexpr (kFmt == kWoInt8) {
-                    acc[m] = dot;
-                } else if constexpr (kFmt == kWoNf4) {
-                    acc[m] = __builtin_fmaf(sc, dot, acc[m]);
-                } else {
+                float xs = 0.0f;
+                if constexpr (kFmt == kWoAwq) {
                     const h16x2 ones = {(h16)1.0f, (h16)1.0f};
-                    float xs = 0.0f;
 #pragma unroll
                     for (int p = 0; p < kCols / 2; ++p)
                         xs = __builtin_amdgcn_fdot2(ones, __builtin_bit_cast(h16x2, xw[p]), xs, false);
-                    acc[m] = __builtin_fmaf(sc, dot, __builtin_fmaf(mn, xs, acc[m]));
+                }
+#pragma unroll
+                for (int r = 0; r < RW; ++r) {
+                    float dot = kFmt == kWoInt8 ? acc[r][m] : 0.0f;
+#pragma unroll
+                    for (int p = 0; p < kCols / 2; ++p)
+                        dot = __builtin_amdgcn_fdot2(wv[r][p], __builtin_bit_cast(h16x2, xw[p]), dot, false);
+                    if constexpr (kFmt == kWoInt8) acc[r][m] = dot;
+                    else if constexpr (kFmt == kWoNf4) acc[r][m] = __builtin_fmaf(sc[r], dot, acc[r][m]);
+                    else acc[r][m] = __builtin_fmaf(sc[r], dot, __builtin_fmaf(mn[r], xs, acc[r][m]));
                 }
             }
         }
     }
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = wave_sum(acc[m]);
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = wave_sum(acc[r][m]);
     if constexpr (kSplit > 1) {
         if (lane == 0) {
 #pragma unroll
-            for (int m = 0; m < MR; ++m) part[wave][m] = acc[m];
+            for (int r = 0; r < RW; ++r)
+#pragma unroll
+                for (int m = 0; m < MR; ++m) part[wave][r][m] = acc[r][m];
         }
         __syncthreads();
 #pragma unroll
-        for (int m = 0; m < MR; ++m) {
-            float sum = 0.0f;
+        for (int r = 0; r < RW; ++r)
 #pragma unroll
-            for (int p = 0; p < kSplit; ++p) sum += part[set * kSplit + p][m];
-            acc[m] = sum;
-        }
+            for (int m = 0; m < MR; ++m) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int p = 0; p < kSplit; ++p) sum += part[set * kSplit + p][r][m];
+                acc[r][m] = sum;
+            }
     }
-    if (piece == 0 && n < a.N) {
+    if (piece == 0) {
         float mine = 0.0f;
 #pragma unroll
-        for (int m = 0; m < MR; ++m)
-            if (lane == m) mine = acc[m];
-        if (lane < MR && lane < M) {
-            if constexpr (kFmt == kWoInt8) mine *= static_cast<const float*>(a.scales)[row];
+        for (int r = 0; r < RW; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (lane == r * MR + m) mine = acc[r][m];
+        const int r = lane / MR, m = lane % MR;
+        if (lane < RW * MR && m < M && n0 + r < a.N) {
+            const int n = n0 + r;
+            if constexpr (kFmt == kWoInt8) mine *= static_cast<const float*>(a.scales)[n];
             if (a.bias) mine += (float)a.bias[n];
-            a.y[(size_t)lane * a.N + n] = to_half(mine);
+            a.y[(size_t)m * a.N + n] = to_half(mine);
         }
     }
+}
+
+template <int kFmt, int MR, int kSplit, int RW>
+void launch_gemv_cfg(const h16* x, const WoGemv& a, int M, hipStream_t st) {
+    constexpr int kRows = kWavesPerBlock / kSplit * RW;
+    wo_gemv<kFmt, MR, kSplit, RW><<<dim3((unsigned)((a.N + kRows - 1) / kRows)), kBlock, 0, st>>>(x, a, M);
 }
 
 template <int kFmt, int MR>
 void launch_gemv_rows(const h16* x, const WoGemv& a, int M, hipStream_t st) {
     constexpr int kCols = kFmt == kWoInt8 ? 16 : 32;
     const int nchunks = a.K / kCols;
-    // Thousands of waves in flight, and no wave with less than half a round of chunks.
-    int split = 1;
+    // Thousands of waves in flight, and no wave with less than half a round of chunks; with rows to spare and short
+    // rows, two or four rows per wave (each activation chunk loaded once for them).
+    int split = 1, rw = 1;
     while (split < 4 && (long)a.N * split < 4096 && nchunks / (2 * split) >= kWave / 2) split *= 2;
-    const int rows = kWavesPerBlock / split;
-    const dim3 grid((unsigned)((a.N + rows - 1) / rows));
-    if (split == 1) wo_gemv<kFmt, MR, 1><<<grid, kBlock, 0, st>>>(x, a, M);
-    else if (split == 2) wo_gemv<kFmt, MR, 2><<<grid, kBlock, 0, st>>>(x, a, M);
-    else wo_gemv<kFmt, MR, 4><<<grid, kBlock, 0, st>>>(x, a, M);
+    while (split == 1 && rw < 4 && a.N / (2 * rw) >= 8192 && nchunks * rw <= 256 && MR * rw * 2 <= 8) rw *= 2;
+    if constexpr (MR <= 2) {
+        if (rw == 4) return launch_gemv_cfg<kFmt, MR, 1, 4>(x, a, M, st);
+    }
+    if constexpr (MR <= 4) {
+        if (rw >= 2) return launch_gemv_cfg<kFmt, MR, 1, 2>(x, a, M, st);
+    }
+    if (split == 1) launch_gemv_cfg<kFmt, MR, 1, 1>(x, a, M, st);
+    else if (split == 2) launch_gemv_cfg<kFmt, MR, 2, 1>(x, a, M, st);
+    else launch_gemv_cfg<kFmt, MR, 4, 1>(x, a, M, st);
 }
 
 template <int kFmt>
