@@ -17,9 +17,16 @@
  *               ("rne", what a device kernel that made no other error stores).
  *
  * Parity status (what pins each function is listed in tests/test_oracle_*.py):
- *   every function below is pinned by the compiled reference (oracle/_ref,
- *   bit-for-bit) where that builds, by committed golden vectors made from it,
- *   and by closed forms / invariants that do not retype its formula.
+ *   the functions that restate src/cpu (layer kernels, int8 quantisers and
+ *   linear layers, weight-only dequantisers, BitNet) are pinned by the compiled
+ *   reference (oracle/_ref, bit-for-bit) where that builds, by committed golden
+ *   vectors made from it, and by closed forms / invariants that do not retype
+ *   their formula. The functions that restate accelerator-only code (the
+ *   quantised KV codec, the Conv-VAE ops) have no CPU counterpart to compile
+ *   and are pinned by what the mathematics fixes: exhaustive code tables,
+ *   Hadamard / Lloyd-Max / signal-to-noise conditions, FP64 convolutions,
+ *   invariance under chunking, im2col + GEMM == direct convolution. One table
+ *   is PARITY UNPINNED: the +-1 pattern of the TurboQuant rotation (see there).
  */
 #ifndef VV_ORACLE_H
 #define VV_ORACLE_H
