@@ -267,8 +267,9 @@ vv_status_t vv_dequant_nf4_dev(const uint8_t* packed, const void* scales_fp16, v
 vv_status_t vv_awq_gemv_dev(const void* x, const uint32_t* packed, const uint32_t* mins,
                             const void* scales, const void* bias, void* y, int N, int K,
                             int group_size, void* stream);
-/* M <= 8 and K % 32 == 0: the one-row kernel; else dequantise into
- * temp_weight_fp16 + vv_gemm_fp16_dev. replaces device.h:199-202
+/* M <= 8 and K % 32 == 0: the one-row kernel; 9..64 rows: the small-M MFMA
+ * kernel where it serves the shape (no scratch); else dequantise into
+ * temp_weight_fp16 + vv_gemm_fp16_dev (the same bits). replaces device.h:199-202
  * (awq_gemv.cu:213-238). */
 vv_status_t vv_awq_gemm_dev(const void* input_fp16, const uint32_t* packed, const uint32_t* mins,
                             const void* scales, void* output_fp16, void* temp_weight_fp16,

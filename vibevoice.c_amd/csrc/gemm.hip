@@ -247,6 +247,8 @@ constexpr int kSkinnyWaves = 8;
 struct SkinnyProjs {
     const void* w[3];
     const void* scales[3];      // INT8: FP32 per weight row; NF4: FP16 absmax per 64 elements; FP16: unused
+    const void* mins[3];        // INT4 {scale, min}: FP16 per group, beside the scales
+    int gshift;                 // INT4 {scale, min}: log2 of the group size
     const h16* bias[3];
     h16* y[3];
     int n[3];
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
     const int wave = tid >> 6;
     const int r16 = lane & 15, ks = lane >> 4;
     const int which = ((int)blockIdx.x >= projs.first[1]) + ((int)blockIdx.x >= projs.first[2]);
-    const WoSource B = {projs.w[which], projs.scales[which], nullptr, 0};
+    const WoSource B = {projs.w[which], projs.scales[which], projs.mins[which], projs.gshift};
     const h16* __restrict__ bias = projs.bias[which];
     h16* __restrict__ C = projs.y[which];
     const int N = projs.n[which], vec_store = projs.vec[which];
@@ -369,6 +371,7 @@ void launch_skinny(const h16* A, const SkinnyProjs& projs, int blocks, int M, in
                    float beta, hipStream_t st, int format = kWoF16) {
     if (format == kWoInt8) launch_skinny_as<kWoInt8>(A, projs, blocks, M, K, alpha, beta, st);
     else if (format == kWoNf4) launch_skinny_as<kWoNf4>(A, projs, blocks, M, K, alpha, beta, st);
+    else if (format == kWoAwq) launch_skinny_as<kWoAwq>(A, projs, blocks, M, K, alpha, beta, st);
     else launch_skinny_as<kWoF16>(A, projs, blocks, M, K, alpha, beta, st);
 }
 
@@ -493,6 +496,30 @@ int forced_tile() {
 
 }  // namespace
 }  // namespace vv
+
+// For linear_wonly.hip: y[M][N] = A[M][K] x W^T for one INT4 {scale, min} weight through the small-M kernel (the
+// format is not one of the public entry point's), or VV_ERR_UNSUPPORTED (nothing launched) where
+// vv_gemm_fp16_dev would not hand the shape to that kernel.
+__attribute__((visibility("hidden")))
+vv_status_t vv_skinny_int4_minmax(const void* A, const void* w, const void* scales, const void* mins, int gshift,
+                                  void* y, int M, int N, int K, void* stream) {
+    if (M < 9 || M > 64 || K % 8 != 0 || !vv::aligned16(A) || !vv::skinny_serves(M, N) ||
+        (reinterpret_cast<uintptr_t>(w) & 3u) || (reinterpret_cast<uintptr_t>(scales) & 1u) ||
+        (reinterpret_cast<uintptr_t>(mins) & 1u))
+        return VV_ERR_UNSUPPORTED;
+    vv::SkinnyProjs p = {};
+    p.w[0] = w;
+    p.scales[0] = scales;
+    p.mins[0] = mins;
+    p.gshift = gshift;
+    p.y[0] = static_cast<vv::h16*>(y);
+    p.n[0] = N;
+    p.vec[0] = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(y) & 7u) == 0);
+    const int blocks = (N + 15) / 16;
+    p.first[1] = p.first[2] = blocks;
+    vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, 1.0f, 0.0f, vv::as_stream(stream), vv::kWoAwq);
+    return vv::launch_status();
+}
 
 extern "C" {
 

@@ -21,6 +21,11 @@
 //               either way.
 #include "wonly.hpp"
 
+// gemm.hip: one INT4 {scale, min} weight through the small-M MFMA kernel, or VV_ERR_UNSUPPORTED.
+__attribute__((visibility("hidden")))
+vv_status_t vv_skinny_int4_minmax(const void* A, const void* w, const void* scales, const void* mins, int gshift,
+                                  void* y, int M, int N, int K, void* stream);
+
 namespace vv {
 namespace {
 
@@ -256,12 +261,15 @@ vv_status_t dequant(const WoSource& src, void* out, size_t n_elements, int K, hi
 template <int kFmt>
 vv_status_t gemm_via_fp16(const void* input, const WoSource& src, void* output, void* temp, int M, int N, int K,
                           void* stream) {
-    if constexpr (kFmt != kWoAwq) {
-        if (M >= 9 && M <= 64) {
+    if (M >= 9 && M <= 64) {
+        vv_status_t s;
+        if constexpr (kFmt == kWoAwq) {
+            s = vv_skinny_int4_minmax(input, src.w, src.scales, src.mins, src.gshift, output, M, N, K, stream);
+        } else {
             const vv_skinny_proj_t p = {src.w, src.scales, nullptr, output, N};
-            const vv_status_t s = vv_skinny_linear_dev(input, kFmt, &p, 1, M, K, 1.0f, stream);
-            if (s != VV_ERR_UNSUPPORTED) return s;
+            s = vv_skinny_linear_dev(input, kFmt, &p, 1, M, K, 1.0f, stream);
         }
+        if (s != VV_ERR_UNSUPPORTED) return s;
     }
     if (!temp) return VV_ERR_NULL_PTR;
     if (!aligned16(temp)) return VV_ERR_UNSUPPORTED;
