@@ -273,11 +273,13 @@ __global__ __launch_bounds__(kBlock) void bn_requant(const float* __restrict__ y
 
 // ── int8 head + argmax ──────────────────────────────────────────────────────
 
-constexpr int kHeadRowsPerWave = 8;
+constexpr int kHeadRowsPerWave = 32;
 constexpr int kHeadRows = kWavesPerBlock * kHeadRowsPerWave;
 
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
 
+// A half-wave per vocabulary row (K = 1536 is exactly three 16-byte chunks per lane), two pairs of rows in flight;
+// kWide: 16-byte loads (K % 16 == 0, operands on 16 bytes), else 4-byte ones.
 template <bool kWide>
 __global__ __launch_bounds__(kBlock) void bn_head(const int8_t* __restrict__ q, const float* __restrict__ scale,
                                                   const int8_t* __restrict__ w, const float* __restrict__ w_scale,
@@ -286,34 +288,50 @@ __global__ __launch_bounds__(kBlock) void bn_head(const int8_t* __restrict__ q, 
     __shared__ float best_v[kWavesPerBlock];
     __shared__ int best_i[kWavesPerBlock];
     const int wave = wave_in_block(), lane = lane_id();
+    const int l32 = lane & 31, half = lane >> 5;
     const float s = *scale;
     float bv = -FLT_MAX;
     int bi = 0x7fffffff;
     const int r0 = (int)blockIdx.x * kHeadRows + wave * kHeadRowsPerWave;
-    for (int r = 0; r < kHeadRowsPerWave; ++r) {
-        const int n = r0 + r;
-        if (n >= V) break;
-        const int8_t* wr = w + (size_t)n * K;
-        int acc = 0;
-        if constexpr (kWide) {
-            const i32x4* w4 = reinterpret_cast<const i32x4*>(wr);
-            const i32x4* x4 = reinterpret_cast<const i32x4*>(q);
-            for (int i = lane; i < K / 16; i += kWave) {
-                const i32x4 a = __builtin_nontemporal_load(w4 + i), b = x4[i];
-                acc = __builtin_amdgcn_sdot4(a.x, b.x, acc, false);
-                acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);
-                acc = __builtin_amdgcn_sdot4(a.z, b.z, acc, false);
-                acc = __builtin_amdgcn_sdot4(a.w, b.w, acc, false);
+    for (int r = 0; r < kHeadRowsPerWave; r += 4) {
+        int acc[2] = {0, 0};
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int n = min(r0 + r + 2 * u + half, V - 1);
+            const int8_t* wr = w + (size_t)n * K;
+            if constexpr (kWide) {
+                const i32x4* w4 = reinterpret_cast<const i32x4*>(wr);
+                const i32x4* x4 = reinterpret_cast<const i32x4*>(q);
+                for (int i = l32; i < K / 16; i += 32) {
+                    const i32x4 a = __builtin_nontemporal_load(w4 + i), b = x4[i];
+                    acc[u] = __builtin_amdgcn_sdot4(a.x, b.x, acc[u], false);
+                    acc[u] = __builtin_amdgcn_sdot4(a.y, b.y, acc[u], false);
+                    acc[u] = __builtin_amdgcn_sdot4(a.z, b.z, acc[u], false);
+                    acc[u] = __builtin_amdgcn_sdot4(a.w, b.w, acc[u], false);
+                }
+            } else {
+                const int* w1 = reinterpret_cast<const int*>(wr);
+                const int* x1 = reinterpret_cast<const int*>(q);
+                for (int i = l32; i < K / 4; i += 32) acc[u] = __builtin_amdgcn_sdot4(w1[i], x1[i], acc[u], false);
             }
-        } else {
-            const int* w1 = reinterpret_cast<const int*>(wr);
-            const int* x1 = reinterpret_cast<const int*>(q);
-            for (int i = lane; i < K / 4; i += kWave) acc = __builtin_amdgcn_sdot4(w1[i], x1[i], acc, false);
         }
-        acc = wave_sum_int(acc);
-        float v = (float)acc * w_scale[n];
-        v = v / s;
-        if (better(v, n, bv, bi)) { bv = v; bi = n; }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) acc[u] += __shfl_xor(acc[u], o);       // inside each half-wave
+            const int n = r0 + r + 2 * u + half;
+            if (n < V) {
+                float v = (float)acc[u] * w_scale[n];
+                v = v / s;
+                if (better(v, n, bv, bi)) { bv = v; bi = n; }
+            }
+        }
+    }
+    // the two half-waves hold different rows: meet them, then the waves
+    {
+        const float ov = __shfl_xor(bv, 32);
+        const int oi = __shfl_xor(bi, 32);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
     }
     if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
     __syncthreads();
