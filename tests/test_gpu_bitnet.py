@@ -155,3 +155,56 @@ def test_argument_checks():
     assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 6, p, None, p, s) == I                        # K % 4
     assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 64, p, None, None, s) == N
     assert dev.vv_i8_head_argmax_scratch_bytes(0) == 0
+
+
+def test_bitnet_decode_ops_replay_from_a_graph():
+    """Every per-token value (activation scale, row sum, the head's scale) is read from device memory, so a captured
+    quantise -> ternary product -> int8 head sequence replays on new inputs: each replay equals the eager run."""
+    import ctypes as C
+    rng = np.random.default_rng(9)
+    K, N, V = 1536, 1536, 4000
+    codes = oracle.ternary_pack(rng.integers(-1, 2, (N, K)).astype(np.int8))
+    wh = rng.integers(-127, 128, (V, N), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.01, V).astype(np.float32)
+    d_codes, d_wh, d_ws = D(codes), D(wh), D(ws)
+    d_x = torch.zeros((1, K), dtype=torch.float32, device="cuda")
+    d_q = torch.zeros((1, K), dtype=torch.int8, device="cuda")
+    d_s = torch.zeros(1, dtype=torch.float32, device="cuda")
+    d_sum = torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_y = torch.zeros((1, N), dtype=torch.float32, device="cuda")
+    d_q2 = torch.zeros((1, N), dtype=torch.int8, device="cuda")
+    d_s2 = torch.zeros(1, dtype=torch.float32, device="cuda")
+    d_tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_val = torch.zeros(1, dtype=torch.float32, device="cuda")
+    d_scr = torch.empty(dev.vv_i8_head_argmax_scratch_bytes(V), dtype=torch.uint8, device="cuda")
+
+    def step(st):
+        ok(dev.vv_act_quant_i8_dev(P(d_x), 0, 1, K, P(d_q), P(d_s), P(d_sum), st))
+        ok(dev.vv_ternary_gemm_dev(P(d_q), P(d_sum), P(d_s), P(d_codes), 0.02, None, None, P(d_y), 0, 1, N, K, st))
+        ok(dev.vv_act_quant_i8_dev(P(d_y), 0, 1, N, P(d_q2), P(d_s2), None, st))
+        ok(dev.vv_i8_head_argmax_dev(P(d_q2), P(d_s2), P(d_wh), P(d_ws), V, N, P(d_tok), P(d_val), P(d_scr), st))
+
+    s = C.c_void_p()
+    assert dev.vv_dev_stream_create(C.byref(s)) == dev.VV_OK
+    st = s.value
+    torch.cuda.synchronize()
+    assert dev.vv_dev_graph_begin(st) == dev.VV_OK
+    step(st)
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(st, C.byref(g)) == dev.VV_OK and g.value
+    seen = set()
+    for i in range(5):
+        x = (rng.standard_normal((1, K)) * (1 + i)).astype(np.float32)
+        d_x.copy_(torch.from_numpy(x))
+        torch.cuda.synchronize()
+        assert dev.vv_dev_graph_launch(g.value, st) == dev.VV_OK
+        assert dev.vv_dev_stream_sync(st) == dev.VV_OK
+        got = (int(host(d_tok)[0]), float(host(d_val)[0]))
+        q, sc, sm = oracle.bn_act_quant(x)
+        _, y = oracle.ternary_linear(q, sc, codes, 0.02, None)
+        q2, s2, _ = oracle.bn_act_quant(y)
+        assert got == oracle.i8_head_argmax(q2[0], float(s2[0]), wh, ws)
+        seen.add(got[0])
+    assert len(seen) > 1                                           # the replays really saw different inputs
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(st)
