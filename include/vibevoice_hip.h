@@ -246,7 +246,8 @@ vv_status_t vv_nf4_gemv_dev(const void* x, const uint8_t* packed, const void* sc
                             const void* bias, void* y, int N, int K, void* stream);
 /* M <= 8 (K % 32 == 0): the one-row kernel over up to eight rows, no scratch.
  * 9..64 rows: the small-M MFMA kernel where vv_skinny_linear_dev serves the
- * shape, no scratch. Otherwise the weight is dequantised into temp_weight_fp16
+ * shape, else the tile kernel with the weight dequantised on its way in; no
+ * scratch either way. Otherwise the weight is dequantised into temp_weight_fp16
  * [N][K] (NULL there: VV_ERR_NULL_PTR) and vv_gemm_fp16_dev runs; the last two
  * give the same bits. block_size must be 64. replaces device.h:174-178
  * (gemm.cu:468-500). */
@@ -268,7 +269,8 @@ vv_status_t vv_awq_gemv_dev(const void* x, const uint32_t* packed, const uint32_
                             const void* scales, const void* bias, void* y, int N, int K,
                             int group_size, void* stream);
 /* M <= 8 and K % 32 == 0: the one-row kernel; 9..64 rows: the small-M MFMA
- * kernel where it serves the shape (no scratch); else dequantise into
+ * kernel or the tile kernel with the weight dequantised on its way in (no
+ * scratch); else dequantise into
  * temp_weight_fp16 + vv_gemm_fp16_dev (the same bits). replaces device.h:199-202
  * (awq_gemv.cu:213-238). */
 vv_status_t vv_awq_gemm_dev(const void* input_fp16, const uint32_t* packed, const uint32_t* mins,
@@ -283,9 +285,10 @@ vv_status_t vv_dequant_awq_dev(const uint32_t* packed, const uint32_t* mins, con
  * once per output. replaces device.h:216-218 (int8_gemv.cu:72-101). */
 vv_status_t vv_int8_gemv_dev(const void* x, const int8_t* q, const float* scales,
                              const void* bias, void* y, int N, int K, void* stream);
-/* M <= 8 the one-row kernel, 9..64 the small-M MFMA kernel where it serves (no
- * scratch), else dequantise + vv_gemm_fp16_dev; the last two give the same
- * bits. No bias. replaces device.h:223-226 (int8_gemv.cu:194-223). */
+/* M <= 8 the one-row kernel, 9..64 the small-M MFMA kernel where it serves, else
+ * the tile kernel with the weight dequantised on its way in (no scratch either
+ * way), above that dequantise + vv_gemm_fp16_dev; all of the last three give
+ * the same bits. No bias. replaces device.h:223-226 (int8_gemv.cu:194-223). */
 vv_status_t vv_int8_gemm_dev(const void* input_fp16, const int8_t* q, const float* scales,
                              void* output_fp16, void* temp_weight_fp16, int M, int N, int K,
                              void* stream);

@@ -97,6 +97,33 @@ __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
     mfma_tile<F16Op, BM, BN, WM, WN, kSlab / 8, kFull, kAhead>(A, B, M, N, K / 8, epilogue);
 }
 
+// The same tile loop with the weight rows dequantised on their way in (wonly.hpp): the K order of gemm_tile, so
+// the bits of dequantising into FP16 first and running gemm_tile on that.
+template <int kFmt>
+struct WoRows {
+    static constexpr bool kPlain = false;
+    WoSource src;
+    const float* book;
+    int K;
+    __device__ __forceinline__ u32x4 load(int row, int slot) const { return wo_slot<kFmt>(src, book, (size_t)row, K, slot); }
+};
+
+template <int BM, int BN, int WM, int WN, int kSlab, bool kFull, int kFmt>
+__global__ __launch_bounds__(WM * WN * kWave) void gemm_tile_wo(
+    const h16* __restrict__ A, WoSource B, h16* __restrict__ C, int M, int N, int K, int vec_store) {
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    __shared__ float book[16];
+    if constexpr (kFmt == kWoNf4) {
+        if (threadIdx.x < 16) book[threadIdx.x] = kNf4Book[threadIdx.x];
+        __syncthreads();
+    }
+    auto epilogue = [=](const f32x16 (&acc)[TN][TM], int m0, int n0, int frow, int fhalf) {
+        store_tile<TM, TN>(acc, C, M, N, m0, n0, frow, fhalf, 1.0f, 0.0f, vec_store);
+    };
+    const WoRows<kFmt> rows = {B, book, K};
+    mfma_tile<F16Op, BM, BN, WM, WN, kSlab / 8, kFull, 1>(A, nullptr, M, N, K / 8, epilogue, rows);
+}
+
 // The 256x256 tile with the slabs copied from global memory straight into LDS
 // (mfma_dma.hpp). Needs K % 32 == 0.
 __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
@@ -519,6 +546,37 @@ vv_status_t vv_skinny_int4_minmax(const void* A, const void* w, const void* scal
     p.first[1] = p.first[2] = blocks;
     vv::launch_skinny(static_cast<const vv::h16*>(A), p, blocks, M, K, 1.0f, 0.0f, vv::as_stream(stream), vv::kWoAwq);
     return vv::launch_status();
+}
+
+// For linear_wonly.hip: y[M][N] = A[M][K] x W^T, 9 <= M <= 64, for one weight in a weight-only format through the
+// LDS-tiled kernel with the weight dequantised on its way in: no scratch, the bits of dequantise + vv_gemm_fp16_dev
+// where that tiles. VV_ERR_UNSUPPORTED (nothing launched) outside what it covers.
+template <int kFmt>
+static vv_status_t tile_wo(const vv::h16* A, const vv::WoSource& B, vv::h16* C, int M, int N, int K, hipStream_t st) {
+    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    // Unpacking a slot costs about what multiplying it does: four waves per tile even when two would hold the rows
+    // (measured faster for every format from 17 rows on; the tile shape changes no bit).
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+    if (K % 64 == 0) vv::gemm_tile_wo<64, 64, 2, 2, 64, true, kFmt><<<grid, 4 * vv::kWave, 0, st>>>(A, B, C, M, N, K, vec);
+    else vv::gemm_tile_wo<64, 64, 2, 2, 64, false, kFmt><<<grid, 4 * vv::kWave, 0, st>>>(A, B, C, M, N, K, vec);
+    return vv::launch_status();
+}
+
+__attribute__((visibility("hidden")))
+vv_status_t vv_gemm_tile_weight_only(int format, const void* A, const void* w, const void* scales, const void* mins,
+                                     int gshift, void* y, int M, int N, int K, void* stream) {
+    if (M < 9 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || !vv::aligned16(A) || vv::skinny_serves(M, N))
+        return VV_ERR_UNSUPPORTED;
+    const uintptr_t at = reinterpret_cast<uintptr_t>(w);
+    if ((format == vv::kWoInt8 ? (at & 7u) : (at & 3u)) != 0) return VV_ERR_UNSUPPORTED;
+    const vv::WoSource B = {w, scales, mins, gshift};
+    const vv::h16* a = static_cast<const vv::h16*>(A);
+    vv::h16* c = static_cast<vv::h16*>(y);
+    hipStream_t st = vv::as_stream(stream);
+    if (format == vv::kWoInt8) return tile_wo<vv::kWoInt8>(a, B, c, M, N, K, st);
+    if (format == vv::kWoNf4) return tile_wo<vv::kWoNf4>(a, B, c, M, N, K, st);
+    if (format == vv::kWoAwq) return tile_wo<vv::kWoAwq>(a, B, c, M, N, K, st);
+    return VV_ERR_UNSUPPORTED;
 }
 
 extern "C" {

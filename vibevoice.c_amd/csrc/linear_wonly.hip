@@ -26,6 +26,12 @@ __attribute__((visibility("hidden")))
 vv_status_t vv_skinny_int4_minmax(const void* A, const void* w, const void* scales, const void* mins, int gshift,
                                   void* y, int M, int N, int K, void* stream);
 
+// gemm.hip: the same 9..64 rows where the small-M kernel declines, through the LDS-tiled kernel with the weight
+// dequantised on its way in; VV_ERR_UNSUPPORTED outside what it covers.
+__attribute__((visibility("hidden")))
+vv_status_t vv_gemm_tile_weight_only(int format, const void* A, const void* w, const void* scales, const void* mins,
+                                     int gshift, void* y, int M, int N, int K, void* stream);
+
 namespace vv {
 namespace {
 
@@ -269,6 +275,8 @@ vv_status_t gemm_via_fp16(const void* input, const WoSource& src, void* output, 
             const vv_skinny_proj_t p = {src.w, src.scales, nullptr, output, N};
             s = vv_skinny_linear_dev(input, kFmt, &p, 1, M, K, 1.0f, stream);
         }
+        if (s != VV_ERR_UNSUPPORTED) return s;
+        s = vv_gemm_tile_weight_only(kFmt, input, src.w, src.scales, src.mins, src.gshift, output, M, N, K, stream);
         if (s != VV_ERR_UNSUPPORTED) return s;
     }
     if (!temp) return VV_ERR_NULL_PTR;

@@ -31,10 +31,15 @@ struct Const { static constexpr int value = kValue; };
 //   epi(acc, m0, n0, frow, fhalf)            register 4g + r of lane l: column
 //                                            n0 + 32a + 8g + 4(l/32) + r of row
 //                                            m0 + 32b + l % 32, for acc[a][b]
+// Where the W rows come from: PlainRows reads 16-byte slots of a row-major operand (the default); any other source
+// produces slot `slot` of row `row` itself (weights dequantised on their way in): kPlain = false and
+// u32x4 load(int row, int slot) const.
+struct PlainRows { static constexpr bool kPlain = true; };
+
 template <typename Op, int BM, int BN, int WM, int WN, int kSlabChunks, bool kFull, int kAhead,
-          typename Epi>
+          typename Epi, typename BSrc = PlainRows>
 __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void* __restrict__ B,
-                                          int M, int N, int kchunks, const Epi& epi) {
+                                          int M, int N, int kchunks, const Epi& epi, const BSrc& bsrc = BSrc()) {
     constexpr int NT = WM * WN * kWave;
     constexpr int kSteps = kSlabChunks / 2;   // MFMA K steps per slab (two slots each)
     typedef typename Op::Acc Acc;
@@ -67,6 +72,7 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
     const char* a_base = static_cast<const char*>(A) + (size_t)m_blk * row_bytes;
     const char* b_base = static_cast<const char*>(B) + (size_t)n_blk * row_bytes;
     uint32_t a_off[LA], b_off[LB];
+    int b_row[LB];                                       // for a BSrc that is not plain rows
     const int my_slot = tid % kSlabChunks;               // NT is a multiple of the slots per row
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
@@ -77,6 +83,7 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
     for (int i = 0; i < LB; ++i) {
         const int row = min((tid + i * NT) / kSlabChunks, N - 1 - n_blk);
         b_off[i] = (uint32_t)row * row_bytes + (uint32_t)my_slot * 16u;
+        b_row[i] = n_blk + row;
     }
     // LDS side: the i-th store of a thread lands NT slots after its first (the
     // swizzle term depends on row bits 1..3 only and NT / slots is a multiple
@@ -97,8 +104,12 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
         for (int i = 0; i < LA; ++i)
             ra[set][i] = live ? *reinterpret_cast<const u32x4*>(a_base + adv + a_off[i]) : zero;
 #pragma unroll
-        for (int i = 0; i < LB; ++i)
-            rb[set][i] = live ? *reinterpret_cast<const u32x4*>(b_base + adv + b_off[i]) : zero;
+        for (int i = 0; i < LB; ++i) {
+            if constexpr (BSrc::kPlain)
+                rb[set][i] = live ? *reinterpret_cast<const u32x4*>(b_base + adv + b_off[i]) : zero;
+            else
+                rb[set][i] = live ? bsrc.load(b_row[i], slab * kSlabChunks + my_slot) : zero;
+        }
     };
     auto stage = [&](auto set_c, int buf) {
         constexpr int set = decltype(set_c)::value;
