@@ -149,3 +149,21 @@ def test_the_library_defines_every_symbol_of_the_reference_seam():
     assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
                              "vv_embedding_rmsnorm_dev", "vv_gemv_multi_dev", "vv_gemv_swiglu_dev",
                              "vv_kv_rotate_dev", "vv_kv_unrotate_dev"}
+
+
+HOST_ARCHIVE = os.path.join(ROOT, "oracle", "_ref", "host", "libvv_ref_host.a")
+
+
+@pytest.mark.skipif(not os.path.exists(HOST_ARCHIVE), reason="oracle/_ref/host not built (needs the reference tree)")
+def test_the_reference_host_code_links_against_this_library_alone():
+    """The reference's host side (decoder, KV cache, pipeline, Conv-VAE front end, connectors, loaders ...), compiled
+    where it lies into oracle/_ref/host/libvv_ref_host.a: every vv_ symbol it leaves undefined is one this library
+    defines, so an engine links with -lvibevoice_hip and nothing else for the accelerator."""
+    undefined = subprocess.run(["nm", "-u", HOST_ARCHIVE], capture_output=True, text=True).stdout
+    defined = subprocess.run(["nm", "--defined-only", HOST_ARCHIVE], capture_output=True, text=True).stdout
+    want = {l.split()[-1] for l in undefined.splitlines() if l.strip().startswith("U vv_")}
+    have_host = {l.split()[-1] for l in defined.splitlines() if len(l.split()) == 3 and l.split()[-1].startswith("vv_")}
+    need = want - have_host
+    out = subprocess.check_output(["nm", "-D", "--defined-only", dev.LIB_PATH], text=True)
+    ours = {l.split()[-1] for l in out.splitlines() if " T vv_" in l}
+    assert len(need) >= 60 and not (need - ours), sorted(need - ours)
