@@ -292,27 +292,28 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
             del xq, sx, c
         del w8, sw
     # And as W4A8: 4-bit codes with a scale and a zero point per 128 columns (any bytes are valid codes).
-    out["w4a8"], out["w4a8_gemv"] = {}, {}
+    out["w4a8"], out["w4a8_gemv"], out["w4a8_chunk"] = {}, {}, {}
     G = 128
     for name, n, k in shapes:
         w4 = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
         sz = torch.stack([torch.rand(n, k // G, device="cuda") * 0.02 + 0.002,
                           torch.randint(0, 16, (n, k // G), device="cuda").float()], dim=-1).half().contiguous()
-        for m, key, layout in ((T, "w4a8", 3), (1, "w4a8_gemv", 2)):
+        # T rows (prefill), one row (decode) and 29 rows (a streaming chunk: the weights are still the bytes)
+        for m, key, layout in ((T, "w4a8", 3), (1, "w4a8_gemv", 2), (29, "w4a8_chunk", 3)):
             xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
             sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
             c = torch.empty(m, n, dtype=torch.float16, device="cuda")
             xs = xq.view(m, k // 32, 32).sum(-1, dtype=torch.int32).contiguous()     # what the quantiser writes
             sec = timed(lambda: dev.vv_w4a8_linear_dev(xq.data_ptr(), layout, sx.data_ptr(), xs.data_ptr(), w4.data_ptr(),
                                                        sz.data_ptr(), G, None, None, c.data_ptr(), 0, m, n, k, 0,
-                                                       st), 5 if m > 1 else 50)
-            if m > 1:
+                                                       st), 5 if m > 64 else 50)
+            if m > 64:
                 tops = 2.0 * m * n * k / sec / 1e12
                 out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TOPs": tops,
                                   "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
             else:
-                gb = (n * k / 2 + n * (k // G) * 4 + k + 2.0 * n) / sec / 1e9
-                out[key][name] = {"N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                gb = (n * k / 2 + n * (k // G) * 4 + m * (k + 2.0 * n)) / sec / 1e9
+                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del xq, sx, c
         # the same codes against FP16 activations (W4A16)
@@ -1088,6 +1089,8 @@ def main() -> int:
                     f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
             for name, d in layer[kind + "_gemv"].items():
                 log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        for name, d in layer["w4a8_chunk"].items():
+            log(f"  w4a8 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         for name, d in layer["w4a16"].items():
             log(f"  w4a16 {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")

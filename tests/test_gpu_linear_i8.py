@@ -289,7 +289,13 @@ def want_w4(p, bias=False, res=False):
 W4_SHAPES = [(1, 64, 32, 32), (3, 50, 192, 96), (1, 40, 8192, 4096), (8, 37, 18944, 32), (1, 18944, 3584, 128), (1, 3584, 3584, 128), (1, 512, 18944, 128), (2, 77, 256, 256), (5, 136, 640, 32),
              (8, 300, 640, 64), (8, 64, 1024, 512), (9, 64, 64, 32), (16, 30, 96, 32), (17, 77, 256, 256),
              (33, 136, 640, 32), (64, 300, 640, 64), (65, 64, 1024, 512), (100, 130, 160, 32), (130, 101, 224, 32),
-             (285, 3584, 3584, 128), (300, 4608, 1536, 128), (921, 512, 3584, 128)]
+             (285, 3584, 3584, 128), (300, 4608, 1536, 128), (921, 512, 3584, 128),
+             # at most 64 rows in the MMA order with groups of 64, 128, 256: the streamed kernel, whole and partial
+             # rounds of eight groups, ragged N
+             (9, 100, 1152, 128), (29, 3584, 3584, 128), (28, 520, 18944, 128), (33, 77, 1280, 64),
+             (64, 136, 2304, 256), (40, 4608, 1536, 128), (32, 31, 64, 64), (5, 33, 8192, 128),
+             # five to eight rows: the streamed kernel reads the GEMV's order of the activations as well
+             (8, 3584, 3584, 128), (7, 100, 1152, 128), (6, 520, 2304, 256), (5, 77, 1280, 64)]
 
 
 @pytest.mark.parametrize("M,N,K,G", W4_SHAPES)
@@ -305,6 +311,11 @@ def test_w4a8_bit_exact_against_oracle(M, N, K, G):
         assert np.array_equal(run_w4(p, lay, True, True), want16), f"f16 layout {lay}"
         same_f32(run_w4(p, lay, f32=True), plain32, f"f32 plain layout {lay}")
         same_f32(run_w4(p, lay, True, True, f32=True, xsum=True), want32, f"f32 layout {lay} with xsum")
+        if lay == L_MMA and M <= 64:     # asked for by name, the LDS-tiled kernel serves these rows too
+            same_f32(run_w4(p, lay, True, True, f32=True, path=MMA), want32, "f32 tiled")
+        if lay == L_GEMV and M > 4:      # and the GEMV beyond the four rows AUTO gives it
+            same_f32(run_w4(p, lay, True, True, f32=True, path=GEMV), want32, "f32 gemv by name")
+            same_f32(run_w4(p, lay, True, True, f32=True, path=GEMV, xsum=True), want32, "f32 gemv by name, xsum")
 
 
 @pytest.mark.parametrize("M,N,K,G", [(1, 256, 3584, 128), (7, 300, 640, 64), (40, 136, 640, 32), (300, 264, 1024, 512)])
@@ -369,13 +380,16 @@ def test_w4a8_follows_the_device_quantiser():
         same_f32(d_y.cpu().numpy(), want32, f"layout {lay}")
 
 
-@pytest.mark.parametrize("M,layout", [(2, L_GEMV), (40, L_MMA)])
+@pytest.mark.parametrize("M,layout", [(2, L_GEMV), (40, L_MMA), (7, L_GEMV), (6, L_GEMV)])
 def test_i8_linear_multi_w4(M, layout):
+    """One launch for all projections or one call each (M = 6: wide projections of
+    more than four rows go one by one), the same bits."""
     K, G = 512, 128
+    sizes = (9000, 8000, 136) if M == 6 else (512, 128, 136)
     base = w4_problem(M, 8, K, G, 80 + M)
     d_xq, d_sx = i8_dev(base["orders"][layout]), i8_dev(base["sx"])
     keep, projs, wants = [], (dev.I8Proj * 3)(), []
-    for i, N in enumerate((512, 128, 136)):
+    for i, N in enumerate(sizes):
         p = w4_problem(M, N, K, G, 90 + i)
         d_w, d_sz = i8_dev(p["gpu"]), i8_dev(p["sz"])
         d_b = to_dev(p["bias"]) if i != 1 else None

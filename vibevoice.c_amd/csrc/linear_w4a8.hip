@@ -525,6 +525,260 @@ bool launch_w4_tile(const W4Args& a, hipStream_t st) {
     return true;
 }
 
+// ── M <= 64 in the MMA order, groups of 64, 128 or 256 columns: streamed weights ─
+// With so few activation rows a tile grid has too few workgroups to pull the
+// codes out of HBM, and the in-order addition of the groups forbids splitting K
+// between accumulators. The int32 sum of one group is exact in any order,
+// though: a workgroup owns 32 weight rows, its eight waves take the eight groups
+// of a round one each and leave the group's sums in LDS, and the waves that
+// own a quarter of the output tile then add the round's groups in order,
+// acc += s_g * (float)sum_g, as every other path does.
+//
+// One 32x32x32 MFMA pair covers 64 columns: lane (row, half) loads the 16 bytes
+// of codes of chunk 2p + half of its weight row and the 32 bytes of that chunk
+// of its activation row; the first MFMA meets nibble slots 0..3 of the four
+// words with activation bytes 0..15, the second slots 4..7 with bytes 16..31.
+// No byte is loaded twice, and both chunks of a pair lie in one group.
+constexpr int kStreamWaves = 8;
+
+// A lane of the MFMA order reads 16 bytes of its own row, so one load touches 32
+// cache lines; kViaLds (groups of 128 columns) loads whole runs of a row instead
+// (four lanes a weight row's 64 bytes of the group, eight lanes an activation
+// row's 128) and turns them into the MFMA order through a piece of LDS of the
+// wave's own. The operands of the next round are requested before the sums of
+// this one are handed over; requesting further ahead measured slower.
+template <int kMT, int kPairs, bool kViaLds, bool kGemvOrder>
+__global__ __launch_bounds__(kStreamWaves * kWave) void w4a8_stream(W4Args a) {
+    static_assert(!kViaLds || kPairs == 2, "the staged loads are laid out for groups of 128 columns");
+    constexpr int kGroups = kStreamWaves;          // groups per round, one per wave
+    extern __shared__ u32x4 lds[];                 // sums[kGroups][kMT][4][64] int32x4, then scl[kGroups][32] float
+    i32x4* sums = reinterpret_cast<i32x4*>(lds);
+    float* scl = reinterpret_cast<float*>(lds + kGroups * kMT * 4 * kWave);
+    u32x4* stage = lds + kGroups * kMT * 4 * kWave + kGroups * 32 / 4;     // kViaLds: 4 KB per wave
+    const int wave = wave_in_block(), lane = lane_id();
+    const int row32 = lane & 31, half = lane >> 5;
+    const int n_blk = (int)blockIdx.x * 32;
+    const int ng = a.K / a.G;
+    const int nrounds = (ng + kGroups - 1) / kGroups;
+    const int wr = min(n_blk + row32, a.N - 1);
+    const u32x4* wrow = reinterpret_cast<const u32x4*>(a.packed + (size_t)wr * (a.K / 8));
+    const uint32_t* zrow = a.sz + (size_t)wr * ng;
+    const u32x4* xrow[kMT];
+#pragma unroll
+    for (int y = 0; y < kMT; ++y)
+        xrow[y] = reinterpret_cast<const u32x4*>(a.xq + (size_t)min(y * 32 + row32, a.M - 1) * a.K);
+    // Wave 4 y + q adds output rows 8 q + 4 half + r (r = 0..3) of activation tile y. (Sharing the
+    // adds between all eight waves when there is one tile measured slower.)
+    const bool adds = wave < kMT * 4;
+    const int ay = wave >> 2, aq = wave & 3;
+    const i32x4* my_sums = sums + (ay * 4 + aq) * kWave + lane;
+    const float* my_scl = scl + 8 * aq + 4 * half;
+    f32x4 facc = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4 w[kPairs], x[kMT][kPairs][2];
+    uint32_t zw = 0;
+    auto fetch = [&](int round) {
+        const int g = min(round * kGroups + wave, ng - 1);
+        if constexpr (kViaLds) {
+            // Whole runs of a row per load: 4 lanes cover a weight row's 64 bytes of the group, 8 lanes an
+            // activation row's 128 bytes.
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int row = min(n_blk + (lane >> 2) + 16 * i, a.N - 1);
+                w[i] = reinterpret_cast<const u32x4*>(a.packed + (size_t)row * (a.K / 8))[g * 4 + (lane & 3)];
+            }
+#pragma unroll
+            for (int y = 0; y < kMT; ++y)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = min(y * 32 + (lane >> 3) + 8 * i, a.M - 1);
+                    x[y][i >> 1][i & 1] =
+                        reinterpret_cast<const u32x4*>(a.xq + (size_t)row * a.K)[g * 8 + (lane & 7)];
+                }
+        } else {
+            const int c0 = g * (2 * kPairs) + half;
+#pragma unroll
+            for (int p = 0; p < kPairs; ++p) {
+                w[p] = wrow[c0 + 2 * p];
+#pragma unroll
+                for (int y = 0; y < kMT; ++y) {
+                    x[y][p][0] = xrow[y][2 * (c0 + 2 * p)];
+                    x[y][p][1] = xrow[y][2 * (c0 + 2 * p) + 1];
+                }
+            }
+        }
+        zw = zrow[g];
+    };
+    auto add_group = [&](int j) {
+#pragma clang fp contract(off)
+        const i32x4 s = my_sums[j * (kMT * 4 * kWave)];
+        const f32x4 sc = *reinterpret_cast<const f32x4*>(my_scl + j * 32);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float term = sc[r] * (float)s[r];
+            facc[r] = facc[r] + term;
+        }
+    };
+    // The group sums of one round go through LDS to the adding waves.
+    auto hand_over = [&](const i32x16 (&acc)[kMT], float scale, int round) {
+        __syncthreads();           // the previous round's sums have been added
+        if (round * kGroups + wave < ng) {
+#pragma unroll
+            for (int y = 0; y < kMT; ++y)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const i32x4 s = {acc[y][4 * q], acc[y][4 * q + 1], acc[y][4 * q + 2], acc[y][4 * q + 3]};
+                    sums[((wave * kMT + y) * 4 + q) * kWave + lane] = s;
+                }
+            if (half == 0) scl[wave * 32 + row32] = scale;
+        }
+        __syncthreads();
+        if (adds) {
+            const int live = ng - round * kGroups;
+            if (live >= kGroups) {
+#pragma unroll
+                for (int j = 0; j < kGroups; ++j) add_group(j);
+            } else {
+#pragma unroll 1
+                for (int j = 0; j < live; ++j) add_group(j);
+            }
+        }
+    };
+    auto group_sums = [&](i32x16 (&acc)[kMT]) {
+        const uint32_t z4 = sz_zero4(zw);
+        u32x4 wf[kPairs], xf[kMT][kPairs][2];
+        if constexpr (kViaLds) {
+            // Through this wave's own piece of LDS into the MFMA order; LDS serves a wave's accesses in
+            // the order they were issued, so the piece is reused without a barrier.
+            u32x4* buf = stage + wave * 256;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int row = (lane >> 2) + 16 * i;
+                buf[row * 4 + swz<32>(row, lane & 3)] = w[i];
+            }
+#pragma unroll
+            for (int p = 0; p < 2; ++p) wf[p] = buf[row32 * 4 + swz<32>(row32, half + 2 * p)];
+#pragma unroll
+            for (int y = 0; y < kMT; ++y) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = (lane >> 3) + 8 * i;
+                    buf[row * 8 + swz<64>(row, lane & 7)] = x[y][i >> 1][i & 1];
+                }
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    xf[y][p][0] = buf[row32 * 8 + swz<64>(row32, 2 * (half + 2 * p))];
+                    xf[y][p][1] = buf[row32 * 8 + swz<64>(row32, 2 * (half + 2 * p) + 1)];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < kPairs; ++p) {
+                wf[p] = w[p];
+#pragma unroll
+                for (int y = 0; y < kMT; ++y) {
+                    xf[y][p][0] = x[y][p][0];
+                    xf[y][p][1] = x[y][p][1];
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < kPairs; ++p) {
+            i32x4 lo, hi;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t even = wf[p][t] & 0x0F0F0F0Fu;           // slots 0,2,4,6
+                const uint32_t odd = (wf[p][t] >> 4) & 0x0F0F0F0Fu;     // slots 1,3,5,7
+                if constexpr (kGemvOrder) {
+                    // activation bytes 8t..8t+3 meet the even slots of word t, 8t+4..8t+7 the odd ones
+                    (t < 2 ? lo : hi)[2 * (t & 1)] = (int)minus_zero(even, z4);
+                    (t < 2 ? lo : hi)[2 * (t & 1) + 1] = (int)minus_zero(odd, z4);
+                } else {
+                    lo[t] = (int)minus_zero(__builtin_amdgcn_perm(odd, even, 0x05010400u), z4);
+                    hi[t] = (int)minus_zero(__builtin_amdgcn_perm(odd, even, 0x07030602u), z4);
+                }
+            }
+#pragma unroll
+            for (int y = 0; y < kMT; ++y) {
+                const i32x4 x0 = __builtin_bit_cast(i32x4, xf[y][p][0]);
+                const i32x4 x1 = __builtin_bit_cast(i32x4, xf[y][p][1]);
+                if (p == 0) {
+                    const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    acc[y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, x0, zero, 0, 0, 0);
+                } else {
+                    acc[y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo, x0, acc[y], 0, 0, 0);
+                }
+                acc[y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(hi, x1, acc[y], 0, 0, 0);
+            }
+        }
+    };
+    fetch(0);
+    for (int round = 0; round < nrounds; ++round) {
+        i32x16 acc[kMT];
+        group_sums(acc);
+        const float scale = sz_scale(zw);
+        fetch(min(round + 1, nrounds - 1));       // past the end: the last round again, unused
+        hand_over(acc, scale, round);
+    }
+    if (adds) {
+        const int m = ay * 32 + row32, n = n_blk + 8 * aq + 4 * half;
+        if (m < a.M && n < a.N) {
+            const float t[4] = {facc[0], facc[1], facc[2], facc[3]};
+            w4_store4(a, m, n, t);
+        }
+    }
+}
+
+template <int kMT, int kPairs, bool kGemvOrder>
+bool launch_w4_stream_cfg(const W4Args& a, hipStream_t st) {
+    constexpr bool kViaLds = kPairs == 2;
+    constexpr size_t kLds = (size_t)kStreamWaves * kMT * 4 * kWave * 16 + (size_t)kStreamWaves * 32 * sizeof(float) +
+                            (kViaLds ? (size_t)kStreamWaves * 4096 : 0);
+    if constexpr (kLds > 64 * 1024) {
+        // above the default limit of dynamic LDS: raised once per thread and device
+        static thread_local int ready_device = -1;
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess) return false;
+        if (ready_device != device) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(w4a8_stream<kMT, kPairs, kViaLds, kGemvOrder>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds) != hipSuccess) {
+                (void)hipGetLastError();
+                return false;
+            }
+            ready_device = device;
+        }
+    }
+    w4a8_stream<kMT, kPairs, kViaLds, kGemvOrder>
+        <<<dim3((unsigned)((a.N + 31) / 32)), kStreamWaves * kWave, kLds, st>>>(a);
+    return true;
+}
+
+bool w4_stream_serves(int M, int N, int G) {
+    if (M > 64 || (G != 64 && G != 128 && G != 256)) return false;
+    if (M > 32 && (N + 63) / 64 >= 256) return false;     // enough 64 x 64 tiles to fill the chip
+    if (M > 32 && G == 256) return false;                   // two tiles of its operands do not fit the registers
+    return true;
+}
+
+// false: not this kernel's shape (nothing launched). gemv_order: the activations are in the GEMV's order.
+bool launch_w4_stream(const W4Args& a, bool gemv_order, hipStream_t st) {
+    if (!w4_stream_serves(a.M, a.N, a.G) || (gemv_order && a.M > 32)) return false;
+    if (gemv_order) {
+        return a.G == 64 ? launch_w4_stream_cfg<1, 1, true>(a, st)
+             : a.G == 128 ? launch_w4_stream_cfg<1, 2, true>(a, st) : launch_w4_stream_cfg<1, 4, true>(a, st);
+    }
+    if (a.M <= 32) {
+        return a.G == 64 ? launch_w4_stream_cfg<1, 1, false>(a, st)
+             : a.G == 128 ? launch_w4_stream_cfg<1, 2, false>(a, st) : launch_w4_stream_cfg<1, 4, false>(a, st);
+    }
+    return a.G == 64 ? launch_w4_stream_cfg<2, 1, false>(a, st) : launch_w4_stream_cfg<2, 2, false>(a, st);
+}
+
+// From five activation rows on the streamed kernel beats the GEMV, which goes through the weights once
+// per row in its arithmetic.
+constexpr int kGemvBestRows = 4;
+constexpr int kStreamMinRows = 2048;      // weight rows; below, the GEMV's one workgroup per few rows fills the chip better
+
 enum I8Path : int { kPathAuto = 0, kPathGemv = 1, kPathMma = 2, kPathSimt = 3 };
 
 }  // namespace
@@ -540,6 +794,11 @@ vv_status_t vv_w4a8_gemv_multi(const int8_t* xq, int x_layout, const float* sx, 
     if (K <= 0 || K % 32 != 0 || group_size <= 0 || group_size % 32 != 0 || K % group_size != 0)
         return VV_ERR_UNSUPPORTED;
     if (!vv::aligned16(xq) || (xsum && (reinterpret_cast<uintptr_t>(xsum) & 3u))) return VV_ERR_UNSUPPORTED;
+    // Wide projections of more than four rows go one by one to the streamed kernel, which wins there
+    // by more than a launch; the short ones of attention stay together.
+    long rows = 0;
+    for (int i = 0; i < n; ++i) rows += projs[i].N;
+    if (M > vv::kGemvBestRows && rows >= 16384 && vv::w4_stream_serves(M, projs[0].N, group_size)) return VV_ERR_UNSUPPORTED;
     vv::W4Args a = {};
     a.xq = xq;
     a.sx = sx;
@@ -575,6 +834,7 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
         return VV_ERR_UNSUPPORTED;
     if (!vv::aligned16(xq) || !vv::aligned16(packed) || (reinterpret_cast<uintptr_t>(sz) & 3u))
         return VV_ERR_UNSUPPORTED;
+    const bool path_auto = path == vv::kPathAuto;
     if (path == vv::kPathAuto) path = x_layout == vv::kLayoutGemv ? vv::kPathGemv : vv::kPathMma;
     // Each kernel family reads one order of the activations.
     if ((path == vv::kPathGemv) != (x_layout == vv::kLayoutGemv)) return VV_ERR_UNSUPPORTED;
@@ -600,6 +860,8 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
 
     if (path == vv::kPathGemv) {
         // xsum (may be NULL) is only read here: the other kernels take the zero point off the codes
+        if (path_auto && M > vv::kGemvBestRows && N >= vv::kStreamMinRows && vv::launch_w4_stream(a, true, st))
+            return vv::launch_status();
         const int mr = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : 8;
         vv::W4Segs segs = {};
         segs.packed[0] = a.packed;
@@ -617,6 +879,8 @@ vv_status_t vv_w4a8_linear_dev(const int8_t* xq, int x_layout, const float* sx, 
         else vv::w4a8_gemv<8><<<grid, vv::kBlock, 0, st>>>(a);
         return vv::launch_status();
     }
+    // Asked for by name, the MMA path is the LDS-tiled kernel at every M.
+    if (path_auto && vv::launch_w4_stream(a, false, st)) return vv::launch_status();
     const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     if (M > 64 && wg128 >= 256) {
         if (!vv::launch_w4_tile<128, 128, 2, 2, 4>(a, st)) return VV_ERR_CUDA_LAUNCH;
