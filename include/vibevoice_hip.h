@@ -155,7 +155,10 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
  * order of xq inside every run of 32 columns: VV_Q8_W4_GEMV (2) for the GEMV
  * (M <= 8, K <= 20480), VV_Q8_W4_MMA (3) for the matrix-core tiles (any M);
  * AUTO takes the family the layout belongs to, and a family asked for with the
- * other layout declines (VV_ERR_UNSUPPORTED), as in the reference. xsum (the
+ * other layout declines (VV_ERR_UNSUPPORTED), as in the reference. Within a
+ * family AUTO may pick a third kernel that streams the weights (at most 64
+ * rows, group_size 64, 128 or 256; either order); a path asked for by name is
+ * the GEMV or the LDS-tiled kernel itself. xsum (the
  * quantiser's int32 [M][K/32] sums, may be NULL) saves the GEMV some integer
  * work and is not read otherwise; the result does not depend on it. Group
  * sums are exact int32 and the groups are added in order in FP32, nothing
