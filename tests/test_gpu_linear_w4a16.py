@@ -79,7 +79,8 @@ def test_dequant_bit_exact(N, K, G):
 
 
 WEIGHTS = [(3584, 3584, 128, False), (512, 3584, 128, False), (18944, 3584, 128, False), (3584, 18944, 128, False),
-           (1536, 8960, 32, True), (256, 1536, 64, True), (100, 96, 32, False), (8200, 512, 256, False)]
+           (1536, 8960, 32, True), (256, 1536, 64, True), (100, 96, 32, False), (8200, 512, 256, False),
+           (8216, 320, 64, True)]     # 32 weight rows per workgroup, a scale per chunk pair, a ragged last step
 
 
 @pytest.mark.parametrize("N,K,G,sym", WEIGHTS)

@@ -13,8 +13,8 @@
 //   w4a16_gemv      M <= 4: lanes take whole chunks, v_dot2_f32_f16 against the
 //                   natural half2 pairs of x; K split over waves or several
 //                   rows per wave by shape; up to three projections per launch
-//   w4a16_skinny    5 <= M <= 64: codes straight into 16x16x32 MFMA operands, K
-//                   split over the eight waves of a workgroup
+//   w4a16_skinny    5 <= M <= 64: codes dequantised in registers into 16x16x32
+//                   MFMA operands, K split over the eight waves of a workgroup
 //   w4a16_tile      larger M: the LDS-tiled 32x32x16 FP16 MFMA loop with the
 //                   codes dequantised on their way into LDS
 //   w4a16_gather    out[m][j] = x[m][perm[j]] (act-order checkpoints)
@@ -261,74 +261,101 @@ struct TileArgs {
 };
 
 // ── 5 <= M <= 64 ───────────────────────────────────────────────────────────
-// Sixteen weight rows per workgroup, K split over its eight waves, the codes
-// going from global memory straight into 16x16x32 MFMA operands: one chunk of
+// Sixteen or 32 weight rows per workgroup, K split over its eight waves, the
+// codes dequantised in registers into 16x16x32 MFMA operands: one chunk of
 // codes is one K step, lane (row, q) dequantises the chunk's q-th run of eight
 // columns (four half2 from the four words) and meets the same eight columns of
-// up to 64 activation rows. Bound by the code bytes; no LDS until the waves'
-// partial tiles are added.
+// up to 64 activation rows. Every chunk is loaded from global memory once (by
+// one lane of the four that need it) and passed round through LDS; the waves'
+// partial tiles are added at the end. Every workgroup reads all the
+// activations, which is most of the L2 traffic from 16 rows on.
 constexpr int kSkinnyWaves = 8;
 
-template <int kMT>
+template <int kMT, int kNT>
 __global__ __launch_bounds__(kSkinnyWaves * kWave) void w4a16_skinny(TileArgs a) {
-    __shared__ f32x4 part[kSkinnyWaves][kMT][kWave];
+    __shared__ f32x4 part[kSkinnyWaves][kMT * kNT][kWave];
+    __shared__ u32x4 staged[kSkinnyWaves][kNT][kWave];      // a wave's own 16 rows x 4 chunks of codes per tile
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, ks = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16;
+    const int n0 = (int)blockIdx.x * (16 * kNT);
     const int ncodes = a.K / 32, ng = a.K >> a.gshift;
-    const int row = min(n0 + r16, a.N - 1);
-    const u32x4* wrow = a.packed + (size_t)row * ncodes;
-    const uint32_t* szrow = a.sz + (size_t)row * ng;
+    // The four lanes of an operand row would each load the row's whole chunk for a quarter of its bits;
+    // instead lane l loads chunk l % 4 of row l / 4 once (64 bytes of a row side by side) and the wave
+    // hands the chunks round through its piece of LDS, which serves a wave's accesses in order.
+    const uint32_t* szrow[kNT];
+    const u32x4* lrow[kNT];
+#pragma unroll
+    for (int j = 0; j < kNT; ++j) {
+        szrow[j] = a.sz + (size_t)min(n0 + 16 * j + r16, a.N - 1) * ng;
+        lrow[j] = a.packed + (size_t)min(n0 + 16 * j + (lane >> 2), a.N - 1) * ncodes;
+    }
+    const int put = (lane >> 2) * 4 + swz<32>(lane >> 2, lane & 3);
+    const bool one_group = a.gshift >= 7;               // the four chunks of a step share their scale
     const u32x4* arow[kMT];
 #pragma unroll
     for (int t = 0; t < kMT; ++t)
         arow[t] = reinterpret_cast<const u32x4*>(a.a + (size_t)min(16 * t + r16, a.M - 1) * a.K);
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    f32x4 acc[kMT];
+    f32x4 acc[kMT][kNT];
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < kMT; ++t)
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) acc[t][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int c0 = wave * 4; c0 < ncodes; c0 += kSkinnyWaves * 4) {
-        u32x4 codes[4], x[kMT][4];
-        uint32_t gsz[4];
+        u32x4 mine[kNT], x[kMT][4];
+        uint32_t gsz[kNT][4];
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) {
+            mine[j] = __builtin_nontemporal_load(lrow[j] + min(c0 + (lane & 3), ncodes - 1));
+            if (one_group) gsz[j][0] = szrow[j][(c0 * 32) >> a.gshift];
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const bool live = c0 + u < ncodes;
             const int c = live ? c0 + u : ncodes - 1;
-            codes[u] = __builtin_nontemporal_load(wrow + c);
-            gsz[u] = szrow[(c * 32) >> a.gshift];
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) gsz[j][u] = one_group ? gsz[j][0] : szrow[j][(c * 32) >> a.gshift];
 #pragma unroll
             for (int t = 0; t < kMT; ++t) x[t][u] = live ? arow[t][c * 4 + ks] : zero;   // a dead step adds zero
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const GroupConst gc = group_const(gsz[u]);
-            u32x4 w;
-            w.x = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].x, ks, gc));
-            w.y = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].y, ks, gc));
-            w.z = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].z, ks, gc));
-            w.w = __builtin_bit_cast(uint32_t, dequant_pair(codes[u].w, ks, gc));
+        for (int j = 0; j < kNT; ++j) staged[wave][j][put] = mine[j];
 #pragma unroll
-            for (int t = 0; t < kMT; ++t)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, w),
-                                                                __builtin_bit_cast(h16x8, x[t][u]), acc[t], 0, 0, 0);
-        }
+        for (int j = 0; j < kNT; ++j)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const u32x4 codes = staged[wave][j][r16 * 4 + swz<32>(r16, u)];
+                const GroupConst gc = group_const(gsz[j][u]);
+                u32x4 w;
+                w.x = __builtin_bit_cast(uint32_t, dequant_pair(codes.x, ks, gc));
+                w.y = __builtin_bit_cast(uint32_t, dequant_pair(codes.y, ks, gc));
+                w.z = __builtin_bit_cast(uint32_t, dequant_pair(codes.z, ks, gc));
+                w.w = __builtin_bit_cast(uint32_t, dequant_pair(codes.w, ks, gc));
+#pragma unroll
+                for (int t = 0; t < kMT; ++t)
+                    acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, w),
+                                                                       __builtin_bit_cast(h16x8, x[t][u]), acc[t][j],
+                                                                       0, 0, 0);
+            }
     }
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    for (int t = 0; t < kMT; ++t)
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) part[wave][t * kNT + j][lane] = acc[t][j];
     __syncthreads();
 
-    // register r of lane l: column n0 + 4(l / 16) + r of row 16t + l % 16
-    if (tid < kMT * kWave) {
-        const int t = tid >> 6;
-        f32x4 sum = part[0][t][lane];
+    // register r of lane l: column n0 + 16 j + 4(l / 16) + r of row 16t + l % 16
+    if (tid < kMT * kNT * kWave) {
+        const int tile = tid >> 6, t = tile / kNT, j = tile % kNT;
+        f32x4 sum = part[0][tile][lane];
 #pragma unroll
         for (int w = 1; w < kSkinnyWaves; ++w) {
-            const f32x4 p = part[w][t][lane];
+            const f32x4 p = part[w][tile][lane];
 #pragma unroll
             for (int r = 0; r < 4; ++r) sum[r] += p[r];
         }
-        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        const int m = 16 * t + r16, n = n0 + 16 * j + 4 * ks;
         if (m < a.M && n < a.N) {
             h16* crow = a.c + (size_t)m * a.N;
             if (a.vec && n + 3 < a.N) {
@@ -633,13 +660,19 @@ vv_status_t vv_w4a16_gemm_dev(const void* A, const void* packed, const void* sz,
     a.gshift = gs;
     a.vec = (N % 4 == 0) && !(reinterpret_cast<uintptr_t>(C) & 7u) && !(bias && (reinterpret_cast<uintptr_t>(bias) & 7u));
     // Beyond 16 rows a wide layer re-reads the activations once per 16 columns: tiles serve it better.
-    if (M <= 16 || (M <= 64 && (N + 63) / 64 < 200)) {
-        const dim3 grid((unsigned)((N + 15) / 16));
+    if (M <= 32 || (M <= 64 && (N + 63) / 64 < 200)) {
         constexpr int kThreads = vv::kSkinnyWaves * vv::kWave;
-        if (M <= 16) vv::w4a16_skinny<1><<<grid, kThreads, 0, st>>>(a);
-        else if (M <= 32) vv::w4a16_skinny<2><<<grid, kThreads, 0, st>>>(a);
-        else if (M <= 48) vv::w4a16_skinny<3><<<grid, kThreads, 0, st>>>(a);
-        else vv::w4a16_skinny<4><<<grid, kThreads, 0, st>>>(a);
+        // Every workgroup reads all the activations: with 256+ workgroups left, 32 weight rows each
+        // halve that traffic (gate or up at 28 rows: 36 -> 27 us; down, 112 workgroups: 38 -> 46).
+        const bool two = M <= 32 && N >= 8192;
+        const dim3 grid((unsigned)((N + (two ? 31 : 15)) / (two ? 32 : 16)));
+        if (two) {
+            if (M <= 16) vv::w4a16_skinny<1, 2><<<grid, kThreads, 0, st>>>(a);
+            else vv::w4a16_skinny<2, 2><<<grid, kThreads, 0, st>>>(a);
+        } else if (M <= 16) vv::w4a16_skinny<1, 1><<<grid, kThreads, 0, st>>>(a);
+        else if (M <= 32) vv::w4a16_skinny<2, 1><<<grid, kThreads, 0, st>>>(a);
+        else if (M <= 48) vv::w4a16_skinny<3, 1><<<grid, kThreads, 0, st>>>(a);
+        else vv::w4a16_skinny<4, 1><<<grid, kThreads, 0, st>>>(a);
         return vv::launch_status();
     }
     const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
