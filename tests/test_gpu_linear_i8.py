@@ -380,6 +380,42 @@ def test_w4a8_follows_the_device_quantiser():
         same_f32(d_y.cpu().numpy(), want32, f"layout {lay}")
 
 
+@pytest.mark.parametrize("M,layout", [(6, L_GEMV), (29, L_MMA)])
+def test_w4a8_streamed_rows_replay_from_a_graph(M, layout):
+    """Quantiser + W4A8 layer at the row counts of the streamed kernel, captured once (the kernel's first use may
+    fall inside the capture) and replayed on new activations, the program's own work in between: every replay
+    gives the oracle's bits."""
+    N, K, G = 2080, 3584, 128
+    p = w4_problem(M, N, K, G, 23)
+    d_w, d_sz = i8_dev(p["gpu"]), i8_dev(p["sz"])
+    d_x = torch.zeros((M, K), dtype=torch.float16, device="cuda")
+    d_xq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    d_sx = torch.empty(M, dtype=torch.float32, device="cuda")
+    d_xs = torch.empty((M, K // 32), dtype=torch.int32, device="cuda")
+    d_y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    s = C.c_void_p()
+    assert dev.vv_dev_stream_create(C.byref(s)) == dev.VV_OK
+    st = s.value
+    torch.cuda.synchronize()
+    assert dev.vv_dev_graph_begin(st) == dev.VV_OK
+    ok(dev.vv_act_quant_dev(d_x.data_ptr(), M, K, layout, d_xq.data_ptr(), d_sx.data_ptr(), d_xs.data_ptr(), st))
+    ok(dev.vv_w4a8_linear_dev(d_xq.data_ptr(), layout, d_sx.data_ptr(), d_xs.data_ptr(), d_w.data_ptr(),
+                              d_sz.data_ptr(), G, None, None, d_y.data_ptr(), 1, M, N, K, AUTO, st))
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(st, C.byref(g)) == dev.VV_OK and g.value
+    for i in range(3):
+        x = oracle.normal_f16((M, K), 30 + i, std=1.0 + i)
+        d_x.copy_(torch.from_numpy(x.view(np.float16)))
+        torch.cuda.synchronize()
+        assert dev.vv_dev_graph_launch(g.value, st) == dev.VV_OK
+        assert dev.vv_dev_stream_sync(st) == dev.VV_OK
+        xq, sx, _ = oracle.quant_act_q8(oracle.widen(x), 0, want_xsum=False)
+        want32, _ = oracle.w4a8_linear(xq, sx, p["packed"], p["scales"], p["zeros"], G)
+        same_f32(d_y.cpu().numpy(), want32, f"replay {i}")
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(st)
+
+
 @pytest.mark.parametrize("M,layout", [(2, L_GEMV), (40, L_MMA), (7, L_GEMV), (6, L_GEMV)])
 def test_i8_linear_multi_w4(M, layout):
     """One launch for all projections or one call each (M = 6: wide projections of
