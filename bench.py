@@ -317,21 +317,21 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del xq, sx, c
         # the same codes against FP16 activations (W4A16)
-        for m, key in ((T, "w4a16"), (1, "w4a16_gemv")):
+        for m, key in ((T, "w4a16"), (1, "w4a16_gemv"), (29, "w4a16_chunk")):
             out.setdefault(key, {})
             a = torch.randn(m, k, dtype=torch.float16, device="cuda")
             c = torch.empty(m, n, dtype=torch.float16, device="cuda")
             dense = torch.empty(n * k, dtype=torch.float16, device="cuda")     # the decoder's dequant scratch
             sec = timed(lambda: dev.vv_w4a16_gemm_dev(a.data_ptr(), w4.data_ptr(), sz.data_ptr(), None, c.data_ptr(),
                                                       dense.data_ptr(), n * k * 2, m, n, k, G, st),
-                        5 if m > 1 else 50)
-            if m > 1:
+                        5 if m > 64 else 50)
+            if m > 64:
                 tf = 2.0 * m * n * k / sec / 1e12
                 out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TFLOPs": tf,
                                   "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
             else:
-                gb = (n * k / 2 + n * (k // G) * 4 + 2.0 * k + 2.0 * n) / sec / 1e9
-                out[key][name] = {"N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                gb = (n * k / 2 + n * (k // G) * 4 + m * (2.0 * k + 2.0 * n)) / sec / 1e9
+                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del a, c, dense
         del w4, sz
@@ -1096,6 +1096,8 @@ def main() -> int:
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         for name, d in layer["w4a16_gemv"].items():
             log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        for name, d in layer["w4a16_chunk"].items():
+            log(f"  w4a16 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
         for name, d in layer["weight_only"].items():
             log(f"  weight-only {name:18s} N={d['N']} K={d['K']}: one row {d['M1_us']:7.2f} us {d['M1_GBps']:7.1f} GB/s, "
                 f"29 rows {d['M29_us']:7.2f} us, dequantise {d['dequant_us']:7.2f} us {d['dequant_GBps']:7.1f} GB/s")
