@@ -538,6 +538,23 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv,
 vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv,
                            void* out, int n_q_heads, int cache_len,
                            const int* d_cache_len, void* scratch, void* stream);
+/* vv_attn_decode without the scratch argument, for callers that cannot
+ * allocate device memory (code under graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the slices' partial states live in a
+ * file-scope device array of the library, 8.25 MiB per GPU, held until the
+ * process ends. It calls no hipMalloc, hipFree or other allocating routine.
+ * Same arguments, results (bit for bit) and status codes as vv_attn_decode;
+ * additionally VV_ERR_INVALID_ARG when the split path would need more than
+ * VV_ATTN_DECODE_STATIC_MAX_Q_HEADS query heads of partial states, and
+ * VV_ERR_CUDA when the array's address cannot be resolved. All calls on one
+ * GPU share that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race, so serialise them or use vv_attn_decode with a buffer per
+ * context. The array's address is resolved at the first call on each device:
+ * make that call outside a graph capture. No counterpart in the reference. */
+#define VV_ATTN_DECODE_STATIC_MAX_Q_HEADS 64
+vv_status_t vv_attn_decode_static(int backend, const void* q, const vv_kv_view_t* kv,
+                                  void* out, int n_q_heads, int cache_len,
+                                  const int* d_cache_len, void* stream);
 /* The older entry points for raw FP16 caches: the cache as two pointers
  * instead of a view, otherwise vv_attn_scratch_bytes, vv_attn_decode_shape,
  * vv_attn_decode and vv_attn_prefill. replace device.h:621-655. */

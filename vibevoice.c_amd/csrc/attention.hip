@@ -25,6 +25,8 @@
 //                leave (max, sum, unnormalised O) in the caller's scratch
 //                and decode_merge folds them.
 //   rows_generic any head_dim <= 256, any alignment: one wave per (row, head).
+#include <atomic>
+
 #include "vv_common.hpp"
 
 namespace vv {
@@ -922,6 +924,13 @@ bool shape_ok(int n_q_heads, int n_kv_heads, int head_dim) {
            head_dim <= 256;
 }
 
+// Whether a decode over this view runs decode128 (and, past 1024 positions, needs the
+// partial-state buffer) rather than the wave-per-head kernel.
+bool decode_on_matrix_cores(const void* q, const vv_kv_view_t* kv) {
+    return packed_format(kv->format) ||
+           (kv->head_dim == kD && aligned16(q) && aligned16(kv->k) && aligned16(kv->v));
+}
+
 }  // namespace
 }  // namespace vv
 
@@ -994,36 +1003,35 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     return vv::launch_status();
 }
 
-vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, void* out,
-                           int n_q_heads, int cache_len, const int* d_cache_len, void* scratch,
-                           void* stream) {
-    (void)backend;
-    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
-    if (cache_len <= 0) return VV_OK;
-    if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
-    const bool packed = vv::packed_format(kv->format);
-    if (kv->format != vv::kFormatFp16 && !packed) return VV_ERR_UNSUPPORTED;
-    if (!vv::shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
-    if (packed && (!vv::packed_view_ok(kv) || !vv::aligned16(q))) return VV_ERR_UNSUPPORTED;
-    hipStream_t st = vv::as_stream(stream);
-    const float scale_log2 = vv::kLog2e / sqrtf((float)kv->head_dim);
-    const vv::h16* Q = static_cast<const vv::h16*>(q);
-    const vv::h16* K = static_cast<const vv::h16*>(kv->k);
-    const vv::h16* V = static_cast<const vv::h16*>(kv->v);
-    vv::h16* O = static_cast<vv::h16*>(out);
-    const vv::KvSource src = {kv->k, kv->v, static_cast<const vv::h16*>(kv->k_meta),
-                              static_cast<const vv::h16*>(kv->v_meta), kv->page_table};
-    if (packed || (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v))) {
-        const int n_parts = vv::decode_parts(cache_len);
-        if (n_parts > 1 && !scratch) return VV_ERR_NULL_PTR;
+}  // extern "C" (reopened below)
+
+namespace vv {
+namespace {
+
+// The split decode: decode128 over the slices, then decode_merge. `parts` holds
+// the slices' partial states (vv_attn_scratch_bytes() of device memory); every
+// (head, slice) record the merge reads is written by decode128 in the same call,
+// empty slices included, so the buffer needs no clearing between calls.
+vv_status_t attn_decode_launch(const void* q, const vv_kv_view_t* kv, void* out, int n_q_heads,
+                               int cache_len, const int* d_cache_len, float* parts,
+                               hipStream_t st) {
+    const bool packed = packed_format(kv->format);
+    const float scale_log2 = kLog2e / sqrtf((float)kv->head_dim);
+    const h16* Q = static_cast<const h16*>(q);
+    const h16* K = static_cast<const h16*>(kv->k);
+    const h16* V = static_cast<const h16*>(kv->v);
+    h16* O = static_cast<h16*>(out);
+    const KvSource src = {kv->k, kv->v, static_cast<const h16*>(kv->k_meta),
+                          static_cast<const h16*>(kv->v_meta), kv->page_table};
+    if (decode_on_matrix_cores(q, kv)) {
+        const int n_parts = decode_parts(cache_len);
+        if (n_parts > 1 && !parts) return VV_ERR_NULL_PTR;
         const int group = n_q_heads / kv->n_kv_heads;
         const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads, (unsigned)((group + 31) / 32));
-        float* parts = static_cast<float*>(scratch);
-#define VV_DECODE(F)                                                                                       \
-    vv::decode128<vv::F><<<grid, vv::kWave, 0, st>>>(Q, src, O, parts, n_q_heads, kv->n_kv_heads, cache_len, \
-                                                     d_cache_len, n_parts, scale_log2)
+#define VV_DECODE(F)                                                                                  \
+    decode128<F><<<grid, kWave, 0, st>>>(Q, src, O, parts, n_q_heads, kv->n_kv_heads, cache_len,     \
+                                         d_cache_len, n_parts, scale_log2)
         if (packed) {
-            using namespace vv;
             VV_FOR_PACKED_FORMAT(kv->format, VV_DECODE)
         } else {
             VV_DECODE(kFmtFp16);
@@ -1031,17 +1039,93 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, v
 #undef VV_DECODE
         if (n_parts > 1) {
             if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
-            vv::decode_merge<<<dim3((unsigned)n_q_heads), vv::kMergeThreads, 0, st>>>(
-                static_cast<const float*>(scratch), O, n_parts);
+            decode_merge<<<dim3((unsigned)n_q_heads), kMergeThreads, 0, st>>>(parts, O, n_parts);
         }
     } else {
         // One row: position cache_len - 1 sees everything, so no mask is needed.
         const dim3 grid(1u, (unsigned)n_q_heads);
-        vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
-                                                     kv->n_kv_heads, kv->head_dim, 1, 0, cache_len,
-                                                     d_cache_len, 0, scale_log2);
+        rows_generic<<<grid, kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads, kv->n_kv_heads,
+                                             kv->head_dim, 1, 0, cache_len, d_cache_len, 0, scale_log2);
     }
-    return vv::launch_status();
+    return launch_status();
+}
+
+// Argument checks shared by the two decode entry points; VV_OK means "launch".
+vv_status_t attn_decode_check(const void* q, const vv_kv_view_t* kv, const void* out, int n_q_heads) {
+    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
+    if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
+    const bool packed = packed_format(kv->format);
+    if (kv->format != kFormatFp16 && !packed) return VV_ERR_UNSUPPORTED;
+    if (!shape_ok(n_q_heads, kv->n_kv_heads, kv->head_dim)) return VV_ERR_UNSUPPORTED;
+    if (packed && (!packed_view_ok(kv) || !aligned16(q))) return VV_ERR_UNSUPPORTED;
+    return VV_OK;
+}
+
+// ── the library's own partial-state buffer, for callers that cannot allocate ──
+// One array per GPU the library runs on, held until the process ends. In host
+// code the array's name is only a handle for hipGetSymbolAddress: the device
+// address is looked up once per device (with that device current) and only that
+// address is ever handed to a kernel.
+constexpr int kStaticMaxQHeads = VV_ATTN_DECODE_STATIC_MAX_Q_HEADS;
+constexpr size_t kStaticFloats = (size_t)kStaticMaxQHeads * kMaxParts * kPartFloats;   // 8.25 MiB
+static __device__ __align__(256) float scratch[kStaticFloats];
+
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+float* static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        p = static_cast<float*>(sym);      // every thread that races here finds the same address
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    return p;
+}
+
+}  // namespace
+}  // namespace vv
+
+extern "C" {
+
+vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv, void* out,
+                           int n_q_heads, int cache_len, const int* d_cache_len, void* scratch,
+                           void* stream) {
+    (void)backend;
+    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
+    if (cache_len <= 0) return VV_OK;
+    const vv_status_t rc = vv::attn_decode_check(q, kv, out, n_q_heads);
+    if (rc != VV_OK) return rc;
+    return vv::attn_decode_launch(q, kv, out, n_q_heads, cache_len, d_cache_len,
+                                  static_cast<float*>(scratch), vv::as_stream(stream));
+}
+
+/* vv_attn_decode with the slices' partial states in the library's own
+ * file-scope device array instead of a caller's buffer: no hipMalloc, hipFree
+ * or other allocating call, here or below. */
+vv_status_t vv_attn_decode_static(int backend, const void* q, const vv_kv_view_t* kv, void* out,
+                                  int n_q_heads, int cache_len, const int* d_cache_len,
+                                  void* stream) {
+    (void)backend;
+    if (!q || !kv || !out) return VV_ERR_NULL_PTR;
+    if (cache_len <= 0) return VV_OK;
+    const vv_status_t rc = vv::attn_decode_check(q, kv, out, n_q_heads);
+    if (rc != VV_OK) return rc;
+    float* parts = nullptr;
+    if (vv::decode_on_matrix_cores(q, kv) && vv::decode_parts(cache_len) > 1) {
+        // the partial states are [n_q_heads][slices][head_dim + 4] floats, head_dim 128 on this path
+        if (n_q_heads > vv::kStaticMaxQHeads) return VV_ERR_INVALID_ARG;
+        parts = vv::static_scratch();
+        if (!parts) return VV_ERR_CUDA;
+    }
+    return vv::attn_decode_launch(q, kv, out, n_q_heads, cache_len, d_cache_len, parts,
+                                  vv::as_stream(stream));
 }
 
 /* The older entry points for raw FP16 caches (device.h:621-655): the same

@@ -19,6 +19,7 @@ VV_ERR_UNSUPPORTED = -7
 VV_ERR_CUDA = -100
 VV_ERR_CUDA_OOM = -101
 VV_ERR_CUDA_LAUNCH = -102
+VV_ATTN_DECODE_STATIC_MAX_Q_HEADS = 64    # include/vibevoice_hip.h
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
                         "libvibevoice_hip.so")
@@ -96,6 +97,7 @@ SIGNATURES = {
     "vv_attn_decode_shape": (_i, [_i, _i, _i, _i]),
     "vv_attn_prefill": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, C.c_bool, _vp, _vp]),
     "vv_attn_decode": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "vv_attn_decode_static": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "vv_kv_quant_store_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_bool, _i, _i, _i, _vp, _i, _i, _vp]),
     "vv_kv_dequant_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "vv_gqa_attention_decode_q_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
