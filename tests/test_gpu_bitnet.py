@@ -11,6 +11,10 @@ from gpu_util import dev, ok, stream
 
 pytestmark = pytest.mark.gpu
 
+NOT_BUILT = ("BitNet's requantiser and int8 tied head are not built in this backend (their first versions followed "
+             "the reference's CUDA kernels too closely and were removed; the component is outside the layer-kernel "
+             "scope): the entry points answer VV_ERR_UNSUPPORTED")
+
 
 def D(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -94,19 +98,16 @@ def test_int8_product_bit_exact(M, N, K):
     assert np.array_equal(host(d_acc), acc)
     assert np.array_equal(host(d_y).view(np.uint32), y.view(np.uint32))
     assert float(host(d_am)[0]) == am
-    # then the requantisation that follows it in the encoder, reading the folded maximum from device memory
-    for relu in (False, True):
-        want_q, want_inv = oracle.i8s_requant(y, am, relu)
-        d_rq = torch.full((M, N), 99, dtype=torch.int8, device="cuda")
-        d_inv = torch.zeros(1, dtype=torch.float32, device="cuda")
-        ok(dev.vv_i8s_requant_dev(P(d_y), M * N, P(d_am), int(relu), P(d_rq), P(d_inv), stream()))
-        assert np.array_equal(host(d_rq), want_q) and float(host(d_inv)[0]) == want_inv
+    # the requantisation that follows it in the encoder is not built in this backend
+    d_rq = torch.full((M, N), 99, dtype=torch.int8, device="cuda")
+    assert dev.vv_i8s_requant_dev(P(d_y), M * N, P(d_am), 0, P(d_rq), None, stream()) == dev.VV_ERR_UNSUPPORTED
     # accumulators only
     d_acc.fill_(-7)
     ok(dev.vv_i8_gemm_dev(P(d_a), None, P(d_w), 0.004, None, P(d_acc), None, None, M, N, K, stream()))
     assert np.array_equal(host(d_acc), acc)
 
 
+@pytest.mark.skip(reason=NOT_BUILT)
 def test_requant_of_all_zero_tensor():
     d_y = torch.zeros(1000, dtype=torch.float32, device="cuda")
     d_am = torch.zeros(1, dtype=torch.float32, device="cuda")
@@ -116,6 +117,7 @@ def test_requant_of_all_zero_tensor():
     assert host(d_q).max() == 0 and host(d_q).min() == 0 and float(host(d_inv)[0]) == 0.0
 
 
+@pytest.mark.skip(reason=NOT_BUILT)
 @pytest.mark.parametrize("V,K", [(40, 64), (1000, 1536), (151936, 1536), (777, 100)])
 def test_int8_head_argmax(V, K):
     rng = np.random.default_rng(V + K)
@@ -151,12 +153,12 @@ def test_argument_checks():
     assert dev.vv_ternary_gemm_dev(p, p, p, p, 1.0, None, p, None, 0, 1, 8, 64, s) == I           # K % 128
     assert dev.vv_i8_gemm_dev(p, None, p, 1.0, None, None, p, None, 1, 8, 64, s) == N             # y without a_scale
     assert dev.vv_i8_gemm_dev(p, p, p, 1.0, None, p, None, None, 0, 8, 64, s) == I
-    assert dev.vv_i8s_requant_dev(p, 0, p, 0, p, None, s) == I
-    assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 6, p, None, p, s) == I                        # K % 4
-    assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 64, p, None, None, s) == N
+    assert dev.vv_i8s_requant_dev(p, 8, p, 0, p, None, s) == dev.VV_ERR_UNSUPPORTED               # not built
+    assert dev.vv_i8_head_argmax_dev(p, p, p, p, 8, 64, p, None, p, s) == dev.VV_ERR_UNSUPPORTED  # not built
     assert dev.vv_i8_head_argmax_scratch_bytes(0) == 0
 
 
+@pytest.mark.skip(reason=NOT_BUILT)
 def test_bitnet_decode_ops_replay_from_a_graph():
     """Every per-token value (activation scale, row sum, the head's scale) is read from device memory, so a captured
     quantise -> ternary product -> int8 head sequence replays on new inputs: each replay equals the eager run."""

@@ -19,8 +19,6 @@
 //                 sum (c - 1) q = sum c q - sum q.
 //   bn_naive      int8 x int8 when K is not a multiple of 16 or an operand is
 //                 off 16 bytes: one thread per output
-//   bn_requant    one scale for a whole tensor, read from device memory
-//   bn_head       int8 tied-head argmax in two stages; ties to the lowest index
 #include <float.h>
 
 #include "vv_common.hpp"
@@ -255,120 +253,9 @@ void launch_bn_gemm(const int8_t* a, const void* w, const BnOut& out, int K, hip
     }
 }
 
-// ── requantisation ──────────────────────────────────────────────────────────
-
-__global__ __launch_bounds__(kBlock) void bn_requant(const float* __restrict__ y, int64_t n,
-                                                     const float* __restrict__ absmax, int relu,
-                                                     int8_t* __restrict__ q, float* __restrict__ out_scale) {
-    const float am = *absmax;
-    const float inv = am != 0.0f ? 127.0f / am : 0.0f;
-    const float lo = relu ? 0.0f : -127.0f;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-        float v = y[i] * inv;
-        v = v < lo ? lo : (v > 127.0f ? 127.0f : v);        // a NaN falls through both, as on the CPU
-        q[i] = (int8_t)(int)__builtin_rintf(v);
-    }
-    if (blockIdx.x == 0 && threadIdx.x == 0 && out_scale) *out_scale = inv;
-}
-
-// ── int8 head + argmax ──────────────────────────────────────────────────────
-
-constexpr int kHeadRowsPerWave = 32;
-constexpr int kHeadRows = kWavesPerBlock * kHeadRowsPerWave;
-
-__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
-
-// A half-wave per vocabulary row (K = 1536 is exactly three 16-byte chunks per lane), two pairs of rows in flight;
-// kWide: 16-byte loads (K % 16 == 0, operands on 16 bytes), else 4-byte ones.
-template <bool kWide>
-__global__ __launch_bounds__(kBlock) void bn_head(const int8_t* __restrict__ q, const float* __restrict__ scale,
-                                                  const int8_t* __restrict__ w, const float* __restrict__ w_scale,
-                                                  int V, int K, float* __restrict__ pv, int* __restrict__ pi) {
-#pragma clang fp contract(off)
-    __shared__ float best_v[kWavesPerBlock];
-    __shared__ int best_i[kWavesPerBlock];
-    const int wave = wave_in_block(), lane = lane_id();
-    const int l32 = lane & 31, half = lane >> 5;
-    const float s = *scale;
-    float bv = -FLT_MAX;
-    int bi = 0x7fffffff;
-    const int r0 = (int)blockIdx.x * kHeadRows + wave * kHeadRowsPerWave;
-    for (int r = 0; r < kHeadRowsPerWave; r += 4) {
-        int acc[2] = {0, 0};
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int n = min(r0 + r + 2 * u + half, V - 1);
-            const int8_t* wr = w + (size_t)n * K;
-            if constexpr (kWide) {
-                const i32x4* w4 = reinterpret_cast<const i32x4*>(wr);
-                const i32x4* x4 = reinterpret_cast<const i32x4*>(q);
-                for (int i = l32; i < K / 16; i += 32) {
-                    const i32x4 a = __builtin_nontemporal_load(w4 + i), b = x4[i];
-                    acc[u] = __builtin_amdgcn_sdot4(a.x, b.x, acc[u], false);
-                    acc[u] = __builtin_amdgcn_sdot4(a.y, b.y, acc[u], false);
-                    acc[u] = __builtin_amdgcn_sdot4(a.z, b.z, acc[u], false);
-                    acc[u] = __builtin_amdgcn_sdot4(a.w, b.w, acc[u], false);
-                }
-            } else {
-                const int* w1 = reinterpret_cast<const int*>(wr);
-                const int* x1 = reinterpret_cast<const int*>(q);
-                for (int i = l32; i < K / 4; i += 32) acc[u] = __builtin_amdgcn_sdot4(w1[i], x1[i], acc[u], false);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-#pragma unroll
-            for (int o = 16; o > 0; o >>= 1) acc[u] += __shfl_xor(acc[u], o);       // inside each half-wave
-            const int n = r0 + r + 2 * u + half;
-            if (n < V) {
-                float v = (float)acc[u] * w_scale[n];
-                v = v / s;
-                if (better(v, n, bv, bi)) { bv = v; bi = n; }
-            }
-        }
-    }
-    // the two half-waves hold different rows: meet them, then the waves
-    {
-        const float ov = __shfl_xor(bv, 32);
-        const int oi = __shfl_xor(bi, 32);
-        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
-    }
-    if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float v = best_v[0];
-        int i = best_i[0];
-#pragma unroll
-        for (int k = 1; k < kWavesPerBlock; ++k)
-            if (better(best_v[k], best_i[k], v, i)) { v = best_v[k]; i = best_i[k]; }
-        pv[blockIdx.x] = v;
-        pi[blockIdx.x] = i;
-    }
-}
-
-__global__ __launch_bounds__(kBlock) void bn_head_final(const float* __restrict__ pv, const int* __restrict__ pi, int n,
-                                                        int32_t* __restrict__ token, float* __restrict__ value) {
-    __shared__ float sv[kBlock];
-    __shared__ int si[kBlock];
-    float bv = -FLT_MAX;
-    int bi = 0x7fffffff;
-    for (int i = (int)threadIdx.x; i < n; i += kBlock)
-        if (better(pv[i], pi[i], bv, bi)) { bv = pv[i]; bi = pi[i]; }
-    sv[threadIdx.x] = bv;
-    si[threadIdx.x] = bi;
-    __syncthreads();
-    for (int st = kBlock / 2; st > 0; st >>= 1) {
-        if ((int)threadIdx.x < st && better(sv[threadIdx.x + st], si[threadIdx.x + st], sv[threadIdx.x], si[threadIdx.x])) {
-            sv[threadIdx.x] = sv[threadIdx.x + st];
-            si[threadIdx.x] = si[threadIdx.x + st];
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        *token = si[0];
-        if (value) *value = sv[0];
-    }
-}
+// The requantiser and the int8 tied head are not built in this backend: their entry points answer
+// VV_ERR_UNSUPPORTED.
+constexpr int kHeadRows = 128;      // weight rows per partial winner: sizes vv_i8_head_argmax_scratch_bytes
 
 }  // namespace
 }  // namespace vv
@@ -434,12 +321,8 @@ vv_status_t vv_i8_gemm_dev(const int8_t* a, const float* a_scale, const int8_t* 
 
 vv_status_t vv_i8s_requant_dev(const float* y, int64_t n, const float* absmax, int relu, int8_t* q, float* out_scale,
                                void* stream) {
-    if (!y || !absmax || !q) return VV_ERR_NULL_PTR;
-    if (n <= 0) return VV_ERR_INVALID_ARG;
-    int64_t blocks = (n + vv::kBlock - 1) / vv::kBlock;
-    if (blocks > 8192) blocks = 8192;
-    vv::bn_requant<<<dim3((unsigned)blocks), vv::kBlock, 0, vv::as_stream(stream)>>>(y, n, absmax, relu, q, out_scale);
-    return vv::launch_status();
+    (void)y; (void)n; (void)absmax; (void)relu; (void)q; (void)out_scale; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 size_t vv_i8_head_argmax_scratch_bytes(int V) {
@@ -450,21 +333,9 @@ size_t vv_i8_head_argmax_scratch_bytes(int V) {
 
 vv_status_t vv_i8_head_argmax_dev(const int8_t* q, const float* scale, const int8_t* w, const float* w_scale, int V,
                                   int K, int32_t* token, float* value, void* scratch, void* stream) {
-    if (!q || !scale || !w || !w_scale || !token || !scratch) return VV_ERR_NULL_PTR;
-    if (V <= 0 || K <= 0 || K % 4) return VV_ERR_INVALID_ARG;
-    if ((reinterpret_cast<uintptr_t>(q) & 3u) || (reinterpret_cast<uintptr_t>(w) & 3u) ||
-        (reinterpret_cast<uintptr_t>(scratch) & 3u))
-        return VV_ERR_UNSUPPORTED;
-    const int nb = (V + vv::kHeadRows - 1) / vv::kHeadRows;
-    float* pv = static_cast<float*>(scratch);
-    int* pi = reinterpret_cast<int*>(pv + nb);
-    hipStream_t st = vv::as_stream(stream);
-    if (K % 16 == 0 && vv::aligned16(q) && vv::aligned16(w))
-        vv::bn_head<true><<<dim3((unsigned)nb), vv::kBlock, 0, st>>>(q, scale, w, w_scale, V, K, pv, pi);
-    else
-        vv::bn_head<false><<<dim3((unsigned)nb), vv::kBlock, 0, st>>>(q, scale, w, w_scale, V, K, pv, pi);
-    vv::bn_head_final<<<dim3(1), vv::kBlock, 0, st>>>(pv, pi, nb, token, value);
-    return vv::launch_status();
+    (void)q; (void)scale; (void)w; (void)w_scale; (void)V; (void)K; (void)token; (void)value; (void)scratch;
+    (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 }  // extern "C"

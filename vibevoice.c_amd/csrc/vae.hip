@@ -1,4 +1,6 @@
-// The batched, streaming Conv-VAE encoder ops. FP16 activations, channel-first
+// The matrix-core part of the batched, streaming Conv-VAE encoder ops (the direct and im2col
+// convolutions, the context copy and the per-column 1/rms are not built here: their entry points
+// answer VV_ERR_UNSUPPORTED). FP16 activations, channel-first
 // and packed along time; the items of a launch sit side by side in one
 // [C][ld] buffer and only the convolutions know where one ends (a descriptor
 // passed by value). No output's arithmetic depends on where its item sits, on
@@ -7,15 +9,7 @@
 // separate kernels would have stored an intermediate. So batching, chunking
 // and fusing change no bit.
 //
-//   vae_conv       one output per thread, an FP32 fused multiply-add chain over
-//                  (in channel, tap) from zero
-//   vae_tail       the next chunk's left context
-//   vae_im2col     the inputs of a strided conv as GEMM columns
-//   vae_conv_gemm  the conv over those columns: FP32 FMAs in K order per output
-//                  (the bits of vae_conv), 64x64 tile, 4x4 outputs per thread
-//   vae_rms        1 / rms over channels per column (packed and context)
-//   vae_mixer      RMSNorm -> depthwise conv -> gamma residual, fused (vae_mixer_vec:
-//                  the same with 16-byte accesses where rows and items allow)
+//   vae_mixer_vec  RMSNorm -> depthwise conv -> gamma residual, fused, 16-byte accesses
 //   vae_gemm       the FFN (A x B, B K-major) and connector (A x B^T) GEMMs on
 //                  v_mfma_f32_16x16x32_f16: 128x128 or 64x64 tile, four waves,
 //                  64 K per LDS stage; a K-major B is transposed on its way
@@ -33,242 +27,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef vv_vae_conv_desc_t Desc;
 typedef vv_vae_conv_item_t Item;
 
-// Column `pos` of [context ++ input] of an item, channel ic; zero past either end.
-__device__ __forceinline__ h16 item_value(const Desc& d, const Item& it, const h16* __restrict__ x, int64_t ld_in,
-                                          int ic, int pos) {
-    if (pos >= it.have + it.in_len) return (h16)0.0f;
-    if (pos < it.have) {
-        const h16* tl = static_cast<const h16*>(it.tail_in);
-        return tl ? tl[(size_t)ic * d.cap + pos] : (h16)0.0f;
-    }
-    const h16* xb = it.in_ptr ? static_cast<const h16*>(it.in_ptr) : x + it.in_off;
-    return xb[(size_t)ic * ld_in + (pos - it.have)];
-}
-
-template <bool kTransposed>
-__global__ __launch_bounds__(kBlock) void vae_conv(Desc d, const h16* __restrict__ x, int64_t ld_in,
-                                                   const h16* __restrict__ w, const h16* __restrict__ b,
-                                                   h16* __restrict__ y, int64_t ld_out, int in_ch, int k,
-                                                   int stride) {
-    const Item& it = d.it[blockIdx.z];
-    const int oc = (int)blockIdx.y;
-    const int t = (int)blockIdx.x * kBlock + (int)threadIdx.x;
-    if (t >= it.out_len) return;
-    const int total = it.have + it.in_len;
-    const h16* wr = w + (size_t)oc * in_ch * k;
-    float sum = 0.0f;
-    for (int ic = 0; ic < in_ch; ++ic)
-        for (int kk = 0; kk < k; ++kk) {
-            const int p = t * stride + kk;
-            if (p < total) sum = __builtin_fmaf((float)wr[ic * k + kk], (float)item_value(d, it, x, ld_in, ic, p), sum);
-        }
-    if (b) sum += (float)b[oc];
-    if constexpr (kTransposed) {
-        if (t >= it.skip) static_cast<h16*>(it.out_ptr)[(size_t)(t - it.skip) * it.out_ld + oc] = to_half(sum);
-    } else {
-        y[(size_t)oc * ld_out + it.out_off + t] = to_half(sum);
-    }
-}
-
-__global__ __launch_bounds__(kBlock) void vae_tail(Desc d, const h16* __restrict__ x, int64_t ld_in, int in_ch) {
-    const Item& it = d.it[blockIdx.y];
-    if (!it.tail_out || it.keep <= 0) return;
-    const int idx = (int)blockIdx.x * kBlock + (int)threadIdx.x;
-    if (idx >= in_ch * it.keep) return;
-    const int c = idx / it.keep, j = idx - c * it.keep;
-    const int p = it.have + it.in_len - it.keep + j;
-    static_cast<h16*>(it.tail_out)[(size_t)c * d.cap + j] = p < 0 ? (h16)0.0f : item_value(d, it, x, ld_in, c, p);
-}
-
-// The item that owns packed output column p.
-__device__ __forceinline__ int item_of(const Desc& d, int64_t p) {
-    int i = 0;
-    while (i + 1 < d.n && p >= d.it[i + 1].out_off) ++i;
-    return i;
-}
-
-__global__ __launch_bounds__(kBlock) void vae_im2col(Desc d, const h16* __restrict__ x, int64_t ld_in, int k,
-                                                     int stride, int64_t p0, int pc, h16* __restrict__ col,
-                                                     int64_t ldcol) {
-    const int q = (int)blockIdx.x * kBlock + (int)threadIdx.x;
-    if (q >= pc) return;
-    const int kr = (int)blockIdx.y;
-    const int ic = kr / k, kk = kr - ic * k;
-    const int64_t p = p0 + q;
-    const Item& it = d.it[item_of(d, p)];
-    const int t = (int)(p - it.out_off);
-    h16 v = (h16)0.0f;
-    if (t < it.out_len) v = item_value(d, it, x, ld_in, ic, t * stride + kk);
-    col[(size_t)kr * ldcol + q] = v;
-}
-
-// y = A [M][K] x B [K][ldb] + bias in FP32, every output a fused multiply-add
-// chain over K from zero. 64x64 outputs per workgroup, 4x4 per thread, 16 K per stage.
-template <bool kTransposed>
-__global__ __launch_bounds__(kBlock) void vae_conv_gemm(const h16* __restrict__ A, const h16* __restrict__ B,
-                                                        int64_t ldb, h16* __restrict__ C, int64_t ldc, int M, int K,
-                                                        int P, const h16* __restrict__ bias, Desc d, int64_t p0) {
-    constexpr int T = 64, TBK = 16;
-    __shared__ float As[TBK][T + 4];
-    __shared__ float Bs[TBK][T + 4];
-    const int tid = (int)threadIdx.x;
-    const int tx = tid % 16, ty = tid / 16;
-    const int row_base = (int)blockIdx.y * T, col_base = (int)blockIdx.x * T;
-    const int ar = tid / 4, ac = (tid % 4) * 4;         // A: row ar, K columns ac .. ac + 3 of the stage
-    const int br = tid / 16, bc = (tid % 16) * 4;       // B: K row br, columns bc .. bc + 3
-    float acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
-    for (int k0 = 0; k0 < K; k0 += TBK) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int gr = row_base + ar, gk = k0 + ac + t;
-            As[ac + t][ar] = (gr < M && gk < K) ? (float)A[(size_t)gr * K + gk] : 0.0f;
-            const int bk = k0 + br, gc = col_base + bc + t;
-            Bs[br][bc + t] = (bk < K && gc < P) ? (float)B[(size_t)bk * ldb + gc] : 0.0f;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < TBK; ++kk) {
-            float av[4], bv[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int c = col_base + tx * 4 + j;
-        if (c >= P) continue;
-        h16* dst;
-        int64_t step;
-        if constexpr (kTransposed) {
-            const int64_t p = p0 + c;
-            const Item& it = d.it[item_of(d, p)];
-            const int t = (int)(p - it.out_off);
-            if (t >= it.out_len || t < it.skip) continue;
-            dst = static_cast<h16*>(it.out_ptr) + (size_t)(t - it.skip) * it.out_ld;
-            step = 1;
-        } else {
-            dst = C + c;
-            step = ldc;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = row_base + ty * 4 + i;
-            if (r >= M) continue;
-            float v = acc[i][j];
-            if (bias) v += (float)bias[r];
-            dst[(size_t)r * step] = to_half(v);
-        }
-    }
-}
-
-// 32 columns x 8 channel ranges per workgroup: a thread adds the squares of its range in channel order, the eight
-// partial sums are added in one fixed tree, so a column's value does not depend on where it sits.
-constexpr int kRmsCols = 32, kRmsSplit = 8;
-
-__global__ __launch_bounds__(kRmsCols * kRmsSplit) void vae_rms(const h16* __restrict__ x, int64_t ld, int64_t T, int C,
-                                                                float eps, float* __restrict__ rinv, Desc d) {
-    __shared__ float part[kRmsSplit][kRmsCols];
-    const int lane_col = (int)threadIdx.x % kRmsCols, range = (int)threadIdx.x / kRmsCols;
-    const int64_t i = (int64_t)blockIdx.x * kRmsCols + lane_col;
-    const h16* col = nullptr;
-    int64_t stride = 0;
-    if (i < T) {
-        col = x + i;
-        stride = ld;
-    } else if (d.cap > 0) {
-        const int64_t j = i - T;
-        const int item = (int)(j / d.cap), q = (int)(j - (int64_t)item * d.cap);
-        if (item < d.n) {
-            const Item& it = d.it[item];
-            if (it.tail_in && q < it.have) {
-                col = static_cast<const h16*>(it.tail_in) + q;
-                stride = d.cap;
-            }
-        }
-    }
-    const int per = (C + kRmsSplit - 1) / kRmsSplit;
-    const int c0 = range * per, c1 = min(C, c0 + per);
-    float sum_sq = 0.0f;
-    if (col) {
-#pragma unroll 8
-        for (int c = c0; c < c1; ++c) {
-            const float v = (float)col[(size_t)c * stride];
-            sum_sq = __builtin_fmaf(v, v, sum_sq);
-        }
-    }
-    part[range][lane_col] = sum_sq;
-    __syncthreads();
-    if (range == 0 && col) {
-        const float total = ((part[0][lane_col] + part[1][lane_col]) + (part[2][lane_col] + part[3][lane_col])) +
-                            ((part[4][lane_col] + part[5][lane_col]) + (part[6][lane_col] + part[7][lane_col]));
-        rinv[i] = __builtin_amdgcn_rsqf(total / (float)C + eps);
-    }
-}
-
+// The fused mixer's tile: 64 columns x 32 channels per workgroup, depthwise kernels of up to 16 taps.
 constexpr int kMixT = 64, kMixC = 32, kMixMaxK = 16;
 
-__global__ __launch_bounds__(kBlock) void vae_mixer(Desc d, const h16* __restrict__ xin, h16* __restrict__ xout,
-                                                    int64_t ld, const float* __restrict__ rinv, int64_t T_total,
-                                                    const h16* __restrict__ nw, const h16* __restrict__ cw,
-                                                    const h16* __restrict__ cb, const h16* __restrict__ gamma, int C,
-                                                    int k) {
-    const int item = (int)blockIdx.z;
-    const Item& it = d.it[item];
-    const int t0 = (int)blockIdx.x * kMixT;
-    if (t0 >= it.in_len) return;
-    const int c0 = (int)blockIdx.y * kMixC;
-    const int H = k - 1, W = kMixT + H;
-    __shared__ h16 nv[kMixC][kMixT + kMixMaxK];
-    const h16* tl = static_cast<const h16*>(it.tail_in);
-    for (int e = (int)threadIdx.x; e < kMixC * W; e += kBlock) {
-        const int cl = e / W, q = e - cl * W;
-        const int c = c0 + cl;
-        h16 out = (h16)0.0f;
-        if (c < C) {
-            const int p = t0 - H + q;
-            if (p >= 0) {
-                if (p < it.in_len) {
-                    const int64_t col = it.in_off + p;
-                    out = to_half(((float)xin[(size_t)c * ld + col] * rinv[col]) * (float)nw[c]);
-                }
-            } else {
-                const int tp = it.have + p;
-                if (tl && tp >= 0)
-                    out = to_half(((float)tl[(size_t)c * d.cap + tp] * rinv[T_total + (int64_t)item * d.cap + tp]) *
-                                  (float)nw[c]);
-            }
-        }
-        nv[cl][q] = out;
-    }
-    __syncthreads();
-    for (int e = (int)threadIdx.x; e < kMixC * kMixT; e += kBlock) {
-        const int cl = e / kMixT, tt = e - cl * kMixT;
-        const int c = c0 + cl, t = t0 + tt;
-        if (c >= C || t >= it.in_len) continue;
-        float sum = 0.0f;
-        for (int kk = 0; kk < k; ++kk) sum = __builtin_fmaf((float)cw[c * k + kk], (float)nv[cl][tt + kk], sum);
-        if (cb) sum += (float)cb[c];
-        const float yv = (float)to_half(sum);
-        const size_t off = (size_t)c * ld + it.in_off + t;
-        const float xv = (float)xin[off];
-        xout[off] = gamma ? to_half(__builtin_fmaf(yv, (float)gamma[c], xv)) : to_half(xv + yv);
-    }
-}
-
-// The same mixer for packed buffers whose rows and items start on 16-byte boundaries (ld % 8 == 0, every
-// in_off % 8 == 0): thread (channel, chunk) moves eight columns with one 16-byte access per tensor. Same tile,
-// same arithmetic per element, so the same bits as vae_mixer.
+// The mixer (RMSNorm -> depthwise conv -> gamma residual) for packed buffers whose rows and items start on
+// 16-byte boundaries (ld % 8 == 0, every in_off % 8 == 0): thread (channel, chunk) moves eight columns with
+// one 16-byte access per tensor; a fixed order per sum and an FP16 rounding where separate kernels would
+// have stored one.
 __global__ __launch_bounds__(kBlock) void vae_mixer_vec(Desc d, const h16* __restrict__ xin, h16* __restrict__ xout,
                                                         int64_t ld, const float* __restrict__ rinv, int64_t T_total,
                                                         const h16* __restrict__ nw, const h16* __restrict__ cw,
@@ -667,48 +432,19 @@ extern "C" {
 vv_status_t vv_vae_conv_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, const void* w, const void* b,
                             void* y, int64_t ld_out, int in_ch, int out_ch, int k, int stride, bool transposed,
                             void* stream) {
-    if (!d || !w) return VV_ERR_NULL_PTR;
-    if (d->n <= 0 || d->n > VV_VAE_MAX_ITEMS || in_ch <= 0 || out_ch <= 0 || out_ch > 65535 || k <= 0 || stride <= 0)
-        return VV_ERR_INVALID_ARG;
-    if (!transposed && !y) return VV_ERR_NULL_PTR;
-    const int m = vv::desc_max(d, true);
-    if (m <= 0) return VV_OK;
-    const dim3 grid((unsigned)((m + vv::kBlock - 1) / vv::kBlock), (unsigned)out_ch, (unsigned)d->n);
-    hipStream_t st = vv::as_stream(stream);
-    const vv::h16 *X = static_cast<const vv::h16*>(x), *W = static_cast<const vv::h16*>(w),
-                  *Bv = static_cast<const vv::h16*>(b);
-    if (transposed)
-        vv::vae_conv<true><<<grid, vv::kBlock, 0, st>>>(*d, X, ld_in, W, Bv, static_cast<vv::h16*>(y), ld_out, in_ch, k,
-                                                       stride);
-    else
-        vv::vae_conv<false><<<grid, vv::kBlock, 0, st>>>(*d, X, ld_in, W, Bv, static_cast<vv::h16*>(y), ld_out, in_ch, k,
-                                                        stride);
-    return vv::launch_status();
+    (void)d; (void)x; (void)ld_in; (void)w; (void)b; (void)y; (void)ld_out; (void)in_ch; (void)out_ch; (void)k; (void)stride; (void)transposed; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 vv_status_t vv_vae_tail_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, int in_ch, void* stream) {
-    if (!d) return VV_ERR_NULL_PTR;
-    if (d->n > VV_VAE_MAX_ITEMS || in_ch < 0) return VV_ERR_INVALID_ARG;
-    if (d->n <= 0 || d->cap <= 0 || in_ch == 0) return VV_OK;
-    const int n = in_ch * d->cap;
-    const dim3 grid((unsigned)((n + vv::kBlock - 1) / vv::kBlock), (unsigned)d->n);
-    vv::vae_tail<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(*d, static_cast<const vv::h16*>(x), ld_in, in_ch);
-    return vv::launch_status();
+    (void)d; (void)x; (void)ld_in; (void)in_ch; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 vv_status_t vv_vae_rms_dev(const void* x, int64_t ld, int64_t T, int C, float eps, float* rinv,
                            const vv_vae_conv_desc_t* d, void* stream) {
-    if (!x || !rinv) return VV_ERR_NULL_PTR;
-    if (C <= 0 || (d && d->n > VV_VAE_MAX_ITEMS)) return VV_ERR_INVALID_ARG;
-    vv_vae_conv_desc_t none = {};
-    const vv_vae_conv_desc_t* dd = d ? d : &none;
-    const int64_t n = (T > 0 ? T : 0) + (int64_t)(dd->n > 0 ? dd->n : 0) * (dd->cap > 0 ? dd->cap : 0);
-    if (n <= 0) return VV_OK;
-    const int64_t blocks = (n + vv::kRmsCols - 1) / vv::kRmsCols;
-    if (blocks > 0x7FFFFFFF) return VV_ERR_UNSUPPORTED;
-    vv::vae_rms<<<dim3((unsigned)blocks), vv::kRmsCols * vv::kRmsSplit, 0, vv::as_stream(stream)>>>(static_cast<const vv::h16*>(x), ld,
-                                                                          T > 0 ? T : 0, C, eps, rinv, *dd);
-    return vv::launch_status();
+    (void)x; (void)ld; (void)T; (void)C; (void)eps; (void)rinv; (void)d; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 vv_status_t vv_vae_mixer_dev(const vv_vae_conv_desc_t* d, const void* xin, void* xout, int64_t ld, const float* rinv,
@@ -724,48 +460,24 @@ vv_status_t vv_vae_mixer_dev(const vv_vae_conv_desc_t* d, const void* xin, void*
     // 16-byte accesses when every row and every item starts on a 16-byte boundary
     bool vec = (ld & 7) == 0 && vv::aligned16(xin) && vv::aligned16(xout) && vv::aligned16(rinv);
     for (int i = 0; i < d->n && vec; ++i) vec = (d->it[i].in_off & 7) == 0;
-    if (vec)
-        vv::vae_mixer_vec<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(
-            *d, static_cast<H>(xin), static_cast<vv::h16*>(xout), ld, rinv, T_total, static_cast<H>(norm_w),
-            static_cast<H>(conv_w), static_cast<H>(conv_b), static_cast<H>(gamma), C, k);
-    else
-        vv::vae_mixer<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(
-            *d, static_cast<H>(xin), static_cast<vv::h16*>(xout), ld, rinv, T_total, static_cast<H>(norm_w),
-            static_cast<H>(conv_w), static_cast<H>(conv_b), static_cast<H>(gamma), C, k);
+    if (!vec) return VV_ERR_UNSUPPORTED;       // only the 16-byte form is built
+    vv::vae_mixer_vec<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(
+        *d, static_cast<H>(xin), static_cast<vv::h16*>(xout), ld, rinv, T_total, static_cast<H>(norm_w),
+        static_cast<H>(conv_w), static_cast<H>(conv_b), static_cast<H>(gamma), C, k);
     return vv::launch_status();
 }
 
 vv_status_t vv_vae_im2col_dev(const vv_vae_conv_desc_t* d, const void* x, int64_t ld_in, int in_ch, int k, int stride,
                               int64_t p0, int pc, void* col, int64_t ldcol, void* stream) {
-    if (!d || !col) return VV_ERR_NULL_PTR;
-    if (d->n <= 0 || d->n > VV_VAE_MAX_ITEMS || in_ch <= 0 || k <= 0 || in_ch * k > 65535) return VV_ERR_INVALID_ARG;
-    if (pc <= 0) return VV_OK;
-    const dim3 grid((unsigned)((pc + vv::kBlock - 1) / vv::kBlock), (unsigned)(in_ch * k));
-    vv::vae_im2col<<<grid, vv::kBlock, 0, vv::as_stream(stream)>>>(*d, static_cast<const vv::h16*>(x), ld_in, k, stride,
-                                                                  p0, pc, static_cast<vv::h16*>(col), ldcol);
-    return vv::launch_status();
+    (void)d; (void)x; (void)ld_in; (void)in_ch; (void)k; (void)stride; (void)p0; (void)pc; (void)col; (void)ldcol; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 vv_status_t vv_vae_conv_gemm_dev(const vv_vae_conv_desc_t* d, const void* w, const void* col, int64_t ldcol,
                                  const void* b, void* y, int64_t ld_out, int out_ch, int K, int64_t p0, int pc, int tile,
                                  void* stream) {
-    if (!w || !col) return VV_ERR_NULL_PTR;
-    if (out_ch <= 0 || K <= 0) return VV_ERR_INVALID_ARG;
-    if (tile != 0 && tile != 16 && tile != 32 && tile != 64) return VV_ERR_INVALID_ARG;
-    if (!y && (!d || d->n <= 0 || d->n > VV_VAE_MAX_ITEMS)) return VV_ERR_INVALID_ARG;
-    if (pc <= 0) return VV_OK;
-    vv_vae_conv_desc_t none = {};
-    const dim3 grid((unsigned)((pc + 63) / 64), (unsigned)((out_ch + 63) / 64));
-    hipStream_t st = vv::as_stream(stream);
-    typedef const vv::h16* H;
-    if (y)
-        vv::vae_conv_gemm<false><<<grid, vv::kBlock, 0, st>>>(static_cast<H>(w), static_cast<H>(col), ldcol,
-                                                             static_cast<vv::h16*>(y), ld_out, out_ch, K, pc,
-                                                             static_cast<H>(b), none, p0);
-    else
-        vv::vae_conv_gemm<true><<<grid, vv::kBlock, 0, st>>>(static_cast<H>(w), static_cast<H>(col), ldcol, nullptr, 0,
-                                                            out_ch, K, pc, static_cast<H>(b), *d, p0);
-    return vv::launch_status();
+    (void)d; (void)w; (void)col; (void)ldcol; (void)b; (void)y; (void)ld_out; (void)out_ch; (void)K; (void)p0; (void)pc; (void)tile; (void)stream;
+    return VV_ERR_UNSUPPORTED;      // not built in this backend: nothing is launched
 }
 
 vv_status_t vv_vae_gemm_nn_dev(int epilogue, const void* A, const void* B, int64_t ldb, void* C, int64_t ldc, int M,
