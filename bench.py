@@ -166,6 +166,79 @@ def time_kernel(torch, wl: Workload, name: str, launches: int, reps: int, st: in
     return per[0], per[len(per) // 2]
 
 
+# The shapes BASELINE.json's configs name, and the 2048-row chunk the reference's chunked prefill
+# actually launches (src/inference/decoder.c:1147-1174).
+CONFIG_SHAPES = [("add+norm", 512), ("add+norm", 2048), ("add+norm", 4096), ("rope", 2048),
+                 ("swiglu", 2048), ("swiglu", 4096), ("gather+norm", 2048)]
+LLC_BYTES = 256 << 20            # the last-level cache in front of HBM (plus 4 MB of L2 per XCD)
+CONFIG_FOOTPRINT = 4 * LLC_BYTES   # rotate over at least this many bytes of distinct tensors
+
+
+def configs_leg(torch, dev, wl: "Workload", st: int, launches: int = 120, reps: int = 5) -> list:
+    """Every (kernel, T) of CONFIG_SHAPES, cold: the launches rotate over enough distinct buffer
+    sets that their joint footprint is four times the last-level cache, so no launch finds its
+    inputs cached by an earlier one. These launches last 3-70 us, less than Python needs to issue
+    one, so the stream is first kept busy by a few full-size SwiGLU launches while the timed
+    launches are queued behind them; the start event sits between the two groups. The time per
+    launch therefore includes the gap between dependent kernels of one stream, as in the product."""
+    out = []
+    for name, T in CONFIG_SHAPES:
+        nbytes = algorithmic_bytes(T)[name]
+        nsets = max(3, -(-CONFIG_FOOTPRINT // nbytes))
+        gen = torch.Generator(device="cuda").manual_seed(T)
+
+        def randn(*shape, std=1.0):
+            return (torch.randn(*shape, generator=gen, device="cuda") * std).half()
+
+        sets = []
+        for _ in range(nsets):
+            if name == "add+norm":
+                d = {"residual": randn(T, H), "x": randn(T, H),
+                     "normed": torch.empty(T, H, dtype=torch.float16, device="cuda")}
+            elif name == "rope":
+                d = {"q": randn(T, NQ, HD), "k": randn(T, NK, HD)}
+            elif name == "swiglu":
+                d = {"gate": randn(T, I_FF, std=2.0), "up": randn(T, I_FF, std=2.0),
+                     "out": torch.empty(T, I_FF, dtype=torch.float16, device="cuda")}
+            else:
+                d = {"ids": torch.randint(0, V, (T,), generator=gen, device="cuda", dtype=torch.int32),
+                     "hidden": torch.empty(T, H, dtype=torch.float16, device="cuda"),
+                     "normed": torch.empty(T, H, dtype=torch.float16, device="cuda")}
+            sets.append(d)
+        small = Workload.__new__(Workload)
+        small.torch, small.dev, small.T, small.nsets = torch, dev, T, nsets
+        small.table, small.weight, small.sets = wl.table, wl.weight, sets
+        n = max(launches, 2 * nsets)
+        for i in range(nsets):
+            small.launch(name, i, st)
+        torch.cuda.synchronize()
+        per, queued_ahead = [], True
+        for _ in range(reps):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            for i in range(8):                      # ~2 ms of work ahead of the timed launches
+                wl.launch("swiglu", i, st)
+            e0.record()
+            for i in range(n):
+                small.launch(name, i, st)
+            e1.record()
+            queued_ahead = queued_ahead and not e0.query()     # still busy ahead of us: the queue never ran dry
+            e1.synchronize()
+            per.append(e0.elapsed_time(e1) * 1e-3 / n)
+        per.sort()
+        med = per[len(per) // 2]
+        out.append({"kernel": name, "rows": T, "bytes": nbytes, "us": med * 1e6, "us_best": per[0] * 1e6,
+                    "GBps": nbytes / med / 1e9, "frac": nbytes / med / 1e9 / HBM_PEAK_GBPS,
+                    "rows_per_s": T / med, "buffer_sets": nsets, "footprint_MB": nsets * nbytes / 1e6,
+                    "cold": True, "launches_queued_ahead_of_the_gpu": bool(queued_ahead)})
+        log(f"  config {name:12s} T={T:5d} {med * 1e6:8.2f} us  {nbytes / med / 1e9:8.1f} GB/s  "
+            f"{100 * nbytes / med / 1e9 / HBM_PEAK_GBPS:5.1f} % of peak  ({nsets} sets, cold"
+            f"{'' if queued_ahead else ', issue-bound'})")
+        del sets, small
+        torch.cuda.empty_cache()
+    return out
+
+
 def decode_graph_leg(torch, dev, wl1) -> dict:
     """One token's worth of this library's launches (per layer: norm -> RoPE(Q,K) with the
     position read from device memory -> add+norm -> SwiGLU -> add+norm), issued directly and
@@ -902,7 +975,7 @@ def cpu_baseline(rows: int) -> dict:
         simd = oracle.ref.vv_cpu_simd_name().decode()
     else:
         threads, simd = oracle.lib.vvo_threads(), "scalar"
-    vocab = 8192                                   # a table slice: the gather cost is per row
+    vocab = V                                      # the whole [152064, 3584] table: 1.09 GB of host memory
     table = oracle.normal_f16((vocab, H), 1, std=0.02)
     ids = oracle.ids(rows, 2, vocab)
     w = oracle.normal_f16((H,), 3, mean=1.0, std=0.1)
@@ -968,8 +1041,8 @@ def cpu_baseline(rows: int) -> dict:
         "cores": threads,
         "kind": "reference" if use_ref else "port",
         "simd": simd,
-        "sample": f"the same step on {rows} of {T_FULL} rows (embedding table cut to {vocab} "
-                  "rows), best of 5 after a warm-up call",
+        "sample": f"the same step on {rows} of {T_FULL} rows (the whole {vocab}-row embedding table), "
+                  "best of 5 after a warm-up call",
         "rows_per_s": rows / total,
         "ms_per_step_sample": total * 1e3,
         "kernels": per,
@@ -985,6 +1058,7 @@ def main() -> int:
     ap.add_argument("--sets", type=int, default=3, help="rotating buffer sets")
     ap.add_argument("--launches", type=int, default=20, help="back-to-back launches per event pair")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-config (smaller T) leg")
     ap.add_argument("--only", default=None, help="time only this kernel (profiling aid)")
     ap.add_argument("--reps", type=int, default=5, help="event-timed repetitions per kernel")
     ap.add_argument("--unfused", action="store_true",
@@ -1130,6 +1204,11 @@ def main() -> int:
                 f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at "
                 f"{d['weight_GBps']:.0f} GB/s ({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
 
+    # ── BASELINE.json's config shapes and the 2048-row prefill chunk, cold ──
+    configs = []
+    if not args.only and not args.no_configs:
+        configs = configs_leg(torch, dev, wl, st)
+
     # ── decode shape (T = 1): launch-bound, reported as microseconds per launch ──
     decode = {}
     if not args.only:
@@ -1167,8 +1246,12 @@ def main() -> int:
         "kernels": per,
         "roofline": {"kernel": dominant, "bound": "hbm", "achieved": per[dominant]["GBps"],
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": per[dominant]["frac_of_peak"], "traffic": traffic},
+                     "frac": per[dominant]["frac_of_peak"], "traffic": traffic,
+                     "traffic_source": "profiles/pmc_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                       "of this kernel at this shape, recorded earlier, not measured in this run"},
     }
+    if configs:
+        result["configs"] = configs
     if unfused:
         result["unfused"] = unfused
     if layer:

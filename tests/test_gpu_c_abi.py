@@ -6,8 +6,30 @@ import subprocess
 
 import pytest
 
+import functools
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 EXE = os.path.join(HERE, "c", "abi_layer_ops")
+# Written by __graft_entry__.build() when it compiled the reference's test programs (oracle/Makefile,
+# which needs the reference tree). It travels with the built programs, so where it is present a missing
+# program is a broken build or a lost file and fails loudly; a checkout built without the reference
+# tree has neither and skips.
+REF_MARKER = os.path.join(os.path.dirname(HERE), "oracle", "ref_built.marker")
+
+
+def needs_ref_program(path):
+    def wrap(fn):
+        @functools.wraps(fn)
+        def run(*a, **kw):
+            if not os.path.exists(path):
+                rel = os.path.relpath(path, os.path.dirname(HERE))
+                if os.path.exists(REF_MARKER):
+                    pytest.fail(f"{rel} is missing although the reference's test programs were built "
+                                f"({os.path.relpath(REF_MARKER, os.path.dirname(HERE))} is present)")
+                pytest.skip(f"{rel} not built (needs the reference tree)")
+            return fn(*a, **kw)
+        return run
+    return wrap
 
 
 @pytest.mark.gpu
@@ -28,8 +50,7 @@ REF_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_device_mem
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(REF_EXE),
-                    reason="oracle/_ref/test_device_memory_hip not built (needs the reference tree)")
+@needs_ref_program(REF_EXE)
 def test_reference_own_device_memory_test_passes_on_this_backend():
     """The reference's tests/test_device_memory.c, compiled unmodified by
     oracle/Makefile and linked against libvibevoice_hip.so: copies, fills,
@@ -44,8 +65,7 @@ LAYER_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_prefill_
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(LAYER_EXE),
-                    reason="oracle/_ref/test_prefill_append_hip not built (needs the reference tree)")
+@needs_ref_program(LAYER_EXE)
 def test_reference_layer_runner_passes_on_this_backend():
     """The reference's tests/test_prefill_append.c with the reference's own
     decoder and KV cache (compiled unmodified by oracle/Makefile) driving this
@@ -67,8 +87,7 @@ ATTN_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_attention
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(ATTN_EXE),
-                    reason="oracle/_ref/test_attention_hip not built (needs the reference tree)")
+@needs_ref_program(ATTN_EXE)
 def test_reference_own_attention_test_passes_on_this_backend():
     """The reference's tests/test_attention.c, unmodified: prefill attention at
     28 query / 4 KV heads of 128 against its FP64 reference, at lengths on and
@@ -85,8 +104,7 @@ POOL_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_kv_pool_h
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(POOL_EXE),
-                    reason="oracle/_ref/test_kv_pool_hip not built (needs the reference tree)")
+@needs_ref_program(POOL_EXE)
 def test_reference_own_kv_pool_test_passes_on_this_backend():
     """The reference's tests/test_kv_pool.c with the reference's KV cache code:
     the paged pool's bookkeeping against the device page table this backend
@@ -101,8 +119,7 @@ INT8_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_int8_line
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(INT8_EXE),
-                    reason="oracle/_ref/test_int8_linear_hip not built (needs the reference tree)")
+@needs_ref_program(INT8_EXE)
 def test_reference_own_int8_linear_test_passes_on_this_backend():
     """The reference's tests/test_int8_linear.c: its CPU quantiser and linear
     kernels, then this backend's activation quantisers (plain and fused, four
@@ -123,8 +140,7 @@ W4A16_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_w4a16_hi
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(W4A16_EXE),
-                    reason="oracle/_ref/test_w4a16_hip not built (needs the reference tree)")
+@needs_ref_program(W4A16_EXE)
 def test_reference_own_w4a16_test_passes_on_this_backend():
     """The reference's tests/test_w4a16.c: AWQ, GPTQ (symmetric, act-order) and
     load-time INT4 weights made and repacked by the reference's host code, then
@@ -142,8 +158,7 @@ POS_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_decode_pos
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(KVQ_EXE),
-                    reason="oracle/_ref/test_kv_quant_hip not built (needs the reference tree)")
+@needs_ref_program(KVQ_EXE)
 def test_reference_own_kv_quant_test_passes_on_this_backend():
     """The reference's tests/test_kv_quant.c: a cache shaped like Qwen2's keys
     stored in both FP8 and all four TurboQuant formats, unpacked, attended to
@@ -157,8 +172,7 @@ def test_reference_own_kv_quant_test_passes_on_this_backend():
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(POS_EXE),
-                    reason="oracle/_ref/test_decode_position_hip not built (needs the reference tree)")
+@needs_ref_program(POS_EXE)
 def test_reference_own_decode_position_test_passes_on_this_backend():
     """The reference's tests/test_decode_position.c: everything a captured decode
     step reads from a device int (position add, the row copy, FP16 and
@@ -176,8 +190,7 @@ CONCURRENT_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_con
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(ATTN_BACKENDS_EXE),
-                    reason="oracle/_ref/test_attn_backends_hip not built (needs the reference tree)")
+@needs_ref_program(ATTN_BACKENDS_EXE)
 def test_reference_own_attention_interface_test_passes_on_this_backend():
     """The reference's tests/test_attn_backends.c: every backend name over slab
     and paged caches in FP16, FP8 and TurboQuant, prefill and decode at two head
@@ -193,8 +206,7 @@ def test_reference_own_attention_interface_test_passes_on_this_backend():
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(CONCURRENT_EXE),
-                    reason="oracle/_ref/test_concurrent_decode_hip not built (needs the reference tree)")
+@needs_ref_program(CONCURRENT_EXE)
 def test_reference_own_concurrent_decode_test_passes_on_this_backend():
     """The reference's tests/test_concurrent_decode.c: four threads, each with
     its own stream and scratch, decode over slab caches and over pages of one
@@ -209,8 +221,7 @@ SKINNY_EXE = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "test_skinny_
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.exists(SKINNY_EXE),
-                    reason="oracle/_ref/test_skinny_hip not built (needs the reference tree)")
+@needs_ref_program(SKINNY_EXE)
 def test_reference_own_small_m_test_passes_on_this_backend():
     """The reference's tests/test_skinny.c: dense FP16, per-channel INT8 and NF4
     linear layers at every row count where a tiling changes between 9 and 64,

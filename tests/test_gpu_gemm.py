@@ -107,6 +107,13 @@ def test_gemm_edges():
     want = (2.0 * oracle.widen(bits_of(c))).astype(np.float16).view(np.uint16)
     ok(dev.vv_gemm_fp16_dev(p, p, c.data_ptr(), 2, 8, 0, 1.0, 2.0, stream()))
     assert np.array_equal(bits_of(c), want)
+    # the same at shapes that would otherwise run the 128- and 256-wide tile kernels: no operand is read
+    for fn, M, N in ((dev.vv_gemm_fp16_dev, 300, 512), (dev.vv_gemm_fp16_dev, 1024, 2048),
+                     (dev.vv_gemm_fp16_tile_dev, 300, 512)):
+        c = to_dev(oracle.normal_f16((M, N), 10))
+        want = (2.0 * oracle.widen(bits_of(c))).astype(np.float16).view(np.uint16)
+        ok(fn(p, p, c.data_ptr(), M, N, 0, 1.0, 2.0, stream()))
+        assert np.array_equal(bits_of(c), want)
 
 
 def skinny(d_a, ws, biases, M, K, alpha=1.0):

@@ -465,7 +465,9 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
     const h16* b = static_cast<const h16*>(B);
     h16* c = static_cast<h16*>(C);
 
-    if (K % 8 != 0 || !aligned16(A) || !aligned16(B)) {
+    // K == 0 goes here too (C = beta * C): the tile kernels' first slab fetch is
+    // unconditional and would read past an empty operand.
+    if (K == 0 || K % 8 != 0 || !aligned16(A) || !aligned16(B)) {
         const size_t blocks = ((size_t)M * N + kBlock - 1) / kBlock;
         gemm_naive<<<dim3((unsigned)blocks), kBlock, 0, st>>>(a, b, c, M, N, K, alpha, beta);
         return launch_status();

@@ -246,7 +246,11 @@ vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias
     if (fast) {
         // items per thread: enough for one position, then as many positions per
         // workgroup as fit (at most kPosPerBlock); VV_ROPE_ITEMS=1|2|4 forces (A/B aid)
-        static const int forced_items = getenv("VV_ROPE_ITEMS") ? atoi(getenv("VV_ROPE_ITEMS")) : 0;
+        static const int forced_items = [] {
+            const char* e = getenv("VV_ROPE_ITEMS");
+            const int v = e ? atoi(e) : 0;
+            return (v == 1 || v == 2 || v == 4) ? v : 0;       // anything else: not forced
+        }();
         const int tasks = (nq + nk) * 8;
         int items = forced_items ? forced_items : 1;
         while (items * kBlock < tasks) items *= 2;          // <= kMaxItems by the head limit
