@@ -126,6 +126,79 @@ __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
     }
 }
 
+// ── one wave per row, kCpl chunks per lane ──────────────────────────────
+// For launches of a few thousand rows. With a workgroup per row the chip holds
+// about 1024 rows at a time (four 7-wave workgroups per compute unit), so a
+// 2048-row prefill chunk runs as two dependent rounds of load -> reduce -> store
+// and never has more than half of its reads in flight. Here a row is one wave
+// with all of its loads (kCpl per tensor) issued back to back: 2048 rows are
+// 2048 waves, two per SIMD, every byte of the launch requested in the first
+// microsecond, no LDS and no barrier. The sum of squares keeps the workgroup
+// kernel's order bit for bit: group j of 64 chunks is reduced like wave j of
+// that kernel (same DPP tree), and the groups are added in order from zero.
+template <int kCpl, int kMode, bool kStream>
+__global__ __launch_bounds__(kBlock) void norm_rows_wave(
+    const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
+    const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float inv_n,
+    float eps) {
+    const int row = (int)blockIdx.x * ((int)blockDim.x >> 6) + wave_in_block();
+    if (row >= rows) return;                      // whole waves leave; nothing below synchronises
+    const int lane = lane_id();
+    constexpr bool kGathers = kMode == kGather || kMode == kGatherOnly;
+    constexpr bool kStreamSrc = kStream && !kGathers;
+    const size_t src_row = kGathers ? (size_t)ids[row] : (size_t)row;
+    const Chunk* s = src + src_row * (size_t)nchunks;
+    const size_t out_base = (size_t)row * (size_t)nchunks;
+
+    Chunk a[kCpl], b[kCpl], w[kCpl];
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        if (c < nchunks) {
+            a[j] = load_chunk_as<kStreamSrc>(s + c);
+            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
+        }
+    }
+    if (kMode == kGatherOnly) {
+#pragma unroll
+        for (int j = 0; j < kCpl; ++j) {
+            const int c = j * kWave + lane;
+            if (c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        if (c < nchunks) w[j] = load_chunk(weight + c);
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        float acc = 0.0f;
+        if (c < nchunks) {
+            f32x8 x = unpack(a[j]);
+            if (kMode == kAdd) {
+                const f32x8 res = unpack(b[j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = res[i] + x[i];
+                a[j] = pack(x);                   // the stored residual; the norm reads that value
+                x = unpack(a[j]);
+            }
+            if (kMode == kAdd || kMode == kGather) store_chunk_as<kStream>(state + out_base + c, a[j]);
+            acc = chunk_sumsq(x, 0.0f);
+        }
+        total += wave_sum(acc);
+    }
+    const float inv = inv_rms(total, inv_n, eps);
+#pragma unroll
+    for (int j = 0; j < kCpl; ++j) {
+        const int c = j * kWave + lane;
+        if (c < nchunks) store_chunk_as<kStream>(normed + out_base + c, scale_chunk(a[j], inv, w[j]));
+    }
+}
+
 // ── one workgroup per row, any width, any alignment ──────────────────────
 // Two passes; the second re-reads what the first one left in `state` (kAdd,
 // kGather) or the source row (kPlain), which the caches still hold. Thread t
@@ -204,18 +277,58 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         const Chunk* w = static_cast<const Chunk*>(weight);
         Chunk* o = static_cast<Chunk*>(normed);
         const bool full = nchunks == cpt * threads;
-        // Two rows per workgroup for the narrow (one chunk per thread) case once there
-        // are enough rows to fill the chip several times over; VV_HIP_ROWS_PER_WG=1|2 forces.
+        // Which kernel: measured cold on MI355X at hidden 3584 with streaming accesses, a
+        // launch of R rows (times in us, workgroup per row / two rows per workgroup / wave
+        // per row):        R = 1024          2048            3072           6144          14449
+        //   add+norm    6.8  6.9  6.2   11.7 12.0 10.1  16.5 17.0 15.5  29.8 30.6 31.1  66.8 67.1 68.9
+        //   gather+norm 7.2  5.8  5.8   11.5  9.8  8.4  15.6 14.4 12.2  27.1 25.2 23.2  58.4 54.6 53.7
+        //   norm        4.1  4.4  5.3    7.6  6.3  6.5  10.1 10.2  8.7  17.3 16.7 15.7  38.0 34.2 37.0
+        // A workgroup per row keeps ~1024 rows on the chip at once, so a few thousand rows
+        // run as two or three dependent rounds; a wave per row has them all resident with
+        // every load issued at the start. Long launches hide that and prefer light waves.
+        // Row counts are scaled to hidden 3584 (448 chunks) for other widths.
+        // VV_HIP_ROWS_PER_WG=1|2 forces a workgroup kernel, VV_HIP_NORM_WAVE=0|1 the wave kernel.
         static const int forced_rows = [] {
             const char* e = getenv("VV_HIP_ROWS_PER_WG");
             return (e && (e[0] == '1' || e[0] == '2')) ? e[0] - '0' : 0;
         }();
-        // Measured at T = 14449, hidden 3584: two rows per workgroup is faster for the
-        // one-input modes (norm 37.3 -> 34.6 us, gather+norm 58.8 -> 55.2 us) and
-        // slightly slower for add+norm (66.6 -> 67.5 us), which already has two loads
-        // per thread in flight.
-        const int rpw = forced_rows ? forced_rows
-                                    : ((cpt == 1 && rows >= 4096 && kMode != kAdd) ? 2 : 1);
+        static const int forced_wave = [] {
+            const char* e = getenv("VV_HIP_NORM_WAVE");
+            return (e && (e[0] == '0' || e[0] == '1')) ? e[0] - '0' : -1;
+        }();
+        const long eq_rows = (long)rows * nchunks / 448;       // rows of 448 chunks with the same bytes
+        bool wave = false;
+        int rpw = 1;
+        if (cpt == 1) {
+            if (kMode == kAdd) wave = eq_rows >= 896 && eq_rows <= 4608;
+            else if (kMode == kPlain) {
+                wave = eq_rows >= 2560 && eq_rows < 7168;
+                rpw = eq_rows >= 1536 ? 2 : 1;
+            } else if (kMode == kGather) {
+                wave = eq_rows >= 768;
+                rpw = eq_rows >= 256 ? 2 : 1;
+            } else {
+                rpw = eq_rows >= 4096 ? 2 : 1;      // gather only: 32.4 us at 14449 rows (80 % of peak)
+            }
+        }
+        if (forced_rows) { rpw = forced_rows; wave = false; }
+        if (forced_wave >= 0 && !forced_rows) wave = forced_wave == 1;
+        if (wave && cpt == 1 && nchunks <= 8 * kWave) {
+            const dim3 wgrid((unsigned)((rows + kWavesPerBlock - 1) / kWavesPerBlock));
+#define VV_WAVE_CASE(C)                                                                           \
+    case C:                                                                                      \
+        if (stream) norm_rows_wave<C, kMode, true><<<wgrid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, \
+                                                                             nchunks, inv_n, eps);    \
+        else norm_rows_wave<C, kMode, false><<<wgrid, kBlock, 0, st>>>(s, stt, ids, w, o, rows,       \
+                                                                       nchunks, inv_n, eps);          \
+        break;
+            switch ((nchunks + kWave - 1) / kWave) {
+                VV_WAVE_CASE(1) VV_WAVE_CASE(2) VV_WAVE_CASE(3) VV_WAVE_CASE(4)
+                VV_WAVE_CASE(5) VV_WAVE_CASE(6) VV_WAVE_CASE(7) VV_WAVE_CASE(8)
+            }
+#undef VV_WAVE_CASE
+            return launch_status();
+        }
         const bool two = rpw == 2 && cpt == 1;
         const dim3 grid((unsigned)(two ? (rows + 1) / 2 : rows));
 #define VV_WG_LAUNCH(C, R, S, F)                                                          \

@@ -161,6 +161,79 @@ __global__ __launch_bounds__(kBlock) void rope128(RopeArgs a, FreqTable freqs, i
     }
 }
 
+// head_dim == 128, at most 32 heads in all: ONE WAVE PER POSITION, for launches
+// of a few thousand positions. With a workgroup per position a 2048-row prefill
+// chunk is a bit more than one round of workgroups on the chip, each a
+// load -> barrier -> store chain; here it is 2048 independent waves, all
+// resident at once, with no LDS and no barrier. Lane l is (chunk pair c = l % 8,
+// head group l / 8) and takes heads l / 8, l / 8 + 8, ... (four items for 32
+// heads): its eight loads go out first; then the lane computes the cosine and
+// sine of ONE pair index (l, of 64) and collects the eight it needs, pairs
+// 8c .. 8c + 7, from lanes 8c .. 8c + 7 by cross-lane reads. Same angle, same
+// sincosf, same unfused rotation as rope128: the same bits.
+constexpr int kWaveItems = 4;
+
+template <bool kBias, bool kStream>
+__global__ __launch_bounds__(kBlock) void rope128_wave(RopeArgs a, FreqTable freqs) {
+    const int row = (int)blockIdx.x * ((int)blockDim.x >> 6) + wave_in_block();
+    if (row >= a.rows) return;                    // whole waves leave; nothing below synchronises
+    const int lane = lane_id(), c = lane & 7, hg = lane >> 3;
+    const int heads = a.nq + a.nk;
+    const int first = a.d_position ? *a.d_position : a.position_offset;
+    float my_freq = freqs.f[lane];
+
+    Chunk* lo_p[kWaveItems];
+    Chunk lo[kWaveItems], hi[kWaveItems];
+    bool live[kWaveItems];
+#pragma unroll
+    for (int k = 0; k < kWaveItems; ++k) {
+        const int want = hg + 8 * k;
+        live[k] = want < heads;
+        const int head = live[k] ? want : heads - 1;
+        h16* base = head < a.nq
+            ? a.q + ((size_t)row * (size_t)a.nq + (size_t)head) * 128u
+            : a.k + ((size_t)row * (size_t)a.nk + (size_t)(head - a.nq)) * 128u;
+        lo_p[k] = reinterpret_cast<Chunk*>(base) + c;
+        lo[k] = load_chunk_as<kStream>(lo_p[k]);
+        hi[k] = load_chunk_as<kStream>(lo_p[k] + 8);
+        if (kBias) {
+            const h16* bias = head < a.nq
+                ? (a.q_bias ? a.q_bias + (size_t)head * 128u : nullptr)
+                : (a.k_bias ? a.k_bias + (size_t)(head - a.nq) * 128u : nullptr);
+            if (bias) {
+                const Chunk* bp = reinterpret_cast<const Chunk*>(bias) + c;
+                lo[k] = add_bias(lo[k], load_chunk(bp));
+                hi[k] = add_bias(hi[k], load_chunk(bp + 8));
+            }
+        }
+    }
+    asm volatile("" : "+v"(my_freq));             // the frequency is waited for here, not the tensor data
+
+    float my_s, my_c;
+    sincosf((float)(first + row) * my_freq, &my_s, &my_c);
+    f32x8 cv, sv;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        cv[i] = __shfl(my_c, 8 * c + i);
+        sv[i] = __shfl(my_s, 8 * c + i);
+    }
+#pragma unroll
+    for (int k = 0; k < kWaveItems; ++k) {
+        if (live[k]) {
+            const f32x8 x0 = unpack(lo[k]), x1 = unpack(hi[k]);
+            f32x8 y0, y1;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const Pair r = rotate(x0[i], x1[i], cv[i], sv[i]);
+                y0[i] = r.lo;
+                y1[i] = r.hi;
+            }
+            store_chunk_as<kStream>(lo_p[k], pack(y0));
+            store_chunk_as<kStream>(lo_p[k] + 8, pack(y1));
+        }
+    }
+}
+
 // Any even head_dim <= 256, any alignment: one workgroup per position,
 // 2-byte accesses.
 __global__ __launch_bounds__(kBlock) void rope_generic(RopeArgs a, FreqTable freqs) {
@@ -261,6 +334,25 @@ vv_status_t launch_rope(void* q, void* k, const void* q_bias, const void* k_bias
         const dim3 grid((unsigned)((rows + posb - 1) / posb));
         const bool stream = use_streaming(2u * (size_t)rows * (size_t)(nq + nk) * 128u * 2u);
         const bool exact = (nq + nk) * 8 == kBlock;
+        // A wave per position for launches that would otherwise be one to three rounds of
+        // workgroups: measured cold at 28 + 4 heads, workgroup / wave per position:
+        // 1024 rows 4.7 / 4.3 us, 2048 rows 7.7 / 7.1 us, 4096 rows 12.8 / 12.8 us,
+        // 14449 rows 38.5 / 40.3 us. VV_ROPE_WAVE=0|1 forces.
+        static const int forced_wave = [] {
+            const char* e = getenv("VV_ROPE_WAVE");
+            return (e && (e[0] == '0' || e[0] == '1')) ? e[0] - '0' : -1;
+        }();
+        const long eq_rows = (long)rows * (nq + nk) / 32;
+        bool wave = eq_rows >= 768 && eq_rows <= 3584;
+        if (forced_wave >= 0) wave = forced_wave == 1;
+        if (wave && nq + nk <= 8 * kWaveItems && !forced_items) {
+            const dim3 wgrid((unsigned)((rows + kWavesPerBlock - 1) / kWavesPerBlock));
+            if (has_bias && stream)  rope128_wave<true, true><<<wgrid, kBlock, 0, st>>>(a, freqs);
+            else if (has_bias)       rope128_wave<true, false><<<wgrid, kBlock, 0, st>>>(a, freqs);
+            else if (stream)         rope128_wave<false, true><<<wgrid, kBlock, 0, st>>>(a, freqs);
+            else                     rope128_wave<false, false><<<wgrid, kBlock, 0, st>>>(a, freqs);
+            return launch_status();
+        }
 #define VV_ROPE_LAUNCH(B, S, E, I) rope128<B, S, E, I><<<grid, kBlock, 0, st>>>(a, freqs, posb)
 #define VV_ROPE_ITEMS(B, S, E)                          \
     do {                                                \

@@ -32,12 +32,13 @@ __device__ __forceinline__ void store_chunk(Chunk* p, const Chunk& c) { *p = c; 
 
 // Streaming forms (the "nt" bit on global_load/global_store): the line is
 // touched once and should be the first to leave the caches. On MI355X a plain
-// copy moves 5.7 TB/s with ordinary accesses and 6.3 TB/s with these; the
-// hosts pick them when a launch's footprint exceeds what the last-level cache
-// could keep for the next kernel anyway (kStreamBytes), and ordinary accesses
-// below that, so a decode step or a prefill chunk leaves its output cached for
-// the GEMM that consumes it.
-constexpr size_t kStreamBytes = (size_t)96 << 20;
+// copy moves 5.7 TB/s with ordinary accesses and 6.3 TB/s with these, and the
+// gap is wider for short launches against a last-level cache that earlier
+// kernels left full of written lines (a 2048-row add+norm: 13.5 us with ordinary
+// accesses, 11.7 us with these; its stores alone are worth 20 %). The hosts pick
+// them from kStreamBytes per launch on; below that (a decode step, a handful of
+// rows) ordinary accesses leave the output in L2 for the kernel that consumes it.
+constexpr size_t kStreamBytes = (size_t)2 << 20;
 
 __device__ __forceinline__ Chunk load_chunk_stream(const Chunk* p) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
