@@ -151,6 +151,54 @@ def test_add_rmsnorm_other_widths(rows, hidden):
     assert_fp16_close(bits_of(d_n), nref, nrne, f"add+rmsnorm [{rows},{hidden}]")
 
 
+@pytest.mark.parametrize("rows,hidden", [(900, 3584), (1000, 3584), (2049, 3584), (5000, 3584), (3000, 1536),
+                                         (4001, 1000), (1300, 4096), (9000, 512)])
+def test_mid_size_launches_every_row_kernel_agrees(rows, hidden):
+    """Launches of a thousand to a few thousand rows run one wave per row (full and partial
+    last groups of 64 chunks), shorter and longer ones a workgroup per row or per two rows, and
+    the switch-over differs by op: the fused ops must still equal their two-call sequences bit
+    for bit, whichever kernels the two sides run, and both must match the oracle."""
+    res = oracle.normal_f16((rows, hidden), 21 + rows)
+    x = oracle.normal_f16((rows, hidden), 22 + rows)
+    w = weight(hidden)
+    want_res, nref, nrne = oracle.add_rmsnorm_f16(res, x, w, EPS)
+    d_res, d_x, d_w = to_dev(res), to_dev(x), to_dev(w)
+    d_n = torch.full((rows, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_add_rmsnorm_dev(d_res.data_ptr(), d_x.data_ptr(), d_w.data_ptr(), d_n.data_ptr(),
+                              rows, hidden, EPS, stream()))
+    assert np.array_equal(bits_of(d_res), want_res), "updated residual must be bit-exact"
+    assert_fp16_close(bits_of(d_n), nref, nrne, f"add+rmsnorm [{rows},{hidden}]")
+    e_res, e_x = to_dev(res), to_dev(x)
+    ok(dev.vv_residual_add_dev(e_res.data_ptr(), e_x.data_ptr(), rows * hidden, stream()))
+    ok(dev.vv_rmsnorm_dev(e_res.data_ptr(), d_w.data_ptr(), e_x.data_ptr(), rows, hidden, EPS, stream()))
+    assert np.array_equal(bits_of(e_res), bits_of(d_res))
+    assert np.array_equal(bits_of(e_x), bits_of(d_n))
+    # a row normalised alone (one-row launch: workgroup kernel) gives the bits it got in the batch
+    for r in (0, rows // 2, rows - 1):
+        one = torch.empty(hidden, dtype=torch.float16, device="cuda")
+        ok(dev.vv_rmsnorm_dev(d_res.data_ptr() + r * hidden * 2, d_w.data_ptr(), one.data_ptr(), 1, hidden,
+                              EPS, stream()))
+        assert np.array_equal(bits_of(one), bits_of(d_n)[r])
+    # gather + norm against gather, then norm
+    vocab = 3000
+    table = oracle.normal_f16((vocab, hidden), 23, std=0.02)
+    ids = oracle.ids(rows, 24 + rows, vocab)
+    ids[0], ids[-1] = vocab - 1, 0
+    d_t, d_i = to_dev(table), torch.from_numpy(ids).cuda()
+    g_h = torch.full((rows, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    g_n = torch.full((rows, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_embedding_rmsnorm_dev(d_t.data_ptr(), d_i.data_ptr(), d_w.data_ptr(), g_h.data_ptr(),
+                                    g_n.data_ptr(), rows, hidden, EPS, stream()))
+    assert np.array_equal(bits_of(g_h), oracle.embedding_f16(table, ids)), "gather is not bit-exact"
+    u_h = torch.full((rows, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    u_n = torch.full((rows, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_embedding_dev(d_t.data_ptr(), d_i.data_ptr(), u_h.data_ptr(), rows, hidden, stream()))
+    ok(dev.vv_rmsnorm_dev(u_h.data_ptr(), d_w.data_ptr(), u_n.data_ptr(), rows, hidden, EPS, stream()))
+    assert np.array_equal(bits_of(u_h), bits_of(g_h)) and np.array_equal(bits_of(u_n), bits_of(g_n))
+    ref, rne = oracle.rmsnorm_f16(bits_of(g_h), w, EPS)
+    assert_fp16_close(bits_of(g_n), ref, rne, f"gather+rmsnorm [{rows},{hidden}]")
+
+
 # ── RoPE (config 3) ─────────────────────────────────────────────────────────
 
 def rope_check(got_bits, x_bits, off, theta, what):
@@ -247,6 +295,44 @@ def test_bias_rope_equals_bias_add_then_rope():
     assert np.array_equal(bits_of(f_q), bits_of(a_q)) and np.array_equal(bits_of(f_k), bits_of(a_k))
     biased_q = oracle.bias_add_f16(q.reshape(T, -1), qb).reshape(T, NQ, HD)
     rope_check(bits_of(f_q), biased_q, off, 1e6, "bias+rope Q")
+
+
+@pytest.mark.parametrize("T,off", [(1000, 0), (3001, 8192), (770, 31000)])
+def test_rope_mid_size_launches_agree_with_short_ones(T, off):
+    """A thousand to a few thousand positions run one wave per position, other lengths a
+    workgroup per position: same angle, same sincosf, same rotation, so the same bits - checked
+    against one-row launches, the device-side position and the bias form, then the oracle."""
+    q = oracle.normal_f16((T, NQ, HD), 950 + T)
+    k = oracle.normal_f16((T, NK, HD), 951 + T)
+    d_q, d_k = to_dev(q), to_dev(k)
+    ok(dev.vv_rope_qk_dev(d_q.data_ptr(), d_k.data_ptr(), T, NQ, NK, HD, off, None, 1e6, stream()))
+    rope_check(bits_of(d_q), q, off, 1e6, f"rope Q T={T}")
+    rope_check(bits_of(d_k), k, off, 1e6, f"rope K T={T}")
+    for r in (0, 1, T // 2, T - 1):
+        one_q, one_k = to_dev(q[r:r + 1]), to_dev(k[r:r + 1])
+        ok(dev.vv_rope_qk_dev(one_q.data_ptr(), one_k.data_ptr(), 1, NQ, NK, HD, off + r, None, 1e6, stream()))
+        assert np.array_equal(bits_of(one_q)[0], bits_of(d_q)[r]) and np.array_equal(bits_of(one_k)[0], bits_of(d_k)[r])
+    p_q, p_k = to_dev(q), to_dev(k)
+    d_pos = torch.tensor([off], dtype=torch.int32, device="cuda")
+    ok(dev.vv_rope_qk_dev(p_q.data_ptr(), p_k.data_ptr(), T, NQ, NK, HD, 0, d_pos.data_ptr(), 1e6, stream()))
+    assert np.array_equal(bits_of(p_q), bits_of(d_q)) and np.array_equal(bits_of(p_k), bits_of(d_k))
+    s_k = to_dev(k)                                  # K alone: 4 heads, a short launch in workgroup form
+    ok(dev.vv_rope_dev(s_k.data_ptr(), T, NK, HD, off, None, 1e6, stream()))
+    assert np.array_equal(bits_of(s_k), bits_of(d_k))
+    qb = oracle.normal_f16((NQ * HD,), 952, std=0.5)
+    kb = oracle.normal_f16((NK * HD,), 953, std=0.5)
+    a_q, a_k, d_qb, d_kb = to_dev(q), to_dev(k), to_dev(qb), to_dev(kb)
+    ok(dev.vv_bias_add_dev(a_q.data_ptr(), d_qb.data_ptr(), T, NQ * HD, stream()))
+    ok(dev.vv_bias_add_dev(a_k.data_ptr(), d_kb.data_ptr(), T, NK * HD, stream()))
+    ok(dev.vv_rope_qk_dev(a_q.data_ptr(), a_k.data_ptr(), T, NQ, NK, HD, off, None, 1e6, stream()))
+    f_q, f_k = to_dev(q), to_dev(k)
+    ok(dev.vv_bias_rope_qk_dev(f_q.data_ptr(), f_k.data_ptr(), d_qb.data_ptr(), None, T, NQ, NK, HD, off, None,
+                               1e6, stream()))
+    assert np.array_equal(bits_of(f_q), bits_of(a_q)) and np.array_equal(bits_of(f_k), bits_of(d_k))
+    f_q, f_k = to_dev(q), to_dev(k)
+    ok(dev.vv_bias_rope_qk_dev(f_q.data_ptr(), f_k.data_ptr(), d_qb.data_ptr(), d_kb.data_ptr(), T, NQ, NK, HD,
+                               off, None, 1e6, stream()))
+    assert np.array_equal(bits_of(f_q), bits_of(a_q)) and np.array_equal(bits_of(f_k), bits_of(a_k))
 
 
 # ── SwiGLU (config 4) ───────────────────────────────────────────────────────

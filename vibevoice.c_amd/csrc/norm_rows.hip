@@ -133,69 +133,87 @@ __global__ __launch_bounds__(kMaxWgThreads) void norm_rows_wg(
 // and never has more than half of its reads in flight. Here a row is one wave
 // with all of its loads (kCpl per tensor) issued back to back: 2048 rows are
 // 2048 waves, two per SIMD, every byte of the launch requested in the first
-// microsecond, no LDS and no barrier. The sum of squares keeps the workgroup
+// microsecond; the only barrier publishes the weight row, which the four waves
+// of a workgroup share through LDS. The sum of squares keeps the workgroup
 // kernel's order bit for bit: group j of 64 chunks is reduced like wave j of
 // that kernel (same DPP tree), and the groups are added in order from zero.
-template <int kCpl, int kMode, bool kStream>
+template <int kCpl, int kMode, bool kStream, bool kFull>      // kFull: nchunks == 64 * kCpl
 __global__ __launch_bounds__(kBlock) void norm_rows_wave(
     const Chunk* src, Chunk* state, const int32_t* __restrict__ ids,
     const Chunk* __restrict__ weight, Chunk* normed, int rows, int nchunks, float inv_n,
     float eps) {
-    const int row = (int)blockIdx.x * ((int)blockDim.x >> 6) + wave_in_block();
-    if (row >= rows) return;                      // whole waves leave; nothing below synchronises
-    const int lane = lane_id();
+    // The weight row goes through LDS once per workgroup instead of once per wave: measured
+    // cold against each wave loading its own copy, gather+norm 8.1 / 8.4 us at 2048 rows and
+    // 16.8 / 17.3 us at 4096, norm 6.0 / 6.6 us at 2048.
+    __shared__ Chunk wsh[kCpl * kWave];
     constexpr bool kGathers = kMode == kGather || kMode == kGatherOnly;
     constexpr bool kStreamSrc = kStream && !kGathers;
+    constexpr int kWeightLoads = (kCpl * kWave + kBlock - 1) / kBlock;
+    const int lane = lane_id();
+    const int want = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
+    const bool live = want < rows;               // a wave past the end re-reads the last row, stores nothing
+    const int row = live ? want : rows - 1;
+
+    // All loads are unconditional (an index past the end is clamped and its value unused), so
+    // the code up to the stores is one straight line and the waits count loads exactly. The
+    // weight chunks are requested first: loads are counted in order, so waiting for them does
+    // not wait for the row.
+    Chunk wmine[kWeightLoads];
+    if (kMode != kGatherOnly) {
+#pragma unroll
+        for (int i = 0; i < kWeightLoads; ++i)
+            wmine[i] = load_chunk(weight + min(i * kBlock + (int)threadIdx.x, nchunks - 1));
+    }
     const size_t src_row = kGathers ? (size_t)ids[row] : (size_t)row;
     const Chunk* s = src + src_row * (size_t)nchunks;
     const size_t out_base = (size_t)row * (size_t)nchunks;
 
-    Chunk a[kCpl], b[kCpl], w[kCpl];
+    Chunk a[kCpl], b[kCpl];
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (c < nchunks) {
-            a[j] = load_chunk_as<kStreamSrc>(s + c);
-            if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
-        }
+        const int c = kFull ? j * kWave + lane : min(j * kWave + lane, nchunks - 1);
+        a[j] = load_chunk_as<kStreamSrc>(s + c);
+        if (kMode == kAdd) b[j] = load_chunk_as<kStream>(state + out_base + c);
     }
     if (kMode == kGatherOnly) {
+        if (!live) return;
 #pragma unroll
         for (int j = 0; j < kCpl; ++j) {
             const int c = j * kWave + lane;
-            if (c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
+            if (kFull || c < nchunks) store_chunk_as<kStream>(state + out_base + c, a[j]);
         }
         return;
     }
 #pragma unroll
-    for (int j = 0; j < kCpl; ++j) {
-        const int c = j * kWave + lane;
-        if (c < nchunks) w[j] = load_chunk(weight + c);
-    }
+    for (int i = 0; i < kWeightLoads; ++i)      // clamped duplicates write the same bytes to the same slot
+        wsh[min(i * kBlock + (int)threadIdx.x, nchunks - 1)] = wmine[i];
+    __syncthreads();
+    if (!live) return;                           // no barrier below
+
     float total = 0.0f;
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
-        float acc = 0.0f;
-        if (c < nchunks) {
-            f32x8 x = unpack(a[j]);
-            if (kMode == kAdd) {
-                const f32x8 res = unpack(b[j]);
+        f32x8 x = unpack(a[j]);
+        if (kMode == kAdd) {
+            const f32x8 res = unpack(b[j]);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) x[i] = res[i] + x[i];
-                a[j] = pack(x);                   // the stored residual; the norm reads that value
-                x = unpack(a[j]);
-            }
-            if (kMode == kAdd || kMode == kGather) store_chunk_as<kStream>(state + out_base + c, a[j]);
-            acc = chunk_sumsq(x, 0.0f);
+            for (int i = 0; i < 8; ++i) x[i] = res[i] + x[i];
+            a[j] = pack(x);                       // the stored residual; the norm reads that value
+            x = unpack(a[j]);
         }
-        total += wave_sum(acc);
+        if ((kMode == kAdd || kMode == kGather) && (kFull || c < nchunks))
+            store_chunk_as<kStream>(state + out_base + c, a[j]);
+        const float acc = chunk_sumsq(x, 0.0f);
+        total += wave_sum((kFull || c < nchunks) ? acc : 0.0f);
     }
     const float inv = inv_rms(total, inv_n, eps);
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
-        if (c < nchunks) store_chunk_as<kStream>(normed + out_base + c, scale_chunk(a[j], inv, w[j]));
+        if (kFull || c < nchunks)
+            store_chunk_as<kStream>(normed + out_base + c,
+                                    scale_chunk(a[j], inv, wsh[kFull ? c : min(c, nchunks - 1)]));
     }
 }
 
@@ -278,11 +296,11 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         Chunk* o = static_cast<Chunk*>(normed);
         const bool full = nchunks == cpt * threads;
         // Which kernel: measured cold on MI355X at hidden 3584 with streaming accesses, a
-        // launch of R rows (times in us, workgroup per row / two rows per workgroup / wave
-        // per row):        R = 1024          2048            3072           6144          14449
-        //   add+norm    6.8  6.9  6.2   11.7 12.0 10.1  16.5 17.0 15.5  29.8 30.6 31.1  66.8 67.1 68.9
-        //   gather+norm 7.2  5.8  5.8   11.5  9.8  8.4  15.6 14.4 12.2  27.1 25.2 23.2  58.4 54.6 53.7
-        //   norm        4.1  4.4  5.3    7.6  6.3  6.5  10.1 10.2  8.7  17.3 16.7 15.7  38.0 34.2 37.0
+        // launch of R rows (us; workgroup per row / two rows per workgroup / wave per row):
+        //             R = 1024            2048             4096             8192            14449
+        //   add+norm    6.8  6.9  6.3   11.7 12.0 10.5   20.9 21.6 20.7   38.6 39.4 40.2   66.9 67.1 69.6
+        //   gather+norm 7.2  5.9  5.1   11.5  9.8  8.1   19.4 18.1 16.8   34.8 32.7 32.7   58.4 54.3 55.4
+        //   norm        4.1  4.4  3.9    7.7  6.3  6.0   12.7 12.3 11.2   22.0 20.9 20.8   37.2 34.4 34.7
         // A workgroup per row keeps ~1024 rows on the chip at once, so a few thousand rows
         // run as two or three dependent rounds; a wave per row has them all resident with
         // every load issued at the start. Long launches hide that and prefer light waves.
@@ -300,12 +318,13 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         bool wave = false;
         int rpw = 1;
         if (cpt == 1) {
-            if (kMode == kAdd) wave = eq_rows >= 896 && eq_rows <= 4608;
-            else if (kMode == kPlain) {
-                wave = eq_rows >= 2560 && eq_rows < 7168;
+            if (kMode == kAdd) {
+                wave = eq_rows >= 896 && eq_rows <= 4608;
+            } else if (kMode == kPlain) {
+                wave = eq_rows >= 1024 && eq_rows < 10240;
                 rpw = eq_rows >= 1536 ? 2 : 1;
             } else if (kMode == kGather) {
-                wave = eq_rows >= 768;
+                wave = eq_rows >= 768 && eq_rows < 10240;
                 rpw = eq_rows >= 256 ? 2 : 1;
             } else {
                 rpw = eq_rows >= 4096 ? 2 : 1;      // gather only: 32.4 us at 14449 rows (80 % of peak)
@@ -315,17 +334,22 @@ vv_status_t launch_rows(const void* src, void* state, const int32_t* ids, const 
         if (forced_wave >= 0 && !forced_rows) wave = forced_wave == 1;
         if (wave && cpt == 1 && nchunks <= 8 * kWave) {
             const dim3 wgrid((unsigned)((rows + kWavesPerBlock - 1) / kWavesPerBlock));
-#define VV_WAVE_CASE(C)                                                                           \
-    case C:                                                                                      \
-        if (stream) norm_rows_wave<C, kMode, true><<<wgrid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, \
-                                                                             nchunks, inv_n, eps);    \
-        else norm_rows_wave<C, kMode, false><<<wgrid, kBlock, 0, st>>>(s, stt, ids, w, o, rows,       \
-                                                                       nchunks, inv_n, eps);          \
-        break;
+#define VV_WAVE_LAUNCH(C, S, F)                                                               \
+    norm_rows_wave<C, kMode, S, F><<<wgrid, kBlock, 0, st>>>(s, stt, ids, w, o, rows, nchunks, \
+                                                            inv_n, eps)
+#define VV_WAVE_CASE(C)                                                  \
+    case C: {                                                           \
+        const bool wfull = nchunks == C * kWave;                        \
+        if (stream && wfull)  VV_WAVE_LAUNCH(C, true, true);            \
+        else if (stream)      VV_WAVE_LAUNCH(C, true, false);           \
+        else if (wfull)       VV_WAVE_LAUNCH(C, false, true);           \
+        else                  VV_WAVE_LAUNCH(C, false, false);          \
+    } break;
             switch ((nchunks + kWave - 1) / kWave) {
                 VV_WAVE_CASE(1) VV_WAVE_CASE(2) VV_WAVE_CASE(3) VV_WAVE_CASE(4)
                 VV_WAVE_CASE(5) VV_WAVE_CASE(6) VV_WAVE_CASE(7) VV_WAVE_CASE(8)
             }
+#undef VV_WAVE_LAUNCH
 #undef VV_WAVE_CASE
             return launch_status();
         }
