@@ -677,6 +677,29 @@ vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias,
                                 int n_kv_heads, int head_dim, int position_offset,
                                 const int* d_position, float theta, void* stream);
 
+/* addition: the cosines and sines of seq_len consecutive positions, computed once for
+ * every layer that rotates at those positions (src/inference/decoder.c:850-855 runs
+ * the same rotation in each of the 28 layers): table[row][i] = {cos, sin} of
+ * (float)(first + row) * theta^(-2i/head_dim), i < head_dim/2, as FP32 pairs
+ * (8 * seq_len * head_dim/2 bytes, 16-byte aligned), first = *d_position when
+ * d_position is given, else position_offset. The angle and the full-range sincosf
+ * are those of vv_rope_dev, so a rotation that reads the table gives its bits. */
+vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int position_offset,
+                              const int* d_position, float theta, void* stream);
+
+/* addition: a rotary projection in ONE launch, the q or k leg of decoder.c:825-855
+ * (vv_gemm_fp16_dev, vv_bias_add_dev, vv_rope_dev) with the bias and the rotation
+ * done in the GEMM's store: C[M, n_heads*head_dim] = rope(fp16(A[M,K] W[N,K]^T) +
+ * bias), row m rotated by row m of a vv_rope_table_dev table. Each step rounds to
+ * FP16 where the separate calls store, so the result equals vv_gemm_fp16_dev then
+ * vv_bias_rope_qk_dev bit for bit, and the projection is written once instead of
+ * written, read and written again. bias may be NULL. head_dim must be 128 and C,
+ * bias and the table 16-byte aligned (else VV_ERR_UNSUPPORTED, nothing launched);
+ * up to 64 rows, K % 8 != 0 or unaligned A / W run the two steps one after the other. */
+vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias, void* C,
+                                  int M, int n_heads, int head_dim, int K,
+                                  const void* rope_table, void* stream);
+
 /* addition: one activation row through up to three projections in ONE launch
  * (the decode step's q/k/v): y_i[N_i] = x[K] . W_i^T (+ bias_i). Equals
  * vv_gemm_fp16_dev(M = 1) followed by vv_bias_add_dev per projection bit for

@@ -135,6 +135,83 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     mfma_dma<F16Op>(A, B, M, N, K * 2, epilogue);
 }
 
+// The projection epilogue of a rotary attention layer in the GEMM's store: C = rope(fp16(A W^T) + bias)
+// for heads of 128 columns. The wave's two N tiles are 64 columns apart (kPairN), so register 4g + r of
+// acc[0] and of acc[1] are columns n and n + 64 of one head: the rotate-half pair. Every step rounds where
+// the separate launches round - the product to FP16 (the GEMM's store), the biased value to FP16 (the bias
+// add's store), then the unfused rotation of the rope kernels on cos/sin read from a table that holds
+// their sincosf values - so the result equals GEMM, then bias + RoPE, bit for bit.
+template <int TM>
+__device__ __forceinline__ void store_tile_rope(const f32x16 (&acc)[2][TM], h16* __restrict__ C,
+                                                const h16* __restrict__ bias, const float2* __restrict__ table,
+                                                int M, int N, int m0, int n0, int frow, int fhalf, float alpha,
+                                                float beta) {
+    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+    if (n0 >= N) return;                         // whole heads: the wave's 64 + 64 columns are all in or all out
+    const int pair0 = n0 & 127;                  // 0 or 32: the first rotation pair of tile 0
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const int m = m0 + b * 32 + frow;
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+        const float2* trow = table + (size_t)m * 64;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int col = 8 * g + 4 * fhalf;
+            const int n = n0 + col;
+            h16x4 lo, hi;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                lo[r] = to_half(finish(acc[0][b][4 * g + r], alpha, beta, (h16)0.0f));
+                hi[r] = to_half(finish(acc[1][b][4 * g + r], alpha, beta, (h16)0.0f));
+            }
+            if (bias) {
+                const h16x4 blo = *reinterpret_cast<const h16x4*>(bias + n);
+                const h16x4 bhi = *reinterpret_cast<const h16x4*>(bias + n + 64);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    lo[r] = to_half((float)lo[r] + (float)blo[r]);
+                    hi[r] = to_half((float)hi[r] + (float)bhi[r]);
+                }
+            }
+            const float4 cs01 = *reinterpret_cast<const float4*>(trow + pair0 + col);
+            const float4 cs23 = *reinterpret_cast<const float4*>(trow + pair0 + col + 2);
+            const float cv[4] = {cs01.x, cs01.z, cs23.x, cs23.z};
+            const float sv[4] = {cs01.y, cs01.w, cs23.y, cs23.w};
+            h16x4 olo, ohi;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const Pair p = rotate((float)lo[r], (float)hi[r], cv[r], sv[r]);
+                olo[r] = to_half(p.lo);
+                ohi[r] = to_half(p.hi);
+            }
+            *reinterpret_cast<h16x4*>(crow + n) = olo;
+            *reinterpret_cast<h16x4*>(crow + n + 64) = ohi;
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int kSlab, bool kFull, int kAhead>
+__global__ __launch_bounds__(WM * WN * kWave) void gemm_tile_rope(
+    const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
+    const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    auto epilogue = [=](const f32x16 (&acc)[TN][TM], int m0, int n0, int frow, int fhalf) {
+        store_tile_rope<TM>(acc, C, bias, table, M, N, m0, n0, frow, fhalf, alpha, beta);
+    };
+    mfma_tile<F16Op, BM, BN, WM, WN, kSlab / 8, kFull, kAhead, decltype(epilogue), PlainRows, true>(
+        A, B, M, N, K / 8, epilogue);
+}
+
+__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma_rope(
+    const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
+    const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
+    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
+        store_tile_rope<4>(acc, C, bias, table, M, N, m0, n0, frow, fhalf, alpha, beta);
+    };
+    mfma_dma<F16Op, true>(A, B, M, N, K * 2, epilogue);
+}
+
 // M == 1: bound by the weight bytes. kSplit waves share an output column (a
 // weight row), each streaming a contiguous 1/kSplit of it with non-temporal
 // 16-byte loads, four in flight; their sums meet in LDS. Narrow outputs take
@@ -515,6 +592,50 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
     return launch_status();
 }
 
+// C = rope(fp16(A W^T) + bias) in the GEMM's store, for the shapes the LDS-tiled kernels serve: the
+// same tile rule as gemm() above 64 rows, except that the two small tiles give way to 64 x 128 (the
+// narrowest block that holds a whole head; all tile shapes add K in the same order). false: nothing
+// launched (up to 64 rows, where gemm() streams the weights in another K order, and odd K).
+template <int BM, int BN, int WM, int WN, int kSlab, int kAhead>
+void launch_tile_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N,
+                      int K, hipStream_t st) {
+    const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    if (K % kSlab == 0)
+        gemm_tile_rope<BM, BN, WM, WN, kSlab, true, kAhead><<<grid, WM * WN * kWave, 0, st>>>(
+            A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
+    else
+        gemm_tile_rope<BM, BN, WM, WN, kSlab, false, kAhead><<<grid, WM * WN * kWave, 0, st>>>(
+            A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
+}
+
+bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N, int K,
+               hipStream_t st, int choice) {
+    if (M <= 64 || K <= 0 || K % 8 != 0) return false;
+    if (choice == kAuto) {
+        const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+        const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+        choice = wg256 >= 512 ? k256 : wg128 >= 256 ? k128 : k64;
+    }
+    if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
+        static thread_local int ready_device = -1;
+        int device = 0;
+        if (hipGetDevice(&device) == hipSuccess &&
+            (ready_device == device ||
+             hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma_rope),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLdsBytes) == hipSuccess)) {
+            ready_device = device;
+            const dim3 grid((unsigned)((N + kDmaTile - 1) / kDmaTile), (unsigned)((M + kDmaTile - 1) / kDmaTile));
+            gemm_dma_rope<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
+            return true;
+        }
+        (void)hipGetLastError();
+    }
+    if (choice == k256 || choice == k256regs) launch_tile_rope<256, 256, 2, 4, 32, 2>(A, B, bias, table, C, M, N, K, st);
+    else if (choice == k128) launch_tile_rope<128, 128, 2, 2, 64, 2>(A, B, bias, table, C, M, N, K, st);
+    else launch_tile_rope<64, 128, 2, 2, 64, 1>(A, B, bias, table, C, M, N, K, st);
+    return true;
+}
+
 int forced_tile() {
     static const int v = [] {
         const char* e = getenv("VV_GEMM_TILE");
@@ -580,6 +701,9 @@ vv_status_t vv_gemm_tile_weight_only(int format, const void* A, const void* w, c
     if (format == vv::kWoAwq) return tile_wo<vv::kWoAwq>(a, B, c, M, N, K, st);
     return VV_ERR_UNSUPPORTED;
 }
+
+// rope.hip: x[rows][heads][128] = rope(x + bias), cos/sin from a vv_rope_table_dev table.
+vv_status_t vv_rope128_from_table(void* x, const void* bias, const void* table, int rows, int heads, void* stream);
 
 extern "C" {
 
@@ -671,6 +795,25 @@ vv_status_t vv_gemv_swiglu_dev(const void* x, const void* w_gate, const void* w_
     else if (split == 2) vv::gemv_multi<2, 1><<<grid, vv::kBlock, 0, st>>>(a, p, K);
     else vv::gemv_multi<4, 1><<<grid, vv::kBlock, 0, st>>>(a, p, K);
     return vv::launch_status();
+}
+
+vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias, void* C, int M,
+                                  int n_heads, int head_dim, int K, const void* rope_table, void* stream) {
+    if (!A || !W || !C || !rope_table) return VV_ERR_NULL_PTR;
+    if (M <= 0 || n_heads <= 0) return VV_OK;
+    if (K < 0) return VV_ERR_INVALID_ARG;
+    if (head_dim != 128 || !vv::aligned16(C) || !vv::aligned16(rope_table) || (bias && !vv::aligned16(bias)))
+        return VV_ERR_UNSUPPORTED;
+    const int N = n_heads * 128;
+    if (vv::aligned16(A) && vv::aligned16(W) &&
+        vv::gemm_rope(static_cast<const vv::h16*>(A), static_cast<const vv::h16*>(W),
+                      static_cast<const vv::h16*>(bias), static_cast<const float2*>(rope_table),
+                      static_cast<vv::h16*>(C), M, N, K, vv::as_stream(stream), vv::forced_tile()))
+        return vv::launch_status();
+    // What the fused kernels do not cover: the two steps one after the other, on the same table.
+    const vv_status_t s = vv::gemm(A, W, C, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
+    if (s != VV_OK) return s;
+    return vv_rope128_from_table(C, bias, rope_table, M, n_heads, stream);
 }
 
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M, int N, int K,

@@ -33,7 +33,11 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_byte_ad
                  : "memory", "m0");
 }
 
-template <typename Op, typename Epi>
+// kPairN: a wave's two N tiles are 64 columns apart instead of adjacent - wave wn takes columns
+// 128 (wn / 2) + 32 (wn % 2) + {0, 64} of the block - so that an epilogue finds columns n and n + 64
+// (the rotate-half pair of a 128-wide head) in the same lane and register of acc[0] and acc[1]. The
+// products and their order per output element do not change.
+template <typename Op, bool kPairN = false, typename Epi>
 __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
                                          int row_bytes, const Epi& epi) {
     typedef typename Op::Acc Acc;
@@ -91,7 +95,9 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
     for (int step = 0; step < 2; ++step)
         f_idx[step] = frow * kSlabChunks + swz<32>(frow, step * 2 + fhalf);
     const int fa_base = wm * TM * 32 * kSlabChunks;
-    const int fb_base = kDmaTile * kSlabChunks + wn * TN * 32 * kSlabChunks;
+    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 32;      // first column of tile a = 0
+    constexpr int kTileStrideN = kPairN ? 64 : 32;
+    const int fb_base = kDmaTile * kSlabChunks + wave_n0 * kSlabChunks;
 
     // Fragment reads run a whole slab ahead: while the 16 MFMAs of slab s execute
     // from one register set, the operands of slab s + 1 come in from LDS into the
@@ -103,7 +109,7 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
         const u32x4* st = dma_lds + (slab % kDmaStages) * kDmaStageSlots;
 #pragma unroll
         for (int a = 0; a < TN; ++a)
-            fw[set][step][a] = st[fb_base + a * 32 * kSlabChunks + f_idx[step]];
+            fw[set][step][a] = st[fb_base + a * kTileStrideN * kSlabChunks + f_idx[step]];
 #pragma unroll
         for (int b = 0; b < TM; ++b)
             fx[set][step][b] = st[fa_base + b * 32 * kSlabChunks + f_idx[step]];
@@ -150,7 +156,7 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
     if (slab < nslabs) one_slab(Const<0>{}, Const<1>{}, slab);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus copies land before the LDS is released
 
-    epi(acc, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf);
+    epi(acc, m_blk + wm * TM * 32, n_blk + wave_n0, frow, fhalf);
 }
 
 }  // namespace vv

@@ -36,8 +36,12 @@ struct Const { static constexpr int value = kValue; };
 // u32x4 load(int row, int slot) const.
 struct PlainRows { static constexpr bool kPlain = true; };
 
+// kPairN (wave tiles of two N tiles, BN a multiple of 128): the two N tiles of a wave are 64 columns
+// apart - wave wn takes columns 128 (wn / 2) + 32 (wn % 2) + {0, 64} of the block - so that an epilogue
+// finds columns n and n + 64 in the same lane and register of acc[0] and acc[1]; epi's n0 is then the
+// first column of tile 0. The products and their order per output element do not change.
 template <typename Op, int BM, int BN, int WM, int WN, int kSlabChunks, bool kFull, int kAhead,
-          typename Epi, typename BSrc = PlainRows>
+          typename Epi, typename BSrc = PlainRows, bool kPairN = false>
 __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void* __restrict__ B,
                                           int M, int N, int kchunks, const Epi& epi, const BSrc& bsrc = BSrc()) {
     constexpr int NT = WM * WN * kWave;
@@ -137,7 +141,10 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
     for (int step = 0; step < kSteps; ++step)
         f_idx[step] = frow * kSlabChunks + swz<kSlabChunks * 8>(frow, step * 2 + fhalf);
     const int fa_base = wm * TM * 32 * kSlabChunks;
-    const int fb_base = kASlots + wn * TN * 32 * kSlabChunks;
+    static_assert(!kPairN || (TN == 2 && BN % 128 == 0), "paired N tiles: two tiles per wave, whole heads per block");
+    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 32;      // first column of tile a = 0
+    constexpr int kTileStrideN = kPairN ? 64 : 32;
+    const int fb_base = kASlots + wave_n0 * kSlabChunks;
 
     // One slab: the operand fragments of step s + 1 are read from LDS before
     // the MFMAs of step s are issued.
@@ -148,7 +155,7 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
             constexpr int set = decltype(set_c)::value;
 #pragma unroll
             for (int a = 0; a < TN; ++a)
-                fw[set][a] = src[fb_base + a * 32 * kSlabChunks + f_idx[step]];
+                fw[set][a] = src[fb_base + a * kTileStrideN * kSlabChunks + f_idx[step]];
 #pragma unroll
             for (int b = 0; b < TM; ++b)
                 fx[set][b] = src[fa_base + b * 32 * kSlabChunks + f_idx[step]];
@@ -201,7 +208,7 @@ __device__ __forceinline__ void mfma_tile(const void* __restrict__ A, const void
         }
     }
 
-    epi(acc, m_blk + wm * TM * 32, n_blk + wn * TN * 32, frow, fhalf);
+    epi(acc, m_blk + wm * TM * 32, n_blk + wave_n0, frow, fhalf);
 }
 
 }  // namespace vv

@@ -20,7 +20,7 @@
 //     (never the fast intrinsics, whose error grows with |angle|).
 #include <math.h>
 
-#include "vv_common.hpp"
+#include "row_math.hpp"
 
 namespace vv {
 namespace {
@@ -47,21 +47,6 @@ __device__ __forceinline__ Chunk add_bias(const Chunk& v, const Chunk& b) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = x[i] + y[i];
     return pack(r);      // rounded to FP16 before the rotation, as bias_add then rope would
-}
-
-// The rotation itself, in the CPU path's arithmetic: four products, one
-// subtraction, one addition, none of them fused, so that the only difference
-// from the CPU result is the last bits of sin/cos.
-struct Pair {
-    float lo, hi;
-};
-__device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
-#pragma clang fp contract(off)
-    const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
-    Pair r;
-    r.lo = ac - bs;
-    r.hi = as + bc;
-    return r;
 }
 
 // head_dim == 128, 16-byte aligned tensors, at most kMaxFastHeads heads in all.
@@ -277,6 +262,53 @@ __global__ __launch_bounds__(kBlock) void rope_generic(RopeArgs a, FreqTable fre
     }
 }
 
+// The cosines and sines of a run of positions, once for every layer that rotates at those
+// positions: table[row][i] = {cos, sin}((float)(first + row) * inv_freq[i]), i < head_dim / 2 -
+// the angle and the sincosf of the rope kernels, so a rotation that reads the table gives their bits.
+__global__ __launch_bounds__(kBlock) void rope_table(float2* __restrict__ table, int rows, int half,
+                                                     int position_offset, const int* __restrict__ d_position,
+                                                     FreqTable freqs) {
+    const int idx = (int)blockIdx.x * kBlock + (int)threadIdx.x;
+    if (idx >= rows * half) return;
+    const int row = idx / half, i = idx - row * half;
+    const int first = d_position ? *d_position : position_offset;
+    float s, c;
+    sincosf((float)(first + row) * freqs.f[i], &s, &c);
+    table[idx] = make_float2(c, s);
+}
+
+// x[row][head][:] = rope(x (+ bias)) with cos/sin read from such a table: the form of
+// vv_bias_rope_qk_dev for callers that hold one. One thread per (row, head, chunk pair), head_dim 128.
+__global__ __launch_bounds__(kBlock) void rope128_from_table(h16* __restrict__ x, const h16* __restrict__ bias,
+                                                             const float2* __restrict__ table, int rows,
+                                                             int heads) {
+    const size_t item = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (item >= (size_t)rows * heads * 8) return;
+    const int c = (int)(item & 7);
+    const size_t rh = item >> 3;
+    const int head = (int)(rh % heads);
+    const size_t row = rh / heads;
+    Chunk* lo_p = reinterpret_cast<Chunk*>(x + rh * 128u) + c;
+    Chunk lo = load_chunk(lo_p), hi = load_chunk(lo_p + 8);
+    if (bias) {
+        const Chunk* bp = reinterpret_cast<const Chunk*>(bias + (size_t)head * 128u) + c;
+        lo = add_bias(lo, load_chunk(bp));
+        hi = add_bias(hi, load_chunk(bp + 8));
+    }
+    const float2* t = table + row * 64 + c * 8;
+    const f32x8 x0 = unpack(lo), x1 = unpack(hi);
+    f32x8 y0, y1;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float2 cs = t[i];
+        const Pair r = rotate(x0[i], x1[i], cs.x, cs.y);
+        y0[i] = r.lo;
+        y1[i] = r.hi;
+    }
+    store_chunk(lo_p, pack(y0));
+    store_chunk(lo_p + 8, pack(y1));
+}
+
 // The table depends only on (theta, head_dim); each host thread remembers the
 // last one it built (thread-local, so concurrent callers never share state).
 const FreqTable& host_freqs(float theta, int head_dim) {
@@ -404,4 +436,28 @@ vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias, const void
                            position_offset, d_position, theta, vv::as_stream(stream));
 }
 
+vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int position_offset,
+                              const int* d_position, float theta, void* stream) {
+    if (!table) return VV_ERR_NULL_PTR;
+    if (seq_len <= 0 || head_dim <= 0) return VV_OK;
+    if ((head_dim & 1) || head_dim > 2 * vv::kMaxPairs) return VV_ERR_UNSUPPORTED;
+    if (reinterpret_cast<uintptr_t>(table) & 7u) return VV_ERR_INVALID_ARG;
+    const int half = head_dim / 2;
+    const size_t n = (size_t)seq_len * (size_t)half;
+    vv::rope_table<<<dim3((unsigned)((n + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0, vv::as_stream(stream)>>>(
+        static_cast<float2*>(table), seq_len, half, position_offset, d_position, vv::host_freqs(theta, head_dim));
+    return vv::launch_status();
+}
+
 }  // extern "C"
+
+// For gemm.hip: x[rows][heads][128] = rope(x + bias) with cos/sin from a vv_rope_table_dev table
+// (16-byte aligned x and bias, table rows 0 .. rows - 1).
+__attribute__((visibility("hidden")))
+vv_status_t vv_rope128_from_table(void* x, const void* bias, const void* table, int rows, int heads, void* stream) {
+    const size_t items = (size_t)rows * (size_t)heads * 8u;
+    vv::rope128_from_table<<<dim3((unsigned)((items + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
+                             vv::as_stream(stream)>>>(static_cast<vv::h16*>(x), static_cast<const vv::h16*>(bias),
+                                                      static_cast<const float2*>(table), rows, heads);
+    return vv::launch_status();
+}

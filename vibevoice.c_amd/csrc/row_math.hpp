@@ -89,6 +89,23 @@ __device__ __forceinline__ Chunk scale_chunk(const Chunk& x16, float inv, const 
     return pack(x);
 }
 
+// ── RoPE ─────────────────────────────────────────────────────────────────
+
+// The rotation of one (lo, hi) pair in the CPU path's arithmetic: four products,
+// one subtraction, one addition, none of them fused, so that the only difference
+// from the CPU result is the last bits of sin/cos.
+struct Pair {
+    float lo, hi;
+};
+__device__ __forceinline__ Pair rotate(float a, float b, float c, float s) {
+#pragma clang fp contract(off)
+    const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+    Pair r;
+    r.lo = ac - bs;
+    r.hi = as + bc;
+    return r;
+}
+
 // ── SwiGLU ───────────────────────────────────────────────────────────────
 
 // silu(g) * u in the CPU path's association, (g / (1 + e^-g)) * u, with the
