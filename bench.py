@@ -507,11 +507,49 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
     out["attn_prefill"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf,
                            "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
     scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
-    sec = timed(lambda: dev.vv_attn_decode(2, q.data_ptr(), C.addressof(view), o.data_ptr(), NQ, T, None,
-                                           scratch.data_ptr(), st), 50)
-    gb = 2.0 * T * NK * HD * 2 / sec / 1e9
-    out["attn_decode"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS,
-                          "note": "two launches; the host's launch rate bounds this figure"}
+    # Decode reads each layer's cache once per token: 28 caches in rotation (829 MB at T = 14449, so nothing
+    # is served from the last-level cache), issued one by one and as one captured graph replayed.
+    caches = [(torch.randn(T, NK, HD, dtype=torch.float16, device="cuda"),
+               torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")) for _ in range(28)]
+    views = [dev.KvView(k=kk.data_ptr(), v=vv.data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                        format=0, n_kv_heads=NK, head_dim=HD) for kk, vv in caches]
+
+    ds = C.c_void_p()                      # a stream of its own: the default stream cannot be captured
+    assert dev.vv_dev_stream_create(C.byref(ds)) == 0
+
+    def decode_all():
+        for vw in views:
+            assert dev.vv_attn_decode(2, q.data_ptr(), C.addressof(vw), o.data_ptr(), NQ, T, None,
+                                      scratch.data_ptr(), ds.value) == 0
+
+    def wall(fn, reps=10):                 # host clock around a drained stream, median of three
+        fn()
+        assert dev.vv_dev_stream_sync(ds.value) == 0
+        per = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            assert dev.vv_dev_stream_sync(ds.value) == 0
+            per.append((time.perf_counter() - t0) / reps)
+        return sorted(per)[1]
+
+    torch.cuda.synchronize()
+    sec = wall(decode_all) / len(views)
+    assert dev.vv_dev_graph_begin(ds.value) == 0
+    decode_all()
+    g = C.c_void_p()
+    assert dev.vv_dev_graph_end(ds.value, C.byref(g)) == 0 and g.value
+    sec_graph = wall(lambda: dev.vv_dev_graph_launch(g.value, ds.value)) / len(views)
+    dev.vv_dev_graph_destroy(g.value)
+    dev.vv_dev_stream_destroy(ds.value)
+    nbytes = 2.0 * T * NK * HD * 2
+    out["attn_decode"] = {"cache_len": T, "caches_in_rotation": len(views), "us": sec * 1e6, "GBps": nbytes / sec / 1e9,
+                          "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS, "graph_us": sec_graph * 1e6,
+                          "graph_GBps": nbytes / sec_graph / 1e9,
+                          "note": "two launches per call (slices, then their merge); about 8 us of it is launch and "
+                                  "memory latency, the same at 1000 positions"}
+    del caches, views
     # The same two over an FP8 (E4M3) cache: half the cache bytes, widened on their way into the tile.
     k8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
     v8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
@@ -596,12 +634,21 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
     def gemm(x, wt, y, n, kk):
         assert dev.vv_gemm_fp16_dev(P(x), P(wt), P(y), T, n, kk, 1.0, 0.0, st) == 0
 
-    def layer():
+    # cos/sin of the prompt's positions: once per forward pass, shared by the 28 layers
+    rope_table = torch.empty(T, HD // 2, 2, dtype=torch.float32, device="cuda")
+    assert dev.vv_rope_table_dev(P(rope_table), T, HD, 0, None, THETA, st) == 0
+
+    def layer(fused=True):
         assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0
-        gemm(normed, wq, q, QD, H)
-        gemm(normed, wk, k, KD, H)
+        if fused:       # bias + RoPE in the projection's store
+            assert dev.vv_gemm_bias_rope_dev(P(normed), P(wq), P(bq), P(q), T, NQ, HD, H, P(rope_table), st) == 0
+            assert dev.vv_gemm_bias_rope_dev(P(normed), P(wk), P(bk), P(k), T, NK, HD, H, P(rope_table), st) == 0
+        else:
+            gemm(normed, wq, q, QD, H)
+            gemm(normed, wk, k, KD, H)
         gemm(normed, wv, v, KD, H)
-        assert dev.vv_bias_rope_qk_dev(P(q), P(k), P(bq), P(bk), T, NQ, NK, HD, 0, None, THETA, st) == 0
+        if not fused:
+            assert dev.vv_bias_rope_qk_dev(P(q), P(k), P(bq), P(bk), T, NQ, NK, HD, 0, None, THETA, st) == 0
         assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
         assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, T, 0, T, True, None, st) == 0
         gemm(attn, wo, proj, H, QD)
@@ -612,22 +659,26 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
         gemm(gate, wd, proj, H, I_FF)
         assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
 
-    layer()
-    torch.cuda.synchronize()
-    per = []
-    for _ in range(3):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        layer()
-        e1.record()
-        e1.synchronize()
-        per.append(e0.elapsed_time(e1))
-    per.sort()
-    ms = per[1]
+    def time_layer(fused):
+        layer(fused)
+        torch.cuda.synchronize()
+        per = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            layer(fused)
+            e1.record()
+            e1.synchronize()
+            per.append(e0.elapsed_time(e1))
+        per.sort()
+        return per[1]
+
+    ms_separate = time_layer(False)
+    ms = time_layer(True)
     assert bool(torch.isfinite(hidden).all())
     flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
-    return {"rows": T, "ms_per_layer": ms, "TFLOPs": flops / ms / 1e9, "layers_assumed": 28,
-            "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
+    return {"rows": T, "ms_per_layer": ms, "ms_per_layer_rope_as_its_own_launch": ms_separate,
+            "TFLOPs": flops / ms / 1e9, "layers_assumed": 28, "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
 
 
 def prefill_layer_quant_leg(torch, dev, T: int, st: int, kind: str) -> dict:
@@ -1209,7 +1260,8 @@ def main() -> int:
         log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         d = layer["attn_decode"]
-        log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s "
+            f"(replayed from a graph: {d['graph_us']:.2f} us {d['graph_GBps']:.1f} GB/s)")
         d = layer["attn_prefill_fp8"]
         log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
         d = layer["attn_decode_fp8"]

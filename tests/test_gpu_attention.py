@@ -143,7 +143,8 @@ def test_paged_cache_matches_contiguous(rows, nq, nkv, off):
         assert np.array_equal(outs[0], outs[1])
 
 
-@pytest.mark.parametrize("nq,nkv,hd", [(28, 4, 128), (2, 1, 128), (40, 1, 128), (12, 2, 128), (4, 2, 64)])
+# groups of 7, 2, 40 (beyond the streaming kernel), 6, 16 and 12 query heads per KV head; head_dim 64: the generic kernel
+@pytest.mark.parametrize("nq,nkv,hd", [(28, 4, 128), (2, 1, 128), (40, 1, 128), (12, 2, 128), (4, 2, 64), (32, 2, 128), (24, 2, 128)])
 @pytest.mark.parametrize("cache_len", [1, 17, 64, 65, 255, 257, 1000, 5000, 14449, 40000])
 def test_decode_against_oracle(nq, nkv, hd, cache_len):
     q, k, v = make(1, nq, nkv, hd, cache_len, cache_len + nq)

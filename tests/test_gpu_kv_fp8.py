@@ -143,6 +143,15 @@ def test_prefill_equals_fp16_cache_of_decoded_values(fmt, q_len, q_offset, kv_le
     assert err < (0.5 if fmt == E4M3 else 1.0), err      # half a step of a value near 6: 3 or 2 mantissa bits
 
 
+def same_attention(a_bits, b_bits, what):
+    """A packed cache and the FP16 cache of its decoded values hold the same numbers; their decodes run
+    different kernels (the FP16 cache streams, the packed ones go through the LDS tile), so the results
+    agree to the rounding of the probabilities (FP16, 2^-11 relative) rather than bit for bit."""
+    a, b = oracle.widen(a_bits).astype(np.float64), oracle.widen(b_bits).astype(np.float64)
+    err = np.abs(a - b).max() / max(np.abs(b).max(), 1e-9)
+    assert err <= 1e-3, f"{what}: packed and FP16 decodes differ by {err:.2e} of the largest output"
+
+
 @pytest.mark.parametrize("fmt", [E4M3, E5M2])
 @pytest.mark.parametrize("cache_len,paged", [(1, False), (64, False), (65, False), (1500, False), (14449, False), (700, True)])
 def test_decode_equals_fp16_cache_of_decoded_values(fmt, cache_len, paged):
@@ -171,7 +180,7 @@ def test_decode_equals_fp16_cache_of_decoded_values(fmt, cache_len, paged):
         ok(dev.vv_attn_decode(FA2, d_q.data_ptr(), C.addressof(vw), d_o.data_ptr(), nq, cache_len, d_len.data_ptr(),
                               scratch.data_ptr(), stream()))
         outs.append(bits_of(d_o))
-    assert np.array_equal(outs[0], outs[1])
+    same_attention(outs[0], outs[1], f"fp8 decode, cache {cache_len}")
     if not paged:
         d_o = torch.full((1, nq, HD), float("nan"), dtype=torch.float16, device="cuda")
         d_kq, d_vq = u8(kq), u8(vq)

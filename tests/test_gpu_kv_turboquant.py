@@ -41,6 +41,16 @@ def qwen_like(n, seed):
     return oracle.narrow(k), oracle.narrow(v)
 
 
+
+
+def same_attention(a_bits, b_bits, what):
+    """A packed cache and the FP16 cache of its decoded values hold the same numbers; their decodes run
+    different kernels (the FP16 cache streams, the packed ones go through the LDS tile), so the results
+    agree to the rounding of the probabilities (FP16, 2^-11 relative) rather than bit for bit."""
+    a, b = oracle.widen(a_bits).astype(np.float64), oracle.widen(b_bits).astype(np.float64)
+    err = np.abs(a - b).max() / max(np.abs(b).max(), 1e-9)
+    assert err <= 1e-3, f"{what}: packed and FP16 decodes differ by {err:.2e} of the largest output"
+
 def test_rotation_bit_exact_and_inverse():
     x = oracle.normal_f16((5, 28, HD), 1, std=2.0)
     d_x = to_dev(x)
@@ -131,7 +141,7 @@ def test_decode_equals_fp16_cache_of_unpacked_vectors_and_tracks_fp16_attention(
         ok(dev.vv_attn_decode(FA2, d_q.data_ptr(), C.addressof(vw), d_o.data_ptr(), nq, cache_len, None,
                               scratch.data_ptr(), stream()))
         outs.append(bits_of(d_o))
-    assert np.array_equal(outs[0], outs[1])
+    same_attention(outs[0], outs[1], f"TurboQuant decode, cache {cache_len}")
     # the older entry point, then the recipe's last step
     d_ks, d_vs, d_km, d_vm = u8(ks), u8(vs), to_dev(km), to_dev(vm)
     d_o = torch.full((1, nq, HD), float("nan"), dtype=torch.float16, device="cuda")

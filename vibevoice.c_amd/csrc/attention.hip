@@ -531,6 +531,187 @@ __global__ __launch_bounds__(kWave) void decode128(
     }
 }
 
+// ── decode over an FP16 cache, head_dim 128, groups of up to 16 query heads ───
+// The decode is a stream of the cache: 512 bytes per position and KV head, used once,
+// and a launch lives for a few microseconds, so what counts is that every byte is
+// requested at once and that a wave has little code to run when its bytes arrive (a
+// wave's first pass over its code is a chain of instruction-cache misses). A
+// workgroup of sixteen waves owns a slice of the positions of one KV head; wave w
+// takes the 16-key blocks w, w + 16, ... of the slice, one block at a time with the
+// next block's eight loads (16 bytes per lane each) in flight. At 14k positions a
+// wave has exactly one block: the whole cache is in flight from the first
+// microsecond, 2048 short waves per KV head. Both products run on the matrix cores
+// with the group's query heads in the place of rows:
+//   scores   S^T = K Q^T (16x16x32): the K rows go from global memory straight into
+//            the A operand - lane (key l % 16, j = l / 16) holds channels
+//            32 s + 8 j .. + 7 in step s, the query fragment the same channels - and
+//            lane (head l % 16, j) ends up with keys 4 j .. 4 j + 3 of the block.
+//   softmax  online per head in FP32, base-2 domain; maximum and sum cross the four
+//            j groups by lane exchange. The probabilities, rounded to FP16, are
+//            already the B operand of the second product (16x16x16, k = key).
+//   O^T      = V^T P^T: lane (chunk c = l % 16, j) loads keys 4 j .. 4 j + 3 of chunk
+//            c as stored and writes, per channel, the four keys as 8 bytes into the
+//            wave's own LDS tile [e][c][16 keys] (channel 8 c + e); the 16 channels
+//            {8 c + e} of one e form an A tile, so writes and reads alike touch each
+//            bank once per 32 lanes. Lane (head l % 16, j') accumulates channels
+//            32 j' + 8 r + e in FP32.
+// Only V passes through LDS, and only inside its own wave (no workgroup barrier in
+// the loop). The waves' states meet in LDS and the workgroup leaves one (max, sum,
+// unnormalised O) record per head in `parts`, for decode_merge.
+constexpr int kStreamWaves = 16;
+constexpr int kStreamThreads = kStreamWaves * kWave;
+constexpr int kStreamOStride = kD + 1;          // floats per head in the waves' exchange (odd: spreads banks)
+// A wave's LDS: V^T of a block (4 KB), later its O for kHeads heads.
+constexpr int stream_tile_bytes(int heads) { return heads * kStreamOStride * 4 < 4096 ? 4096 : (heads * kStreamOStride * 4 + 15) / 16 * 16; }
+
+__device__ __forceinline__ float xor_lanes16(float v) { return __shfl_xor(v, 16); }
+
+template <int kHeads>      // the group's query heads, padded: 8 or 16
+__global__ __launch_bounds__(kStreamThreads) void decode_stream(
+    const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V,
+    const int* __restrict__ page_table, float* __restrict__ parts, int n_q_heads, int n_kv_heads,
+    int cache_len, const int* __restrict__ d_cache_len, int n_parts, float scale_log2) {
+    // Per wave: V^T of the block in hand, [e][c][16 keys] halves; after its loop the wave's O instead,
+    // [head][kStreamOStride] floats (a wave touches no other wave's tile before the barrier).
+    __shared__ __attribute__((aligned(16))) char tile_lds[kStreamWaves][stream_tile_bytes(kHeads)];
+    __shared__ float m_lds[kStreamWaves][16], l_lds[kStreamWaves][16];
+    auto o_of = [&](int w) { return reinterpret_cast<float*>(tile_lds[w]); };
+
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = wave_in_block();
+    const int c = lane & 15, j = lane >> 4;        // c: key (scores) / head (softmax, O) / chunk (V loads)
+    h16 (*vt)[16][16] = reinterpret_cast<h16 (*)[16][16]>(tile_lds[wave]);
+    const int part = (int)blockIdx.x, kvh = (int)blockIdx.y;
+    const int group = n_q_heads / n_kv_heads;
+    const int len = d_cache_len ? *d_cache_len : cache_len;
+    const int per = (((len + n_parts - 1) / n_parts) + 15) & ~15;
+    const int begin = part * per, end = min(len, begin + per);
+    const size_t row_halves = (size_t)n_kv_heads * kD;
+
+    // Block n of this wave starts at key begin + 16 (wave + 16 n). Keys past the slice repeat its last
+    // key (finite values; their scores are masked).
+    Chunk kr[4], vr[4];
+    auto fetch = [&](int key0) {
+        const int tk = min(key0 + c, end - 1);
+        const Chunk* kp = reinterpret_cast<const Chunk*>(K + (size_t)cache_row(page_table, tk) * row_halves +
+                                                         (size_t)kvh * kD);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) kr[s] = load_chunk_stream(kp + 4 * s + j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tv = min(key0 + 4 * j + i, end - 1);
+            vr[i] = load_chunk_stream(reinterpret_cast<const Chunk*>(
+                V + (size_t)cache_row(page_table, tv) * row_halves + (size_t)kvh * kD) + c);
+        }
+    };
+    int key0 = begin + 16 * wave;
+    if (key0 < end) fetch(key0);
+
+    // The query fragments of this lane's head: channels 32 s + 8 j .. + 7 of step s.
+    h16x8 qf[4];
+    {
+        const Chunk* qp = reinterpret_cast<const Chunk*>(Q + (size_t)(kvh * group + min(c, group - 1)) * kD);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) qf[s] = __builtin_bit_cast(h16x8, load_chunk(qp + 4 * s + j));
+    }
+
+    f32x4 o[8];                                    // o[e][r]: channel 32 j + 8 r + e of head c
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = -INFINITY, l = 0.0f;
+
+    for (; key0 < end; key0 += 16 * kStreamWaves) {
+        // scores: lane (head c, j) gets keys key0 + 4 j + r
+        f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, kr[s]), qf[s], sc, 0, 0, 0);
+        h16x8 v4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
+        const int next = key0 + 16 * kStreamWaves;
+        if (next < end) fetch(next);               // the same for the whole wave
+
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sc[r] = key0 + 4 * j + r < end ? sc[r] : -INFINITY;
+            mx = fmaxf(mx, sc[r]);
+        }
+        mx = fmaxf(mx, xor_lanes16(mx));
+        mx = fmaxf(mx, other_half(mx)) * scale_log2;
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        if (__builtin_amdgcn_ballot_w64(m_new > m && m > -INFINITY) != 0) {
+            const float alpha = exp2_fast(m - m_use);
+            l *= alpha;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[e][r] *= alpha;
+        }
+        m = m_new;
+
+        // V^T of the block into the wave's tile: four keys of one channel per 8-byte slot
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
+            *reinterpret_cast<h16x4*>(&vt[e][c][4 * j]) = w;
+        }
+        h16x4 pf;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = exp2_fast(fmaf(sc[r], scale_log2, -m_use));
+            l += p;
+            pf[r] = (h16)p;
+        }
+        // the wave's own LDS traffic only: in order per wave, no workgroup barrier needed
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const h16x4 vf = *reinterpret_cast<const h16x4*>(&vt[e][c][4 * j]);
+            o[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf, o[e], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();                   // the next block overwrites the tile
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // the wave's denominators meet across the four j groups; then the waves
+    l += xor_lanes16(l);
+    l += other_half(l);
+    if (j == 0) {
+        m_lds[wave][c] = m;
+        l_lds[wave][c] = l;
+    }
+    if (c < group) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o_of(wave)[c * kStreamOStride + 32 * j + 8 * r + e] = o[e][r];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < group * kD; idx += kStreamThreads) {
+        const int h = idx >> 7, ch = idx & (kD - 1);
+        float m_all = -INFINITY;
+#pragma unroll 4
+        for (int w = 0; w < kStreamWaves; ++w) m_all = fmaxf(m_all, m_lds[w][h]);
+        float ov = 0.0f, l_all = 0.0f;
+#pragma unroll 4
+        for (int w = 0; w < kStreamWaves; ++w) {
+            const float mw = m_lds[w][h];
+            const float f = mw == -INFINITY ? 0.0f : exp2_fast(mw - m_all);
+            ov = fmaf(o_of(w)[h * kStreamOStride + ch], f, ov);
+            l_all = fmaf(l_lds[w][h], f, l_all);
+        }
+        float* dst = parts + ((size_t)(kvh * group + h) * n_parts + part) * kPartFloats;
+        dst[ch] = ov;
+        if (ch == 0) { dst[kD] = m_all; dst[kD + 1] = l_all; }
+    }
+}
+
 // Folds the slices of one head. The first n_parts threads turn the slices'
 // maxima into weights 2^(m_p - m_all) (kept in LDS) and sum the weighted
 // denominators; then 8 groups of 128 threads take every 8th slice for one
@@ -547,6 +728,13 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge(const float* __res
     const int d = tid % kD, grp = tid / kD;
     const float* src = parts + (size_t)head * n_parts * kPartFloats;
 
+    // The first 64 slices' values are requested before the maxima are exchanged: one trip to memory, not two.
+    float v0[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int p = grp + u * kMergeGroups;
+        v0[u] = p < n_parts ? src[p * kPartFloats + d] : 0.0f;
+    }
     const bool mine = tid < n_parts;
     const float m = mine ? src[tid * kPartFloats + kD] : -INFINITY;
     const float l = mine ? src[tid * kPartFloats + kD + 1] : 0.0f;
@@ -566,7 +754,12 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge(const float* __res
     for (int w = 0; w < kMergeThreads / kWave; ++w) l_all += s_red[1][w];
 
     float o = 0.0f;
-    for (int p0 = grp; p0 < n_parts; p0 += 8 * kMergeGroups) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int p = grp + u * kMergeGroups;
+        if (p < n_parts) o = fmaf(v0[u], s_f[p], o);
+    }
+    for (int p0 = grp + 8 * kMergeGroups; p0 < n_parts; p0 += 8 * kMergeGroups) {
         float v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -893,6 +1086,21 @@ int decode_parts(int cache_len) {
     return n;
 }
 
+// Slices of the streaming decode (FP16 caches): as many workgroups as the chip has compute units
+// (one slice per 64 keys until then), never more slices than the packed formats' kernel would use, so
+// the partial-state buffer of vv_attn_scratch_bytes() holds either.
+int stream_parts(int cache_len, int n_kv_heads) {
+    static const int wgs = [] {
+        const char* e = getenv("VV_DEC_WGS");
+        const int v = e ? atoi(e) : 0;
+        return v > 0 ? v : 256;
+    }();
+    int most = kMinParts;
+    while (most * n_kv_heads < wgs && most < kMaxParts) most *= 2;
+    const int n = decode_parts(cache_len);
+    return n < most ? n : most;
+}
+
 bool fp8_format(int kv_format) { return kv_format == kFmtE4M3 || kv_format == kFmtE5M2; }
 bool tq_format(int kv_format) { return kv_format >= kFmtTq4 && kv_format <= kFmtTq15; }
 bool packed_format(int kv_format) { return fp8_format(kv_format) || tq_format(kv_format); }
@@ -1023,7 +1231,20 @@ vv_status_t attn_decode_launch(const void* q, const vv_kv_view_t* kv, void* out,
     h16* O = static_cast<h16*>(out);
     const KvSource src = {kv->k, kv->v, static_cast<const h16*>(kv->k_meta),
                           static_cast<const h16*>(kv->v_meta), kv->page_table};
-    if (decode_on_matrix_cores(q, kv)) {
+    const int q_group = n_q_heads / kv->n_kv_heads;
+    if (!packed && q_group <= 16 && decode_on_matrix_cores(q, kv)) {
+        if (!parts) return VV_ERR_NULL_PTR;
+        const int n_parts = stream_parts(cache_len, kv->n_kv_heads);
+        const dim3 grid((unsigned)n_parts, (unsigned)kv->n_kv_heads);
+        if (q_group <= 8)
+            decode_stream<8><<<grid, kStreamThreads, 0, st>>>(Q, K, V, kv->page_table, parts, n_q_heads, kv->n_kv_heads,
+                                                             cache_len, d_cache_len, n_parts, scale_log2);
+        else
+            decode_stream<16><<<grid, kStreamThreads, 0, st>>>(Q, K, V, kv->page_table, parts, n_q_heads, kv->n_kv_heads,
+                                                              cache_len, d_cache_len, n_parts, scale_log2);
+        if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
+        decode_merge<<<dim3((unsigned)n_q_heads), kMergeThreads, 0, st>>>(parts, O, n_parts);
+    } else if (decode_on_matrix_cores(q, kv)) {
         const int n_parts = decode_parts(cache_len);
         if (n_parts > 1 && !parts) return VV_ERR_NULL_PTR;
         const int group = n_q_heads / kv->n_kv_heads;
