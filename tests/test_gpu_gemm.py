@@ -47,7 +47,8 @@ def run(fn, d_a, d_b, d_c, M, N, K, alpha=1.0, beta=0.0):
 SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520), (49, 16, 1024), (64, 3584, 3584), (1, 3584, 3584), (3, 512, 3584), (8, 1000, 1536), (9, 64, 64),
           (29, 3584, 3584), (29, 512, 3584), (33, 4608, 1536), (64, 256, 512), (100, 128, 72),
           (285, 3584, 3584), (130, 101, 200), (257, 37, 8), (48, 512, 256), (70, 3584, 18944), (29, 18944, 512),
-          (4100, 8200, 72), (4097, 8192, 64)]     # enough 256x256 workgroups for the eight-wave tile
+          (4100, 8200, 72), (4097, 8192, 64),     # enough 256x256 workgroups for the eight-wave tile
+          (4100, 8200, 192), (4097, 8192, 128), (4100, 8200, 96)]    # ... fed in 128-byte slabs (K % 64 == 0), or in 64-byte ones
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

@@ -135,6 +135,16 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     mfma_dma<F16Op>(A, B, M, N, K * 2, epilogue);
 }
 
+// The same tile fed in slabs of 64 halves (whole cache lines per row; mfma_dma.hpp). Needs K % 64 == 0.
+__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64(
+    const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
+    int K, float alpha, float beta, int vec_store) {
+    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
+        store_tile<4, 2>(acc, C, M, N, m0, n0, frow, fhalf, alpha, beta, vec_store);
+    };
+    mfma_dma64<F16Op>(A, B, M, N, K * 2, epilogue);
+}
+
 // The projection epilogue of a rotary attention layer in the GEMM's store: C = rope(fp16(A W^T) + bias)
 // for heads of 128 columns. The wave's two N tiles are 64 columns apart (kPairN), so register 4g + r of
 // acc[0] and of acc[1] are columns n and n + 64 of one head: the rotate-half pair. Every step rounds where
@@ -210,6 +220,15 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma_rope(
         store_tile_rope<4>(acc, C, bias, table, M, N, m0, n0, frow, fhalf, alpha, beta);
     };
     mfma_dma<F16Op, true>(A, B, M, N, K * 2, epilogue);
+}
+
+__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64_rope(
+    const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
+    const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
+    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
+        store_tile_rope<4>(acc, C, bias, table, M, N, m0, n0, frow, fhalf, alpha, beta);
+    };
+    mfma_dma64<F16Op, true>(A, B, M, N, K * 2, epilogue);
 }
 
 // M == 1: bound by the weight bytes. kSplit waves share an output column (a
@@ -507,22 +526,33 @@ void launch_tile(const void* A, const void* B, void* C, int M, int N, int K, flo
             alpha, beta, vec);
 }
 
-bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
-                hipStream_t st) {
-    // 128 KB of LDS per workgroup is above the default limit: raised once per thread and device.
-    static thread_local int ready_device = -1;
+// 128 KB of LDS per workgroup is above the default limit: raised once per thread, device and kernel.
+template <typename Kernel>
+bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes) {
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return false;
     if (ready_device != device) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)kDmaLdsBytes) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)bytes) != hipSuccess) {
             (void)hipGetLastError();
             return false;
         }
         ready_device = device;
     }
+    return true;
+}
+
+bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+                hipStream_t st) {
+    static thread_local int ready32 = -1, ready64 = -1;
     const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    if (K % (kDma64SlabBytes / 2) == 0) {
+        if (!allow_big_lds(gemm_dma64, ready64, kDma64LdsBytes)) return false;
+        gemm_dma64<<<dim3(dma64_grid(M, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
+            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha, beta, vec);
+        return true;
+    }
+    if (!allow_big_lds(gemm_dma, ready32, kDmaLdsBytes)) return false;
     const dim3 grid((unsigned)((N + kDmaTile - 1) / kDmaTile), (unsigned)((M + kDmaTile - 1) / kDmaTile));
     gemm_dma<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(
         static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha,
@@ -617,18 +647,17 @@ bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table,
         choice = wg256 >= 512 ? k256 : wg128 >= 256 ? k128 : k64;
     }
     if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
-        static thread_local int ready_device = -1;
-        int device = 0;
-        if (hipGetDevice(&device) == hipSuccess &&
-            (ready_device == device ||
-             hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma_rope),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLdsBytes) == hipSuccess)) {
-            ready_device = device;
+        static thread_local int ready32 = -1, ready64 = -1;
+        if (K % (kDma64SlabBytes / 2) == 0 && allow_big_lds(gemm_dma64_rope, ready64, kDma64LdsBytes)) {
+            gemm_dma64_rope<<<dim3(dma64_grid(M, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(A, B, bias, table, C, M, N,
+                                                                                              K, 1.0f, 0.0f);
+            return true;
+        }
+        if (K % (kDma64SlabBytes / 2) != 0 && allow_big_lds(gemm_dma_rope, ready32, kDmaLdsBytes)) {
             const dim3 grid((unsigned)((N + kDmaTile - 1) / kDmaTile), (unsigned)((M + kDmaTile - 1) / kDmaTile));
             gemm_dma_rope<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
             return true;
         }
-        (void)hipGetLastError();
     }
     if (choice == k256 || choice == k256regs) launch_tile_rope<256, 256, 2, 4, 32, 2>(A, B, bias, table, C, M, N, K, st);
     else if (choice == k128) launch_tile_rope<128, 128, 2, 2, 64, 2>(A, B, bias, table, C, M, N, K, st);

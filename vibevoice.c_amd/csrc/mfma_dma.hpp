@@ -159,4 +159,154 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
     epi(acc, m_blk + wm * TM * 32, n_blk + wave_n0, frow, fhalf);
 }
 
+// ── The same tile with slabs of 128 bytes per row (K = 64 halves, 128 int8) ──────────────────
+// What the measurements on MI355X said about the loop above, and what this one does about it:
+//   * A wave issues in order: a block of LDS reads followed by a block of MFMAs leaves the matrix
+//     pipe idle during the first and the LDS idle during the second, and both waves of a SIMD do
+//     the same thing at the same time (they leave the barrier together). Here every LDS read and
+//     every copy request is issued directly behind an MFMA, one per MFMA, in the order in which
+//     the next K step first uses the fragments.
+//   * A copy of 64 bytes per row touches half a 128-byte cache line; the other half is fetched
+//     again for the next slab (the L1 is far too small to keep it). Here a row's whole line comes
+//     in one copy: half the requests to L2, half the barriers per MFMA.
+//   * Workgroups are handed to the eight XCDs in turn, so in launch order the 32 workgroups that
+//     run together on one XCD share one row of tiles and nothing of the other operand. Here the
+//     workgroups of an XCD walk 4 x 8 blocks of tiles (12 operand tiles per 32 instead of 33).
+//   * The clock is not a constant: under this load the device runs at 1.6-1.8 GHz of its 2.4, and
+//     a loop that wastes fewer cycles is answered with a lower clock. What is left to gain is
+//     energy per product, not cycles.
+// Two stages of 64 KB. Fragments are read one K step ahead; the barrier sits before the last K
+// step of a slab, when every wave has read all of the slab (its last step was read during the
+// step before), so the stage is free for the slab after next, whose eight copies per wave are
+// issued behind that step's MFMAs and have a whole slab of MFMAs to land. Rows must be whole
+// slabs: K % 64 == 0 for FP16. The grid is one-dimensional: dma64_grid() workgroups.
+constexpr int kDma64SlabBytes = 128;
+constexpr int kDma64StageSlots = 2 * kDmaTile * (kDma64SlabBytes / 16);      // 4096 slots: A rows, then B rows
+constexpr size_t kDma64LdsBytes = (size_t)2 * kDma64StageSlots * 16;
+constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 workgroups, one per CU of an XCD
+
+inline unsigned dma64_grid(int M, int N) {
+    const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
+    return (unsigned)(((gx + kSuperN - 1) / kSuperN) * ((gy + kSuperM - 1) / kSuperM) * (kSuperM * kSuperN));
+}
+
+template <typename Op, bool kPairN = false, typename Epi>
+__device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
+                                           int row_bytes, const Epi& epi) {
+    typedef typename Op::Acc Acc;
+    constexpr int kSlabChunks = kDma64SlabBytes / 16;     // 8
+    constexpr int WN = 4, TM = 4, TN = 2;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
+    constexpr int kLoads = kDma64StageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 8
+    static_assert(kLoads == 8, "one copy request behind each MFMA of a K step");
+    extern __shared__ u32x4 dma_lds[];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    // Workgroup -> tile: workgroup i runs on XCD i % 8 as its (i / 8)-th; an XCD takes whole blocks of tiles.
+    const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
+    const int blocks_x = (gx + kSuperN - 1) / kSuperN;
+    const int xcd = (int)blockIdx.x & 7, nth = (int)blockIdx.x >> 3;
+    const int seq = ((nth >> 5) * 8 + xcd) * 32 + (nth & 31);
+    const int block = seq >> 5, within = seq & 31;
+    const int block_y = block / blocks_x, block_x = block - block_y * blocks_x;
+    const int tile_m = block_y * kSuperM + (within >> 3), tile_n = block_x * kSuperN + (within & 7);
+    if (tile_m >= gy || tile_n >= gx) return;             // the whole workgroup, before any barrier
+    const int m_blk = tile_m * kDmaTile, n_blk = tile_n * kDmaTile;
+    const int nslabs = row_bytes / kDma64SlabBytes;
+    const uint32_t lds0 =
+        (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
+
+    // Copy i of this wave fills slots (wave + 8i) * 64 .. + 63 of a stage: 8 rows x 8 slots, a whole line per
+    // row. The lane owns (row, physical slot) and fetches the logical slot that the swizzle maps there.
+    const char* src[kLoads];
+    uint32_t dst[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const int slot0 = (wave + kDmaWaves * i) * kWave;
+        const int p = slot0 + lane;
+        const int row = p / kSlabChunks, phys = p % kSlabChunks;
+        const int logical = swz<64>(row, phys);
+        const bool is_b = row >= kDmaTile;
+        const int r = is_b ? row - kDmaTile : row;
+        const char* base = is_b ? static_cast<const char*>(B) + (size_t)min(n_blk + r, N - 1) * row_bytes
+                                : static_cast<const char*>(A) + (size_t)min(m_blk + r, M - 1) * row_bytes;
+        src[i] = base + logical * 16;
+        dst[i] = lds0 + (uint32_t)slot0 * 16u;
+    }
+    auto request = [&](int slab, int i) {        // slab -> stage slab % 2; past the end: the last slab again
+        const size_t adv = (size_t)min(slab, nslabs - 1) * kDma64SlabBytes;
+        const uint32_t stage = (uint32_t)(slab & 1) * (kDma64StageSlots * 16u);
+        lds_dma16(src[i] + adv, dst[i] + stage);
+    };
+
+    Acc acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+
+    const int frow = lane & 31, fhalf = lane >> 5;
+    int f_idx[4];
+#pragma unroll
+    for (int step = 0; step < 4; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 2 + fhalf);
+    const int fa_base = wm * TM * 32 * kSlabChunks;
+    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 32;      // first column of tile a = 0
+    constexpr int kTileStrideN = kPairN ? 64 : 32;
+    const int fb_base = kDmaTile * kSlabChunks + wave_n0 * kSlabChunks;
+
+    u32x4 fw[2][TN], fx[2][TM];                  // [set][tile]: the K step in hand and the next
+    // Fragment i of a step, in the order in which the step's MFMAs first use them: w0, x0, x1, x2, x3, w1.
+    auto read = [&](auto set_c, int slab, int step, int i) {
+        constexpr int set = decltype(set_c)::value;
+        const u32x4* st = dma_lds + (slab & 1) * kDma64StageSlots;
+        if (i == 0) fw[set][0] = st[fb_base + f_idx[step]];
+        else if (i == 5) fw[set][1] = st[fb_base + kTileStrideN * kSlabChunks + f_idx[step]];
+        else fx[set][i - 1] = st[fa_base + (i - 1) * 32 * kSlabChunks + f_idx[step]];
+    };
+    auto k_step = [&](auto cur_c, auto nxt_c, int slab, auto step_c) {
+        constexpr int set = decltype(cur_c)::value;
+        constexpr int step = decltype(step_c)::value;
+        if constexpr (step == 3) {
+            // the next slab has landed (this wave's copies; the barrier adds the others') and every wave has
+            // this slab's last fragments in registers
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        const int nslab = step == 3 ? slab + 1 : slab;
+        constexpr int nstep = (step + 1) & 3;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_barrier(0);
+            acc[i / TM][i % TM] = Op::mfma(fw[set][i / TM], fx[set][i % TM], acc[i / TM][i % TM]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i < 6) read(nxt_c, nslab, nstep, i);
+            if constexpr (step == 3) request(slab + 2, i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) request(0, i);
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) request(1, i);
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // slab 0; slab 1 is waited for at the first barrier
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 6; ++i) read(Const<0>{}, 0, 0, i);
+    for (int slab = 0; slab < nslabs; ++slab) {
+        k_step(Const<0>{}, Const<1>{}, slab, Const<0>{});
+        k_step(Const<1>{}, Const<0>{}, slab, Const<1>{});
+        k_step(Const<0>{}, Const<1>{}, slab, Const<2>{});
+        k_step(Const<1>{}, Const<0>{}, slab, Const<3>{});
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the surplus copies and reads land before the LDS is released
+
+    epi(acc, m_blk + wm * TM * 32, n_blk + wave_n0, frow, fhalf);
+}
+
 }  // namespace vv
