@@ -405,6 +405,244 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
     }
 }
 
+// ── prefill over an FP16 cache, head_dim 128: the same arithmetic as prefill128, pipelined ─────
+// A wave issues in order, so a tile done as "all the score MFMAs, then the softmax, then all the
+// O MFMAs" leaves the matrix pipe idle through the softmax and the vector ALU idle through the
+// MFMAs; measured, the softmax of a tile costs about what its 32 MFMAs cost. Here the loop is
+// skewed by one tile: while the vector ALU turns tile j's scores into probabilities, the matrix
+// pipe computes tile j + 1's scores, a slice of the one issued behind each MFMA of the other; then
+// the O^T += V^T P^T MFMAs of tile j run with tile j + 1's V^T transposition (and the loads of
+// tile j + 2's V) behind them. K goes from global memory straight into LDS (two buffers, two tiles
+// ahead, no registers, no commit); V is transposed on its way in as before, into two buffers, so
+// one barrier per tile remains. V^T rows are 128 bytes: channel 8 d + e sits in row 16 e + d (so
+// the eight rows a thread writes are 16 rows apart and a wave's writes spread over the banks), its
+// 16-byte units XOR-ed with (row / 2) % 8, and the keys inside a row are ordered so that the eight
+// keys a lane multiplies in one step are one unit: 16-byte reads, bank-conflict free. The values
+// and their order of summation are those of prefill128: the same bits.
+// Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
+// alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
+constexpr int kVtRowHalves = 64;                 // one V^T row: 64 keys, 128 bytes, 8 units of 16 bytes
+struct PipeTiles {
+    Chunk k[2][kKeyTile * 16];                   // [buffer][key][16 slots], slot ^ (key & 15)
+    __align__(16) h16 vt[2][kD * kVtRowHalves];  // [buffer][row 16 e + dchunk][unit ^ ((row >> 1) & 7)][8 keys]
+};
+__device__ __forceinline__ void copy16_to_lds(const void* gptr, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_byte_addr), "v"(gptr) : "memory", "m0");
+}
+__global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
+    const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V, const int* __restrict__ page_table,
+    h16* __restrict__ O, int n_q_heads, int n_kv_heads, int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
+    __shared__ PipeTiles tiles;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, half = lane >> 5;
+    const int head = (int)blockIdx.x;
+    const int kvh = head / (n_q_heads / n_kv_heads);
+    const int q0 = (int)(gridDim.y - 1 - blockIdx.y) * kQTile;
+    const int qw0 = q0 + wave * 32;
+    const int qrow = qw0 + col;
+    const int q_abs = q_offset + qrow;
+    int wg_limit = kv_len;
+    if (causal) wg_limit = min(kv_len, q_offset + min(q0 + kQTile, q_len));
+    const int ntiles = (wg_limit + kKeyTile - 1) / kKeyTile;
+    const int last_key = kv_len - 1;
+    const size_t row_halves = (size_t)n_kv_heads * kD;
+    const uint32_t lds_k0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)&tiles.k[0][0]);
+
+    h16x8 qf[kD / 16];
+    load_query(qf, Q + ((size_t)min(qrow, q_len - 1) * n_q_heads + head) * kD, half);
+    RowState st;
+    st.reset();
+
+    // K tile j -> buffer j & 1, straight into LDS: copy c of this wave fills slots 64 (4 wave + c) .. + 63:
+    // keys 4 (4 wave + c) .. + 3, the lane owning (key, physical slot) and fetching the logical slot.
+    auto request_k = [&](int j) {
+        const int t0 = j * kKeyTile;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
+            const int row = cache_row(page_table, min(t0 + key, last_key));
+            const Chunk* g = reinterpret_cast<const Chunk*>(K + (size_t)row * row_halves + (size_t)kvh * kD) + (phys ^ (key & 15));
+            copy16_to_lds(g, lds_k0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave + c) * 1024u);
+        }
+    };
+    // V tile: a thread takes four consecutive keys 4 kg .. + 3 of one 8-channel chunk.
+    const int dchunk = tid & 15, kg = tid >> 4;
+    Chunk vr[4];
+    auto fetch_v = [&](int j) {
+        const int t0 = j * kKeyTile;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = cache_row(page_table, min(t0 + 4 * kg + i, last_key));
+            vr[i] = load_chunk(reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + dchunk);
+        }
+    };
+    // key 32 a + 16 sp + 8 x + 4 h + i sits at position 32 a + 16 sp + 8 h + 4 x + i of its row, so that the eight
+    // keys a lane multiplies in one step are one 16-byte unit; kg = 8 a + 4 sp + 2 x + h
+    const int v_unit = (kg >> 2) * 2 + (kg & 1), v_sub = (kg >> 1) & 1;     // unit 2 (2a + sp) + h, half-unit x
+    auto commit_v = [&](int j) {
+        h16x8 v4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int row = 16 * e + dchunk;
+            const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
+            *reinterpret_cast<h16x4*>(&tiles.vt[j & 1][row * kVtRowHalves + ((v_unit ^ ((row >> 1) & 7)) * 8) + 4 * v_sub]) = w;
+        }
+    };
+    auto scores = [&](int j, f32x16 (&s)[2]) {
+        const Chunk* kb = tiles.k[j & 1];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[a][r] = 0.0f;
+#pragma unroll
+            for (int s8 = 0; s8 < kD / 16; ++s8) {
+                const int row = 32 * a + col, slot = 2 * s8 + half;
+                const h16x8 kf = __builtin_bit_cast(h16x8, kb[row * 16 + (slot ^ (row & 15))]);
+                s[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s8], s[a], 0, 0, 0);
+            }
+        }
+    };
+
+    if (ntiles > 0) {
+        request_k(0);
+        request_k(1);
+        fetch_v(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        commit_v(0);
+        fetch_v(1);
+    }
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");          // K 0 and K 1 landed; V 1 may fly
+    __syncthreads();
+    f32x16 s_cur[2];
+    if (ntiles > 0) scores(0, s_cur);
+    __syncthreads();                                          // K 0 is read: its buffer may take K 2
+
+    for (int j = 0; j < ntiles; ++j) {
+        const int t0 = j * kKeyTile;
+        if (t0 + kKeyTile > kv_len || (causal && t0 + kKeyTile - 1 > q_offset + qw0)) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const bool seen = key < kv_len && (!causal || key <= q_abs);
+                    s_cur[a][r] = seen ? s_cur[a][r] : -INFINITY;
+                }
+        }
+        // block 1: the next tile's scores on the matrix pipe, this tile's softmax on the vector ALU, a slice of
+        // the one behind each MFMA of the other
+        f32x16 s_next[2];
+        request_k(j + 2);                                     // into the buffer tile j's K has left
+        const Chunk* kb = tiles.k[(j + 1) & 1];
+        auto k_frag = [&](int k) {                            // step k = 8 a + s8
+            const int row = 32 * (k >> 3) + col, slot = 2 * (k & 7) + half;
+            return __builtin_bit_cast(h16x8, kb[row * 16 + (slot ^ (row & 15))]);
+        };
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_next[a][r] = 0.0f;
+        h16x8 kf[3];
+        kf[0] = k_frag(0);
+        kf[1] = k_frag(1);
+        float mx = -INFINITY, m_new = 0.0f, m_use = 0.0f, sum = 0.0f;
+        h16x8 pf[4];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (k + 2 < 16) kf[(k + 2) % 3] = k_frag(k + 2);
+            s_next[k >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[k % 3], qf[k & 7], s_next[k >> 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (k < 4) {
+#pragma unroll
+                for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_cur[q >> 4][q & 15]);
+                if (k == 3) {
+                    mx = fmaxf(mx, other_half(mx)) * scale_log2;
+                    m_new = fmaxf(st.m, mx);
+                    m_use = m_new == -INFINITY ? 0.0f : m_new;
+                }
+            } else {
+#pragma unroll
+                for (int q = (k - 4) * 32 / 12; q < (k - 3) * 32 / 12; ++q) {
+                    const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -m_use));
+                    sum += p;
+                    pf[q >> 3][q & 7] = (h16)p;
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        sum += other_half(sum);
+        if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
+            const float alpha = exp2_fast(st.m - m_use);
+            st.l *= alpha;
+#pragma unroll
+            for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+        }
+        st.l += sum;
+        st.m = m_new;
+        // block 2: O^T += V^T P^T on the matrix pipe; behind its MFMAs the next tile's V^T goes into its buffer
+        // and the tile after that is asked for
+        const h16* vb = tiles.vt[j & 1];
+        auto v_frag = [&](int k) {                            // step k = 4 u + t
+            const int row = 32 * (k & 3) + col;
+            return *reinterpret_cast<const h16x8*>(&vb[row * kVtRowHalves + (((2 * (k >> 2) + half) ^ ((row >> 1) & 7)) * 8)]);
+        };
+        h16x8 vf[3];
+        vf[0] = v_frag(0);
+        vf[1] = v_frag(1);
+        h16x8 v4[4];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (k + 2 < 16) vf[(k + 2) % 3] = v_frag(k + 2);
+            st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (k == 3) {
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");      // V j+1 in registers (the four K copies just issued may fly)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
+            }
+            if (k >= 4 && k < 12) {
+                const int e = k - 4, row = 16 * e + dchunk;
+                const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
+                *reinterpret_cast<h16x4*>(&tiles.vt[(j + 1) & 1][row * kVtRowHalves + ((v_unit ^ ((row >> 1) & 7)) * 8) + 4 * v_sub]) = w;
+            }
+            if (k >= 12) {
+                const int i = k - 12;
+                const int row = cache_row(page_table, min((j + 2) * kKeyTile + 4 * kg + i, last_key));
+                vr[i] = load_chunk(reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + dchunk);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");      // K j+2 landed (V j+2 may fly)
+        __syncthreads();
+#pragma unroll
+        for (int a = 0; a < 2; ++a) s_cur[a] = s_next[a];
+    }
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no copy may land after the workgroup has gone
+    if (qrow < q_len) {
+        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+        h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
+        // register 4 g + r of tile t is LDS row 32 t + 8 g + 4 half + r = 16 e + dchunk: channel 8 dchunk + e
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = 32 * t + 8 * g + 4 * half + r;
+                    op[8 * (row & 15) + (row >> 4)] = to_half(st.o[t][4 * g + r] * inv);
+                }
+    }
+}
+
+
 // ── any head_dim <= 256: one wave per (query row, head) ──────────────────
 __global__ __launch_bounds__(kWave) void rows_generic(
     const h16* Q, const h16* Kc, const h16* Vc, const int* page_table, h16* O, int n_q_heads,
@@ -1199,9 +1437,9 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
 #undef VV_PREFILL
     } else if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
                vv::aligned16(out)) {
-        const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
-        vv::prefill128<vv::kFmtFp16><<<grid, vv::kBlock, 0, st>>>(Q, src, O, n_q_heads, kv->n_kv_heads, q_len,
-                                                                  q_offset, kv_len, causal ? 1 : 0, scale_log2);
+        const dim3 grid((unsigned)n_q_heads, (unsigned)((q_len + vv::kQTile - 1) / vv::kQTile));
+        vv::prefill_pipe<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads, kv->n_kv_heads, q_len,
+                                                      q_offset, kv_len, causal ? 1 : 0, scale_log2);
     } else {
         const dim3 grid((unsigned)q_len, (unsigned)n_q_heads);
         vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,

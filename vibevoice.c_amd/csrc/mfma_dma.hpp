@@ -187,7 +187,9 @@ constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 wor
 
 inline unsigned dma64_grid(int M, int N) {
     const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
-    return (unsigned)(((gx + kSuperN - 1) / kSuperN) * ((gy + kSuperM - 1) / kSuperM) * (kSuperM * kSuperN));
+    // workgroup i runs block 8 (i / 256) + i % 8: whole groups of eight blocks, or the last ones stay half done
+    const int blocks = ((gx + kSuperN - 1) / kSuperN) * ((gy + kSuperM - 1) / kSuperM);
+    return (unsigned)((blocks + 7) / 8 * 8 * (kSuperM * kSuperN));
 }
 
 template <typename Op, bool kPairN = false, typename Epi>
