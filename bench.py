@@ -339,7 +339,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0        # MI355X dense FP16 matrix rate
 MFMA_I8_PEAK_TOPS = 5000.0           # and the dense int8 one
 
 
-def layer_leg(torch, dev, T: int, st: int) -> dict:
+def layer_leg(torch, dev, T: int, st: int, fp16_only: bool = False) -> dict:
     """The rest of a dense Qwen2-7B layer at the same prompt length: the four projection shapes of
     the FP16 GEMM and causal GQA attention at M = T (matrix-core bound: TFLOP/s against the dense
     FP16 peak), and the decode forms (one row: bound by the weight / cache bytes, GB/s). Not part of
@@ -380,121 +380,122 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del a, c
         del w
-    # The same four projections as W8A8 (int8 x int8 on the matrix cores, per-row / per-channel scales).
-    out["w8a8"], out["w8a8_gemv"] = {}, {}
-    for name, n, k in shapes:
-        w8 = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
-        sw = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
-        for m, key in ((T, "w8a8"), (1, "w8a8_gemv")):
-            xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
-            sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
-            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-            sec = timed(lambda: dev.vv_w8a8_linear_dev(xq.data_ptr(), sx.data_ptr(), w8.data_ptr(), sw.data_ptr(),
-                                                       None, None, c.data_ptr(), 0, m, n, k, 0, st),
-                        5 if m > 1 else 50)
-            if m > 1:
-                tops = 2.0 * m * n * k / sec / 1e12
-                out[key][name] = {"M": m, "N": n, "K": k, "us": sec * 1e6, "TOPs": tops,
-                                  "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
-            else:
-                gb = (n * k + k + 6.0 * n) / sec / 1e9
-                out[key][name] = {"N": n, "K": k, "us": sec * 1e6, "GBps": gb,
-                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
-            del xq, sx, c
-        del w8, sw
-    # And as W4A8: 4-bit codes with a scale and a zero point per 128 columns (any bytes are valid codes).
-    out["w4a8"], out["w4a8_gemv"], out["w4a8_chunk"] = {}, {}, {}
-    G = 128
-    for name, n, k in shapes:
-        w4 = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
-        sz = torch.stack([torch.rand(n, k // G, device="cuda") * 0.02 + 0.002,
-                          torch.randint(0, 16, (n, k // G), device="cuda").float()], dim=-1).half().contiguous()
-        # T rows (prefill), one row (decode) and 29 rows (a streaming chunk: the weights are still the bytes)
-        for m, key, layout in ((T, "w4a8", 3), (1, "w4a8_gemv", 2), (29, "w4a8_chunk", 3)):
-            xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
-            sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
-            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-            xs = xq.view(m, k // 32, 32).sum(-1, dtype=torch.int32).contiguous()     # what the quantiser writes
-            sec = timed(lambda: dev.vv_w4a8_linear_dev(xq.data_ptr(), layout, sx.data_ptr(), xs.data_ptr(), w4.data_ptr(),
-                                                       sz.data_ptr(), G, None, None, c.data_ptr(), 0, m, n, k, 0,
-                                                       st), 5 if m > 64 else 50)
-            if m > 64:
-                tops = 2.0 * m * n * k / sec / 1e12
-                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TOPs": tops,
-                                  "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
-            else:
-                gb = (n * k / 2 + n * (k // G) * 4 + m * (k + 2.0 * n)) / sec / 1e9
-                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
-                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
-            del xq, sx, c
-        # the same codes against FP16 activations (W4A16)
-        for m, key in ((T, "w4a16"), (1, "w4a16_gemv"), (29, "w4a16_chunk")):
-            out.setdefault(key, {})
-            a = torch.randn(m, k, dtype=torch.float16, device="cuda")
-            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-            dense = torch.empty(n * k, dtype=torch.float16, device="cuda")     # the decoder's dequant scratch
-            sec = timed(lambda: dev.vv_w4a16_gemm_dev(a.data_ptr(), w4.data_ptr(), sz.data_ptr(), None, c.data_ptr(),
-                                                      dense.data_ptr(), n * k * 2, m, n, k, G, st),
-                        5 if m > 64 else 50)
-            if m > 64:
-                tf = 2.0 * m * n * k / sec / 1e12
-                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TFLOPs": tf,
-                                  "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
-            else:
-                gb = (n * k / 2 + n * (k // G) * 4 + m * (2.0 * k + 2.0 * n)) / sec / 1e9
-                out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
-                                  "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
-            del a, c, dense
-        del w4, sz
-    # The older weight-only formats on FP16 activations: one row (decode), 29 rows (a streaming
-    # chunk, the small-M kernel where it serves) and the dequantiser that feeds the FP16 GEMM.
-    out["weight_only"] = {}
-    for fmt in ("int8", "nf4", "int4"):
+    if not fp16_only:
+        # The same four projections as W8A8 (int8 x int8 on the matrix cores, per-row / per-channel scales).
+        out["w8a8"], out["w8a8_gemv"] = {}, {}
         for name, n, k in shapes:
-            if fmt == "int8":
-                wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
-                sc = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
-                mn, wbytes = None, n * k + 4.0 * n
-            else:
-                wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
-                per = 64 if fmt == "nf4" else G
-                sc = (torch.rand(n * k // per, device="cuda") * 0.02 + 0.002).half()
-                mn = (-torch.rand(n * k // per, device="cuda") * 0.1).half() if fmt == "int4" else None
-                wbytes = n * k / 2 + (2.0 if fmt == "nf4" else 4.0) * n * k / per
-            dense = torch.empty(n * k, dtype=torch.float16, device="cuda")
-            P = lambda t: t.data_ptr() if t is not None else None
-
-            def run(m, a, c):
-                if fmt == "int8":
-                    return dev.vv_int8_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, st)
-                if fmt == "nf4":
-                    return dev.vv_nf4_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, 64, st)
-                return dev.vv_awq_gemm_dev(P(a), P(wq), P(mn), P(sc), P(c), P(dense), m, n, k, G, st)
-
-            def run_dequant():
-                if fmt == "int8":
-                    return dev.vv_dequant_int8_dev(P(wq), P(sc), P(dense), n, k, st)
-                if fmt == "nf4":
-                    return dev.vv_dequant_nf4_dev(P(wq), P(sc), P(dense), n * k, 64, st)
-                return dev.vv_dequant_awq_dev(P(wq), P(mn), P(sc), P(dense), n, k, G, st)
-
-            d = {"N": n, "K": k}
-            for m in (1, 29):
+            w8 = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+            sw = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
+            for m, key in ((T, "w8a8"), (1, "w8a8_gemv")):
+                xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+                sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
+                c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                sec = timed(lambda: dev.vv_w8a8_linear_dev(xq.data_ptr(), sx.data_ptr(), w8.data_ptr(), sw.data_ptr(),
+                                                           None, None, c.data_ptr(), 0, m, n, k, 0, st),
+                            5 if m > 1 else 50)
+                if m > 1:
+                    tops = 2.0 * m * n * k / sec / 1e12
+                    out[key][name] = {"M": m, "N": n, "K": k, "us": sec * 1e6, "TOPs": tops,
+                                      "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
+                else:
+                    gb = (n * k + k + 6.0 * n) / sec / 1e9
+                    out[key][name] = {"N": n, "K": k, "us": sec * 1e6, "GBps": gb,
+                                      "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+                del xq, sx, c
+            del w8, sw
+        # And as W4A8: 4-bit codes with a scale and a zero point per 128 columns (any bytes are valid codes).
+        out["w4a8"], out["w4a8_gemv"], out["w4a8_chunk"] = {}, {}, {}
+        G = 128
+        for name, n, k in shapes:
+            w4 = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
+            sz = torch.stack([torch.rand(n, k // G, device="cuda") * 0.02 + 0.002,
+                              torch.randint(0, 16, (n, k // G), device="cuda").float()], dim=-1).half().contiguous()
+            # T rows (prefill), one row (decode) and 29 rows (a streaming chunk: the weights are still the bytes)
+            for m, key, layout in ((T, "w4a8", 3), (1, "w4a8_gemv", 2), (29, "w4a8_chunk", 3)):
+                xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+                sx = torch.rand(m, dtype=torch.float32, device="cuda") * 1e-2
+                c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                xs = xq.view(m, k // 32, 32).sum(-1, dtype=torch.int32).contiguous()     # what the quantiser writes
+                sec = timed(lambda: dev.vv_w4a8_linear_dev(xq.data_ptr(), layout, sx.data_ptr(), xs.data_ptr(), w4.data_ptr(),
+                                                           sz.data_ptr(), G, None, None, c.data_ptr(), 0, m, n, k, 0,
+                                                           st), 5 if m > 64 else 50)
+                if m > 64:
+                    tops = 2.0 * m * n * k / sec / 1e12
+                    out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TOPs": tops,
+                                      "frac_of_mfma_peak": tops / MFMA_I8_PEAK_TOPS}
+                else:
+                    gb = (n * k / 2 + n * (k // G) * 4 + m * (k + 2.0 * n)) / sec / 1e9
+                    out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                                      "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+                del xq, sx, c
+            # the same codes against FP16 activations (W4A16)
+            for m, key in ((T, "w4a16"), (1, "w4a16_gemv"), (29, "w4a16_chunk")):
+                out.setdefault(key, {})
                 a = torch.randn(m, k, dtype=torch.float16, device="cuda")
                 c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-                assert run(m, a, c) == 0
-                sec = timed(lambda: run(m, a, c), 50)
-                d[f"M{m}_us"] = sec * 1e6
-                if m == 1:
-                    d["M1_GBps"] = (wbytes + 2.0 * k + 2.0 * n) / sec / 1e9
-                    d["M1_frac_of_hbm_peak"] = d["M1_GBps"] / HBM_PEAK_GBPS
-                del a, c
-            assert run_dequant() == 0
-            sec = timed(run_dequant, 20)
-            d["dequant_us"] = sec * 1e6
-            d["dequant_GBps"] = (wbytes + 2.0 * n * k) / sec / 1e9
-            out["weight_only"][f"{fmt} {name}"] = d
-            del wq, sc, mn, dense
+                dense = torch.empty(n * k, dtype=torch.float16, device="cuda")     # the decoder's dequant scratch
+                sec = timed(lambda: dev.vv_w4a16_gemm_dev(a.data_ptr(), w4.data_ptr(), sz.data_ptr(), None, c.data_ptr(),
+                                                          dense.data_ptr(), n * k * 2, m, n, k, G, st),
+                            5 if m > 64 else 50)
+                if m > 64:
+                    tf = 2.0 * m * n * k / sec / 1e12
+                    out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "TFLOPs": tf,
+                                      "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+                else:
+                    gb = (n * k / 2 + n * (k // G) * 4 + m * (2.0 * k + 2.0 * n)) / sec / 1e9
+                    out[key][name] = {"M": m, "N": n, "K": k, "group": G, "us": sec * 1e6, "GBps": gb,
+                                      "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+                del a, c, dense
+            del w4, sz
+        # The older weight-only formats on FP16 activations: one row (decode), 29 rows (a streaming
+        # chunk, the small-M kernel where it serves) and the dequantiser that feeds the FP16 GEMM.
+        out["weight_only"] = {}
+        for fmt in ("int8", "nf4", "int4"):
+            for name, n, k in shapes:
+                if fmt == "int8":
+                    wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+                    sc = torch.rand(n, dtype=torch.float32, device="cuda") * 1e-2
+                    mn, wbytes = None, n * k + 4.0 * n
+                else:
+                    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device="cuda")
+                    per = 64 if fmt == "nf4" else G
+                    sc = (torch.rand(n * k // per, device="cuda") * 0.02 + 0.002).half()
+                    mn = (-torch.rand(n * k // per, device="cuda") * 0.1).half() if fmt == "int4" else None
+                    wbytes = n * k / 2 + (2.0 if fmt == "nf4" else 4.0) * n * k / per
+                dense = torch.empty(n * k, dtype=torch.float16, device="cuda")
+                P = lambda t: t.data_ptr() if t is not None else None
+
+                def run(m, a, c):
+                    if fmt == "int8":
+                        return dev.vv_int8_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, st)
+                    if fmt == "nf4":
+                        return dev.vv_nf4_gemm_dev(P(a), P(wq), P(sc), P(c), P(dense), m, n, k, 64, st)
+                    return dev.vv_awq_gemm_dev(P(a), P(wq), P(mn), P(sc), P(c), P(dense), m, n, k, G, st)
+
+                def run_dequant():
+                    if fmt == "int8":
+                        return dev.vv_dequant_int8_dev(P(wq), P(sc), P(dense), n, k, st)
+                    if fmt == "nf4":
+                        return dev.vv_dequant_nf4_dev(P(wq), P(sc), P(dense), n * k, 64, st)
+                    return dev.vv_dequant_awq_dev(P(wq), P(mn), P(sc), P(dense), n, k, G, st)
+
+                d = {"N": n, "K": k}
+                for m in (1, 29):
+                    a = torch.randn(m, k, dtype=torch.float16, device="cuda")
+                    c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                    assert run(m, a, c) == 0
+                    sec = timed(lambda: run(m, a, c), 50)
+                    d[f"M{m}_us"] = sec * 1e6
+                    if m == 1:
+                        d["M1_GBps"] = (wbytes + 2.0 * k + 2.0 * n) / sec / 1e9
+                        d["M1_frac_of_hbm_peak"] = d["M1_GBps"] / HBM_PEAK_GBPS
+                    del a, c
+                assert run_dequant() == 0
+                sec = timed(run_dequant, 20)
+                d["dequant_us"] = sec * 1e6
+                d["dequant_GBps"] = (wbytes + 2.0 * n * k) / sec / 1e9
+                out["weight_only"][f"{fmt} {name}"] = d
+                del wq, sc, mn, dense
     q = torch.randn(T, NQ, HD, dtype=torch.float16, device="cuda")
     k_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
     v_ = torch.randn(T, NK, HD, dtype=torch.float16, device="cuda")
@@ -550,63 +551,66 @@ def layer_leg(torch, dev, T: int, st: int) -> dict:
                           "note": "two launches per call (slices, then their merge); about 8 us of it is launch and "
                                   "memory latency, the same at 1000 positions"}
     del caches, views
-    # The same two over an FP8 (E4M3) cache: half the cache bytes, widened on their way into the tile.
-    k8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
-    v8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
-    view8 = dev.KvView(k=k8.data_ptr(), v=v8.data_ptr(), k_meta=None, v_meta=None, page_table=None,
-                       format=1, n_kv_heads=NK, head_dim=HD)
-    sec = timed(lambda: dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, 0, T,
-                                            True, None, st), 3)
-    tf = 4.0 * NQ * HD * T * (T + 1) / 2 / sec / 1e12
-    out["attn_prefill_fp8"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf, "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
-    sec = timed(lambda: dev.vv_attn_decode(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, None,
-                                           scratch.data_ptr(), st), 50)
-    gb = 2.0 * T * NK * HD / sec / 1e9
-    out["attn_decode_fp8"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
-    del q, k_, v_, o, k8, v8
-    # BitNet's integer layers at the 1.5B shape (hidden 1536, FFN 8960, vocabulary 151936): quantise, one decode row
-    # and a 512-row prefill through the ternary gate projection.
-    Hb, Fb, Vb, Mb = 1536, 8960, 151936, 512
-    bn = {}
-    xb = torch.randn(Mb, Hb, dtype=torch.float16, device="cuda")
-    qb = torch.empty(Mb, Hb, dtype=torch.int8, device="cuda")
-    sb = torch.empty(Mb, dtype=torch.float32, device="cuda")
-    smb = torch.empty(Mb, dtype=torch.int32, device="cuda")
-    sec = timed(lambda: dev.vv_act_quant_i8_dev(xb.data_ptr(), 1, Mb, Hb, qb.data_ptr(), sb.data_ptr(), smb.data_ptr(), st), 50)
-    bn["act_quant_512x1536_us"] = sec * 1e6
-    codes = torch.randint(0, 3, (Fb, Hb // 4, 4), dtype=torch.uint8, device="cuda")
-    codes = (codes[..., 0] << 6 | codes[..., 1] << 4 | codes[..., 2] << 2 | codes[..., 3]).contiguous()
-    yb = torch.empty(Mb, Fb, dtype=torch.float16, device="cuda")
-    for m in (1, Mb):
-        sec = timed(lambda: dev.vv_ternary_gemm_dev(qb.data_ptr(), smb.data_ptr(), sb.data_ptr(), codes.data_ptr(), 0.02,
-                                                    None, None, yb.data_ptr(), 1, m, Fb, Hb, st), 50)
-        bn[f"ternary_{Fb}x{Hb}_M{m}_us"] = sec * 1e6
-    # (the int8 tied head is not built in this backend: no leg)
-    out["bitnet"] = bn
-    del xb, qb, sb, smb, codes, yb
-    # Conv-VAE encoder ops at a deep stage's shape: 512 channels, 24000 packed columns in one item.
-    Cv, Tv, kv = 512, 24000, 7
-    d = dev.VaeConvDesc()
-    d.n, d.cap = 1, kv - 1
-    d.it[0].in_len = d.it[0].out_len = Tv
-    xv = torch.randn(Cv, Tv, dtype=torch.float16, device="cuda")
-    xo = torch.empty_like(xv)
-    rv = torch.empty(Tv, dtype=torch.float32, device="cuda")
-    nwv = torch.randn(Cv, dtype=torch.float16, device="cuda")
-    cwv = torch.randn(Cv, kv, dtype=torch.float16, device="cuda") * 0.3
-    vae = {}
-    rv.copy_(torch.rsqrt(xv.float().pow(2).mean(0) + 1e-5))     # the per-column 1/rms op is not built in this backend
-    sec = timed(lambda: dev.vv_vae_mixer_dev(C.addressof(d), xv.data_ptr(), xo.data_ptr(), Tv, rv.data_ptr(), Tv,
-                                             nwv.data_ptr(), cwv.data_ptr(), None, nwv.data_ptr(), Cv, kv, st), 50)
-    vae["mixer_us"] = sec * 1e6
-    vae["mixer_GBps"] = 4.0 * Cv * Tv / sec / 1e9
-    w1 = torch.randn(4 * Cv, Cv, dtype=torch.float16, device="cuda") * Cv ** -0.5
-    hv = torch.empty(4 * Cv, Tv, dtype=torch.float16, device="cuda")
-    sec = timed(lambda: dev.vv_vae_gemm_nn_dev(0, w1.data_ptr(), xv.data_ptr(), Tv, hv.data_ptr(), Tv, 4 * Cv, Cv, Tv,
-                                               None, None, rv.data_ptr(), nwv.data_ptr(), 0, st), 20)
-    vae["ffn_up_gelu_us"] = sec * 1e6
-    vae["ffn_up_gelu_TFLOPs"] = 2.0 * 4 * Cv * Cv * Tv / sec / 1e12
-    out["vae"] = vae
+    if not fp16_only:
+        # The same two over an FP8 (E4M3) cache: half the cache bytes, widened on their way into the tile.
+        k8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
+        v8 = torch.randint(0, 0x78, (T, NK, HD), dtype=torch.uint8, device="cuda")
+        view8 = dev.KvView(k=k8.data_ptr(), v=v8.data_ptr(), k_meta=None, v_meta=None, page_table=None,
+                           format=1, n_kv_heads=NK, head_dim=HD)
+        sec = timed(lambda: dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, 0, T,
+                                                True, None, st), 3)
+        tf = 4.0 * NQ * HD * T * (T + 1) / 2 / sec / 1e12
+        out["attn_prefill_fp8"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf, "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+        sec = timed(lambda: dev.vv_attn_decode(2, q.data_ptr(), C.addressof(view8), o.data_ptr(), NQ, T, None,
+                                               scratch.data_ptr(), st), 50)
+        gb = 2.0 * T * NK * HD / sec / 1e9
+        out["attn_decode_fp8"] = {"cache_len": T, "us": sec * 1e6, "GBps": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
+        del k8, v8
+    del q, k_, v_, o
+    if not fp16_only:
+        # BitNet's integer layers at the 1.5B shape (hidden 1536, FFN 8960, vocabulary 151936): quantise, one decode row
+        # and a 512-row prefill through the ternary gate projection.
+        Hb, Fb, Vb, Mb = 1536, 8960, 151936, 512
+        bn = {}
+        xb = torch.randn(Mb, Hb, dtype=torch.float16, device="cuda")
+        qb = torch.empty(Mb, Hb, dtype=torch.int8, device="cuda")
+        sb = torch.empty(Mb, dtype=torch.float32, device="cuda")
+        smb = torch.empty(Mb, dtype=torch.int32, device="cuda")
+        sec = timed(lambda: dev.vv_act_quant_i8_dev(xb.data_ptr(), 1, Mb, Hb, qb.data_ptr(), sb.data_ptr(), smb.data_ptr(), st), 50)
+        bn["act_quant_512x1536_us"] = sec * 1e6
+        codes = torch.randint(0, 3, (Fb, Hb // 4, 4), dtype=torch.uint8, device="cuda")
+        codes = (codes[..., 0] << 6 | codes[..., 1] << 4 | codes[..., 2] << 2 | codes[..., 3]).contiguous()
+        yb = torch.empty(Mb, Fb, dtype=torch.float16, device="cuda")
+        for m in (1, Mb):
+            sec = timed(lambda: dev.vv_ternary_gemm_dev(qb.data_ptr(), smb.data_ptr(), sb.data_ptr(), codes.data_ptr(), 0.02,
+                                                        None, None, yb.data_ptr(), 1, m, Fb, Hb, st), 50)
+            bn[f"ternary_{Fb}x{Hb}_M{m}_us"] = sec * 1e6
+        # (the int8 tied head is not built in this backend: no leg)
+        out["bitnet"] = bn
+        del xb, qb, sb, smb, codes, yb
+        # Conv-VAE encoder ops at a deep stage's shape: 512 channels, 24000 packed columns in one item.
+        Cv, Tv, kv = 512, 24000, 7
+        d = dev.VaeConvDesc()
+        d.n, d.cap = 1, kv - 1
+        d.it[0].in_len = d.it[0].out_len = Tv
+        xv = torch.randn(Cv, Tv, dtype=torch.float16, device="cuda")
+        xo = torch.empty_like(xv)
+        rv = torch.empty(Tv, dtype=torch.float32, device="cuda")
+        nwv = torch.randn(Cv, dtype=torch.float16, device="cuda")
+        cwv = torch.randn(Cv, kv, dtype=torch.float16, device="cuda") * 0.3
+        vae = {}
+        rv.copy_(torch.rsqrt(xv.float().pow(2).mean(0) + 1e-5))     # the per-column 1/rms op is not built in this backend
+        sec = timed(lambda: dev.vv_vae_mixer_dev(C.addressof(d), xv.data_ptr(), xo.data_ptr(), Tv, rv.data_ptr(), Tv,
+                                                 nwv.data_ptr(), cwv.data_ptr(), None, nwv.data_ptr(), Cv, kv, st), 50)
+        vae["mixer_us"] = sec * 1e6
+        vae["mixer_GBps"] = 4.0 * Cv * Tv / sec / 1e9
+        w1 = torch.randn(4 * Cv, Cv, dtype=torch.float16, device="cuda") * Cv ** -0.5
+        hv = torch.empty(4 * Cv, Tv, dtype=torch.float16, device="cuda")
+        sec = timed(lambda: dev.vv_vae_gemm_nn_dev(0, w1.data_ptr(), xv.data_ptr(), Tv, hv.data_ptr(), Tv, 4 * Cv, Cv, Tv,
+                                                   None, None, rv.data_ptr(), nwv.data_ptr(), 0, st), 20)
+        vae["ffn_up_gelu_us"] = sec * 1e6
+        vae["ffn_up_gelu_TFLOPs"] = 2.0 * 4 * Cv * Cv * Tv / sec / 1e12
+        out["vae"] = vae
     return out
 
 
@@ -1156,6 +1160,11 @@ def main() -> int:
     ap.add_argument("--layer", action="store_true",
                     help="also time the dense GEMM and attention entry points at the layer's shapes "
                          "(reported under 'layer'; not part of the step)")
+    ap.add_argument("--layer-fp16", action="store_true",
+                    help="like --layer, but only the FP16 GEMM and attention legs and the whole-layer / whole-token "
+                         "figures built on them (no quantised, BitNet or Conv-VAE legs): short enough to profile")
+    ap.add_argument("--no-token", action="store_true",
+                    help="with --layer / --layer-fp16: skip the whole-token decode legs (thousands of small launches)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
                          "five times: the known-size reference for rocprofv3 byte counters")
@@ -1231,29 +1240,30 @@ def main() -> int:
                 f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (not part of the step)")
 
     layer = {}
-    if args.layer:
-        layer = layer_leg(torch, dev, T, st)
+    if args.layer or args.layer_fp16:
+        fp16_only = not args.layer
+        layer = layer_leg(torch, dev, T, st, fp16_only)
         for name, d in layer["gemm"].items():
             log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         for name, d in layer["gemv"].items():
             log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for kind in ("w8a8", "w4a8"):
+        for kind in () if fp16_only else ("w8a8", "w4a8"):
             for name, d in layer[kind].items():
                 log(f"  {kind} {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TOPs']:7.1f} TOP/s "
                     f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
             for name, d in layer[kind + "_gemv"].items():
                 log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer["w4a8_chunk"].items():
+        for name, d in layer.get("w4a8_chunk", {}).items():
             log(f"  w4a8 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer["w4a16"].items():
+        for name, d in layer.get("w4a16", {}).items():
             log(f"  w4a16 {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
-        for name, d in layer["w4a16_gemv"].items():
+        for name, d in layer.get("w4a16_gemv", {}).items():
             log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer["w4a16_chunk"].items():
+        for name, d in layer.get("w4a16_chunk", {}).items():
             log(f"  w4a16 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer["weight_only"].items():
+        for name, d in layer.get("weight_only", {}).items():
             log(f"  weight-only {name:18s} N={d['N']} K={d['K']}: one row {d['M1_us']:7.2f} us {d['M1_GBps']:7.1f} GB/s, "
                 f"29 rows {d['M29_us']:7.2f} us, dequantise {d['dequant_us']:7.2f} us {d['dequant_GBps']:7.1f} GB/s")
         d = layer["attn_prefill"]
@@ -1262,32 +1272,35 @@ def main() -> int:
         d = layer["attn_decode"]
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s "
             f"(replayed from a graph: {d['graph_us']:.2f} us {d['graph_GBps']:.1f} GB/s)")
-        d = layer["attn_prefill_fp8"]
-        log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
-        d = layer["attn_decode_fp8"]
-        log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        d = layer["bitnet"]
-        log("  BitNet (1536 / 8960 / 151936): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
-        d = layer["vae"]
-        log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
+        if not fp16_only:
+            d = layer["attn_prefill_fp8"]
+            log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
+            d = layer["attn_decode_fp8"]
+            log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+            d = layer["bitnet"]
+            log("  BitNet (1536 / 8960 / 151936): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
+            d = layer["vae"]
+            log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
         layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
-        log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention); "
+        log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
+            f"{d['ms_per_layer_rope_as_its_own_launch']:.2f} ms with bias + RoPE as a launch of its own); "
             f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
-        for kind in ("w8a8", "w4a8", "w4a16"):
+        for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
             torch.cuda.empty_cache()
             layer["prefill_layer_" + kind] = d = prefill_layer_quant_leg(torch, dev, T, st, kind)
             log(f"  prefill layer, {kind} projections: {d['ms_per_layer']:.2f} ms ({d['Tops']:.0f} TOP/s over linears + "
                 f"attention); 28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
-        layer["decode_token"] = d = decode_token_leg(torch, dev, T)
-        log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
-            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
-            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
-        layer["decode_token_fused"] = d = decode_token_leg(torch, dev, T, fused=True)
-        log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
-            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
-            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+        if not args.no_token:
+            layer["decode_token"] = d = decode_token_leg(torch, dev, T)
+            log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+                f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+            layer["decode_token_fused"] = d = decode_token_leg(torch, dev, T, fused=True)
+            log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+                f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
 
-        for kind in ("w4a16", "w8a8", "w4a8"):
+        for kind in () if fp16_only or args.no_token else ("w4a16", "w8a8", "w4a8"):
             torch.cuda.empty_cache()
             layer["decode_token_" + kind] = d = decode_token_quant_leg(torch, dev, T, kind)
             log(f"  decode token, {kind} projections: {d['calls']} calls, eager {d['eager_ms']:.3f} ms, "

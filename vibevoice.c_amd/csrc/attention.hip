@@ -417,10 +417,16 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
 // one barrier per tile remains. V^T rows are 128 bytes: channel 8 d + e sits in row 16 e + d (so
 // the eight rows a thread writes are 16 rows apart and a wave's writes spread over the banks), its
 // 16-byte units XOR-ed with (row / 2) % 8, and the keys inside a row are ordered so that the eight
-// keys a lane multiplies in one step are one unit: 16-byte reads, bank-conflict free. The values
-// and their order of summation are those of prefill128: the same bits.
+// keys a lane multiplies in one step are one unit: 16-byte reads. The values and their order of
+// summation are those of prefill128: the same bits.
+// The loop is unrolled by two so that the buffers are compile-time constants (LDS addresses are a
+// per-lane offset plus an immediate) and the two score sets swap roles without a copy; contiguous
+// caches are addressed as a uniform base per tile plus a per-lane offset that never changes; the
+// probabilities are converted two at a time. What is left is bound by the vector ALU: about 280
+// vector instructions and 33 exponentials per tile and wave against 32 MFMAs.
 // Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
 // alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
+template <int kValue> struct Parity { static constexpr int value = kValue; };
 constexpr int kVtRowHalves = 64;                 // one V^T row: 64 keys, 128 bytes, 8 units of 16 bytes
 struct PipeTiles {
     Chunk k[2][kKeyTile * 16];                   // [buffer][key][16 slots], slot ^ (key & 15)
@@ -456,26 +462,52 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
 
     // K tile j -> buffer j & 1, straight into LDS: copy c of this wave fills slots 64 (4 wave + c) .. + 63:
     // keys 4 (4 wave + c) .. + 3, the lane owning (key, physical slot) and fetching the logical slot.
+    // Contiguous cache, tile wholly inside it: a uniform base per tile plus a 32-bit offset per lane that never
+    // changes, so a copy costs no vector instruction. Otherwise (pages, the cache's last rows): an address per lane.
+    uint32_t k_off[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
+        k_off[c] = (uint32_t)(((size_t)key * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)((phys ^ (key & 15)) * 16);
+    }
     auto request_k = [&](int j) {
         const int t0 = j * kKeyTile;
+        const uint32_t lds_at = lds_k0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave) * 1024u;
+        if (!page_table && t0 + kKeyTile <= kv_len) {
+            const char* base = reinterpret_cast<const char*>(K) + (size_t)t0 * row_halves * 2u;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
-            const int row = cache_row(page_table, min(t0 + key, last_key));
-            const Chunk* g = reinterpret_cast<const Chunk*>(K + (size_t)row * row_halves + (size_t)kvh * kD) + (phys ^ (key & 15));
-            copy16_to_lds(g, lds_k0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave + c) * 1024u);
+            for (int c = 0; c < 4; ++c)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             : : "s"(lds_at + (uint32_t)c * 1024u), "v"(k_off[c]), "s"(base) : "memory", "m0");
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
+                const int row = cache_row(page_table, min(t0 + key, last_key));
+                const Chunk* g = reinterpret_cast<const Chunk*>(K + (size_t)row * row_halves + (size_t)kvh * kD) + (phys ^ (key & 15));
+                copy16_to_lds(g, lds_at + (uint32_t)c * 1024u);
+            }
         }
     };
     // V tile: a thread takes four consecutive keys 4 kg .. + 3 of one 8-channel chunk.
     const int dchunk = tid & 15, kg = tid >> 4;
     Chunk vr[4];
-    auto fetch_v = [&](int j) {
-        const int t0 = j * kKeyTile;
+    uint32_t v_off[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 4; ++i) v_off[i] = (uint32_t)(((size_t)(4 * kg + i) * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)dchunk * 16u;
+    auto fetch_v1 = [&](int j, int i) {
+        const int t0 = j * kKeyTile;
+        if (!page_table && t0 + kKeyTile <= kv_len) {
+            const char* base = reinterpret_cast<const char*>(V) + (size_t)t0 * row_halves * 2u;
+            vr[i] = load_chunk(reinterpret_cast<const Chunk*>(base + v_off[i]));
+        } else {
             const int row = cache_row(page_table, min(t0 + 4 * kg + i, last_key));
             vr[i] = load_chunk(reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + dchunk);
         }
+    };
+    auto fetch_v = [&](int j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fetch_v1(j, i);
     };
     // key 32 a + 16 sp + 8 x + 4 h + i sits at position 32 a + 16 sp + 8 h + 4 x + i of its row, so that the eight
     // keys a lane multiplies in one step are one 16-byte unit; kg = 8 a + 4 sp + 2 x + h
@@ -506,21 +538,43 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         }
     };
 
-    if (ntiles > 0) {
-        request_k(0);
-        request_k(1);
-        fetch_v(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        commit_v(0);
-        fetch_v(1);
-    }
+    // (q_len, kv_len > 0: every workgroup has at least one tile. The prologue is unconditional so that the
+    // compiler knows the query loads have been waited for when the loop starts; on a path around it, it
+    // would wait for them - and with them for every copy in flight - inside the loop.)
+    request_k(0);
+    request_k(1);
+    fetch_v(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    commit_v(0);
+    fetch_v(1);
     asm volatile("s_waitcnt vmcnt(4)" ::: "memory");          // K 0 and K 1 landed; V 1 may fly
     __syncthreads();
-    f32x16 s_cur[2];
-    if (ntiles > 0) scores(0, s_cur);
+    // a lane's fragment positions inside a tile never change: row col (+ 32 a) of K, slot 2 s8 + half swizzled;
+    // row col (+ 32 t) of V^T, unit 2 u + half swizzled ((32 t + col) / 2 % 8 = col / 2 % 8)
+    int kf_idx[8], vf_idx[4];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) kf_idx[s8] = col * 16 + ((2 * s8 + half) ^ (col & 15));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) vf_idx[u] = col * kVtRowHalves + (((2 * u + half) ^ ((col >> 1) & 7)) * 8);
+    f32x16 s_pp[2][2];                        // the scores of the tile in hand and of the next, by tile parity
+    scores(0, s_pp[0]);
     __syncthreads();                                          // K 0 is read: its buffer may take K 2
 
-    for (int j = 0; j < ntiles; ++j) {
+    // Byte offsets of this lane's fragments from the start of a K / V^T buffer: with the buffer a compile-time
+    // constant (the loop is unrolled by two) the rest of an LDS address is an immediate.
+    uint32_t kf_byte[8], vf_byte[4];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) kf_byte[s8] = (uint32_t)kf_idx[s8] * 16u;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) vf_byte[u] = (uint32_t)vf_idx[u] * 2u;
+    const uint32_t vw_byte = (uint32_t)(dchunk * kVtRowHalves + 4 * v_sub) * 2u;      // V^T write: row 16 e + dchunk
+    // ... whose unit swizzle, (row / 2) % 8 = (8 e + dchunk / 2) % 8, does not depend on e
+    const uint32_t vw_unit = (uint32_t)((v_unit ^ ((dchunk >> 1) & 7)) * 16);
+    // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
+    auto body = [&](int j, auto parity_c) {
+        constexpr int P = decltype(parity_c)::value;
+        f32x16 (&s_cur)[2] = s_pp[P];
+        f32x16 (&s_next)[2] = s_pp[P ^ 1];
         const int t0 = j * kKeyTile;
         if (t0 + kKeyTile > kv_len || (causal && t0 + kKeyTile - 1 > q_offset + qw0)) {
 #pragma unroll
@@ -532,14 +586,10 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                     s_cur[a][r] = seen ? s_cur[a][r] : -INFINITY;
                 }
         }
-        // block 1: the next tile's scores on the matrix pipe, this tile's softmax on the vector ALU, a slice of
-        // the one behind each MFMA of the other
-        f32x16 s_next[2];
         request_k(j + 2);                                     // into the buffer tile j's K has left
-        const Chunk* kb = tiles.k[(j + 1) & 1];
+        const char* kb = reinterpret_cast<const char*>(&tiles.k[P ^ 1][0]);
         auto k_frag = [&](int k) {                            // step k = 8 a + s8
-            const int row = 32 * (k >> 3) + col, slot = 2 * (k & 7) + half;
-            return __builtin_bit_cast(h16x8, kb[row * 16 + (slot ^ (row & 15))]);
+            return __builtin_bit_cast(h16x8, *reinterpret_cast<const Chunk*>(kb + (k >> 3) * 8192 + kf_byte[k & 7]));
         };
 #pragma unroll
         for (int a = 0; a < 2; ++a)
@@ -569,11 +619,20 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                 for (int q = (k - 4) * 32 / 12; q < (k - 3) * 32 / 12; ++q) {
                     const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -m_use));
                     sum += p;
-                    pf[q >> 3][q & 7] = (h16)p;
+                    s_cur[q >> 4][q & 15] = p;
                 }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        // two probabilities per conversion (v_cvt_pk_f16_f32, round to nearest even like the single one)
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int q = 0; q < 32; q += 2) {
+            const f32x2 two = {s_cur[q >> 4][q & 15], s_cur[q >> 4][(q & 15) + 1]};
+            const h16x2 h = __builtin_convertvector(two, h16x2);
+            pf[q >> 3][q & 7] = h[0];
+            pf[q >> 3][(q & 7) + 1] = h[1];
+        }
         sum += other_half(sum);
         if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
             const float alpha = exp2_fast(st.m - m_use);
@@ -587,10 +646,10 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         st.m = m_new;
         // block 2: O^T += V^T P^T on the matrix pipe; behind its MFMAs the next tile's V^T goes into its buffer
         // and the tile after that is asked for
-        const h16* vb = tiles.vt[j & 1];
+        const char* vb = reinterpret_cast<const char*>(&tiles.vt[P][0]);
+        char* vw = reinterpret_cast<char*>(&tiles.vt[P ^ 1][0]);
         auto v_frag = [&](int k) {                            // step k = 4 u + t
-            const int row = 32 * (k & 3) + col;
-            return *reinterpret_cast<const h16x8*>(&vb[row * kVtRowHalves + (((2 * (k >> 2) + half) ^ ((row >> 1) & 7)) * 8)]);
+            return *reinterpret_cast<const h16x8*>(vb + (k & 3) * 32 * kVtRowHalves * 2 + vf_byte[k >> 2]);
         };
         h16x8 vf[3];
         vf[0] = v_frag(0);
@@ -608,21 +667,21 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                 for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
             }
             if (k >= 4 && k < 12) {
-                const int e = k - 4, row = 16 * e + dchunk;
+                const int e = k - 4;
                 const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
-                *reinterpret_cast<h16x4*>(&tiles.vt[(j + 1) & 1][row * kVtRowHalves + ((v_unit ^ ((row >> 1) & 7)) * 8) + 4 * v_sub]) = w;
+                *reinterpret_cast<h16x4*>(vw + e * 16 * kVtRowHalves * 2 + vw_byte + vw_unit) = w;
             }
-            if (k >= 12) {
-                const int i = k - 12;
-                const int row = cache_row(page_table, min((j + 2) * kKeyTile + 4 * kg + i, last_key));
-                vr[i] = load_chunk(reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + dchunk);
-            }
+            if (k >= 12) fetch_v1(j + 2, k - 12);
         }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(4)" ::: "memory");      // K j+2 landed (V j+2 may fly)
         __syncthreads();
-#pragma unroll
-        for (int a = 0; a < 2; ++a) s_cur[a] = s_next[a];
+    };
+    // An odd tile count is rounded up: the extra tile lies wholly past the keys the workgroup may see, so it
+    // is masked, its probabilities are zeros and the state does not move.
+    for (int j = 0; j < ntiles; j += 2) {
+        body(j, Parity<0>{});
+        body(j + 1, Parity<1>{});
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no copy may land after the workgroup has gone
