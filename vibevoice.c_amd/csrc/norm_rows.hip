@@ -207,8 +207,10 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
             a[j] = pack(x);                       // the stored residual; the norm reads that value
             x = unpack(a[j]);
         }
-        if ((kMode == kAdd || kMode == kGather) && (kFull || c < nchunks))
-            store_chunk_as<kStream>(state + out_base + c, a[j]);
+        // The updated residual goes out as soon as it is known; the gathered row waits until the normed row
+        // is out (cold at 2048 / 4096 rows: add+norm 10.4 / 20.7 us storing here against 10.6 / 21.2 us
+        // storing last; gather+norm 8.6 us storing here against 8.3 us storing last).
+        if (kMode == kAdd && (kFull || c < nchunks)) store_chunk_as<kStream>(state + out_base + c, a[j]);
         const float acc = chunk_sumsq(x, 0.0f);
         total += wave_sum((kFull || c < nchunks) ? acc : 0.0f);
     }
@@ -216,9 +218,11 @@ __global__ __launch_bounds__(kBlock) void norm_rows_wave(
 #pragma unroll
     for (int j = 0; j < kCpl; ++j) {
         const int c = j * kWave + lane;
-        if (kFull || c < nchunks)
+        if (kFull || c < nchunks) {
             store_chunk_as<kStream>(normed + out_base + c,
                                     scale_chunk(a[j], inv, wsh[kFull ? c : min(c, nchunks - 1)]));
+            if (kMode == kGather) store_chunk_as<kStream>(state + out_base + c, a[j]);
+        }
     }
 }
 
