@@ -49,7 +49,9 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           (285, 3584, 3584), (130, 101, 200), (257, 37, 8), (48, 512, 256), (70, 3584, 18944), (29, 18944, 512),
           (4100, 8200, 72), (4097, 8192, 64),     # enough 256x256 workgroups for the eight-wave tile
           (4100, 8200, 192), (4097, 8192, 128), (4100, 8200, 96),
-          (2048, 18944, 64), (2300, 16400, 128)]       # 20 and 90 blocks of 4 x 8 tiles: not a multiple of the eight XCDs    # ... fed in 128-byte slabs (K % 64 == 0), or in 64-byte ones
+          # 256x256 tiles in 4 x 8 blocks dealt to the eight XCDs: 18 and 128 whole blocks with ragged edges, no whole
+          # block at all (7 tile columns), whole blocks only
+          (2048, 18944, 64), (2300, 16400, 128), (19000, 1792, 64), (4096, 8192, 64)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

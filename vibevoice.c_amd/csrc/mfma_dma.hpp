@@ -170,8 +170,14 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
 //     again for the next slab (the L1 is far too small to keep it). Here a row's whole line comes
 //     in one copy: half the requests to L2, half the barriers per MFMA.
 //   * Workgroups are handed to the eight XCDs in turn, so in launch order the 32 workgroups that
-//     run together on one XCD share one row of tiles and nothing of the other operand. Here the
-//     workgroups of an XCD walk 4 x 8 blocks of tiles (12 operand tiles per 32 instead of 33).
+//     run together on one XCD share one row of tiles and nothing of the other operand. Here an XCD
+//     walks whole 4 x 8 blocks of tiles (12 operand tiles per 32 instead of 33), the eight XCDs
+//     eight consecutive blocks at a time, so they also read the same operand rows at the same
+//     time and share them in the memory-side cache. Only as many blocks as divide by eight are
+//     dealt out whole; the tiles of the others and of the ragged right and bottom edges are
+//     numbered behind them and cut into eight equal runs, so every XCD has the same number of
+//     tiles (whole blocks only leave the same XCDs a round short again and again: 584 against
+//     480 tiles at 57 x 74).
 //   * The clock is not a constant: under this load the device runs at 1.6-1.8 GHz of its 2.4, and
 //     a loop that wastes fewer cycles is answered with a lower clock. What is left to gain is
 //     energy per product, not cycles.
@@ -185,12 +191,58 @@ constexpr int kDma64StageSlots = 2 * kDmaTile * (kDma64SlabBytes / 16);      // 
 constexpr size_t kDma64LdsBytes = (size_t)2 * kDma64StageSlots * 16;
 constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 workgroups, one per CU of an XCD
 
-inline unsigned dma64_grid(int M, int N) {
-    const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
-    // workgroup i runs block 8 (i / 256) + i % 8: whole groups of eight blocks, or the last ones stay half done
-    const int blocks = ((gx + kSuperN - 1) / kSuperN) * ((gy + kSuperM - 1) / kSuperM);
-    return (unsigned)((blocks + 7) / 8 * 8 * (kSuperM * kSuperN));
-}
+// The numbering above for a gy x gx grid of tiles. `whole`: tiles per XCD that come in whole blocks;
+// `run`: the length of an XCD's run of the remaining `rest` tiles.
+struct Dma64Map {
+    int gx, gy, fx, fy, whole, run, rest, spare, right;
+    __host__ __device__ Dma64Map(int M, int N) {
+        gx = (N + kDmaTile - 1) / kDmaTile;
+        gy = (M + kDmaTile - 1) / kDmaTile;
+        fx = gx / kSuperN;                                // whole blocks per row of blocks
+        fy = gy / kSuperM;
+        const int blocks = fx * fy;
+        whole = (blocks / 8) * (kSuperM * kSuperN);
+        spare = (blocks % 8) * (kSuperM * kSuperN);       // tiles of the whole blocks that are not dealt out
+        right = gy * (gx - fx * kSuperN);                 // tiles right of the last whole block, every row
+        rest = spare + right + (gy - fy * kSuperM) * fx * kSuperN;
+        run = (rest + 7) / 8;
+    }
+    __host__ __device__ unsigned grid() const { return (unsigned)(8 * (whole + run)); }
+    // Tile of workgroup `wg` (it runs on XCD wg % 8 as that XCD's (wg / 8)-th); false: none.
+    __device__ __forceinline__ bool tile(int wg, int& tile_m, int& tile_n) const {
+        const int xcd = wg & 7, nth = wg >> 3;
+        int block, within;
+        if (nth < whole) {
+            block = (nth >> 5) * 8 + xcd;
+            within = nth & 31;
+        } else {
+            int e = xcd * run + (nth - whole);
+            if (e >= rest) return false;
+            if (e >= spare) {
+                e -= spare;
+                if (e < right) {
+                    const int wr = gx - fx * kSuperN;
+                    tile_m = e / wr;
+                    tile_n = fx * kSuperN + e % wr;
+                } else {
+                    e -= right;
+                    const int hb = gy - fy * kSuperM;
+                    tile_m = fy * kSuperM + e % hb;
+                    tile_n = e / hb;
+                }
+                return true;
+            }
+            block = (whole >> 5) * 8 + (e >> 5);
+            within = e & 31;
+        }
+        const int block_y = block / fx;
+        tile_m = block_y * kSuperM + (within >> 3);
+        tile_n = (block - block_y * fx) * kSuperN + (within & 7);
+        return true;
+    }
+};
+
+inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N).grid(); }
 
 template <typename Op, bool kPairN = false, typename Epi>
 __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
@@ -206,15 +258,9 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    // Workgroup -> tile: workgroup i runs on XCD i % 8 as its (i / 8)-th; an XCD takes whole blocks of tiles.
-    const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
-    const int blocks_x = (gx + kSuperN - 1) / kSuperN;
-    const int xcd = (int)blockIdx.x & 7, nth = (int)blockIdx.x >> 3;
-    const int seq = ((nth >> 5) * 8 + xcd) * 32 + (nth & 31);
-    const int block = seq >> 5, within = seq & 31;
-    const int block_y = block / blocks_x, block_x = block - block_y * blocks_x;
-    const int tile_m = block_y * kSuperM + (within >> 3), tile_n = block_x * kSuperN + (within & 7);
-    if (tile_m >= gy || tile_n >= gx) return;             // the whole workgroup, before any barrier
+    const Dma64Map map(M, N);
+    int tile_m, tile_n;
+    if (!map.tile((int)blockIdx.x, tile_m, tile_n)) return;      // the whole workgroup, before any barrier
     const int m_blk = tile_m * kDmaTile, n_blk = tile_n * kDmaTile;
     const int nslabs = row_bytes / kDma64SlabBytes;
     const uint32_t lds0 =
