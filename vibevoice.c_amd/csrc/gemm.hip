@@ -34,6 +34,7 @@ namespace vv {
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float finish(float acc, float alpha, float beta, h16 old) {
     return alpha * acc + beta * (float)old;
@@ -84,7 +85,45 @@ struct F16Op {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, w),
                                                       __builtin_bit_cast(h16x8, x), c, 0, 0, 0);
     }
+    typedef f32x4 Acc16;
+    static __device__ __forceinline__ Acc16 mfma16(u32x4 w, u32x4 x, Acc16 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, w),
+                                                      __builtin_bit_cast(h16x8, x), c, 0, 0, 0);
+    }
 };
+
+// A wave's 4 x 8 accumulator tiles of 16 x 16 (mfma_dma64) to C: register r of lane l holds column
+// n0 + 16 a + 4 (l / 16) + r of row m0 + 16 b + l % 16 of acc[a][b].
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[4][8], h16* __restrict__ C, int M, int N, int m0,
+                                             int n0, int lane, float alpha, float beta, int vec_store) {
+    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const int m = m0 + b * 16 + (lane & 15);
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int n = n0 + a * 16 + 4 * (lane >> 4);
+            if (n >= N) continue;
+            if (vec_store && n + 3 < N) {
+                h16x4 old = {0, 0, 0, 0};
+                if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = to_half(finish(acc[a][b][r], alpha, beta, old[r]));
+                *reinterpret_cast<h16x4*>(crow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) {
+                        const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                        crow[n + r] = to_half(finish(acc[a][b][r], alpha, beta, old));
+                    }
+            }
+        }
+    }
+}
 
 template <int BM, int BN, int WM, int WN, int kSlab, bool kFull, int kAhead>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile(
@@ -139,8 +178,8 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
 __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64(
     const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
     int K, float alpha, float beta, int vec_store) {
-    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
-        store_tile<4, 2>(acc, C, M, N, m0, n0, frow, fhalf, alpha, beta, vec_store);
+    auto epilogue = [=](const f32x4 (&acc)[4][8], int m0, int n0, int lane) {
+        store_tile16(acc, C, M, N, m0, n0, lane, alpha, beta, vec_store);
     };
     mfma_dma64<F16Op>(A, B, M, N, K * 2, epilogue);
 }
@@ -201,6 +240,57 @@ __device__ __forceinline__ void store_tile_rope(const f32x16 (&acc)[2][TM], h16*
     }
 }
 
+// The same store for mfma_dma64's 16 x 16 tiles (kPairN: tiles a and a + 2 are 64 columns apart, tile a at
+// column 16 (a % 2) + 64 (a / 2) of the wave's head half): register r of acc[a][b] and of acc[a + 2][b] are the
+// rotate-half pair.
+__device__ __forceinline__ void store_tile16_rope(const f32x4 (&acc)[4][8], h16* __restrict__ C,
+                                                  const h16* __restrict__ bias, const float2* __restrict__ table,
+                                                  int M, int N, int m0, int n0, int lane, float alpha, float beta) {
+    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+    if (n0 >= N) return;                         // whole heads: the wave's 32 + 32 columns are all in or all out
+    const int pair0 = n0 & 127;                  // 0 or 32: the first rotation pair of tile 0
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const int m = m0 + b * 16 + (lane & 15);
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+        const float2* trow = table + (size_t)m * 64;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int col = 16 * a + 4 * (lane >> 4);
+            const int n = n0 + col;
+            h16x4 lo, hi;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                lo[r] = to_half(finish(acc[a][b][r], alpha, beta, (h16)0.0f));
+                hi[r] = to_half(finish(acc[a + 2][b][r], alpha, beta, (h16)0.0f));
+            }
+            if (bias) {
+                const h16x4 blo = *reinterpret_cast<const h16x4*>(bias + n);
+                const h16x4 bhi = *reinterpret_cast<const h16x4*>(bias + n + 64);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    lo[r] = to_half((float)lo[r] + (float)blo[r]);
+                    hi[r] = to_half((float)hi[r] + (float)bhi[r]);
+                }
+            }
+            const float4 cs01 = *reinterpret_cast<const float4*>(trow + pair0 + col);
+            const float4 cs23 = *reinterpret_cast<const float4*>(trow + pair0 + col + 2);
+            const float cv[4] = {cs01.x, cs01.z, cs23.x, cs23.z};
+            const float sv[4] = {cs01.y, cs01.w, cs23.y, cs23.w};
+            h16x4 olo, ohi;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const Pair p = rotate((float)lo[r], (float)hi[r], cv[r], sv[r]);
+                olo[r] = to_half(p.lo);
+                ohi[r] = to_half(p.hi);
+            }
+            *reinterpret_cast<h16x4*>(crow + n) = olo;
+            *reinterpret_cast<h16x4*>(crow + n + 64) = ohi;
+        }
+    }
+}
+
 template <int BM, int BN, int WM, int WN, int kSlab, bool kFull, int kAhead>
 __global__ __launch_bounds__(WM * WN * kWave) void gemm_tile_rope(
     const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
@@ -225,8 +315,8 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma_rope(
 __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64_rope(
     const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
     const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
-    auto epilogue = [=](const f32x16 (&acc)[2][4], int m0, int n0, int frow, int fhalf) {
-        store_tile_rope<4>(acc, C, bias, table, M, N, m0, n0, frow, fhalf, alpha, beta);
+    auto epilogue = [=](const f32x4 (&acc)[4][8], int m0, int n0, int lane) {
+        store_tile16_rope(acc, C, bias, table, M, N, m0, n0, lane, alpha, beta);
     };
     mfma_dma64<F16Op, true>(A, B, M, N, K * 2, epilogue);
 }
@@ -360,7 +450,6 @@ inline int gemv_split(int N) { return N >= 16384 ? 1 : N >= 8192 ? 2 : 4; }
 // of each weight row), two lines in flight per iteration; the eight partial
 // tiles meet in LDS. The activations (M x K, at most 2.4 MB) come from L1/L2.
 // The K order differs from gemm_tile's, so the bits may too (same bounds).
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyWaves = 8;
 
 // Up to three projections of the same activations in one launch (q/k/v,
@@ -542,14 +631,43 @@ bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes) {
     return true;
 }
 
+// Rows of the 256x256 tiles' launch when the last round of workgroups would run mostly empty. Every XCD takes
+// an eighth of the tiles, 32 at a time, so a launch costs ceil(tiles / 8 / 32) rounds; 57 x 14 tiles (14449 rows
+// into 3584 columns) are 3.1 rounds and cost four. The rows that spill into a round of their own go to the
+// 128x128 tile kernel instead, whose rounds are short (priced at 0.45 of a 256x256 round, measured at K = 18944;
+// less for shorter K): 54 rows of tiles in three rounds, the other 625 rows in one short one. 0: no split pays
+// (at least a twentieth of the time).
+int dma64_split_rows(int M, int N) {
+    const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
+    auto rounds = [](long tiles) { return (double)(((tiles + 7) / 8 + 31) / 32); };
+    const double whole = rounds((long)gx * gy);
+    double best = whole * 0.95;
+    int best_rows = 0;
+    for (int r = gy - 1; r >= 1 && r >= gy - 16; --r) {
+        const int tail = M - r * kDmaTile;
+        const long small = (long)((tail + 127) / 128) * ((N + 127) / 128);
+        const double cost = rounds((long)gx * r) + 0.45 * (double)((small + 255) / 256);
+        if (cost < best) {
+            best = cost;
+            best_rows = r * kDmaTile;
+        }
+    }
+    return best_rows;
+}
+
 bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
                 hipStream_t st) {
     static thread_local int ready32 = -1, ready64 = -1;
     const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
     if (K % (kDma64SlabBytes / 2) == 0) {
         if (!allow_big_lds(gemm_dma64, ready64, kDma64LdsBytes)) return false;
-        gemm_dma64<<<dim3(dma64_grid(M, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
-            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha, beta, vec);
+        const int head = dma64_split_rows(M, N);
+        const int rows = head ? head : M;
+        gemm_dma64<<<dim3(dma64_grid(rows, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
+            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), rows, N, K, alpha, beta, vec);
+        if (head)
+            launch_tile<128, 128, 2, 2, 64, 2>(static_cast<const h16*>(A) + (size_t)head * K, B,
+                                               static_cast<h16*>(C) + (size_t)head * N, M - head, N, K, alpha, beta, st);
         return true;
     }
     if (!allow_big_lds(gemm_dma, ready32, kDmaLdsBytes)) return false;
@@ -649,8 +767,13 @@ bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table,
     if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
         static thread_local int ready32 = -1, ready64 = -1;
         if (K % (kDma64SlabBytes / 2) == 0 && allow_big_lds(gemm_dma64_rope, ready64, kDma64LdsBytes)) {
-            gemm_dma64_rope<<<dim3(dma64_grid(M, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(A, B, bias, table, C, M, N,
-                                                                                              K, 1.0f, 0.0f);
+            const int head = dma64_split_rows(M, N);         // the rows gemm() gives to this tile, so the same bits
+            const int rows = head ? head : M;
+            gemm_dma64_rope<<<dim3(dma64_grid(rows, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
+                A, B, bias, table, C, rows, N, K, 1.0f, 0.0f);
+            if (head)
+                launch_tile_rope<128, 128, 2, 2, 64, 2>(A + (size_t)head * K, B, bias, table + (size_t)head * 64,
+                                                        C + (size_t)head * N, M - head, N, K, st);
             return true;
         }
         if (K % (kDma64SlabBytes / 2) != 0 && allow_big_lds(gemm_dma_rope, ready32, kDmaLdsBytes)) {

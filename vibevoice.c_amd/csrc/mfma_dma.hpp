@@ -244,14 +244,25 @@ struct Dma64Map {
 
 inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N).grid(); }
 
+// The wave tile is 128 (m) x 64 (n) in TN x TM = 4 x 8 products of 16 x 16 over K steps of 32 (Op::mfma16: the
+// 16x16x32 matrix instructions move a fifth fewer register bytes per product than the 32x32x16 ones, and under the
+// power limit that is speed: 1.7-1.9 against 1.5-1.6 PFLOP/s for the bare instruction streams on random
+// operands). A fragment is 16 rows x 64 bytes: lane l reads slot K step * 4 + l / 16 of row l % 16.
+//   Op::Acc16                                4-wide accumulator vector
+//   Op::mfma16(u32x4 w, u32x4 x, Acc16 c)    one 16x16 product over a K step
+//   epi(acc, m0, n0, lane)                   register r of lane l: column n0 + off(a) + 4 (l / 16) + r of row
+//                                            m0 + 16 b + l % 16, for acc[a][b]; off(a) = 16 a, or with kPairN
+//                                            16 (a % 2) + 64 (a / 2): tiles a and a + 2 are 64 columns apart
+// The MFMAs of a step run x tile by x tile, so an x fragment is dead after four MFMAs and the next step's
+// takes its registers at once: only the four w fragments and two of the eight x fragments are held twice.
 template <typename Op, bool kPairN = false, typename Epi>
 __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
                                            int row_bytes, const Epi& epi) {
-    typedef typename Op::Acc Acc;
+    typedef typename Op::Acc16 Acc;
     constexpr int kSlabChunks = kDma64SlabBytes / 16;     // 8
-    constexpr int WN = 4, TM = 4, TN = 2;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
+    constexpr int WN = 4, TM = 8, TN = 4;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
     constexpr int kLoads = kDma64StageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 8
-    static_assert(kLoads == 8, "one copy request behind each MFMA of a K step");
+    static_assert(kLoads == 8, "the copy requests of a slab go behind eight MFMAs of its last K step");
     extern __shared__ u32x4 dma_lds[];
 
     const int tid = (int)threadIdx.x;
@@ -295,45 +306,76 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
 #pragma unroll
         for (int b = 0; b < TM; ++b)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+            for (int r = 0; r < 4; ++r) acc[a][b][r] = 0;
 
-    const int frow = lane & 31, fhalf = lane >> 5;
-    int f_idx[4];
+    const int frow = lane & 15, fquarter = lane >> 4;
+    int f_idx[2];
 #pragma unroll
-    for (int step = 0; step < 4; ++step)
-        f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 2 + fhalf);
-    const int fa_base = wm * TM * 32 * kSlabChunks;
-    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 32;      // first column of tile a = 0
-    constexpr int kTileStrideN = kPairN ? 64 : 32;
+    for (int step = 0; step < 2; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 4 + fquarter);
+    const int fa_base = wm * TM * 16 * kSlabChunks;
+    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 16;      // first column of tile a = 0
     const int fb_base = kDmaTile * kSlabChunks + wave_n0 * kSlabChunks;
+    auto w_off = [](int a) { return (kPairN ? (a & 1) * 16 + (a >> 1) * 64 : a * 16) * kSlabChunks; };
 
-    u32x4 fw[2][TN], fx[2][TM];                  // [set][tile]: the K step in hand and the next
-    // Fragment i of a step, in the order in which the step's MFMAs first use them: w0, x0, x1, x2, x3, w1.
-    auto read = [&](auto set_c, int slab, int step, int i) {
+    // w: the K step in hand and the next. x: one set, refilled in place, except the last two tiles of a step,
+    // which are held twice like w (their refill could only follow the step's last MFMAs, and the reads of a
+    // step must be back when the next begins).
+    constexpr int kSingle = TM - 2;
+    u32x4 fw[2][TN], fx[kSingle], fxl[2][TM - kSingle];
+    auto read_w = [&](auto set_c, int slab, int step, int a) {
         constexpr int set = decltype(set_c)::value;
-        const u32x4* st = dma_lds + (slab & 1) * kDma64StageSlots;
-        if (i == 0) fw[set][0] = st[fb_base + f_idx[step]];
-        else if (i == 5) fw[set][1] = st[fb_base + kTileStrideN * kSlabChunks + f_idx[step]];
-        else fx[set][i - 1] = st[fa_base + (i - 1) * 32 * kSlabChunks + f_idx[step]];
+        fw[set][a] = dma_lds[(slab & 1) * kDma64StageSlots + fb_base + w_off(a) + f_idx[step]];
     };
+    auto read_x = [&](auto set_c, int slab, int step, int b) {
+        constexpr int set = decltype(set_c)::value;
+        const u32x4 v = dma_lds[(slab & 1) * kDma64StageSlots + fa_base + b * 16 * kSlabChunks + f_idx[step]];
+        if (b < kSingle) fx[b] = v;
+        else fxl[set][b - kSingle] = v;
+    };
+    // One K step: 32 MFMAs, x tile by x tile. Reads and copy requests go behind MFMAs, one each; the next
+    // step's x fragment b < 6 can go anywhere behind the last MFMA of x tile b (it takes that fragment's
+    // registers). Step 0 reads step 1 of the same slab. Step 1 first issues eight MFMAs; behind the barrier
+    // that follows every wave has read all of this slab and the next slab has landed (this wave's copies;
+    // the barrier adds the others'): then come the reads of the next slab's step 0 and the eight copy
+    // requests of the slab after next into the stage just freed. The last read of a step is eight MFMAs
+    // from its end.
     auto k_step = [&](auto cur_c, auto nxt_c, int slab, auto step_c) {
         constexpr int set = decltype(cur_c)::value;
         constexpr int step = decltype(step_c)::value;
-        if constexpr (step == 3) {
-            // the next slab has landed (this wave's copies; the barrier adds the others') and every wave has
-            // this slab's last fragments in registers
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            __syncthreads();
-        }
-        const int nslab = step == 3 ? slab + 1 : slab;
-        constexpr int nstep = (step + 1) & 3;
+        constexpr int nstep = step ^ 1;
+        const int nslab = slab + step;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_sched_barrier(0);
-            acc[i / TM][i % TM] = Op::mfma(fw[set][i / TM], fx[set][i % TM], acc[i / TM][i % TM]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (i < 6) read(nxt_c, nslab, nstep, i);
-            if constexpr (step == 3) request(slab + 2, i);
+        for (int b = 0; b < TM; ++b) {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+                if (step == 1 && b == 2 && a == 0) {
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    __syncthreads();
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                acc[a][b] = Op::mfma16(fw[set][a], b < kSingle ? fx[b] : fxl[set][b - kSingle], acc[a][b]);
+                __builtin_amdgcn_sched_barrier(0);
+                const int slot = (b - 2 * step) * TN + a;          // step 1: counted from the barrier
+                if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
+                else if (slot == 1) read_x(nxt_c, nslab, nstep, step == 0 ? 6 : 0);
+                else if (slot == 2) read_w(nxt_c, nslab, nstep, 1);
+                else if (slot == 3) read_x(nxt_c, nslab, nstep, step == 0 ? 0 : 2);
+                else if (slot == 4) read_w(nxt_c, nslab, nstep, 2);
+                else if (slot == 5) read_w(nxt_c, nslab, nstep, 3);
+                else if (slot == 6) read_x(nxt_c, nslab, nstep, step == 0 ? 7 : 1);
+                else if (slot == 7) read_x(nxt_c, nslab, nstep, step == 0 ? 1 : 3);
+                else if (slot == 8 && step == 1) read_x(nxt_c, nslab, nstep, 6);
+                else if (slot == 9 && step == 1) read_x(nxt_c, nslab, nstep, 7);
+                else if (slot == 11) read_x(nxt_c, nslab, nstep, step == 0 ? 2 : 4);
+                else if (slot == 15) read_x(nxt_c, nslab, nstep, step == 0 ? 3 : 5);
+                else if (slot == 19 && step == 0) read_x(nxt_c, nslab, nstep, 4);
+                else if (slot == 23 && step == 0) read_x(nxt_c, nslab, nstep, 5);
+                else if constexpr (step == 1) {
+                    const int i = slot == 10 ? 0 : slot >= 12 && slot <= 14 ? slot - 11 : slot >= 16 && slot <= 19 ? slot - 12 : -1;
+                    if (i >= 0) request(slab + 2, i);
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -345,16 +387,16 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // slab 0; slab 1 is waited for at the first barrier
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 6; ++i) read(Const<0>{}, 0, 0, i);
+    for (int a = 0; a < TN; ++a) read_w(Const<0>{}, 0, 0, a);
+#pragma unroll
+    for (int b = 0; b < TM; ++b) read_x(Const<0>{}, 0, 0, b);
     for (int slab = 0; slab < nslabs; ++slab) {
         k_step(Const<0>{}, Const<1>{}, slab, Const<0>{});
         k_step(Const<1>{}, Const<0>{}, slab, Const<1>{});
-        k_step(Const<0>{}, Const<1>{}, slab, Const<2>{});
-        k_step(Const<1>{}, Const<0>{}, slab, Const<3>{});
     }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the surplus copies and reads land before the LDS is released
 
-    epi(acc, m_blk + wm * TM * 32, n_blk + wave_n0, frow, fhalf);
+    epi(acc, m_blk + wm * TM * 16, n_blk + wave_n0, lane);
 }
 
 }  // namespace vv
