@@ -5,9 +5,9 @@ Bars: the stated one for FP16 outputs (scaled error <= 2e-3) and an
 elementwise one of our own: half an FP16 ulp of the exact value plus 1e-5 of
 sum_k |a||b| (FP32 accumulation over K <= 18944 stays well inside that).
 Bit-exact: every tile shape against the 128x128 tile (same K order; above 64
-rows, where the tile kernels run) except the 256x256 tile on the 16x16x32
-instructions, which is held to it within the FP32 summation order and to
-itself bit for bit; beta = 0 never reading C, M <= 0 / N <= 0 launching nothing.
+rows, where the tile kernels run) except the tiles on the 16x16x32
+instructions, which are held to it within the FP32 summation order and to
+themselves bit for bit; beta = 0 never reading C, M <= 0 / N <= 0 launching nothing.
 """
 import numpy as np
 import pytest
@@ -52,7 +52,9 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           (4100, 8200, 192), (4097, 8192, 128), (4100, 8200, 96),
           # 256x256 tiles in 4 x 8 blocks dealt to the eight XCDs: 18 and 128 whole blocks with ragged edges, no whole
           # block at all (7 tile columns), whole blocks only
-          (2048, 18944, 64), (2300, 16400, 128), (19000, 1792, 64), (4096, 8192, 64)]
+          (2048, 18944, 64), (2300, 16400, 128), (19000, 1792, 64), (4096, 8192, 64),
+          # the 128x128 tile fed the same way: 17 x 17, 9 x 32 and 113 x 4 tiles
+          (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -67,10 +69,11 @@ def test_gemm_against_oracle_and_tile(M, N, K):
     d_t = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     tile = run(dev.vv_gemm_fp16_tile_dev, d_a, d_b, d_t, M, N, K)
     check(tile, ref, mag, f"tile {M}x{N}x{K}")
-    big = -(-M // 256) * -(-N // 256) >= 512 and K % 64 == 0
+    big = K % 64 == 0 and (-(-M // 256) * -(-N // 256) >= 512 or (M > 64 and -(-M // 128) * -(-N // 128) >= 256))
     if big:
-        # the 256x256 tile fed in 128-byte slabs multiplies with the 16x16x32 instructions, which add 32
-        # products at a time where the other tiles add 16: same sums, another rounding of the FP32 partials
+        # the tiles fed in 128-byte slabs (the choice from 256 tiles of 128x128 on, K % 64 == 0) multiply with the
+        # 16x16x32 instructions, which add 32 products at a time where the other tiles add 16: same sums, another
+        # rounding of the FP32 partials
         diff = np.abs(oracle.widen(got) - oracle.widen(tile))
         assert np.all(diff <= 2.0 ** -9 * mag + 2.0 ** -14), "tile shapes must agree to FP32 summation order"
         again = run(dev.vv_gemm_fp16_dev, d_a, d_b, torch.zeros_like(d_c), M, N, K)

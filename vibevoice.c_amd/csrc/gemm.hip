@@ -92,13 +92,14 @@ struct F16Op {
     }
 };
 
-// A wave's 4 x 8 accumulator tiles of 16 x 16 (mfma_dma64) to C: register r of lane l holds column
+// A wave's 4 x TM accumulator tiles of 16 x 16 (mfma_dma64) to C: register r of lane l holds column
 // n0 + 16 a + 4 (l / 16) + r of row m0 + 16 b + l % 16 of acc[a][b].
-__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[4][8], h16* __restrict__ C, int M, int N, int m0,
+template <int TM>
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[4][TM], h16* __restrict__ C, int M, int N, int m0,
                                              int n0, int lane, float alpha, float beta, int vec_store) {
     typedef h16 h16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < TM; ++b) {
         const int m = m0 + b * 16 + (lane & 15);
         if (m >= M) continue;
         h16* crow = C + (size_t)m * N;
@@ -174,14 +175,17 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
     mfma_dma<F16Op>(A, B, M, N, K * 2, epilogue);
 }
 
-// The same tile fed in slabs of 64 halves (whole cache lines per row; mfma_dma.hpp). Needs K % 64 == 0.
-__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64(
+// The 256x256 or 128x128 tile fed in slabs of 64 halves (whole cache lines per row; mfma_dma.hpp). Needs
+// K % 64 == 0.
+template <int kTile, int kStages>
+__global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma64(
     const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
     int K, float alpha, float beta, int vec_store) {
-    auto epilogue = [=](const f32x4 (&acc)[4][8], int m0, int n0, int lane) {
-        store_tile16(acc, C, M, N, m0, n0, lane, alpha, beta, vec_store);
+    constexpr int TM = Dma64Shape<kTile>::TM;
+    auto epilogue = [=](const f32x4 (&acc)[4][TM], int m0, int n0, int lane) {
+        store_tile16<TM>(acc, C, M, N, m0, n0, lane, alpha, beta, vec_store);
     };
-    mfma_dma64<F16Op>(A, B, M, N, K * 2, epilogue);
+    mfma_dma64<F16Op, kTile, false, kStages>(A, B, M, N, K * 2, epilogue);
 }
 
 // The projection epilogue of a rotary attention layer in the GEMM's store: C = rope(fp16(A W^T) + bias)
@@ -243,14 +247,15 @@ __device__ __forceinline__ void store_tile_rope(const f32x16 (&acc)[2][TM], h16*
 // The same store for mfma_dma64's 16 x 16 tiles (kPairN: tiles a and a + 2 are 64 columns apart, tile a at
 // column 16 (a % 2) + 64 (a / 2) of the wave's head half): register r of acc[a][b] and of acc[a + 2][b] are the
 // rotate-half pair.
-__device__ __forceinline__ void store_tile16_rope(const f32x4 (&acc)[4][8], h16* __restrict__ C,
+template <int TM>
+__device__ __forceinline__ void store_tile16_rope(const f32x4 (&acc)[4][TM], h16* __restrict__ C,
                                                   const h16* __restrict__ bias, const float2* __restrict__ table,
                                                   int M, int N, int m0, int n0, int lane, float alpha, float beta) {
     typedef h16 h16x4 __attribute__((ext_vector_type(4)));
     if (n0 >= N) return;                         // whole heads: the wave's 32 + 32 columns are all in or all out
     const int pair0 = n0 & 127;                  // 0 or 32: the first rotation pair of tile 0
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < TM; ++b) {
         const int m = m0 + b * 16 + (lane & 15);
         if (m >= M) continue;
         h16* crow = C + (size_t)m * N;
@@ -312,13 +317,15 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma_rope(
     mfma_dma<F16Op, true>(A, B, M, N, K * 2, epilogue);
 }
 
-__global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma64_rope(
+template <int kTile, int kStages>
+__global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma64_rope(
     const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
     const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
-    auto epilogue = [=](const f32x4 (&acc)[4][8], int m0, int n0, int lane) {
-        store_tile16_rope(acc, C, bias, table, M, N, m0, n0, lane, alpha, beta);
+    constexpr int TM = Dma64Shape<kTile>::TM;
+    auto epilogue = [=](const f32x4 (&acc)[4][TM], int m0, int n0, int lane) {
+        store_tile16_rope<TM>(acc, C, bias, table, M, N, m0, n0, lane, alpha, beta);
     };
-    mfma_dma64<F16Op, true>(A, B, M, N, K * 2, epilogue);
+    mfma_dma64<F16Op, kTile, true, kStages>(A, B, M, N, K * 2, epilogue);
 }
 
 // M == 1: bound by the weight bytes. kSplit waves share an output column (a
@@ -634,8 +641,8 @@ bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes) {
 // Rows of the 256x256 tiles' launch when the last round of workgroups would run mostly empty. Every XCD takes
 // an eighth of the tiles, 32 at a time, so a launch costs ceil(tiles / 8 / 32) rounds; 57 x 14 tiles (14449 rows
 // into 3584 columns) are 3.1 rounds and cost four. The rows that spill into a round of their own go to the
-// 128x128 tile kernel instead, whose rounds are short (priced at 0.45 of a 256x256 round, measured at K = 18944;
-// less for shorter K): 54 rows of tiles in three rounds, the other 625 rows in one short one. 0: no split pays
+// 128x128 tile instead, whose rounds are short (a third of a 256x256 round, measured at K = 3584 and 18944;
+// priced at 0.35): 54 rows of tiles in three rounds, the other 625 rows in one short one. 0: no split pays
 // (at least a twentieth of the time).
 int dma64_split_rows(int M, int N) {
     const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
@@ -646,7 +653,7 @@ int dma64_split_rows(int M, int N) {
     for (int r = gy - 1; r >= 1 && r >= gy - 16; --r) {
         const int tail = M - r * kDmaTile;
         const long small = (long)((tail + 127) / 128) * ((N + 127) / 128);
-        const double cost = rounds((long)gx * r) + 0.45 * (double)((small + 255) / 256);
+        const double cost = rounds((long)gx * r) + 0.35 * (double)((small + 255) / 256);
         if (cost < best) {
             best = cost;
             best_rows = r * kDmaTile;
@@ -655,19 +662,41 @@ int dma64_split_rows(int M, int N) {
     return best_rows;
 }
 
+template <int kTile, int kStages = 2>
+bool launch_dma64(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+                  hipStream_t st) {
+    typedef Dma64Shape<kTile, kStages> Shape;
+    static thread_local int ready = -1;
+    if (!allow_big_lds(gemm_dma64<kTile, kStages>, ready, Shape::kLdsBytes)) return false;
+    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    gemm_dma64<kTile, kStages><<<dim3(dma64_grid<kTile>(M, N)), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(
+        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha, beta, vec);
+    return true;
+}
+
+// The 128x128 tile: fed by copies straight into LDS when K is a multiple of 64 (four stages deep when no
+// compute unit gets a second workgroup to fill its waits, two otherwise), through registers otherwise.
+bool dma128_alone(int M, int N) { return (long)((M + 127) / 128) * ((N + 127) / 128) <= 256; }
+
+void launch_128(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+                hipStream_t st) {
+    if (K % (kDma64SlabBytes / 2) == 0 &&
+        (dma128_alone(M, N) ? launch_dma64<128, 4>(A, B, C, M, N, K, alpha, beta, st)
+                            : launch_dma64<128, 2>(A, B, C, M, N, K, alpha, beta, st)))
+        return;
+    launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st);
+}
+
 bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
                 hipStream_t st) {
-    static thread_local int ready32 = -1, ready64 = -1;
+    static thread_local int ready32 = -1;
     const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
     if (K % (kDma64SlabBytes / 2) == 0) {
-        if (!allow_big_lds(gemm_dma64, ready64, kDma64LdsBytes)) return false;
         const int head = dma64_split_rows(M, N);
-        const int rows = head ? head : M;
-        gemm_dma64<<<dim3(dma64_grid(rows, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
-            static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), rows, N, K, alpha, beta, vec);
+        if (!launch_dma64<256>(A, B, C, head ? head : M, N, K, alpha, beta, st)) return false;
         if (head)
-            launch_tile<128, 128, 2, 2, 64, 2>(static_cast<const h16*>(A) + (size_t)head * K, B,
-                                               static_cast<h16*>(C) + (size_t)head * N, M - head, N, K, alpha, beta, st);
+            launch_128(static_cast<const h16*>(A) + (size_t)head * K, B, static_cast<h16*>(C) + (size_t)head * N,
+                       M - head, N, K, alpha, beta, st);
         return true;
     }
     if (!allow_big_lds(gemm_dma, ready32, kDmaLdsBytes)) return false;
@@ -678,7 +707,9 @@ bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, floa
     return true;
 }
 
-enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4, k256regs = 5 };
+// k128: the 128x128 tile through registers (the tile of vv_gemm_fp16_tile_dev); k128dma: that tile fed by copies
+// straight into LDS where K allows, what the automatic choice takes.
+enum TileChoice : int { kAuto = 0, k128 = 1, k64 = 2, k32 = 3, k256 = 4, k256regs = 5, k128dma = 6 };
 
 vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, float alpha,
                  float beta, void* stream, int choice, bool allow_gemv) {
@@ -726,9 +757,10 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         // round on.
         const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128 : (M > 32) ? k64 : k32;
+        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128dma : (M > 32) ? k64 : k32;
     }
     switch (choice) {
+        case k128dma: launch_128(A, B, C, M, N, K, alpha, beta, st); break;
         case k256:
             if (K % (kDmaSlabBytes / 2) == 0 && launch_dma(A, B, C, M, N, K, alpha, beta, st)) break;
             [[fallthrough]];
@@ -756,33 +788,52 @@ void launch_tile_rope(const h16* A, const h16* B, const h16* bias, const float2*
             A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
 }
 
+template <int kTile, int kStages = 2>
+bool launch_dma64_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N,
+                       int K, hipStream_t st) {
+    typedef Dma64Shape<kTile, kStages> Shape;
+    static thread_local int ready = -1;
+    if (!allow_big_lds(gemm_dma64_rope<kTile, kStages>, ready, Shape::kLdsBytes)) return false;
+    gemm_dma64_rope<kTile, kStages><<<dim3(dma64_grid<kTile>(M, N)), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(
+        A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
+    return true;
+}
+
+void launch_128_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N, int K,
+                     hipStream_t st) {
+    if (K % (kDma64SlabBytes / 2) == 0 &&
+        (dma128_alone(M, N) ? launch_dma64_rope<128, 4>(A, B, bias, table, C, M, N, K, st)
+                            : launch_dma64_rope<128, 2>(A, B, bias, table, C, M, N, K, st)))
+        return;
+    launch_tile_rope<128, 128, 2, 2, 64, 2>(A, B, bias, table, C, M, N, K, st);
+}
+
 bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N, int K,
                hipStream_t st, int choice) {
     if (M <= 64 || K <= 0 || K % 8 != 0) return false;
     if (choice == kAuto) {
         const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-        choice = wg256 >= 512 ? k256 : wg128 >= 256 ? k128 : k64;
+        choice = wg256 >= 512 ? k256 : wg128 >= 256 ? k128dma : k64;
     }
     if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
-        static thread_local int ready32 = -1, ready64 = -1;
-        if (K % (kDma64SlabBytes / 2) == 0 && allow_big_lds(gemm_dma64_rope, ready64, kDma64LdsBytes)) {
+        static thread_local int ready32 = -1;
+        if (K % (kDma64SlabBytes / 2) == 0) {
             const int head = dma64_split_rows(M, N);         // the rows gemm() gives to this tile, so the same bits
-            const int rows = head ? head : M;
-            gemm_dma64_rope<<<dim3(dma64_grid(rows, N)), kDmaWaves * kWave, kDma64LdsBytes, st>>>(
-                A, B, bias, table, C, rows, N, K, 1.0f, 0.0f);
-            if (head)
-                launch_tile_rope<128, 128, 2, 2, 64, 2>(A + (size_t)head * K, B, bias, table + (size_t)head * 64,
-                                                        C + (size_t)head * N, M - head, N, K, st);
-            return true;
-        }
-        if (K % (kDma64SlabBytes / 2) != 0 && allow_big_lds(gemm_dma_rope, ready32, kDmaLdsBytes)) {
+            if (launch_dma64_rope<256>(A, B, bias, table, C, head ? head : M, N, K, st)) {
+                if (head)
+                    launch_128_rope(A + (size_t)head * K, B, bias, table + (size_t)head * 64, C + (size_t)head * N,
+                                    M - head, N, K, st);
+                return true;
+            }
+        } else if (allow_big_lds(gemm_dma_rope, ready32, kDmaLdsBytes)) {
             const dim3 grid((unsigned)((N + kDmaTile - 1) / kDmaTile), (unsigned)((M + kDmaTile - 1) / kDmaTile));
             gemm_dma_rope<<<grid, kDmaWaves * kWave, kDmaLdsBytes, st>>>(A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
             return true;
         }
     }
     if (choice == k256 || choice == k256regs) launch_tile_rope<256, 256, 2, 4, 32, 2>(A, B, bias, table, C, M, N, K, st);
+    else if (choice == k128dma) launch_128_rope(A, B, bias, table, C, M, N, K, st);
     else if (choice == k128) launch_tile_rope<128, 128, 2, 2, 64, 2>(A, B, bias, table, C, M, N, K, st);
     else launch_tile_rope<64, 128, 2, 2, 64, 1>(A, B, bias, table, C, M, N, K, st);
     return true;

@@ -181,23 +181,40 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
 //   * The clock is not a constant: under this load the device runs at 1.6-1.8 GHz of its 2.4, and
 //     a loop that wastes fewer cycles is answered with a lower clock. What is left to gain is
 //     energy per product, not cycles.
-// Two stages of 64 KB. Fragments are read one K step ahead; the barrier sits before the last K
-// step of a slab, when every wave has read all of the slab (its last step was read during the
-// step before), so the stage is free for the slab after next, whose eight copies per wave are
-// issued behind that step's MFMAs and have a whole slab of MFMAs to land. Rows must be whole
-// slabs: K % 64 == 0 for FP16. The grid is one-dimensional: dma64_grid() workgroups.
+// Two stages of 64 KB, two K steps of 32 to a slab. Fragments are read one K step ahead; the
+// barrier sits in the last K step of a slab, when every wave has read all of the slab (its last
+// step was read during the step before), so the stage is free for the slab after next, whose
+// eight copies per wave are issued behind that step's MFMAs and have a whole slab of MFMAs to
+// land. Rows must be whole slabs: K % 64 == 0 for FP16. The grid is one-dimensional:
+// dma64_grid() workgroups.
+// The same loop serves a 128x128 tile (four waves of 64 x 64) for shapes and leftovers that do not fill the
+// chip with 256x256 tiles: with two stages (64 KB of LDS) two workgroups share a compute unit, the barrier
+// of one hidden behind the other; with four stages a workgroup that has the unit to itself asks for a slab
+// three slabs ahead (its slabs are 512 matrix-core cycles long, a copy's way from memory takes four times that).
 constexpr int kDma64SlabBytes = 128;
-constexpr int kDma64StageSlots = 2 * kDmaTile * (kDma64SlabBytes / 16);      // 4096 slots: A rows, then B rows
-constexpr size_t kDma64LdsBytes = (size_t)2 * kDma64StageSlots * 16;
-constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 workgroups, one per CU of an XCD
+constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 workgroups
+
+template <int kTile, int kStages = 2>
+struct Dma64Shape {
+    static_assert(kTile == 256 || kTile == 128, "tile sizes with a schedule");
+    static_assert(kStages == 2 || kStages == 4, "a slab's stage is slab % kStages");
+    static constexpr int kWaves = kTile / 32;                     // 2 x 4 or 2 x 2 waves
+    static constexpr int WN = kWaves / 2;
+    static constexpr int TM = kTile / 2 / 16, TN = 4;             // wave tile (kTile / 2) x 64 in 16 x 16 products
+    static constexpr int kStageSlots = 2 * kTile * (kDma64SlabBytes / 16);   // A rows, then B rows
+    static constexpr size_t kLdsBytes = (size_t)kStages * kStageSlots * 16;
+    static constexpr int kLoads = kStageSlots / kWave / kWaves;   // wave-wide copies per wave per slab
+    static_assert(kLoads == 8, "the copy requests of a slab go behind eight MFMAs of its last K step");
+};
+constexpr size_t kDma64LdsBytes = Dma64Shape<256>::kLdsBytes;
 
 // The numbering above for a gy x gx grid of tiles. `whole`: tiles per XCD that come in whole blocks;
 // `run`: the length of an XCD's run of the remaining `rest` tiles.
 struct Dma64Map {
     int gx, gy, fx, fy, whole, run, rest, spare, right;
-    __host__ __device__ Dma64Map(int M, int N) {
-        gx = (N + kDmaTile - 1) / kDmaTile;
-        gy = (M + kDmaTile - 1) / kDmaTile;
+    __host__ __device__ Dma64Map(int M, int N, int tile) {
+        gx = (N + tile - 1) / tile;
+        gy = (M + tile - 1) / tile;
         fx = gx / kSuperN;                                // whole blocks per row of blocks
         fy = gy / kSuperM;
         const int blocks = fx * fy;
@@ -242,61 +259,63 @@ struct Dma64Map {
     }
 };
 
-inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N).grid(); }
+template <int kTile = 256>
+inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N, kTile).grid(); }
 
-// The wave tile is 128 (m) x 64 (n) in TN x TM = 4 x 8 products of 16 x 16 over K steps of 32 (Op::mfma16: the
-// 16x16x32 matrix instructions move a fifth fewer register bytes per product than the 32x32x16 ones, and under the
-// power limit that is speed: 1.7-1.9 against 1.5-1.6 PFLOP/s for the bare instruction streams on random
-// operands). A fragment is 16 rows x 64 bytes: lane l reads slot K step * 4 + l / 16 of row l % 16.
+// The wave tile is TN x TM = 4 x 8 (4 x 4 for the 128x128 tile) products of 16 x 16 over K steps of 32
+// (Op::mfma16: the 16x16x32 matrix instructions move a fifth fewer register bytes per product than the
+// 32x32x16 ones, and under the power limit that is speed: 1.7-1.9 against 1.5-1.6 PFLOP/s for the bare
+// instruction streams on random operands). A fragment is 16 rows x 64 bytes: lane l reads slot
+// K step * 4 + l / 16 of row l % 16.
 //   Op::Acc16                                4-wide accumulator vector
 //   Op::mfma16(u32x4 w, u32x4 x, Acc16 c)    one 16x16 product over a K step
 //   epi(acc, m0, n0, lane)                   register r of lane l: column n0 + off(a) + 4 (l / 16) + r of row
 //                                            m0 + 16 b + l % 16, for acc[a][b]; off(a) = 16 a, or with kPairN
 //                                            16 (a % 2) + 64 (a / 2): tiles a and a + 2 are 64 columns apart
 // The MFMAs of a step run x tile by x tile, so an x fragment is dead after four MFMAs and the next step's
-// takes its registers at once: only the four w fragments and two of the eight x fragments are held twice.
-template <typename Op, bool kPairN = false, typename Epi>
+// takes its registers at once: only the four w fragments and the last two x fragments are held twice.
+template <typename Op, int kTile = 256, bool kPairN = false, int kStages = 2, typename Epi>
 __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
                                            int row_bytes, const Epi& epi) {
     typedef typename Op::Acc16 Acc;
+    typedef Dma64Shape<kTile, kStages> Shape;
     constexpr int kSlabChunks = kDma64SlabBytes / 16;     // 8
-    constexpr int WN = 4, TM = 8, TN = 4;                 // 2 x 4 waves, wave tile 128 (m) x 64 (n)
-    constexpr int kLoads = kDma64StageSlots / kWave / kDmaWaves;   // wave-wide copies per wave per slab: 8
-    static_assert(kLoads == 8, "the copy requests of a slab go behind eight MFMAs of its last K step");
+    constexpr int WN = Shape::WN, TM = Shape::TM, TN = Shape::TN, kLoads = Shape::kLoads;
+    constexpr int kStageSlots = Shape::kStageSlots;
     extern __shared__ u32x4 dma_lds[];
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const Dma64Map map(M, N);
+    const Dma64Map map(M, N, kTile);
     int tile_m, tile_n;
     if (!map.tile((int)blockIdx.x, tile_m, tile_n)) return;      // the whole workgroup, before any barrier
-    const int m_blk = tile_m * kDmaTile, n_blk = tile_n * kDmaTile;
+    const int m_blk = tile_m * kTile, n_blk = tile_n * kTile;
     const int nslabs = row_bytes / kDma64SlabBytes;
     const uint32_t lds0 =
         (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
 
-    // Copy i of this wave fills slots (wave + 8i) * 64 .. + 63 of a stage: 8 rows x 8 slots, a whole line per
-    // row. The lane owns (row, physical slot) and fetches the logical slot that the swizzle maps there.
+    // Copy i of this wave fills slots (wave + waves * i) * 64 .. + 63 of a stage: 8 rows x 8 slots, a whole
+    // line per row. The lane owns (row, physical slot) and fetches the logical slot that the swizzle maps there.
     const char* src[kLoads];
     uint32_t dst[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-        const int slot0 = (wave + kDmaWaves * i) * kWave;
+        const int slot0 = (wave + Shape::kWaves * i) * kWave;
         const int p = slot0 + lane;
         const int row = p / kSlabChunks, phys = p % kSlabChunks;
         const int logical = swz<64>(row, phys);
-        const bool is_b = row >= kDmaTile;
-        const int r = is_b ? row - kDmaTile : row;
+        const bool is_b = row >= kTile;
+        const int r = is_b ? row - kTile : row;
         const char* base = is_b ? static_cast<const char*>(B) + (size_t)min(n_blk + r, N - 1) * row_bytes
                                 : static_cast<const char*>(A) + (size_t)min(m_blk + r, M - 1) * row_bytes;
         src[i] = base + logical * 16;
         dst[i] = lds0 + (uint32_t)slot0 * 16u;
     }
-    auto request = [&](int slab, int i) {        // slab -> stage slab % 2; past the end: the last slab again
+    auto request = [&](int slab, int i) {        // slab -> stage slab % kStages; past the end: the last slab again
         const size_t adv = (size_t)min(slab, nslabs - 1) * kDma64SlabBytes;
-        const uint32_t stage = (uint32_t)(slab & 1) * (kDma64StageSlots * 16u);
+        const uint32_t stage = (uint32_t)(slab & (kStages - 1)) * (kStageSlots * 16u);
         lds_dma16(src[i] + adv, dst[i] + stage);
     };
 
@@ -315,7 +334,7 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
         f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 4 + fquarter);
     const int fa_base = wm * TM * 16 * kSlabChunks;
     const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 16;      // first column of tile a = 0
-    const int fb_base = kDmaTile * kSlabChunks + wave_n0 * kSlabChunks;
+    const int fb_base = kTile * kSlabChunks + wave_n0 * kSlabChunks;
     auto w_off = [](int a) { return (kPairN ? (a & 1) * 16 + (a >> 1) * 64 : a * 16) * kSlabChunks; };
 
     // w: the K step in hand and the next. x: one set, refilled in place, except the last two tiles of a step,
@@ -325,55 +344,71 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     u32x4 fw[2][TN], fx[kSingle], fxl[2][TM - kSingle];
     auto read_w = [&](auto set_c, int slab, int step, int a) {
         constexpr int set = decltype(set_c)::value;
-        fw[set][a] = dma_lds[(slab & 1) * kDma64StageSlots + fb_base + w_off(a) + f_idx[step]];
+        fw[set][a] = dma_lds[(slab & (kStages - 1)) * kStageSlots + fb_base + w_off(a) + f_idx[step]];
     };
     auto read_x = [&](auto set_c, int slab, int step, int b) {
         constexpr int set = decltype(set_c)::value;
-        const u32x4 v = dma_lds[(slab & 1) * kDma64StageSlots + fa_base + b * 16 * kSlabChunks + f_idx[step]];
+        const u32x4 v = dma_lds[(slab & (kStages - 1)) * kStageSlots + fa_base + b * 16 * kSlabChunks + f_idx[step]];
         if (b < kSingle) fx[b] = v;
         else fxl[set][b - kSingle] = v;
     };
-    // One K step: 32 MFMAs, x tile by x tile. Reads and copy requests go behind MFMAs, one each; the next
-    // step's x fragment b < 6 can go anywhere behind the last MFMA of x tile b (it takes that fragment's
-    // registers). Step 0 reads step 1 of the same slab. Step 1 first issues eight MFMAs; behind the barrier
-    // that follows every wave has read all of this slab and the next slab has landed (this wave's copies;
-    // the barrier adds the others'): then come the reads of the next slab's step 0 and the eight copy
-    // requests of the slab after next into the stage just freed. The last read of a step is eight MFMAs
-    // from its end.
+    // One K step: TM x 4 MFMAs, x tile by x tile. Reads and copy requests go behind MFMAs, one each; the
+    // next step's x fragment b < TM - 2 can go anywhere behind the last MFMA of x tile b (it takes that
+    // fragment's registers). Step 0 reads step 1 of the same slab. In step 1, behind the barrier, every wave
+    // has read all of this slab and the next slab has landed (this wave's copies; the barrier adds the
+    // others'): then come the reads of the next slab's step 0 and the eight copy requests of the slab after
+    // next into the stage just freed. The last read of a step is eight MFMAs from its end. With 32 MFMAs to
+    // a step, step 1 issues eight before the barrier, so that the last read of step 0 is back when the wave
+    // gets there; with 16 the barrier comes first and the other workgroup of the compute unit fills the wait.
     auto k_step = [&](auto cur_c, auto nxt_c, int slab, auto step_c) {
         constexpr int set = decltype(cur_c)::value;
         constexpr int step = decltype(step_c)::value;
         constexpr int nstep = step ^ 1;
+        constexpr int kBefore = TM == 8 ? 2 : 0;                   // x tiles of step 1 ahead of the barrier
         const int nslab = slab + step;
 #pragma unroll
         for (int b = 0; b < TM; ++b) {
 #pragma unroll
             for (int a = 0; a < TN; ++a) {
-                if (step == 1 && b == 2 && a == 0) {
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                if (step == 1 && b == kBefore && a == 0) {
+                    // this wave's copies of the next slab are in: only those of the slabs behind it may still fly
+                    if constexpr (kStages == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
                     __syncthreads();
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 acc[a][b] = Op::mfma16(fw[set][a], b < kSingle ? fx[b] : fxl[set][b - kSingle], acc[a][b]);
                 __builtin_amdgcn_sched_barrier(0);
-                const int slot = (b - 2 * step) * TN + a;          // step 1: counted from the barrier
-                if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
-                else if (slot == 1) read_x(nxt_c, nslab, nstep, step == 0 ? 6 : 0);
-                else if (slot == 2) read_w(nxt_c, nslab, nstep, 1);
-                else if (slot == 3) read_x(nxt_c, nslab, nstep, step == 0 ? 0 : 2);
-                else if (slot == 4) read_w(nxt_c, nslab, nstep, 2);
-                else if (slot == 5) read_w(nxt_c, nslab, nstep, 3);
-                else if (slot == 6) read_x(nxt_c, nslab, nstep, step == 0 ? 7 : 1);
-                else if (slot == 7) read_x(nxt_c, nslab, nstep, step == 0 ? 1 : 3);
-                else if (slot == 8 && step == 1) read_x(nxt_c, nslab, nstep, 6);
-                else if (slot == 9 && step == 1) read_x(nxt_c, nslab, nstep, 7);
-                else if (slot == 11) read_x(nxt_c, nslab, nstep, step == 0 ? 2 : 4);
-                else if (slot == 15) read_x(nxt_c, nslab, nstep, step == 0 ? 3 : 5);
-                else if (slot == 19 && step == 0) read_x(nxt_c, nslab, nstep, 4);
-                else if (slot == 23 && step == 0) read_x(nxt_c, nslab, nstep, 5);
-                else if constexpr (step == 1) {
-                    const int i = slot == 10 ? 0 : slot >= 12 && slot <= 14 ? slot - 11 : slot >= 16 && slot <= 19 ? slot - 12 : -1;
-                    if (i >= 0) request(slab + 2, i);
+                const int slot = (b - kBefore * step) * TN + a;    // step 1: counted from the barrier
+                if constexpr (TM == 8) {
+                    if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
+                    else if (slot == 1) read_x(nxt_c, nslab, nstep, step == 0 ? 6 : 0);
+                    else if (slot == 2) read_w(nxt_c, nslab, nstep, 1);
+                    else if (slot == 3) read_x(nxt_c, nslab, nstep, step == 0 ? 0 : 2);
+                    else if (slot == 4) read_w(nxt_c, nslab, nstep, 2);
+                    else if (slot == 5) read_w(nxt_c, nslab, nstep, 3);
+                    else if (slot == 6) read_x(nxt_c, nslab, nstep, step == 0 ? 7 : 1);
+                    else if (slot == 7) read_x(nxt_c, nslab, nstep, step == 0 ? 1 : 3);
+                    else if (slot == 8 && step == 1) read_x(nxt_c, nslab, nstep, 6);
+                    else if (slot == 9 && step == 1) read_x(nxt_c, nslab, nstep, 7);
+                    else if (slot == 11) read_x(nxt_c, nslab, nstep, step == 0 ? 2 : 4);
+                    else if (slot == 15) read_x(nxt_c, nslab, nstep, step == 0 ? 3 : 5);
+                    else if (slot == 19 && step == 0) read_x(nxt_c, nslab, nstep, 4);
+                    else if (slot == 23 && step == 0) read_x(nxt_c, nslab, nstep, 5);
+                    else if constexpr (step == 1) {
+                        const int i = slot == 10 ? 0 : slot >= 12 && slot <= 14 ? slot - 11 : slot >= 16 && slot <= 19 ? slot - 12 : -1;
+                        if (i >= 0) request(slab + kStages, i);
+                    }
+                } else {
+                    if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
+                    else if (slot == 1) read_w(nxt_c, nslab, nstep, 1);
+                    else if (slot == 2) read_w(nxt_c, nslab, nstep, 2);
+                    else if (slot == 3) read_x(nxt_c, nslab, nstep, 0);
+                    else if (slot == 4) read_w(nxt_c, nslab, nstep, 3);
+                    else if (slot == 5) read_x(nxt_c, nslab, nstep, 2);
+                    else if (slot == 6) read_x(nxt_c, nslab, nstep, 3);
+                    else if (slot == 7) read_x(nxt_c, nslab, nstep, 1);
+                    else if constexpr (step == 1) request(slab + kStages, slot - 8);
                 }
             }
         }
@@ -381,10 +416,12 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     };
 
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) request(0, i);
+    for (int s = 0; s < kStages; ++s)
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) request(1, i);
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // slab 0; slab 1 is waited for at the first barrier
+        for (int i = 0; i < kLoads; ++i) request(s, i);
+    // slab 0; slab 1 is waited for at the first barrier
+    if constexpr (kStages == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
     __syncthreads();
 #pragma unroll
     for (int a = 0; a < TN; ++a) read_w(Const<0>{}, 0, 0, a);
