@@ -33,6 +33,15 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_byte_ad
                  : "memory", "m0");
 }
 
+// The same copy with the address as a wave-uniform base plus a 32-bit byte offset per lane: the base advances
+// in scalar registers, so a loop spends no vector instruction on the addresses.
+__device__ __forceinline__ void lds_dma16_at(const void* base, uint32_t lane_offset, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_byte_addr), "v"(lane_offset), "s"(base)
+                 : "memory", "m0");
+}
+
 // kPairN: a wave's two N tiles are 64 columns apart instead of adjacent - wave wn takes columns
 // 128 (wn / 2) + 32 (wn % 2) + {0, 64} of the block - so that an epilogue finds columns n and n + 64
 // (the rotate-half pair of a 128-wide head) in the same lane and register of acc[0] and acc[1]. The
@@ -297,26 +306,25 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
         (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
 
     // Copy i of this wave fills slots (wave + waves * i) * 64 .. + 63 of a stage: 8 rows x 8 slots, a whole
-    // line per row. The lane owns (row, physical slot) and fetches the logical slot that the swizzle maps there.
-    const char* src[kLoads];
-    uint32_t dst[kLoads];
+    // line per row; copies 0 .. 3 are A rows, 4 .. 7 B rows. The lane owns (row, physical slot) and fetches the
+    // logical slot that the swizzle maps there: a byte offset from the tile's first row, the same for every slab.
+    const char* a_tile = static_cast<const char*>(A) + (size_t)m_blk * row_bytes;
+    const char* b_tile = static_cast<const char*>(B) + (size_t)n_blk * row_bytes;
+    uint32_t src[kLoads], dst[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int slot0 = (wave + Shape::kWaves * i) * kWave;
         const int p = slot0 + lane;
         const int row = p / kSlabChunks, phys = p % kSlabChunks;
         const int logical = swz<64>(row, phys);
-        const bool is_b = row >= kTile;
-        const int r = is_b ? row - kTile : row;
-        const char* base = is_b ? static_cast<const char*>(B) + (size_t)min(n_blk + r, N - 1) * row_bytes
-                                : static_cast<const char*>(A) + (size_t)min(m_blk + r, M - 1) * row_bytes;
-        src[i] = base + logical * 16;
+        const int r = i < kLoads / 2 ? min(row, M - 1 - m_blk) : min(row - kTile, N - 1 - n_blk);
+        src[i] = (uint32_t)r * (uint32_t)row_bytes + (uint32_t)logical * 16u;
         dst[i] = lds0 + (uint32_t)slot0 * 16u;
     }
     auto request = [&](int slab, int i) {        // slab -> stage slab % kStages; past the end: the last slab again
         const size_t adv = (size_t)min(slab, nslabs - 1) * kDma64SlabBytes;
         const uint32_t stage = (uint32_t)(slab & (kStages - 1)) * (kStageSlots * 16u);
-        lds_dma16(src[i] + adv, dst[i] + stage);
+        lds_dma16_at((i < kLoads / 2 ? a_tile : b_tile) + adv, src[i], dst[i] + stage);
     };
 
     Acc acc[TN][TM];
@@ -352,12 +360,13 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
         if (b < kSingle) fx[b] = v;
         else fxl[set][b - kSingle] = v;
     };
-    // One K step: TM x 4 MFMAs, x tile by x tile. Reads and copy requests go behind MFMAs, one each; the
+    // One K step: TM x 4 MFMAs, x tile by x tile. Reads and copy requests go behind MFMAs; the
     // next step's x fragment b < TM - 2 can go anywhere behind the last MFMA of x tile b (it takes that
     // fragment's registers). Step 0 reads step 1 of the same slab. In step 1, behind the barrier, every wave
     // has read all of this slab and the next slab has landed (this wave's copies; the barrier adds the
-    // others'): then come the reads of the next slab's step 0 and the eight copy requests of the slab after
-    // next into the stage just freed. The last read of a step is eight MFMAs from its end. With 32 MFMAs to
+    // others'): then come the eight copy requests of the slab after next into the stage just freed, behind
+    // the first eight MFMAs, and with them the reads of the next slab's step 0. The last read of a step is
+    // eight MFMAs from its end. With 32 MFMAs to
     // a step, step 1 issues eight before the barrier, so that the last read of step 0 is back when the wave
     // gets there; with 16 the barrier comes first and the other workgroup of the compute unit fills the wait.
     auto k_step = [&](auto cur_c, auto nxt_c, int slab, auto step_c) {
@@ -380,6 +389,10 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                 acc[a][b] = Op::mfma16(fw[set][a], b < kSingle ? fx[b] : fxl[set][b - kSingle], acc[a][b]);
                 __builtin_amdgcn_sched_barrier(0);
                 const int slot = (b - kBefore * step) * TN + a;    // step 1: counted from the barrier
+                if constexpr (step == 1) {
+                    // the copies first: their way from memory is longer than the slab they have to make it in
+                    if (slot >= 0 && slot < kLoads) request(slab + kStages, slot);
+                }
                 if constexpr (TM == 8) {
                     if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
                     else if (slot == 1) read_x(nxt_c, nslab, nstep, step == 0 ? 6 : 0);
@@ -395,10 +408,6 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                     else if (slot == 15) read_x(nxt_c, nslab, nstep, step == 0 ? 3 : 5);
                     else if (slot == 19 && step == 0) read_x(nxt_c, nslab, nstep, 4);
                     else if (slot == 23 && step == 0) read_x(nxt_c, nslab, nstep, 5);
-                    else if constexpr (step == 1) {
-                        const int i = slot == 10 ? 0 : slot >= 12 && slot <= 14 ? slot - 11 : slot >= 16 && slot <= 19 ? slot - 12 : -1;
-                        if (i >= 0) request(slab + kStages, i);
-                    }
                 } else {
                     if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
                     else if (slot == 1) read_w(nxt_c, nslab, nstep, 1);
@@ -408,7 +417,6 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                     else if (slot == 5) read_x(nxt_c, nslab, nstep, 2);
                     else if (slot == 6) read_x(nxt_c, nslab, nstep, 3);
                     else if (slot == 7) read_x(nxt_c, nslab, nstep, 1);
-                    else if constexpr (step == 1) request(slab + kStages, slot - 8);
                 }
             }
         }
