@@ -54,7 +54,7 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           # block at all (7 tile columns), whole blocks only
           (2048, 18944, 64), (2300, 16400, 128), (19000, 1792, 64), (4096, 8192, 64),
           # the 128x128 tile fed the same way: 17 x 17, 9 x 32 and 113 x 4 tiles
-          (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128)]
+          (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128), (70, 33000, 64)]      # ... and one row of 258 tiles
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
