@@ -93,16 +93,17 @@ struct F16Op {
 };
 
 // A wave's 4 x TM accumulator tiles of 16 x 16 (mfma_dma64) to C: register r of lane l holds column
-// n0 + 16 a + 4 (l / 16) + r of row m0 + 16 b + l % 16 of acc[a][b].
+// n0 + 16 a + 4 (l / 16) + r of row m0 + 16 b + l % 16 of acc[a][b]. C's rows are ldc halves apart (the launch
+// may cover a range of C's columns).
 template <int TM>
-__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[4][TM], h16* __restrict__ C, int M, int N, int m0,
-                                             int n0, int lane, float alpha, float beta, int vec_store) {
+__device__ __forceinline__ void store_tile16(const f32x4 (&acc)[4][TM], h16* __restrict__ C, int M, int N, int ldc,
+                                             int m0, int n0, int lane, float alpha, float beta, int vec_store) {
     typedef h16 h16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int b = 0; b < TM; ++b) {
         const int m = m0 + b * 16 + (lane & 15);
         if (m >= M) continue;
-        h16* crow = C + (size_t)m * N;
+        h16* crow = C + (size_t)m * ldc;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int n = n0 + a * 16 + 4 * (lane >> 4);
@@ -180,10 +181,10 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma(
 template <int kTile, int kStages>
 __global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma64(
     const h16* __restrict__ A, const h16* __restrict__ B, h16* __restrict__ C, int M, int N,
-    int K, float alpha, float beta, int vec_store) {
+    int K, int ldc, float alpha, float beta, int vec_store) {
     constexpr int TM = Dma64Shape<kTile>::TM;
     auto epilogue = [=](const f32x4 (&acc)[4][TM], int m0, int n0, int lane) {
-        store_tile16<TM>(acc, C, M, N, m0, n0, lane, alpha, beta, vec_store);
+        store_tile16<TM>(acc, C, M, N, ldc, m0, n0, lane, alpha, beta, vec_store);
     };
     mfma_dma64<F16Op, kTile, false, kStages>(A, B, M, N, K * 2, epilogue);
 }
@@ -250,7 +251,8 @@ __device__ __forceinline__ void store_tile_rope(const f32x16 (&acc)[2][TM], h16*
 template <int TM>
 __device__ __forceinline__ void store_tile16_rope(const f32x4 (&acc)[4][TM], h16* __restrict__ C,
                                                   const h16* __restrict__ bias, const float2* __restrict__ table,
-                                                  int M, int N, int m0, int n0, int lane, float alpha, float beta) {
+                                                  int M, int N, int ldc, int m0, int n0, int lane, float alpha,
+                                                  float beta) {
     typedef h16 h16x4 __attribute__((ext_vector_type(4)));
     if (n0 >= N) return;                         // whole heads: the wave's 32 + 32 columns are all in or all out
     const int pair0 = n0 & 127;                  // 0 or 32: the first rotation pair of tile 0
@@ -258,7 +260,7 @@ __device__ __forceinline__ void store_tile16_rope(const f32x4 (&acc)[4][TM], h16
     for (int b = 0; b < TM; ++b) {
         const int m = m0 + b * 16 + (lane & 15);
         if (m >= M) continue;
-        h16* crow = C + (size_t)m * N;
+        h16* crow = C + (size_t)m * ldc;
         const float2* trow = table + (size_t)m * 64;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
@@ -320,10 +322,10 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void gemm_dma_rope(
 template <int kTile, int kStages>
 __global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma64_rope(
     const h16* __restrict__ A, const h16* __restrict__ B, const h16* __restrict__ bias,
-    const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, float alpha, float beta) {
+    const float2* __restrict__ table, h16* __restrict__ C, int M, int N, int K, int ldc, float alpha, float beta) {
     constexpr int TM = Dma64Shape<kTile>::TM;
     auto epilogue = [=](const f32x4 (&acc)[4][TM], int m0, int n0, int lane) {
-        store_tile16_rope<TM>(acc, C, bias, table, M, N, m0, n0, lane, alpha, beta);
+        store_tile16_rope<TM>(acc, C, bias, table, M, N, ldc, m0, n0, lane, alpha, beta);
     };
     mfma_dma64<F16Op, kTile, true, kStages>(A, B, M, N, K * 2, epilogue);
 }
@@ -638,39 +640,52 @@ bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes) {
     return true;
 }
 
-// Rows of the 256x256 tiles' launch when the last round of workgroups would run mostly empty. Every XCD takes
-// an eighth of the tiles, 32 at a time, so a launch costs ceil(tiles / 8 / 32) rounds; 57 x 14 tiles (14449 rows
-// into 3584 columns) are 3.1 rounds and cost four. The rows that spill into a round of their own go to the
-// 128x128 tile instead, whose rounds are short (a third of a 256x256 round, measured at K = 3584 and 18944;
-// priced at 0.35): 54 rows of tiles in three rounds, the other 625 rows in one short one. 0: no split pays
-// (at least a twentieth of the time).
-int dma64_split_rows(int M, int N) {
+// The part of C that the 256x256 tiles' launch covers when its last round of workgroups would run mostly empty.
+// Every XCD takes an eighth of the tiles, 32 at a time, so a launch costs ceil(tiles / 8 / 32) rounds: 57 x 14
+// tiles (14449 rows into 3584 columns) are 3.1 rounds and cost four, 8 x 74 (a 2048-row chunk into 18944
+// columns) are 2.3 and cost three. The rows - or the columns - that spill into a round of their own go to the
+// 128x128 tile instead, whose rounds are short: 0.42 of a 256x256 round when no compute unit gets a second
+// workgroup (at most 256 tiles, four stages), 0.6 per 512 tiles otherwise (measured at K = 3584 and 18944).
+// 54 rows of tiles in three rounds and the other 625 rows in one short one; 64 columns of tiles in two rounds
+// and the other 2560 columns in one short one. {0, 0}: no split pays (at least a twentieth of the time).
+struct Dma64Split { int rows, cols; };
+
+Dma64Split dma64_split(int M, int N) {
     const int gx = (N + kDmaTile - 1) / kDmaTile, gy = (M + kDmaTile - 1) / kDmaTile;
     auto rounds = [](long tiles) { return (double)(((tiles + 7) / 8 + 31) / 32); };
-    const double whole = rounds((long)gx * gy);
-    double best = whole * 0.95;
-    int best_rows = 0;
+    auto rest = [](int m, int n) {
+        const long small = (long)((m + 127) / 128) * ((n + 127) / 128);
+        return small <= 256 ? 0.42 : 0.6 * (double)((small + 511) / 512);
+    };
+    double best = rounds((long)gx * gy) * 0.95;
+    Dma64Split split = {0, 0};
     for (int r = gy - 1; r >= 1 && r >= gy - 16; --r) {
-        const int tail = M - r * kDmaTile;
-        const long small = (long)((tail + 127) / 128) * ((N + 127) / 128);
-        const double cost = rounds((long)gx * r) + 0.35 * (double)((small + 255) / 256);
+        const double cost = rounds((long)gx * r) + rest(M - r * kDmaTile, N);
         if (cost < best) {
             best = cost;
-            best_rows = r * kDmaTile;
+            split = {r * kDmaTile, 0};
         }
     }
-    return best_rows;
+    for (int c = gx - 1; c >= 1 && c >= gx - 16; --c) {
+        const double cost = rounds((long)gy * c) + rest(M, N - c * kDmaTile);
+        if (cost < best) {
+            best = cost;
+            split = {0, c * kDmaTile};
+        }
+    }
+    return split;
 }
 
+// C's rows are ldc halves apart: the launch may cover a range of C's columns (B's rows).
 template <int kTile, int kStages = 2>
-bool launch_dma64(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+bool launch_dma64(const void* A, const void* B, void* C, int M, int N, int K, int ldc, float alpha, float beta,
                   hipStream_t st) {
     typedef Dma64Shape<kTile, kStages> Shape;
     static thread_local int ready = -1;
     if (!allow_big_lds(gemm_dma64<kTile, kStages>, ready, Shape::kLdsBytes)) return false;
-    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    const int vec = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
     gemm_dma64<kTile, kStages><<<dim3(dma64_grid<kTile>(M, N)), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(
-        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, alpha, beta, vec);
+        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<h16*>(C), M, N, K, ldc, alpha, beta, vec);
     return true;
 }
 
@@ -678,12 +693,15 @@ bool launch_dma64(const void* A, const void* B, void* C, int M, int N, int K, fl
 // compute unit gets a second workgroup to fill its waits, two otherwise), through registers otherwise.
 bool dma128_alone(int M, int N) { return (long)((M + 127) / 128) * ((N + 127) / 128) <= 256; }
 
+bool launch_dma128(const void* A, const void* B, void* C, int M, int N, int K, int ldc, float alpha, float beta,
+                   hipStream_t st) {
+    return dma128_alone(M, N) ? launch_dma64<128, 4>(A, B, C, M, N, K, ldc, alpha, beta, st)
+                              : launch_dma64<128, 2>(A, B, C, M, N, K, ldc, alpha, beta, st);
+}
+
 void launch_128(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
                 hipStream_t st) {
-    if (K % (kDma64SlabBytes / 2) == 0 &&
-        (dma128_alone(M, N) ? launch_dma64<128, 4>(A, B, C, M, N, K, alpha, beta, st)
-                            : launch_dma64<128, 2>(A, B, C, M, N, K, alpha, beta, st)))
-        return;
+    if (K % (kDma64SlabBytes / 2) == 0 && launch_dma128(A, B, C, M, N, K, N, alpha, beta, st)) return;
     launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st);
 }
 
@@ -692,11 +710,16 @@ bool launch_dma(const void* A, const void* B, void* C, int M, int N, int K, floa
     static thread_local int ready32 = -1;
     const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
     if (K % (kDma64SlabBytes / 2) == 0) {
-        const int head = dma64_split_rows(M, N);
-        if (!launch_dma64<256>(A, B, C, head ? head : M, N, K, alpha, beta, st)) return false;
-        if (head)
-            launch_128(static_cast<const h16*>(A) + (size_t)head * K, B, static_cast<h16*>(C) + (size_t)head * N,
-                       M - head, N, K, alpha, beta, st);
+        const h16* a = static_cast<const h16*>(A);
+        const h16* b = static_cast<const h16*>(B);
+        h16* c = static_cast<h16*>(C);
+        const Dma64Split sp = dma64_split(M, N);
+        // the 128x128 part first: should its launch be refused, the 256x256 tiles take everything
+        if (sp.cols && launch_dma128(a, b + (size_t)sp.cols * K, c + sp.cols, M, N - sp.cols, K, N, alpha, beta, st))
+            return launch_dma64<256>(a, b, c, M, sp.cols, K, N, alpha, beta, st) ||
+                   launch_dma64<256>(a, b, c, M, N, K, N, alpha, beta, st);
+        if (!launch_dma64<256>(a, b, c, sp.rows ? sp.rows : M, N, K, N, alpha, beta, st)) return false;
+        if (sp.rows) launch_128(a + (size_t)sp.rows * K, b, c + (size_t)sp.rows * N, M - sp.rows, N, K, alpha, beta, st);
         return true;
     }
     if (!allow_big_lds(gemm_dma, ready32, kDmaLdsBytes)) return false;
@@ -790,21 +813,24 @@ void launch_tile_rope(const h16* A, const h16* B, const h16* bias, const float2*
 
 template <int kTile, int kStages = 2>
 bool launch_dma64_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N,
-                       int K, hipStream_t st) {
+                       int K, int ldc, hipStream_t st) {
     typedef Dma64Shape<kTile, kStages> Shape;
     static thread_local int ready = -1;
     if (!allow_big_lds(gemm_dma64_rope<kTile, kStages>, ready, Shape::kLdsBytes)) return false;
     gemm_dma64_rope<kTile, kStages><<<dim3(dma64_grid<kTile>(M, N)), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(
-        A, B, bias, table, C, M, N, K, 1.0f, 0.0f);
+        A, B, bias, table, C, M, N, K, ldc, 1.0f, 0.0f);
     return true;
+}
+
+bool launch_dma128_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N,
+                        int K, int ldc, hipStream_t st) {
+    return dma128_alone(M, N) ? launch_dma64_rope<128, 4>(A, B, bias, table, C, M, N, K, ldc, st)
+                              : launch_dma64_rope<128, 2>(A, B, bias, table, C, M, N, K, ldc, st);
 }
 
 void launch_128_rope(const h16* A, const h16* B, const h16* bias, const float2* table, h16* C, int M, int N, int K,
                      hipStream_t st) {
-    if (K % (kDma64SlabBytes / 2) == 0 &&
-        (dma128_alone(M, N) ? launch_dma64_rope<128, 4>(A, B, bias, table, C, M, N, K, st)
-                            : launch_dma64_rope<128, 2>(A, B, bias, table, C, M, N, K, st)))
-        return;
+    if (K % (kDma64SlabBytes / 2) == 0 && launch_dma128_rope(A, B, bias, table, C, M, N, K, N, st)) return;
     launch_tile_rope<128, 128, 2, 2, 64, 2>(A, B, bias, table, C, M, N, K, st);
 }
 
@@ -819,11 +845,16 @@ bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table,
     if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
         static thread_local int ready32 = -1;
         if (K % (kDma64SlabBytes / 2) == 0) {
-            const int head = dma64_split_rows(M, N);         // the rows gemm() gives to this tile, so the same bits
-            if (launch_dma64_rope<256>(A, B, bias, table, C, head ? head : M, N, K, st)) {
-                if (head)
-                    launch_128_rope(A + (size_t)head * K, B, bias, table + (size_t)head * 64, C + (size_t)head * N,
-                                    M - head, N, K, st);
+            const Dma64Split sp = dma64_split(M, N);         // the split of gemm(), so the same bits
+            if (sp.cols && launch_dma128_rope(A, B + (size_t)sp.cols * K, bias ? bias + sp.cols : nullptr, table,
+                                              C + sp.cols, M, N - sp.cols, K, N, st)) {
+                if (launch_dma64_rope<256>(A, B, bias, table, C, M, sp.cols, K, N, st) ||
+                    launch_dma64_rope<256>(A, B, bias, table, C, M, N, K, N, st))
+                    return true;
+            } else if (launch_dma64_rope<256>(A, B, bias, table, C, sp.rows ? sp.rows : M, N, K, N, st)) {
+                if (sp.rows)
+                    launch_128_rope(A + (size_t)sp.rows * K, B, bias, table + (size_t)sp.rows * 64,
+                                    C + (size_t)sp.rows * N, M - sp.rows, N, K, st);
                 return true;
             }
         } else if (allow_big_lds(gemm_dma_rope, ready32, kDmaLdsBytes)) {
