@@ -361,11 +361,12 @@ def layer_leg(torch, dev, T: int, st: int, fp16_only: bool = False) -> dict:
         per.sort()
         return per[len(per) // 2]
 
-    out = {"gemm": {}, "gemv": {}}
+    # "gemm_chunk": the same projections at 2048 rows, the reference's prefill chunk (decoder.c:1147-1174)
+    out = {"gemm": {}, "gemm_chunk": {}, "gemv": {}}
     shapes = (("q_o_proj", H, H), ("kv_proj", NK * HD, H), ("gate_up_proj", I_FF, H), ("down_proj", H, I_FF))
     for name, n, k in shapes:
         w = torch.randn(n, k, dtype=torch.float16, device="cuda") * k ** -0.5
-        for m, key in ((T, "gemm"), (1, "gemv")):
+        for m, key in ((T, "gemm"), (2048, "gemm_chunk"), (1, "gemv")):
             a = torch.randn(m, k, dtype=torch.float16, device="cuda")
             c = torch.empty(m, n, dtype=torch.float16, device="cuda")
             sec = timed(lambda: dev.vv_gemm_fp16_dev(a.data_ptr(), w.data_ptr(), c.data_ptr(), m, n, k,
@@ -1243,7 +1244,7 @@ def main() -> int:
     if args.layer or args.layer_fp16:
         fp16_only = not args.layer
         layer = layer_leg(torch, dev, T, st, fp16_only)
-        for name, d in layer["gemm"].items():
+        for name, d in list(layer["gemm"].items()) + list(layer.get("gemm_chunk", {}).items()):
             log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
                 f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         for name, d in layer["gemv"].items():

@@ -54,7 +54,9 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           # block at all (7 tile columns), whole blocks only
           (2048, 18944, 64), (2300, 16400, 128), (19000, 1792, 64), (4096, 8192, 64),
           # the 128x128 tile fed the same way: 17 x 17, 9 x 32 and 113 x 4 tiles
-          (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128), (70, 33000, 64)]      # ... and one row of 258 tiles
+          (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128), (70, 33000, 64),      # ... and one row of 258 tiles
+          # the 64x64 tile fed the same way: 256 tiles or fewer (eight stages), more (four), ragged, one slab
+          (2048, 512, 3584), (285, 3584, 3584), (130, 200, 64), (1000, 1100, 192), (65, 64, 128)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -69,10 +71,10 @@ def test_gemm_against_oracle_and_tile(M, N, K):
     d_t = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     tile = run(dev.vv_gemm_fp16_tile_dev, d_a, d_b, d_t, M, N, K)
     check(tile, ref, mag, f"tile {M}x{N}x{K}")
-    big = K % 64 == 0 and (-(-M // 256) * -(-N // 256) >= 512 or (M > 64 and -(-M // 128) * -(-N // 128) >= 256))
+    big = K % 64 == 0 and M > 64
     if big:
-        # the tiles fed in 128-byte slabs (the choice from 256 tiles of 128x128 on, K % 64 == 0) multiply with the
-        # 16x16x32 instructions, which add 32 products at a time where the other tiles add 16: same sums, another
+        # the tiles fed in 128-byte slabs (the choice above 64 rows when K % 64 == 0) multiply with the 16x16x32
+        # instructions, which add 32 products at a time where the other tiles add 16: same sums, another
         # rounding of the FP32 partials
         diff = np.abs(oracle.widen(got) - oracle.widen(tile))
         assert np.all(diff <= 2.0 ** -9 * mag + 2.0 ** -14), "tile shapes must agree to FP32 summation order"

@@ -72,7 +72,7 @@ def fused(d_a, d_w, d_bias, M, heads, K, table):
 # through registers), ragged edges in both directions, an odd head count, and row counts up to 64, which
 # run the two steps one after the other.
 SHAPES = [(65, 1, 64), (100, 4, 3584), (130, 3, 200), (257, 28, 512), (2048, 28, 256), (2048, 4, 3584),
-          (4100, 64, 72), (4097, 64, 64), (4100, 63, 96), (4100, 63, 192), (4097, 64, 128), (2048, 148, 64), (19000, 14, 64), (2100, 17, 192), (14449, 4, 128), (1, 28, 3584), (29, 4, 3584), (64, 28, 512), (16, 2, 40)]
+          (4100, 64, 72), (4097, 64, 64), (4100, 63, 96), (4100, 63, 192), (4097, 64, 128), (2048, 148, 64), (19000, 14, 64), (2100, 17, 192), (14449, 4, 128), (2048, 4, 3584), (285, 28, 512), (130, 2, 64), (1, 28, 3584), (29, 4, 3584), (64, 28, 512), (16, 2, 40)]
 
 
 @pytest.mark.parametrize("M,heads,K", SHAPES)

@@ -699,6 +699,17 @@ bool launch_dma128(const void* A, const void* B, void* C, int M, int N, int K, i
                               : launch_dma64<128, 2>(A, B, C, M, N, K, ldc, alpha, beta, st);
 }
 
+// The 64x64 tile fed the same way, for more than 64 rows (up to 64 the small-M kernels and their bit-for-bit
+// contract with the register-fed tiles rule): eight stages while every workgroup has a compute unit to itself.
+bool dma64_serves(int M, int K) { return M > 64 && K % (kDma64SlabBytes / 2) == 0; }
+
+bool launch_dma_small(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
+                      hipStream_t st) {
+    const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+    return tiles <= 256 ? launch_dma64<64, 8>(A, B, C, M, N, K, N, alpha, beta, st)
+                        : launch_dma64<64, 4>(A, B, C, M, N, K, N, alpha, beta, st);
+}
+
 void launch_128(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta,
                 hipStream_t st) {
     if (K % (kDma64SlabBytes / 2) == 0 && launch_dma128(A, B, C, M, N, K, N, alpha, beta, st)) return;
@@ -772,6 +783,7 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         launch_skinny(a, projs, blocks, M, K, alpha, beta, st);
         return launch_status();
     }
+    const bool auto_choice = choice == kAuto;
     if (choice == kAuto) {
         // The largest tile that still fills the 256 compute units: 256x256
         // (eight waves, the fewest L1 and LDS bytes per MFMA; fed by direct
@@ -780,7 +792,10 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         // round on.
         const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= 256) ? k128dma : (M > 32) ? k64 : k32;
+        // (copy-fed, four stages deep, the 128x128 tile already pays with half the compute units busy:
+        // 1024 x 3584 x 3584 in 31 us as 224 tiles of 128, 50 us as 896 tiles of 64; at 112 tiles the 64s win)
+        const long enough128 = K % (kDma64SlabBytes / 2) == 0 ? 128 : 256;
+        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= enough128) ? k128dma : (M > 32) ? k64 : k32;
     }
     switch (choice) {
         case k128dma: launch_128(A, B, C, M, N, K, alpha, beta, st); break;
@@ -789,7 +804,10 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
             [[fallthrough]];
         case k256regs: launch_tile<256, 256, 2, 4, 32, 2>(A, B, C, M, N, K, alpha, beta, st); break;
         case k128: launch_tile<128, 128, 2, 2, 64, 2>(A, B, C, M, N, K, alpha, beta, st); break;
-        case k64:  launch_tile<64, 64, 2, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
+        case k64:
+            if (auto_choice && dma64_serves(M, K) && launch_dma_small(A, B, C, M, N, K, alpha, beta, st)) break;
+            launch_tile<64, 64, 2, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st);
+            break;
         default:   launch_tile<32, 64, 1, 2, 64, 1>(A, B, C, M, N, K, alpha, beta, st); break;
     }
     return launch_status();
@@ -840,7 +858,11 @@ bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table,
     if (choice == kAuto) {
         const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
         const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-        choice = wg256 >= 512 ? k256 : wg128 >= 256 ? k128dma : k64;
+        const long enough128 = K % (kDma64SlabBytes / 2) == 0 ? 128 : 256;       // as in gemm()
+        choice = wg256 >= 512 ? k256 : wg128 >= enough128 ? k128dma : k64;
+        // gemm() gives these shapes to the copy-fed 64x64 tile, which is narrower than a head: the caller runs
+        // the two steps one after the other (on the 16x16x32 instruction like that tile, so the bits agree)
+        if (choice == k64 && dma64_serves(M, K)) return false;
     }
     if (choice == k256 && K % (kDmaSlabBytes / 2) == 0) {
         static thread_local int ready32 = -1;
@@ -875,7 +897,7 @@ int forced_tile() {
         const char* e = getenv("VV_GEMM_TILE");
         return e ? atoi(e) : 0;
     }();
-    return (v >= 0 && v <= 5) ? v : 0;
+    return (v >= 0 && v <= 6) ? v : 0;
 }
 
 }  // namespace

@@ -200,14 +200,20 @@ __device__ __forceinline__ void mfma_dma(const void* __restrict__ A, const void*
 // chip with 256x256 tiles: with two stages (64 KB of LDS) two workgroups share a compute unit, the barrier
 // of one hidden behind the other; with four stages a workgroup that has the unit to itself asks for a slab
 // three slabs ahead (its slabs are 512 matrix-core cycles long, a copy's way from memory takes four times that).
+// And a 64x64 tile (two waves of 32 x 64) for the shapes with too few 128x128 tiles to fill the chip: its slab
+// is 16 KB, bound by the copy path (256 clocks) rather than by its 16 MFMAs per wave, so it asks seven slabs
+// ahead (eight stages) when a workgroup has the compute unit to itself and three (four stages) otherwise.
 constexpr int kDma64SlabBytes = 128;
 constexpr int kSuperM = 4, kSuperN = 8;           // tiles per XCD block: 32 workgroups
 
 template <int kTile, int kStages = 2>
 struct Dma64Shape {
-    static_assert(kTile == 256 || kTile == 128, "tile sizes with a schedule");
-    static_assert(kStages == 2 || kStages == 4, "a slab's stage is slab % kStages");
-    static constexpr int kWaves = kTile / 32;                     // 2 x 4 or 2 x 2 waves
+    static_assert(kTile == 256 || kTile == 128 || kTile == 64, "tile sizes with a schedule");
+    static_assert(kStages == 2 || kStages == 4 || kStages == 8, "a slab's stage is slab % kStages");
+    // Slabs asked for ahead of the one in hand. With eight stages seven: a wave then has at most 56 copies
+    // in flight, which its six-bit counter can still tell apart.
+    static constexpr int kAhead = kStages == 8 ? 7 : kStages;
+    static constexpr int kWaves = kTile / 32;                     // 2 x 4, 2 x 2 or 2 x 1 waves
     static constexpr int WN = kWaves / 2;
     static constexpr int TM = kTile / 2 / 16, TN = 4;             // wave tile (kTile / 2) x 64 in 16 x 16 products
     static constexpr int kStageSlots = 2 * kTile * (kDma64SlabBytes / 16);   // A rows, then B rows
@@ -349,7 +355,7 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     // which are held twice like w (their refill could only follow the step's last MFMAs, and the reads of a
     // step must be back when the next begins).
     constexpr int kSingle = TM - 2;
-    u32x4 fw[2][TN], fx[kSingle], fxl[2][TM - kSingle];
+    u32x4 fw[2][TN], fx[kSingle > 0 ? kSingle : 1], fxl[2][TM - kSingle];
     auto read_w = [&](auto set_c, int slab, int step, int a) {
         constexpr int set = decltype(set_c)::value;
         fw[set][a] = dma_lds[(slab & (kStages - 1)) * kStageSlots + fb_base + w_off(a) + f_idx[step]];
@@ -381,8 +387,9 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
             for (int a = 0; a < TN; ++a) {
                 if (step == 1 && b == kBefore && a == 0) {
                     // this wave's copies of the next slab are in: only those of the slabs behind it may still fly
-                    if constexpr (kStages == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                    else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+                    if constexpr (Shape::kAhead == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    else if constexpr (Shape::kAhead == 4) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(40) lgkmcnt(0)" ::: "memory");
                     __syncthreads();
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -391,7 +398,7 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                 const int slot = (b - kBefore * step) * TN + a;    // step 1: counted from the barrier
                 if constexpr (step == 1) {
                     // the copies first: their way from memory is longer than the slab they have to make it in
-                    if (slot >= 0 && slot < kLoads) request(slab + kStages, slot);
+                    if (slot >= 0 && slot < kLoads) request(slab + Shape::kAhead, slot);
                 }
                 if constexpr (TM == 8) {
                     if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
@@ -408,7 +415,7 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                     else if (slot == 15) read_x(nxt_c, nslab, nstep, step == 0 ? 3 : 5);
                     else if (slot == 19 && step == 0) read_x(nxt_c, nslab, nstep, 4);
                     else if (slot == 23 && step == 0) read_x(nxt_c, nslab, nstep, 5);
-                } else {
+                } else if constexpr (TM == 4) {
                     if (slot == 0) read_w(nxt_c, nslab, nstep, 0);
                     else if (slot == 1) read_w(nxt_c, nslab, nstep, 1);
                     else if (slot == 2) read_w(nxt_c, nslab, nstep, 2);
@@ -417,6 +424,9 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
                     else if (slot == 5) read_x(nxt_c, nslab, nstep, 2);
                     else if (slot == 6) read_x(nxt_c, nslab, nstep, 3);
                     else if (slot == 7) read_x(nxt_c, nslab, nstep, 1);
+                } else {                                           // TM == 2: both x fragments are held twice
+                    if (slot < 4) read_w(nxt_c, nslab, nstep, slot);
+                    else if (slot < 6) read_x(nxt_c, nslab, nstep, slot - 4);
                 }
             }
         }
@@ -424,12 +434,13 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     };
 
 #pragma unroll
-    for (int s = 0; s < kStages; ++s)
+    for (int s = 0; s < Shape::kAhead; ++s)
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) request(s, i);
     // slab 0; slab 1 is waited for at the first barrier
-    if constexpr (kStages == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    if constexpr (Shape::kAhead == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (Shape::kAhead == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(48)" ::: "memory");
     __syncthreads();
 #pragma unroll
     for (int a = 0; a < TN; ++a) read_w(Const<0>{}, 0, 0, a);
