@@ -508,6 +508,14 @@ def layer_leg(torch, dev, T: int, st: int, fp16_only: bool = False) -> dict:
     tf = 4.0 * NQ * HD * T * (T + 1) / 2 / sec / 1e12
     out["attn_prefill"] = {"rows": T, "us": sec * 1e6, "TFLOPs": tf,
                            "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+    # The product's launch shape: the prompt's last 2048-row chunk (decoder.c:1147-1174) against the whole cache.
+    if T > 2048:
+        rows, off = 2048, T - 2048
+        sec = timed(lambda: dev.vv_attn_prefill(2, q.data_ptr(), C.addressof(view), o.data_ptr(), NQ, rows, off, T,
+                                                True, None, st), 5)
+        tf = 4.0 * NQ * HD * (rows * off + rows * (rows + 1) / 2) / sec / 1e12
+        out["attn_prefill_chunk"] = {"rows": rows, "q_offset": off, "kv_len": T, "us": sec * 1e6, "TFLOPs": tf,
+                                     "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
     scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
     # Decode reads each layer's cache once per token: 28 caches in rotation (829 MB at T = 14449, so nothing
     # is served from the last-level cache), issued one by one and as one captured graph replayed.
@@ -1270,6 +1278,10 @@ def main() -> int:
         d = layer["attn_prefill"]
         log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+        if "attn_prefill_chunk" in layer:
+            d = layer["attn_prefill_chunk"]
+            log(f"  attention prefill, rows {d['q_offset']}..{T - 1} against {T} keys: {d['us']:9.1f} us "
+                f"{d['TFLOPs']:7.1f} TFLOP/s ({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
         d = layer["attn_decode"]
         log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s "
             f"(replayed from a graph: {d['graph_us']:.2f} us {d['graph_GBps']:.1f} GB/s)")
