@@ -30,6 +30,11 @@ struct I8Op {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, w),
                                                      __builtin_bit_cast(i32x4, x), c, 0, 0, 0);
     }
+    typedef i32x4 Acc16;                      // 16 x 16 over 64 bytes of K (mfma_dma64); integer sums: the same value
+    static __device__ __forceinline__ Acc16 mfma16(u32x4 w, u32x4 x, Acc16 c) {
+        return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, w),
+                                                     __builtin_bit_cast(i32x4, x), c, 0, 0, 0);
+    }
 };
 
 struct I8Out {
@@ -129,6 +134,31 @@ __global__ __launch_bounds__(kDmaWaves * kWave) void i8_dma(const int8_t* __rest
         i8_epilogue<4, 2>(acc, out, m0, n0, frow, fhalf);
     };
     mfma_dma<I8Op>(xq, w, out.M, out.N, K, epilogue);
+}
+
+// The 256x256, 128x128 and 64x64 tiles fed in slabs of 128 bytes per row (whole cache lines) on the 16x16x64
+// instruction (mfma_dma.hpp): K % 128 == 0. Register r of lane l holds column n0 + 16 a + 4 (l / 16) + r of row
+// m0 + 16 b + l % 16 of acc[a][b].
+template <int kTile, int kStages>
+__global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void i8_dma64(const int8_t* __restrict__ xq,
+                                                                                const int8_t* __restrict__ w,
+                                                                                I8Out out, int K) {
+    constexpr int TM = Dma64Shape<kTile>::TM;
+    auto epilogue = [=](const i32x4 (&acc)[4][TM], int m0, int n0, int lane) {
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int m = m0 + b * 16 + (lane & 15);
+            if (m >= out.M) continue;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const int n = n0 + a * 16 + 4 * (lane >> 4);
+                if (n >= out.N) continue;
+                const int t[4] = {acc[a][b][0], acc[a][b][1], acc[a][b][2], acc[a][b][3]};
+                i8_store4(out, m, n, t);
+            }
+        }
+    };
+    mfma_dma64<I8Op, kTile, false, kStages>(xq, w, out.M, out.N, K, epilogue);
 }
 
 __device__ __forceinline__ int wave_sum_i32(int v) {
@@ -315,6 +345,67 @@ bool launch_i8_dma(const int8_t* xq, const int8_t* w, const I8Out& out, int K, h
     return true;
 }
 
+template <int kTile, int kStages>
+bool launch_i8_dma64(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
+    typedef Dma64Shape<kTile, kStages> Shape;
+    static thread_local int ready_device = -1;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return false;
+    if (ready_device != device) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(i8_dma64<kTile, kStages>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)Shape::kLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        ready_device = device;
+    }
+    i8_dma64<kTile, kStages><<<dim3(dma64_grid<kTile>(out.M, out.N)), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(
+        xq, w, out, K);
+    return true;
+}
+
+// Rows [first, first + rows) of a product as a product of its own.
+I8Out i8_rows(const I8Out& o, int first, int rows) {
+    I8Out r = o;
+    r.sx = o.sx + first;
+    if (o.res) r.res = o.res + (size_t)first * o.N;
+    r.y = o.y_f32 ? static_cast<void*>(static_cast<float*>(o.y) + (size_t)first * o.N)
+                  : static_cast<void*>(static_cast<h16*>(o.y) + (size_t)first * o.N);
+    r.M = rows;
+    return r;
+}
+
+// The tile rule of the FP16 GEMM's copy-fed kernels (gemm.hip), for more than 64 rows and K % 128 == 0; the rows
+// that would spill into a mostly empty last round of 256x256 tiles go to the 128x128 tile. false: nothing launched.
+bool launch_i8_dma64_auto(const int8_t* xq, const int8_t* w, const I8Out& out, int K, hipStream_t st) {
+    const int M = out.M, N = out.N;
+    const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const long wg64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+    auto small = [&](const int8_t* x, const I8Out& o) {
+        const long tiles = (long)((o.M + 127) / 128) * ((o.N + 127) / 128);
+        return tiles <= 256 ? launch_i8_dma64<128, 4>(x, w, o, K, st) : launch_i8_dma64<128, 2>(x, w, o, K, st);
+    };
+    if (wg256 >= 512) {
+        // rows of tiles in whole rounds of 8 x 32 workgroups, the rest as one short launch, where that pays
+        const int gx = (N + 255) / 256, gy = (M + 255) / 256;
+        auto rounds = [](long tiles) { return (double)(((tiles + 7) / 8 + 31) / 32); };
+        double best = rounds((long)gx * gy) * 0.95;
+        int head = 0;
+        for (int r = gy - 1; r >= 1 && r >= gy - 16; --r) {
+            const long rest = (long)((M - r * 256 + 127) / 128) * ((N + 127) / 128);
+            const double cost = rounds((long)gx * r) + (rest <= 256 ? 0.42 : 0.6 * (double)((rest + 511) / 512));
+            if (cost < best) { best = cost; head = r * 256; }
+        }
+        if (!head) return launch_i8_dma64<256, 2>(xq, w, out, K, st);
+        if (!small(xq + (size_t)head * K, i8_rows(out, head, M - head))) return false;
+        return launch_i8_dma64<256, 2>(xq, w, i8_rows(out, 0, head), K, st) ||
+               launch_i8_dma64<256, 2>(xq, w, out, K, st);
+    }
+    if (wg128 >= 128) return small(xq, out);
+    return wg64 <= 256 ? launch_i8_dma64<64, 8>(xq, w, out, K, st) : launch_i8_dma64<64, 4>(xq, w, out, K, st);
+}
+
 template <int MR, int kSplit, int RW>
 void launch_i8_gemv_cfg(const int8_t* xq, I8Segs segs, int n_segs, int K, hipStream_t st) {
     constexpr int kRows = kWavesPerBlock / kSplit * RW;
@@ -407,7 +498,8 @@ vv_status_t vv_w8a8_linear_dev(const int8_t* xq, const float* sx, const int8_t* 
     const long wg256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     const long wg128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     static const bool no_dma = [] { const char* e = getenv("VV_I8_NO_DMA"); return e && e[0] == '1'; }();
-    if (wg256 >= 512 && K % vv::kDmaSlabBytes == 0 && !no_dma && vv::launch_i8_dma(xq, w, out, K, st)) {}
+    if (M > 64 && K % vv::kDma64SlabBytes == 0 && !no_dma && vv::launch_i8_dma64_auto(xq, w, out, K, st)) {}
+    else if (wg256 >= 512 && K % vv::kDmaSlabBytes == 0 && !no_dma && vv::launch_i8_dma(xq, w, out, K, st)) {}
     else if (wg256 >= 512) vv::launch_i8_tile<256, 256, 2, 4, 4, 2>(xq, w, out, K, st);
     else if (M > 64 && wg128 >= 256) vv::launch_i8_tile<128, 128, 2, 2, 8, 2>(xq, w, out, K, st);
     else if (M > 32) vv::launch_i8_tile<64, 64, 2, 2, 8, 1>(xq, w, out, K, st);
