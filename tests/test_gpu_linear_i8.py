@@ -61,7 +61,10 @@ def same_f32(got, want, what):
 SHAPES = [(1, 64, 16), (1, 3584, 3584), (1, 18944, 3584), (1, 8200, 512), (2, 100, 48), (3, 512, 3584), (5, 77, 1040),
           (8, 1000, 1536), (9, 64, 64), (16, 30, 48), (29, 512, 3584), (33, 77, 528), (64, 256, 512),
           (65, 3584, 128), (100, 130, 80), (130, 101, 208), (257, 37, 16), (285, 3584, 3584), (300, 4608, 272),
-          (4100, 8200, 64)]
+          (4100, 8200, 64),
+          # K % 128 == 0 above 64 rows: the copy-fed 256x256 tiles with the last rows split off, the 128x128 tile
+          # with two and with four stages (the 64x64 one: 65 and 285 rows above)
+          (4100, 8200, 128), (2100, 2100, 256), (1100, 2048, 128)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
