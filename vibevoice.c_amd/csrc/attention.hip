@@ -411,27 +411,34 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
 // MFMAs; measured, the softmax of a tile costs about what its 32 MFMAs cost. Here the loop is
 // skewed by one tile: while the vector ALU turns tile j's scores into probabilities, the matrix
 // pipe computes tile j + 1's scores, a slice of the one issued behind each MFMA of the other; then
-// the O^T += V^T P^T MFMAs of tile j run with tile j + 1's V^T transposition (and the loads of
-// tile j + 2's V) behind them. K goes from global memory straight into LDS (two buffers, two tiles
-// ahead, no registers, no commit); V is transposed on its way in as before, into two buffers, so
-// one barrier per tile remains. V^T rows are 128 bytes: channel 8 d + e sits in row 16 e + d (so
-// the eight rows a thread writes are 16 rows apart and a wave's writes spread over the banks), its
-// 16-byte units XOR-ed with (row / 2) % 8, and the keys inside a row are ordered so that the eight
-// keys a lane multiplies in one step are one unit: 16-byte reads. The values and their order of
-// summation are those of prefill128: the same bits.
+// the O^T += V^T P^T MFMAs of tile j run. K and V both go from global memory straight into LDS, row
+// major as they lie in the cache (two buffers each, no registers, no commit, one barrier per tile):
+// the V^T operand is transposed on its way OUT of LDS (ds_read_b64_tr_b16: four keys of sixteen
+// channels per group of sixteen lanes, two reads per fragment), which takes the tile's transposition -
+// four loads, sixteen byte permutes and eight LDS writes per thread and tile - off the vector ALU
+// that bounds this kernel (1812 -> 1691 us at 14449 rows). A key's 64-byte quarters rotate with the
+// key, so the four keys of a transposing read lie in four quarters of the banks. A lane multiplies
+// the keys in the order in which its probabilities leave the score MFMAs. The values and their order
+// of summation are those of prefill128: the same bits.
 // The loop is unrolled by two so that the buffers are compile-time constants (LDS addresses are a
 // per-lane offset plus an immediate) and the two score sets swap roles without a copy; contiguous
 // caches are addressed as a uniform base per tile plus a per-lane offset that never changes; the
-// probabilities are converted two at a time. What is left is bound by the vector ALU: about 280
+// probabilities are converted two at a time. What is left is bound by the vector ALU: about 180
 // vector instructions and 33 exponentials per tile and wave against 32 MFMAs.
 // Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
 // alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
 template <int kValue> struct Parity { static constexpr int value = kValue; };
-constexpr int kVtRowHalves = 64;                 // one V^T row: 64 keys, 128 bytes, 8 units of 16 bytes
 struct PipeTiles {
     Chunk k[2][kKeyTile * 16];                   // [buffer][key][16 slots], slot ^ (key & 15)
-    __align__(16) h16 vt[2][kD * kVtRowHalves];  // [buffer][row 16 e + dchunk][unit ^ ((row >> 1) & 7)][8 keys]
+    Chunk v[2][kKeyTile * 16];                   // [buffer][key][16 slots], slot + 4 (key & 3) mod 16
 };
+// Four keys of sixteen channels, transposed on the way out of LDS: lane t of each group of sixteen lanes
+// points at four consecutive halves, and lane j of the group receives element j % 4 of lanes j / 4, j / 4 + 4,
+// j / 4 + 8, j / 4 + 12. With lane t at channels 4 (t % 4) .. + 3 of key t / 4, lane j gets channel j of keys 0 .. 3.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ s16x4 lds_read_transposed(const char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
+}
 __device__ __forceinline__ void copy16_to_lds(const void* gptr, uint32_t lds_byte_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_byte_addr), "v"(gptr) : "memory", "m0");
 }
@@ -489,38 +496,33 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             }
         }
     };
-    // V tile: a thread takes four consecutive keys 4 kg .. + 3 of one 8-channel chunk.
-    const int dchunk = tid & 15, kg = tid >> 4;
-    Chunk vr[4];
+    // V tile j -> buffer j & 1 the same way (the cache rows of K and V have one layout); the lane owning (key,
+    // physical slot p) fetches logical slot p - 4 (key % 4): a key's 64-byte quarters rotate with the key, so the
+    // four keys a transposing read gathers lie in four different quarters of the banks.
+    const uint32_t lds_v0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)&tiles.v[0][0]);
     uint32_t v_off[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v_off[i] = (uint32_t)(((size_t)(4 * kg + i) * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)dchunk * 16u;
-    auto fetch_v1 = [&](int j, int i) {
+    for (int c = 0; c < 4; ++c) {
+        const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
+        v_off[c] = (uint32_t)(((size_t)key * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)(((phys - 4 * (key & 3)) & 15) * 16);
+    }
+    auto request_v = [&](int j) {
         const int t0 = j * kKeyTile;
+        const uint32_t lds_at = lds_v0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave) * 1024u;
         if (!page_table && t0 + kKeyTile <= kv_len) {
             const char* base = reinterpret_cast<const char*>(V) + (size_t)t0 * row_halves * 2u;
-            vr[i] = load_chunk(reinterpret_cast<const Chunk*>(base + v_off[i]));
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             : : "s"(lds_at + (uint32_t)c * 1024u), "v"(v_off[c]), "s"(base) : "memory", "m0");
         } else {
-            const int row = cache_row(page_table, min(t0 + 4 * kg + i, last_key));
-            vr[i] = load_chunk(reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + dchunk);
-        }
-    };
-    auto fetch_v = [&](int j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fetch_v1(j, i);
-    };
-    // key 32 a + 16 sp + 8 x + 4 h + i sits at position 32 a + 16 sp + 8 h + 4 x + i of its row, so that the eight
-    // keys a lane multiplies in one step are one 16-byte unit; kg = 8 a + 4 sp + 2 x + h
-    const int v_unit = (kg >> 2) * 2 + (kg & 1), v_sub = (kg >> 1) & 1;     // unit 2 (2a + sp) + h, half-unit x
-    auto commit_v = [&](int j) {
-        h16x8 v4[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int row = 16 * e + dchunk;
-            const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
-            *reinterpret_cast<h16x4*>(&tiles.vt[j & 1][row * kVtRowHalves + ((v_unit ^ ((row >> 1) & 7)) * 8) + 4 * v_sub]) = w;
+            for (int c = 0; c < 4; ++c) {
+                const int key = 4 * (4 * wave + c) + (lane >> 4), phys = lane & 15;
+                const int row = cache_row(page_table, min(t0 + key, last_key));
+                const Chunk* g = reinterpret_cast<const Chunk*>(V + (size_t)row * row_halves + (size_t)kvh * kD) + ((phys - 4 * (key & 3)) & 15);
+                copy16_to_lds(g, lds_at + (uint32_t)c * 1024u);
+            }
         }
     };
     auto scores = [&](int j, f32x16 (&s)[2]) {
@@ -543,33 +545,34 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     // would wait for them - and with them for every copy in flight - inside the loop.)
     request_k(0);
     request_k(1);
-    fetch_v(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    commit_v(0);
-    fetch_v(1);
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");          // K 0 and K 1 landed; V 1 may fly
+    request_v(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // K 0, K 1 and V 0 landed
     __syncthreads();
     // a lane's fragment positions inside a tile never change: row col (+ 32 a) of K, slot 2 s8 + half swizzled;
     // row col (+ 32 t) of V^T, unit 2 u + half swizzled ((32 t + col) / 2 % 8 = col / 2 % 8)
-    int kf_idx[8], vf_idx[4];
+    int kf_idx[8];
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) kf_idx[s8] = col * 16 + ((2 * s8 + half) ^ (col & 15));
-#pragma unroll
-    for (int u = 0; u < 4; ++u) vf_idx[u] = col * kVtRowHalves + (((2 * u + half) ^ ((col >> 1) & 7)) * 8);
     f32x16 s_pp[2][2];                        // the scores of the tile in hand and of the next, by tile parity
     scores(0, s_pp[0]);
     __syncthreads();                                          // K 0 is read: its buffer may take K 2
 
     // Byte offsets of this lane's fragments from the start of a K / V^T buffer: with the buffer a compile-time
     // constant (the loop is unrolled by two) the rest of an LDS address is an immediate.
-    uint32_t kf_byte[8], vf_byte[4];
+    uint32_t kf_byte[8], vt_byte[4];
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) kf_byte[s8] = (uint32_t)kf_idx[s8] * 16u;
+    // V^T fragments: channel tile t (32 channels), key step u (16 keys). A lane multiplies, in this order, keys
+    // 16 u + 4 half + 0 .. 3 and 16 u + 8 + 4 half + 0 .. 3 (where its probabilities sit after the score MFMAs):
+    // two transposing reads of four keys each. In its group of sixteen lanes, lane t points at key t / 4 of the
+    // four and at channels 32 t' + 16 (group % 2) + 4 (t % 4) .. + 3; the key's quarter rotation depends on t / 4
+    // alone, so the address is one register per channel tile plus an immediate for (u, which four, buffer).
 #pragma unroll
-    for (int u = 0; u < 4; ++u) vf_byte[u] = (uint32_t)vf_idx[u] * 2u;
-    const uint32_t vw_byte = (uint32_t)(dchunk * kVtRowHalves + 4 * v_sub) * 2u;      // V^T write: row 16 e + dchunk
-    // ... whose unit swizzle, (row / 2) % 8 = (8 e + dchunk / 2) % 8, does not depend on e
-    const uint32_t vw_unit = (uint32_t)((v_unit ^ ((dchunk >> 1) & 7)) * 16);
+    for (int t = 0; t < 4; ++t) {
+        const int tin = lane & 15, kk = tin >> 2;
+        const int slot = 4 * ((t + kk) & 3) + 2 * ((lane >> 4) & 1) + ((tin & 3) >> 1);
+        vt_byte[t] = (uint32_t)((4 * half + kk) * 256 + slot * 16 + (tin & 1) * 8);
+    }
     // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
     auto body = [&](int j, auto parity_c) {
         constexpr int P = decltype(parity_c)::value;
@@ -587,6 +590,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                 }
         }
         request_k(j + 2);                                     // into the buffer tile j's K has left
+        request_v(j + 1);                                     // into the buffer tile j - 1's V has left
         const char* kb = reinterpret_cast<const char*>(&tiles.k[P ^ 1][0]);
         auto k_frag = [&](int k) {                            // step k = 8 a + s8
             return __builtin_bit_cast(h16x8, *reinterpret_cast<const Chunk*>(kb + (k >> 3) * 8192 + kf_byte[k & 7]));
@@ -644,37 +648,27 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         }
         st.l += sum;
         st.m = m_new;
-        // block 2: O^T += V^T P^T on the matrix pipe; behind its MFMAs the next tile's V^T goes into its buffer
-        // and the tile after that is asked for
-        const char* vb = reinterpret_cast<const char*>(&tiles.vt[P][0]);
-        char* vw = reinterpret_cast<char*>(&tiles.vt[P ^ 1][0]);
+        // block 2: O^T += V^T P^T on the matrix pipe, the V^T fragments transposed out of the row-major tile
+        const char* vb = reinterpret_cast<const char*>(&tiles.v[P][0]);
         auto v_frag = [&](int k) {                            // step k = 4 u + t
-            return *reinterpret_cast<const h16x8*>(vb + (k & 3) * 32 * kVtRowHalves * 2 + vf_byte[k >> 2]);
+            const char* at = vb + vt_byte[k & 3] + (k >> 2) * 4096;
+            const s16x4 lo = lds_read_transposed(at), hi = lds_read_transposed(at + 2048);
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            return __builtin_bit_cast(h16x8, both);
         };
         h16x8 vf[3];
         vf[0] = v_frag(0);
         vf[1] = v_frag(1);
-        h16x8 v4[4];
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             __builtin_amdgcn_sched_barrier(0);
             if (k + 2 < 16) vf[(k + 2) % 3] = v_frag(k + 2);
             st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (k == 3) {
-                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");      // V j+1 in registers (the four K copies just issued may fly)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) v4[i] = __builtin_bit_cast(h16x8, vr[i]);
-            }
-            if (k >= 4 && k < 12) {
-                const int e = k - 4;
-                const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
-                *reinterpret_cast<h16x4*>(vw + e * 16 * kVtRowHalves * 2 + vw_byte + vw_unit) = w;
-            }
-            if (k >= 12) fetch_v1(j + 2, k - 12);
         }
         __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");      // K j+2 landed (V j+2 may fly)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // K j+2 and V j+1 landed
         __syncthreads();
     };
     // An odd tile count is rounded up: the extra tile lies wholly past the keys the workgroup may see, so it
@@ -688,16 +682,17 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     if (qrow < q_len) {
         const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
         h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
-        // register 4 g + r of tile t is LDS row 32 t + 8 g + 4 half + r = 16 e + dchunk: channel 8 dchunk + e
+        // register 4 g + r of tile t is channel 32 t + 8 g + 4 half + r
+        typedef h16 h16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
+            for (int g = 0; g < 4; ++g) {
+                h16x4 o4;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = 32 * t + 8 * g + 4 * half + r;
-                    op[8 * (row & 15) + (row >> 4)] = to_half(st.o[t][4 * g + r] * inv);
-                }
+                for (int r = 0; r < 4; ++r) o4[r] = to_half(st.o[t][4 * g + r] * inv);
+                *reinterpret_cast<h16x4*>(op + 32 * t + 8 * g + 4 * half) = o4;
+            }
     }
 }
 
