@@ -660,6 +660,10 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         h16x8 vf[3];
         vf[0] = v_frag(0);
         vf[1] = v_frag(1);
+        // Block 2 is matrix work alone and block 1 is bound by its vector work: where the SIMD's other wave
+        // (of the compute unit's second workgroup) is in block 1, it goes first, and these MFMAs fill the
+        // matrix pipe under its softmax (1.5-2 % at 14449 rows).
+        __builtin_amdgcn_s_setprio(0);
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             __builtin_amdgcn_sched_barrier(0);
@@ -667,12 +671,14 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(1);
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // K j+2 and V j+1 landed
         __syncthreads();
     };
     // An odd tile count is rounded up: the extra tile lies wholly past the keys the workgroup may see, so it
     // is masked, its probabilities are zeros and the state does not move.
+    __builtin_amdgcn_s_setprio(1);                            // block 1's priority; block 2 lowers it for itself
     for (int j = 0; j < ntiles; j += 2) {
         body(j, Parity<0>{});
         body(j + 1, Parity<1>{});
