@@ -42,7 +42,38 @@ constexpr int kMaxParts = 256;       // decode slices per KV head
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float other_half(float v) { return __shfl_xor(v, 32); }
+// A value and its partner's, 32 (or 16) lanes away, combined in the vector ALU: the gfx950 lane swaps exchange
+// the odd rows of one register with the even rows of another (rows of 32 or 16 lanes), so from two copies of v
+// one register ends up with the lower row's values in both rows of a pair and the other with the upper row's.
+// No trip through the LDS crossbar and no counter to wait for; max and + commute, so every lane gets the bits
+// that v (op) shuffle-xor(v) gave it. (As instructions: the compiler's builtin for them hands back the first
+// register twice. The two wait states are what it puts between a vector write and a swap that reads it.)
+__device__ __forceinline__ void swap_rows32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_rows16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_xor32(float v) {
+    float a = v, b = v;
+    swap_rows32(a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    float a = v, b = v;
+    swap_rows32(a, b);
+    return a + b;
+}
+__device__ __forceinline__ float max_xor16(float v) {
+    float a = v, b = v;
+    swap_rows16(a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_xor16(float v) {
+    float a = v, b = v;
+    swap_rows16(a, b);
+    return a + b;
+}
 
 __device__ __forceinline__ int cache_row(const int* page_table, int t) {
     return page_table ? page_table[t / kPage] * kPage + t % kPage : t;
@@ -285,7 +316,7 @@ __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], 
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
-    mx = fmaxf(mx, other_half(mx)) * scale_log2;
+    mx = max_xor32(mx) * scale_log2;
     const float m_new = fmaxf(st.m, mx);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
     float sum = 0.0f;
@@ -297,7 +328,7 @@ __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], 
             s[a][r] = p;
             sum += p;
         }
-    sum += other_half(sum);
+    sum = sum_xor32(sum);
     if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
         const float alpha = exp2_fast(st.m - m_use);
         st.l *= alpha;
@@ -614,7 +645,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
 #pragma unroll
                 for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_cur[q >> 4][q & 15]);
                 if (k == 3) {
-                    mx = fmaxf(mx, other_half(mx)) * scale_log2;
+                    mx = max_xor32(mx) * scale_log2;
                     m_new = fmaxf(st.m, mx);
                     m_use = m_new == -INFINITY ? 0.0f : m_new;
                 }
@@ -637,7 +668,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             pf[q >> 3][q & 7] = h[0];
             pf[q >> 3][(q & 7) + 1] = h[1];
         }
-        sum += other_half(sum);
+        sum = sum_xor32(sum);
         if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
             const float alpha = exp2_fast(st.m - m_use);
             st.l *= alpha;
@@ -862,8 +893,6 @@ constexpr int kStreamOStride = kD + 1;          // floats per head in the waves'
 // A wave's LDS: V^T of a block (4 KB), later its O for kHeads heads.
 constexpr int stream_tile_bytes(int heads) { return heads * kStreamOStride * 4 < 4096 ? 4096 : (heads * kStreamOStride * 4 + 15) / 16 * 16; }
 
-__device__ __forceinline__ float xor_lanes16(float v) { return __shfl_xor(v, 16); }
-
 template <int kHeads>      // the group's query heads, padded: 8 or 16
 __global__ __launch_bounds__(kStreamThreads) void decode_stream(
     const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V,
@@ -936,8 +965,7 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
             sc[r] = key0 + 4 * j + r < end ? sc[r] : -INFINITY;
             mx = fmaxf(mx, sc[r]);
         }
-        mx = fmaxf(mx, xor_lanes16(mx));
-        mx = fmaxf(mx, other_half(mx)) * scale_log2;
+        mx = max_xor32(max_xor16(mx)) * scale_log2;
         const float m_new = fmaxf(m, mx);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         if (__builtin_amdgcn_ballot_w64(m_new > m && m > -INFINITY) != 0) {
@@ -978,8 +1006,7 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
     }
 
     // the wave's denominators meet across the four j groups; then the waves
-    l += xor_lanes16(l);
-    l += other_half(l);
+    l = sum_xor32(sum_xor16(l));
     if (j == 0) {
         m_lds[wave][c] = m;
         l_lds[wave][c] = l;
