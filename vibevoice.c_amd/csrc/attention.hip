@@ -455,7 +455,10 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
 // per-lane offset plus an immediate) and the two score sets swap roles without a copy; contiguous
 // caches are addressed as a uniform base per tile plus a per-lane offset that never changes; the
 // probabilities are converted two at a time. What is left is bound by the vector ALU: about 180
-// vector instructions and 33 exponentials per tile and wave against 32 MFMAs.
+// vector instructions and 33 exponentials per tile and wave against 32 MFMAs. The softmax block runs
+// at a higher wave priority than the V^T P^T block (the SIMD's other wave belongs to the compute
+// unit's other workgroup and is in any phase to this one), and the two exchanges between the halves
+// of a wave are lane swaps in the vector ALU (max_xor32, sum_xor32): 1691 -> 1531 us together.
 // Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
 // alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
 template <int kValue> struct Parity { static constexpr int value = kValue; };
