@@ -607,11 +607,9 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         const int slot = 4 * ((t + kk) & 3) + 2 * ((lane >> 4) & 1) + ((tin & 3) >> 1);
         vt_byte[t] = (uint32_t)((4 * half + kk) * 256 + slot * 16 + (tin & 1) * 8);
     }
-    // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
-    auto body = [&](int j, auto parity_c) {
-        constexpr int P = decltype(parity_c)::value;
-        f32x16 (&s_cur)[2] = s_pp[P];
-        f32x16 (&s_next)[2] = s_pp[P ^ 1];
+    // Tile j's scores lose what the row may not see: only a tile that reaches past the cache end or past the
+    // wave's first row's position has anything to hide.
+    auto hide = [&](int j, f32x16 (&sc)[2]) {
         const int t0 = j * kKeyTile;
         if (t0 + kKeyTile > kv_len || (causal && t0 + kKeyTile - 1 > q_offset + qw0)) {
 #pragma unroll
@@ -620,9 +618,22 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                 for (int r = 0; r < 16; ++r) {
                     const int key = t0 + 32 * a + 8 * (r >> 2) + 4 * half + (r & 3);
                     const bool seen = key < kv_len && (!causal || key <= q_abs);
-                    s_cur[a][r] = seen ? s_cur[a][r] : -INFINITY;
+                    sc[a][r] = seen ? sc[a][r] : -INFINITY;
                 }
         }
+    };
+    // The row maximum (scaled) of the tile in hand: taken while the vector ALU has nothing else to do, behind the
+    // first V^T P^T MFMAs of the tile before (behind the first scores in the prologue).
+    hide(0, s_pp[0]);
+    float mx_cur = -INFINITY;
+#pragma unroll
+    for (int q = 0; q < 32; ++q) mx_cur = fmaxf(mx_cur, s_pp[0][q >> 4][q & 15]);
+    mx_cur = max_xor32(mx_cur) * scale_log2;
+    // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
+    auto body = [&](int j, auto parity_c) {
+        constexpr int P = decltype(parity_c)::value;
+        f32x16 (&s_cur)[2] = s_pp[P];
+        f32x16 (&s_next)[2] = s_pp[P ^ 1];
         request_k(j + 2);                                     // into the buffer tile j's K has left
         request_v(j + 1);                                     // into the buffer tile j - 1's V has left
         const char* kb = reinterpret_cast<const char*>(&tiles.k[P ^ 1][0]);
@@ -636,7 +647,9 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         h16x8 kf[3];
         kf[0] = k_frag(0);
         kf[1] = k_frag(1);
-        float mx = -INFINITY, m_new = 0.0f, m_use = 0.0f, sum = 0.0f;
+        float sum = 0.0f;
+        const float m_new = fmaxf(st.m, mx_cur);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         h16x8 pf[4];
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
@@ -644,21 +657,11 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             if (k + 2 < 16) kf[(k + 2) % 3] = k_frag(k + 2);
             s_next[k >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[k % 3], qf[k & 7], s_next[k >> 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (k < 4) {
 #pragma unroll
-                for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_cur[q >> 4][q & 15]);
-                if (k == 3) {
-                    mx = max_xor32(mx) * scale_log2;
-                    m_new = fmaxf(st.m, mx);
-                    m_use = m_new == -INFINITY ? 0.0f : m_new;
-                }
-            } else {
-#pragma unroll
-                for (int q = (k - 4) * 32 / 12; q < (k - 3) * 32 / 12; ++q) {
-                    const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -m_use));
-                    sum += p;
-                    s_cur[q >> 4][q & 15] = p;
-                }
+            for (int q = 2 * k; q < 2 * k + 2; ++q) {
+                const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -m_use));
+                sum += p;
+                s_cur[q >> 4][q & 15] = p;
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -698,12 +701,20 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         // (of the compute unit's second workgroup) is in block 1, it goes first, and these MFMAs fill the
         // matrix pipe under its softmax (1.5-2 % at 14449 rows).
         __builtin_amdgcn_s_setprio(0);
+        hide(j + 1, s_next);
+        float mx = -INFINITY;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             __builtin_amdgcn_sched_barrier(0);
             if (k + 2 < 16) vf[(k + 2) % 3] = v_frag(k + 2);
             st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+            if (k < 4) {                                      // the next tile's row maximum, where the vector ALU idles
+#pragma unroll
+                for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_next[q >> 4][q & 15]);
+            } else if (k == 4) {
+                mx_cur = max_xor32(mx) * scale_log2;
+            }
         }
         __builtin_amdgcn_s_setprio(1);
         __builtin_amdgcn_sched_barrier(0);
