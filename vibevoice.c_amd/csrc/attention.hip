@@ -458,7 +458,9 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
 // vector instructions and 33 exponentials per tile and wave against 32 MFMAs. The softmax block runs
 // at a higher wave priority than the V^T P^T block (the SIMD's other wave belongs to the compute
 // unit's other workgroup and is in any phase to this one), and the two exchanges between the halves
-// of a wave are lane swaps in the vector ALU (max_xor32, sum_xor32): 1691 -> 1531 us together.
+// of a wave are lane swaps in the vector ALU (max_xor32, sum_xor32); the row maximum of the next tile
+// is taken behind the first V^T P^T MFMAs, so that the exponentials spread over all sixteen score
+// MFMAs: 1691 -> 1501 us together.
 // Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
 // alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
 template <int kValue> struct Parity { static constexpr int value = kValue; };
