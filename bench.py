@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused layer kernels at the Qwen2-7B prefill shape.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layer] [--only NAME]
 
 One "step" is one pass of the hot path over a T = 14449 token prompt:
   gather+norm   vv_embedding_rmsnorm_dev   table [152064,3584] -> hidden, normed
@@ -17,7 +17,11 @@ left by the previous one. Reported:
              algorithmic byte count, rows/s, fraction of the 8 TB/s HBM peak;
   roofline   the dominant kernel (SwiGLU: 63 % of the step's bytes);
   cpu_baseline  the reference's CPU kernels (or our restatement of them) on the
-             host's cores, on the same T = 14449 step (about 10 s including input generation).
+             host's cores, on the same T = 14449 step (about 10 s including input generation);
+  configs    the reference's own launch shapes (512-4096 rows), cold;
+  layer      the FP16 GEMM and attention entry points at the layer's shapes (not part of
+             `value`; --no-layer skips them, --layer / --layer-fp16 add the quantised and
+             whole-token legs).
 Prints one JSON line on stdout; progress goes to stderr.
 """
 from __future__ import annotations
@@ -1174,6 +1178,9 @@ def main() -> int:
                          "figures built on them (no quantised, BitNet or Conv-VAE legs): short enough to profile")
     ap.add_argument("--no-token", action="store_true",
                     help="with --layer / --layer-fp16: skip the whole-token decode legs (thousands of small launches)")
+    ap.add_argument("--no-layer", action="store_true",
+                    help="skip the FP16 GEMM and attention legs that a plain run reports under 'layer' "
+                         "(the --layer-fp16 legs without the whole-token ones)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (vv_dev_memcpy_d2d_at at index 0) "
                          "five times: the known-size reference for rocprofv3 byte counters")
@@ -1249,7 +1256,11 @@ def main() -> int:
                 f"{100 * unfused[name]['frac_of_peak']:5.1f} % of peak  (not part of the step)")
 
     layer = {}
-    if args.layer or args.layer_fp16:
+    # a plain run carries the FP16 GEMM / attention figures too (a dozen seconds; never part of `value`)
+    default_layer = not (args.layer or args.layer_fp16 or args.no_layer or args.only)
+    if default_layer:
+        args.no_token = True
+    if args.layer or args.layer_fp16 or default_layer:
         fp16_only = not args.layer
         layer = layer_leg(torch, dev, T, st, fp16_only)
         for name, d in list(layer["gemm"].items()) + list(layer.get("gemm_chunk", {}).items()):
