@@ -1155,6 +1155,79 @@ def cpu_baseline(rows: int) -> dict:
     }
 
 
+def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
+    """The GEMM / attention / whole-layer legs reported under 'layer' (none of them part of `value`)."""
+    layer = layer_leg(torch, dev, T, st, fp16_only)
+    for name, d in list(layer["gemm"].items()) + list(layer.get("gemm_chunk", {}).items()):
+        log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+            f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+    for name, d in layer["gemv"].items():
+        log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+    for kind in () if fp16_only else ("w8a8", "w4a8"):
+        for name, d in layer[kind].items():
+            log(f"  {kind} {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TOPs']:7.1f} TOP/s "
+                f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
+        for name, d in layer[kind + "_gemv"].items():
+            log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+    for name, d in layer.get("w4a8_chunk", {}).items():
+        log(f"  w4a8 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+    for name, d in layer.get("w4a16", {}).items():
+        log(f"  w4a16 {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+            f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+    for name, d in layer.get("w4a16_gemv", {}).items():
+        log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+    for name, d in layer.get("w4a16_chunk", {}).items():
+        log(f"  w4a16 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+    for name, d in layer.get("weight_only", {}).items():
+        log(f"  weight-only {name:18s} N={d['N']} K={d['K']}: one row {d['M1_us']:7.2f} us {d['M1_GBps']:7.1f} GB/s, "
+            f"29 rows {d['M29_us']:7.2f} us, dequantise {d['dequant_us']:7.2f} us {d['dequant_GBps']:7.1f} GB/s")
+    d = layer["attn_prefill"]
+    log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+        f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+    if "attn_prefill_chunk" in layer:
+        d = layer["attn_prefill_chunk"]
+        log(f"  attention prefill, rows {d['q_offset']}..{T - 1} against {T} keys: {d['us']:9.1f} us "
+            f"{d['TFLOPs']:7.1f} TFLOP/s ({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+    d = layer["attn_decode"]
+    log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s "
+        f"(replayed from a graph: {d['graph_us']:.2f} us {d['graph_GBps']:.1f} GB/s)")
+    if not fp16_only:
+        d = layer["attn_prefill_fp8"]
+        log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
+        d = layer["attn_decode_fp8"]
+        log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
+        d = layer["bitnet"]
+        log("  BitNet (1536 / 8960 / 151936): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
+        d = layer["vae"]
+        log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
+    layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
+    log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
+        f"{d['ms_per_layer_rope_as_its_own_launch']:.2f} ms with bias + RoPE as a launch of its own); "
+        f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
+    for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
+        torch.cuda.empty_cache()
+        layer["prefill_layer_" + kind] = d = prefill_layer_quant_leg(torch, dev, T, st, kind)
+        log(f"  prefill layer, {kind} projections: {d['ms_per_layer']:.2f} ms ({d['Tops']:.0f} TOP/s over linears + "
+            f"attention); 28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
+    if not args.no_token:
+        layer["decode_token"] = d = decode_token_leg(torch, dev, T)
+        log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+        layer["decode_token_fused"] = d = decode_token_leg(torch, dev, T, fused=True)
+        log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
+            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
+            f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+
+    for kind in () if fp16_only or args.no_token else ("w4a16", "w8a8", "w4a8"):
+        torch.cuda.empty_cache()
+        layer["decode_token_" + kind] = d = decode_token_quant_leg(torch, dev, T, kind)
+        log(f"  decode token, {kind} projections: {d['calls']} calls, eager {d['eager_ms']:.3f} ms, "
+            f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at "
+            f"{d['weight_GBps']:.0f} GB/s ({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+    return layer
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1260,76 +1333,14 @@ def main() -> int:
     default_layer = not (args.layer or args.layer_fp16 or args.no_layer or args.only)
     if default_layer:
         args.no_token = True
-    if args.layer or args.layer_fp16 or default_layer:
-        fp16_only = not args.layer
-        layer = layer_leg(torch, dev, T, st, fp16_only)
-        for name, d in list(layer["gemm"].items()) + list(layer.get("gemm_chunk", {}).items()):
-            log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
-                f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
-        for name, d in layer["gemv"].items():
-            log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for kind in () if fp16_only else ("w8a8", "w4a8"):
-            for name, d in layer[kind].items():
-                log(f"  {kind} {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TOPs']:7.1f} TOP/s "
-                    f"({100 * d['frac_of_mfma_peak']:.1f} % of the int8 matrix peak)")
-            for name, d in layer[kind + "_gemv"].items():
-                log(f"  {kind} gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer.get("w4a8_chunk", {}).items():
-            log(f"  w4a8 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer.get("w4a16", {}).items():
-            log(f"  w4a16 {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
-                f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
-        for name, d in layer.get("w4a16_gemv", {}).items():
-            log(f"  w4a16 gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer.get("w4a16_chunk", {}).items():
-            log(f"  w4a16 {d['M']} rows {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-        for name, d in layer.get("weight_only", {}).items():
-            log(f"  weight-only {name:18s} N={d['N']} K={d['K']}: one row {d['M1_us']:7.2f} us {d['M1_GBps']:7.1f} GB/s, "
-                f"29 rows {d['M29_us']:7.2f} us, dequantise {d['dequant_us']:7.2f} us {d['dequant_GBps']:7.1f} GB/s")
-        d = layer["attn_prefill"]
-        log(f"  attention prefill T={T}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
-            f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
-        if "attn_prefill_chunk" in layer:
-            d = layer["attn_prefill_chunk"]
-            log(f"  attention prefill, rows {d['q_offset']}..{T - 1} against {T} keys: {d['us']:9.1f} us "
-                f"{d['TFLOPs']:7.1f} TFLOP/s ({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
-        d = layer["attn_decode"]
-        log(f"  attention decode, cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s "
-            f"(replayed from a graph: {d['graph_us']:.2f} us {d['graph_GBps']:.1f} GB/s)")
-        if not fp16_only:
-            d = layer["attn_prefill_fp8"]
-            log(f"  attention prefill, FP8 cache: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s")
-            d = layer["attn_decode_fp8"]
-            log(f"  attention decode, FP8 cache {T}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
-            d = layer["bitnet"]
-            log("  BitNet (1536 / 8960 / 151936): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
-            d = layer["vae"]
-            log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
-        layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
-        log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
-            f"{d['ms_per_layer_rope_as_its_own_launch']:.2f} ms with bias + RoPE as a launch of its own); "
-            f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
-        for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
-            torch.cuda.empty_cache()
-            layer["prefill_layer_" + kind] = d = prefill_layer_quant_leg(torch, dev, T, st, kind)
-            log(f"  prefill layer, {kind} projections: {d['ms_per_layer']:.2f} ms ({d['Tops']:.0f} TOP/s over linears + "
-                f"attention); 28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
-        if not args.no_token:
-            layer["decode_token"] = d = decode_token_leg(torch, dev, T)
-            log(f"  decode token, {d['layers']} layers, cache {T}: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
-                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
-                f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
-            layer["decode_token_fused"] = d = decode_token_leg(torch, dev, T, fused=True)
-            log(f"  decode token, fused additions: {d['launches']} launches, eager {d['eager_ms']:.3f} ms, "
-                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at {d['weight_GBps']:.0f} GB/s "
-                f"({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
-
-        for kind in () if fp16_only or args.no_token else ("w4a16", "w8a8", "w4a8"):
-            torch.cuda.empty_cache()
-            layer["decode_token_" + kind] = d = decode_token_quant_leg(torch, dev, T, kind)
-            log(f"  decode token, {kind} projections: {d['calls']} calls, eager {d['eager_ms']:.3f} ms, "
-                f"graph {d['graph_ms']:.3f} ms = {d['tokens_per_s']:.0f} tokens/s, weights at "
-                f"{d['weight_GBps']:.0f} GB/s ({100 * d['frac_of_hbm_peak']:.1f} % of peak)")
+    if args.layer or args.layer_fp16:
+        layer = layer_legs(torch, dev, T, st, args, not args.layer)
+    elif default_layer:
+        try:                                  # the line's own figures must not depend on these legs
+            layer = layer_legs(torch, dev, T, st, args, True)
+        except Exception as e:  # noqa: BLE001
+            log(f"  layer legs failed: {e!r}")
+            layer = {"error": repr(e)}
 
     # ── BASELINE.json's config shapes and the 2048-row prefill chunk, cold ──
     configs = []
