@@ -56,7 +56,9 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           # the 128x128 tile fed the same way: 17 x 17, 9 x 32 and 113 x 4 tiles
           (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128), (70, 33000, 64),      # ... and one row of 258 tiles
           # the 64x64 tile fed the same way: 256 tiles or fewer (eight stages), more (four), ragged, one slab
-          (2048, 512, 3584), (285, 3584, 3584), (130, 200, 64), (1000, 1100, 192), (65, 64, 128)]
+          (2048, 512, 3584), (285, 3584, 3584), (130, 200, 64), (1000, 1100, 192), (65, 64, 128),
+          # one row, few long weight rows: two output columns per wave (an odd count leaves the last wave one)
+          (1, 3584, 18944), (1, 37, 8192), (1, 1, 8200)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -203,7 +205,7 @@ def gemv_multi(d_x, ws, biases, K):
 
 
 @pytest.mark.parametrize("Ns,K", [((3584, 512, 512), 3584), ((1536, 256, 256), 1536), ((18944, 18944), 3584),
-                                  ((9000,), 520), ((37, 5, 101), 72)])
+                                  ((9000,), 520), ((37, 5, 101), 72), ((3584,), 18944), ((37, 5), 8192)])
 def test_gemv_multi_equals_gemv_then_bias(Ns, K):
     """One decode row through several projections in one launch == the separate calls, bit for bit."""
     d_x = to_dev(oracle.normal_f16((1, K), 61))
