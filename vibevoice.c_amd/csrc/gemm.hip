@@ -25,6 +25,8 @@
 //   gemv_row<kSplit>        M == 1 (a decode step): one to four waves per
 //                           output column stream that weight row once with
 //                           non-temporal 16-byte loads.
+//   gemv_rows<kSplit, kR>   M == 1 over few long weight rows: kR output
+//                           columns per wave, summed in gemv_row's order.
 //   gemm_naive              K not a multiple of 8, or pointers off 16 bytes.
 #include "mfma_dma.hpp"
 #include "row_math.hpp"
