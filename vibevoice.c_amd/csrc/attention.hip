@@ -1137,6 +1137,23 @@ __global__ __launch_bounds__(kBlock) void kv_store_fp16(
     v_store[dst] = v[i];
 }
 
+// The same in 16-byte chunks, for rows that are whole chunks at aligned addresses (any n_kv_heads x 128): a thread
+// asks for its K and V chunks before it reads the position and the page, so a decode step's store is three trips
+// to memory in a row (arguments; position, K and V together; page), not five, and a prefill's moves 16 bytes an access.
+__global__ __launch_bounds__(kBlock) void kv_store_fp16_chunks(
+    const Chunk* __restrict__ k, const Chunk* __restrict__ v, Chunk* __restrict__ k_store,
+    Chunk* __restrict__ v_store, int row_chunks, int pos, const int* __restrict__ d_pos, int n_chunks,
+    const int* __restrict__ page_table) {
+    const int i = (int)blockIdx.x * kBlock + (int)threadIdx.x;
+    if (i >= n_chunks) return;
+    const Chunk kc = load_chunk(k + i), vc = load_chunk(v + i);
+    const int p = i / row_chunks, e = i - p * row_chunks;
+    const int t = (d_pos ? *d_pos : pos) + p;
+    const size_t dst = (size_t)cache_row(page_table, t) * row_chunks + e;
+    store_chunk(k_store + dst, kc);
+    store_chunk(v_store + dst, vc);
+}
+
 // ── FP8 cache store (src/cuda/kv_quant.cu:57-84, kv_codec.cuh:66-128) ──────
 // One value to E4M3 (bias 7, largest finite 448 = 0x7E) or E5M2 (bias 15,
 // largest finite 57344 = 0x7B) in integer arithmetic: zero and NaN give a signed
@@ -1779,6 +1796,16 @@ vv_status_t vv_kv_store_dev(const void* k_fp16, const void* v_fp16, void* k_stor
     }
     const int row = n_kv_heads * head_dim;
     const size_t n = (size_t)n_positions * row;
+    if (row % 8 == 0 && n / 8 <= 0x7fffffffu && vv::aligned16(k_fp16) && vv::aligned16(v_fp16) &&
+        vv::aligned16(k_store) && vv::aligned16(v_store)) {
+        const int n_chunks = (int)(n / 8);
+        vv::kv_store_fp16_chunks<<<dim3((unsigned)((n_chunks + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
+                                   vv::as_stream(stream)>>>(
+            static_cast<const vv::Chunk*>(k_fp16), static_cast<const vv::Chunk*>(v_fp16),
+            static_cast<vv::Chunk*>(k_store), static_cast<vv::Chunk*>(v_store), row / 8, pos, d_pos, n_chunks,
+            page_table);
+        return vv::launch_status();
+    }
     vv::kv_store_fp16<<<dim3((unsigned)((n + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
                         vv::as_stream(stream)>>>(
         static_cast<const vv::h16*>(k_fp16), static_cast<const vv::h16*>(v_fp16),
