@@ -119,6 +119,34 @@ def paged_cache(k, v, nkv, hd, seed):
     return pool_k, pool_v, table, perm
 
 
+@pytest.mark.parametrize("nkv,hd,shift", [(4, 128, 0), (3, 20, 0), (2, 64, 1), (1, 8, 0)])
+def test_kv_store_fp16_places_rows(nkv, hd, shift):
+    """FP16 append at a host and at a device-side position: rows of whole 16-byte chunks, rows that are not
+    (3 x 20 halves), and a source that is not 16-byte aligned (one half off) all land where they belong."""
+    cap, n1, n2 = 40, 7, 5
+    rng = np.random.default_rng(3)
+    k = rng.standard_normal((n1 + n2, nkv, hd)).astype(np.float16)
+    v = rng.standard_normal((n1 + n2, nkv, hd)).astype(np.float16)
+    flat_k = torch.zeros((n1 + n2) * nkv * hd + 8, dtype=torch.float16, device="cuda")
+    flat_v = torch.zeros_like(flat_k)
+    flat_k[shift:shift + k.size] = torch.from_numpy(k.reshape(-1)).cuda()
+    flat_v[shift:shift + v.size] = torch.from_numpy(v.reshape(-1)).cuda()
+    ck = torch.full((cap, nkv, hd), float("nan"), dtype=torch.float16, device="cuda")
+    cv = torch.full((cap, nkv, hd), float("nan"), dtype=torch.float16, device="cuda")
+    row = nkv * hd * 2
+    ok(dev.vv_kv_store_dev(flat_k.data_ptr() + 2 * shift, flat_v.data_ptr() + 2 * shift, ck.data_ptr(), cv.data_ptr(),
+                           None, None, None, False, nkv, hd, 3, None, n1, FP16, None, stream()))
+    d_pos = torch.tensor([3 + n1], dtype=torch.int32, device="cuda")
+    ok(dev.vv_kv_store_dev(flat_k.data_ptr() + 2 * shift + n1 * row, flat_v.data_ptr() + 2 * shift + n1 * row,
+                           ck.data_ptr(), cv.data_ptr(), None, None, None, False, nkv, hd, 0, d_pos.data_ptr(), n2,
+                           FP16, None, stream()))
+    torch.cuda.synchronize()
+    got_k, got_v = ck.cpu().numpy(), cv.cpu().numpy()
+    assert np.array_equal(got_k[3:3 + n1 + n2].view(np.uint16), k.view(np.uint16))
+    assert np.array_equal(got_v[3:3 + n1 + n2].view(np.uint16), v.view(np.uint16))
+    assert np.isnan(got_k[:3].astype(np.float32)).all() and np.isnan(got_k[3 + n1 + n2:].astype(np.float32)).all()
+
+
 @pytest.mark.parametrize("rows,nq,nkv,off", [(100, 4, 2, 150), (1, 28, 4, 300)])
 def test_paged_cache_matches_contiguous(rows, nq, nkv, off):
     hd, kv_len = 128, off + rows
