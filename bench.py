@@ -385,6 +385,27 @@ def layer_leg(torch, dev, T: int, st: int, fp16_only: bool = False) -> dict:
                                   "frac_of_hbm_peak": gb / HBM_PEAK_GBPS}
             del a, c
         del w
+    # gate, up and SwiGLU in one GEMM (vv_gemm_swiglu_dev) against the three launches it replaces
+    out["gemm_swiglu"] = {}
+    wg = torch.randn(I_FF, H, dtype=torch.float16, device="cuda") * H ** -0.5
+    wu = torch.randn(I_FF, H, dtype=torch.float16, device="cuda") * H ** -0.5
+    for m in (T, 2048):
+        a = torch.randn(m, H, dtype=torch.float16, device="cuda")
+        g, u = (torch.empty(m, I_FF, dtype=torch.float16, device="cuda") for _ in range(2))
+
+        def three():
+            dev.vv_gemm_fp16_dev(a.data_ptr(), wg.data_ptr(), g.data_ptr(), m, I_FF, H, 1.0, 0.0, st)
+            dev.vv_gemm_fp16_dev(a.data_ptr(), wu.data_ptr(), u.data_ptr(), m, I_FF, H, 1.0, 0.0, st)
+            dev.vv_swiglu_dev(g.data_ptr(), u.data_ptr(), g.data_ptr(), m * I_FF, st)
+        sec = timed(lambda: dev.vv_gemm_swiglu_dev(a.data_ptr(), wg.data_ptr(), wu.data_ptr(), None, None,
+                                                   g.data_ptr(), m, I_FF, H, st), 5)
+        sec3 = timed(three, 5)
+        tf = 4.0 * m * I_FF * H / sec / 1e12
+        out["gemm_swiglu"][f"M{m}"] = {"M": m, "N": I_FF, "K": H, "us": sec * 1e6, "TFLOPs": tf,
+                                       "frac_of_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS,
+                                       "us_two_gemms_and_swiglu": sec3 * 1e6}
+        del a, g, u
+    del wg, wu
     if not fp16_only:
         # The same four projections as W8A8 (int8 x int8 on the matrix cores, per-row / per-channel scales).
         out["w8a8"], out["w8a8_gemv"] = {}, {}
@@ -670,9 +691,12 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
         assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, T, 0, T, True, None, st) == 0
         gemm(attn, wo, proj, H, QD)
         assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n2), P(normed), T, H, EPS, st) == 0
-        gemm(normed, wg, gate, I_FF, H)
-        gemm(normed, wu, up, I_FF, H)
-        assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), T * I_FF, st) == 0
+        if fused:       # gate, up and SwiGLU in one GEMM: gate and up are never written
+            assert dev.vv_gemm_swiglu_dev(P(normed), P(wg), P(wu), None, None, P(gate), T, I_FF, H, st) == 0
+        else:
+            gemm(normed, wg, gate, I_FF, H)
+            gemm(normed, wu, up, I_FF, H)
+            assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), T * I_FF, st) == 0
         gemm(gate, wd, proj, H, I_FF)
         assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
 
@@ -694,7 +718,7 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
     ms = time_layer(True)
     assert bool(torch.isfinite(hidden).all())
     flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
-    return {"rows": T, "ms_per_layer": ms, "ms_per_layer_rope_as_its_own_launch": ms_separate,
+    return {"rows": T, "ms_per_layer": ms, "ms_per_layer_reference_api_calls": ms_separate,
             "TFLOPs": flops / ms / 1e9, "layers_assumed": 28, "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
 
 
@@ -1161,6 +1185,10 @@ def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
     for name, d in list(layer["gemm"].items()) + list(layer.get("gemm_chunk", {}).items()):
         log(f"  gemm {name:13s} M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
             f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak)")
+    for name, d in layer.get("gemm_swiglu", {}).items():
+        log(f"  gemm gate+up+swiglu M={d['M']} N={d['N']} K={d['K']}: {d['us']:9.1f} us {d['TFLOPs']:7.1f} TFLOP/s "
+            f"({100 * d['frac_of_mfma_peak']:.1f} % of the FP16 matrix peak); as two GEMMs and SwiGLU "
+            f"{d['us_two_gemms_and_swiglu']:.1f} us")
     for name, d in layer["gemv"].items():
         log(f"  gemv {name:13s} N={d['N']} K={d['K']}: {d['us']:7.2f} us {d['GBps']:7.1f} GB/s")
     for kind in () if fp16_only else ("w8a8", "w4a8"):
@@ -1202,7 +1230,7 @@ def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
         log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
     layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
     log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
-        f"{d['ms_per_layer_rope_as_its_own_launch']:.2f} ms with bias + RoPE as a launch of its own); "
+        f"{d['ms_per_layer_reference_api_calls']:.2f} ms with bias + RoPE and SwiGLU as launches of their own); "
         f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
     for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
         torch.cuda.empty_cache()

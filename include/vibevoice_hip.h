@@ -709,6 +709,18 @@ vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias
 vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int n_proj,
                               int K, void* stream);
 
+/* addition: a prefill's MLP front half in one GEMM, out[M, N] = silu(fp16(A Wg^T)) *
+ * fp16(A Wu^T) for A[M, K], Wg and Wu [N, K] (decoder.c:966-977: two
+ * vv_gemm_fp16_dev and vv_swiglu_dev). Gate and up are rounded to FP16 where the
+ * two GEMMs store and go through the SwiGLU kernel's own function in the GEMM's
+ * store, so the result equals the three calls bit for bit and gate and up are
+ * never written. Fused for M > 64, K % 64 == 0 and 16-byte aligned A, Wg, Wu;
+ * every other shape runs the three calls through the caller's `gate` and `up`
+ * buffers ([M, N] each; NULL: VV_ERR_UNSUPPORTED for those shapes, nothing
+ * launched). The fused path does not touch `gate` and `up`. */
+vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_up, void* gate,
+                               void* up, void* out, int M, int N, int K, void* stream);
+
 /* addition: the decode step's MLP front half in one launch,
  * y[N] = silu(x . Wg^T) * (x . Wu^T): equals two vv_gemm_fp16_dev(M = 1) and
  * vv_swiglu_dev bit for bit (decoder.c:966-977) without writing gate and up. */

@@ -332,6 +332,50 @@ __global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma
     mfma_dma64<F16Op, kTile, true, kStages>(A, B, M, N, K * 2, epilogue);
 }
 
+// The front half of a gated MLP in one GEMM: out = silu(fp16(A Wg^T)) * fp16(A Wu^T). A tile multiplies 256 rows of A
+// with 128 rows of Wg and the same 128 rows of Wu (mfma_dma64's two-operand layout), so acc[a] and acc[a + 2] of a
+// wave are one output element's gate and up products. Both are rounded to FP16 where the two GEMMs' stores round,
+// then the SwiGLU kernel's own function runs on them: the result equals vv_gemm_fp16_dev twice and vv_swiglu_dev
+// bit for bit, without gate and up ever going to memory (2 x 547 MB written and read again at 14449 x 18944).
+template <int TM>
+__device__ __forceinline__ void store_tile16_swiglu(const f32x4 (&acc)[4][TM], h16* __restrict__ out, int M, int N,
+                                                    int m0, int n0, int lane) {
+    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+    const bool vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+        const int m = m0 + b * 16 + (lane & 15);
+        if (m >= M) continue;
+        h16* orow = out + (size_t)m * N;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int n = n0 + a * 16 + 4 * (lane >> 4);
+            if (n >= N) continue;
+            h16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                o[r] = to_half(swiglu1((float)to_half(acc[a][b][r]), (float)to_half(acc[a + 2][b][r])));
+            if (vec && n + 3 < N) {
+                *reinterpret_cast<h16x4*>(orow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) orow[n + r] = o[r];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(Dma64Shape<256>::kWaves * kWave, 2) void gemm_dma64_swiglu(
+    const h16* __restrict__ A, const h16* __restrict__ Wg, const h16* __restrict__ Wu, h16* __restrict__ out, int M,
+    int N, int K) {
+    constexpr int TM = Dma64Shape<256>::TM;
+    auto epilogue = [=](const f32x4 (&acc)[4][TM], int m0, int n0, int lane) {
+        store_tile16_swiglu<TM>(acc, out, M, N, m0, n0, lane);
+    };
+    mfma_dma64<F16Op, 256, 2, 2>(A, Wg, M, N, K * 2, epilogue, Wu);
+}
+
 // M == 1: bound by the weight bytes. kSplit waves share an output column (a
 // weight row), each streaming a contiguous 1/kSplit of it with non-temporal
 // 16-byte loads, four in flight; their sums meet in LDS. Narrow outputs take
@@ -1137,6 +1181,33 @@ vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias
     const vv_status_t s = vv::gemm(A, W, C, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
     if (s != VV_OK) return s;
     return vv_rope128_from_table(C, bias, rope_table, M, n_heads, stream);
+}
+
+vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_up, void* gate, void* up,
+                               void* out, int M, int N, int K, void* stream) {
+    if (!A || !w_gate || !w_up || !out) return VV_ERR_NULL_PTR;
+    if (M <= 0 || N <= 0) return VV_OK;
+    if (K < 0) return VV_ERR_INVALID_ARG;
+    // The fused tile where vv_gemm_fp16_dev itself would run its copy-fed 16x16x32 tiles (they all add K in one
+    // order, whatever their size): more than 64 rows of whole 64-half slabs at 16-byte aligned addresses.
+    if (vv::dma64_serves(M, K) && K > 0 && vv::aligned16(A) && vv::aligned16(w_gate) && vv::aligned16(w_up)) {
+        typedef vv::Dma64Shape<256, 2> Shape;
+        static thread_local int ready = -1;
+        if (vv::allow_big_lds(vv::gemm_dma64_swiglu, ready, Shape::kLdsBytes)) {
+            vv::gemm_dma64_swiglu<<<dim3(vv::dma64_grid<256>(M, 2 * N)), Shape::kWaves * vv::kWave, Shape::kLdsBytes,
+                                    vv::as_stream(stream)>>>(
+                static_cast<const vv::h16*>(A), static_cast<const vv::h16*>(w_gate),
+                static_cast<const vv::h16*>(w_up), static_cast<vv::h16*>(out), M, N, K);
+            return vv::launch_status();
+        }
+    }
+    // Everything else: the three steps one after the other, through the caller's gate and up buffers.
+    if (!gate || !up || (size_t)M * (size_t)N > 0x7fffffffu) return VV_ERR_UNSUPPORTED;
+    vv_status_t s = vv::gemm(A, w_gate, gate, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
+    if (s != VV_OK) return s;
+    s = vv::gemm(A, w_up, up, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
+    if (s != VV_OK) return s;
+    return vv_swiglu_dev(gate, up, out, M * N, stream);
 }
 
 vv_status_t vv_gemm_fp16_tile_dev(const void* A, const void* B, void* C, int M, int N, int K,

@@ -289,9 +289,15 @@ inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N, kTile).grid(); 
 //                                            16 (a % 2) + 64 (a / 2): tiles a and a + 2 are 64 columns apart
 // The MFMAs of a step run x tile by x tile, so an x fragment is dead after four MFMAs and the next step's
 // takes its registers at once: only the four w fragments and the last two x fragments are held twice.
-template <typename Op, int kTile = 256, bool kPairN = false, int kStages = 2, typename Epi>
+// kPairN = 2 (256x256 tile only): TWO B operands of N rows each. A tile's 256 B rows are rows n .. n + 127 of B and
+// the same rows of B2, and wave wn takes columns 32 wn .. + 31 of both: acc[a] and acc[a + 2] are the products of
+// one output column with the two matrices (gate and up of a gated MLP), in the same lane and register. N counts
+// the columns of one matrix; a tile covers 128 of them; the epilogue's n0 is the first of the wave's 32.
+template <typename Op, int kTile = 256, int kPairN = 0, int kStages = 2, typename Epi>
 __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const void* __restrict__ B, int M, int N,
-                                           int row_bytes, const Epi& epi) {
+                                           int row_bytes, const Epi& epi, const void* __restrict__ B2 = nullptr) {
+    static_assert(kPairN != 2 || kTile == 256, "the two-operand layout is the 256x256 tile's");
+    constexpr int kTileN = kPairN == 2 ? kTile / 2 : kTile;          // columns of C (of one matrix) per tile
     typedef typename Op::Acc16 Acc;
     typedef Dma64Shape<kTile, kStages> Shape;
     constexpr int kSlabChunks = kDma64SlabBytes / 16;     // 8
@@ -303,10 +309,10 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const Dma64Map map(M, N, kTile);
+    const Dma64Map map(M, kPairN == 2 ? 2 * N : N, kTile);
     int tile_m, tile_n;
     if (!map.tile((int)blockIdx.x, tile_m, tile_n)) return;      // the whole workgroup, before any barrier
-    const int m_blk = tile_m * kTile, n_blk = tile_n * kTile;
+    const int m_blk = tile_m * kTile, n_blk = tile_n * kTileN;
     const int nslabs = row_bytes / kDma64SlabBytes;
     const uint32_t lds0 =
         (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
@@ -316,6 +322,7 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     // logical slot that the swizzle maps there: a byte offset from the tile's first row, the same for every slab.
     const char* a_tile = static_cast<const char*>(A) + (size_t)m_blk * row_bytes;
     const char* b_tile = static_cast<const char*>(B) + (size_t)n_blk * row_bytes;
+    const char* b2_tile = kPairN == 2 ? static_cast<const char*>(B2) + (size_t)n_blk * row_bytes : b_tile;
     uint32_t src[kLoads], dst[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
@@ -323,14 +330,17 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
         const int p = slot0 + lane;
         const int row = p / kSlabChunks, phys = p % kSlabChunks;
         const int logical = swz<64>(row, phys);
-        const int r = i < kLoads / 2 ? min(row, M - 1 - m_blk) : min(row - kTile, N - 1 - n_blk);
+        // two operands: the B rows of copies 4, 5 are rows 0 .. 127 of B's tile, those of copies 6, 7 of B2's
+        const int b_row = kPairN == 2 ? (row - kTile) % kTileN : row - kTile;
+        const int r = i < kLoads / 2 ? min(row, M - 1 - m_blk) : min(b_row, N - 1 - n_blk);
         src[i] = (uint32_t)r * (uint32_t)row_bytes + (uint32_t)logical * 16u;
         dst[i] = lds0 + (uint32_t)slot0 * 16u;
     }
     auto request = [&](int slab, int i) {        // slab -> stage slab % kStages; past the end: the last slab again
         const size_t adv = (size_t)min(slab, nslabs - 1) * kDma64SlabBytes;
         const uint32_t stage = (uint32_t)(slab & (kStages - 1)) * (kStageSlots * 16u);
-        lds_dma16_at((i < kLoads / 2 ? a_tile : b_tile) + adv, src[i], dst[i] + stage);
+        const char* tile = i < kLoads / 2 ? a_tile : (kPairN == 2 && i >= 3 * kLoads / 4) ? b2_tile : b_tile;
+        lds_dma16_at(tile + adv, src[i], dst[i] + stage);
     };
 
     Acc acc[TN][TM];
@@ -347,9 +357,13 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     for (int step = 0; step < 2; ++step)
         f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 4 + fquarter);
     const int fa_base = wm * TM * 16 * kSlabChunks;
-    const int wave_n0 = kPairN ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 16;      // first column of tile a = 0
+    // first B row of the wave's tile a = 0, and tile a's distance from it
+    const int wave_n0 = kPairN == 2 ? wn * 32 : kPairN == 1 ? (wn >> 1) * 128 + (wn & 1) * 32 : wn * TN * 16;
     const int fb_base = kTile * kSlabChunks + wave_n0 * kSlabChunks;
-    auto w_off = [](int a) { return (kPairN ? (a & 1) * 16 + (a >> 1) * 64 : a * 16) * kSlabChunks; };
+    auto w_off = [](int a) {
+        return (kPairN == 2 ? (a & 1) * 16 + (a >> 1) * 128 : kPairN == 1 ? (a & 1) * 16 + (a >> 1) * 64 : a * 16) *
+               kSlabChunks;
+    };
 
     // w: the K step in hand and the next. x: one set, refilled in place, except the last two tiles of a step,
     // which are held twice like w (their refill could only follow the step's last MFMAs, and the reads of a

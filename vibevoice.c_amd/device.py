@@ -111,6 +111,7 @@ SIGNATURES = {
     "vv_argmax_dev": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "vv_skinny_linear_dev": (_i, [_vp, _i, _vp, _i, _i, _i, _f, _vp]),
     "vv_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vv_gemm_swiglu_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "vv_w4a16_gemv_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "vv_w4a16_gemv_multi_dev": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "vv_w4a16_gather_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
