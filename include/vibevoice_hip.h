@@ -717,7 +717,8 @@ vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int 
  * never written. Fused for M > 64, K % 64 == 0 and 16-byte aligned A, Wg, Wu;
  * every other shape runs the three calls through the caller's `gate` and `up`
  * buffers ([M, N] each; NULL: VV_ERR_UNSUPPORTED for those shapes, nothing
- * launched). The fused path does not touch `gate` and `up`. */
+ * launched). The fused path does not touch `gate` and `up`; `out` may be `gate`
+ * (as vv_swiglu_dev's output may be its gate input). */
 vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_up, void* gate,
                                void* up, void* out, int M, int N, int K, void* stream);
 
