@@ -1190,7 +1190,8 @@ vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_
     if (K < 0) return VV_ERR_INVALID_ARG;
     // The fused tile where vv_gemm_fp16_dev itself would run its copy-fed 16x16x32 tiles (they all add K in one
     // order, whatever their size): more than 64 rows of whole 64-half slabs at 16-byte aligned addresses.
-    if (vv::dma64_serves(M, K) && K > 0 && vv::aligned16(A) && vv::aligned16(w_gate) && vv::aligned16(w_up)) {
+    if (vv::dma64_serves(M, K) && K > 0 && N <= (1 << 29) && vv::aligned16(A) && vv::aligned16(w_gate) &&
+        vv::aligned16(w_up)) {
         typedef vv::Dma64Shape<256, 2> Shape;
         static thread_local int ready = -1;
         if (vv::allow_big_lds(vv::gemm_dma64_swiglu, ready, Shape::kLdsBytes)) {
