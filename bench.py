@@ -650,8 +650,9 @@ def layer_leg(torch, dev, T: int, st: int, fp16_only: bool = False) -> dict:
 
 def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
     """One dense decoder layer over the whole T-row prompt, in the reference decoder's op order
-    (decoder.c:706-991) on this library's entry points: norm, q/k/v GEMMs, bias + RoPE, causal
-    attention over the chunk's own K/V, o GEMM, add+norm, gate/up GEMMs, SwiGLU, down GEMM, add+norm.
+    (decoder.c:706-991), from its normed input to the next layer's: q/k/v GEMMs, bias + RoPE, causal
+    attention over the chunk's own K/V, o GEMM, add + norm, gate/up GEMMs, SwiGLU, down GEMM, add + norm -
+    once on this library's fused entry points, once on the calls of the reference's device.h alone.
     Random weights. Reports the layer time and what 28 such layers make in prompt tokens per second."""
     import ctypes as C
     f16 = dict(dtype=torch.float16, device="cuda")
@@ -677,28 +678,41 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
     assert dev.vv_rope_table_dev(P(rope_table), T, HD, 0, None, THETA, st) == 0
 
     def layer(fused=True):
-        assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0
-        if fused:       # bias + RoPE in the projection's store
+        """One layer from its normed input to the next layer's normed input. fused: this library's fused
+        entry points; else only the calls of the reference's device.h, in decoder.c's order (706-991)."""
+        if fused:
+            # bias + RoPE in the q / k projections' store
             assert dev.vv_gemm_bias_rope_dev(P(normed), P(wq), P(bq), P(q), T, NQ, HD, H, P(rope_table), st) == 0
             assert dev.vv_gemm_bias_rope_dev(P(normed), P(wk), P(bk), P(k), T, NK, HD, H, P(rope_table), st) == 0
+            gemm(normed, wv, v, KD, H)
+            assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
         else:
             gemm(normed, wq, q, QD, H)
             gemm(normed, wk, k, KD, H)
-        gemm(normed, wv, v, KD, H)
-        if not fused:
-            assert dev.vv_bias_rope_qk_dev(P(q), P(k), P(bq), P(bk), T, NQ, NK, HD, 0, None, THETA, st) == 0
-        assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
+            gemm(normed, wv, v, KD, H)
+            assert dev.vv_bias_add_dev(P(q), P(bq), T, QD, st) == 0
+            assert dev.vv_bias_add_dev(P(k), P(bk), T, KD, st) == 0
+            assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
+            assert dev.vv_rope_dev(P(q), T, NQ, HD, 0, None, THETA, st) == 0
+            assert dev.vv_rope_dev(P(k), T, NK, HD, 0, None, THETA, st) == 0
         assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, T, 0, T, True, None, st) == 0
         gemm(attn, wo, proj, H, QD)
-        assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n2), P(normed), T, H, EPS, st) == 0
-        if fused:       # gate, up and SwiGLU in one GEMM: gate and up are never written
+        if fused:
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n2), P(normed), T, H, EPS, st) == 0
+            # gate, up and SwiGLU in one GEMM: gate and up are never written
             assert dev.vv_gemm_swiglu_dev(P(normed), P(wg), P(wu), None, None, P(gate), T, I_FF, H, st) == 0
         else:
+            assert dev.vv_residual_add_dev(P(hidden), P(proj), T * H, st) == 0
+            assert dev.vv_rmsnorm_dev(P(hidden), P(n2), P(normed), T, H, EPS, st) == 0
             gemm(normed, wg, gate, I_FF, H)
             gemm(normed, wu, up, I_FF, H)
             assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), T * I_FF, st) == 0
         gemm(gate, wd, proj, H, I_FF)
-        assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
+        if fused:       # the residual add and the next layer's input norm in one launch
+            assert dev.vv_add_rmsnorm_dev(P(hidden), P(proj), P(n1), P(normed), T, H, EPS, st) == 0
+        else:
+            assert dev.vv_residual_add_dev(P(hidden), P(proj), T * H, st) == 0
+            assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0
 
     def time_layer(fused):
         layer(fused)
@@ -714,6 +728,7 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
         per.sort()
         return per[1]
 
+    assert dev.vv_rmsnorm_dev(P(hidden), P(n1), P(normed), T, H, EPS, st) == 0      # layer 0's input norm
     ms_separate = time_layer(False)
     ms = time_layer(True)
     assert bool(torch.isfinite(hidden).all())
@@ -1230,7 +1245,7 @@ def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
         log("  Conv-VAE ops (512 channels x 24000 columns): " + ", ".join(f"{k} {v:.1f}" for k, v in d.items()))
     layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
     log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
-        f"{d['ms_per_layer_reference_api_calls']:.2f} ms with bias + RoPE and SwiGLU as launches of their own); "
+        f"{d['ms_per_layer_reference_api_calls']:.2f} ms on the calls of the reference's device.h alone); "
         f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
     for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
         torch.cuda.empty_cache()
