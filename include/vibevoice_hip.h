@@ -715,7 +715,8 @@ vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int 
  * two GEMMs store and go through the SwiGLU kernel's own function in the GEMM's
  * store, so the result equals the three calls bit for bit and gate and up are
  * never written. Fused for M > 64, K % 64 == 0 and 16-byte aligned A, Wg, Wu;
- * every other shape runs the three calls through the caller's `gate` and `up`
+ * one row runs vv_gemv_swiglu_dev; every other shape runs the three calls through
+ * the caller's `gate` and `up`
  * buffers ([M, N] each; NULL: VV_ERR_UNSUPPORTED for those shapes, nothing
  * launched). The fused path does not touch `gate` and `up`; `out` may be `gate`
  * (as vv_swiglu_dev's output may be its gate input). */

@@ -59,7 +59,17 @@ def test_fused_equals_the_three_calls(M, N, K):
     assert st == dev.VV_OK and np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("M,N,K", [(64, 300, 128), (9, 100, 64), (1, 512, 256), (200, 96, 72), (300, 64, 8)])
+@pytest.mark.parametrize("N,K", [(512, 256), (18944, 3584), (37, 8)])
+def test_one_row_runs_the_decode_launch(N, K):
+    d_a = to_dev(oracle.normal_f16((1, K), 41))
+    d_g = to_dev(oracle.normal_f16((N, K), 42, std=K ** -0.5))
+    d_u = to_dev(oracle.normal_f16((N, K), 43, std=K ** -0.5))
+    _, _, want = separate(d_a, d_g, d_u, 1, N, K)
+    st, got, _ = fused(d_a, d_g, d_u, 1, N, K, buffers=False)
+    assert st == dev.VV_OK and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 300, 128), (9, 100, 64), (2, 512, 256), (200, 96, 72), (300, 64, 8)])
 def test_other_shapes_run_the_three_calls(M, N, K):
     """Up to 64 rows, or rows that are not whole 64-half slabs: through the caller's buffers, or declined."""
     d_a = to_dev(oracle.normal_f16((M, K), 21))

@@ -1202,6 +1202,8 @@ vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_
             return vv::launch_status();
         }
     }
+    // One row: the decode step's own fused launch (equal to the three calls by its own contract).
+    if (M == 1 && vv_gemv_swiglu_dev(A, w_gate, w_up, out, N, K, stream) == VV_OK) return VV_OK;
     // Everything else: the three steps one after the other, through the caller's gate and up buffers.
     if (!gate || !up || (size_t)M * (size_t)N > 0x7fffffffu) return VV_ERR_UNSUPPORTED;
     vv_status_t s = vv::gemm(A, w_gate, gate, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
