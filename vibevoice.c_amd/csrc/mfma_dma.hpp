@@ -285,7 +285,7 @@ inline unsigned dma64_grid(int M, int N) { return Dma64Map(M, N, kTile).grid(); 
 //   Op::Acc16                                4-wide accumulator vector
 //   Op::mfma16(u32x4 w, u32x4 x, Acc16 c)    one 16x16 product over a K step
 //   epi(acc, m0, n0, lane)                   register r of lane l: column n0 + off(a) + 4 (l / 16) + r of row
-//                                            m0 + 16 b + l % 16, for acc[a][b]; off(a) = 16 a, or with kPairN
+//                                            m0 + 16 b + l % 16, for acc[a][b]; off(a) = 16 a, or with kPairN = 1
 //                                            16 (a % 2) + 64 (a / 2): tiles a and a + 2 are 64 columns apart
 // The MFMAs of a step run x tile by x tile, so an x fragment is dead after four MFMAs and the next step's
 // takes its registers at once: only the four w fragments and the last two x fragments are held twice.
