@@ -461,8 +461,8 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
 // of a wave are lane swaps in the vector ALU (max_xor32, sum_xor32); the row maximum of the next tile
 // is taken behind the first V^T P^T MFMAs, so that the exponentials spread over all sixteen score
 // MFMAs: 1691 -> 1501 us together.
-// Workgroups are ordered heaviest first across ALL heads (the head is the fast grid index), which
-// alone is worth 12 % of a causal 14k prompt over "heaviest first per head".
+// Workgroups are ordered heaviest first across ALL heads, which alone is worth 12 % of a causal 14k
+// prompt over "heaviest first per head"; the query heads of one KV head share an XCD (see the kernel).
 template <int kValue> struct Parity { static constexpr int value = kValue; };
 struct PipeTiles {
     Chunk k[2][kKeyTile * 16];                   // [buffer][key][16 slots], slot ^ (key & 15)
@@ -485,9 +485,17 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
-    const int head = (int)blockIdx.x;
-    const int kvh = head / (n_q_heads / n_kv_heads);
-    const int q0 = (int)(gridDim.y - 1 - blockIdx.y) * kQTile;
+    // Workgroup i runs on XCD i % 8 as that XCD's (i / 8)-th. The query heads of one KV head that work on the same
+    // rows read the same K and V tiles at the same time: such a group is kept on ONE XCD (one L2), its members next
+    // to each other in that XCD's order, and the groups are dealt to the XCDs heaviest rows first.
+    const int group_heads = n_q_heads / n_kv_heads;
+    const int n_row_tiles = (q_len + kQTile - 1) / kQTile;
+    const int xcd = (int)blockIdx.x & 7, nth = (int)blockIdx.x >> 3;
+    const int group = (nth / group_heads) * 8 + xcd;              // (row tile, KV head), heaviest first
+    if (group >= n_row_tiles * n_kv_heads) return;                // the whole workgroup, before any barrier
+    const int kvh = group % n_kv_heads;
+    const int head = kvh * group_heads + nth % group_heads;
+    const int q0 = (n_row_tiles - 1 - group / n_kv_heads) * kQTile;
     const int qw0 = q0 + wave * 32;
     const int qrow = qw0 + col;
     const int q_abs = q_offset + qrow;
@@ -1557,7 +1565,8 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
 #undef VV_PREFILL
     } else if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
                vv::aligned16(out)) {
-        const dim3 grid((unsigned)n_q_heads, (unsigned)((q_len + vv::kQTile - 1) / vv::kQTile));
+        const int groups = kv->n_kv_heads * ((q_len + vv::kQTile - 1) / vv::kQTile);     // see the kernel's numbering
+        const dim3 grid((unsigned)(8 * ((groups + 7) / 8) * (n_q_heads / kv->n_kv_heads)));
         vv::prefill_pipe<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads, kv->n_kv_heads, q_len,
                                                       q_offset, kv_len, causal ? 1 : 0, scale_log2);
     } else {
