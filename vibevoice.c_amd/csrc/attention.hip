@@ -1555,7 +1555,15 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
     vv::h16* O = static_cast<vv::h16*>(out);
     const vv::KvSource src = {kv->k, kv->v, static_cast<const vv::h16*>(kv->k_meta),
                               static_cast<const vv::h16*>(kv->v_meta), kv->page_table};
-    if (packed) {
+    // A/B aid for the parity tests: the plain tile kernel on an FP16 cache (same bits as the pipelined one).
+    const char* force_tile = getenv("VV_ATTN_PREFILL_TILE");
+    const bool tile_fp16 = !packed && force_tile && force_tile[0] == '1' && kv->head_dim == vv::kD &&
+                           vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) && vv::aligned16(out);
+    if (tile_fp16) {
+        const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
+        vv::prefill128<vv::kFmtFp16><<<grid, vv::kBlock, 0, st>>>(Q, src, O, n_q_heads, kv->n_kv_heads, q_len,
+                                                                  q_offset, kv_len, causal ? 1 : 0, scale_log2);
+    } else if (packed) {
         const dim3 grid((unsigned)((q_len + vv::kQTile - 1) / vv::kQTile), (unsigned)n_q_heads);
 #define VV_PREFILL(F)                                                                                          \
     vv::prefill128<vv::F><<<grid, vv::kBlock, 0, st>>>(Q, src, O, n_q_heads, kv->n_kv_heads, q_len, q_offset, \
