@@ -681,11 +681,10 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
         """One layer from its normed input to the next layer's normed input. fused: this library's fused
         entry points; else only the calls of the reference's device.h, in decoder.c's order (706-991)."""
         if fused:
-            # bias + RoPE in the q / k projections' store
-            assert dev.vv_gemm_bias_rope_dev(P(normed), P(wq), P(bq), P(q), T, NQ, HD, H, P(rope_table), st) == 0
-            assert dev.vv_gemm_bias_rope_dev(P(normed), P(wk), P(bk), P(k), T, NK, HD, H, P(rope_table), st) == 0
-            gemm(normed, wv, v, KD, H)
-            assert dev.vv_bias_add_dev(P(v), P(bv), T, KD, st) == 0
+            # q / k / v with bias + RoPE in the store (one grid of equal tiles up to ~9000 rows, else one launch
+            # per projection with bias + RoPE in the q / k stores)
+            assert dev.vv_gemm_qkv_rope_dev(P(normed), P(wq), P(wk), P(wv), P(bq), P(bk), P(bv), P(q), P(k), P(v), T,
+                                            NQ, NK, HD, H, P(rope_table), None, None, None, 0, None, st) == 0
         else:
             gemm(normed, wq, q, QD, H)
             gemm(normed, wk, k, KD, H)
@@ -734,6 +733,126 @@ def prefill_layer_leg(torch, dev, T: int, st: int) -> dict:
     assert bool(torch.isfinite(hidden).all())
     flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
     return {"rows": T, "ms_per_layer": ms, "ms_per_layer_reference_api_calls": ms_separate,
+            "TFLOPs": flops / ms / 1e9, "layers_assumed": 28, "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
+
+
+def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
+    """One dense decoder layer over a T-row prompt THE WAY THE REFERENCE RUNS IT (decoder.c:1095-1241): chunks of
+    at most 2048 rows (7 x 2048 + 113 at T = 14449), each through the layer in decoder_layer_impl's order
+    (decoder.c:706-991) - q/k/v projections, bias, RoPE, KV append at the chunk's positions, causal attention of the
+    chunk against the cache grown so far, o projection, add + norm, gate/up, SwiGLU, down, add + norm - once on this
+    library's fused entry points (q/k/v + bias + RoPE + append in one launch), once on the calls of the reference's
+    device.h alone. Random weights; the normed input of every chunk (the previous layer's output) is made before
+    the clock starts. Reports ms per layer, per chunk, and the q/k/v leg of a full chunk alone."""
+    import ctypes as C
+    f16 = dict(dtype=torch.float16, device="cuda")
+    QD, KD = NQ * HD, NK * HD
+    w = lambda *shape, std: torch.randn(*shape, **f16) * std
+    wq, wk, wv, wo = w(QD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(H, QD, std=QD ** -0.5)
+    wg, wu, wd = w(I_FF, H, std=H ** -0.5), w(I_FF, H, std=H ** -0.5), w(H, I_FF, std=I_FF ** -0.5)
+    bq, bk, bv = w(QD, std=0.1), w(KD, std=0.1), w(KD, std=0.1)
+    n1, n2 = 1 + w(H, std=0.1), 1 + w(H, std=0.1)
+    C_ROWS = min(chunk, T)
+    hidden0, normed_in = w(T, H, std=1.0), torch.empty(T, H, **f16)
+    hidden = torch.empty(T, H, **f16)
+    normed, proj = torch.empty(C_ROWS, H, **f16), torch.empty(C_ROWS, H, **f16)
+    q, attn = torch.empty(C_ROWS, QD, **f16), torch.empty(C_ROWS, QD, **f16)
+    k, v = torch.empty(C_ROWS, KD, **f16), torch.empty(C_ROWS, KD, **f16)
+    gate, up = torch.empty(C_ROWS, I_FF, **f16), torch.empty(C_ROWS, I_FF, **f16)
+    kc, vc = torch.empty(T, KD, **f16), torch.empty(T, KD, **f16)
+    view = dev.KvView(k=kc.data_ptr(), v=vc.data_ptr(), k_meta=None, v_meta=None, page_table=None, format=0,
+                      n_kv_heads=NK, head_dim=HD)
+    P = lambda t: t.data_ptr()
+    rope_table = torch.empty(T, HD // 2, 2, dtype=torch.float32, device="cuda")
+    assert dev.vv_rope_table_dev(P(rope_table), T, HD, 0, None, THETA, st) == 0
+    assert dev.vv_rmsnorm_dev(P(hidden0), P(n1), P(normed_in), T, H, EPS, st) == 0
+    chunks = [(s0, min(chunk, T - s0)) for s0 in range(0, T, chunk)]
+
+    def gemm(x, wt, y, m, n, kk):
+        assert dev.vv_gemm_fp16_dev(x, P(wt), P(y), m, n, kk, 1.0, 0.0, st) == 0
+
+    def qkv(start, n, fused):
+        x = P(normed_in) + start * H * 2
+        if fused:
+            assert dev.vv_gemm_qkv_rope_dev(x, P(wq), P(wk), P(wv), P(bq), P(bk), P(bv), P(q), None, None, n, NQ, NK,
+                                            HD, H, P(rope_table) + start * HD * 4, P(kc), P(vc), None, start, None,
+                                            st) == 0
+            return
+        gemm(x, wq, q, n, QD, H)
+        gemm(x, wk, k, n, KD, H)
+        gemm(x, wv, v, n, KD, H)
+        assert dev.vv_bias_add_dev(P(q), P(bq), n, QD, st) == 0
+        assert dev.vv_bias_add_dev(P(k), P(bk), n, KD, st) == 0
+        assert dev.vv_bias_add_dev(P(v), P(bv), n, KD, st) == 0
+        assert dev.vv_rope_dev(P(q), n, NQ, HD, start, None, THETA, st) == 0
+        assert dev.vv_rope_dev(P(k), n, NK, HD, start, None, THETA, st) == 0
+        # the contiguous cache's append (kv_cache.c:238-245): two device copies
+        assert dev.vv_dev_memcpy_d2d(P(kc) + start * KD * 2, P(k), n * KD * 2, st) == 0
+        assert dev.vv_dev_memcpy_d2d(P(vc) + start * KD * 2, P(v), n * KD * 2, st) == 0
+
+    def one_chunk(start, n, fused):
+        h = P(hidden) + start * H * 2
+        qkv(start, n, fused)
+        assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, n, start, start + n, True, None, st) == 0
+        gemm(P(attn), wo, proj, n, H, QD)
+        if fused:
+            assert dev.vv_add_rmsnorm_dev(h, P(proj), P(n2), P(normed), n, H, EPS, st) == 0
+            assert dev.vv_gemm_swiglu_dev(P(normed), P(wg), P(wu), P(gate), P(up), P(gate), n, I_FF, H, st) == 0
+        else:
+            assert dev.vv_residual_add_dev(h, P(proj), n * H, st) == 0
+            assert dev.vv_rmsnorm_dev(h, P(n2), P(normed), n, H, EPS, st) == 0
+            gemm(P(normed), wg, gate, n, I_FF, H)
+            gemm(P(normed), wu, up, n, I_FF, H)
+            assert dev.vv_swiglu_dev(P(gate), P(up), P(gate), n * I_FF, st) == 0
+        gemm(P(gate), wd, proj, n, H, I_FF)
+        if fused:       # the residual add and the next layer's input norm in one launch
+            assert dev.vv_add_rmsnorm_dev(h, P(proj), P(n1), P(normed), n, H, EPS, st) == 0
+        else:
+            assert dev.vv_residual_add_dev(h, P(proj), n * H, st) == 0
+            assert dev.vv_rmsnorm_dev(h, P(n1), P(normed), n, H, EPS, st) == 0
+
+    def time_layer(fused):
+        per, per_chunk = [], None
+        for rep in range(4):
+            hidden.copy_(hidden0)
+            torch.cuda.synchronize()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(chunks) + 1)]
+            ev[0].record()
+            for i, (s0, n) in enumerate(chunks):
+                one_chunk(s0, n, fused)
+                ev[i + 1].record()
+            ev[-1].synchronize()
+            if rep:                                      # the first pass warms up
+                per.append((ev[0].elapsed_time(ev[-1]), [ev[i].elapsed_time(ev[i + 1]) for i in range(len(chunks))]))
+        per.sort(key=lambda t: t[0])
+        return per[len(per) // 2]
+
+    def time_qkv(fused, launches=10):
+        s0, n = chunks[-2] if len(chunks) > 1 else chunks[0]
+        qkv(s0, n, fused)
+        per = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(launches):
+                qkv(s0, n, fused)
+            e1.record()
+            e1.synchronize()
+            per.append(e0.elapsed_time(e1) * 1e3 / launches)
+        per.sort()
+        return n, per[1]
+
+    ms_api, chunks_api = time_layer(False)
+    ms, chunks_ms = time_layer(True)
+    assert bool(torch.isfinite(hidden).all())
+    rows_qkv, us_qkv = time_qkv(True)
+    _, us_qkv_api = time_qkv(False)
+    flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
+    return {"rows": T, "chunk_rows": [n for _, n in chunks], "ms_per_layer": ms, "ms_per_chunk": chunks_ms,
+            "ms_per_layer_reference_api_calls": ms_api, "ms_per_chunk_reference_api_calls": chunks_api,
+            "launches_per_chunk": 7, "launches_per_chunk_reference_api_calls": 20,
+            "qkv_leg": {"rows": rows_qkv, "us": us_qkv, "us_reference_api_calls": us_qkv_api,
+                        "TFLOPs": 2.0 * rows_qkv * (QD + 2 * KD) * H / us_qkv / 1e6},
             "TFLOPs": flops / ms / 1e9, "layers_assumed": 28, "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
 
 
@@ -1246,6 +1365,13 @@ def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
     layer["prefill_layer"] = d = prefill_layer_leg(torch, dev, T, st)
     log(f"  prefill layer, T={T}: {d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s over GEMMs + attention; "
         f"{d['ms_per_layer_reference_api_calls']:.2f} ms on the calls of the reference's device.h alone); "
+        f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
+    torch.cuda.empty_cache()
+    layer["prefill_chunked"] = d = prefill_chunked_leg(torch, dev, T, st)
+    log(f"  prefill layer in {len(d['chunk_rows'])} chunks of <= 2048 rows (the reference's launch pattern), T={T}: "
+        f"{d['ms_per_layer']:.2f} ms ({d['TFLOPs']:.0f} TFLOP/s; {d['ms_per_layer_reference_api_calls']:.2f} ms on the "
+        f"calls of the reference's device.h alone); q/k/v + bias + RoPE + append of {d['qkv_leg']['rows']} rows "
+        f"{d['qkv_leg']['us']:.1f} us in one launch, {d['qkv_leg']['us_reference_api_calls']:.1f} us in ten; "
         f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
     for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
         torch.cuda.empty_cache()

@@ -681,9 +681,12 @@ vv_status_t vv_bias_rope_qk_dev(void* q, void* k, const void* q_bias,
  * every layer that rotates at those positions (src/inference/decoder.c:850-855 runs
  * the same rotation in each of the 28 layers): table[row][i] = {cos, sin} of
  * (float)(first + row) * theta^(-2i/head_dim), i < head_dim/2, as FP32 pairs
- * (8 * seq_len * head_dim/2 bytes, 16-byte aligned), first = *d_position when
- * d_position is given, else position_offset. The angle and the full-range sincosf
- * are those of vv_rope_dev, so a rotation that reads the table gives its bits. */
+ * (8 * seq_len * head_dim/2 bytes; a table that is not 16-byte aligned is
+ * VV_ERR_UNSUPPORTED, the status its readers return for one), first = *d_position
+ * when d_position is given, else position_offset. The angle and the full-range
+ * sincosf are those of vv_rope_dev, so a rotation that reads the table gives its
+ * bits. vv_gemm_bias_rope_dev and vv_gemm_qkv_rope_dev read rows of 64 pairs: they
+ * need a table built with head_dim == 128. */
 vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int position_offset,
                               const int* d_position, float theta, void* stream);
 
@@ -699,6 +702,30 @@ vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int positi
 vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias, void* C,
                                   int M, int n_heads, int head_dim, int K,
                                   const void* rope_table, void* stream);
+
+/* addition: the q, k and v projections of a prefill chunk in ONE launch - the whole of
+ * decoder.c:815-867 on the dense FP16 path (quant_linear_group :478-505 = three
+ * vv_gemm_fp16_dev + vv_bias_add_dev, vv_rope_dev twice :849-855, the KV append
+ * :864-867): q[M, n_q_heads*128] = rope(fp16(x Wq^T) + bq), k likewise with Wk / bk,
+ * v[M, n_kv_heads*128] = fp16(x Wv^T) + bv, row m rotated by row m of a
+ * vv_rope_table_dev table (built with head_dim 128 for the chunk's positions). With
+ * k_cache / v_cache (FP16 [positions][n_kv_heads][128], contiguous or behind a table
+ * of 64-position pages) the k and v rows also land at positions first .. first+M-1,
+ * first = *d_pos when d_pos is given, else pos; k and v may then be NULL. Every step
+ * rounds to FP16 where the separate calls store: the result equals
+ * vv_gemm_bias_rope_dev (q), vv_gemm_bias_rope_dev (k), vv_gemm_fp16_dev +
+ * vv_bias_add_dev (v) and vv_kv_store_dev bit for bit. One grid of equal tiles serves
+ * 7 query heads per KV head with head_dim 128 (28 + 4 heads: a tile is one q or k head
+ * plus 16 columns of v), more than 64 rows, K % 64 == 0; other shapes run the separate
+ * calls through k and v (VV_ERR_UNSUPPORTED if those are NULL). Biases may be NULL.
+ * q, k, v, the caches, the biases and the table must be 16-byte aligned
+ * (VV_ERR_UNSUPPORTED otherwise, nothing launched). */
+vv_status_t vv_gemm_qkv_rope_dev(const void* x, const void* wq, const void* wk, const void* wv,
+                                 const void* bq, const void* bk, const void* bv, void* q,
+                                 void* k, void* v, int M, int n_q_heads, int n_kv_heads,
+                                 int head_dim, int K, const void* rope_table, void* k_cache,
+                                 void* v_cache, const int* page_table, int pos,
+                                 const int* d_pos, void* stream);
 
 /* addition: one activation row through up to three projections in ONE launch
  * (the decode step's q/k/v): y_i[N_i] = x[K] . W_i^T (+ bias_i). Equals

@@ -149,7 +149,8 @@ def test_the_library_defines_every_symbol_of_the_reference_seam():
     assert have - wanted == {"vv_add_rmsnorm_dev", "vv_rope_qk_dev", "vv_bias_rope_qk_dev",
                              "vv_embedding_rmsnorm_dev", "vv_gemv_multi_dev", "vv_gemv_swiglu_dev",
                              "vv_kv_rotate_dev", "vv_kv_unrotate_dev", "vv_attn_decode_static",
-                             "vv_rope_table_dev", "vv_gemm_bias_rope_dev", "vv_gemm_swiglu_dev"}
+                             "vv_rope_table_dev", "vv_gemm_bias_rope_dev", "vv_gemm_swiglu_dev",
+                             "vv_gemm_qkv_rope_dev"}
 
 
 HOST_ARCHIVE = os.path.join(ROOT, "oracle", "_ref", "host", "libvv_ref_host.a")

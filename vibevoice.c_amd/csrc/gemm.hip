@@ -332,6 +332,120 @@ __global__ __launch_bounds__(Dma64Shape<kTile>::kWaves * kWave, 2) void gemm_dma
     mfma_dma64<F16Op, kTile, true, kStages>(A, B, M, N, K * 2, epilogue);
 }
 
+// The q, k and v projections of a chunk of rows in one grid (mfma_dma64_qkv): tile (tile_m, head) holds 128 rows
+// of one q or k head - bias and RoPE in the store, as gemm_dma64_rope - and of v's columns 16 head .. + 15 (bias
+// in the store). k and v rows go to plain [rows, n_kv_heads * 128] buffers and / or into an FP16 KV cache at
+// positions first .. first + M - 1 (contiguous, or through a table of 64-position pages), so neither the bias
+// add nor the append needs a launch of its own. Every step rounds where the separate launches round.
+struct QkvArgs {
+    const h16 *x, *wq, *wk, *wv, *bq, *bk, *bv;
+    const float2* table;
+    h16 *q, *k, *v, *k_cache, *v_cache;
+    const int* page_table;
+    const int* d_pos;
+    int pos, M, K, n_q_heads, n_kv_heads;
+};
+
+template <int kStages>
+__global__ __launch_bounds__(QkvShape<kStages>::kWaves * kWave, 2) void gemm_dma64_qkv(const QkvArgs g) {
+    typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+    // Workgroup i runs on XCD i % 8 as its (i / 8)-th: an XCD takes eight heads (XCD % 4) and every other row
+    // tile (XCD / 4), eight row tiles at a time, so the 64 workgroups it runs together share 8 + 8 operand tiles.
+    const int xcd = (int)blockIdx.x & 7, nth = (int)blockIdx.x >> 3;
+    const int n_heads = g.n_q_heads + g.n_kv_heads;
+    const int head_groups = n_heads / 8;                       // 4 for 28 + 4 heads
+    const int m_par = 8 / head_groups;                         // XCDs that share a group of heads: 2
+    const int head = (xcd % head_groups) * 8 + (nth & 7);
+    const int tile_m = (nth >> 3) * m_par + xcd / head_groups;
+    const int m_blk = tile_m * 128;
+    if (m_blk >= g.M) return;                                  // the whole workgroup, before any barrier
+    const bool is_q = head < g.n_q_heads;
+    const int kv_head = head - g.n_q_heads;
+    const size_t row_bytes = (size_t)g.K * 2;
+    const char* x = reinterpret_cast<const char*>(g.x) + (size_t)m_blk * row_bytes;
+    const char* w_head = reinterpret_cast<const char*>(is_q ? g.wq + (size_t)head * 128 * g.K
+                                                            : g.wk + (size_t)kv_head * 128 * g.K);
+    const char* w_strip = reinterpret_cast<const char*>(g.wv + (size_t)head * kQkvStrip * g.K);
+    const h16* bias = is_q ? g.bq : g.bk;
+    if (bias) bias += (is_q ? head : kv_head) * 128;
+    const int kv_row = g.n_kv_heads * 128;
+    const int first = g.d_pos ? *g.d_pos : g.pos;
+
+    auto epilogue = [&](const f32x4 (&acc)[4][4], const f32x4 (&accv)[2], int m0, int wn, int lane) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int m = m_blk + m0 + 16 * ((b + 2 * wn) & 3) + (lane & 15);
+            if (m >= g.M) continue;
+            const float2* trow = g.table + (size_t)m * 64;
+            size_t cache_at = 0;
+            if (g.k_cache) {
+                const int t = first + m;
+                cache_at = (size_t)(g.page_table ? g.page_table[t >> 6] * 64 + (t & 63) : t) * kv_row;
+            }
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const int col = 32 * wn + 16 * a + 4 * (lane >> 4);        // the pair is (col, col + 64) of the head
+                h16x4 lo, hi;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    lo[r] = to_half(acc[a][b][r]);
+                    hi[r] = to_half(acc[a + 2][b][r]);
+                }
+                if (bias) {
+                    const h16x4 blo = *reinterpret_cast<const h16x4*>(bias + col);
+                    const h16x4 bhi = *reinterpret_cast<const h16x4*>(bias + col + 64);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        lo[r] = to_half((float)lo[r] + (float)blo[r]);
+                        hi[r] = to_half((float)hi[r] + (float)bhi[r]);
+                    }
+                }
+                const float4 cs01 = *reinterpret_cast<const float4*>(trow + col);
+                const float4 cs23 = *reinterpret_cast<const float4*>(trow + col + 2);
+                const float cv[4] = {cs01.x, cs01.z, cs23.x, cs23.z};
+                const float sv[4] = {cs01.y, cs01.w, cs23.y, cs23.w};
+                h16x4 olo, ohi;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const Pair p = rotate((float)lo[r], (float)hi[r], cv[r], sv[r]);
+                    olo[r] = to_half(p.lo);
+                    ohi[r] = to_half(p.hi);
+                }
+                if (is_q) {
+                    h16* dst = g.q + ((size_t)m * g.n_q_heads + head) * 128 + col;
+                    *reinterpret_cast<h16x4*>(dst) = olo;
+                    *reinterpret_cast<h16x4*>(dst + 64) = ohi;
+                } else {
+                    if (g.k) {
+                        h16* dst = g.k + (size_t)m * kv_row + kv_head * 128 + col;
+                        *reinterpret_cast<h16x4*>(dst) = olo;
+                        *reinterpret_cast<h16x4*>(dst + 64) = ohi;
+                    }
+                    if (g.k_cache) {
+                        h16* dst = g.k_cache + cache_at + kv_head * 128 + col;
+                        *reinterpret_cast<h16x4*>(dst) = olo;
+                        *reinterpret_cast<h16x4*>(dst + 64) = ohi;
+                    }
+                }
+            }
+            if (b < 2) {                                                   // the strip of v: product, then bias
+                const int col = head * kQkvStrip + 4 * (lane >> 4);
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = to_half(accv[b][r]);
+                if (g.bv) {
+                    const h16x4 bb = *reinterpret_cast<const h16x4*>(g.bv + col);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] = to_half((float)o[r] + (float)bb[r]);
+                }
+                if (g.v) *reinterpret_cast<h16x4*>(g.v + (size_t)m * kv_row + col) = o;
+                if (g.v_cache) *reinterpret_cast<h16x4*>(g.v_cache + cache_at + col) = o;
+            }
+        }
+    };
+    mfma_dma64_qkv<F16Op, kStages>(x, w_head, w_strip, g.M - m_blk, (int)row_bytes, epilogue);
+}
+
 // The front half of a gated MLP in one GEMM: out = silu(fp16(A Wg^T)) * fp16(A Wu^T). A tile multiplies 256 rows of A
 // with 128 rows of Wg and the same 128 rows of Wu (mfma_dma64's two-operand layout), so acc[a] and acc[a + 2] of a
 // wave are one output element's gate and up products. Both are rounded to FP16 where the two GEMMs' stores round,
@@ -1003,6 +1117,27 @@ bool gemm_rope(const h16* A, const h16* B, const h16* bias, const float2* table,
     return true;
 }
 
+// The fused q / k / v tile serves: 7 query heads per KV head of 128 channels in groups of eight heads, more than 64
+// rows of whole 64-half slabs (where the separate calls run their copy-fed 16x16x32 tiles too: same K order).
+bool qkv_serves(int M, int n_q_heads, int n_kv_heads, int head_dim, int K) {
+    const int n_heads = n_q_heads + n_kv_heads;
+    return head_dim == 128 && n_kv_heads * 128 == n_heads * kQkvStrip && n_heads % 8 == 0 && 8 % (n_heads / 8) == 0 &&
+           dma64_serves(M, K) && (size_t)K * 2 * 144 < 0x7fffffffu;
+}
+
+template <int kStages>
+bool launch_qkv(const QkvArgs& g, hipStream_t st) {
+    typedef QkvShape<kStages> Shape;
+    static thread_local int ready = -1;
+    if (!allow_big_lds(gemm_dma64_qkv<kStages>, ready, Shape::kLdsBytes)) return false;
+    const int n_heads = g.n_q_heads + g.n_kv_heads;
+    const int m_par = 8 / (n_heads / 8);
+    const int gy = (g.M + 127) / 128;
+    const unsigned grid = 64u * (unsigned)((gy + m_par - 1) / m_par);
+    gemm_dma64_qkv<kStages><<<dim3(grid), Shape::kWaves * kWave, Shape::kLdsBytes, st>>>(g);
+    return true;
+}
+
 int forced_tile() {
     static const int v = [] {
         const char* e = getenv("VV_GEMM_TILE");
@@ -1181,6 +1316,52 @@ vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias
     const vv_status_t s = vv::gemm(A, W, C, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
     if (s != VV_OK) return s;
     return vv_rope128_from_table(C, bias, rope_table, M, n_heads, stream);
+}
+
+vv_status_t vv_gemm_qkv_rope_dev(const void* x, const void* wq, const void* wk, const void* wv, const void* bq,
+                                 const void* bk, const void* bv, void* q, void* k, void* v, int M, int n_q_heads,
+                                 int n_kv_heads, int head_dim, int K, const void* rope_table, void* k_cache,
+                                 void* v_cache, const int* page_table, int pos, const int* d_pos, void* stream) {
+    if (!x || !wq || !wk || !wv || !q || !rope_table) return VV_ERR_NULL_PTR;
+    if ((!k || !v) && (!k_cache || !v_cache)) return VV_ERR_NULL_PTR;
+    if ((k_cache == nullptr) != (v_cache == nullptr)) return VV_ERR_NULL_PTR;
+    if (M <= 0 || n_q_heads <= 0 || n_kv_heads <= 0) return VV_OK;
+    if (K < 0 || pos < 0) return VV_ERR_INVALID_ARG;
+    const void* aligned[] = {q, k, v, k_cache, v_cache, rope_table, bq, bk, bv};
+    for (const void* p : aligned)
+        if (p && !vv::aligned16(p)) return VV_ERR_UNSUPPORTED;
+    if (head_dim != 128) return VV_ERR_UNSUPPORTED;
+    // From the row count at which the q projection fills the chip with 256x256 tiles (two rounds of them), the
+    // separate launches are faster (14449 rows: 490 against 539 us); below, the equal tiles are (2048 rows: 73
+    // against 109 us).
+    const bool big_tiles = (long)((M + 255) / 256) * ((n_q_heads * 128 + 255) / 256) >= 512 && k && v;
+    if (vv::forced_tile() == 0 && !big_tiles && vv::qkv_serves(M, n_q_heads, n_kv_heads, head_dim, K) && vv::aligned16(x) &&
+        vv::aligned16(wq) && vv::aligned16(wk) && vv::aligned16(wv)) {
+        typedef const vv::h16* H;
+        const vv::QkvArgs g = {static_cast<H>(x), static_cast<H>(wq), static_cast<H>(wk), static_cast<H>(wv),
+                               static_cast<H>(bq), static_cast<H>(bk), static_cast<H>(bv),
+                               static_cast<const float2*>(rope_table), static_cast<vv::h16*>(q),
+                               static_cast<vv::h16*>(k), static_cast<vv::h16*>(v), static_cast<vv::h16*>(k_cache),
+                               static_cast<vv::h16*>(v_cache), page_table, d_pos, pos, M, K, n_q_heads, n_kv_heads};
+        // up to 256 tiles a workgroup has its compute unit to itself and asks for its slabs four ahead
+        const long tiles = (long)((M + 127) / 128) * (n_q_heads + n_kv_heads);
+        if (tiles <= 256 ? vv::launch_qkv<4>(g, vv::as_stream(stream)) : vv::launch_qkv<2>(g, vv::as_stream(stream)))
+            return vv::launch_status();
+    }
+    // Everything else: the separate launches, through the caller's k and v buffers.
+    if (!k || !v) return VV_ERR_UNSUPPORTED;
+    vv_status_t s = vv_gemm_bias_rope_dev(x, wq, bq, q, M, n_q_heads, head_dim, K, rope_table, stream);
+    if (s != VV_OK) return s;
+    s = vv_gemm_bias_rope_dev(x, wk, bk, k, M, n_kv_heads, head_dim, K, rope_table, stream);
+    if (s != VV_OK) return s;
+    const int nkv = n_kv_heads * head_dim;
+    s = vv::gemm(x, wv, v, M, nkv, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
+    if (s != VV_OK) return s;
+    if (bv && (s = vv_bias_add_dev(v, bv, M, nkv, stream)) != VV_OK) return s;
+    if (k_cache)
+        return vv_kv_store_dev(k, v, k_cache, v_cache, nullptr, nullptr, nullptr, false, n_kv_heads, head_dim, pos,
+                               d_pos, M, 0, page_table, stream);
+    return VV_OK;
 }
 
 vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_up, void* gate, void* up,

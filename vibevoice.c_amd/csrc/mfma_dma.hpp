@@ -469,4 +469,178 @@ __device__ __forceinline__ void mfma_dma64(const void* __restrict__ A, const voi
     epi(acc, m_blk + wm * TM * 16, n_blk + wave_n0, lane);
 }
 
+// ── The q, k and v projections of a chunk of rows in ONE grid of equal tiles ─────────────────
+// A decoder with 7 query heads per KV head of 128 channels (28 + 4 heads: 3584 + 512 + 512 output columns)
+// has as many q and k heads, 32, as v has 16-column strips: a tile is 128 rows x (one head of q or k + one
+// strip of v) = 128 x 144 outputs, and 2048 rows are 16 x 32 = 512 equal tiles - one full round of two
+// workgroups per compute unit, where 128 x 128 tiles over the 4608 columns would be 576 (a round and an
+// eighth). The loop is mfma_dma64's for the 128 x 128 tile (four waves of 64 x 64, kPairN = 1: a head's columns
+// n and n + 64 in one lane) with a ninth copy per slab for the 16 v rows (waves 0 and 1 issue it), one more
+// fragment read and two more MFMAs per K step and wave: the strip's eight 16 x 16 products go two to a wave,
+// against the x fragments b = 0, 1 of the step - wave wn numbers its four row tiles from 2 wn (row tile
+// (b + 2 wn) % 4 is its b-th), so that the two waves that share rows take different halves of the strip
+// and the schedule needs no branch. Every output element adds K in mfma_dma64's order.
+//   epi(acc, accv, m0, wn, lane)   acc[a][b]: as mfma_dma64 with kPairN = 1, row m0 + 16 ((b + 2 wn) % 4) + l % 16;
+//                                  accv[j]: v column 4 (l / 16) + r of the strip, row m0 + 16 ((j + 2 wn) % 4) + l % 16
+constexpr int kQkvStrip = 16;                                  // v columns per tile
+template <int kStages>
+struct QkvShape {
+    static_assert(kStages == 2 || kStages == 4, "a slab's stage is slab % kStages");
+    static constexpr int kAhead = kStages;
+    static constexpr int kWaves = 4;
+    static constexpr int kStageSlots = (128 + 128 + kQkvStrip) * (kDma64SlabBytes / 16);   // x rows, head rows, v rows
+    static constexpr size_t kLdsBytes = (size_t)kStages * kStageSlots * 16;
+};
+
+// x: the tile's first row (rows_left of them exist); w_head: the head's 128 weight rows; w_strip: the strip's 16.
+template <typename Op, int kStages, typename Epi>
+__device__ __forceinline__ void mfma_dma64_qkv(const char* __restrict__ x, const char* __restrict__ w_head,
+                                               const char* __restrict__ w_strip, int rows_left, int row_bytes,
+                                               const Epi& epi) {
+    typedef typename Op::Acc16 Acc;
+    typedef QkvShape<kStages> Shape;
+    constexpr int kSlabChunks = kDma64SlabBytes / 16;     // 8
+    constexpr int WN = 2, TM = 4, TN = 4, kLoads = 8;
+    constexpr int kStageSlots = Shape::kStageSlots;
+    extern __shared__ u32x4 dma_lds[];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const bool strip_wave = wave < 2;                     // the waves that copy the strip's rows
+    const int nslabs = row_bytes / kDma64SlabBytes;
+    const uint32_t lds0 =
+        (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dma_lds);
+
+    // Copies 0 .. 3 of a wave are x rows, 4 .. 7 head rows (8 rows x 8 slots each, as in mfma_dma64); copy 8 of
+    // waves 0 and 1 is eight rows of the strip.
+    uint32_t src[kLoads + 1], dst[kLoads + 1];
+#pragma unroll
+    for (int i = 0; i <= kLoads; ++i) {
+        const int slot0 = (wave + Shape::kWaves * i) * kWave;
+        const int p = slot0 + lane;
+        const int row = p / kSlabChunks, phys = p % kSlabChunks;
+        const int logical = swz<64>(row, phys);
+        const int r = i < kLoads / 2 ? min(row, rows_left - 1) : i < kLoads ? row - 128 : row - 256;
+        src[i] = (uint32_t)r * (uint32_t)row_bytes + (uint32_t)logical * 16u;
+        dst[i] = lds0 + (uint32_t)slot0 * 16u;
+    }
+    auto request = [&](int slab, int i) {        // slab -> stage slab % kStages; past the end: the last slab again
+        const size_t adv = (size_t)min(slab, nslabs - 1) * kDma64SlabBytes;
+        const uint32_t stage = (uint32_t)(slab & (kStages - 1)) * (kStageSlots * 16u);
+        const char* tile = i < kLoads / 2 ? x : i < kLoads ? w_head : w_strip;
+        lds_dma16_at(tile + adv, src[i], dst[i] + stage);
+    };
+
+    Acc acc[TN][TM], accv[2];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b) acc[a][b][r] = 0;
+        accv[0][r] = accv[1][r] = 0;
+    }
+
+    const int frow = lane & 15, fquarter = lane >> 4;
+    int f_idx[2];
+#pragma unroll
+    for (int step = 0; step < 2; ++step)
+        f_idx[step] = frow * kSlabChunks + swz<64>(frow, step * 4 + fquarter);
+    int x_off[TM];                                        // the wave's b-th row tile is tile (b + 2 wn) % 4 of its 64 rows
+#pragma unroll
+    for (int b = 0; b < TM; ++b) x_off[b] = (wm * TM + ((b + 2 * wn) & 3)) * 16 * kSlabChunks;
+    const int fb_base = 128 * kSlabChunks + wn * 32 * kSlabChunks;
+    constexpr int kStripBase = 256 * kSlabChunks;
+    auto w_off = [](int a) { return ((a & 1) * 16 + (a >> 1) * 64) * kSlabChunks; };
+
+    // w and the strip fragment: the K step in hand and the next. x: tiles 0, 1 one set, refilled in place behind
+    // their last MFMA; tiles 2, 3 held twice.
+    u32x4 fw[2][TN], fv[2], fx[2], fxl[2][2];
+    auto read_w = [&](auto set_c, int slab, int step, int a) {
+        constexpr int set = decltype(set_c)::value;
+        fw[set][a] = dma_lds[(slab & (kStages - 1)) * kStageSlots + fb_base + w_off(a) + f_idx[step]];
+    };
+    auto read_v = [&](auto set_c, int slab, int step) {
+        constexpr int set = decltype(set_c)::value;
+        fv[set] = dma_lds[(slab & (kStages - 1)) * kStageSlots + kStripBase + f_idx[step]];
+    };
+    auto read_x = [&](auto set_c, int slab, int step, int b) {
+        constexpr int set = decltype(set_c)::value;
+        const u32x4 v = dma_lds[(slab & (kStages - 1)) * kStageSlots + x_off[b] + f_idx[step]];
+        if (b < 2) fx[b] = v;
+        else fxl[set][b - 2] = v;
+    };
+    // One K step: 18 MFMAs, x tile by x tile (tiles 0 and 1: four head products and the strip's). The reads of the
+    // next step and, in step 1 behind the barrier, the copy requests of the slab after next go one behind each MFMA.
+    auto k_step = [&](auto cur_c, auto nxt_c, int slab, auto step_c) {
+        constexpr int set = decltype(cur_c)::value;
+        constexpr int step = decltype(step_c)::value;
+        constexpr int nstep = step ^ 1;
+        const int nslab = slab + step;
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+#pragma unroll
+            for (int a = 0; a < (b < 2 ? TN + 1 : TN); ++a) {
+                if (step == 1 && b == 0 && a == 0) {
+                    // this wave's copies of the next slab are in: only those of the slabs behind it may still fly
+                    if constexpr (Shape::kAhead == 2) {
+                        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    } else {
+                        if (strip_wave) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
+                        else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+                    }
+                    __syncthreads();
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const u32x4 xf = b < 2 ? fx[b] : fxl[set][b - 2];
+                if (a < TN) acc[a][b] = Op::mfma16(fw[set][a], xf, acc[a][b]);
+                else accv[b] = Op::mfma16(fv[set], xf, accv[b]);
+                __builtin_amdgcn_sched_barrier(0);
+                const int slot = b < 2 ? b * (TN + 1) + a : 2 * (TN + 1) + (b - 2) * TN + a;
+                if constexpr (step == 1) {
+                    if (slot < kLoads) request(slab + Shape::kAhead, slot);
+                    else if (slot == kLoads && strip_wave) request(slab + Shape::kAhead, kLoads);
+                }
+                if (slot < 4) read_w(nxt_c, nslab, nstep, slot);
+                else if (slot == 4) read_x(nxt_c, nslab, nstep, 0);
+                else if (slot == 5) read_v(nxt_c, nslab, nstep);
+                else if (slot == 6) read_x(nxt_c, nslab, nstep, 2);
+                else if (slot == 7) read_x(nxt_c, nslab, nstep, 3);
+                else if (slot == 9) read_x(nxt_c, nslab, nstep, 1);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+#pragma unroll
+    for (int s = 0; s < Shape::kAhead; ++s) {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) request(s, i);
+        if (strip_wave) request(s, kLoads);
+    }
+    // slab 0; slab 1 is waited for at the first barrier
+    if constexpr (Shape::kAhead == 2) {
+        if (strip_wave) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else {
+        if (strip_wave) asm volatile("s_waitcnt vmcnt(27)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < TN; ++a) read_w(Const<0>{}, 0, 0, a);
+    read_v(Const<0>{}, 0, 0);
+#pragma unroll
+    for (int b = 0; b < TM; ++b) read_x(Const<0>{}, 0, 0, b);
+    for (int slab = 0; slab < nslabs; ++slab) {
+        k_step(Const<0>{}, Const<1>{}, slab, Const<0>{});
+        k_step(Const<1>{}, Const<0>{}, slab, Const<1>{});
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the surplus copies and reads land before the LDS is released
+
+    epi(acc, accv, wm * TM * 16, wn, lane);
+}
+
 }  // namespace vv

@@ -441,7 +441,7 @@ vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int positi
     if (!table) return VV_ERR_NULL_PTR;
     if (seq_len <= 0 || head_dim <= 0) return VV_OK;
     if ((head_dim & 1) || head_dim > 2 * vv::kMaxPairs) return VV_ERR_UNSUPPORTED;
-    if (reinterpret_cast<uintptr_t>(table) & 7u) return VV_ERR_INVALID_ARG;
+    if (reinterpret_cast<uintptr_t>(table) & 15u) return VV_ERR_UNSUPPORTED;    // its readers load 16 bytes at a time
     const int half = head_dim / 2;
     const size_t n = (size_t)seq_len * (size_t)half;
     vv::rope_table<<<dim3((unsigned)((n + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0, vv::as_stream(stream)>>>(

@@ -157,6 +157,7 @@ SIGNATURES = {
     "vv_bias_rope_qk_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "vv_rope_table_dev": (_i, [_vp, _i, _i, _i, _vp, _f, _vp]),
     "vv_gemm_bias_rope_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "vv_gemm_qkv_rope_dev": (_i, [_vp] * 10 + [_i] * 5 + [_vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "vv_embedding_rmsnorm_dev": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "vv_dev_alloc": (_i, [C.POINTER(_vp), _sz]),
     "vv_dev_alloc_pinned": (_i, [C.POINTER(_vp), _sz]),
