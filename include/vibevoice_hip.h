@@ -546,7 +546,9 @@ vv_status_t vv_attn_decode(int backend, const void* q, const vv_kv_view_t* kv,
  * Same arguments, results (bit for bit) and status codes as vv_attn_decode;
  * additionally VV_ERR_INVALID_ARG when the split path would need more than
  * VV_ATTN_DECODE_STATIC_MAX_Q_HEADS query heads of partial states, and
- * VV_ERR_CUDA when the array's address cannot be resolved. All calls on one
+ * VV_ERR_CUDA when the array's address cannot be resolved or the stream belongs
+ * to another device than the current one (each GPU has its own array, and the
+ * current device's is the one the call can name). All calls on one
  * GPU share that GPU's array: calls that overlap on one GPU (two streams, two
  * threads) race, so serialise them or use vv_attn_decode with a buffer per
  * context. The array's address is resolved at the first call on each device:

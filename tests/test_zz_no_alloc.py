@@ -55,10 +55,16 @@ def _check(c):
 def test_static_scratch_decode_matches_caller_scratch_twice():
     big = _case(28, 4, 128, 14449, 11)        # 256 slices
     small = _case(12, 2, 128, 3000, 23)       # 64 slices, fewer heads: a subset of the array
+    # a first call resolves the array's address (and loads the kernels); from then on the device's free memory -
+    # which a hipMalloc inside the library would move, unlike torch's own counters - must stay where it is
+    _run_pair(small)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]
     _run_pair(big)
     _run_pair(small)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.cuda.memory_allocated() == before
     _check(big)
     _check(small)

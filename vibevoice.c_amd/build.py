@@ -22,7 +22,11 @@ LIB = os.path.join(LIBDIR, "libvibevoice_hip.so")
 ARCH = "gfx950"
 
 # -packed-fp32-ops off: scalar FP32 arithmetic is never fused into v_pk_*_f32.
-DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# -amdgpu-kernarg-preload-count: the first 16 dwords of a kernel's arguments arrive in scalar registers with the
+# wave instead of being fetched by its first instructions - one memory round trip less before a kernel's first
+# load (a 512-row add+norm 4.20 -> 3.95 us, a one-row launch 2.4 -> 2.1 us; long kernels do not notice).
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
             "-Wno-unused-parameter", f"--offload-arch={ARCH}"] + DEVICE_FLAGS
 

@@ -917,6 +917,11 @@ constexpr int kStreamOStride = kD + 1;          // floats per head in the waves'
 // A wave's LDS: V^T of a block (4 KB), later its O for kHeads heads.
 constexpr int stream_tile_bytes(int heads) { return heads * kStreamOStride * 4 < 4096 ? 4096 : (heads * kStreamOStride * 4 + 15) / 16 * 16; }
 
+// Where channel ch of a head sits in the waves' exchange: the upper two of the four 32-channel blocks turned by 16, so
+// that the four lanes that hold one (e, r) of the same head in their four blocks write four different banks
+// (with a plain layout blocks j and j + 2 are 64 floats apart: every store a two-way conflict).
+__device__ __forceinline__ int stream_o_slot(int ch) { return (ch & ~31) | ((ch + ((ch >> 2) & 16)) & 31); }
+
 template <int kHeads>      // the group's query heads, padded: 8 or 16
 __global__ __launch_bounds__(kStreamThreads) void decode_stream(
     const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V,
@@ -1039,7 +1044,7 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
 #pragma unroll
         for (int e = 0; e < 8; ++e)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o_of(wave)[c * kStreamOStride + 32 * j + 8 * r + e] = o[e][r];
+            for (int r = 0; r < 4; ++r) o_of(wave)[c * kStreamOStride + stream_o_slot(32 * j + 8 * r + e)] = o[e][r];
     }
     __syncthreads();
     for (int idx = tid; idx < group * kD; idx += kStreamThreads) {
@@ -1052,7 +1057,7 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
         for (int w = 0; w < kStreamWaves; ++w) {
             const float mw = m_lds[w][h];
             const float f = mw == -INFINITY ? 0.0f : exp2_fast(mw - m_all);
-            ov = fmaf(o_of(w)[h * kStreamOStride + ch], f, ov);
+            ov = fmaf(o_of(w)[h * kStreamOStride + stream_o_slot(ch)], f, ov);
             l_all = fmaf(l_lds[w][h], f, l_all);
         }
         float* dst = parts + ((size_t)(kvh * group + h) * n_parts + part) * kPartFloats;
@@ -1669,9 +1674,12 @@ static __device__ __align__(256) float scratch[kStaticFloats];
 constexpr int kMaxDevices = 64;
 std::atomic<float*> g_scratch_ptr[kMaxDevices];
 
-float* static_scratch() {
-    int dev = -1;
+// The array of the device the stream belongs to (the current device for the default stream), which must be the
+// current device: a symbol's address can only be asked of the current device.
+float* static_scratch(hipStream_t st) {
+    int dev = -1, stream_dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    if (st && hipStreamGetDevice(st, &stream_dev) == hipSuccess && stream_dev != dev) return nullptr;
     float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!p) {
         void* sym = nullptr;
@@ -1717,7 +1725,7 @@ vv_status_t vv_attn_decode_static(int backend, const void* q, const vv_kv_view_t
     if (vv::decode_on_matrix_cores(q, kv) && vv::decode_parts(cache_len) > 1) {
         // the partial states are [n_q_heads][slices][head_dim + 4] floats, head_dim 128 on this path
         if (n_q_heads > vv::kStaticMaxQHeads) return VV_ERR_INVALID_ARG;
-        parts = vv::static_scratch();
+        parts = vv::static_scratch(vv::as_stream(stream));
         if (!parts) return VV_ERR_CUDA;
     }
     return vv::attn_decode_launch(q, kv, out, n_q_heads, cache_len, d_cache_len, parts,
