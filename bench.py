@@ -769,6 +769,8 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
     view = dev.KvView(k=kc.data_ptr(), v=vc.data_ptr(), k_meta=None, v_meta=None, page_table=None, format=0,
                       n_kv_heads=NK, head_dim=HD)
     P = lambda t: t.data_ptr()
+    # the context's attention scratch, which the reference's decoder hands to every attention call (decoder.c:755, 893)
+    attn_scratch = torch.empty(dev.vv_attn_scratch_bytes(NQ, NK, HD), dtype=torch.uint8, device="cuda")
     rope_table = torch.empty(T, HD // 2, 2, dtype=torch.float32, device="cuda")
     assert dev.vv_rope_table_dev(P(rope_table), T, HD, 0, None, THETA, st) == 0
     assert dev.vv_rmsnorm_dev(P(hidden0), P(n1), P(normed_in), T, H, EPS, st) == 0
@@ -799,7 +801,8 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
     def one_chunk(start, n, fused):
         h = P(hidden) + start * H * 2
         qkv(start, n, fused)
-        assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, n, start, start + n, True, None, st) == 0
+        assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, n, start, start + n, True, P(attn_scratch),
+                                   st) == 0
         gemm(P(attn), wo, proj, n, H, QD)
         if fused:
             assert dev.vv_add_rmsnorm_dev(h, P(proj), P(n2), P(normed), n, H, EPS, st) == 0

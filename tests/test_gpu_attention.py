@@ -204,6 +204,55 @@ def test_decode_against_oracle(nq, nkv, hd, cache_len):
     check(one, ref, vmax, "prefill of one row")
 
 
+def prefill_with_scratch(d_q, view, nq, hd, rows, off, kv_len, scratch):
+    d_o = torch.full((rows, nq, hd), float("nan"), dtype=torch.float16, device="cuda")
+    ok(dev.vv_attn_prefill(FA2, d_q.data_ptr(), C.addressof(view), d_o.data_ptr(), nq, rows, off, kv_len, True,
+                           scratch.data_ptr(), stream()))
+    return bits_of(d_o)
+
+
+# few rows against a long cache: with the caller's scratch the keys are cut into runs (a short chunk on top of a
+# filled cache, src/inference/decoder.c:1095-1115). Rows, heads, offset: one row tile at the end of a long cache,
+# a ragged one, several tiles whose causal limits differ (the last runs are empty for the first tiles), one row.
+SPLIT = [(113, 28, 4, 14336), (37, 4, 2, 5000), (300, 4, 1, 3000), (1, 2, 1, 4000), (128, 8, 2, 1000), (600, 4, 2, 700)]
+
+
+@pytest.mark.parametrize("rows,nq,nkv,off", SPLIT)
+def test_prefill_split_over_the_keys(rows, nq, nkv, off):
+    hd, kv_len = 128, off + rows
+    q, k, v = make(rows, nq, nkv, hd, kv_len, 3 * rows + off)
+    ref = oracle.attention_prefill_f32(oracle.widen(q), oracle.widen(k), oracle.widen(v), off, kv_len, True)
+    d_q = to_dev(q)
+    pad = np.full((8, nkv, hd), 0x7E00, np.uint16)             # NaN past the cache's end
+    vw = view_of(to_dev(np.concatenate([k, pad])), to_dev(np.concatenate([v, pad])), nkv, hd)
+    vmax = float(np.abs(oracle.widen(v)).max())
+    scratch = torch.full((dev.vv_attn_scratch_bytes(nq, nkv, hd) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    got = prefill_with_scratch(d_q, vw, nq, hd, rows, off, kv_len, scratch)
+    check(got, ref, vmax, "split prefill")
+    assert not np.isnan(scratch[:8].cpu().numpy()).any(), "this shape was meant to take the split path"
+    # the one-launch form of the same call agrees to the rounding of the runs' partial sums
+    whole = prefill(d_q, vw, nq, hd, rows, off, kv_len)
+    d = np.abs(oracle.widen(got).astype(np.float64) - oracle.widen(whole).astype(np.float64))
+    assert d.max() <= 2.0 ** -9 * vmax
+    # the same bits again, and from a paged cache
+    assert np.array_equal(prefill_with_scratch(d_q, vw, nq, hd, rows, off, kv_len, scratch), got)
+    pool_k, pool_v, table, _ = paged_cache(k, v, nkv, hd, 9)
+    assert np.array_equal(prefill_with_scratch(d_q, view_of(pool_k, pool_v, nkv, hd, table), nq, hd, rows, off, kv_len,
+                                               scratch), got)
+
+
+def test_prefill_scratch_is_left_alone_when_there_is_nothing_to_split():
+    """Enough rows to fill the chip, or too few keys for two runs: one launch, the scratch untouched."""
+    for rows, nq, nkv, off in ((2048, 28, 4, 0), (64, 4, 2, 100)):
+        hd, kv_len = 128, off + rows
+        q, k, v = make(rows, nq, nkv, hd, kv_len, 5)
+        d_q, vw = to_dev(q), view_of(to_dev(k), to_dev(v), nkv, hd)
+        scratch = torch.full((dev.vv_attn_scratch_bytes(nq, nkv, hd) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+        got = prefill_with_scratch(d_q, vw, nq, hd, rows, off, kv_len, scratch)
+        assert np.array_equal(got, prefill(d_q, vw, nq, hd, rows, off, kv_len))
+        assert bool(torch.isnan(scratch).all())
+
+
 def test_declines_and_edges():
     hd, nkv, nq = 128, 1, 2
     d = torch.zeros((4, nq, hd), dtype=torch.float16, device="cuda")

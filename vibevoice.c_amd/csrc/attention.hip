@@ -25,6 +25,7 @@
 //                leave (max, sum, unnormalised O) in the caller's scratch
 //                and decode_merge folds them.
 //   rows_generic any head_dim <= 256, any alignment: one wave per (row, head).
+#include <algorithm>
 #include <atomic>
 
 #include "vv_common.hpp"
@@ -81,6 +82,8 @@ __device__ __forceinline__ int cache_row(const int* page_table, int t) {
 
 // ── head_dim 128 on the matrix cores: the pieces both forms share ─────────
 constexpr int kD = 128;
+constexpr int kPartFloats = kD + 4;        // a partial state: 128 channels, max, sum, 2 unused (16-byte rows)
+constexpr int kPrefillSplitRows = 2048;    // (rows x key runs) of a split prefill the caller's scratch holds per query head
 constexpr int kQTile = 128;          // query rows per prefill workgroup (32 per wave)
 constexpr int kKeyTile = 64;         // keys per LDS tile
 constexpr int kVtStride = kKeyTile + 4;   // halves per transposed-V row: 136 B
@@ -478,9 +481,15 @@ __device__ __forceinline__ s16x4 lds_read_transposed(const char* p) {
 __device__ __forceinline__ void copy16_to_lds(const void* gptr, uint32_t lds_byte_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_byte_addr), "v"(gptr) : "memory", "m0");
 }
+// kSplit: the keys are cut into `n_runs` runs of `tiles_per_part` tiles (an even number); a workgroup takes one run
+// of what it would have taken alone and leaves each row's state - 128 unnormalised channels, the
+// scaled maximum, the sum - in `parts` as record (row, head, run) for prefill_merge. For a few rows against a long
+// cache: one row tile is 28 workgroups that each walk the whole cache, tile after tile, on a chip of 256 units.
+template <bool kSplit>
 __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V, const int* __restrict__ page_table,
-    h16* __restrict__ O, int n_q_heads, int n_kv_heads, int q_len, int q_offset, int kv_len, int causal, float scale_log2) {
+    h16* __restrict__ O, int n_q_heads, int n_kv_heads, int q_len, int q_offset, int kv_len, int causal, float scale_log2,
+    float* __restrict__ parts, int n_runs, int tiles_per_part) {
     __shared__ PipeTiles tiles;
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -491,7 +500,13 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     const int group_heads = n_q_heads / n_kv_heads;
     const int n_row_tiles = (q_len + kQTile - 1) / kQTile;
     const int xcd = (int)blockIdx.x & 7, nth = (int)blockIdx.x >> 3;
-    const int group = (nth / group_heads) * 8 + xcd;              // (row tile, KV head), heaviest first
+    int group = (nth / group_heads) * 8 + xcd;                    // (row tile, KV head), heaviest first
+    int run = 0;                                                  // kSplit: (run, row tile, KV head) dealt the same way
+    if (kSplit) {
+        run = group / (n_row_tiles * n_kv_heads);
+        group -= run * (n_row_tiles * n_kv_heads);
+        if (run >= n_runs) return;
+    }
     if (group >= n_row_tiles * n_kv_heads) return;                // the whole workgroup, before any barrier
     const int kvh = group % n_kv_heads;
     const int head = kvh * group_heads + nth % group_heads;
@@ -501,10 +516,22 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     const int q_abs = q_offset + qrow;
     int wg_limit = kv_len;
     if (causal) wg_limit = min(kv_len, q_offset + min(q0 + kQTile, q_len));
-    const int ntiles = (wg_limit + kKeyTile - 1) / kKeyTile;
+    int ntiles = (wg_limit + kKeyTile - 1) / kKeyTile;
     const int last_key = kv_len - 1;
     const size_t row_halves = (size_t)n_kv_heads * kD;
     const uint32_t lds_k0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)&tiles.k[0][0]);
+    int tile0 = 0;                                                // first key tile of this workgroup's run
+    if (kSplit) {
+        tile0 = run * tiles_per_part;
+        ntiles = min(tiles_per_part, ntiles - tile0);
+        if (ntiles <= 0) {                                        // nothing the rows may see in this run: empty states
+            if (qrow < q_len) {
+                float* rec = parts + (((size_t)qrow * n_q_heads + head) * n_runs + run) * kPartFloats;
+                for (int i = half; i < kPartFloats; i += 2) rec[i] = i == kD ? -INFINITY : 0.0f;
+            }
+            return;                                               // the whole workgroup, before any barrier
+        }
+    }
 
     h16x8 qf[kD / 16];
     load_query(qf, Q + ((size_t)min(qrow, q_len - 1) * n_q_heads + head) * kD, half);
@@ -522,7 +549,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         k_off[c] = (uint32_t)(((size_t)key * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)((phys ^ (key & 15)) * 16);
     }
     auto request_k = [&](int j) {
-        const int t0 = j * kKeyTile;
+        const int t0 = (tile0 + j) * kKeyTile;
         const uint32_t lds_at = lds_k0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave) * 1024u;
         if (!page_table && t0 + kKeyTile <= kv_len) {
             const char* base = reinterpret_cast<const char*>(K) + (size_t)t0 * row_halves * 2u;
@@ -551,7 +578,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         v_off[c] = (uint32_t)(((size_t)key * row_halves + (size_t)kvh * kD) * 2u) + (uint32_t)(((phys - 4 * (key & 3)) & 15) * 16);
     }
     auto request_v = [&](int j) {
-        const int t0 = j * kKeyTile;
+        const int t0 = (tile0 + j) * kKeyTile;
         const uint32_t lds_at = lds_v0 + (uint32_t)(j & 1) * (kKeyTile * 256u) + (uint32_t)(4 * wave) * 1024u;
         if (!page_table && t0 + kKeyTile <= kv_len) {
             const char* base = reinterpret_cast<const char*>(V) + (size_t)t0 * row_halves * 2u;
@@ -620,7 +647,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     // Tile j's scores lose what the row may not see: only a tile that reaches past the cache end or past the
     // wave's first row's position has anything to hide.
     auto hide = [&](int j, f32x16 (&sc)[2]) {
-        const int t0 = j * kKeyTile;
+        const int t0 = (tile0 + j) * kKeyTile;
         if (t0 + kKeyTile > kv_len || (causal && t0 + kKeyTile - 1 > q_offset + qw0)) {
 #pragma unroll
             for (int a = 0; a < 2; ++a)
@@ -740,6 +767,20 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no copy may land after the workgroup has gone
+    if (kSplit) {
+        if (qrow < q_len) {
+            float* rec = parts + (((size_t)qrow * n_q_heads + head) * n_runs + run) * kPartFloats;
+            // register 4 g + r of tile t is channel 32 t + 8 g + 4 half + r
+#pragma unroll
+            for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    *reinterpret_cast<float4*>(rec + 32 * t + 8 * g + 4 * half) =
+                        float4{st.o[t][4 * g], st.o[t][4 * g + 1], st.o[t][4 * g + 2], st.o[t][4 * g + 3]};
+            if (half == 0) *reinterpret_cast<float2*>(rec + kD) = float2{st.m, st.l};
+        }
+        return;
+    }
     if (qrow < q_len) {
         const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
         h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
@@ -757,6 +798,42 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     }
 }
 
+
+// The runs of a split prefill folded: one wave per (row, head), two channels per lane, the runs in order. A run's
+// record is 128 unnormalised channels, its scaled maximum and its sum; a run that saw no key has maximum -inf.
+__global__ __launch_bounds__(kBlock) void prefill_merge(const float* __restrict__ parts, h16* __restrict__ O,
+                                                        int rows_heads, int n_parts) {
+    constexpr int kMostRuns = 16;                          // what vv_attn_prefill cuts a prefill into at most
+    const int item = (int)blockIdx.x * kWavesPerBlock + wave_in_block();
+    if (item >= rows_heads) return;
+    const int lane = lane_id();
+    const float* rec = parts + (size_t)item * n_parts * kPartFloats;
+    // every run's values are asked for before the first is used: one trip to memory
+    float m[kMostRuns], l[kMostRuns];
+    float2 v[kMostRuns];
+#pragma unroll
+    for (int p = 0; p < kMostRuns; ++p) {
+        const float* r = rec + (size_t)min(p, n_parts - 1) * kPartFloats;
+        m[p] = p < n_parts ? r[kD] : -INFINITY;
+        l[p] = r[kD + 1];
+        v[p] = *reinterpret_cast<const float2*>(r + 2 * lane);
+    }
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < kMostRuns; ++p) m_all = fmaxf(m_all, m[p]);
+    float o0 = 0.0f, o1 = 0.0f, l_all = 0.0f;
+#pragma unroll
+    for (int p = 0; p < kMostRuns; ++p) {
+        const float f = m[p] == -INFINITY ? 0.0f : exp2_fast(m[p] - m_all);
+        o0 = fmaf(v[p].x, f, o0);
+        o1 = fmaf(v[p].y, f, o1);
+        l_all = fmaf(l[p], f, l_all);
+    }
+    const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+    typedef h16 h16x2v __attribute__((ext_vector_type(2)));
+    const h16x2v out = {to_half(o0 * inv), to_half(o1 * inv)};
+    *reinterpret_cast<h16x2v*>(O + (size_t)item * kD + 2 * lane) = out;
+}
 
 // ── any head_dim <= 256: one wave per (query row, head) ──────────────────
 __global__ __launch_bounds__(kWave) void rows_generic(
@@ -810,7 +887,6 @@ __global__ __launch_bounds__(kWave) void rows_generic(
 // the heads sharing a KV head take the place of the prefill's query rows, so
 // the slice's K and V are read once for all of them. n_parts == 1 writes O;
 // otherwise each slice leaves (max, sum, unnormalised O) per head in `parts`.
-constexpr int kPartFloats = kD + 4;        // per (head, slice): 128 channels, max, sum, 2 unused (16-byte rows)
 
 template <int kFmt>
 __global__ __launch_bounds__(kWave) void decode128(
@@ -1532,7 +1608,9 @@ int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads, int
 size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim) {
     (void)n_kv_heads;
     if (n_q_heads <= 0 || head_dim <= 0) return 0;
-    return (size_t)n_q_heads * vv::kMaxParts * ((size_t)head_dim + 4) * sizeof(float);
+    // per query head: the decode's slices, or the (rows x key runs) of a short prefill split over the keys
+    constexpr size_t kRecords = vv::kMaxParts > vv::kPrefillSplitRows ? vv::kMaxParts : vv::kPrefillSplitRows;
+    return (size_t)n_q_heads * kRecords * ((size_t)head_dim + 4) * sizeof(float);
 }
 
 int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_len) {
@@ -1543,7 +1621,7 @@ int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_l
 vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, void* out,
                             int n_q_heads, int q_len, int q_offset, int kv_len, bool causal,
                             void* scratch, void* stream) {
-    (void)backend; (void)scratch;
+    (void)backend;
     if (!q || !kv || !out) return VV_ERR_NULL_PTR;
     if (q_len <= 0 || kv_len <= 0) return VV_OK;
     if (!kv->k || !kv->v) return VV_ERR_NULL_PTR;
@@ -1578,10 +1656,34 @@ vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv, 
 #undef VV_PREFILL
     } else if (kv->head_dim == vv::kD && vv::aligned16(q) && vv::aligned16(kv->k) && vv::aligned16(kv->v) &&
                vv::aligned16(out)) {
-        const int groups = kv->n_kv_heads * ((q_len + vv::kQTile - 1) / vv::kQTile);     // see the kernel's numbering
-        const dim3 grid((unsigned)(8 * ((groups + 7) / 8) * (n_q_heads / kv->n_kv_heads)));
-        vv::prefill_pipe<<<grid, vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads, kv->n_kv_heads, q_len,
-                                                      q_offset, kv_len, causal ? 1 : 0, scale_log2);
+        const int row_tiles = (q_len + vv::kQTile - 1) / vv::kQTile;
+        const int groups = kv->n_kv_heads * row_tiles;                                   // see the kernel's numbering
+        const unsigned gx = (unsigned)(8 * ((groups + 7) / 8) * (n_q_heads / kv->n_kv_heads));
+        // Few rows against many keys: the keys are cut into runs, as many as give every compute unit two
+        // workgroups, as the caller's scratch holds, and as leave a run eight tiles or more.
+        const int key_tiles = ((causal ? std::min(kv_len, q_offset + q_len) : kv_len) + vv::kKeyTile - 1) / vv::kKeyTile;
+        int runs = 1;
+        if (scratch && vv::aligned16(scratch) && q_len <= vv::kPrefillSplitRows)
+            runs = std::min(std::min(512 / (row_tiles * n_q_heads), 16),
+                            std::min(vv::kPrefillSplitRows / q_len, key_tiles / 8));
+        if (runs >= 2) {
+            int per = (key_tiles + runs - 1) / runs;
+            per += per & 1;                                        // whole pairs of tiles: the loop is unrolled by two
+            runs = (key_tiles + per - 1) / per;
+            float* parts = static_cast<float*>(scratch);
+            const unsigned gsplit = (unsigned)(8 * ((groups * runs + 7) / 8) * (n_q_heads / kv->n_kv_heads));
+            vv::prefill_pipe<true><<<dim3(gsplit), vv::kBlock, 0, st>>>(
+                Q, K, V, kv->page_table, O, n_q_heads, kv->n_kv_heads, q_len, q_offset, kv_len, causal ? 1 : 0,
+                scale_log2, parts, runs, per);
+            if (hipGetLastError() != hipSuccess) return VV_ERR_CUDA_LAUNCH;
+            const int items = q_len * n_q_heads;
+            vv::prefill_merge<<<dim3((unsigned)((items + vv::kWavesPerBlock - 1) / vv::kWavesPerBlock)), vv::kBlock, 0,
+                                st>>>(parts, O, items, runs);
+        } else {
+            vv::prefill_pipe<false><<<dim3(gx), vv::kBlock, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
+                                                                     kv->n_kv_heads, q_len, q_offset, kv_len,
+                                                                     causal ? 1 : 0, scale_log2, nullptr, 1, 0);
+        }
     } else {
         const dim3 grid((unsigned)q_len, (unsigned)n_q_heads);
         vv::rows_generic<<<grid, vv::kWave, 0, st>>>(Q, K, V, kv->page_table, O, n_q_heads,
@@ -1734,8 +1836,9 @@ vv_status_t vv_attn_decode_static(int backend, const void* q, const vv_kv_view_t
 
 /* The older entry points for raw FP16 caches (device.h:621-655): the same
  * kernels, the cache given as two pointers instead of a view. */
-size_t vv_gqa_decode_scratch_bytes(int n_q_heads, int head_dim) {
-    return vv_attn_scratch_bytes(n_q_heads, 1, head_dim);
+size_t vv_gqa_decode_scratch_bytes(int n_q_heads, int head_dim) {      // the decode's slices alone
+    if (n_q_heads <= 0 || head_dim <= 0) return 0;
+    return (size_t)n_q_heads * vv::kMaxParts * ((size_t)head_dim + 4) * sizeof(float);
 }
 
 int vv_gqa_decode_shape(int cache_len) { return vv::decode_parts(cache_len); }
