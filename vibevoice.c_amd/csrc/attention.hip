@@ -978,20 +978,17 @@ __global__ __launch_bounds__(kWave) void decode128(
 //   softmax  online per head in FP32, base-2 domain; maximum and sum cross the four
 //            j groups by lane exchange. The probabilities, rounded to FP16, are
 //            already the B operand of the second product (16x16x16, k = key).
-//   O^T      = V^T P^T: lane (chunk c = l % 16, j) loads keys 4 j .. 4 j + 3 of chunk
-//            c as stored and writes, per channel, the four keys as 8 bytes into the
-//            wave's own LDS tile [e][c][16 keys] (channel 8 c + e); the 16 channels
-//            {8 c + e} of one e form an A tile, so writes and reads alike touch each
-//            bank once per 32 lanes. Lane (head l % 16, j') accumulates channels
-//            32 j' + 8 r + e in FP32.
-// Only V passes through LDS, and only inside its own wave (no workgroup barrier in
-// the loop). The waves' states meet in LDS and the workgroup leaves one (max, sum,
-// unnormalised O) record per head in `parts`, for decode_merge.
+//   O^T      = V^T P^T: lane (chunk c = l % 16, j) loads keys 4 j .. 4 j + 3 of chunk c as stored; element e of
+//            those four rows are the four keys of channel 8 c + e, which is exactly this lane's share of the A
+//            operand of the tile "channels {8 c + e}" (row c, keys 4 j .. + 3): the transposition costs a pick
+//            of halves, no LDS. Lane (head l % 16, j') accumulates channels 32 j' + 8 r + e in FP32.
+// Nothing passes through LDS in the loop. The waves' states meet in LDS once and the workgroup leaves one (max,
+// sum, unnormalised O) record per head in `parts`, for decode_merge.
 constexpr int kStreamWaves = 16;
 constexpr int kStreamThreads = kStreamWaves * kWave;
 constexpr int kStreamOStride = kD + 1;          // floats per head in the waves' exchange (odd: spreads banks)
-// A wave's LDS: V^T of a block (4 KB), later its O for kHeads heads.
-constexpr int stream_tile_bytes(int heads) { return heads * kStreamOStride * 4 < 4096 ? 4096 : (heads * kStreamOStride * 4 + 15) / 16 * 16; }
+// A wave's LDS: its O for kHeads heads.
+constexpr int stream_tile_bytes(int heads) { return (heads * kStreamOStride * 4 + 15) / 16 * 16; }
 
 // Where channel ch of a head sits in the waves' exchange: the upper two of the four 32-channel blocks turned by 16, so
 // that the four lanes that hold one (e, r) of the same head in their four blocks write four different banks
@@ -1003,8 +1000,7 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
     const h16* __restrict__ Q, const h16* __restrict__ K, const h16* __restrict__ V,
     const int* __restrict__ page_table, float* __restrict__ parts, int n_q_heads, int n_kv_heads,
     int cache_len, const int* __restrict__ d_cache_len, int n_parts, float scale_log2) {
-    // Per wave: V^T of the block in hand, [e][c][16 keys] halves; after its loop the wave's O instead,
-    // [head][kStreamOStride] floats (a wave touches no other wave's tile before the barrier).
+    // Per wave: its O after the loop, [head][kStreamOStride] floats.
     __shared__ __attribute__((aligned(16))) char tile_lds[kStreamWaves][stream_tile_bytes(kHeads)];
     __shared__ float m_lds[kStreamWaves][16], l_lds[kStreamWaves][16];
     auto o_of = [&](int w) { return reinterpret_cast<float*>(tile_lds[w]); };
@@ -1012,7 +1008,6 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = wave_in_block();
     const int c = lane & 15, j = lane >> 4;        // c: key (scores) / head (softmax, O) / chunk (V loads)
-    h16 (*vt)[16][16] = reinterpret_cast<h16 (*)[16][16]>(tile_lds[wave]);
     const int part = (int)blockIdx.x, kvh = (int)blockIdx.y;
     const int group = n_q_heads / n_kv_heads;
     const int len = d_cache_len ? *d_cache_len : cache_len;
@@ -1083,12 +1078,6 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
         }
         m = m_new;
 
-        // V^T of the block into the wave's tile: four keys of one channel per 8-byte slot
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const h16x4 w = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
-            *reinterpret_cast<h16x4*>(&vt[e][c][4 * j]) = w;
-        }
         h16x4 pf;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -1096,18 +1085,14 @@ __global__ __launch_bounds__(kStreamThreads) void decode_stream(
             l += p;
             pf[r] = (h16)p;
         }
-        // the wave's own LDS traffic only: in order per wave, no workgroup barrier needed
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // V^T P^T: lane (chunk c, j) holds keys 4 j .. 4 j + 3 of channels 8 c .. 8 c + 7 as they were stored; the four
+        // keys of ONE channel 8 c + e are this lane's part of the A operand of tile e (row c = channel 8 c + e, keys
+        // 4 j .. + 3), so the transposition is a pick of element e from the four rows: no trip through LDS.
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const h16x4 vf = *reinterpret_cast<const h16x4*>(&vt[e][c][4 * j]);
+            const h16x4 vf = {v4[0][e], v4[1][e], v4[2][e], v4[3][e]};
             o[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf, o[e], 0, 0, 0);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();                   // the next block overwrites the tile
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 
     // the wave's denominators meet across the four j groups; then the waves
