@@ -513,7 +513,9 @@ typedef struct vv_kv_view {
  * replaces device.h:545-546 (src/cuda/attention_fi.cu:554-583). */
 int vv_attn_resolve(int requested, int kv_format, bool paged, int n_q_heads,
                     int n_kv_heads, int head_dim);
-/* n_q_heads * 256 * (head_dim + 4) floats: the decode slices' partial states.
+/* n_q_heads * 2048 * (head_dim + 4) floats: room for the decode slices' partial
+ * states (256 per head) and for the partial states of a short prefill split
+ * over the keys (rows x key runs <= 2048 per head); one buffer per context.
  * replaces device.h:554 (attention_fi.cu:585-589). */
 size_t vv_attn_scratch_bytes(int n_q_heads, int n_kv_heads, int head_dim);
 /* The number of slices the decode splits `cache_len` positions into: 16 up to
@@ -525,6 +527,11 @@ int vv_attn_decode_shape(int backend, int n_q_heads, int n_kv_heads, int cache_l
  * positions of the cache; Q, O [q_len][n_q_heads][head_dim] FP16; causal:
  * query p sees positions <= p. head_dim 128 with 16-byte aligned pointers
  * runs on the matrix cores, any other head_dim <= 256 a wave per row.
+ * scratch (vv_attn_scratch_bytes() of device memory, 16-byte aligned, or NULL):
+ * with it, few rows against many keys on an FP16 cache (fewer workgroups than
+ * fill the chip, at least sixteen 64-key tiles) are split over the keys into
+ * up to 16 runs whose partial states a second launch folds - the same values
+ * to the rounding of the runs' partial sums; without it every call is one launch.
  * A format other than FP16, head_dim > 256 or n_q_heads % n_kv_heads != 0:
  * VV_ERR_UNSUPPORTED. replaces device.h:575-578 (attention_fi.cu:600-632). */
 vv_status_t vv_attn_prefill(int backend, const void* q, const vv_kv_view_t* kv,
@@ -558,7 +565,8 @@ vv_status_t vv_attn_decode_static(int backend, const void* q, const vv_kv_view_t
                                   void* out, int n_q_heads, int cache_len,
                                   const int* d_cache_len, void* stream);
 /* The older entry points for raw FP16 caches: the cache as two pointers
- * instead of a view, otherwise vv_attn_scratch_bytes, vv_attn_decode_shape,
+ * instead of a view, otherwise vv_attn_scratch_bytes (the decode's 256 slices per
+ * head alone: these prefill forms take no scratch), vv_attn_decode_shape,
  * vv_attn_decode and vv_attn_prefill. replace device.h:621-655. */
 size_t vv_gqa_decode_scratch_bytes(int n_q_heads, int head_dim);
 int vv_gqa_decode_shape(int cache_len);
