@@ -43,6 +43,17 @@ constexpr int kMaxParts = 256;       // decode slices per KV head
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+// The reference exponent of a row's online softmax. It need not be the running maximum: any value within a
+// fixed distance below it keeps every probability bounded (here by 2^kMaxSlack = 256, far inside FP16 and
+// harmless to the FP32 sums), and the quotient O / l does not depend on it. So the reference moves - and O and
+// l are rescaled, 65 multiplies per lane - only when a tile's maximum passes it by more than kMaxSlack, which
+// after a row's first tile almost never happens, instead of whenever the maximum creeps up (on random scores:
+// in nearly half of all tiles, since some one of a wave's 32 rows finds a new maximum). A row's rule depends on
+// that row's scores alone. Units: base-2 exponents.
+constexpr float kMaxSlack = 8.0f;
+__device__ __forceinline__ float next_reference(float m, float tile_max) {
+    return tile_max > m + kMaxSlack ? tile_max : m;           // m = -inf: any finite maximum replaces it
+}
 // A value and its partner's, 32 (or 16) lanes away, combined in the vector ALU: the gfx950 lane swaps exchange
 // the odd rows of one register with the even rows of another (rows of 32 or 16 lanes), so from two copies of v
 // one register ends up with the lower row's values in both rows of a pair and the other with the upper row's.
@@ -98,7 +109,7 @@ struct KvTile {
 // register 4g + r of tile t is channel 32t + 8g + 4*(lane / 32) + r.
 struct RowState {
     f32x16 o[kD / 32];
-    float m, l;                                   // running max (base-2 domain) and sum
+    float m, l;                                   // reference exponent (next_reference; base-2 domain) and sum
     __device__ __forceinline__ void reset() {
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
@@ -310,8 +321,8 @@ __device__ __forceinline__ void tile_scores(const KvTile& tile, const h16x8 (&qf
 // Online-softmax update of the row state, then O^T += V^T P^T over the tile's
 // four 16-key steps. Slot e of this lane in step (a, sp) is register 8*sp + e
 // of s[a], i.e. key 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte
-// reads of V^T below. O is rescaled only when some row's maximum moved (after
-// the first few tiles it rarely does): the factor is exactly 1 otherwise.
+// reads of V^T below. O is rescaled only when some row's reference exponent
+// moved (next_reference): the factor is exactly 1 otherwise.
 __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], RowState& st,
                                             int col, int half, float scale_log2) {
     float mx = -INFINITY;
@@ -320,7 +331,7 @@ __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], 
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
     mx = max_xor32(mx) * scale_log2;
-    const float m_new = fmaxf(st.m, mx);
+    const float m_new = next_reference(st.m, mx);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
     float sum = 0.0f;
 #pragma unroll
@@ -685,7 +696,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         kf[0] = k_frag(0);
         kf[1] = k_frag(1);
         float sum = 0.0f;
-        const float m_new = fmaxf(st.m, mx_cur);
+        const float m_new = next_reference(st.m, mx_cur);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         h16x8 pf[4];
 #pragma unroll
