@@ -43,17 +43,8 @@ constexpr int kMaxParts = 256;       // decode slices per KV head
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
-// The reference exponent of a row's online softmax. It need not be the running maximum: any value within a
-// fixed distance below it keeps every probability bounded (here by 2^kMaxSlack = 256, far inside FP16 and
-// harmless to the FP32 sums), and the quotient O / l does not depend on it. So the reference moves - and O and
-// l are rescaled, 65 multiplies per lane - only when a tile's maximum passes it by more than kMaxSlack, which
-// after a row's first tile almost never happens, instead of whenever the maximum creeps up (on random scores:
-// in nearly half of all tiles, since some one of a wave's 32 rows finds a new maximum). A row's rule depends on
-// that row's scores alone. Units: base-2 exponents.
+// The slack of a row's reference exponent below its running maximum, in base-2 exponents (RowState).
 constexpr float kMaxSlack = 8.0f;
-__device__ __forceinline__ float next_reference(float m, float tile_max) {
-    return tile_max > m + kMaxSlack ? tile_max : m;           // m = -inf: any finite maximum replaces it
-}
 // A value and its partner's, 32 (or 16) lanes away, combined in the vector ALU: the gfx950 lane swaps exchange
 // the odd rows of one register with the even rows of another (rows of 32 or 16 lanes), so from two copies of v
 // one register ends up with the lower row's values in both rows of a pair and the other with the upper row's.
@@ -105,19 +96,46 @@ struct KvTile {
     float lev[16];                                // TurboQuant caches: the format's level table
 };
 
-// Per-lane state of one query row (lane % 32) over the keys seen so far: O^T
-// register 4g + r of tile t is channel 32t + 8g + 4*(lane / 32) + r.
+// Per-lane state of one query row (lane % 32) over the keys seen so far: O^T register 4g + r of tile t is
+// channel 32t + 8g + 4*(lane / 32) + r. o and l are on the scale 2^-m_use, and l is THIS LANE's share of the
+// row's sum (its keys of every tile; the two halves of a wave are added once, at the end: row_sum).
+// The reference exponent of the online softmax need not be the running maximum: any value within a fixed
+// distance below it keeps every probability bounded (here by 2^kMaxSlack = 256, far inside FP16 and harmless to
+// the FP32 sums), and the quotient O / l does not depend on it. m_use is the reference (the raw score it was
+// taken from times scale_log2; 0 while the row has seen no key) and bar that raw score + the slack in raw units:
+// only a tile with a score above the bar moves the reference - after a row's first tile almost none does,
+// where a reference that follows the maximum moves in nearly half of all tiles on random scores (some one of
+// a wave's 32 rows finds a new maximum). Every lane can tell from its own scores whether a tile is above its
+// row's bar, so a tile that moves no reference costs no exchange between lanes and no arithmetic on the state
+// (65 multiplies per lane). A row's rule depends on that row's scores alone.
 struct RowState {
     f32x16 o[kD / 32];
-    float m, l;                                   // reference exponent (next_reference; base-2 domain) and sum
+    float bar, m_use, l;                          // bar = -inf: the row has seen no key (then m_use = 0)
     __device__ __forceinline__ void reset() {
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
-        m = -INFINITY;
+        bar = -INFINITY;
+        m_use = 0.0f;
         l = 0.0f;
     }
+    // mx: this lane's raw maximum of the tile at hand. Called (by the whole wave) when some lane's is above its bar.
+    __device__ __forceinline__ void move_reference(float mx, float scale_log2) {
+        mx = max_xor32(mx);
+        const bool moves = mx > bar;                                                  // then mx is finite
+        const float use = moves ? mx * scale_log2 : m_use;
+        const float alpha = bar == -INFINITY ? 0.0f : exp2_fast(m_use - use);         // exactly 1 where nothing moves
+        l *= alpha;
+#pragma unroll
+        for (int t = 0; t < kD / 32; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+        bar = moves ? mx + kMaxSlack / scale_log2 : bar;
+        m_use = use;
+    }
+    __device__ __forceinline__ float reference() const { return bar == -INFINITY ? -INFINITY : m_use; }
+    __device__ __forceinline__ float row_sum() const { return sum_xor32(l); }
 };
 
 // Keys t0 .. t0+63 of KV head kvh, first into registers (fetch: issued a tile
@@ -322,7 +340,7 @@ __device__ __forceinline__ void tile_scores(const KvTile& tile, const h16x8 (&qf
 // four 16-key steps. Slot e of this lane in step (a, sp) is register 8*sp + e
 // of s[a], i.e. key 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte
 // reads of V^T below. O is rescaled only when some row's reference exponent
-// moved (next_reference): the factor is exactly 1 otherwise.
+// moves (RowState::move_reference).
 __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], RowState& st,
                                             int col, int half, float scale_log2) {
     float mx = -INFINITY;
@@ -330,29 +348,15 @@ __device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], 
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
-    mx = max_xor32(mx) * scale_log2;
-    const float m_new = next_reference(st.m, mx);
-    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-    float sum = 0.0f;
+    if (__builtin_amdgcn_ballot_w64(mx > st.bar) != 0) st.move_reference(mx, scale_log2);
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float p = exp2_fast(fmaf(s[a][r], scale_log2, -m_use));
+            const float p = exp2_fast(fmaf(s[a][r], scale_log2, -st.m_use));
             s[a][r] = p;
-            sum += p;
+            st.l += p;
         }
-    sum = sum_xor32(sum);
-    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
-        const float alpha = exp2_fast(st.m - m_use);
-        st.l *= alpha;
-#pragma unroll
-        for (int t = 0; t < kD / 32; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
-    }
-    st.l += sum;
-    st.m = m_new;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int a = u >> 1, sp = u & 1;
@@ -436,7 +440,8 @@ __global__ __launch_bounds__(kBlock, 2) void prefill128(
     }
 
     if (qrow < q_len) {
-        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+        const float l_row = st.row_sum();
+        const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
         h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
@@ -673,10 +678,12 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     // The row maximum (scaled) of the tile in hand: taken while the vector ALU has nothing else to do, behind the
     // first V^T P^T MFMAs of the tile before (behind the first scores in the prologue).
     hide(0, s_pp[0]);
-    float mx_cur = -INFINITY;
+    {
+        float mx = -INFINITY;
 #pragma unroll
-    for (int q = 0; q < 32; ++q) mx_cur = fmaxf(mx_cur, s_pp[0][q >> 4][q & 15]);
-    mx_cur = max_xor32(mx_cur) * scale_log2;
+        for (int q = 0; q < 32; ++q) mx = fmaxf(mx, s_pp[0][q >> 4][q & 15]);
+        st.move_reference(mx, scale_log2);
+    }
     // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
     auto body = [&](int j, auto parity_c) {
         constexpr int P = decltype(parity_c)::value;
@@ -695,9 +702,6 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         h16x8 kf[3];
         kf[0] = k_frag(0);
         kf[1] = k_frag(1);
-        float sum = 0.0f;
-        const float m_new = next_reference(st.m, mx_cur);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         h16x8 pf[4];
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
@@ -707,8 +711,8 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int q = 2 * k; q < 2 * k + 2; ++q) {
-                const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -m_use));
-                sum += p;
+                const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -st.m_use));
+                st.l += p;
                 s_cur[q >> 4][q & 15] = p;
             }
         }
@@ -722,17 +726,9 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             pf[q >> 3][q & 7] = h[0];
             pf[q >> 3][(q & 7) + 1] = h[1];
         }
-        sum = sum_xor32(sum);
-        if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
-            const float alpha = exp2_fast(st.m - m_use);
-            st.l *= alpha;
-#pragma unroll
-            for (int t = 0; t < kD / 32; ++t)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
-        }
-        st.l += sum;
-        st.m = m_new;
+        // (the compiler would sink the exponentials past the branch in hide() to their first use, out from under
+        // the MFMAs they were placed behind: their results are pinned here)
+        asm volatile("" : "+v"(pf[0]), "+v"(pf[1]), "+v"(pf[2]), "+v"(pf[3]), "+v"(st.l));
         // block 2: O^T += V^T P^T on the matrix pipe, the V^T fragments transposed out of the row-major tile
         const char* vb = reinterpret_cast<const char*>(&tiles.v[P][0]);
         auto v_frag = [&](int k) {                            // step k = 4 u + t
@@ -757,15 +753,14 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
             if (k + 2 < 16) vf[(k + 2) % 3] = v_frag(k + 2);
             st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (k < 4) {                                      // the next tile's row maximum, where the vector ALU idles
+            if (k < 4) {                                      // this lane's maximum of the next tile, where the vector ALU idles
 #pragma unroll
                 for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_next[q >> 4][q & 15]);
-            } else if (k == 4) {
-                mx_cur = max_xor32(mx) * scale_log2;
             }
         }
         __builtin_amdgcn_s_setprio(1);
         __builtin_amdgcn_sched_barrier(0);
+        if (__builtin_amdgcn_ballot_w64(mx > st.bar) != 0) st.move_reference(mx, scale_log2);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // K j+2 and V j+1 landed
         __syncthreads();
     };
@@ -778,6 +773,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no copy may land after the workgroup has gone
+    const float l_row = st.row_sum();
     if (kSplit) {
         if (qrow < q_len) {
             float* rec = parts + (((size_t)qrow * n_q_heads + head) * n_runs + run) * kPartFloats;
@@ -788,12 +784,12 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
                 for (int g = 0; g < 4; ++g)
                     *reinterpret_cast<float4*>(rec + 32 * t + 8 * g + 4 * half) =
                         float4{st.o[t][4 * g], st.o[t][4 * g + 1], st.o[t][4 * g + 2], st.o[t][4 * g + 3]};
-            if (half == 0) *reinterpret_cast<float2*>(rec + kD) = float2{st.m, st.l};
+            if (half == 0) *reinterpret_cast<float2*>(rec + kD) = float2{st.reference(), l_row};
         }
         return;
     }
     if (qrow < q_len) {
-        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+        const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
         h16* op = O + ((size_t)qrow * n_q_heads + head) * kD;
         // register 4 g + r of tile t is channel 32 t + 8 g + 4 half + r
         typedef h16 h16x4 __attribute__((ext_vector_type(4)));
@@ -947,7 +943,8 @@ __global__ __launch_bounds__(kWave) void decode128(
 
     if (g >= group) return;
     if (n_parts == 1) {
-        const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+        const float l_row = st.row_sum();
+        const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
         h16* op = O + (size_t)head * kD;
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
@@ -960,7 +957,8 @@ __global__ __launch_bounds__(kWave) void decode128(
             }
     } else {
         float* dst = parts + ((size_t)head * n_parts + part) * kPartFloats;
-        if (half == 0) { dst[kD] = st.m; dst[kD + 1] = st.l; }
+        const float l_row = st.row_sum();
+        if (half == 0) { dst[kD] = st.reference(); dst[kD + 1] = l_row; }
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
