@@ -99,44 +99,74 @@ struct KvTile {
 // Per-lane state of one query row (lane % 32) over the keys seen so far: O^T register 4g + r of tile t is
 // channel 32t + 8g + 4*(lane / 32) + r. o and l are on the scale 2^-m_use, and l is THIS LANE's share of the
 // row's sum (its keys of every tile; the two halves of a wave are added once, at the end: row_sum).
-// The reference exponent of the online softmax need not be the running maximum: any value within a fixed
-// distance below it keeps every probability bounded (here by 2^kMaxSlack = 256, far inside FP16 and harmless to
-// the FP32 sums), and the quotient O / l does not depend on it. m_use is the reference (the raw score it was
-// taken from times scale_log2; 0 while the row has seen no key) and bar that raw score + the slack in raw units:
-// only a tile with a score above the bar moves the reference - after a row's first tile almost none does,
-// where a reference that follows the maximum moves in nearly half of all tiles on random scores (some one of
-// a wave's 32 rows finds a new maximum). Every lane can tell from its own scores whether a tile is above its
-// row's bar, so a tile that moves no reference costs no exchange between lanes and no arithmetic on the state
-// (65 multiplies per lane). A row's rule depends on that row's scores alone.
+// The reference exponent m_use of the online softmax need not be the running maximum: with any value not far
+// below it the probabilities stay inside FP16 and the FP32 sums, and the quotient O / l does not depend on it. So
+// a tile's probabilities are formed with the reference AS IT STANDS, with no look at the tile's maximum, and each
+// lane compares the sum of its 32 against a bar (thr): none of them can be larger than their sum. Only where a
+// sum passes the bar - or a row has seen no key yet (thr < 0: any sum passes) - are the rows' maxima taken and
+// exchanged, the reference moved up where a row's maximum is more than kMaxSlack above it, O and l rescaled, and
+// the tile's probabilities formed again (settle; the raw scores are still there). After a row's first tile that
+// almost never happens, where a reference that follows the maximum moves in nearly half of all tiles on random
+// scores (some one of a wave's 32 rows finds a new maximum): a tile costs no maximum, no exchange between lanes
+// and no arithmetic on the state. A row's rule depends on that row's scores alone.
+constexpr float kSumBar = 32768.0f;               // 2^15: a lane's 32 probabilities of a tile, each below FP16's 65504
 struct RowState {
     f32x16 o[kD / 32];
-    float bar, m_use, l;                          // bar = -inf: the row has seen no key (then m_use = 0)
+    float thr, m_use, l;                          // thr < 0: the row has seen no key (then m_use = 0), else kSumBar
     __device__ __forceinline__ void reset() {
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
-        bar = -INFINITY;
+        thr = -1.0f;
         m_use = 0.0f;
         l = 0.0f;
     }
-    // mx: this lane's raw maximum of the tile at hand. Called (by the whole wave) when some lane's is above its bar.
-    __device__ __forceinline__ void move_reference(float mx, float scale_log2) {
+    // mx: this lane's raw maximum of the tile at hand. Called by the whole wave.
+    __device__ __forceinline__ void settle(float mx, float scale_log2) {
         mx = max_xor32(mx);
-        const bool moves = mx > bar;                                                  // then mx is finite
-        const float use = moves ? mx * scale_log2 : m_use;
-        const float alpha = bar == -INFINITY ? 0.0f : exp2_fast(m_use - use);         // exactly 1 where nothing moves
+        const bool unseen = thr < 0.0f;
+        const float top = mx * scale_log2;
+        const bool moves = unseen ? mx > -INFINITY : top > m_use + kMaxSlack;
+        const float use = moves ? top : m_use;
+        const float alpha = unseen ? 0.0f : exp2_fast(m_use - use);                   // exactly 1 where nothing moves
         l *= alpha;
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-        bar = moves ? mx + kMaxSlack / scale_log2 : bar;
         m_use = use;
+        thr = unseen && !moves ? -1.0f : kSumBar;
     }
-    __device__ __forceinline__ float reference() const { return bar == -INFINITY ? -INFINITY : m_use; }
+    __device__ __forceinline__ float reference() const { return thr < 0.0f ? -INFINITY : m_use; }
     __device__ __forceinline__ float row_sum() const { return sum_xor32(l); }
 };
+// A lane's 32 scores of a tile -> probabilities on the reference m_use, rounded to FP16 two per conversion
+// (v_cvt_pk_f16_f32) into the B operand's slots (score q of the tile: slot q % 8 of key step q / 8), and their
+// FP32 sum in this order.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void probabilities(const f32x16 (&s)[2], float scale_log2, float m_use, h16x8 (&pf)[4],
+                                              float& sum) {
+    sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 32; q += 2) {
+        const f32x2 two = {exp2_fast(fmaf(s[q >> 4][q & 15], scale_log2, -m_use)),
+                           exp2_fast(fmaf(s[q >> 4][(q & 15) + 1], scale_log2, -m_use))};
+        sum += two[0];
+        sum += two[1];
+        const h16x2 h = __builtin_convertvector(two, h16x2);
+        pf[q >> 3][q & 7] = h[0];
+        pf[q >> 3][(q & 7) + 1] = h[1];
+    }
+}
+__device__ __forceinline__ float lane_max(const f32x16 (&s)[2]) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
+    return mx;
+}
 
 // Keys t0 .. t0+63 of KV head kvh, first into registers (fetch: issued a tile
 // ahead, so the loads fly while the previous tile is computed), then into LDS
@@ -340,36 +370,27 @@ __device__ __forceinline__ void tile_scores(const KvTile& tile, const h16x8 (&qf
 // four 16-key steps. Slot e of this lane in step (a, sp) is register 8*sp + e
 // of s[a], i.e. key 32a + 16sp + 8(e / 4) + 4*half + e % 4: the two 8-byte
 // reads of V^T below. O is rescaled only when some row's reference exponent
-// moves (RowState::move_reference).
-__device__ __forceinline__ void tile_update(const KvTile& tile, f32x16 (&s)[2], RowState& st,
+// moves (RowState::settle).
+__device__ __forceinline__ void tile_update(const KvTile& tile, const f32x16 (&s)[2], RowState& st,
                                             int col, int half, float scale_log2) {
-    float mx = -INFINITY;
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[a][r]);
-    if (__builtin_amdgcn_ballot_w64(mx > st.bar) != 0) st.move_reference(mx, scale_log2);
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float p = exp2_fast(fmaf(s[a][r], scale_log2, -st.m_use));
-            s[a][r] = p;
-            st.l += p;
-        }
+    h16x8 pf[4];
+    float sum;
+    probabilities(s, scale_log2, st.m_use, pf, sum);
+    if (__builtin_amdgcn_ballot_w64(sum > st.thr) != 0) {
+        st.settle(lane_max(s), scale_log2);
+        probabilities(s, scale_log2, st.m_use, pf, sum);
+    }
+    st.l += sum;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int a = u >> 1, sp = u & 1;
-        h16x8 pf;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pf[e] = (h16)s[a][8 * sp + e];
 #pragma unroll
         for (int t = 0; t < kD / 32; ++t) {
             const h16* base = &tile.vt[(32 * t + col) * kVtStride + 32 * a + 16 * sp + 4 * half];
             const h16x4 lo = *reinterpret_cast<const h16x4*>(base);
             const h16x4 hi = *reinterpret_cast<const h16x4*>(base + 8);
             const h16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, st.o[t], 0, 0, 0);
+            st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[u], st.o[t], 0, 0, 0);
         }
     }
 }
@@ -678,12 +699,6 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     // The row maximum (scaled) of the tile in hand: taken while the vector ALU has nothing else to do, behind the
     // first V^T P^T MFMAs of the tile before (behind the first scores in the prologue).
     hide(0, s_pp[0]);
-    {
-        float mx = -INFINITY;
-#pragma unroll
-        for (int q = 0; q < 32; ++q) mx = fmaxf(mx, s_pp[0][q >> 4][q & 15]);
-        st.move_reference(mx, scale_log2);
-    }
     // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
     auto body = [&](int j, auto parity_c) {
         constexpr int P = decltype(parity_c)::value;
@@ -703,32 +718,33 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         kf[0] = k_frag(0);
         kf[1] = k_frag(1);
         h16x8 pf[4];
+        float sum = 0.0f;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             __builtin_amdgcn_sched_barrier(0);
             if (k + 2 < 16) kf[(k + 2) % 3] = k_frag(k + 2);
             s_next[k >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[k % 3], qf[k & 7], s_next[k >> 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int q = 2 * k; q < 2 * k + 2; ++q) {
-                const float p = exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -st.m_use));
-                st.l += p;
-                s_cur[q >> 4][q & 15] = p;
+            {                                                 // scores 2 k, 2 k + 1: as in probabilities()
+                const int q = 2 * k;
+                const f32x2 two = {exp2_fast(fmaf(s_cur[q >> 4][q & 15], scale_log2, -st.m_use)),
+                                   exp2_fast(fmaf(s_cur[q >> 4][(q & 15) + 1], scale_log2, -st.m_use))};
+                sum += two[0];
+                sum += two[1];
+                const h16x2 h = __builtin_convertvector(two, h16x2);
+                pf[q >> 3][q & 7] = h[0];
+                pf[q >> 3][(q & 7) + 1] = h[1];
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        // two probabilities per conversion (v_cvt_pk_f16_f32, round to nearest even like the single one)
-        typedef float f32x2 __attribute__((ext_vector_type(2)));
-#pragma unroll
-        for (int q = 0; q < 32; q += 2) {
-            const f32x2 two = {s_cur[q >> 4][q & 15], s_cur[q >> 4][(q & 15) + 1]};
-            const h16x2 h = __builtin_convertvector(two, h16x2);
-            pf[q >> 3][q & 7] = h[0];
-            pf[q >> 3][(q & 7) + 1] = h[1];
+        // (the compiler would sink the conversions past the branches below to their first use, out from under the
+        // MFMAs they were placed behind: their results are pinned here)
+        asm volatile("" : "+v"(pf[0]), "+v"(pf[1]), "+v"(pf[2]), "+v"(pf[3]), "+v"(sum));
+        if (__builtin_amdgcn_ballot_w64(sum > st.thr) != 0) {     // rare (RowState): the reference settles, the tile again
+            st.settle(lane_max(s_cur), scale_log2);
+            probabilities(s_cur, scale_log2, st.m_use, pf, sum);
         }
-        // (the compiler would sink the exponentials past the branch in hide() to their first use, out from under
-        // the MFMAs they were placed behind: their results are pinned here)
-        asm volatile("" : "+v"(pf[0]), "+v"(pf[1]), "+v"(pf[2]), "+v"(pf[3]), "+v"(st.l));
+        st.l += sum;
         // block 2: O^T += V^T P^T on the matrix pipe, the V^T fragments transposed out of the row-major tile
         const char* vb = reinterpret_cast<const char*>(&tiles.v[P][0]);
         auto v_frag = [&](int k) {                            // step k = 4 u + t
@@ -746,21 +762,14 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         // matrix pipe under its softmax (1.5-2 % at 14449 rows).
         __builtin_amdgcn_s_setprio(0);
         hide(j + 1, s_next);
-        float mx = -INFINITY;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
             __builtin_amdgcn_sched_barrier(0);
             if (k + 2 < 16) vf[(k + 2) % 3] = v_frag(k + 2);
             st.o[k & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[k % 3], pf[k >> 2], st.o[k & 3], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (k < 4) {                                      // this lane's maximum of the next tile, where the vector ALU idles
-#pragma unroll
-                for (int q = 8 * k; q < 8 * k + 8; ++q) mx = fmaxf(mx, s_next[q >> 4][q & 15]);
-            }
         }
         __builtin_amdgcn_s_setprio(1);
         __builtin_amdgcn_sched_barrier(0);
-        if (__builtin_amdgcn_ballot_w64(mx > st.bar) != 0) st.move_reference(mx, scale_log2);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // K j+2 and V j+1 landed
         __syncthreads();
     };
