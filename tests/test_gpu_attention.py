@@ -253,6 +253,77 @@ def test_prefill_scratch_is_left_alone_when_there_is_nothing_to_split():
         assert bool(torch.isnan(scratch).all())
 
 
+def structured(kind, rows, nq, nkv, hd, kv_len, seed):
+    """Scores with a shape along the keys instead of noise alone: the tile kernels form a tile's probabilities on the
+    softmax reference as it stands and settle it only where a lane's sum passes 2^15 (attention.hip, RowState), so
+    these are the inputs on which that happens in tile after tile, never again after the first, or once, mid-way.
+    q is about one in every channel, so a key's score is about the sum of its channels."""
+    rng = np.random.default_rng(seed)
+    q = (1.0 + 0.05 * rng.standard_normal((rows, nq, hd))).astype(np.float16)
+    noise = 0.02 * rng.standard_normal((kv_len, nkv, hd))
+    t = np.arange(kv_len, dtype=np.float64)[:, None, None]
+    if kind == "rising":          # 5.1 a key raw = 0.65 in base-2 exponents: 42 a tile of 64 keys
+        k = 0.04 * t + noise
+    elif kind == "falling":       # the first tile holds the maximum; later probabilities fall to nothing
+        k = 0.04 * (kv_len - 1 - t) + noise
+    else:                         # "spike": noise, one key 49 base-2 exponents above it in the sixth tile
+        k = 3.0 * noise
+        k[333] = 3.0
+    v = rng.standard_normal((kv_len, nkv, hd))
+    return bits_of_np(q), bits_of_np(k.astype(np.float16)), bits_of_np(v.astype(np.float16))
+
+
+def bits_of_np(a):
+    return np.ascontiguousarray(a).view(np.uint16)
+
+
+@pytest.mark.parametrize("kind", ["rising", "falling", "spike"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_prefill_where_the_softmax_reference_moves(kind, causal):
+    rows, nq, nkv, hd, kv_len = 200, 4, 2, 128, 700
+    off = kv_len - rows
+    q, k, v = structured(kind, rows, nq, nkv, hd, kv_len, 17)
+    ref = oracle.attention_prefill_f32(oracle.widen(q), oracle.widen(k), oracle.widen(v), off, kv_len, causal)
+    d_q, vw = to_dev(q), view_of(to_dev(k), to_dev(v), nkv, hd)
+    vmax = float(np.abs(oracle.widen(v)).max())
+    got = prefill(d_q, vw, nq, hd, rows, off, kv_len, causal)
+    check(got, ref, vmax, f"{kind} scores")
+    # the plain tile kernel: the same state and the same helpers, so the same bits
+    import os
+    os.environ["VV_ATTN_PREFILL_TILE"] = "1"
+    try:
+        tile = prefill(d_q, vw, nq, hd, rows, off, kv_len, causal)
+    finally:
+        os.environ.pop("VV_ATTN_PREFILL_TILE", None)
+    assert np.array_equal(tile, got)
+
+
+@pytest.mark.parametrize("kind", ["rising", "falling", "spike"])
+def test_split_prefill_and_decode_where_the_softmax_reference_moves(kind):
+    """The runs of a split prefill and the slices of a decode hand on (reference, sum, O) records: their references
+    differ by hundreds of base-2 exponents here."""
+    rows, nq, nkv, hd, kv_len = 100, 4, 2, 128, 1200
+    off = kv_len - rows
+    q, k, v = structured(kind, rows, nq, nkv, hd, kv_len, 23)
+    ref = oracle.attention_prefill_f32(oracle.widen(q), oracle.widen(k), oracle.widen(v), off, kv_len, True)
+    d_q, vw = to_dev(q), view_of(to_dev(k), to_dev(v), nkv, hd)
+    vmax = float(np.abs(oracle.widen(v)).max())
+    scratch = torch.full((dev.vv_attn_scratch_bytes(nq, nkv, hd) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    got = prefill_with_scratch(d_q, vw, nq, hd, rows, off, kv_len, scratch)
+    assert not np.isnan(scratch[:8].cpu().numpy()).any(), "this shape was meant to take the split path"
+    check(got, ref, vmax, f"{kind} scores, split prefill")
+    # one decode row over the same cache: 4 query heads (the streaming kernel) and 34 on 2 KV heads (the tile
+    # kernel's decode form, which shares the prefill's state)
+    for heads in (4, 34):
+        q1 = np.ascontiguousarray(np.resize(q[-1:], (1, heads, hd)))
+        ref1 = oracle.attention_prefill_f32(oracle.widen(q1), oracle.widen(k), oracle.widen(v), kv_len - 1, kv_len, True)
+        d_o = torch.full((1, heads, hd), float("nan"), dtype=torch.float16, device="cuda")
+        sc = torch.empty(dev.vv_attn_scratch_bytes(heads, nkv, hd), dtype=torch.uint8, device="cuda")
+        ok(dev.vv_attn_decode(FA2, to_dev(q1).data_ptr(), C.addressof(vw), d_o.data_ptr(), heads, kv_len, None,
+                              sc.data_ptr(), stream()))
+        check(bits_of(d_o), ref1, vmax, f"{kind} scores, decode with {heads} heads")
+
+
 def test_declines_and_edges():
     hd, nkv, nq = 128, 1, 2
     d = torch.zeros((4, nq, hd), dtype=torch.float16, device="cuda")
