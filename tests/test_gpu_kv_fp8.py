@@ -190,6 +190,27 @@ def test_decode_equals_fp16_cache_of_decoded_values(fmt, cache_len, paged):
         assert np.array_equal(bits_of(d_o), outs[0])
 
 
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+@pytest.mark.parametrize("cache_len", [65, 1500, 14449])
+def test_decode_bit_for_bit_where_both_caches_run_the_tile_kernel(fmt, cache_len):
+    """Seventeen query heads per KV head are more than the FP16 cache's streaming decode kernel takes, so the FP16
+    cache of the decoded values runs the tile kernel too: the packed decode must then equal it in every bit -
+    one wrong code on a small channel would show."""
+    nq = 17 * NKV
+    k, v, kq, vq, k16, v16 = fp8_cache(fmt, cache_len, 40 + cache_len % 89)
+    d_q = to_dev(oracle.normal_f16((1, nq, HD), 8))
+    scratch = torch.empty(dev.vv_attn_scratch_bytes(nq, NKV, HD), dtype=torch.uint8, device="cuda")
+    outs = []
+    for kk, vv_, f in ((u8(kq), u8(vq), fmt), (to_dev(k16), to_dev(v16), 0)):
+        d_o = torch.full((1, nq, HD), float("nan"), dtype=torch.float16, device="cuda")
+        vw = view(kk, vv_, f)
+        ok(dev.vv_attn_decode(FA2, d_q.data_ptr(), C.addressof(vw), d_o.data_ptr(), nq, cache_len, None,
+                              scratch.data_ptr(), stream()))
+        outs.append(bits_of(d_o))
+    assert not np.isnan(oracle.widen(outs[0])).any()
+    assert np.array_equal(outs[0], outs[1])
+
+
 def test_formats_and_shapes_not_served():
     P = torch.zeros(4096, dtype=torch.float16, device="cuda").data_ptr()
     for fmt in (7, 9):                # FP32 (the CPU path's), no such format

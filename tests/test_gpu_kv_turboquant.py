@@ -163,6 +163,28 @@ def test_decode_equals_fp16_cache_of_unpacked_vectors_and_tracks_fp16_attention(
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("cache_len", [65, 3000])
+def test_decode_bit_for_bit_where_both_caches_run_the_tile_kernel(fmt, cache_len):
+    """Seventeen query heads per KV head are more than the FP16 cache's streaming decode kernel takes, so the FP16
+    cache of the unpacked vectors runs the tile kernel too: the packed decode must then equal it in every bit."""
+    nq = 17 * NKV
+    k, v = qwen_like(cache_len, 9 + cache_len)
+    ks, km = oracle.kv_store_tq(k, oracle.kv_build_ref(k), fmt)
+    vs, vm = oracle.kv_store_tq(v, None, fmt)
+    k16, v16 = oracle.kv_unpack(ks, km, fmt), oracle.kv_unpack(vs, vm, fmt)
+    d_q = to_dev(oracle.kv_rotate(oracle.normal_f16((1, nq, HD), 13, std=0.6)))
+    scratch = torch.empty(dev.vv_attn_scratch_bytes(nq, NKV, HD), dtype=torch.uint8, device="cuda")
+    outs = []
+    for vw in (view(u8(ks), u8(vs), to_dev(km), to_dev(vm), fmt), view(to_dev(k16), to_dev(v16), None, None, 0)):
+        d_o = torch.full((1, nq, HD), float("nan"), dtype=torch.float16, device="cuda")
+        ok(dev.vv_attn_decode(FA2, d_q.data_ptr(), C.addressof(vw), d_o.data_ptr(), nq, cache_len, None,
+                              scratch.data_ptr(), stream()))
+        outs.append(bits_of(d_o))
+    assert not np.isnan(oracle.widen(outs[0])).any()
+    assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
 def test_prefill_equals_fp16_cache_of_unpacked_vectors(fmt):
     nq, q_len, q_offset, kv_len = 28, 70, 130, 200
     k, v = qwen_like(kv_len, 11)
