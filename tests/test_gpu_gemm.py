@@ -57,6 +57,12 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           (2100, 2100, 192), (1100, 4096, 64), (14449, 512, 128), (70, 33000, 64),      # ... and one row of 258 tiles
           # the 64x64 tile fed the same way: 256 tiles or fewer (eight stages), more (four), ragged, one slab
           (2048, 512, 3584), (285, 3584, 3584), (130, 200, 64), (1000, 1100, 192), (65, 64, 128),
+          # 17 .. 64 rows, K in whole 64-K lines: the weight-streaming kernel that fetches the activations by whole cache
+          # lines (two, three and four row tiles; ragged N; one line; five lines, so that three waves have none; a long K)
+          (17, 100, 320), (33, 52, 64), (40, 3584, 18944), (64, 3584, 1088), (48, 30, 4096), (20, 3584, 3584),
+          (2, 264, 3584), (5, 3584, 18944), (16, 18944, 3584), (13, 50, 64),
+          # 17 .. 64 rows, N too wide for that kernel: one row of 128x128 tiles (and just below their bar: 64-wide ones)
+          (24, 18944, 3584), (64, 16300, 128), (33, 16200, 128),
           # one row, few long weight rows: two output columns per wave (an odd count leaves the last wave one)
           (1, 3584, 18944), (1, 37, 8192), (1, 1, 8200)]
 
@@ -73,9 +79,10 @@ def test_gemm_against_oracle_and_tile(M, N, K):
     d_t = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     tile = run(dev.vv_gemm_fp16_tile_dev, d_a, d_b, d_t, M, N, K)
     check(tile, ref, mag, f"tile {M}x{N}x{K}")
-    big = K % 64 == 0 and M > 64
+    big = K % 64 == 0 and (M > 64 or (M > 16 and N >= 16257))      # the latter: one row of at least 128 tiles of 128
     if big:
-        # the tiles fed in 128-byte slabs (the choice above 64 rows when K % 64 == 0) multiply with the 16x16x32
+        # the tiles fed in 128-byte slabs (the choice above 64 rows, and from 17 rows on where N is very wide, when
+        # K % 64 == 0) multiply with the 16x16x32
         # instructions, which add 32 products at a time where the other tiles add 16: same sums, another
         # rounding of the FP32 partials
         diff = np.abs(oracle.widen(got) - oracle.widen(tile))

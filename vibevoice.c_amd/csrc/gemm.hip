@@ -22,6 +22,9 @@
 //                           straight into 16x16x32 MFMA operands, K split
 //                           over the eight waves of a workgroup; bound by the
 //                           weight bytes.
+//   gemm_skinny_lines<kMT>  the same for FP16 weights and K % 64 == 0: both
+//                           operands come by whole cache lines through each
+//                           wave's own LDS ring (same bits).
 //   gemv_row<kSplit>        M == 1 (a decode step): one to four waves per
 //                           output column stream that weight row once with
 //                           non-temporal 16-byte loads.
@@ -698,6 +701,50 @@ struct SkinnyProjs {
     int vec[3];
 };
 
+// The eight waves' partial tiles, already in `part`, summed in wave order and stored: register r of lane l is column
+// n0 + 4(l / 16) + r of row 16t + l % 16. A bias, when given, is added to the rounded FP16 product and rounded again.
+template <int kMT>
+__device__ __forceinline__ void skinny_store(const f32x4 (*part)[kMT][kWave], h16* __restrict__ C,
+                                             const h16* __restrict__ bias, int M, int N, int n0, int vec_store,
+                                             float alpha, float beta) {
+    const int tid = (int)threadIdx.x, lane = tid & 63, r16 = lane & 15, ks = lane >> 4;
+    if (tid < kMT * kWave) {
+        const int t = tid >> 6;
+        f32x4 sum = part[0][t][lane];
+#pragma unroll
+        for (int w = 1; w < kSkinnyWaves; ++w) {
+            const f32x4 p = part[w][t][lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[r] += p[r];
+        }
+        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        if (m < M && n < N) {
+            h16* crow = C + (size_t)m * N;
+            if (vec_store && n + 3 < N) {
+                typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+                h16x4 old = {0, 0, 0, 0};
+                if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+                h16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    o[r] = to_half(finish(sum[r], alpha, beta, old[r]));
+                    if (bias) o[r] = to_half((float)o[r] + (float)bias[n + r]);
+                }
+                *reinterpret_cast<h16x4*>(crow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) {
+                        const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                        h16 o = to_half(finish(sum[r], alpha, beta, old));
+                        if (bias) o = to_half((float)o + (float)bias[n + r]);
+                        crow[n + r] = o;
+                    }
+            }
+        }
+    }
+}
+
 template <int kMT, int kFmt>
 __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
     const h16* __restrict__ A, SkinnyProjs projs, int M, int K, float alpha, float beta) {
@@ -753,43 +800,120 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
 #pragma unroll
     for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
     __syncthreads();
+    skinny_store<kMT>(part, C, bias, M, N, n0, vec_store, alpha, beta);
+}
 
-    // Register r of lane l is column n0 + 4(l / 16) + r of row 16t + l % 16.
-    if (tid < kMT * kWave) {
-        const int t = tid >> 6;
-        f32x4 sum = part[0][t][lane];
+// The same kernel for FP16 weights and whole 64-K lines (K % 64 == 0), with both operands fetched as WHOLE CACHE
+// LINES. The fragment a lane needs is 16 bytes of one of sixteen rows: a wave's load touches sixteen half lines, and
+// 224 workgroups reading the same activations that way get 8 TB/s out of L2 where whole lines give 19-27 (measured
+// with the two patterns alone: 64 rows x 18944, 65.7 us against 20.2); the weights' gather costs the same way. So a
+// wave copies its line of the activations and of the weights straight into LDS, eight rows of 128 bytes per
+// instruction (lane: row lane / 8, chunk lane % 8 ^ row, so that the fragment reads below find the eight rows of a
+// chunk in eight different groups of banks), kDepth lines ahead, and reads the fragments from there. Its LDS is
+// its own: no barrier, only its own counters (every copy of the loop is issued by hand, in a fixed number per line,
+// so that "all but the last kDepth - 1 lines' copies" is a constant). Same products in the same order: the same
+// bits as gemm_skinny. 64 x 3584 x 18944: 97.9 -> 55.7 us; 24 rows: 53.7 -> 36.7; 8 rows: 32.2 -> 27.7.
+template <int kMT> struct SkinnyLines {
+    static constexpr int kTiles = kMT + 1;                                            // the weights' rows: one more
+    static constexpr int kDepth = kMT == 1 ? 4 : kMT == 2 ? 3 : 2;                    // lines in flight per wave
+    static constexpr int kLineBytes = kTiles * 2048;                                  // 16 rows x 128 bytes a tile
+    static constexpr int kPerLine = 2 * kTiles;                                       // copies per line
+    static constexpr size_t kLdsBytes = (size_t)kSkinnyWaves * kDepth * kLineBytes;   // 128 / 144 / 128 / 160 KB
+    static_assert(kLdsBytes <= 160 * 1024 && kLdsBytes >= sizeof(f32x4) * kSkinnyWaves * kMT * kWave,
+                  "the ring fits, and the partial tiles fit into it");
+    static_assert((kDepth - 1) * kPerLine < 64, "a wave's six-bit load counter");
+};
+
+template <int kMT>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
+    const h16* __restrict__ A, SkinnyProjs projs, int M, int K, float alpha, float beta) {
+    typedef SkinnyLines<kMT> Shape;
+    extern __shared__ __align__(16) char skinny_lds[];
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int which = ((int)blockIdx.x >= projs.first[1]) + ((int)blockIdx.x >= projs.first[2]);
+    const h16* __restrict__ W = static_cast<const h16*>(projs.w[which]);
+    const h16* __restrict__ bias = projs.bias[which];
+    h16* __restrict__ C = projs.y[which];
+    const int N = projs.n[which], vec_store = projs.vec[which];
+    const int n0 = ((int)blockIdx.x - projs.first[which]) * 16;
+    const int nlines = K / 64;
+    const int mine = (nlines - wave + kSkinnyWaves - 1) / kSkinnyWaves;      // lines wave, wave + 8, ...
+
+    const uint32_t ring = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)skinny_lds) +
+                          (uint32_t)wave * (Shape::kDepth * Shape::kLineBytes);
+    // copy j of a line: rows 8 j .. 8 j + 7 of the activations (of the weights' sixteen, for the last tile); this
+    // lane: row 8 j + lane / 8, the chunk whose slot in the row is lane % 8
+    const char* row[2 * Shape::kTiles];
 #pragma unroll
-        for (int w = 1; w < kSkinnyWaves; ++w) {
-            const f32x4 p = part[w][t][lane];
+    for (int j = 0; j < 2 * Shape::kTiles; ++j) {
+        const int r = 8 * j + (lane >> 3);
+        const h16* at = j < 2 * kMT ? A + (size_t)min(r, M - 1) * K : W + (size_t)min(n0 + r - 16 * kMT, N - 1) * K;
+        row[j] = reinterpret_cast<const char*>(at) + (((lane & 7) ^ (lane >> 3)) * 16);
+    }
+    // fragment (tile t, step u): row 16 t + r16 = copy 2 t + r16 / 8, row r16 % 8 of it; chunk 4 u + ks
+    uint32_t frag[2];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sum[r] += p[r];
-        }
-        const int m = 16 * t + r16, n = n0 + 4 * ks;
-        if (m < M && n < N) {
-            h16* crow = C + (size_t)m * N;
-            if (vec_store && n + 3 < N) {
-                typedef h16 h16x4 __attribute__((ext_vector_type(4)));
-                h16x4 old = {0, 0, 0, 0};
-                if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
-                h16x4 o;
+    for (int u = 0; u < 2; ++u) frag[u] = (uint32_t)((r16 >> 3) * 1024 + (r16 & 7) * 128 + (((4 * u + ks) ^ (r16 & 7)) * 16));
+    // the copies of this wave's i-th line, into slot i % kDepth
+    auto request = [&](int i, int slot) {
+        const size_t line = (size_t)(wave + kSkinnyWaves * i) * 128;
+        const uint32_t at = ring + (uint32_t)slot * Shape::kLineBytes;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    o[r] = to_half(finish(sum[r], alpha, beta, old[r]));
-                    if (bias) o[r] = to_half((float)o[r] + (float)bias[n + r]);
-                }
-                *reinterpret_cast<h16x4*>(crow + n) = o;
-            } else {
+        for (int j = 0; j < 2 * Shape::kTiles; ++j)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         : : "s"(at + (uint32_t)j * 1024u), "v"(row[j] + line) : "memory", "m0");
+    };
+
+    f32x4 acc[kMT];
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (n + r < N) {
-                        const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
-                        h16 o = to_half(finish(sum[r], alpha, beta, old));
-                        if (bias) o = to_half((float)o + (float)bias[n + r]);
-                        crow[n + r] = o;
-                    }
+    for (int t = 0; t < kMT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < Shape::kDepth; ++d)
+        if (d < mine) request(d, d);
+    // (unrolled by the depth, so that a line's LDS slot is fixed)
+    for (int i0 = 0; i0 < mine; i0 += Shape::kDepth) {
+#pragma unroll
+        for (int d = 0; d < Shape::kDepth; ++d) {
+            const int i = i0 + d;
+            if (i >= mine) break;
+            // Line i has landed when only the copies of the kDepth - 1 lines behind it are still counted; towards
+            // the end fewer are behind it, and the wave waits for them all (it has nothing left to ask for)
+            if (i + Shape::kDepth - 1 < mine)
+                asm volatile("s_waitcnt vmcnt(%0)" : : "n"((Shape::kDepth - 1) * Shape::kPerLine) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const char* slot = skinny_lds + (size_t)wave * (Shape::kDepth * Shape::kLineBytes) + d * Shape::kLineBytes;
+            u32x4 x[kMT][2], wf[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) wf[u] = *reinterpret_cast<const u32x4*>(slot + kMT * 2048 + frag[u]);
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) x[t][u] = *reinterpret_cast<const u32x4*>(slot + t * 2048 + frag[u]);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int t = 0; t < kMT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, wf[u]),
+                                                                    __builtin_bit_cast(h16x8, x[t][u]),
+                                                                    acc[t], 0, 0, 0);
+            if (i + Shape::kDepth < mine) {
+                // the slot is read (its fragments are in registers) before it is refilled
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                request(i + Shape::kDepth, d);
             }
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                                          // every wave is done with its ring: it becomes `part`
+    f32x4 (*part)[kMT][kWave] = reinterpret_cast<f32x4 (*)[kMT][kWave]>(skinny_lds);
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    __syncthreads();
+    skinny_store<kMT>(part, C, bias, M, N, n0, vec_store, alpha, beta);
 }
 
 // The 64-column tile count below which the weight-streaming kernel beats the
@@ -798,11 +922,35 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
 inline bool few_tiles(int N) { return (long)((N + 63) / 64) < 200; }
 inline bool skinny_serves(int M, int N) { return M >= 2 && (M <= 16 || (M <= 64 && few_tiles(N))); }
 
+template <typename Kernel>
+bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes);
+
+template <int kMT>
+bool launch_skinny_lines(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha, float beta,
+                         hipStream_t st) {
+    static thread_local int ready = -1;
+    if (!allow_big_lds(gemm_skinny_lines<kMT>, ready, SkinnyLines<kMT>::kLdsBytes)) return false;
+    gemm_skinny_lines<kMT><<<dim3((unsigned)blocks), kSkinnyWaves * kWave, SkinnyLines<kMT>::kLdsBytes, st>>>(
+        A, projs, M, K, alpha, beta);
+    return true;
+}
+
 template <int kFmt>
 void launch_skinny_as(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha,
                       float beta, hipStream_t st) {
     constexpr int kThreads = kSkinnyWaves * kWave;
     const dim3 grid((unsigned)blocks);
+    // FP16 weights in whole lines: both operands by whole cache lines through LDS. Should the launch be refused, the
+    // plain kernel below serves.
+    if (kFmt == kWoF16 && K % 64 == 0) {
+        bool aligned = aligned16(A);
+        for (int p = 0; p < 3; ++p) aligned = aligned && (projs.w[p] == nullptr || aligned16(projs.w[p]));
+        if (aligned && (M <= 16 ? launch_skinny_lines<1>(A, projs, blocks, M, K, alpha, beta, st)
+                        : M <= 32 ? launch_skinny_lines<2>(A, projs, blocks, M, K, alpha, beta, st)
+                        : M <= 48 ? launch_skinny_lines<3>(A, projs, blocks, M, K, alpha, beta, st)
+                                  : launch_skinny_lines<4>(A, projs, blocks, M, K, alpha, beta, st)))
+            return;
+    }
     if (M <= 16) gemm_skinny<1, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
     else if (M <= 32) gemm_skinny<2, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
     else if (M <= 48) gemm_skinny<3, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
@@ -1020,7 +1168,10 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         // (copy-fed, four stages deep, the 128x128 tile already pays with half the compute units busy:
         // 1024 x 3584 x 3584 in 31 us as 224 tiles of 128, 50 us as 896 tiles of 64; at 112 tiles the 64s win)
         const long enough128 = K % (kDma64SlabBytes / 2) == 0 ? 128 : 256;
-        choice = wg256 >= 512 ? k256 : (M > 64 && wg128 >= enough128) ? k128dma : (M > 32) ? k64 : k32;
+        // (17 .. 64 rows arrive here when N is too wide for the weight-streaming kernel: one row of 128x128 tiles,
+        // bound by the weight bytes - 24 x 18944 x 3584 in 33 us against 46 us as 64-wide tiles)
+        const bool rows128 = M > 64 || (M > 16 && K % (kDma64SlabBytes / 2) == 0);
+        choice = wg256 >= 512 ? k256 : (rows128 && wg128 >= enough128) ? k128dma : (M > 32) ? k64 : k32;
     }
     switch (choice) {
         case k128dma: launch_128(A, B, C, M, N, K, alpha, beta, st); break;
