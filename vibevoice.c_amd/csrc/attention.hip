@@ -551,6 +551,9 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     const int qw0 = q0 + wave * 32;
     const int qrow = qw0 + col;
     const int q_abs = q_offset + qrow;
+    // A wave whose 32 rows all lie past the chunk's end (a chunk of a few rows against a long cache: three of a
+    // workgroup's four waves) copies its share of every tile and keeps the barriers, and computes nothing.
+    const bool idle = qw0 >= q_len;
     int wg_limit = kv_len;
     if (causal) wg_limit = min(kv_len, q_offset + min(q0 + kQTile, q_len));
     int ntiles = (wg_limit + kKeyTile - 1) / kKeyTile;
@@ -662,7 +665,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) kf_idx[s8] = col * 16 + ((2 * s8 + half) ^ (col & 15));
     f32x16 s_pp[2][2];                        // the scores of the tile in hand and of the next, by tile parity
-    scores(0, s_pp[0]);
+    if (!idle) scores(0, s_pp[0]);
     __syncthreads();                                          // K 0 is read: its buffer may take K 2
 
     // Byte offsets of this lane's fragments from the start of a K / V^T buffer: with the buffer a compile-time
@@ -698,7 +701,7 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
     };
     // The row maximum (scaled) of the tile in hand: taken while the vector ALU has nothing else to do, behind the
     // first V^T P^T MFMAs of the tile before (behind the first scores in the prologue).
-    hide(0, s_pp[0]);
+    if (!idle) hide(0, s_pp[0]);
     // one tile: P = j & 1 names the buffers and which of the two score sets is "this tile"
     auto body = [&](int j, auto parity_c) {
         constexpr int P = decltype(parity_c)::value;
@@ -706,6 +709,11 @@ __global__ __launch_bounds__(kBlock, 2) void prefill_pipe(
         f32x16 (&s_next)[2] = s_pp[P ^ 1];
         request_k(j + 2);                                     // into the buffer tile j's K has left
         request_v(j + 1);                                     // into the buffer tile j - 1's V has left
+        if (idle) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            return;
+        }
         const char* kb = reinterpret_cast<const char*>(&tiles.k[P ^ 1][0]);
         auto k_frag = [&](int k) {                            // step k = 8 a + s8
             return __builtin_bit_cast(h16x8, *reinterpret_cast<const Chunk*>(kb + (k >> 3) * 8192 + kf_byte[k & 7]));
