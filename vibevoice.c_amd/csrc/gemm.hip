@@ -701,23 +701,24 @@ struct SkinnyProjs {
     int vec[3];
 };
 
-// The eight waves' partial tiles, already in `part`, summed in wave order and stored: register r of lane l is column
-// n0 + 4(l / 16) + r of row 16t + l % 16. A bias, when given, is added to the rounded FP16 product and rounded again.
-template <int kMT>
-__device__ __forceinline__ void skinny_store(const f32x4 (*part)[kMT][kWave], h16* __restrict__ C,
+// The eight waves' partial tiles, already in `part`, summed in wave order and stored: register r of lane l of tile
+// (w, t) is column n0 + 16 w + 4(l / 16) + r of row 16t + l % 16. A bias, when given, is added to the rounded FP16
+// product and rounded again.
+template <int kMT, int kWT = 1>
+__device__ __forceinline__ void skinny_store(const f32x4 (*part)[kWT * kMT][kWave], h16* __restrict__ C,
                                              const h16* __restrict__ bias, int M, int N, int n0, int vec_store,
                                              float alpha, float beta) {
     const int tid = (int)threadIdx.x, lane = tid & 63, r16 = lane & 15, ks = lane >> 4;
-    if (tid < kMT * kWave) {
-        const int t = tid >> 6;
-        f32x4 sum = part[0][t][lane];
+    for (int item = tid >> 6; item < kWT * kMT; item += kSkinnyWaves) {
+        const int t = item % kMT;
+        f32x4 sum = part[0][item][lane];
 #pragma unroll
         for (int w = 1; w < kSkinnyWaves; ++w) {
-            const f32x4 p = part[w][t][lane];
+            const f32x4 p = part[w][item][lane];
 #pragma unroll
             for (int r = 0; r < 4; ++r) sum[r] += p[r];
         }
-        const int m = 16 * t + r16, n = n0 + 4 * ks;
+        const int m = 16 * t + r16, n = n0 + 16 * (item / kMT) + 4 * ks;
         if (m < M && n < N) {
             h16* crow = C + (size_t)m * N;
             if (vec_store && n + 3 < N) {
@@ -813,21 +814,23 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny(
 // its own: no barrier, only its own counters (every copy of the loop is issued by hand, in a fixed number per line,
 // so that "all but the last kDepth - 1 lines' copies" is a constant). Same products in the same order: the same
 // bits as gemm_skinny. 64 x 3584 x 18944: 97.9 -> 55.7 us; 24 rows: 53.7 -> 36.7; 8 rows: 32.2 -> 27.7.
-template <int kMT> struct SkinnyLines {
-    static constexpr int kTiles = kMT + 1;                                            // the weights' rows: one more
-    static constexpr int kDepth = kMT == 1 ? 4 : kMT == 2 ? 3 : 2;                    // lines in flight per wave
+// kWT: the weights' tiles of sixteen rows a workgroup takes (16 kWT output columns). Two where the projection is
+// so wide that one would mean a thousand short-lived workgroups: the activations are then copied once for both.
+template <int kMT, int kWT> struct SkinnyLines {
+    static constexpr int kTiles = kMT + kWT;                                          // tiles of a line's slot
+    static constexpr int kDepth = 10 / kTiles < 4 ? 10 / kTiles : 4;                  // lines in flight per wave
     static constexpr int kLineBytes = kTiles * 2048;                                  // 16 rows x 128 bytes a tile
     static constexpr int kPerLine = 2 * kTiles;                                       // copies per line
-    static constexpr size_t kLdsBytes = (size_t)kSkinnyWaves * kDepth * kLineBytes;   // 128 / 144 / 128 / 160 KB
-    static_assert(kLdsBytes <= 160 * 1024 && kLdsBytes >= sizeof(f32x4) * kSkinnyWaves * kMT * kWave,
-                  "the ring fits, and the partial tiles fit into it");
+    static constexpr size_t kLdsBytes = (size_t)kSkinnyWaves * kDepth * kLineBytes;   // 128 .. 160 KB
+    static_assert(kDepth >= 2 && kLdsBytes <= 160 * 1024 &&
+                  kLdsBytes >= sizeof(f32x4) * kSkinnyWaves * kWT * kMT * kWave, "the ring fits, and the partial tiles fit into it");
     static_assert((kDepth - 1) * kPerLine < 64, "a wave's six-bit load counter");
 };
 
-template <int kMT>
+template <int kMT, int kWT>
 __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
     const h16* __restrict__ A, SkinnyProjs projs, int M, int K, float alpha, float beta) {
-    typedef SkinnyLines<kMT> Shape;
+    typedef SkinnyLines<kMT, kWT> Shape;
     extern __shared__ __align__(16) char skinny_lds[];
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -838,13 +841,13 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
     const h16* __restrict__ bias = projs.bias[which];
     h16* __restrict__ C = projs.y[which];
     const int N = projs.n[which], vec_store = projs.vec[which];
-    const int n0 = ((int)blockIdx.x - projs.first[which]) * 16;
+    const int n0 = ((int)blockIdx.x - projs.first[which]) * (16 * kWT);
     const int nlines = K / 64;
     const int mine = (nlines - wave + kSkinnyWaves - 1) / kSkinnyWaves;      // lines wave, wave + 8, ...
 
     const uint32_t ring = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)skinny_lds) +
                           (uint32_t)wave * (Shape::kDepth * Shape::kLineBytes);
-    // copy j of a line: rows 8 j .. 8 j + 7 of the activations (of the weights' sixteen, for the last tile); this
+    // copy j of a line: rows 8 j .. 8 j + 7 of the activations (of the weights' 16 kWT, for the last tiles); this
     // lane: row 8 j + lane / 8, the chunk whose slot in the row is lane % 8
     const char* row[2 * Shape::kTiles];
 #pragma unroll
@@ -867,9 +870,11 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
                          : : "s"(at + (uint32_t)j * 1024u), "v"(row[j] + line) : "memory", "m0");
     };
 
-    f32x4 acc[kMT];
+    f32x4 acc[kWT][kMT];
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int w = 0; w < kWT; ++w)
+#pragma unroll
+        for (int t = 0; t < kMT; ++t) acc[w][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int d = 0; d < Shape::kDepth; ++d)
         if (d < mine) request(d, d);
@@ -886,20 +891,24 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
             else
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             const char* slot = skinny_lds + (size_t)wave * (Shape::kDepth * Shape::kLineBytes) + d * Shape::kLineBytes;
-            u32x4 x[kMT][2], wf[2];
+            u32x4 x[kMT][2], wf[kWT][2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) wf[u] = *reinterpret_cast<const u32x4*>(slot + kMT * 2048 + frag[u]);
+            for (int w = 0; w < kWT; ++w)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) wf[w][u] = *reinterpret_cast<const u32x4*>(slot + (kMT + w) * 2048 + frag[u]);
 #pragma unroll
             for (int t = 0; t < kMT; ++t)
 #pragma unroll
                 for (int u = 0; u < 2; ++u) x[t][u] = *reinterpret_cast<const u32x4*>(slot + t * 2048 + frag[u]);
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int w = 0; w < kWT; ++w)
 #pragma unroll
-                for (int t = 0; t < kMT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, wf[u]),
-                                                                    __builtin_bit_cast(h16x8, x[t][u]),
-                                                                    acc[t], 0, 0, 0);
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int t = 0; t < kMT; ++t)
+                        acc[w][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, wf[w][u]),
+                                                                           __builtin_bit_cast(h16x8, x[t][u]),
+                                                                           acc[w][t], 0, 0, 0);
             if (i + Shape::kDepth < mine) {
                 // the slot is read (its fragments are in registers) before it is refilled
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -909,11 +918,13 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                                          // every wave is done with its ring: it becomes `part`
-    f32x4 (*part)[kMT][kWave] = reinterpret_cast<f32x4 (*)[kMT][kWave]>(skinny_lds);
+    f32x4 (*part)[kWT * kMT][kWave] = reinterpret_cast<f32x4 (*)[kWT * kMT][kWave]>(skinny_lds);
 #pragma unroll
-    for (int t = 0; t < kMT; ++t) part[wave][t][lane] = acc[t];
+    for (int w = 0; w < kWT; ++w)
+#pragma unroll
+        for (int t = 0; t < kMT; ++t) part[wave][w * kMT + t][lane] = acc[w][t];
     __syncthreads();
-    skinny_store<kMT>(part, C, bias, M, N, n0, vec_store, alpha, beta);
+    skinny_store<kMT, kWT>(part, C, bias, M, N, n0, vec_store, alpha, beta);
 }
 
 // The 64-column tile count below which the weight-streaming kernel beats the
@@ -925,14 +936,20 @@ inline bool skinny_serves(int M, int N) { return M >= 2 && (M <= 16 || (M <= 64 
 template <typename Kernel>
 bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes);
 
-template <int kMT>
+template <int kMT, int kWT>
 bool launch_skinny_lines(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha, float beta,
                          hipStream_t st) {
     static thread_local int ready = -1;
-    if (!allow_big_lds(gemm_skinny_lines<kMT>, ready, SkinnyLines<kMT>::kLdsBytes)) return false;
-    gemm_skinny_lines<kMT><<<dim3((unsigned)blocks), kSkinnyWaves * kWave, SkinnyLines<kMT>::kLdsBytes, st>>>(
+    if (!allow_big_lds(gemm_skinny_lines<kMT, kWT>, ready, SkinnyLines<kMT, kWT>::kLdsBytes)) return false;
+    gemm_skinny_lines<kMT, kWT><<<dim3((unsigned)blocks), kSkinnyWaves * kWave, SkinnyLines<kMT, kWT>::kLdsBytes, st>>>(
         A, projs, M, K, alpha, beta);
     return true;
+}
+
+// One projection of up to 16 rows so wide that its 16-column blocks are more than two rounds of workgroups: 32
+// columns each (16 x 18944 x 3584: 32.9 -> 30.6 us; with more rows it gains nothing).
+inline bool skinny_pairs(const SkinnyProjs& projs, int blocks, int M) {
+    return M <= 16 && blocks > 512 && projs.first[1] == blocks && projs.first[2] == blocks;
 }
 
 template <int kFmt>
@@ -945,10 +962,16 @@ void launch_skinny_as(const h16* A, const SkinnyProjs& projs, int blocks, int M,
     if (kFmt == kWoF16 && K % 64 == 0) {
         bool aligned = aligned16(A);
         for (int p = 0; p < 3; ++p) aligned = aligned && (projs.w[p] == nullptr || aligned16(projs.w[p]));
-        if (aligned && (M <= 16 ? launch_skinny_lines<1>(A, projs, blocks, M, K, alpha, beta, st)
-                        : M <= 32 ? launch_skinny_lines<2>(A, projs, blocks, M, K, alpha, beta, st)
-                        : M <= 48 ? launch_skinny_lines<3>(A, projs, blocks, M, K, alpha, beta, st)
-                                  : launch_skinny_lines<4>(A, projs, blocks, M, K, alpha, beta, st)))
+        if (aligned && skinny_pairs(projs, blocks, M)) {
+            SkinnyProjs wide = projs;
+            const int pairs = (blocks + 1) / 2;
+            wide.first[1] = wide.first[2] = pairs;
+            if (launch_skinny_lines<1, 2>(A, wide, pairs, M, K, alpha, beta, st)) return;
+        }
+        if (aligned && (M <= 16 ? launch_skinny_lines<1, 1>(A, projs, blocks, M, K, alpha, beta, st)
+                        : M <= 32 ? launch_skinny_lines<2, 1>(A, projs, blocks, M, K, alpha, beta, st)
+                        : M <= 48 ? launch_skinny_lines<3, 1>(A, projs, blocks, M, K, alpha, beta, st)
+                                  : launch_skinny_lines<4, 1>(A, projs, blocks, M, K, alpha, beta, st)))
             return;
     }
     if (M <= 16) gemm_skinny<1, kFmt><<<grid, kThreads, 0, st>>>(A, projs, M, K, alpha, beta);
