@@ -754,8 +754,10 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
     f16 = dict(dtype=torch.float16, device="cuda")
     QD, KD = NQ * HD, NK * HD
     w = lambda *shape, std: torch.randn(*shape, **f16) * std
-    wq, wk, wv, wo = w(QD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(H, QD, std=QD ** -0.5)
-    wg, wu, wd = w(I_FF, H, std=H ** -0.5), w(I_FF, H, std=H ** -0.5), w(H, I_FF, std=I_FF ** -0.5)
+    def weights():
+        return (w(QD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(KD, H, std=H ** -0.5), w(H, QD, std=QD ** -0.5),
+                w(I_FF, H, std=H ** -0.5), w(I_FF, H, std=H ** -0.5), w(H, I_FF, std=I_FF ** -0.5))
+    layer0 = weights()
     bq, bk, bv = w(QD, std=0.1), w(KD, std=0.1), w(KD, std=0.1)
     n1, n2 = 1 + w(H, std=0.1), 1 + w(H, std=0.1)
     C_ROWS = min(chunk, T)
@@ -779,10 +781,13 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
     def gemm(x, wt, y, m, n, kk):
         assert dev.vv_gemm_fp16_dev(x, P(wt), P(y), m, n, kk, 1.0, 0.0, st) == 0
 
-    def qkv(start, n, fused):
+    def qkv(start, n, fused, ws=layer0):
+        wq, wk, wv = ws[:3]
         x = P(normed_in) + start * H * 2
         if fused:
-            assert dev.vv_gemm_qkv_rope_dev(x, P(wq), P(wk), P(wv), P(bq), P(bk), P(bv), P(q), None, None, n, NQ, NK,
+            # (up to 64 rows the entry point runs the separate launches, which need the k and v buffers)
+            kb, vb = (P(k), P(v)) if n <= 64 else (None, None)
+            assert dev.vv_gemm_qkv_rope_dev(x, P(wq), P(wk), P(wv), P(bq), P(bk), P(bv), P(q), kb, vb, n, NQ, NK,
                                             HD, H, P(rope_table) + start * HD * 4, P(kc), P(vc), None, start, None,
                                             st) == 0
             return
@@ -798,9 +803,10 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
         assert dev.vv_dev_memcpy_d2d(P(kc) + start * KD * 2, P(k), n * KD * 2, st) == 0
         assert dev.vv_dev_memcpy_d2d(P(vc) + start * KD * 2, P(v), n * KD * 2, st) == 0
 
-    def one_chunk(start, n, fused):
+    def one_chunk(start, n, fused, ws=layer0):
+        wo, wg, wu, wd = ws[3:]
         h = P(hidden) + start * H * 2
-        qkv(start, n, fused)
+        qkv(start, n, fused, ws)
         assert dev.vv_attn_prefill(2, P(q), C.addressof(view), P(attn), NQ, n, start, start + n, True, P(attn_scratch),
                                    st) == 0
         gemm(P(attn), wo, proj, n, H, QD)
@@ -851,17 +857,42 @@ def prefill_chunked_leg(torch, dev, T: int, st: int, chunk: int = 2048) -> dict:
         per.sort()
         return n, per[1]
 
+    def time_stream(fused, rows=24, launches=12):
+        """A streaming chunk: `rows` rows through the layer on top of the filled cache (the reference's prefill on a
+        cache that already holds the session, decoder.c:1112-1114), three layers' weights in rotation (1.4 GB: past
+        every cache, as in a 28-layer model)."""
+        s0 = T - rows
+        for ws in layers:
+            one_chunk(s0, rows, fused, ws)
+        per = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(launches):
+                one_chunk(s0, rows, fused, layers[i % len(layers)])
+            e1.record()
+            e1.synchronize()
+            per.append(e0.elapsed_time(e1) * 1e3 / launches)
+        per.sort()
+        return per[1]
+
     ms_api, chunks_api = time_layer(False)
     ms, chunks_ms = time_layer(True)
     assert bool(torch.isfinite(hidden).all())
     rows_qkv, us_qkv = time_qkv(True)
     _, us_qkv_api = time_qkv(False)
+    layers = [layer0, weights(), weights()]
+    stream_rows = 24
+    us_stream, us_stream_api = time_stream(True, stream_rows), time_stream(False, stream_rows)
+    del layers
     flops = 2.0 * T * H * (2 * QD + 2 * KD + 3 * I_FF) + 4.0 * NQ * HD * T * (T + 1) / 2
     return {"rows": T, "chunk_rows": [n for _, n in chunks], "ms_per_layer": ms, "ms_per_chunk": chunks_ms,
             "ms_per_layer_reference_api_calls": ms_api, "ms_per_chunk_reference_api_calls": chunks_api,
             "launches_per_chunk": 7, "launches_per_chunk_reference_api_calls": 20,
             "qkv_leg": {"rows": rows_qkv, "us": us_qkv, "us_reference_api_calls": us_qkv_api,
                         "TFLOPs": 2.0 * rows_qkv * (QD + 2 * KD) * H / us_qkv / 1e6},
+            "stream_chunk": {"rows": stream_rows, "cache_len": T, "us_per_layer": us_stream,
+                             "us_per_layer_reference_api_calls": us_stream_api, "weight_sets_in_rotation": 3},
             "TFLOPs": flops / ms / 1e9, "layers_assumed": 28, "prompt_tokens_per_s": T / (28 * ms * 1e-3)}
 
 
@@ -1382,6 +1413,10 @@ def layer_legs(torch, dev, T: int, st: int, args, fp16_only: bool) -> dict:
         f"calls of the reference's device.h alone); q/k/v + bias + RoPE + append of {d['qkv_leg']['rows']} rows "
         f"{d['qkv_leg']['us']:.1f} us in one launch, {d['qkv_leg']['us_reference_api_calls']:.1f} us in ten; "
         f"28 layers = {d['prompt_tokens_per_s']:.0f} prompt tokens/s")
+    sc = d["stream_chunk"]
+    log(f"  a streaming chunk of {sc['rows']} rows on top of the {sc['cache_len']}-position cache, one layer (three layers' "
+        f"weights in rotation): {sc['us_per_layer']:.1f} us ({sc['us_per_layer_reference_api_calls']:.1f} us on the calls "
+        f"of the reference's device.h alone)")
     for kind in () if fp16_only else ("w8a8", "w4a8", "w4a16"):
         torch.cuda.empty_cache()
         layer["prefill_layer_" + kind] = d = prefill_layer_quant_leg(torch, dev, T, st, kind)

@@ -727,7 +727,9 @@ vv_status_t vv_gemm_bias_rope_dev(const void* A, const void* W, const void* bias
  * vv_bias_add_dev (v) and vv_kv_store_dev bit for bit. One grid of equal tiles serves
  * 7 query heads per KV head with head_dim 128 (28 + 4 heads: a tile is one q or k head
  * plus 16 columns of v), more than 64 rows, K % 64 == 0; other shapes run the separate
- * calls through k and v (VV_ERR_UNSUPPORTED if those are NULL). Biases may be NULL.
+ * calls through k and v (VV_ERR_UNSUPPORTED if those are NULL) - 2 .. 64 rows, a streaming
+ * chunk, as three launches: the three projections with their biases in one launch of the
+ * small-M kernel, one rotation of q and k, the append. Biases may be NULL.
  * q, k, v, the caches, the biases and the table must be 16-byte aligned
  * (VV_ERR_UNSUPPORTED otherwise, nothing launched). */
 vv_status_t vv_gemm_qkv_rope_dev(const void* x, const void* wq, const void* wk, const void* wv,

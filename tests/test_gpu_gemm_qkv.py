@@ -72,7 +72,10 @@ SERVED = [(2048, 28, 4, 3584), (2049, 28, 4, 256), (1000, 28, 4, 3584), (65, 28,
           (4100, 28, 4, 128), (14449, 28, 4, 64), (300, 14, 2, 128), (2100, 14, 2, 64), (130, 7, 1, 320),
           (3000, 7, 1, 64)]
 # what the one-grid tile does not serve: another head ratio, up to 64 rows, rows that are not whole 64-half slabs
-OTHER = [(300, 12, 2, 128), (64, 28, 4, 128), (1, 28, 4, 3584), (200, 28, 4, 72), (100, 4, 4, 64)]
+OTHER = [(300, 12, 2, 128), (64, 28, 4, 128), (1, 28, 4, 3584), (200, 28, 4, 72), (100, 4, 4, 64),
+         # 2 .. 64 rows (a streaming chunk): the three projections in one launch of the weight-streaming kernel, one
+         # rotation of q and k, the append - whole 64-K lines, another K, two rows, another head ratio
+         (24, 28, 4, 3584), (2, 14, 2, 64), (33, 28, 4, 72), (50, 7, 1, 128), (17, 12, 2, 192)]
 
 
 @pytest.mark.parametrize("M,nq,nkv,K", SERVED + OTHER)
@@ -90,7 +93,8 @@ def test_one_launch_equals_the_separate_launches(M, nq, nkv, K, with_bias):
     assert np.array_equal(bits_of(fv), bits_of(v)), "v"
 
 
-@pytest.mark.parametrize("M,nq,nkv,K", [(2048, 28, 4, 256), (333, 28, 4, 64), (700, 14, 2, 128), (300, 12, 2, 128)])
+@pytest.mark.parametrize("M,nq,nkv,K", [(2048, 28, 4, 256), (333, 28, 4, 64), (700, 14, 2, 128), (300, 12, 2, 128),
+                                      (24, 28, 4, 256)])
 @pytest.mark.parametrize("paged", [False, True])
 def test_rows_land_in_the_cache(M, nq, nkv, K, paged):
     """The k and v rows in an FP16 cache at positions pos .. pos + M - 1 == vv_kv_store_dev of the separate
@@ -109,7 +113,7 @@ def test_rows_land_in_the_cache(M, nq, nkv, K, paged):
     want_k, want_v = nan16(cap, nkv, HD), nan16(cap, nkv, HD)
     ok(dev.vv_kv_store_dev(k.data_ptr(), v.data_ptr(), want_k.data_ptr(), want_v.data_ptr(), None, None, None, False,
                            nkv, HD, pos, None, M, 0, ptr(page_table), stream()))
-    served = nq == 7 * nkv
+    served = nq == 7 * nkv and M > 64           # up to 64 rows: separate launches, which need the k and v buffers
     for d_pos in (None, torch.tensor([pos], dtype=torch.int32, device="cuda")):
         for buffers in (True, False):
             kc, vc = nan16(cap, nkv, HD), nan16(cap, nkv, HD)

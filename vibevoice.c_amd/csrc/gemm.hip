@@ -1380,6 +1380,9 @@ vv_status_t vv_gemm_tile_weight_only(int format, const void* A, const void* w, c
 
 // rope.hip: x[rows][heads][128] = rope(x + bias), cos/sin from a vv_rope_table_dev table.
 vv_status_t vv_rope128_from_table(void* x, const void* bias, const void* table, int rows, int heads, void* stream);
+// rope.hip: two tensors of heads_a and heads_b heads rotated in one launch.
+vv_status_t vv_rope128_pair_from_table(void* a, void* b, const void* table, int rows, int heads_a, int heads_b,
+                                       void* stream);
 
 extern "C" {
 
@@ -1524,6 +1527,34 @@ vv_status_t vv_gemm_qkv_rope_dev(const void* x, const void* wq, const void* wk, 
     }
     // Everything else: the separate launches, through the caller's k and v buffers.
     if (!k || !v) return VV_ERR_UNSUPPORTED;
+    // 2 .. 64 rows (a streaming chunk): the three projections with their biases in one launch of the weight-streaming
+    // kernel - which is what each of the calls below would run for its own projection, so the same bits - then one
+    // rotation of the q and k rows, then the append: three launches instead of seven.
+    const int nq_cols = n_q_heads * head_dim, nkv_cols = n_kv_heads * head_dim;
+    if (vv::forced_tile() == 0 && M >= 2 && M <= 64 && K > 0 && K % 8 == 0 && vv::skinny_serves(M, nq_cols) &&
+        vv::skinny_serves(M, nkv_cols) && vv::aligned16(x) && vv::aligned16(wq) && vv::aligned16(wk) && vv::aligned16(wv)) {
+        vv::SkinnyProjs p = {};
+        const void* ws[3] = {wq, wk, wv};
+        const void* bs[3] = {bq, bk, bv};
+        void* ys[3] = {q, k, v};
+        int blocks = 0;
+        for (int i = 0; i < 3; ++i) {
+            p.first[i] = blocks;
+            p.w[i] = ws[i];
+            p.bias[i] = static_cast<const vv::h16*>(bs[i]);
+            p.y[i] = static_cast<vv::h16*>(ys[i]);
+            p.n[i] = i == 0 ? nq_cols : nkv_cols;
+            p.vec[i] = 1;                                      // whole heads of 128 columns, 16-byte aligned rows
+            blocks += (p.n[i] + 15) / 16;
+        }
+        vv::launch_skinny(static_cast<const vv::h16*>(x), p, blocks, M, K, 1.0f, 0.0f, vv::as_stream(stream));
+        vv_status_t s = vv::launch_status();
+        if (s != VV_OK) return s;
+        s = vv_rope128_pair_from_table(q, k, rope_table, M, n_q_heads, n_kv_heads, stream);
+        if (s != VV_OK || !k_cache) return s;
+        return vv_kv_store_dev(k, v, k_cache, v_cache, nullptr, nullptr, nullptr, false, n_kv_heads, head_dim, pos,
+                               d_pos, M, 0, page_table, stream);
+    }
     vv_status_t s = vv_gemm_bias_rope_dev(x, wq, bq, q, M, n_q_heads, head_dim, K, rope_table, stream);
     if (s != VV_OK) return s;
     s = vv_gemm_bias_rope_dev(x, wk, bk, k, M, n_kv_heads, head_dim, K, rope_table, stream);

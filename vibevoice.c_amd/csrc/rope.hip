@@ -309,6 +309,34 @@ __global__ __launch_bounds__(kBlock) void rope128_from_table(h16* __restrict__ x
     store_chunk(lo_p + 8, pack(y1));
 }
 
+// The same rotation of two tensors in one launch (the q and k rows of a chunk): head h < heads_a is a's, the rest b's.
+__global__ __launch_bounds__(kBlock) void rope128_pair_from_table(h16* __restrict__ a, h16* __restrict__ b,
+                                                                  const float2* __restrict__ table, int rows,
+                                                                  int heads_a, int heads_b) {
+    const size_t item = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const int heads = heads_a + heads_b;
+    if (item >= (size_t)rows * heads * 8) return;
+    const int c = (int)(item & 7);
+    const size_t rh = item >> 3;
+    const int head = (int)(rh % heads);
+    const size_t row = rh / heads;
+    h16* x = head < heads_a ? a + (row * heads_a + head) * 128u : b + (row * heads_b + (head - heads_a)) * 128u;
+    Chunk* lo_p = reinterpret_cast<Chunk*>(x) + c;
+    const Chunk lo = load_chunk(lo_p), hi = load_chunk(lo_p + 8);
+    const float2* t = table + row * 64 + c * 8;
+    const f32x8 x0 = unpack(lo), x1 = unpack(hi);
+    f32x8 y0, y1;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float2 cs = t[i];
+        const Pair r = rotate(x0[i], x1[i], cs.x, cs.y);
+        y0[i] = r.lo;
+        y1[i] = r.hi;
+    }
+    store_chunk(lo_p, pack(y0));
+    store_chunk(lo_p + 8, pack(y1));
+}
+
 // The table depends only on (theta, head_dim); each host thread remembers the
 // last one it built (thread-local, so concurrent callers never share state).
 const FreqTable& host_freqs(float theta, int head_dim) {
@@ -450,6 +478,18 @@ vv_status_t vv_rope_table_dev(void* table, int seq_len, int head_dim, int positi
 }
 
 }  // extern "C"
+
+// For gemm.hip: a[rows][heads_a][128] and b[rows][heads_b][128] rotated in place in one launch, cos/sin from a
+// vv_rope_table_dev table (16-byte aligned tensors, table rows 0 .. rows - 1).
+__attribute__((visibility("hidden")))
+vv_status_t vv_rope128_pair_from_table(void* a, void* b, const void* table, int rows, int heads_a, int heads_b,
+                                       void* stream) {
+    const size_t items = (size_t)rows * (size_t)(heads_a + heads_b) * 8u;
+    vv::rope128_pair_from_table<<<dim3((unsigned)((items + vv::kBlock - 1) / vv::kBlock)), vv::kBlock, 0,
+                                  vv::as_stream(stream)>>>(static_cast<vv::h16*>(a), static_cast<vv::h16*>(b),
+                                                           static_cast<const float2*>(table), rows, heads_a, heads_b);
+    return vv::launch_status();
+}
 
 // For gemm.hip: x[rows][heads][128] = rope(x + bias) with cos/sin from a vv_rope_table_dev table
 // (16-byte aligned x and bias, table rows 0 .. rows - 1).
