@@ -753,7 +753,8 @@ vv_status_t vv_gemv_multi_dev(const void* x, const vv_skinny_proj_t* projs, int 
  * vv_gemm_fp16_dev and vv_swiglu_dev). Gate and up are rounded to FP16 where the
  * two GEMMs store and go through the SwiGLU kernel's own function in the GEMM's
  * store, so the result equals the three calls bit for bit and gate and up are
- * never written. Fused for M > 64, K % 64 == 0 and 16-byte aligned A, Wg, Wu;
+ * never written. Fused for M > 64, K % 64 == 0 and 16-byte aligned A, Wg, Wu, and
+ * for 17 .. 64 rows (a streaming chunk) against an N of 12800 or more;
  * one row runs vv_gemv_swiglu_dev; every other shape runs the three calls through
  * the caller's `gate` and `up`
  * buffers ([M, N] each; NULL: VV_ERR_UNSUPPORTED for those shapes, nothing

@@ -62,7 +62,7 @@ SHAPES = [(1, 64, 64), (2, 48, 32), (16, 30, 40), (17, 100, 264), (33, 77, 520),
           (17, 100, 320), (33, 52, 64), (40, 3584, 18944), (64, 3584, 1088), (48, 30, 4096), (20, 3584, 3584),
           (2, 264, 3584), (5, 3584, 18944), (16, 18944, 3584), (13, 50, 64),
           # 17 .. 64 rows, N too wide for that kernel: one row of 128x128 tiles (and just below their bar: 64-wide ones)
-          (24, 18944, 3584), (64, 16300, 128), (33, 16200, 128),
+          (24, 18944, 3584), (64, 16300, 128), (33, 16200, 128), (17, 12800, 64), (48, 13000, 448), (32, 12900, 72),
           # one row, few long weight rows: two output columns per wave (an odd count leaves the last wave one)
           (1, 3584, 18944), (1, 37, 8192), (1, 1, 8200)]
 
@@ -79,10 +79,10 @@ def test_gemm_against_oracle_and_tile(M, N, K):
     d_t = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     tile = run(dev.vv_gemm_fp16_tile_dev, d_a, d_b, d_t, M, N, K)
     check(tile, ref, mag, f"tile {M}x{N}x{K}")
-    big = K % 64 == 0 and (M > 64 or (M > 16 and N >= 16257))      # the latter: one row of at least 128 tiles of 128
+    big = K % 64 == 0 and (M > 64 or (M > 16 and N >= 12800))      # the latter: too wide for the weight-streaming kernel
     if big:
-        # the tiles fed in 128-byte slabs (the choice above 64 rows, and from 17 rows on where N is very wide, when
-        # K % 64 == 0) multiply with the 16x16x32
+        # the tiles fed in 128-byte slabs (the choice above 64 rows when K % 64 == 0) and the kernel that streams 128
+        # columns a workgroup (17 .. 64 rows where N is very wide) multiply with the 16x16x32
         # instructions, which add 32 products at a time where the other tiles add 16: same sums, another
         # rounding of the FP32 partials
         diff = np.abs(oracle.widen(got) - oracle.widen(tile))

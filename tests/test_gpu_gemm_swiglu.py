@@ -83,6 +83,22 @@ def test_other_shapes_run_the_three_calls(M, N, K):
     assert np.isnan(oracle.widen(got)).all(), "declined: nothing launched"
 
 
+@pytest.mark.parametrize("M,N,K", [(24, 18944, 3584), (17, 12800, 64), (64, 13000, 448), (33, 18944, 128), (32, 33000, 64)])
+def test_a_streaming_chunk_against_a_wide_n(M, N, K):
+    """17 .. 64 rows of whole 64-K lines against an N too wide for the small-M kernel: vv_gemm_fp16_dev streams 128
+    columns a workgroup there, and the fused entry point runs that kernel on both matrices at once with SwiGLU in its
+    store - the three calls' bits, with or without the gate and up buffers (which it leaves alone)."""
+    d_a = to_dev(oracle.normal_f16((M, K), 41))
+    d_g = to_dev(oracle.normal_f16((N, K), 42, std=K ** -0.5))
+    d_u = to_dev(oracle.normal_f16((N, K), 43, std=K ** -0.5))
+    gate, up, want = separate(d_a, d_g, d_u, M, N, K)
+    st, got, gate_buf = fused(d_a, d_g, d_u, M, N, K)
+    assert st == dev.VV_OK and np.array_equal(got, want)
+    assert np.isnan(oracle.widen(gate_buf)).all()
+    st, got, _ = fused(d_a, d_g, d_u, M, N, K, buffers=False)
+    assert st == dev.VV_OK and np.array_equal(got, want)
+
+
 def test_against_the_oracle_chain():
     M, N, K = 300, 264, 320
     a, g, u = oracle.normal_f16((M, K), 31), oracle.normal_f16((N, K), 32, std=K ** -0.5), oracle.normal_f16((N, K), 33, std=K ** -0.5)

@@ -927,14 +927,203 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_lines(
     skinny_store<kMT, kWT>(part, C, bias, M, N, n0, vec_store, alpha, beta);
 }
 
+template <typename Kernel>
+bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes);
+
+// 17 .. 64 rows against a very wide N (the gate and up projections of a streaming chunk): a
+// 128x128 tile spends its time on the 128 rows it copies and multiplies whatever the chunk has, and the K-split
+// kernel above has eight waves share 56 lines of a 3584-wide row - seven round trips to memory each, two lines
+// deep. Here a workgroup takes 128 output columns and ALL of K: wave w streams the sixteen weight rows of its own
+// columns through a ring of its own, kDepth - 1 lines ahead, and the chunk's rows - 16 kMT of them, one ring for
+// the workgroup, each wave copying its share of a line - are read by all eight. One barrier per line tells a wave
+// that the others' shares of line i have landed and that all have finished with line i - 1, whose slots the next
+// copies then take. Every copy is whole cache lines (eight rows of 128 bytes, the chunk XOR the row); every output
+// has one accumulator that adds the K steps in order, as the copy-fed tiles do: the same bits as gemm_dma64.
+// kW: waves, i.e. 16-column strips, per workgroup (eight: with four, twice the workgroups, it is 12 % slower). Bare
+// 16-byte loads of the same bytes in the same grid take 24.9 us for 18944 x 3584 (5.45 TB/s), this kernel 28.5 - 34.5
+// from 17 to 64 rows.
+template <int kMT, int kW, int kMats = 1> struct StripShape {
+    static constexpr int kDepth = kMats == 2 ? 4 : kMT <= 4 ? 6 : 4;                  // ring slots (lines)
+    static constexpr int kXCopies = 2 * kMT;                                          // copies of a line of the rows
+    static constexpr int kXLine = kMT * 2048, kWLine = 2048 * kMats;      // a wave's sixteen rows of each matrix
+    static constexpr size_t kLdsBytes = (size_t)kDepth * (kXLine + kW * kWLine);     // 120 / 144 KB; two matrices: 144 / 160
+    static_assert(kLdsBytes <= 160 * 1024, "the rings fit");
+    static_assert(kXCopies <= kW || kXCopies % kW == 0, "a wave's share of a line is fixed");
+    // copies a wave issues per line: its two of the weights, its share of the rows
+    static __device__ __forceinline__ constexpr int x_share(int wave) {
+        return kXCopies >= kW ? kXCopies / kW : (wave < kXCopies ? 1 : 0);
+    }
+    static_assert((kDepth - 2) * (2 * kMats + (kXCopies + kW - 1) / kW) < 64, "a wave's six-bit load counter");
+};
+
+// kMats = 2: the gate and up projections at once - W2 is the second matrix, a wave's ring holds sixteen rows of each,
+// and the store is the SwiGLU of the two products, each rounded to FP16 first (store_tile16_swiglu's arithmetic: the
+// same bits as the two products and vv_swiglu_dev, without gate and up going to memory).
+template <int kMT, int kW, int kMats>
+__global__ __launch_bounds__(kW * kWave) void gemm_strip(
+    const h16* __restrict__ A, const h16* __restrict__ W, const h16* __restrict__ W2, h16* __restrict__ C, int M,
+    int N, int K, float alpha, float beta, int vec_store) {
+    typedef StripShape<kMT, kW, kMats> Shape;
+    extern __shared__ __align__(16) char strip_lds[];
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, ks = lane >> 4;
+    const int n0 = (int)blockIdx.x * (16 * kW) + wave * 16;
+    const int nlines = K / 64;
+    const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)strip_lds);
+    const uint32_t x_ring = lds0, w_ring = lds0 + Shape::kDepth * Shape::kXLine + (uint32_t)wave * (Shape::kDepth * Shape::kWLine);
+    const char* x_lds = strip_lds;
+    const char* w_lds = strip_lds + Shape::kDepth * Shape::kXLine + (size_t)wave * (Shape::kDepth * Shape::kWLine);
+
+    // this lane's part of a copy: row lane / 8 of its eight, the chunk whose slot in the row is lane % 8
+    const int r8 = lane >> 3;
+    const uint32_t in_row = (uint32_t)(((lane & 7) ^ r8) * 16);
+    const char* wrow[2 * kMats];                               // copies 0, 1: W's sixteen rows; 2, 3: W2's
+#pragma unroll
+    for (int j = 0; j < 2 * kMats; ++j)
+        wrow[j] = reinterpret_cast<const char*>((j < 2 ? W : W2) + (size_t)min(n0 + 8 * (j & 1) + r8, N - 1) * K) + in_row;
+    constexpr int kMine = Shape::kXCopies >= kW ? Shape::kXCopies / kW : 1;
+    const char* xrow[kMine];
+    int xcopy[kMine];
+#pragma unroll
+    for (int q = 0; q < kMine; ++q) {
+        xcopy[q] = wave + kW * q;                    // which copy of the line (eight rows each)
+        xrow[q] = reinterpret_cast<const char*>(A + (size_t)min(8 * xcopy[q] + r8, M - 1) * K) + in_row;
+    }
+    const bool copies_x = Shape::kXCopies >= kW || wave < Shape::kXCopies;
+    uint32_t frag[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) frag[u] = (uint32_t)((r16 >> 3) * 1024 + (r16 & 7) * 128 + (((4 * u + ks) ^ (r16 & 7)) * 16));
+
+    auto request = [&](int line, int slot) {
+        const size_t at = (size_t)line * 128;
+#pragma unroll
+        for (int j = 0; j < 2 * kMats; ++j)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         : : "s"(w_ring + (uint32_t)slot * Shape::kWLine + (uint32_t)j * 1024u), "v"(wrow[j] + at) : "memory", "m0");
+        if (copies_x) {
+#pragma unroll
+            for (int q = 0; q < kMine; ++q)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                             : : "s"(x_ring + (uint32_t)slot * Shape::kXLine + (uint32_t)xcopy[q] * 1024u), "v"(xrow[q] + at) : "memory", "m0");
+        }
+    };
+
+    f32x4 acc[kMats][kMT];
+#pragma unroll
+    for (int g = 0; g < kMats; ++g)
+#pragma unroll
+        for (int t = 0; t < kMT; ++t) acc[g][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < Shape::kDepth - 1; ++d)
+        if (d < nlines) request(d, d);
+    // (unrolled by the depth, so that a line's slots are fixed; every wave walks every line: the barriers match)
+    for (int i0 = 0; i0 < nlines; i0 += Shape::kDepth) {
+#pragma unroll
+        for (int d = 0; d < Shape::kDepth; ++d) {
+            const int i = i0 + d;
+            if (i >= nlines) break;
+            // this wave's copies of line i have landed when only those of the kDepth - 2 lines behind it are
+            // still counted; towards the end fewer are behind it, and the wave waits for them all
+            if (i + Shape::kDepth - 2 < nlines) {
+                if (copies_x)
+                    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((Shape::kDepth - 2) * (2 * kMats + kMine)) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(%0)" : : "n"((Shape::kDepth - 2) * 2 * kMats) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __syncthreads();                                  // the others' shares of line i; all are done with line i - 1
+            if (i + Shape::kDepth - 1 < nlines) request(i + Shape::kDepth - 1, (d + Shape::kDepth - 1) % Shape::kDepth);
+            u32x4 x[kMT][2], wf[kMats][2];
+#pragma unroll
+            for (int g = 0; g < kMats; ++g)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+                    wf[g][u] = *reinterpret_cast<const u32x4*>(w_lds + d * Shape::kWLine + g * 2048 + frag[u]);
+#pragma unroll
+            for (int t = 0; t < kMT; ++t)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) x[t][u] = *reinterpret_cast<const u32x4*>(x_lds + d * Shape::kXLine + t * 2048 + frag[u]);
+#pragma unroll
+            for (int g = 0; g < kMats; ++g)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int t = 0; t < kMT; ++t)
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, wf[g][u]),
+                                                                           __builtin_bit_cast(h16x8, x[t][u]),
+                                                                           acc[g][t], 0, 0, 0);
+        }
+    }
+    // register r of lane l of tile t: column n0 + 4 (l / 16) + r of row 16 t + l % 16
+    const int n = n0 + 4 * ks;
+    if (n >= N) return;
+#pragma unroll
+    for (int t = 0; t < kMT; ++t) {
+        const int m = 16 * t + r16;
+        if (m >= M) continue;
+        h16* crow = C + (size_t)m * N;
+        typedef h16 h16x4 __attribute__((ext_vector_type(4)));
+        if constexpr (kMats == 2) {
+            h16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                o[r] = to_half(swiglu1((float)to_half(acc[0][t][r]), (float)to_half(acc[1][t][r])));
+            if (vec_store && n + 3 < N) {
+                *reinterpret_cast<h16x4*>(crow + n) = o;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) crow[n + r] = o[r];
+            }
+        } else if (vec_store && n + 3 < N) {
+            h16x4 old = {0, 0, 0, 0};
+            if (beta != 0.0f) old = *reinterpret_cast<const h16x4*>(crow + n);
+            h16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = to_half(finish(acc[0][t][r], alpha, beta, old[r]));
+            *reinterpret_cast<h16x4*>(crow + n) = o;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) {
+                    const h16 old = beta != 0.0f ? crow[n + r] : (h16)0.0f;
+                    crow[n + r] = to_half(finish(acc[0][t][r], alpha, beta, old));
+                }
+        }
+    }
+}
+
+// B2 given: C = swiglu(fp16(A B^T), fp16(A B2^T)) (alpha and beta unused)
+template <int kMT, int kW, int kMats = 1>
+bool launch_strip(const void* A, const void* B, void* C, int M, int N, int K, float alpha, float beta, hipStream_t st,
+                  const void* B2 = nullptr) {
+    static thread_local int ready = -1;
+    typedef StripShape<kMT, kW, kMats> Shape;
+    if (!allow_big_lds(gemm_strip<kMT, kW, kMats>, ready, Shape::kLdsBytes)) return false;
+    const int vec = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0);
+    gemm_strip<kMT, kW, kMats><<<dim3((unsigned)((N + 16 * kW - 1) / (16 * kW))), kW * kWave, Shape::kLdsBytes, st>>>(
+        static_cast<const h16*>(A), static_cast<const h16*>(B), static_cast<const h16*>(B2), static_cast<h16*>(C), M, N,
+        K, alpha, beta, vec);
+    return true;
+}
+
+
+
 // The 64-column tile count below which the weight-streaming kernel beats the
 // tile kernel for 17..64 rows (M = 29, N = 18944 is 31 us tiled against 46 us
 // streamed; N = 3584, K = 18944 is 136 us against 48 us).
 inline bool few_tiles(int N) { return (long)((N + 63) / 64) < 200; }
 inline bool skinny_serves(int M, int N) { return M >= 2 && (M <= 16 || (M <= 64 && few_tiles(N))); }
 
-template <typename Kernel>
-bool allow_big_lds(Kernel kernel, int& ready_device, size_t bytes);
+// The shapes gemm() hands to gemm_strip: 17 .. 64 rows of whole 64-K lines against an N too wide for the
+// weight-streaming kernel (and not so wide that the 256x256 tiles would fill the chip twice).
+inline bool strip_serves(int M, int N, int K) {
+    return M > 16 && M <= 64 && K > 0 && K % 64 == 0 && !skinny_serves(M, N) &&
+           (long)((M + 255) / 256) * ((N + 255) / 256) < 512;
+}
 
 template <int kMT, int kWT>
 bool launch_skinny_lines(const h16* A, const SkinnyProjs& projs, int blocks, int M, int K, float alpha, float beta,
@@ -1191,9 +1380,15 @@ vv_status_t gemm(const void* A, const void* B, void* C, int M, int N, int K, flo
         // (copy-fed, four stages deep, the 128x128 tile already pays with half the compute units busy:
         // 1024 x 3584 x 3584 in 31 us as 224 tiles of 128, 50 us as 896 tiles of 64; at 112 tiles the 64s win)
         const long enough128 = K % (kDma64SlabBytes / 2) == 0 ? 128 : 256;
-        // (17 .. 64 rows arrive here when N is too wide for the weight-streaming kernel: one row of 128x128 tiles,
-        // bound by the weight bytes - 24 x 18944 x 3584 in 33 us against 46 us as 64-wide tiles)
+        // (17 .. 64 rows arrive here when N is too wide for the weight-streaming kernel; should the kernel below be
+        // refused: one row of 128x128 tiles)
         const bool rows128 = M > 64 || (M > 16 && K % (kDma64SlabBytes / 2) == 0);
+        // 17 .. 64 rows that arrive here (N too wide for the weight-streaming kernel), whole 64-K lines: the kernel
+        // that gives a workgroup 128 columns and all of K (24 x 18944 x 3584: 29 us; 33 us as one row of 128x128 tiles,
+        // which still serve 65 .. 128 rows, where it gains nothing; 46 us as 64-wide tiles)
+        if (strip_serves(M, N, K) && (M <= 32 ? launch_strip<2, 8>(A, B, C, M, N, K, alpha, beta, st)
+                                               : launch_strip<4, 8>(A, B, C, M, N, K, alpha, beta, st)))
+            return launch_status();
         choice = wg256 >= 512 ? k256 : (rows128 && wg128 >= enough128) ? k128dma : (M > 32) ? k64 : k32;
     }
     switch (choice) {
@@ -1590,6 +1785,13 @@ vv_status_t vv_gemm_swiglu_dev(const void* A, const void* w_gate, const void* w_
     }
     // One row: the decode step's own fused launch (equal to the three calls by its own contract).
     if (M == 1 && vv_gemv_swiglu_dev(A, w_gate, w_up, out, N, K, stream) == VV_OK) return VV_OK;
+    // 17 .. 64 rows against a very wide N (a streaming chunk): where vv_gemm_fp16_dev itself would stream 128 columns a
+    // workgroup, the same kernel on both matrices at once, SwiGLU in its store
+    if (vv::forced_tile() == 0 && vv::strip_serves(M, N, K) && vv::aligned16(A) && vv::aligned16(w_gate) &&
+        vv::aligned16(w_up) &&
+        (M <= 32 ? vv::launch_strip<2, 8, 2>(A, w_gate, out, M, N, K, 1.0f, 0.0f, vv::as_stream(stream), w_up)
+                 : vv::launch_strip<4, 8, 2>(A, w_gate, out, M, N, K, 1.0f, 0.0f, vv::as_stream(stream), w_up)))
+        return vv::launch_status();
     // Everything else: the three steps one after the other, through the caller's gate and up buffers.
     if (!gate || !up || (size_t)M * (size_t)N > 0x7fffffffu) return VV_ERR_UNSUPPORTED;
     vv_status_t s = vv::gemm(A, w_gate, gate, M, N, K, 1.0f, 0.0f, stream, vv::forced_tile(), true);
